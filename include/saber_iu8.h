@@ -1,0 +1,220 @@
+/* saber_iu8.h -- C ABI of the MI355X (gfx950) W4A8-iu8 decoder-linear path.
+ *
+ * The reference (GGZ14/saber-engine) crosses into device code through a data-only plugin
+ * boundary: a code object (`.hsaco`) plus a `.manifest.toml`, loaded and launched by its Rust
+ * host crates through a dlopen'd libamdhip64 (include/saber_abi.h:24-30 of the reference).
+ * This library is the C/C++ counterpart of those host crates for this one path, so that a host
+ * without them (or a binding in another language) can resolve, validate, load and launch the
+ * gfx950 code objects exactly as `saber-kernels` + `saber-exec` + `saber-hip` would.
+ * Each entry point names the reference interface it stands in for (paths relative to the
+ * reference tree).
+ *
+ * Conventions: plain pointers and sizes only. Every function returns 0 on success and a
+ * negative SABER_IU8_E_* code on failure; saber_iu8_last_error() returns the message of the
+ * calling thread's last failure. Device pointers are raw HIP device addresses owned by the
+ * caller; `stream` is a hipStream_t passed as void* (NULL = the null stream). All HIP calls of
+ * one context must come from one OS thread (crates/saber-hip/src/lib.rs:11-16).
+ */
+#ifndef SABER_IU8_H
+#define SABER_IU8_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SABER_IU8_ABI_VERSION 1
+
+/* error codes */
+#define SABER_IU8_OK 0
+#define SABER_IU8_E_RULE (-1)      /* a launch rule refused the shape (Error::Rule, macaq_iu8.rs:288-303) */
+#define SABER_IU8_E_PARSE (-2)     /* manifest / code object could not be parsed */
+#define SABER_IU8_E_VALIDATE (-3)  /* manifest does not describe the code object (manifest.rs:228-324) */
+#define SABER_IU8_E_HIP (-4)       /* a HIP call failed (message carries the status) */
+#define SABER_IU8_E_ARG (-5)       /* a null / missing / undersized argument */
+#define SABER_IU8_E_IO (-6)
+#define SABER_IU8_E_NOTLOADED (-7) /* kernel or plugin not in the loaded set */
+
+const char *saber_iu8_last_error(void);
+int saber_iu8_abi_version(void);
+
+/* ------------------------------------------------------------------ weight kinds, layouts */
+
+/* WKind (crates/saber-kernels/src/macaq_iu8.rs:64-72). */
+#define SABER_IU8_W4 0 /* per-row int4 [-8,7]   -> op "gemm_i4a8" */
+#define SABER_IU8_W8 1 /* per-row int8 [-127,127] -> op "gemm_i8a8" */
+
+/* gfx950 device-final layout ids. The reference's pack layouts 17/18 are gfx12 WMMA fragment
+ * orders (crates/saber-mem/src/pack/layout.rs:99-104); a new order is a new id
+ * (include/saber_abi.h:637-643 of the reference). */
+#define SABER_IU8_LAYOUT_I4_ROW_FRAG64 33
+#define SABER_IU8_LAYOUT_I8_ROW_FRAG64 34
+#define SABER_IU8_LAYOUT_A_TILED_I8_64 35
+
+/* Bytes of the A edge for m rows (padded to 16) of k int8 codes (Layout::ATiledI8,
+ * crates/saber-model/src/graph.rs:445-448: same size, gfx950 byte order). */
+size_t saber_iu8_a_bytes(uint32_t m, uint32_t k);
+/* Byte offset of activation (m,k) in the gfx950 A order / of weight byte (n,k) in the W8 order. */
+uint64_t saber_iu8_a_offset(uint32_t m, uint32_t k, uint32_t K);
+/* Byte offset of weight (n,k) in the gfx950 W4 order; *high = 1 when it is the high nibble. */
+uint64_t saber_iu8_w4_offset(uint32_t n, uint32_t k, uint32_t K, uint32_t *high);
+
+/* Offline repack, host memory to host memory. Canonical forms: W4 row-major [N][K/2], low nibble
+ * = even k (the export form, crates/saber-model/src/graph.rs:2591-2592); W8 and A row-major int8.
+ * N % 16 == 0 and K % 128 == 0 or SABER_IU8_E_RULE. `a` rows are padded to 16 with zeros. */
+int saber_iu8_repack_w4(const uint8_t *canonical, uint32_t n, uint32_t k, uint8_t *frag);
+int saber_iu8_repack_w8(const int8_t *rowmajor, uint32_t n, uint32_t k, uint8_t *frag);
+int saber_iu8_repack_a(const int8_t *rowmajor, uint32_t m, uint32_t k, uint8_t *frag);
+int saber_iu8_unpack_a(const uint8_t *frag, uint32_t m, uint32_t k, int8_t *rowmajor);
+/* The reference's gfx12 orders (layouts 17/18 and its A-tiled order) to the gfx950 orders, so a
+ * pack written for the reference can be re-ordered without going back to the export. */
+int saber_iu8_repack_w4_from_gfx12(const uint8_t *frag12, uint32_t n, uint32_t k, uint8_t *frag);
+int saber_iu8_repack_w8_from_gfx12(const uint8_t *frag12, uint32_t n, uint32_t k, uint8_t *frag);
+
+/* ------------------------------------------------------------------ launch descriptors */
+
+/* ArgValue (crates/saber-kernels/src/rules.rs): what the launcher writes into a kernarg slot. */
+#define SABER_IU8_ARG_BUFFER 0      /* device pointer of the named buffer */
+#define SABER_IU8_ARG_NULL_BUFFER 1 /* a named buffer passed as NULL (workspaces at ks == 1) */
+#define SABER_IU8_ARG_I32 2
+#define SABER_IU8_ARG_F32 3
+
+typedef struct {
+  char name[24];
+  uint32_t offset, size; /* natural alignment (abi.rs:111-130) */
+  uint32_t kind;         /* SABER_IU8_ARG_* */
+  int64_t ival;
+  float fval;
+} saber_iu8_slot;
+
+/* WorkspaceKind (crates/saber-kernels/src/rules.rs:473-482; include/saber_abi.h:163-174). */
+#define SABER_IU8_WS_SCRATCH 0    /* undefined at entry, written before read, aliasable */
+#define SABER_IU8_WS_PERSISTENT 1 /* zeroed once at allocation, left zero by the kernel */
+
+typedef struct {
+  char name[24];
+  uint32_t kind;
+  uint64_t bytes;
+  uint32_t zero_once;
+} saber_iu8_workspace;
+
+/* LaunchDescriptor (crates/saber-kernels/src/rules.rs:838-853). */
+typedef struct {
+  char op[24];
+  char plugin[24];
+  char kernel[64];
+  uint32_t grid[3];  /* in workgroups */
+  uint32_t block[3];
+  uint32_t shared_bytes;  /* always 0: LDS is static */
+  uint32_t kernarg_bytes; /* explicit arguments only */
+  uint32_t n_args;
+  saber_iu8_slot args[20];
+  uint32_t n_workspaces;
+  saber_iu8_workspace workspaces[4];
+  uint32_t n_launches; /* 1: split-K reduce is fused */
+  uint32_t ks;         /* grid-level split count (decode), 1 otherwise */
+} saber_iu8_desc;
+
+/* macaq_iu8::resolve(WKind, m, n, k) -> LaunchDescriptor (macaq_iu8.rs:425-427) under the gfx950
+ * launch law. Refuses (SABER_IU8_E_RULE) an empty launch, N % 16 != 0, K % 128 != 0. */
+int saber_iu8_resolve(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *out);
+/* The same descriptor for an explicitly named kernel of the object and split count (the
+ * autotuner's and the parity tests' entry: every variant of one regime gives the same bytes). */
+int saber_iu8_describe(const char *kernel, uint32_t m, uint32_t n, uint32_t k, uint32_t ks, saber_iu8_desc *out);
+/* The activation producer's descriptor (i8_twin's role, macaq_iu8.rs:881-916): bf16 [m,k] rows
+ * -> int8 A edge + f32 scales. */
+int saber_iu8_resolve_quant(uint32_t m, uint32_t k, saber_iu8_desc *out);
+/* SiLU(gate) * up + requant over rows of [gate(n) | up(n)] (abi.rs:315-320, 344-351). */
+int saber_iu8_resolve_silu_mul_quant(uint32_t rows, uint32_t n, saber_iu8_desc *out);
+
+/* abi::signature_for + abi::pack (abi.rs:111-130, 3495): fills names/offsets/sizes of the
+ * explicit arguments of `kernel`; returns the explicit kernarg size in *bytes. */
+int saber_iu8_signature(const char *kernel, saber_iu8_slot *slots, uint32_t cap, uint32_t *n_slots, uint32_t *bytes);
+
+/* A buffer binding: name -> device pointer. */
+typedef struct {
+  const char *name;
+  void *ptr;
+} saber_iu8_binding;
+
+/* pack_kernarg (crates/saber-exec/src/launch.rs:123): the zero-filled kernarg image of `desc`
+ * with 8-byte device pointers / i32 / f32 at their declared offsets. Pure host. */
+int saber_iu8_pack_kernarg(const saber_iu8_desc *desc, const saber_iu8_binding *bufs, uint32_t n_bufs, uint8_t *image,
+                           uint32_t cap, uint32_t *bytes);
+
+/* ------------------------------------------------------------------ manifests and code objects */
+
+/* saber-kbuild's manifest step (crates/saber-kernels/src/bin/saber-kbuild.rs:234-251,
+ * manifest.rs:136-226): reads the code object at `hsaco_path` (clang offload bundle or bare ELF)
+ * and writes `<plugin>.manifest.toml` (schema 1) to `out_path`. build_hash = sha256(preprocessed
+ * source ++ flags) is computed by the caller's build step and passed in. */
+int saber_iu8_manifest_write(const char *hsaco_path, const char *plugin, const char *arch, const char *source,
+                             const char *source_sha256, const char *flags, const char *build_hash, const char *out_path);
+
+/* The loader's three validations (crates/saber-exec/src/loader.rs:249-290): kernarg layout against
+ * the declared signature, one wave size per plugin, manifest against code object (sha256, target,
+ * kernarg size/align, LDS, registers, symbol, per-argument offset/size/value_kind). */
+#define SABER_IU8_REFUSED_KERNARG 1
+#define SABER_IU8_REFUSED_WAVE 2
+#define SABER_IU8_REFUSED_METADATA 3
+/* Returns 0 when the pair loads, SABER_IU8_E_VALIDATE when refused (*refusal names the counter
+ * that moves), SABER_IU8_E_PARSE / _IO when unreadable. */
+int saber_iu8_manifest_validate(const char *manifest_path, const char *arch, int *refusal);
+
+/* sha256 of a file, lowercase hex into out[65]. */
+int saber_iu8_sha256_file(const char *path, char *out65);
+
+/* ------------------------------------------------------------------ contexts, loading, launching */
+
+typedef struct saber_iu8_ctx saber_iu8_ctx;
+
+typedef struct {
+  uint32_t plugins_loaded, kernels_loaded;
+  uint32_t refused_kernarg, refused_wave, refused_metadata; /* loader.rs:249-270 */
+  uint32_t launches;
+} saber_iu8_counters;
+
+/* PluginSet::load_dir (crates/saber-exec/src/loader.rs:318-396): validates every
+ * `*.manifest.toml` under `prebuilt_dir` (the gfx950 directory) and loads the code objects that
+ * pass with hipModuleLoadData on `device`. A refused plugin is skipped and counted, as in the
+ * reference; no plugin at all is SABER_IU8_E_NOTLOADED. */
+int saber_iu8_open(const char *prebuilt_dir, int device, saber_iu8_ctx **out);
+void saber_iu8_close(saber_iu8_ctx *ctx);
+int saber_iu8_get_counters(const saber_iu8_ctx *ctx, saber_iu8_counters *out);
+/* 1 if `kernel` was loaded. */
+int saber_iu8_has_kernel(const saber_iu8_ctx *ctx, const char *kernel);
+
+/* Launcher::launch_op (crates/saber-exec/src/launch.rs:590-660): packs the kernarg image and
+ * calls hipModuleLaunchKernel(f, grid, block, 0, stream, NULL, extra) once. Buffers the
+ * descriptor names must all be bound (workspaces included when ks > 1). Asynchronous, capture-
+ * legal: no allocation, no synchronisation. */
+int saber_iu8_launch(saber_iu8_ctx *ctx, const saber_iu8_desc *desc, const saber_iu8_binding *bufs, uint32_t n_bufs,
+                     void *stream);
+
+/* ------------------------------------------------------------------ operators (resolve + launch) */
+
+/* Per-token int8 quantisation: x bf16 [m,k] -> q (A edge, saber_iu8_a_bytes) + scale f32 [m]. */
+int saber_iu8_quant(saber_iu8_ctx *ctx, const void *x_bf16, void *q, float *scale, uint32_t m, uint32_t k, void *stream);
+
+/* Workspace bytes the resolved GEMM needs (both 0 when it does not split). */
+int saber_iu8_gemm_workspace(int wkind, uint32_t m, uint32_t n, uint32_t k, uint64_t *partial_bytes,
+                             uint64_t *counter_bytes);
+
+/* C[m,n] bf16 = epilogue(A . W^T): a/as from the producer, w in the gfx950 fragment order, ws f32
+ * [n]. `partial` (scratch) and `counter` (zeroed once by the caller, left zero) may be NULL when
+ * saber_iu8_gemm_workspace reports 0. */
+int saber_iu8_gemm(saber_iu8_ctx *ctx, int wkind, const void *a, const float *as, const void *w, const float *ws,
+                   void *c_bf16, uint32_t m, uint32_t n, uint32_t k, void *partial, void *counter, void *stream);
+
+/* The raw int32 accumulators of the same GEMM (16 * sum(a*w) for W4, sum(a*w) for W8), int32
+ * [m,n]: the parity tap. No counterpart in the reference's shipped object (its tests replay
+ * captured bytes, crates/saber-kernels/hip/harness/run_hsaco.cpp:1-15). */
+int saber_iu8_gemm_acc(saber_iu8_ctx *ctx, int wkind, const void *a, const void *w, int32_t *acc, uint32_t m,
+                       uint32_t n, uint32_t k, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SABER_IU8_H */

@@ -1,0 +1,58 @@
+#include "abi.h"
+
+namespace iu8 {
+
+using K = ArgKind;
+
+static const Signature SIG_DEC = {{"a", K::Buffer},  {"w", K::Buffer},
+                                  {"as", K::Buffer}, {"ws", K::Buffer},
+                                  {"decode_partial", K::Buffer}, {"decode_counter", K::Buffer},
+                                  {"c", K::Buffer},  {"m", K::I32},
+                                  {"n", K::I32},     {"k", K::I32}};
+static const Signature SIG_PF = {{"a", K::Buffer}, {"w", K::Buffer}, {"as", K::Buffer}, {"ws", K::Buffer},
+                                 {"c", K::Buffer}, {"m", K::I32},    {"n", K::I32},     {"k", K::I32}};
+static const Signature SIG_QUANT = {{"x", K::Buffer}, {"q", K::Buffer}, {"scale", K::Buffer}, {"k", K::I32}};
+static const Signature SIG_SILU = {{"gu", K::Buffer}, {"q", K::Buffer},       {"scale", K::Buffer},
+                                   {"n", K::I32},     {"row_tok", K::Buffer}, {"meta", K::Buffer}};
+static const Signature SIG_TABLE = {{"out", K::Buffer}};
+static const Signature SIG_MOE_ROUTE = {
+    {"logits", K::Buffer},      {"t", K::I32},           {"e_lo", K::I32},        {"e_loc", K::I32},
+    {"tile_blocks", K::I32},    {"with_shared", K::I32}, {"topk_ids", K::Buffer}, {"topk_w", K::Buffer},
+    {"route_pos", K::Buffer},   {"row_tok", K::Buffer},  {"row_route", K::Buffer}, {"tile_expert", K::Buffer},
+    {"tile_row0", K::Buffer},   {"tile_rows", K::Buffer}, {"expert_cnt", K::Buffer}, {"meta", K::Buffer},
+    {"blk_cnt", K::Buffer},     {"rank", K::Buffer},     {"arrive", K::Buffer}};
+static const Signature SIG_MOE_GROUPED = {
+    {"a", K::Buffer},       {"xptr", K::Buffer}, {"tile_expert", K::Buffer}, {"tile_row0", K::Buffer},
+    {"tile_rows", K::Buffer}, {"row_tok", K::Buffer}, {"meta", K::Buffer},   {"as", K::Buffer},
+    {"p", K::Buffer},       {"cnt", K::Buffer},  {"c", K::Buffer},           {"n", K::I32},
+    {"k", K::I32},          {"pmax", K::I32}};
+static const Signature SIG_MOE_COMBINE = {{"y", K::Buffer},    {"topk_w", K::Buffer}, {"route_pos", K::Buffer},
+                                          {"sgate", K::Buffer}, {"meta", K::Buffer},  {"out", K::Buffer},
+                                          {"h", K::I32}};
+
+static bool starts(const std::string &s, const char *p) { return s.rfind(p, 0) == 0; }
+
+const Signature *signature_for(const std::string &k) {
+  if (starts(k, "macaq_iu8_dec_")) return &SIG_DEC;
+  if (starts(k, "macaq_iu8_pf_")) return &SIG_PF;
+  if (starts(k, "macaq_i8_quant_")) return &SIG_QUANT;
+  if (starts(k, "macaq_i8_silu_mul_quant_")) return &SIG_SILU;
+  if (k == "macaq_silu_bf16_table") return &SIG_TABLE;
+  if (starts(k, "moe_iu8_route_")) return &SIG_MOE_ROUTE;
+  if (starts(k, "moe_iu8_grouped_")) return &SIG_MOE_GROUPED;
+  if (starts(k, "moe_iu8_combine_")) return &SIG_MOE_COMBINE;
+  return nullptr;
+}
+
+uint32_t pack(const Signature &sig, std::vector<std::pair<uint32_t, uint32_t>> &out) {
+  out.clear();
+  uint32_t off = 0;
+  for (const SigArg &a : sig) {
+    off = (off + a.align() - 1) / a.align() * a.align();
+    out.emplace_back(off, a.size());
+    off += a.size();
+  }
+  return off;
+}
+
+}  // namespace iu8

@@ -1,0 +1,207 @@
+#include "rules.h"
+
+#include <cstring>
+
+#include "abi.h"
+#include "util.h"
+
+namespace iu8 {
+
+static const DecVariant DEC_VARIANTS[] = {
+#define IU8_DEC_VARIANT(name, TM, W8, NT, KW, WPB, U, ACC) {#name, TM, W8, NT, KW, WPB, U, ACC},
+#define IU8_PF_VARIANT(name, W8, WMW, WNW, TM, TN, ACC)
+#include "../kernels/iu8_variants.def"
+#undef IU8_DEC_VARIANT
+#undef IU8_PF_VARIANT
+};
+static const PfVariant PF_VARIANTS[] = {
+#define IU8_DEC_VARIANT(name, TM, W8, NT, KW, WPB, U, ACC)
+#define IU8_PF_VARIANT(name, W8, WMW, WNW, TM, TN, ACC) {#name, W8, WMW, WNW, TM, TN, ACC},
+#include "../kernels/iu8_variants.def"
+#undef IU8_DEC_VARIANT
+#undef IU8_PF_VARIANT
+};
+
+const DecVariant *dec_variant(const std::string &name) {
+  for (const DecVariant &v : DEC_VARIANTS)
+    if (name == v.name) return &v;
+  return nullptr;
+}
+const PfVariant *pf_variant(const std::string &name) {
+  for (const PfVariant &v : PF_VARIANTS)
+    if (name == v.name) return &v;
+  return nullptr;
+}
+
+static void copy_name(char *dst, size_t cap, const std::string &s) {
+  snprintf(dst, cap, "%s", s.c_str());
+}
+
+int fill_slots(const std::string &kernel, saber_iu8_desc *d) {
+  const Signature *sig = signature_for(kernel);
+  if (!sig) return fail(SABER_IU8_E_RULE, kernel + ": no declared signature");
+  std::vector<std::pair<uint32_t, uint32_t>> packed;
+  d->kernarg_bytes = pack(*sig, packed);
+  if (sig->size() > sizeof(d->args) / sizeof(d->args[0])) return fail(SABER_IU8_E_RULE, kernel + ": too many arguments");
+  d->n_args = (uint32_t)sig->size();
+  for (size_t i = 0; i < sig->size(); ++i) {
+    saber_iu8_slot &s = d->args[i];
+    memset(&s, 0, sizeof s);
+    copy_name(s.name, sizeof s.name, (*sig)[i].name);
+    s.offset = packed[i].first;
+    s.size = packed[i].second;
+    s.kind = (*sig)[i].kind == ArgKind::Buffer ? SABER_IU8_ARG_BUFFER
+             : (*sig)[i].kind == ArgKind::F32  ? SABER_IU8_ARG_F32
+                                               : SABER_IU8_ARG_I32;
+  }
+  return 0;
+}
+
+void set_i32(saber_iu8_desc *d, const char *name, int64_t v) {
+  for (uint32_t i = 0; i < d->n_args; ++i)
+    if (!strcmp(d->args[i].name, name)) {
+      d->args[i].kind = SABER_IU8_ARG_I32;
+      d->args[i].ival = v;
+    }
+}
+void set_null(saber_iu8_desc *d, const char *name) {
+  for (uint32_t i = 0; i < d->n_args; ++i)
+    if (!strcmp(d->args[i].name, name)) d->args[i].kind = SABER_IU8_ARG_NULL_BUFFER;
+}
+
+static void add_ws(saber_iu8_desc *d, const char *name, uint32_t kind, uint64_t bytes, uint32_t zero_once) {
+  saber_iu8_workspace &w = d->workspaces[d->n_workspaces++];
+  memset(&w, 0, sizeof w);
+  copy_name(w.name, sizeof w.name, name);
+  w.kind = kind;
+  w.bytes = bytes;
+  w.zero_once = zero_once;
+}
+
+static int check_shape(const char *op, uint32_t m, uint32_t n, uint32_t k) {
+  // the reference's refusals (macaq_iu8.rs:288-297), by name
+  if (m == 0 || n == 0 || k == 0)
+    return fail(SABER_IU8_E_RULE, fmt("%s: %u x %u x %u has nothing to do; an empty launch is a caller bug", op, m, n, k));
+  if (n % 16 != 0 || k % 128 != 0)
+    return fail(SABER_IU8_E_RULE,
+                fmt("%s: N=%u must be a multiple of 16 (whole fragments) and K=%u of 128 (the slab)", op, n, k));
+  return 0;
+}
+
+// Double the split until the grid reaches two workgroups a CU, each k-wave keeps >= 2 steps, and
+// the partials stay small next to the weights (they are written and re-read once).
+uint32_t decode_split(uint32_t m, uint32_t n, uint32_t k, uint32_t nblk, uint32_t kw) {
+  const uint32_t steps = k / 128;
+  uint32_t ks = 1;
+  while (nblk * ks < 2 * CU_COUNT && ks < KS_MAX && steps / (ks * 2 * kw) >= 2 &&
+         (uint64_t)(ks * 2) * m * n * 4 * 8 <= (uint64_t)n * k / 2)
+    ks *= 2;
+  return ks;
+}
+
+static int describe_dec(const DecVariant &v, uint32_t m, uint32_t n, uint32_t k, uint32_t ks, saber_iu8_desc *d) {
+  const char *op = v.w8 ? "gemm_i8a8" : "gemm_i4a8";
+  if (int rc = check_shape(op, m, n, k)) return rc;
+  if (m > (uint32_t)v.tm * 16) return fail(SABER_IU8_E_RULE, fmt("%s: %s holds %d rows, M=%u", op, v.name, v.tm * 16, m));
+  if (ks == 0 || ks > k / 128) return fail(SABER_IU8_E_RULE, fmt("%s: split %u of %u K steps", op, ks, k / 128));
+  memset(d, 0, sizeof *d);
+  copy_name(d->op, sizeof d->op, op);
+  copy_name(d->plugin, sizeof d->plugin, "macaq_iu8");
+  copy_name(d->kernel, sizeof d->kernel, v.name);
+  const uint32_t nblk = (n + v.block_n() - 1) / v.block_n();
+  d->grid[0] = nblk, d->grid[1] = 1, d->grid[2] = ks;
+  d->block[0] = v.threads(), d->block[1] = 1, d->block[2] = 1;
+  d->n_launches = 1;
+  d->ks = ks;
+  if (int rc = fill_slots(v.name, d)) return rc;
+  set_i32(d, "m", m);
+  set_i32(d, "n", n);
+  set_i32(d, "k", k);
+  if (ks == 1) {
+    // named-null at ks 1: the kernel must not dereference them (macaq_iu8.rs:447-451)
+    set_null(d, "decode_partial");
+    set_null(d, "decode_counter");
+  } else {
+    add_ws(d, "decode_partial", SABER_IU8_WS_SCRATCH, (uint64_t)ks * m * n * 4, 0);
+    add_ws(d, "decode_counter", SABER_IU8_WS_PERSISTENT, (uint64_t)nblk * 4, 1);
+  }
+  return 0;
+}
+
+static int describe_pf(const PfVariant &v, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *d) {
+  const char *op = v.w8 ? "gemm_i8a8" : "gemm_i4a8";
+  if (int rc = check_shape(op, m, n, k)) return rc;
+  memset(d, 0, sizeof *d);
+  copy_name(d->op, sizeof d->op, op);
+  copy_name(d->plugin, sizeof d->plugin, "macaq_iu8");
+  copy_name(d->kernel, sizeof d->kernel, v.name);
+  d->grid[0] = (n + v.block_n() - 1) / v.block_n();
+  d->grid[1] = (m + v.block_m() - 1) / v.block_m();
+  d->grid[2] = 1;
+  d->block[0] = v.threads(), d->block[1] = 1, d->block[2] = 1;
+  d->n_launches = 1;
+  d->ks = 1;
+  if (int rc = fill_slots(v.name, d)) return rc;
+  set_i32(d, "m", m);
+  set_i32(d, "n", n);
+  set_i32(d, "k", k);
+  return 0;
+}
+
+int describe(const std::string &kernel, uint32_t m, uint32_t n, uint32_t k, uint32_t ks, saber_iu8_desc *out) {
+  if (const DecVariant *v = dec_variant(kernel)) return describe_dec(*v, m, n, k, ks, out);
+  if (const PfVariant *v = pf_variant(kernel)) {
+    if (ks != 1) return fail(SABER_IU8_E_RULE, kernel + ": the prefill tile does not split K");
+    return describe_pf(*v, m, n, k, out);
+  }
+  return fail(SABER_IU8_E_RULE, kernel + ": not a kernel of the macaq_iu8 object");
+}
+
+int resolve(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *out) {
+  if (wkind != SABER_IU8_W4 && wkind != SABER_IU8_W8) return fail(SABER_IU8_E_ARG, "unknown weight kind");
+  const char *tag = wkind == SABER_IU8_W8 ? "w8" : "w4";
+  if (int rc = check_shape(wkind == SABER_IU8_W8 ? "gemm_i8a8" : "gemm_i4a8", m, n, k)) return rc;
+  if (m <= DECODE_MAX_M) {
+    const uint32_t tm = (m + 15) / 16;
+    const std::string name = fmt("macaq_iu8_dec_%s_tm%u", tag, tm);
+    const DecVariant *v = dec_variant(name);
+    if (!v) return fail(SABER_IU8_E_RULE, name + ": no such variant");
+    const uint32_t nblk = (n + v->block_n() - 1) / v->block_n();
+    return describe_dec(*v, m, n, k, decode_split(m, n, k, nblk, v->kw), out);
+  }
+  // prefill: the 256 x 256 tile once it fills the card, the 128 x 128 tile below
+  const uint64_t big = (uint64_t)((m + 255) / 256) * ((n + 255) / 256);
+  const std::string name =
+      big >= CU_COUNT ? fmt("macaq_iu8_pf_%s_tn4_lbk64", tag) : fmt("macaq_iu8_pf_%s_t4x4w2x2", tag);
+  const PfVariant *v = pf_variant(name);
+  if (!v) return fail(SABER_IU8_E_RULE, name + ": no such variant");
+  return describe_pf(*v, m, n, k, out);
+}
+
+static int describe_rows(const char *op, const char *kernel, uint32_t rows, uint32_t width, const char *wname,
+                         saber_iu8_desc *d) {
+  if (rows == 0 || width == 0) return fail(SABER_IU8_E_RULE, fmt("%s: %u rows of %u has nothing to do", op, rows, width));
+  if (width % 64 != 0 || width > 32768)
+    return fail(SABER_IU8_E_RULE, fmt("%s: row width %u must be a multiple of 64 (whole A fragments), at most 32768", op, width));
+  memset(d, 0, sizeof *d);
+  copy_name(d->op, sizeof d->op, op);
+  copy_name(d->plugin, sizeof d->plugin, "macaq_i8q");
+  copy_name(d->kernel, sizeof d->kernel, kernel);
+  d->grid[0] = rows, d->grid[1] = 1, d->grid[2] = 1;
+  d->block[0] = 256, d->block[1] = 1, d->block[2] = 1;
+  d->n_launches = 1;
+  d->ks = 1;
+  if (int rc = fill_slots(kernel, d)) return rc;
+  set_i32(d, wname, width);
+  return 0;
+}
+
+int resolve_quant(uint32_t m, uint32_t k, saber_iu8_desc *out) {
+  return describe_rows("quant_i8", "macaq_i8_quant_t256", m, k, "k", out);
+}
+
+int resolve_silu_mul_quant(uint32_t rows, uint32_t n, saber_iu8_desc *out) {
+  return describe_rows("silu_mul_quant_i8", "macaq_i8_silu_mul_quant_t256", rows, n, "n", out);
+}
+
+}  // namespace iu8

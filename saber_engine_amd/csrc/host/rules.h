@@ -1,0 +1,46 @@
+// The gfx950 launch law of the iu8 path: which kernel, grid, block, split and workspaces a
+// GEMM of m x n x k runs. The counterpart of crates/saber-kernels/src/macaq_iu8.rs
+// (cell :286-358, decode_split :267-279, describe :429-489); the tables are this object's own
+// speed data (256 CUs in 8 XCDs instead of the reference's 64-CU card).
+#pragma once
+#include <string>
+
+#include "../../../include/saber_iu8.h"
+
+namespace iu8 {
+
+struct DecVariant {
+  const char *name;
+  int tm, w8, nt, kw, wpb, u, acc;
+  int block_n() const { return wpb / kw * nt * 16; }
+  int threads() const { return wpb * 64; }
+};
+struct PfVariant {
+  const char *name;
+  int w8, wmw, wnw, tm, tn, acc;
+  int block_m() const { return wmw * tm * 16; }
+  int block_n() const { return wnw * tn * 16; }
+  int threads() const { return wmw * wnw * 64; }
+};
+
+const DecVariant *dec_variant(const std::string &name);
+const PfVariant *pf_variant(const std::string &name);
+
+constexpr uint32_t DECODE_MAX_M = 64;  // the decode band's last row count (macaq_iu8.rs:31)
+constexpr uint32_t KS_MAX = 8;         // the largest grid-level split (macaq_iu8.rs:44)
+constexpr uint32_t CU_COUNT = 256;     // MI355X compute units
+
+// Grid-level split of a decode GEMM whose grid has `nblk` column blocks.
+uint32_t decode_split(uint32_t m, uint32_t n, uint32_t k, uint32_t nblk, uint32_t kw);
+
+int resolve(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *out);
+int describe(const std::string &kernel, uint32_t m, uint32_t n, uint32_t k, uint32_t ks, saber_iu8_desc *out);
+int resolve_quant(uint32_t m, uint32_t k, saber_iu8_desc *out);
+int resolve_silu_mul_quant(uint32_t rows, uint32_t n, saber_iu8_desc *out);
+
+// Fills name/offset/size of every slot from the kernel's signature; kinds default to BUFFER.
+int fill_slots(const std::string &kernel, saber_iu8_desc *d);
+void set_i32(saber_iu8_desc *d, const char *name, int64_t v);
+void set_null(saber_iu8_desc *d, const char *name);
+
+}  // namespace iu8

@@ -1,0 +1,328 @@
+// Loader, launcher and the operator-level entry points: the counterpart of
+// crates/saber-exec/src/loader.rs (PluginSet::load_dir, :318-396), crates/saber-exec/src/launch.rs
+// (pack_kernarg :123, Launcher::launch_op :590-660) and the HIP calls of crates/saber-hip
+// (hipModuleLoadData / hipModuleGetFunction / hipModuleLaunchKernel with a packed-kernarg
+// `extra`, src/ffi.rs:917-995).
+#include <dirent.h>
+#include <hip/hip_runtime_api.h>
+
+#include <algorithm>
+#include <cstring>
+#include <map>
+
+#include "../../../include/saber_iu8.h"
+#include "abi.h"
+#include "manifest.h"
+#include "rules.h"
+#include "util.h"
+
+using namespace iu8;
+
+struct saber_iu8_ctx {
+  int device = 0;
+  std::vector<hipModule_t> modules;
+  std::map<std::string, hipFunction_t> fn;
+  saber_iu8_counters counters{};
+};
+
+static int hip_fail(const char *what, hipError_t e) {
+  return fail(SABER_IU8_E_HIP, fmt("%s: HIP status %d (%s)", what, (int)e, hipGetErrorString(e)));
+}
+
+// Runs the loader's validations on one manifest; fills manifest, blob; names the refusal.
+static int load_and_validate(const std::string &manifest_path, const std::string &arch, Manifest &m,
+                             std::vector<uint8_t> &blob, int *refusal) {
+  if (refusal) *refusal = 0;
+  std::vector<uint8_t> text;
+  if (!read_file(manifest_path, text)) return fail(SABER_IU8_E_IO, manifest_path + ": cannot read");
+  std::string why;
+  if (!manifest_parse_toml(std::string(text.begin(), text.end()), m, &why)) return fail(SABER_IU8_E_PARSE, manifest_path + ": " + why);
+  if (!check_kernarg_layout(m, &why)) {
+    if (refusal) *refusal = SABER_IU8_REFUSED_KERNARG;
+    return fail(SABER_IU8_E_VALIDATE, "refused (kernarg): " + why);
+  }
+  const size_t slash = manifest_path.find_last_of('/');
+  const std::string dir = slash == std::string::npos ? "." : manifest_path.substr(0, slash);
+  if (!read_file(dir + "/" + m.hsaco, blob)) return fail(SABER_IU8_E_IO, dir + "/" + m.hsaco + ": cannot read");
+  CodeObject co;
+  if (!parse_code_object(blob, co, &why)) return fail(SABER_IU8_E_PARSE, m.hsaco + ": " + why);
+  if (!check_wave_size(m, &why)) {
+    if (refusal) *refusal = SABER_IU8_REFUSED_WAVE;
+    return fail(SABER_IU8_E_VALIDATE, "refused (wave): " + why);
+  }
+  if (!validate_against_hsaco(m, blob, co, arch, &why)) {
+    if (refusal) *refusal = SABER_IU8_REFUSED_METADATA;
+    return fail(SABER_IU8_E_VALIDATE, "refused (metadata): " + why);
+  }
+  return 0;
+}
+
+static const void *find_binding(const saber_iu8_binding *bufs, uint32_t n, const char *name, bool *found) {
+  for (uint32_t i = 0; i < n; ++i)
+    if (bufs[i].name && !strcmp(bufs[i].name, name)) {
+      *found = true;
+      return bufs[i].ptr;
+    }
+  *found = false;
+  return nullptr;
+}
+
+extern "C" {
+
+const char *saber_iu8_last_error(void) { return last_error(); }
+int saber_iu8_abi_version(void) { return SABER_IU8_ABI_VERSION; }
+
+int saber_iu8_resolve(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *out) {
+  if (!out) return fail(SABER_IU8_E_ARG, "resolve: null descriptor");
+  return resolve(wkind, m, n, k, out);
+}
+int saber_iu8_describe(const char *kernel, uint32_t m, uint32_t n, uint32_t k, uint32_t ks, saber_iu8_desc *out) {
+  if (!out || !kernel) return fail(SABER_IU8_E_ARG, "describe: null argument");
+  return describe(kernel, m, n, k, ks, out);
+}
+int saber_iu8_resolve_quant(uint32_t m, uint32_t k, saber_iu8_desc *out) {
+  if (!out) return fail(SABER_IU8_E_ARG, "resolve_quant: null descriptor");
+  return resolve_quant(m, k, out);
+}
+int saber_iu8_resolve_silu_mul_quant(uint32_t rows, uint32_t n, saber_iu8_desc *out) {
+  if (!out) return fail(SABER_IU8_E_ARG, "resolve_silu_mul_quant: null descriptor");
+  return resolve_silu_mul_quant(rows, n, out);
+}
+
+int saber_iu8_signature(const char *kernel, saber_iu8_slot *slots, uint32_t cap, uint32_t *n_slots, uint32_t *bytes) {
+  if (!kernel || !slots || !n_slots || !bytes) return fail(SABER_IU8_E_ARG, "signature: null argument");
+  saber_iu8_desc d;
+  memset(&d, 0, sizeof d);
+  if (int rc = fill_slots(kernel, &d)) return rc;
+  if (d.n_args > cap) return fail(SABER_IU8_E_ARG, "signature: slot array too small");
+  memcpy(slots, d.args, sizeof(saber_iu8_slot) * d.n_args);
+  *n_slots = d.n_args;
+  *bytes = d.kernarg_bytes;
+  return 0;
+}
+
+int saber_iu8_pack_kernarg(const saber_iu8_desc *d, const saber_iu8_binding *bufs, uint32_t n_bufs, uint8_t *image,
+                           uint32_t cap, uint32_t *bytes) {
+  if (!d || !image || (!bufs && n_bufs)) return fail(SABER_IU8_E_ARG, "pack_kernarg: null argument");
+  if (cap < d->kernarg_bytes) return fail(SABER_IU8_E_ARG, fmt("pack_kernarg: image of %u B, the kernel takes %u", cap, d->kernarg_bytes));
+  memset(image, 0, d->kernarg_bytes);  // padding is zero-filled (launch.rs:120-122)
+  for (uint32_t i = 0; i < d->n_args; ++i) {
+    const saber_iu8_slot &s = d->args[i];
+    if (s.offset + s.size > d->kernarg_bytes) return fail(SABER_IU8_E_ARG, fmt("%s: slot `%s` past the kernarg block", d->kernel, s.name));
+    switch (s.kind) {
+      case SABER_IU8_ARG_BUFFER: {
+        bool found;
+        const void *p = find_binding(bufs, n_bufs, s.name, &found);
+        if (!found) return fail(SABER_IU8_E_ARG, fmt("%s: buffer `%s` is not bound", d->kernel, s.name));
+        if (!p) return fail(SABER_IU8_E_ARG, fmt("%s: buffer `%s` is bound to NULL", d->kernel, s.name));
+        memcpy(image + s.offset, &p, 8);
+        break;
+      }
+      case SABER_IU8_ARG_NULL_BUFFER:
+        break;
+      case SABER_IU8_ARG_I32: {
+        const int32_t v = (int32_t)s.ival;
+        memcpy(image + s.offset, &v, 4);
+        break;
+      }
+      case SABER_IU8_ARG_F32:
+        memcpy(image + s.offset, &s.fval, 4);
+        break;
+      default:
+        return fail(SABER_IU8_E_ARG, fmt("%s: slot `%s` has unknown kind %u", d->kernel, s.name, s.kind));
+    }
+  }
+  if (bytes) *bytes = d->kernarg_bytes;
+  return 0;
+}
+
+int saber_iu8_sha256_file(const char *path, char *out65) {
+  if (!path || !out65) return fail(SABER_IU8_E_ARG, "sha256_file: null argument");
+  std::vector<uint8_t> b;
+  if (!read_file(path, b)) return fail(SABER_IU8_E_IO, std::string(path) + ": cannot read");
+  snprintf(out65, 65, "%s", sha256_hex(b.data(), b.size()).c_str());
+  return 0;
+}
+
+int saber_iu8_manifest_write(const char *hsaco_path, const char *plugin, const char *arch, const char *source,
+                             const char *source_sha256, const char *flags, const char *build_hash, const char *out_path) {
+  if (!hsaco_path || !plugin || !arch || !source || !source_sha256 || !flags || !build_hash || !out_path)
+    return fail(SABER_IU8_E_ARG, "manifest_write: null argument");
+  std::vector<uint8_t> blob;
+  if (!read_file(hsaco_path, blob)) return fail(SABER_IU8_E_IO, std::string(hsaco_path) + ": cannot read");
+  CodeObject co;
+  std::string why;
+  if (!parse_code_object(blob, co, &why)) return fail(SABER_IU8_E_PARSE, std::string(hsaco_path) + ": " + why);
+  if (co.target.find(arch) == std::string::npos)
+    return fail(SABER_IU8_E_VALIDATE, "code object target " + co.target + " is not " + arch);
+  const std::string hp(hsaco_path);
+  const size_t slash = hp.find_last_of('/');
+  Manifest m = manifest_from_code_object(co, plugin, arch, source, source_sha256, flags, build_hash,
+                                         slash == std::string::npos ? hp : hp.substr(slash + 1),
+                                         sha256_hex(blob.data(), blob.size()));
+  // Name the arguments from the declared signatures (the code object has offsets but no names) and
+  // refuse a kernel that has no signature or does not pack the way it does (manifest.rs:170-207).
+  std::sort(m.kernel.begin(), m.kernel.end(), [](const KernelDecl &x, const KernelDecl &y) { return x.name < y.name; });
+  for (KernelDecl &k : m.kernel) {
+    const Signature *sig = signature_for(k.name);
+    if (!sig) return fail(SABER_IU8_E_VALIDATE, k.name + ": no declared signature for this symbol");
+    if (sig->size() != k.arg.size())
+      return fail(SABER_IU8_E_VALIDATE, fmt("%s: signature has %zu args, code object %zu", k.name.c_str(), sig->size(), k.arg.size()));
+    for (size_t i = 0; i < sig->size(); ++i) k.arg[i].name = (*sig)[i].name;
+  }
+  if (!check_kernarg_layout(m, &why)) return fail(SABER_IU8_E_VALIDATE, why);
+  if (!write_file(out_path, manifest_to_toml(m))) return fail(SABER_IU8_E_IO, std::string(out_path) + ": cannot write");
+  return 0;
+}
+
+int saber_iu8_manifest_validate(const char *manifest_path, const char *arch, int *refusal) {
+  if (!manifest_path) return fail(SABER_IU8_E_ARG, "manifest_validate: null path");
+  Manifest m;
+  std::vector<uint8_t> blob;
+  return load_and_validate(manifest_path, arch ? arch : "", m, blob, refusal);
+}
+
+int saber_iu8_open(const char *prebuilt_dir, int device, saber_iu8_ctx **out) {
+  if (!prebuilt_dir || !out) return fail(SABER_IU8_E_ARG, "open: null argument");
+  *out = nullptr;
+  int ndev = 0;
+  hipError_t e = hipGetDeviceCount(&ndev);
+  if (e != hipSuccess || ndev <= 0) return hip_fail("hipGetDeviceCount (no GPU visible: this path has no CPU fallback)", e);
+  if ((e = hipSetDevice(device)) != hipSuccess) return hip_fail("hipSetDevice", e);
+  hipDeviceProp_t prop;
+  if ((e = hipGetDeviceProperties(&prop, device)) != hipSuccess) return hip_fail("hipGetDeviceProperties", e);
+  std::string arch(prop.gcnArchName);
+  arch = arch.substr(0, arch.find(':'));
+  DIR *dp = opendir(prebuilt_dir);
+  if (!dp) return fail(SABER_IU8_E_IO, std::string(prebuilt_dir) + ": cannot open directory");
+  std::vector<std::string> manifests;
+  while (dirent *de = readdir(dp)) {
+    const std::string f = de->d_name;
+    const std::string suf = ".manifest.toml";
+    if (f.size() > suf.size() && f.compare(f.size() - suf.size(), suf.size(), suf) == 0) manifests.push_back(f);
+  }
+  closedir(dp);
+  std::sort(manifests.begin(), manifests.end());
+  saber_iu8_ctx *ctx = new saber_iu8_ctx();
+  ctx->device = device;
+  std::string first_refusal;
+  for (const std::string &f : manifests) {
+    Manifest m;
+    std::vector<uint8_t> blob;
+    int refusal = 0;
+    const int rc = load_and_validate(std::string(prebuilt_dir) + "/" + f, arch, m, blob, &refusal);
+    if (rc != 0) {
+      if (refusal == SABER_IU8_REFUSED_KERNARG) ctx->counters.refused_kernarg++;
+      else if (refusal == SABER_IU8_REFUSED_WAVE) ctx->counters.refused_wave++;
+      else ctx->counters.refused_metadata++;
+      if (first_refusal.empty()) first_refusal = f + ": " + last_error();
+      continue;
+    }
+    hipModule_t mod;
+    if ((e = hipModuleLoadData(&mod, blob.data())) != hipSuccess) {
+      saber_iu8_close(ctx);
+      return hip_fail(("hipModuleLoadData " + m.hsaco).c_str(), e);
+    }
+    ctx->modules.push_back(mod);
+    ctx->counters.plugins_loaded++;
+    for (const KernelDecl &k : m.kernel) {
+      hipFunction_t fn;
+      if ((e = hipModuleGetFunction(&fn, mod, k.name.c_str())) != hipSuccess) {
+        saber_iu8_close(ctx);
+        return hip_fail(("hipModuleGetFunction " + k.name).c_str(), e);
+      }
+      ctx->fn[k.name] = fn;
+      ctx->counters.kernels_loaded++;
+    }
+  }
+  if (ctx->modules.empty()) {
+    const std::string msg = std::string(prebuilt_dir) + ": no plugin loaded for " + arch +
+                            (first_refusal.empty() ? " (no *.manifest.toml)" : " (" + first_refusal + ")");
+    saber_iu8_close(ctx);
+    return fail(SABER_IU8_E_NOTLOADED, msg);
+  }
+  *out = ctx;
+  return 0;
+}
+
+void saber_iu8_close(saber_iu8_ctx *ctx) {
+  if (!ctx) return;
+  for (hipModule_t m : ctx->modules) (void)hipModuleUnload(m);
+  delete ctx;
+}
+
+int saber_iu8_get_counters(const saber_iu8_ctx *ctx, saber_iu8_counters *out) {
+  if (!ctx || !out) return fail(SABER_IU8_E_ARG, "get_counters: null argument");
+  *out = ctx->counters;
+  return 0;
+}
+
+int saber_iu8_has_kernel(const saber_iu8_ctx *ctx, const char *kernel) {
+  return ctx && kernel && ctx->fn.count(kernel) ? 1 : 0;
+}
+
+int saber_iu8_launch(saber_iu8_ctx *ctx, const saber_iu8_desc *d, const saber_iu8_binding *bufs, uint32_t n_bufs,
+                     void *stream) {
+  if (!ctx || !d) return fail(SABER_IU8_E_ARG, "launch: null argument");
+  auto it = ctx->fn.find(d->kernel);
+  if (it == ctx->fn.end()) return fail(SABER_IU8_E_NOTLOADED, std::string(d->kernel) + ": not in the loaded plugin set");
+  if (d->shared_bytes != 0) return fail(SABER_IU8_E_RULE, std::string(d->kernel) + ": dynamic LDS is not part of this ABI");
+  if (!d->grid[0] || !d->grid[1] || !d->grid[2] || !d->block[0]) return fail(SABER_IU8_E_RULE, std::string(d->kernel) + ": empty grid");
+  alignas(16) uint8_t image[256];
+  uint32_t bytes = 0;
+  if (int rc = saber_iu8_pack_kernarg(d, bufs, n_bufs, image, sizeof image, &bytes)) return rc;
+  size_t sz = bytes;
+  void *extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, image, HIP_LAUNCH_PARAM_BUFFER_SIZE, &sz, HIP_LAUNCH_PARAM_END};
+  const hipError_t e = hipModuleLaunchKernel(it->second, d->grid[0], d->grid[1], d->grid[2], d->block[0], d->block[1],
+                                             d->block[2], 0, (hipStream_t)stream, nullptr, extra);
+  if (e != hipSuccess) return hip_fail(d->kernel, e);
+  ctx->counters.launches++;
+  return 0;
+}
+
+int saber_iu8_quant(saber_iu8_ctx *ctx, const void *x, void *q, float *scale, uint32_t m, uint32_t k, void *stream) {
+  saber_iu8_desc d;
+  if (int rc = resolve_quant(m, k, &d)) return rc;
+  const saber_iu8_binding b[] = {{"x", (void *)x}, {"q", q}, {"scale", scale}};
+  return saber_iu8_launch(ctx, &d, b, 3, stream);
+}
+
+int saber_iu8_gemm_workspace(int wkind, uint32_t m, uint32_t n, uint32_t k, uint64_t *partial_bytes, uint64_t *counter_bytes) {
+  saber_iu8_desc d;
+  if (int rc = resolve(wkind, m, n, k, &d)) return rc;
+  uint64_t p = 0, c = 0;
+  for (uint32_t i = 0; i < d.n_workspaces; ++i) {
+    if (!strcmp(d.workspaces[i].name, "decode_partial")) p = d.workspaces[i].bytes;
+    if (!strcmp(d.workspaces[i].name, "decode_counter")) c = d.workspaces[i].bytes;
+  }
+  if (partial_bytes) *partial_bytes = p;
+  if (counter_bytes) *counter_bytes = c;
+  return 0;
+}
+
+static int launch_gemm(saber_iu8_ctx *ctx, const saber_iu8_desc &d, const void *a, const float *as, const void *w,
+                       const float *ws, void *c, void *partial, void *counter, void *stream) {
+  const saber_iu8_binding b[] = {{"a", (void *)a},   {"w", (void *)w},           {"as", (void *)as},         {"ws", (void *)ws},
+                                 {"c", c},           {"decode_partial", partial}, {"decode_counter", counter}};
+  return saber_iu8_launch(ctx, &d, b, 7, stream);
+}
+
+int saber_iu8_gemm(saber_iu8_ctx *ctx, int wkind, const void *a, const float *as, const void *w, const float *ws,
+                   void *c, uint32_t m, uint32_t n, uint32_t k, void *partial, void *counter, void *stream) {
+  saber_iu8_desc d;
+  if (int rc = resolve(wkind, m, n, k, &d)) return rc;
+  return launch_gemm(ctx, d, a, as, w, ws, c, partial, counter, stream);
+}
+
+int saber_iu8_gemm_acc(saber_iu8_ctx *ctx, int wkind, const void *a, const void *w, int32_t *acc, uint32_t m, uint32_t n,
+                       uint32_t k, void *stream) {
+  if (wkind != SABER_IU8_W4 && wkind != SABER_IU8_W8) return fail(SABER_IU8_E_ARG, "unknown weight kind");
+  const char *tag = wkind == SABER_IU8_W8 ? "w8" : "w4";
+  saber_iu8_desc d;
+  const std::string name = m <= 16 ? fmt("macaq_iu8_dec_%s_tm1_acc", tag) : fmt("macaq_iu8_pf_%s_acc", tag);
+  if (int rc = describe(name, m, n, k, 1, &d)) return rc;
+  // the taps read no scales; bind the accumulator buffer where a pointer is required
+  return launch_gemm(ctx, d, a, (const float *)acc, w, (const float *)acc, acc, nullptr, nullptr, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,74 @@
+// Shared device helpers of the gfx950 W4A8-iu8 kernels: operand orders, the int8 MFMA,
+// the nibble unpack, bf16 rounding and the epilogue contract.
+//
+// OPERAND ORDERS (gfx950 device-final; a wave64 lane reads 16 bytes = one MFMA operand).
+//   A   int8 activations, rows padded to 16. Fragment (mt, kt) = 1024 B at
+//       (mt * K/64 + kt) * 1024; lane l's 16 bytes at l*16 = row mt*16 + l%16,
+//       k = kt*64 + (l/16)*16 + 0..15. Rows past M are never stored from.
+//   W4  int4 [-8,7] two's-complement nibbles. Fragment (nt, kt) = 1024 B at
+//       (nt * K/128 + kt) * 1024; lane l's 4 dwords d0..d3 at l*16 belong to row
+//       nt*16 + l%16; dword j, byte b: low nibble = k0 + b, high nibble = k0 + 4 + b with
+//       k0 = kt*128 + (j/2)*64 + (l/16)*16 + (j%2)*8. Unpacked to the exact int8 16*w
+//       (lo = (d << 4) & 0xF0F0F0F0, hi = d & 0xF0F0F0F0), so {lo(d0),hi(d0),lo(d1),hi(d1)}
+//       is the operand of k-step 2*kt and {lo(d2),hi(d2),lo(d3),hi(d3)} of 2*kt+1, both in
+//       natural k order, and the int32 accumulator holds 16 * sum(a*w).
+//   W8  int8 [-127,127]: the A order by rows of W (fragment (nt, kt) of 16 rows x 64 k).
+// The reference's gfx12 orders (crates/saber-kernels/hip/macaq_iu8.hip:8-18) are wave32 WMMA
+// fragment orders; these are their wave64 MFMA counterparts and keep the same sizes.
+//
+// THE CONTRACT (crates/saber-kernels/hip/macaq_iu8.hip:20-24): acc = exact int32 sum over all
+// of K; y = bf16_rne((f32(acc) * as[m]) * (ws[n] * U)), U = 1/16 for W4 and 1 for W8, each `*`
+// one IEEE f32 multiply. Every translation unit including this header is compiled with
+// -ffp-contract=off.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef int iu8_v4i __attribute__((ext_vector_type(4)));
+typedef unsigned iu8_v4u __attribute__((ext_vector_type(4)));
+typedef unsigned iu8_v2u __attribute__((ext_vector_type(2)));
+typedef unsigned char iu8_u8;
+
+// D[n][m] += sum_k W[n][k] * A[m][k] over 64 k: src0 = weight operand (lane: row n = l%16),
+// src1 = activation operand (lane: row m = l%16); D lane l holds n = 4*(l/16) + 0..3, m = l%16.
+static __device__ __forceinline__ iu8_v4i iu8_mfma(iu8_v4i w, iu8_v4i a, iu8_v4i c) {
+  return __builtin_amdgcn_mfma_i32_16x16x64_i8(w, a, c, 0, 0, 0);
+}
+
+// 16 B of a W4 fragment -> the two k-step operands (int8 = 16 * code).
+static __device__ __forceinline__ void iu8_unpack_w4(iu8_v4u d, iu8_v4i &s0, iu8_v4i &s1) {
+  s0 = iu8_v4i{(int)((d.x << 4) & 0xF0F0F0F0u), (int)(d.x & 0xF0F0F0F0u), (int)((d.y << 4) & 0xF0F0F0F0u),
+               (int)(d.y & 0xF0F0F0F0u)};
+  s1 = iu8_v4i{(int)((d.z << 4) & 0xF0F0F0F0u), (int)(d.z & 0xF0F0F0F0u), (int)((d.w << 4) & 0xF0F0F0F0u),
+               (int)(d.w & 0xF0F0F0F0u)};
+}
+
+// f32 -> bf16 bits, round to nearest even (finite inputs; NaN stays a quiet NaN).
+static __device__ __forceinline__ unsigned iu8_bf16_bits(float x) {
+  const unsigned u = __float_as_uint(x);
+  if (x != x) return (u >> 16) | 0x40u;
+  return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
+}
+static __device__ __forceinline__ float iu8_bf16_f32(unsigned short b) { return __uint_as_float((unsigned)b << 16); }
+
+template <bool W8>
+static __device__ __forceinline__ float iu8_wsu(const float *__restrict__ ws, int n) {
+#pragma clang fp contract(off)
+  return W8 ? ws[n] : ws[n] * 0.0625f;
+}
+static __device__ __forceinline__ float iu8_epi(int acc, float a_scale, float w_scale_u) {
+#pragma clang fp contract(off)
+  const float t = (float)acc * a_scale;
+  return t * w_scale_u;
+}
+
+// The per-token int8 code (crates/saber-kernels/hip/macaq_i8.h:10-13): IEEE divide, clamp,
+// round half to even.
+static __device__ __forceinline__ unsigned iu8_code(float x, float sc) {
+  const float y = fminf(fmaxf(__fdiv_rn(x, sc), -127.f), 127.f);
+  return ((unsigned)(int)__builtin_rintf(y)) & 0xffu;
+}
+
+static __device__ __forceinline__ iu8_v4u iu8_ldg_nt(const iu8_u8 *p) {
+  return __builtin_nontemporal_load((const iu8_v4u *)p);
+}

@@ -1,0 +1,261 @@
+"""Python binding of the C ABI in include/saber_iu8.h (ctypes; no compute happens here).
+
+The names mirror the reference's host interface for this path: `resolve(WKind, m, n, k)`
+(crates/saber-kernels/src/macaq_iu8.rs:425), `PluginSet.load_dir` (crates/saber-exec/src/
+loader.rs:318), `Launcher.launch_op` (crates/saber-exec/src/launch.rs:590).  Device memory and
+streams are the caller's (torch tensors' data_ptr() / torch.cuda streams in the tests).
+
+The library has no CPU fallback: opening a context without a GPU, or before the code objects
+were built, raises.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+PKG = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(PKG)
+LIB_PATH = os.path.join(PKG, "libsaber_iu8.so")
+PREBUILT = os.path.join(ROOT, "prebuilt", "gfx950")
+
+W4, W8 = 0, 1
+ARG_BUFFER, ARG_NULL_BUFFER, ARG_I32, ARG_F32 = 0, 1, 2, 3
+WS_SCRATCH, WS_PERSISTENT = 0, 1
+E_RULE, E_PARSE, E_VALIDATE, E_HIP, E_ARG, E_IO, E_NOTLOADED = -1, -2, -3, -4, -5, -6, -7
+REFUSED_KERNARG, REFUSED_WAVE, REFUSED_METADATA = 1, 2, 3
+
+
+class Slot(C.Structure):
+    _fields_ = [("name", C.c_char * 24), ("offset", C.c_uint32), ("size", C.c_uint32), ("kind", C.c_uint32),
+                ("ival", C.c_int64), ("fval", C.c_float)]
+
+
+class Workspace(C.Structure):
+    _fields_ = [("name", C.c_char * 24), ("kind", C.c_uint32), ("bytes", C.c_uint64), ("zero_once", C.c_uint32)]
+
+
+class Desc(C.Structure):
+    _fields_ = [("op", C.c_char * 24), ("plugin", C.c_char * 24), ("kernel", C.c_char * 64), ("grid", C.c_uint32 * 3),
+                ("block", C.c_uint32 * 3), ("shared_bytes", C.c_uint32), ("kernarg_bytes", C.c_uint32),
+                ("n_args", C.c_uint32), ("args", Slot * 20), ("n_workspaces", C.c_uint32), ("workspaces", Workspace * 4),
+                ("n_launches", C.c_uint32), ("ks", C.c_uint32)]
+
+    def summary(self):
+        g, b = self.grid, self.block
+        return f"{self.kernel.decode()} grid={g[0]}x{g[1]}x{g[2]} block={b[0]} n_launches={self.n_launches}"
+
+    def arg(self, name):
+        for i in range(self.n_args):
+            if self.args[i].name.decode() == name:
+                return self.args[i]
+        return None
+
+    def workspace(self, name):
+        for i in range(self.n_workspaces):
+            if self.workspaces[i].name.decode() == name:
+                return self.workspaces[i]
+        return None
+
+
+class Binding(C.Structure):
+    _fields_ = [("name", C.c_char_p), ("ptr", C.c_void_p)]
+
+
+class Counters(C.Structure):
+    _fields_ = [("plugins_loaded", C.c_uint32), ("kernels_loaded", C.c_uint32), ("refused_kernarg", C.c_uint32),
+                ("refused_wave", C.c_uint32), ("refused_metadata", C.c_uint32), ("launches", C.c_uint32)]
+
+
+class MoeTables(C.Structure):
+    _fields_ = [(n, C.c_void_p) for n in ("topk_ids", "topk_w", "route_pos", "row_tok", "tile_expert", "tile_row0",
+                                          "tile_rows", "expert_cnt", "meta", "scratch")]
+
+
+class IU8Error(RuntimeError):
+    def __init__(self, code, msg):
+        super().__init__(f"[{code}] {msg}")
+        self.code = code
+
+
+_lib = None
+
+
+def lib():
+    """The loaded C library. Raises if it was not built (run __graft_entry__.build())."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise IU8Error(E_NOTLOADED, f"{LIB_PATH} is not built; run `python -m saber_engine_amd.kbuild`")
+        try:  # share the process's HIP runtime with torch when torch is in use
+            import torch  # noqa: F401
+        except Exception:
+            pass
+        L = C.CDLL(LIB_PATH)
+        L.saber_iu8_last_error.restype = C.c_char_p
+        L.saber_iu8_a_bytes.restype = C.c_size_t
+        L.saber_iu8_a_bytes.argtypes = [C.c_uint32, C.c_uint32]
+        L.saber_iu8_a_offset.restype = C.c_uint64
+        L.saber_iu8_a_offset.argtypes = [C.c_uint32] * 3
+        L.saber_iu8_w4_offset.restype = C.c_uint64
+        L.saber_iu8_w4_offset.argtypes = [C.c_uint32] * 3 + [C.POINTER(C.c_uint32)]
+        L.saber_iu8_open.argtypes = [C.c_char_p, C.c_int, C.POINTER(C.c_void_p)]
+        L.saber_iu8_close.argtypes = [C.c_void_p]
+        L.saber_iu8_launch.argtypes = [C.c_void_p, C.POINTER(Desc), C.POINTER(Binding), C.c_uint32, C.c_void_p]
+        L.saber_iu8_quant.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32, C.c_uint32, C.c_void_p]
+        L.saber_iu8_gemm.argtypes = [C.c_void_p, C.c_int] + [C.c_void_p] * 5 + [C.c_uint32] * 3 + [C.c_void_p] * 3
+        L.saber_iu8_gemm_acc.argtypes = [C.c_void_p, C.c_int] + [C.c_void_p] * 3 + [C.c_uint32] * 3 + [C.c_void_p]
+        L.saber_iu8_get_counters.argtypes = [C.c_void_p, C.POINTER(Counters)]
+        L.saber_iu8_has_kernel.argtypes = [C.c_void_p, C.c_char_p]
+        _lib = L
+    return _lib
+
+
+def _check(rc):
+    if rc != 0:
+        raise IU8Error(rc, lib().saber_iu8_last_error().decode())
+
+
+# ---------------------------------------------------------------------------- launch law (host)
+
+def resolve(wkind, m, n, k):
+    d = Desc()
+    _check(lib().saber_iu8_resolve(wkind, m, n, k, C.byref(d)))
+    return d
+
+
+def describe(kernel, m, n, k, ks=1):
+    d = Desc()
+    _check(lib().saber_iu8_describe(kernel.encode(), m, n, k, ks, C.byref(d)))
+    return d
+
+
+def resolve_quant(m, k):
+    d = Desc()
+    _check(lib().saber_iu8_resolve_quant(m, k, C.byref(d)))
+    return d
+
+
+def resolve_silu_mul_quant(rows, n):
+    d = Desc()
+    _check(lib().saber_iu8_resolve_silu_mul_quant(rows, n, C.byref(d)))
+    return d
+
+
+def signature(kernel):
+    slots = (Slot * 24)()
+    n, b = C.c_uint32(), C.c_uint32()
+    _check(lib().saber_iu8_signature(kernel.encode(), slots, 24, C.byref(n), C.byref(b)))
+    return [(slots[i].name.decode(), slots[i].offset, slots[i].size, slots[i].kind) for i in range(n.value)], b.value
+
+
+def _bindings(bufs):
+    arr = (Binding * max(1, len(bufs)))()
+    for i, (name, ptr) in enumerate(bufs.items()):
+        arr[i].name = name.encode()
+        arr[i].ptr = ptr
+    return arr
+
+
+def pack_kernarg(desc, bufs):
+    """bufs: {name: device address}. Returns the kernarg image as bytes."""
+    img = (C.c_uint8 * 256)()
+    n = C.c_uint32()
+    _check(lib().saber_iu8_pack_kernarg(C.byref(desc), _bindings(bufs), len(bufs), img, 256, C.byref(n)))
+    return bytes(img[:n.value])
+
+
+# ---------------------------------------------------------------------------- layouts (host)
+
+def a_bytes(m, k):
+    return lib().saber_iu8_a_bytes(m, k)
+
+
+def repack_w4(canonical):
+    c = np.ascontiguousarray(canonical, dtype=np.uint8)
+    n, k = c.shape[0], c.shape[1] * 2
+    out = np.empty(n * k // 2, np.uint8)
+    _check(lib().saber_iu8_repack_w4(c.ctypes.data_as(C.c_void_p), n, k, out.ctypes.data_as(C.c_void_p)))
+    return out
+
+
+def repack_w8(rowmajor):
+    w = np.ascontiguousarray(rowmajor, dtype=np.int8)
+    n, k = w.shape
+    out = np.empty(n * k, np.uint8)
+    _check(lib().saber_iu8_repack_w8(w.ctypes.data_as(C.c_void_p), n, k, out.ctypes.data_as(C.c_void_p)))
+    return out
+
+
+def repack_weights(W, w8):
+    return repack_w8(W) if w8 else repack_w4(W)
+
+
+def repack_a(rowmajor):
+    a = np.ascontiguousarray(rowmajor, dtype=np.int8)
+    m, k = a.shape
+    out = np.empty(a_bytes(m, k), np.uint8)
+    _check(lib().saber_iu8_repack_a(a.ctypes.data_as(C.c_void_p), m, k, out.ctypes.data_as(C.c_void_p)))
+    return out
+
+
+def unpack_a(frag, m, k):
+    f = np.ascontiguousarray(frag, dtype=np.uint8)
+    out = np.empty((m, k), np.int8)
+    _check(lib().saber_iu8_unpack_a(f.ctypes.data_as(C.c_void_p), m, k, out.ctypes.data_as(C.c_void_p)))
+    return out
+
+
+# ---------------------------------------------------------------------------- manifests (host)
+
+def manifest_validate(path, arch="gfx950"):
+    """Returns (rc, refusal, message)."""
+    refusal = C.c_int(0)
+    rc = lib().saber_iu8_manifest_validate(path.encode(), arch.encode() if arch else None, C.byref(refusal))
+    return rc, refusal.value, lib().saber_iu8_last_error().decode() if rc else ""
+
+
+# ---------------------------------------------------------------------------- device side
+
+class Context:
+    """A loaded plugin set on one device (PluginSet + Launcher)."""
+
+    def __init__(self, prebuilt_dir=PREBUILT, device=0):
+        self._h = C.c_void_p()
+        _check(lib().saber_iu8_open(prebuilt_dir.encode(), device, C.byref(self._h)))
+
+    def close(self):
+        if self._h:
+            lib().saber_iu8_close(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def counters(self):
+        c = Counters()
+        _check(lib().saber_iu8_get_counters(self._h, C.byref(c)))
+        return c
+
+    def has_kernel(self, name):
+        return bool(lib().saber_iu8_has_kernel(self._h, name.encode()))
+
+    def launch(self, desc, bufs, stream=0):
+        _check(lib().saber_iu8_launch(self._h, C.byref(desc), _bindings(bufs), len(bufs), stream))
+
+    def quant(self, x, q, scale, m, k, stream=0):
+        _check(lib().saber_iu8_quant(self._h, x, q, scale, m, k, stream))
+
+    def gemm(self, wkind, a, a_scale, w, w_scale, c, m, n, k, partial=None, counter=None, stream=0):
+        _check(lib().saber_iu8_gemm(self._h, wkind, a, a_scale, w, w_scale, c, m, n, k, partial, counter, stream))
+
+    def gemm_acc(self, wkind, a, w, acc, m, n, k, stream=0):
+        _check(lib().saber_iu8_gemm_acc(self._h, wkind, a, w, acc, m, n, k, stream))
+
+
+def gemm_workspace(wkind, m, n, k):
+    p, c = C.c_uint64(), C.c_uint64()
+    _check(lib().saber_iu8_gemm_workspace(wkind, m, n, k, C.byref(p), C.byref(c)))
+    return p.value, c.value

@@ -1,0 +1,111 @@
+"""Build step of the gfx950 plugin set: the counterpart of the reference's `saber-kbuild`
+(crates/saber-kernels/src/bin/saber-kbuild.rs:186-251) and its source ladder
+(crates/saber-kernels/src/ladder.rs:12-36).
+
+For every kernel stem: resolve `<k>.gfx950.hip -> <k>.gfx95.hip -> <k>.hip`, compile with
+`hipcc --genco --offload-arch=gfx950 -O3 ...`, hash sha256(preprocessed source ++ flags), and
+write `prebuilt/gfx950/<k>.hsaco` + `<k>.manifest.toml` (schema 1, every number read back from
+the code object that was just built). Also builds the host library `libsaber_iu8.so`.
+
+    python -m saber_engine_amd.kbuild            # everything
+    python -m saber_engine_amd.kbuild macaq_iu8  # one plugin
+"""
+import ctypes
+import glob
+import hashlib
+import os
+import subprocess
+import sys
+
+PKG = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(PKG)
+KERNELS = os.path.join(PKG, "csrc", "kernels")
+HOST = os.path.join(PKG, "csrc", "host")
+ARCH = "gfx950"
+PREBUILT = os.path.join(ROOT, "prebuilt", ARCH)
+LIB = os.path.join(PKG, "libsaber_iu8.so")
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+
+# -ffp-contract=off: every product and sum rounds where the source says (the epilogue contract);
+# the packed-fp32 feature is switched off for every device compile of this tree.
+FLAGS = f"--genco --offload-arch={ARCH} -O3 -ffp-contract=off -Xclang -target-feature -Xclang -packed-fp32-ops"
+PLUGINS = ("macaq_iu8", "macaq_i8q", "moe_iu8")
+
+
+def candidates(stem, arch):
+    """Most specific first: gfx950 -> k.gfx950.hip, k.gfx95.hip, k.hip."""
+    out = [f"{stem}.{arch}.hip"]
+    digits = arch[3:] if arch.startswith("gfx") else ""
+    if len(digits) > 2:
+        fam = "gfx" + digits[:2]
+        if fam != arch:
+            out.append(f"{stem}.{fam}.hip")
+    out.append(f"{stem}.hip")
+    return out
+
+
+def resolve_source(stem, arch=ARCH, directory=KERNELS):
+    for c in candidates(stem, arch):
+        p = os.path.join(directory, c)
+        if os.path.isfile(p):
+            return p
+    return None
+
+
+def _run(cmd):
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("command failed: " + " ".join(cmd) + "\n" + r.stderr)
+    return r
+
+
+def build_lib():
+    srcs = sorted(glob.glob(os.path.join(HOST, "*.cpp")))
+    _run([HIPCC, "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-o", LIB] + srcs + ["-I" + os.path.join(ROOT, "include")])
+    return LIB
+
+
+def _lib():
+    L = ctypes.CDLL(LIB)
+    L.saber_iu8_last_error.restype = ctypes.c_char_p
+    return L
+
+
+def build_plugin(stem, out_dir=PREBUILT):
+    src = resolve_source(stem)
+    if src is None:
+        raise FileNotFoundError(f"no source for `{stem}` under {KERNELS}")
+    os.makedirs(out_dir, exist_ok=True)
+    flags = FLAGS.split()
+    pp = _run([HIPCC] + flags + ["-E", "-P", src, "-o", "-"]).stdout.encode()
+    build_hash = hashlib.sha256(pp + FLAGS.encode()).hexdigest()
+    hsaco = os.path.join(out_dir, f"{stem}.hsaco")
+    _run([HIPCC] + flags + [src, "-o", hsaco])
+    with open(src, "rb") as f:
+        src_sha = hashlib.sha256(f.read()).hexdigest()
+    manifest = os.path.join(out_dir, f"{stem}.manifest.toml")
+    L = _lib()
+    rc = L.saber_iu8_manifest_write(hsaco.encode(), stem.encode(), ARCH.encode(), os.path.relpath(src, ROOT).encode(),
+                                    src_sha.encode(), FLAGS.encode(), build_hash.encode(), manifest.encode())
+    if rc != 0:
+        raise RuntimeError(f"manifest for {stem}: {L.saber_iu8_last_error().decode()}")
+    refusal = ctypes.c_int(0)
+    rc = L.saber_iu8_manifest_validate(manifest.encode(), ARCH.encode(), ctypes.byref(refusal))
+    if rc != 0:
+        raise RuntimeError(f"{stem}: the fresh manifest does not validate: {L.saber_iu8_last_error().decode()}")
+    return hsaco, manifest
+
+
+def build_all(stems=None):
+    build_lib()
+    built = []
+    for stem in stems or PLUGINS:
+        if resolve_source(stem) is None:
+            continue
+        built.append(build_plugin(stem))
+    return built
+
+
+if __name__ == "__main__":
+    for h, m in build_all(sys.argv[1:] or None):
+        print("built", os.path.relpath(h, ROOT), os.path.relpath(m, ROOT))
