@@ -1,0 +1,215 @@
+#!/usr/bin/env python3
+"""Benchmark of the W4A8-iu8 decoder-linear hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--m 1] [--no-prefill] [--no-cpu]
+
+A step is one pass of the hot path over one batch: the four W4A8 linears of one 27B-class decoder
+layer (QKV 7168x5120, O 5120x5120, gate+up 34816x5120, down 5120x17408), each as
+per-token int8 quantisation + int4 x int8 GEMM + scale epilogue to bf16, at M tokens (default 1).
+Successive steps walk over LAYERS distinct copies of the weights (> 3x the 256 MB Infinity Cache),
+so every weight byte comes from HBM ("cold"); all inputs are resident in HBM before the timed
+region. The K timed steps are one HIP-graph replay bracketed by synchronisation.
+
+Prints ONE JSON line. `value` is algorithmic GB/s of the whole step (quant + GEMM launches);
+`roofline` is the dominant kernel (the decode GEMM) timed alone with HIP events on its stream;
+`prefill_m2048` carries the second half of the metric (int8 TOPS at M=2048, MFMA roofline);
+`cpu_baseline` is the CPU oracle's vectorised body on the host cores, on a bounded sample.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0      # MI355X published HBM3E bandwidth
+INT8_PEAK_TOPS = 5000.0     # MI355X published dense int8 MFMA peak
+LAYERS = 6                  # distinct weight copies walked by successive steps (6 x 165 MB)
+
+
+def alg_bytes(m, n, k, w8=False):
+    """Algorithmic bytes of one linear: weights + row scales + bf16 activations in + bf16 out."""
+    return (n * k if w8 else n * k // 2) + 4 * n + 2 * m * k + 2 * m * n
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=120)
+    ap.add_argument("--warmup", type=int, default=12)
+    ap.add_argument("--m", type=int, default=1, help="tokens per step (decode band, 1..16)")
+    ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU (no sharding, no collectives); --gpus must be 1", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    from saber_engine_amd import iu8, synth
+
+    assert torch.cuda.is_available(), "bench.py needs an MI355X"
+    dev = torch.device("cuda:0")
+    ctx = iu8.Context()
+    M, K_steps, W_steps = args.m, args.steps, args.warmup
+    linears = synth.LAYER_LINEARS
+
+    # ---- operands: one seeded layer (W -> ws -> A per linear), replicated to LAYERS distinct buffers
+    rng = np.random.default_rng(0)
+    host = {}
+    for name, n, k in linears:
+        Wc, ws = synth.weights(rng, n, k, False)
+        X = synth.activations(rng, max(M, 1), k)
+        host[name] = dict(W=Wc, ws=ws, X=X)
+    dev_w = {name: [] for name, _, _ in linears}
+    dev_ws, dev_x, dev_q, dev_as, dev_c = {}, {}, {}, {}, {}
+    for name, n, k in linears:
+        frag = torch.from_numpy(iu8.repack_w4(host[name]["W"])).to(dev)
+        dev_w[name] = [frag] + [frag.clone() for _ in range(LAYERS - 1)]
+        dev_ws[name] = torch.from_numpy(host[name]["ws"]).to(dev)
+        dev_x[name] = torch.from_numpy(host[name]["X"].view(np.int16)).to(dev)
+        dev_q[name] = torch.zeros(iu8.a_bytes(M, k), dtype=torch.uint8, device=dev)
+        dev_as[name] = torch.zeros(M, dtype=torch.float32, device=dev)
+        dev_c[name] = torch.zeros((M, n), dtype=torch.int16, device=dev)
+    descs = {name: iu8.resolve(iu8.W4, M, n, k) for name, n, k in linears}
+    qdescs = {name: iu8.resolve_quant(M, k) for name, n, k in linears}
+    pbytes = max([d.workspace("decode_partial").bytes for d in descs.values() if d.ks > 1] + [4])
+    cbytes = max([d.workspace("decode_counter").bytes for d in descs.values() if d.ks > 1] + [4])
+    partial = torch.zeros(pbytes // 4, dtype=torch.int32, device=dev)
+    counter = torch.zeros(cbytes // 4, dtype=torch.int32, device=dev)
+
+    stream = torch.cuda.Stream()
+    sh = stream.cuda_stream
+
+    def launch_quant(name):
+        ctx.launch(qdescs[name], dict(x=dev_x[name].data_ptr(), q=dev_q[name].data_ptr(), scale=dev_as[name].data_ptr()), sh)
+
+    def launch_gemm(name, layer):
+        b = dict(a=dev_q[name].data_ptr(), w=dev_w[name][layer].data_ptr(), ws=dev_ws[name].data_ptr(), c=dev_c[name].data_ptr(),
+                 decode_partial=partial.data_ptr(), decode_counter=counter.data_ptr())
+        b["as"] = dev_as[name].data_ptr()
+        ctx.launch(descs[name], b, sh)
+
+    def step(i, gemm_only=False):
+        for name, _, _ in linears:
+            if not gemm_only:
+                launch_quant(name)
+            launch_gemm(name, i % LAYERS)
+
+    def capture(nsteps, gemm_only=False):
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=stream):
+            for i in range(nsteps):
+                step(i, gemm_only)
+        return g
+
+    with torch.cuda.stream(stream):
+        for i in range(W_steps):
+            step(i)
+    stream.synchronize()
+    g_all = capture(K_steps)
+    g_gemm = capture(K_steps, gemm_only=True)
+    with torch.cuda.stream(stream):
+        g_all.replay()
+        g_gemm.replay()
+    torch.cuda.synchronize()
+
+    # ---- the timed region: exactly K steps, one graph replay, bracketed by synchronisation
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    with torch.cuda.stream(stream):
+        g_all.replay()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / K_steps
+    step_bytes = sum(alg_bytes(M, n, k) for _, n, k in linears)
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+
+    # ---- the dominant kernel alone (decode GEMM, 4 launches a step), HIP events on its stream
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    with torch.cuda.stream(stream):
+        ev0.record(stream)
+        g_gemm.replay()
+        ev1.record(stream)
+    torch.cuda.synchronize()
+    gemm_us = ev0.elapsed_time(ev1) * 1e3 / (K_steps * len(linears))
+    gemm_bytes = sum(alg_bytes(M, n, k) - 2 * M * k + M * k + 4 * M for _, n, k in linears) / len(linears)
+    achieved = gemm_bytes / (gemm_us * 1e-6) / 1e9
+    roofline = dict(bound="hbm", kernel=descs["down"].kernel.decode(), achieved=round(achieved, 1), peak=HBM_PEAK_GBPS,
+                    unit="GB/s", frac=round(achieved / HBM_PEAK_GBPS, 4), traffic=None,
+                    avg_launch_us=round(gemm_us, 3), bytes_per_launch=gemm_bytes,
+                    note="mean over the four layer shapes, cold weights (rotating %d copies), graph replay" % LAYERS)
+
+    # ---- parity spot check against the CPU oracle, and the CPU baseline beside it
+    out = dict(metric="W4A8 GEMM GB/s (%HBM) at M=1; int8 TOPS (%MFMA peak) at M=2048", value=round(value, 1), unit="GB/s",
+               n_gpus=1, steps=K_steps, warmup=W_steps, ms_per_step=round(ms_per_step, 5), higher_is_better=True,
+               scaling="weak", vs_baseline=None, dtype="int4 x int8 -> int32 -> bf16", data="synthetic (seed 0)",
+               config=dict(workload="configs[1]: decode-batch W4A8 linear set of one 27B-class layer (QKV, O, gate+up, down), "
+                                    "hidden 5120, TP=1", m=M, layers_rotated=LAYERS, cold=True,
+                           launches_per_step=2 * len(linears), hbm_frac=round(value / HBM_PEAK_GBPS, 4)),
+               roofline=roofline)
+
+    if not args.no_cpu:
+        from oracle import ref
+
+        threads = min(os.cpu_count() or 1, 16)
+        ok = True
+        t_cpu, n_cpu = 0.0, 0
+        while t_cpu < args.cpu_seconds:
+            for name, n, k in linears:
+                c0 = time.perf_counter()
+                r = ref.linear(host[name]["X"][:M], host[name]["W"], host[name]["ws"], False, threads=threads, pin=1)
+                t_cpu += time.perf_counter() - c0
+                if n_cpu == 0:
+                    got = dev_c[name].cpu().numpy().view(np.uint16)
+                    ok = ok and bool(np.array_equal(got, r["C"]))
+            n_cpu += 1
+        isa = {0: "scalar", 1: "avx2", 2: "avx512-vnni"}[ref.lib().w4a8_isa()]
+        out["cpu_baseline"] = dict(value=round(step_bytes * n_cpu / t_cpu / 1e9, 2), unit="GB/s", cores=threads, kind="port",
+                                   sample="%d steps (quant + GEMM + epilogue of the same four linears, M=%d), %s body, "
+                                          "threads pinned one per core, 16-column tiles" % (n_cpu, M, isa))
+        out["parity_vs_oracle"] = ok
+
+    # ---- the second half of the metric: int8 TOPS at M=2048 on the same four shapes
+    if not args.no_prefill:
+        PM = 2048
+        pf = {}
+        tot_ops, tot_us = 0.0, 0.0
+        for name, n, k in linears:
+            d = iu8.resolve(iu8.W4, PM, n, k)
+            q = torch.randint(-127, 128, (iu8.a_bytes(PM, k),), dtype=torch.int8, device=dev).view(torch.uint8)
+            a_s = torch.rand(PM, dtype=torch.float32, device=dev) * 0.05 + 0.01
+            c = torch.zeros((PM, n), dtype=torch.int16, device=dev)
+            b = dict(a=q.data_ptr(), w=dev_w[name][0].data_ptr(), ws=dev_ws[name].data_ptr(), c=c.data_ptr())
+            b["as"] = a_s.data_ptr()
+            reps = 10
+            with torch.cuda.stream(stream):
+                for _ in range(3):
+                    ctx.launch(d, b, sh)
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record(stream)
+                for _ in range(reps):
+                    ctx.launch(d, b, sh)
+                e1.record(stream)
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) * 1e3 / reps
+            ops = 2.0 * PM * n * k
+            pf[name] = dict(kernel=d.kernel.decode(), grid=list(d.grid), us=round(us, 2), tops=round(ops / us / 1e6, 1))
+            tot_ops += ops
+            tot_us += us
+            del q, a_s, c
+        tops = tot_ops / tot_us / 1e6
+        out["prefill_m2048"] = dict(value=round(tops, 1), unit="TOPS", per_linear=pf,
+                                    roofline=dict(bound="mfma", achieved=round(tops / 1e3, 4), peak=INT8_PEAK_TOPS / 1e3,
+                                                  unit="POP/s", frac=round(tops / INT8_PEAK_TOPS, 4), traffic=None))
+    print(json.dumps(out), flush=True)
+    ctx.close()
+
+
+if __name__ == "__main__":
+    main()

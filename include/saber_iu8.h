@@ -129,6 +129,14 @@ int saber_iu8_resolve_quant(uint32_t m, uint32_t k, saber_iu8_desc *out);
 /* SiLU(gate) * up + requant over rows of [gate(n) | up(n)] (abi.rs:315-320, 344-351). */
 int saber_iu8_resolve_silu_mul_quant(uint32_t rows, uint32_t n, saber_iu8_desc *out);
 
+/* A descriptor for any kernel of the loaded objects with an explicit grid (in workgroups) and
+ * block: slots come from the kernel's signature, scalars are then set by name. The replay
+ * harness's form (crates/saber-kernels/hip/harness/run_hsaco.cpp:1-15: "launches exactly what the
+ * descriptor says"); used for the probe kernels and by sweeps. */
+int saber_iu8_describe_raw(const char *kernel, const char *plugin, const uint32_t grid[3], uint32_t block,
+                           saber_iu8_desc *out);
+int saber_iu8_desc_set_i32(saber_iu8_desc *desc, const char *name, int64_t value);
+
 /* abi::signature_for + abi::pack (abi.rs:111-130, 3495): fills names/offsets/sizes of the
  * explicit arguments of `kernel`; returns the explicit kernarg size in *bytes. */
 int saber_iu8_signature(const char *kernel, saber_iu8_slot *slots, uint32_t cap, uint32_t *n_slots, uint32_t *bytes);

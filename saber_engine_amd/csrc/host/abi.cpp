@@ -30,6 +30,11 @@ static const Signature SIG_MOE_COMBINE = {{"y", K::Buffer},    {"topk_w", K::Buf
                                           {"sgate", K::Buffer}, {"meta", K::Buffer},  {"out", K::Buffer},
                                           {"h", K::I32}};
 
+static const Signature SIG_PROBE_READ = {{"src", K::Buffer}, {"out", K::Buffer}, {"n", K::I32}};
+static const Signature SIG_PROBE_COPY = {{"src", K::Buffer}, {"dst", K::Buffer}, {"n", K::I32}};
+static const Signature SIG_PROBE_EMPTY = {{"out", K::Buffer}};
+static const Signature SIG_PROBE_MFMA = {{"out", K::Buffer}, {"n", K::I32}};
+
 static bool starts(const std::string &s, const char *p) { return s.rfind(p, 0) == 0; }
 
 const Signature *signature_for(const std::string &k) {
@@ -38,6 +43,10 @@ const Signature *signature_for(const std::string &k) {
   if (starts(k, "macaq_i8_quant_")) return &SIG_QUANT;
   if (starts(k, "macaq_i8_silu_mul_quant_")) return &SIG_SILU;
   if (k == "macaq_silu_bf16_table") return &SIG_TABLE;
+  if (k == "iu8_probe_read") return &SIG_PROBE_READ;
+  if (k == "iu8_probe_copy") return &SIG_PROBE_COPY;
+  if (k == "iu8_probe_empty") return &SIG_PROBE_EMPTY;
+  if (k == "iu8_probe_mfma") return &SIG_PROBE_MFMA;
   if (starts(k, "moe_iu8_route_")) return &SIG_MOE_ROUTE;
   if (starts(k, "moe_iu8_grouped_")) return &SIG_MOE_GROUPED;
   if (starts(k, "moe_iu8_combine_")) return &SIG_MOE_COMBINE;

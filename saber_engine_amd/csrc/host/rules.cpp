@@ -8,14 +8,14 @@
 namespace iu8 {
 
 static const DecVariant DEC_VARIANTS[] = {
-#define IU8_DEC_VARIANT(name, TM, W8, NT, KW, WPB, U, ACC) {#name, TM, W8, NT, KW, WPB, U, ACC},
+#define IU8_DEC_VARIANT(name, TM, W8, NT, KW, WPB, D, ALDS, ACC) {#name, TM, W8, NT, KW, WPB, D, ALDS, ACC},
 #define IU8_PF_VARIANT(name, W8, WMW, WNW, TM, TN, ACC)
 #include "../kernels/iu8_variants.def"
 #undef IU8_DEC_VARIANT
 #undef IU8_PF_VARIANT
 };
 static const PfVariant PF_VARIANTS[] = {
-#define IU8_DEC_VARIANT(name, TM, W8, NT, KW, WPB, U, ACC)
+#define IU8_DEC_VARIANT(name, TM, W8, NT, KW, WPB, D, ALDS, ACC)
 #define IU8_PF_VARIANT(name, W8, WMW, WNW, TM, TN, ACC) {#name, W8, WMW, WNW, TM, TN, ACC},
 #include "../kernels/iu8_variants.def"
 #undef IU8_DEC_VARIANT
@@ -88,16 +88,10 @@ static int check_shape(const char *op, uint32_t m, uint32_t n, uint32_t k) {
   return 0;
 }
 
-// Double the split until the grid reaches two workgroups a CU, each k-wave keeps >= 2 steps, and
-// the partials stay small next to the weights (they are written and re-read once).
-uint32_t decode_split(uint32_t m, uint32_t n, uint32_t k, uint32_t nblk, uint32_t kw) {
-  const uint32_t steps = k / 128;
-  uint32_t ks = 1;
-  while (nblk * ks < 2 * CU_COUNT && ks < KS_MAX && steps / (ks * 2 * kw) >= 2 &&
-         (uint64_t)(ks * 2) * m * n * 4 * 8 <= (uint64_t)n * k / 2)
-    ks *= 2;
-  return ks;
-}
+// The grid-level split of a decode GEMM. On this card a split costs device-scope fences across
+// the 8 XCDs' L2s (measured: 3-7x the unsplit kernel), and the k-waves of a workgroup already
+// split K through LDS, so the law does not split; `describe` still takes an explicit count.
+uint32_t decode_split(uint32_t, uint32_t, uint32_t, uint32_t, uint32_t) { return 1; }
 
 static int describe_dec(const DecVariant &v, uint32_t m, uint32_t n, uint32_t k, uint32_t ks, saber_iu8_desc *d) {
   const char *op = v.w8 ? "gemm_i8a8" : "gemm_i4a8";
@@ -163,7 +157,15 @@ int resolve(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *out) 
   if (int rc = check_shape(wkind == SABER_IU8_W8 ? "gemm_i8a8" : "gemm_i4a8", m, n, k)) return rc;
   if (m <= DECODE_MAX_M) {
     const uint32_t tm = (m + 15) / 16;
-    const std::string name = fmt("macaq_iu8_dec_%s_tm%u", tag, tm);
+    std::string name = fmt("macaq_iu8_dec_%s_tm%u", tag, tm);
+    if (tm == 1) {
+      // live rows staged in LDS when they fit the 20 KiB or the 80 KiB form, else read from L2
+      uint32_t mr = 1;
+      while (mr < m) mr *= 2;
+      const uint64_t need = (uint64_t)mr * k;
+      if (need > 80 * 1024) name += "_a0";
+      else if (need > 20 * 1024) name += "_a80";
+    }
     const DecVariant *v = dec_variant(name);
     if (!v) return fail(SABER_IU8_E_RULE, name + ": no such variant");
     const uint32_t nblk = (n + v->block_n() - 1) / v->block_n();

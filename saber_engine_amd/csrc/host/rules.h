@@ -11,7 +11,7 @@ namespace iu8 {
 
 struct DecVariant {
   const char *name;
-  int tm, w8, nt, kw, wpb, u, acc;
+  int tm, w8, nt, kw, wpb, depth, alds, acc;
   int block_n() const { return wpb / kw * nt * 16; }
   int threads() const { return wpb * 64; }
 };

@@ -89,6 +89,34 @@ int saber_iu8_resolve_silu_mul_quant(uint32_t rows, uint32_t n, saber_iu8_desc *
   return resolve_silu_mul_quant(rows, n, out);
 }
 
+int saber_iu8_describe_raw(const char *kernel, const char *plugin, const uint32_t grid[3], uint32_t block,
+                           saber_iu8_desc *out) {
+  if (!kernel || !grid || !out) return fail(SABER_IU8_E_ARG, "describe_raw: null argument");
+  if (!grid[0] || !grid[1] || !grid[2] || !block || block > 1024) return fail(SABER_IU8_E_RULE, std::string(kernel) + ": empty or oversized launch");
+  memset(out, 0, sizeof *out);
+  snprintf(out->op, sizeof out->op, "raw");
+  snprintf(out->plugin, sizeof out->plugin, "%s", plugin ? plugin : "");
+  snprintf(out->kernel, sizeof out->kernel, "%s", kernel);
+  for (int i = 0; i < 3; ++i) out->grid[i] = grid[i];
+  out->block[0] = block, out->block[1] = 1, out->block[2] = 1;
+  out->n_launches = 1;
+  out->ks = 1;
+  return fill_slots(kernel, out);
+}
+
+int saber_iu8_desc_set_i32(saber_iu8_desc *desc, const char *name, int64_t value) {
+  if (!desc || !name) return fail(SABER_IU8_E_ARG, "desc_set_i32: null argument");
+  for (uint32_t i = 0; i < desc->n_args; ++i)
+    if (!strcmp(desc->args[i].name, name)) {
+      if (desc->args[i].kind == SABER_IU8_ARG_BUFFER || desc->args[i].kind == SABER_IU8_ARG_NULL_BUFFER)
+        return fail(SABER_IU8_E_ARG, std::string(name) + ": a buffer slot, not a scalar");
+      desc->args[i].kind = SABER_IU8_ARG_I32;
+      desc->args[i].ival = value;
+      return 0;
+    }
+  return fail(SABER_IU8_E_ARG, std::string(desc->kernel) + ": no argument `" + name + "`");
+}
+
 int saber_iu8_signature(const char *kernel, saber_iu8_slot *slots, uint32_t cap, uint32_t *n_slots, uint32_t *bytes) {
   if (!kernel || !slots || !n_slots || !bytes) return fail(SABER_IU8_E_ARG, "signature: null argument");
   saber_iu8_desc d;

@@ -7,12 +7,17 @@
 //
 // Two regimes, two designs.
 //   decode  (M <= 64)  HBM-bound weight streaming. A workgroup owns WN*NT 16-row weight tiles;
-//           its KW "k-waves" interleave over 128-deep K steps of the same tiles, each issuing
-//           128-bit nontemporal loads of packed int4 (one 1-KiB fragment per wave-load), with the
-//           next batch of loads in flight while the current one is unpacked in registers and fed
-//           to v_mfma_i32_16x16x64_i8. The split-K partials of the k-waves are reduced through
-//           LDS (exact int32); an optional grid-level split (gridDim.z) goes through the
-//           `decode_partial` / `decode_counter` workspaces, the last-arriving workgroup summing.
+//           its KW "k-waves" interleave over 128-deep K steps of the same tiles. Every wave keeps
+//           a ring of D steps of 128-bit nontemporal loads of packed int4 in flight (one 1-KiB
+//           fragment per wave-load): a step is consumed (nibble unpack in registers,
+//           v_mfma_i32_16x16x64_i8) and its ring slot re-issued D steps ahead. For M <= 16 the
+//           workgroup's activation rows are staged once in LDS (only the live rows, behind the
+//           first ring of weight loads); lanes of dead rows read row 0, which is harmless: a
+//           row of A only reaches its own row of C, and dead rows are never stored. The k-waves'
+//           partials are reduced through LDS (exact int32). An optional grid-level split
+//           (gridDim.z) goes through the `decode_partial` / `decode_counter` workspaces with the
+//           last-arriving workgroup summing; it costs device-scope fences across the 8 XCDs' L2s
+//           and the launch law does not use it by default.
 //   prefill (M > 64)   MFMA-bound tile GEMM. A workgroup of WMW x WNW waves owns a
 //           (WMW*TM*16) x (WNW*TN*16) output tile; A and W fragments of one 128-deep K step are
 //           staged in LDS in fragment order (W4 stays packed; the unpack happens after the LDS
@@ -21,18 +26,24 @@
 #include "iu8_common.h"
 
 // ============================================================================ decode band
-template <int TM, bool W8, int NT, int KW, int WPB, int U, bool ACC>
+template <int TM, bool W8, int NT, int KW, int WPB, int D, int ALDS, bool ACC>
 __device__ __forceinline__ void iu8_dec_body(const iu8_u8 *__restrict__ A, const iu8_u8 *__restrict__ W,
                                              const float *__restrict__ as, const float *__restrict__ ws,
                                              int *__restrict__ P, int *__restrict__ cnt, void *__restrict__ Cv,
                                              int M, int N, int K) {
   static_assert(WPB % KW == 0, "k-waves divide the workgroup");
+  static_assert(ALDS == 0 || TM == 1, "LDS staging of A is the M <= 16 form");
   constexpr int WN = WPB / KW;
+  constexpr int NTHR = WPB * 64;
   constexpr int WSTEP = W8 ? 2048 : 1024;  // bytes of one 16-row weight tile per 128-deep K step
   constexpr int WV = W8 ? 2 : 1;           // 16-byte loads a lane per step per tile
   constexpr int BN = WN * NT * 16;         // columns a workgroup
-  __shared__ int s_red[(KW > 1 ? KW - 1 : 1) * WN * TM * NT * 256];
+  constexpr int RED = (KW > 1 ? KW - 1 : 1) * WN * TM * NT * 1024;
+  constexpr int ABYTES = ALDS * 1024;
+  // one LDS block: the staged activation rows, re-used for the k-waves' partials at the end
+  __shared__ __attribute__((aligned(16))) iu8_u8 s_mem[ABYTES > RED ? ABYTES : RED];
   __shared__ int s_last;
+  int *s_red = (int *)s_mem;
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -42,17 +53,16 @@ __device__ __forceinline__ void iu8_dec_body(const iu8_u8 *__restrict__ A, const
   const int spb = (steps + Z - 1) / Z;
   const int s_lo = z * spb, s_hi = min(steps, s_lo + spb);
   const int nt0 = (blockIdx.x * WN + wn) * NT;
+  const int ml = lane & 15, lg = lane >> 4;
+  // this wave's steps: s_lo + wk + t*KW, t in [0, T)
+  const int T = s_lo + wk < s_hi ? (s_hi - s_lo - wk + KW - 1) / KW : 0;
 
   const iu8_u8 *wp[NT];
 #pragma unroll
   for (int j = 0; j < NT; ++j) {
     const int ntj = min(nt0 + j, ntiles - 1);  // a tile past N re-reads the last one and stores nothing
-    wp[j] = W + (size_t)ntj * steps * WSTEP + lane * 16;
+    wp[j] = W + ((size_t)ntj * steps + s_lo + wk) * WSTEP + lane * 16;
   }
-  bool live[TM];
-#pragma unroll
-  for (int i = 0; i < TM; ++i) live[i] = i * 16 + (lane & 15) < M;
-  const iu8_u8 *ap = A + lane * 16;
 
   iu8_v4i acc[TM][NT];
 #pragma unroll
@@ -60,69 +70,144 @@ __device__ __forceinline__ void iu8_dec_body(const iu8_u8 *__restrict__ A, const
 #pragma unroll
     for (int j = 0; j < NT; ++j) acc[i][j] = iu8_v4i{0, 0, 0, 0};
 
-  struct Batch {
-    iu8_v4u w[U][NT][WV];
-    iu8_v4i a[U][TM][2];
+  // ---- LDS staging of the live activation rows (issued before the weight ring, waited after it)
+  // MR = staged rows (a power of two >= M); piece p = ((kt*4 + g)*MR + r) holds row r's 16 bytes
+  // of k = (2*s_lo + kt)*64 + g*16.
+  bool staged = false;
+  int mr_shift = 0;
+  constexpr int A_PER = ALDS ? (ABYTES / 16 + NTHR - 1) / NTHR : 1;
+  constexpr bool A_INREG = A_PER <= 8;
+  iu8_v4u areg[A_INREG ? A_PER : 1];
+  int a_pieces = 0;
+  if constexpr (ALDS > 0) {
+    while ((1 << mr_shift) < M) ++mr_shift;
+    a_pieces = ((s_hi - s_lo) * 2 * 4) << mr_shift;
+    staged = M <= 16 && a_pieces * 16 <= ABYTES;
+    if (staged) {
+      auto a_src = [&](int piece) {
+        const int r = piece & ((1 << mr_shift) - 1), g = (piece >> mr_shift) & 3, kt = piece >> (mr_shift + 2);
+        return (const iu8_v4u *)(A + ((size_t)(2 * s_lo + kt) * 1024 + (r + 16 * g) * 16));
+      };
+      if constexpr (A_INREG) {  // few pieces a thread: loads now, LDS stores behind the first weight ring
+#pragma unroll
+        for (int p = 0; p < A_PER; ++p)
+          if (p * NTHR + tid < a_pieces) areg[p] = *a_src(p * NTHR + tid);
+      } else {                  // many: copy before the ring starts
+        for (int piece = tid; piece < a_pieces; piece += NTHR) *(iu8_v4u *)&s_mem[piece * 16] = *a_src(piece);
+      }
+    }
+  }
+
+  // ---- the weight ring
+  iu8_v4u ring[D][NT][WV];
+  iu8_v4i ringa[ALDS ? 1 : D][TM][2];  // direct-from-L2 activation operands when not staged
+  bool live[TM];
+#pragma unroll
+  for (int i = 0; i < TM; ++i) live[i] = i * 16 + ml < M;
+  const iu8_u8 *ap = A + (size_t)(s_lo + wk) * 2048 + lane * 16;
+  auto issue = [&](int slot, int t) {
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int v = 0; v < WV; ++v) ring[slot][j][v] = iu8_ldg_nt(wp[j] + (size_t)t * (KW * WSTEP) + v * 1024);
+    if (!staged) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          ringa[ALDS ? 0 : slot][i][h] = iu8_v4i{0, 0, 0, 0};
+          if (live[i])
+            ringa[ALDS ? 0 : slot][i][h] =
+                *(const iu8_v4i *)(ap + ((size_t)i * ktiles + (size_t)t * (2 * KW) + h) * 1024);
+        }
+    }
   };
-  auto load = [&](Batch &b, int s) {
+  const int a_lane = (((lg << mr_shift) + min(ml, (1 << mr_shift) - 1)) << 4);
+  auto consume = [&](int slot, int t) {
+    iu8_v4i a0[TM], a1[TM];
+    if (ALDS > 0 && staged) {
+      const int kt = 2 * (wk + t * KW);
+      a0[0] = *(const iu8_v4i *)&s_mem[((kt * 4) << (mr_shift + 4)) + a_lane];
+      a1[0] = *(const iu8_v4i *)&s_mem[(((kt + 1) * 4) << (mr_shift + 4)) + a_lane];
+    } else {
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int su = s + u * KW;
-      if (su < s_hi) {
+      for (int i = 0; i < TM; ++i) {
+        a0[i] = ringa[ALDS ? 0 : slot][i][0];
+        a1[i] = ringa[ALDS ? 0 : slot][i][1];
+      }
+    }
 #pragma unroll
-        for (int j = 0; j < NT; ++j)
-#pragma unroll
-          for (int v = 0; v < WV; ++v) b.w[u][j][v] = iu8_ldg_nt(wp[j] + (size_t)su * WSTEP + v * 1024);
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-          for (int h = 0; h < 2; ++h) {
-            b.a[u][i][h] = iu8_v4i{0, 0, 0, 0};
-            if (live[i]) b.a[u][i][h] = *(const iu8_v4i *)(ap + ((size_t)i * ktiles + 2 * su + h) * 1024);
-          }
+    for (int j = 0; j < NT; ++j) {
+      iu8_v4i w0, w1;
+      if constexpr (W8) {
+        w0 = (iu8_v4i)ring[slot][j][0];
+        w1 = (iu8_v4i)ring[slot][j][WV - 1];
       } else {
+        iu8_unpack_w4(ring[slot][j][0], w0, w1);
+      }
 #pragma unroll
-        for (int j = 0; j < NT; ++j)
-#pragma unroll
-          for (int v = 0; v < WV; ++v) b.w[u][j][v] = iu8_v4u{0, 0, 0, 0};
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-          for (int h = 0; h < 2; ++h) b.a[u][i][h] = iu8_v4i{0, 0, 0, 0};
+      for (int i = 0; i < TM; ++i) {
+        acc[i][j] = iu8_mfma(w0, a0[i], acc[i][j]);
+        acc[i][j] = iu8_mfma(w1, a1[i], acc[i][j]);
       }
     }
   };
-  auto compute = [&](const Batch &b) {
-#pragma unroll
-    for (int u = 0; u < U; ++u)
-#pragma unroll
-      for (int j = 0; j < NT; ++j) {
-        iu8_v4i w0, w1;
-        if constexpr (W8) {
-          w0 = (iu8_v4i)b.w[u][j][0];
-          w1 = (iu8_v4i)b.w[u][j][WV - 1];
-        } else {
-          iu8_unpack_w4(b.w[u][j][0], w0, w1);
-        }
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-          acc[i][j] = iu8_mfma(w0, b.a[u][i][0], acc[i][j]);
-          acc[i][j] = iu8_mfma(w1, b.a[u][i][1], acc[i][j]);
-        }
-      }
-  };
 
-  {
-    int s = s_lo + wk;
-    if (s < s_hi) {
-      Batch b0;
-      load(b0, s);
-      for (; s < s_hi; s += KW * U) {
-        Batch b1;
-        load(b1, s + KW * U);  // past the end: zeros, no memory touched
-        compute(b0);
-        b0 = b1;
+  if constexpr (ALDS > 0) {
+    // staged form: the ring never holds activations, so the not-staged fallback of an ALDS kernel
+    // (shape too large for its LDS) loads them at consume time through the one-slot `ringa`
+    if (!staged) {
+      for (int t = 0; t < T; ++t) {
+        issue(0, t);
+        consume(0, t);
       }
+    } else {
+#pragma unroll
+      for (int i = 0; i < D; ++i)
+        if (i < T) issue(i, i);
+      if constexpr (A_INREG) {
+#pragma unroll
+        for (int p = 0; p < A_PER; ++p)
+          if (p * NTHR + tid < a_pieces) *(iu8_v4u *)&s_mem[(p * NTHR + tid) * 16] = areg[p];
+      }
+      __syncthreads();
+      int t0 = 0;
+      for (; t0 + 2 * D <= T; t0 += D) {  // steady state: every slot consumed and re-issued
+#pragma unroll
+        for (int i = 0; i < D; ++i) {
+          consume(i, t0 + i);
+          issue(i, t0 + i + D);
+        }
+      }
+      for (; t0 < T; t0 += D) {  // drain
+#pragma unroll
+        for (int i = 0; i < D; ++i)
+          if (t0 + i < T) {
+            consume(i, t0 + i);
+            if (t0 + i + D < T) issue(i, t0 + i + D);
+          }
+      }
+      __syncthreads();  // every wave is done with the staged rows before s_mem holds partials
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < D; ++i)
+      if (i < T) issue(i, i);
+    int t0 = 0;
+    for (; t0 + 2 * D <= T; t0 += D) {
+#pragma unroll
+      for (int i = 0; i < D; ++i) {
+        consume(i, t0 + i);
+        issue(i, t0 + i + D);
+      }
+    }
+    for (; t0 < T; t0 += D) {
+#pragma unroll
+      for (int i = 0; i < D; ++i)
+        if (t0 + i < T) {
+          consume(i, t0 + i);
+          if (t0 + i + D < T) issue(i, t0 + i + D);
+        }
     }
   }
 
@@ -147,7 +232,7 @@ __device__ __forceinline__ void iu8_dec_body(const iu8_u8 *__restrict__ A, const
     }
   }
 
-  const int ml = lane & 15, nq = (lane >> 4) * 4;
+  const int nq = lg * 4;
   if (Z == 1) {
     if (wk != 0) return;
 #pragma unroll
@@ -199,7 +284,7 @@ __device__ __forceinline__ void iu8_dec_body(const iu8_u8 *__restrict__ A, const
   __threadfence();
   if (tid == 0) cnt[blockIdx.x] = 0;
   const int nb = blockIdx.x * BN, nw4 = min(BN, N - nb) >> 2;
-  for (int idx = tid; idx < nw4 * M; idx += WPB * 64) {
+  for (int idx = tid; idx < nw4 * M; idx += NTHR) {
     const int m = idx / nw4, n = nb + (idx % nw4) * 4;
     iu8_v4i sum = iu8_v4i{0, 0, 0, 0};
     for (int q = 0; q < Z; ++q) sum += __builtin_nontemporal_load((const iu8_v4i *)&P[((size_t)q * M + m) * N + n]);
@@ -215,15 +300,14 @@ __device__ __forceinline__ void iu8_dec_body(const iu8_u8 *__restrict__ A, const
   }
 }
 
-#define IU8_DEC(name, TM, W8, NT, KW, WPB, U, ACC)                                                               \
+#define IU8_DEC(name, TM, W8, NT, KW, WPB, D, ALDS, ACC)                                                         \
   extern "C" __global__ __launch_bounds__(WPB * 64) void name(                                                    \
       const unsigned char *__restrict__ a, const unsigned char *__restrict__ w, const float *__restrict__ as,     \
       const float *__restrict__ ws, int *__restrict__ decode_partial, int *__restrict__ decode_counter,           \
       unsigned short *__restrict__ c, int m, int n, int k) {                                                       \
-    iu8_dec_body<TM, W8, NT, KW, WPB, U, ACC>(a, w, as, ws, decode_partial, decode_counter, c, m, n, k);           \
+    iu8_dec_body<TM, W8, NT, KW, WPB, D, ALDS, ACC>(a, w, as, ws, decode_partial, decode_counter, c, m, n, k);     \
   }
-
-#define IU8_DEC_VARIANT(name, TM, W8, NT, KW, WPB, U, ACC) IU8_DEC(name, TM, W8, NT, KW, WPB, U, ACC)
+#define IU8_DEC_VARIANT(name, TM, W8, NT, KW, WPB, D, ALDS, ACC) IU8_DEC(name, TM, W8, NT, KW, WPB, D, ALDS, ACC)
 #define IU8_PF_VARIANT(name, W8, WMW, WNW, TM, TN, ACC)
 #include "iu8_variants.def"
 #undef IU8_DEC_VARIANT
@@ -344,7 +428,7 @@ __device__ __forceinline__ void iu8_pf_body(const iu8_u8 *__restrict__ A, const 
       const float *__restrict__ ws, unsigned short *__restrict__ c, int m, int n, int k) {                         \
     iu8_pf_body<W8, WMW, WNW, TM, TN, ACC>(a, w, as, ws, c, m, n, k);                                              \
   }
-#define IU8_DEC_VARIANT(name, TM, W8, NT, KW, WPB, U, ACC)
+#define IU8_DEC_VARIANT(name, TM, W8, NT, KW, WPB, D, ALDS, ACC)
 #define IU8_PF_VARIANT(name, W8, WMW, WNW, TM, TN, ACC) IU8_PF(name, W8, WMW, WNW, TM, TN, ACC)
 #include "iu8_variants.def"
 #undef IU8_DEC_VARIANT

@@ -141,6 +141,16 @@ def resolve_silu_mul_quant(rows, n):
     return d
 
 
+def describe_raw(kernel, grid, block, plugin="", **scalars):
+    """Descriptor for any loaded kernel with an explicit launch shape; scalars set by name."""
+    d = Desc()
+    g = (C.c_uint32 * 3)(*grid)
+    _check(lib().saber_iu8_describe_raw(kernel.encode(), plugin.encode(), g, block, C.byref(d)))
+    for name, v in scalars.items():
+        _check(lib().saber_iu8_desc_set_i32(C.byref(d), name.encode(), C.c_int64(int(v))))
+    return d
+
+
 def signature(kernel):
     slots = (Slot * 24)()
     n, b = C.c_uint32(), C.c_uint32()
