@@ -1,0 +1,74 @@
+"""Writes the small golden vectors of tests/golden/ (run from the repo root:
+`python tests/golden/make_fixtures.py`).
+
+The reference holds no input/output vector for the iu8 arithmetic (its GPU gate replays captures
+that are not in its tree), so these vectors are produced HERE by an independent brute-force
+restatement of the written contract in numpy -- float32 IEEE divide / np.rint for the codes, an
+int64 matrix product for the accumulators, float64 products rounded once to float32 for the two
+epilogue multiplies (exact: a product of two float32 fits float64), the bit trick for bf16 -- and
+NOT by the C oracle. The oracle and the HIP path are both checked against them.
+
+kernarg_gfx1201.json holds data read off the reference's committed manifest
+(prebuilt/gfx1201/macaq_iu8.manifest.toml): the explicit kernarg offsets/sizes the host packs.
+"""
+import json
+import os
+import sys
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
+from saber_engine_amd import synth  # noqa: E402  (seeded operand generator only)
+
+
+def bf16_rne_np(x):
+    u = np.asarray(x, np.float32).view(np.uint32).astype(np.uint64)
+    return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+
+
+def brute_linear(Xbits, W, ws, w8):
+    x = synth.bf16_bits_to_f32(Xbits)
+    amax = np.max(np.abs(x), axis=1)
+    sc = np.maximum((amax / np.float32(127.0)).astype(np.float32), np.float32(1e-30))
+    y = (x / sc[:, None]).astype(np.float32)
+    q = np.rint(np.clip(y, -127.0, 127.0)).astype(np.int8)
+    w = W.astype(np.int64) if w8 else synth.unpack_w4(W).astype(np.int64)
+    S = q.astype(np.int64) @ w.T
+    assert np.abs(S).max() < 2 ** 27
+    acc = S if w8 else S * 16
+    wsu = ws if w8 else (ws.astype(np.float64) * 0.0625).astype(np.float32)
+    t = (acc.astype(np.float32).astype(np.float64) * sc[:, None].astype(np.float64)).astype(np.float32)
+    yv = (t.astype(np.float64) * wsu[None, :].astype(np.float64)).astype(np.float32)
+    return q, sc, S.astype(np.int32), bf16_rne_np(yv)
+
+
+def main():
+    cases = [(1, 64, 256, False, 0), (16, 48, 128, False, 1), (5, 32, 256, True, 2), (64, 64, 256, False, 3),
+             (33, 16, 128, True, 4)]
+    out = {}
+    for i, (M, N, K, w8, seed) in enumerate(cases):
+        c = synth.dense_case(M, N, K, w8=w8, seed=seed)
+        if i == 1:
+            c["X"][3, :] = 0  # an all-zero token row: scale 1e-30, codes 0
+        q, sc, S, C = brute_linear(c["X"], c["W"], c["ws"], w8)
+        for k, v in dict(X=c["X"], W=c["W"], ws=c["ws"], q=q, a_scale=sc, S=S, C=C).items():
+            out[f"c{i}_{k}"] = v
+        out[f"c{i}_meta"] = np.array([M, N, K, int(w8)], np.int32)
+    np.savez_compressed(os.path.join(HERE, "dense_small.npz"), **out)
+
+    ref_manifest = "/root/reference/prebuilt/gfx1201/macaq_iu8.manifest.toml"
+    if os.path.exists(ref_manifest):
+        import re
+
+        text = open(ref_manifest).read()
+        table = {}
+        for blk in text.split("[[kernel]]")[1:]:
+            name = re.search(r'name = "(\w+)"', blk).group(1)
+            args = re.findall(r'offset = (\d+)\nsize = (\d+)\nvalue_kind = "(\w+)"\nname = "(\w+)"', blk)
+            table[name] = [dict(name=a[3], offset=int(a[0]), size=int(a[1]), value_kind=a[2]) for a in args]
+        json.dump(table, open(os.path.join(HERE, "kernarg_gfx1201.json"), "w"), indent=1, sort_keys=True)
+
+
+if __name__ == "__main__":
+    main()

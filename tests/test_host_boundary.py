@@ -1,0 +1,302 @@
+"""Host side of the drop-in boundary, no GPU: launch law, kernarg packing against the reference's
+committed manifest, manifest <-> code object validation with negative controls, layouts, and that
+the C-ABI library exports every symbol include/saber_iu8.h declares."""
+import ctypes
+import json
+import os
+import re
+import shutil
+import struct
+
+import numpy as np
+import pytest
+
+from oracle import ref
+from saber_engine_amd import iu8, kbuild, synth
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+GOLD = os.path.join(ROOT, "tests", "golden")
+
+
+@pytest.fixture(scope="module", autouse=True)
+def built():
+    if not os.path.exists(iu8.LIB_PATH) or not os.path.exists(os.path.join(iu8.PREBUILT, "macaq_iu8.manifest.toml")):
+        kbuild.build_all()
+
+
+# ------------------------------------------------------------------ the C ABI surface
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "saber_iu8.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    names = sorted(set(re.findall(r"\b(saber_iu8_[a-z0-9_]+)\s*\(", header)))
+    assert len(names) >= 25
+    lib = ctypes.CDLL(iu8.LIB_PATH)
+    missing = [n for n in names if not hasattr(lib, n)]
+    assert not missing, missing
+    assert lib.saber_iu8_abi_version() == 1
+
+
+def test_descriptor_struct_layout_matches_the_header():
+    # sizes the C side and the ctypes mirror must agree on (a drifted mirror corrupts launches)
+    d = iu8.resolve(iu8.W4, 1, 5120, 5120)
+    assert d.kernel == b"macaq_iu8_dec_w4_tm1" and d.op == b"gemm_i4a8" and d.plugin == b"macaq_iu8"
+    assert d.n_args == 10 and d.kernarg_bytes == 68 and d.n_launches == 1 and d.shared_bytes == 0
+    assert [d.args[i].name.decode() for i in range(10)] == ["a", "w", "as", "ws", "decode_partial", "decode_counter", "c", "m", "n", "k"]
+    assert (d.arg("m").ival, d.arg("n").ival, d.arg("k").ival) == (1, 5120, 5120)
+
+
+# ------------------------------------------------------------------ launch law
+
+def test_resolve_refuses_by_name():
+    for bad in [(0, 64, 128), (1, 0, 128), (1, 64, 0), (1, 40, 128), (1, 64, 192)]:
+        with pytest.raises(iu8.IU8Error) as e:
+            iu8.resolve(iu8.W4, *bad)
+        assert e.value.code == iu8.E_RULE
+    with pytest.raises(iu8.IU8Error):
+        iu8.describe("macaq_iu8_dec_w4_tm1", 17, 64, 128)      # 17 rows do not fit one m-tile
+    with pytest.raises(iu8.IU8Error):
+        iu8.describe("macaq_iu8_pf_w4_tn4_lbk64", 256, 256, 256, ks=2)  # the prefill tile does not split
+    with pytest.raises(iu8.IU8Error):
+        iu8.describe("no_such_kernel", 1, 64, 128)
+
+
+@pytest.mark.parametrize("wk,tag", [(iu8.W4, "w4"), (iu8.W8, "w8")])
+def test_decode_band_routing(wk, tag):
+    for m in (1, 4, 8, 16, 17, 32, 33, 48, 49, 64):
+        d = iu8.resolve(wk, m, 5120, 5120)
+        tm = (m + 15) // 16
+        assert d.kernel.decode().startswith(f"macaq_iu8_dec_{tag}_tm{tm}")
+        assert d.ks == 1 and d.grid[2] == 1 and d.n_workspaces == 0
+        assert d.arg("decode_partial").kind == iu8.ARG_NULL_BUFFER and d.arg("decode_counter").kind == iu8.ARG_NULL_BUFFER
+        assert d.grid[0] * (d.block[0] // 64) >= 5120 // 16 // 4       # the grid covers every 16-column tile
+    assert iu8.resolve(wk, 65, 5120, 5120).kernel.decode().startswith(f"macaq_iu8_pf_{tag}")
+
+
+def test_activation_rows_are_staged_when_they_fit():
+    assert iu8.resolve(iu8.W4, 1, 5120, 17408).kernel == b"macaq_iu8_dec_w4_tm1"        # 17 KiB
+    assert iu8.resolve(iu8.W4, 4, 5120, 5120).kernel == b"macaq_iu8_dec_w4_tm1"         # 20 KiB
+    assert iu8.resolve(iu8.W4, 16, 5120, 5120).kernel == b"macaq_iu8_dec_w4_tm1_a80"    # 80 KiB
+    assert iu8.resolve(iu8.W4, 8, 5120, 17408).kernel == b"macaq_iu8_dec_w4_tm1_a0"     # does not fit
+
+
+def test_explicit_split_declares_its_workspaces():
+    d = iu8.describe("macaq_iu8_dec_w4_tm1", 4, 5120, 17408, ks=4)
+    assert d.ks == 4 and d.grid[2] == 4
+    p, c = d.workspace("decode_partial"), d.workspace("decode_counter")
+    assert p.kind == iu8.WS_SCRATCH and p.bytes == 4 * 4 * 5120 * 4 and not p.zero_once
+    assert c.kind == iu8.WS_PERSISTENT and c.bytes == d.grid[0] * 4 and c.zero_once
+    assert d.arg("decode_partial").kind == iu8.ARG_BUFFER
+
+
+def test_prefill_grid_covers_the_output():
+    for (m, n, k) in [(256, 5120, 5120), (2048, 34816, 5120), (300, 304, 640), (8192, 7168, 5120)]:
+        d = iu8.resolve(iu8.W4, m, n, k)
+        name = d.kernel.decode()
+        bm, bn = (256, 256) if name.endswith("tn4_lbk64") else (128, 128)
+        assert d.grid[0] == -(-n // bn) and d.grid[1] == -(-m // bm) and d.grid[2] == 1 and d.block[0] == 256
+
+
+# ------------------------------------------------------------------ kernarg ABI
+
+def test_signatures_pack_exactly_like_the_reference_manifest():
+    table = json.load(open(os.path.join(GOLD, "kernarg_gfx1201.json")))
+    checked = 0
+    for name, args in table.items():
+        slots, nbytes = iu8.signature(name)
+        assert [(s[0], s[1], s[2]) for s in slots] == [(a["name"], a["offset"], a["size"]) for a in args], name
+        assert [("global_buffer" if s[3] == iu8.ARG_BUFFER else "by_value") for s in slots] == [a["value_kind"] for a in args]
+        assert nbytes == max(a["offset"] + a["size"] for a in args)
+        checked += 1
+    assert checked == 10
+
+
+def test_kernarg_image_built_two_ways_is_byte_identical():
+    d = iu8.describe("macaq_iu8_dec_w4_tm1", 3, 5120, 17408, ks=2)
+    bufs = dict(a=0x7F0000001000, w=0x7F0000002000, ws=0x7F0000004000, decode_partial=0x7F0000005000,
+                decode_counter=0x7F0000006000, c=0x7F0000007000)
+    bufs["as"] = 0x7F0000003000
+    img = iu8.pack_kernarg(d, bufs)
+    want = struct.pack("<7Q3i", bufs["a"], bufs["w"], bufs["as"], bufs["ws"], bufs["decode_partial"], bufs["decode_counter"],
+                       bufs["c"], 3, 5120, 17408)
+    assert img == want and len(img) == 68
+    # ks == 1: the workspace pointers are written as NULL whatever is bound
+    d1 = iu8.resolve(iu8.W4, 3, 5120, 17408)
+    img1 = iu8.pack_kernarg(d1, bufs)
+    assert img1[32:48] == b"\0" * 16 and img1[:32] == want[:32]
+    # a missing or NULL binding is refused, not packed
+    del bufs["ws"]
+    with pytest.raises(iu8.IU8Error) as e:
+        iu8.pack_kernarg(d, bufs)
+    assert e.value.code == iu8.E_ARG
+    bufs["ws"] = 0
+    with pytest.raises(iu8.IU8Error):
+        iu8.pack_kernarg(d, bufs)
+
+
+# ------------------------------------------------------------------ manifests and code objects
+
+def _copy_plugin(tmp_path, stem="macaq_iu8"):
+    for ext in (".hsaco", ".manifest.toml"):
+        shutil.copy(os.path.join(iu8.PREBUILT, stem + ext), tmp_path / (stem + ext))
+    return str(tmp_path / (stem + ".manifest.toml"))
+
+
+def test_every_built_manifest_validates_against_its_code_object():
+    ms = [f for f in os.listdir(iu8.PREBUILT) if f.endswith(".manifest.toml")]
+    assert {"macaq_iu8.manifest.toml", "macaq_i8q.manifest.toml"} <= set(ms)
+    for f in ms:
+        rc, refusal, msg = iu8.manifest_validate(os.path.join(iu8.PREBUILT, f))
+        assert rc == 0 and refusal == 0, msg
+        text = open(os.path.join(iu8.PREBUILT, f)).read()
+        assert 'arch = "gfx950"' in text and "wavefront_size = 64" in text and "wavefront_size = 32" not in text
+        assert "private_segment_fixed_size = 0" in text
+
+
+def test_reference_symbols_and_lds_budget():
+    text = open(os.path.join(iu8.PREBUILT, "macaq_iu8.manifest.toml")).read()
+    for name in json.load(open(os.path.join(GOLD, "kernarg_gfx1201.json"))):
+        assert f'name = "{name}"' in text and f'symbol = "{name}.kd"' in text
+    assert max(int(v) for v in re.findall(r"group_segment_fixed_size = (\d+)", text)) <= 160 * 1024
+    # no kernel of the shipped objects spills to scratch
+    assert set(re.findall(r"private_segment_fixed_size = (\d+)", text)) == {"0"}
+
+
+@pytest.mark.parametrize("edit,counter", [
+    (("offset = 56", "offset = 60", 1), iu8.REFUSED_KERNARG),                  # a drifted kernarg offset
+    (("wavefront_size = 64", "wavefront_size = 32", 1), iu8.REFUSED_WAVE),       # mixed wave sizes in one plugin
+    (("group_segment_fixed_size = ", "group_segment_fixed_size = 1", 1), iu8.REFUSED_METADATA),  # LDS drift
+    (("hsaco_sha256 = \"", "hsaco_sha256 = \"0", 1), iu8.REFUSED_METADATA),       # another build's blob
+    (("arch = \"gfx950\"", "arch = \"gfx1201\"", 1), iu8.REFUSED_METADATA),
+])
+def test_drifted_manifest_is_refused_with_the_right_counter(tmp_path, edit, counter):
+    path = _copy_plugin(tmp_path)
+    text = open(path).read()
+    assert edit[0] in text
+    open(path, "w").write(text.replace(edit[0], edit[1], edit[2]))
+    rc, refusal, msg = iu8.manifest_validate(path, arch="gfx950")
+    assert rc == iu8.E_VALIDATE and refusal == counter, (rc, refusal, msg)
+
+
+def test_tampered_code_object_is_refused(tmp_path):
+    path = _copy_plugin(tmp_path)
+    blob = bytearray(open(tmp_path / "macaq_iu8.hsaco", "rb").read())
+    blob[len(blob) // 2] ^= 0xFF
+    open(tmp_path / "macaq_iu8.hsaco", "wb").write(bytes(blob))
+    rc, refusal, _ = iu8.manifest_validate(path)
+    assert rc in (iu8.E_VALIDATE, iu8.E_PARSE)
+
+
+def test_schema_version_and_garbage_are_parse_errors(tmp_path):
+    path = _copy_plugin(tmp_path)
+    text = open(path).read()
+    open(path, "w").write(text.replace("schema_version = 1", "schema_version = 2"))
+    assert iu8.manifest_validate(path)[0] == iu8.E_PARSE
+    open(path, "w").write("this is not a manifest")
+    assert iu8.manifest_validate(path)[0] == iu8.E_PARSE
+    assert iu8.manifest_validate(str(tmp_path / "absent.manifest.toml"))[0] == iu8.E_IO
+
+
+def test_source_ladder():
+    assert kbuild.candidates("macaq_iu8", "gfx950") == ["macaq_iu8.gfx950.hip", "macaq_iu8.gfx95.hip", "macaq_iu8.hip"]
+    assert kbuild.candidates("k", "gfx1201") == ["k.gfx1201.hip", "k.gfx12.hip", "k.hip"]
+    assert kbuild.resolve_source("macaq_iu8").endswith("macaq_iu8.gfx950.hip")
+    assert kbuild.resolve_source("no_such_kernel") is None
+
+
+def test_open_without_a_gpu_fails_loudly():
+    import torch
+
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    with pytest.raises(iu8.IU8Error) as e:
+        iu8.Context()
+    assert e.value.code == iu8.E_HIP and "no CPU fallback" in str(e.value)
+
+
+# ------------------------------------------------------------------ operand orders
+
+def test_a_order_is_a_bijection_with_16_byte_lane_pieces():
+    L = iu8.lib()
+    M, K = 32, 256
+    offs = np.array([[L.saber_iu8_a_offset(m, k, K) for k in range(K)] for m in range(M)])
+    assert sorted(offs.ravel().tolist()) == list(range(M * K))
+    # lane l of fragment (mt, kt): row mt*16 + l%16, k = kt*64 + (l/16)*16 + 0..15
+    for (m, k) in [(0, 0), (5, 17), (17, 130), (31, 255)]:
+        mt, kt, lane = m // 16, k // 64, (m % 16) + 16 * ((k % 64) // 16)
+        assert offs[m, k] == (mt * (K // 64) + kt) * 1024 + lane * 16 + k % 16
+    rng = np.random.default_rng(0)
+    a = rng.integers(-127, 128, (21, K), dtype=np.int8)
+    frag = iu8.repack_a(a)
+    assert frag.size == 32 * K == iu8.a_bytes(21, K)
+    np.testing.assert_array_equal(iu8.unpack_a(frag, 21, K), a)
+    assert frag.view(np.int8)[offs[7, 33]] == a[7, 33]
+
+
+def test_w4_order_unpacks_to_natural_k_order():
+    L = iu8.lib()
+    N, K = 32, 256
+    rng = np.random.default_rng(1)
+    codes = rng.integers(-8, 8, (N, K), dtype=np.int8)
+    frag = iu8.repack_w4(synth.pack_w4(codes))
+    seen = set()
+    for n in range(N):
+        for k in range(K):
+            hi = ctypes.c_uint32()
+            off = L.saber_iu8_w4_offset(n, k, K, ctypes.byref(hi))
+            seen.add((off, hi.value))
+            nib = (int(frag[off]) >> 4) if hi.value else (int(frag[off]) & 15)
+            assert (nib - 16 if nib >= 8 else nib) == codes[n, k]
+    assert len(seen) == N * K
+    # the device unpack: lo = (d << 4) & 0xF0F0F0F0, hi = d & 0xF0F0F0F0 of lane l's dwords d0..d3 gives
+    # int8 = 16 * code for k = kt*128 + s*64 + (l/16)*16 + 0..15 in order, s = 0 (d0,d1) and 1 (d2,d3)
+    d = frag.view(np.uint32).reshape(N // 16, K // 128, 64, 4)
+    for (nt, kt, lane) in [(0, 0, 0), (1, 1, 37), (0, 1, 63)]:
+        for s in (0, 1):
+            regs = []
+            for j in (2 * s, 2 * s + 1):
+                dj = int(d[nt, kt, lane, j])
+                regs += [(dj << 4) & 0xF0F0F0F0, dj & 0xF0F0F0F0]
+            vals = np.array(regs, np.uint32).view(np.int8)
+            k0 = kt * 128 + s * 64 + (lane // 16) * 16
+            np.testing.assert_array_equal(vals, 16 * codes[nt * 16 + lane % 16, k0:k0 + 16])
+
+
+def test_reference_gfx12_orders_reorder_to_the_same_bytes():
+    # build the reference's fragment orders from the canonical form with the oracle's address
+    # functions, then let the library re-order them: the result must equal the direct repack
+    L = ref.lib()
+    N, K = 32, 256
+    rng = np.random.default_rng(4)
+    codes = rng.integers(-8, 8, (N, K), dtype=np.int8)
+    f12 = np.zeros(N * K // 2, np.uint8)
+    seen = set()
+    for n in range(N):
+        for k in range(K):
+            nib = ctypes.c_uint32()
+            off = L.w4a8_w4_frag_gfx12(n, k, K, ctypes.byref(nib))
+            seen.add((off, nib.value))
+            f12[off] |= (int(codes[n, k]) & 15) << (4 * nib.value)
+    assert len(seen) == N * K
+    out = np.empty_like(f12)
+    assert iu8.lib().saber_iu8_repack_w4_from_gfx12(f12.ctypes.data_as(ctypes.c_void_p), N, K, out.ctypes.data_as(ctypes.c_void_p)) == 0
+    np.testing.assert_array_equal(out, iu8.repack_w4(synth.pack_w4(codes)))
+    w8 = rng.integers(-127, 128, (N, K), dtype=np.int8)
+    g12 = np.zeros(N * K, np.uint8)
+    offs = set()
+    for n in range(N):
+        for k in range(K):
+            off = L.w4a8_a_tiled_gfx12(n, k, K)
+            offs.add(off)
+            g12[off] = w8[n, k].view(np.uint8)
+    assert offs == set(range(N * K))
+    out8 = np.empty_like(g12)
+    assert iu8.lib().saber_iu8_repack_w8_from_gfx12(g12.ctypes.data_as(ctypes.c_void_p), N, K, out8.ctypes.data_as(ctypes.c_void_p)) == 0
+    np.testing.assert_array_equal(out8, iu8.repack_w8(w8))
+
+
+def test_repack_refuses_ragged_shapes():
+    with pytest.raises(iu8.IU8Error):
+        iu8.repack_w4(np.zeros((24, 64), np.uint8))
+    with pytest.raises(iu8.IU8Error):
+        iu8.repack_w8(np.zeros((16, 192), np.int8))
