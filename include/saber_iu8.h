@@ -222,6 +222,62 @@ int saber_iu8_gemm(saber_iu8_ctx *ctx, int wkind, const void *a, const float *as
 int saber_iu8_gemm_acc(saber_iu8_ctx *ctx, int wkind, const void *a, const void *w, int32_t *acc, uint32_t m,
                        uint32_t n, uint32_t k, void *stream);
 
+/* ------------------------------------------------------------------ routed experts (MoE) */
+
+/* The reference has no iu8 MoE; these entry points compose its routing / tile / combine law
+ * (crates/saber-kernels/hip/moe_route.hip, crates/saber-kernels/src/moe.rs) with the iu8 GEMM at
+ * 128 experts, top-8 (the one router symbol this build ships: other widths are refused). */
+
+/* Geometry caps (crates/saber-kernels/src/moe.rs:691-708), no shared expert. */
+uint32_t saber_iu8_moe_rows_cap(uint32_t tokens, uint32_t topk, uint32_t experts);
+uint32_t saber_iu8_moe_tiles_cap(uint32_t tokens, uint32_t topk, uint32_t experts, uint32_t tile_blocks);
+/* tile_blocks the grouped law picks for `tokens`: 1 (16-row tiles, weight-streaming cells) while an
+ * expert averages <= 16 routes, 8 (128-row MFMA tiles) above. */
+uint32_t saber_iu8_moe_tile_blocks(uint32_t tokens, uint32_t topk, uint32_t experts);
+
+/* Device buffers of one routed layer, named as the router kernel's arguments
+ * (crates/saber-kernels/src/abi.rs:354-374); all caller-owned. */
+typedef struct {
+  int32_t *topk_ids;    /* [T * topk] */
+  float *topk_w;        /* [T * topk] */
+  int32_t *route_pos;   /* [T * topk] */
+  int32_t *row_tok;     /* [rows_cap] */
+  int32_t *row_route;   /* [rows_cap] */
+  int32_t *tile_expert; /* [tiles_cap] */
+  int32_t *tile_row0;   /* [tiles_cap] */
+  int32_t *tile_rows;   /* [tiles_cap] */
+  int32_t *expert_cnt;  /* [experts] */
+  int32_t *meta;        /* [8]: [0] tiles, [1] rows, [3] routes, [4] experts touched */
+  int32_t *blk_cnt;     /* [ceil(T / 32) * experts]  scratch */
+  int32_t *rank;        /* [T * topk]                scratch */
+  int32_t *arrive;      /* [1]  persistent: zeroed once by the caller, left zero */
+} saber_iu8_moe_tables;
+
+/* Router + expert-major sort + tile table, one launch. logits bf16 [T, experts]. */
+int saber_iu8_moe_route(saber_iu8_ctx *ctx, const void *logits_bf16, uint32_t tokens, uint32_t experts, uint32_t topk,
+                        uint32_t tile_blocks, const saber_iu8_moe_tables *t, void *stream);
+
+/* Grouped W4 GEMM over the tile table: per tile the expert's weights (gfx950 W4 fragments) at
+ * xptr[2e] and f32 row scales at xptr[2e + 1] (device array of 2 * experts addresses); A rows
+ * gathered through row_tok (gather != 0: a / as are token-major) or in place (a / as are
+ * expert-major); C bf16 [rows_cap, n]. tile_blocks as given to the router. */
+int saber_iu8_moe_grouped(saber_iu8_ctx *ctx, const void *a, const float *as, const void *xptr, void *c_bf16, uint32_t n,
+                          uint32_t k, int gather, uint32_t tokens, uint32_t experts, uint32_t topk, uint32_t tile_blocks,
+                          const saber_iu8_moe_tables *t, void *stream);
+
+/* SiLU(gate)*up + requant over the live expert-major rows: gu bf16 [rows_cap, 2n] -> q (A edge of
+ * rows_cap rows), scale f32 [rows_cap]. Pad rows are skipped. */
+int saber_iu8_moe_silu_mul_quant(saber_iu8_ctx *ctx, const void *gu_bf16, void *q, float *scale, uint32_t n,
+                                 uint32_t rows_cap, const saber_iu8_moe_tables *t, void *stream);
+
+/* Weighted combine: out[t] = bf16(sum_k w[t,k] * Y[pos(t,k)]) in top-k order; y bf16 [rows_cap, h]. */
+int saber_iu8_moe_combine(saber_iu8_ctx *ctx, const void *y_bf16, const saber_iu8_moe_tables *t, void *out_bf16,
+                          uint32_t tokens, uint32_t topk, uint32_t h, void *stream);
+
+/* bf16 silu of every bf16 bit pattern as the device computes it: out u16 [65536] (device). The
+ * parity suite compares it with the host formula for all 65,536 inputs. */
+int saber_iu8_silu_table(saber_iu8_ctx *ctx, void *out_u16, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -64,6 +64,10 @@ void set_i32(saber_iu8_desc *d, const char *name, int64_t v) {
       d->args[i].ival = v;
     }
 }
+void set_buffer(saber_iu8_desc *d, const char *name) {
+  for (uint32_t i = 0; i < d->n_args; ++i)
+    if (!strcmp(d->args[i].name, name)) d->args[i].kind = SABER_IU8_ARG_BUFFER;
+}
 void set_null(saber_iu8_desc *d, const char *name) {
   for (uint32_t i = 0; i < d->n_args; ++i)
     if (!strcmp(d->args[i].name, name)) d->args[i].kind = SABER_IU8_ARG_NULL_BUFFER;
@@ -203,7 +207,11 @@ int resolve_quant(uint32_t m, uint32_t k, saber_iu8_desc *out) {
 }
 
 int resolve_silu_mul_quant(uint32_t rows, uint32_t n, saber_iu8_desc *out) {
-  return describe_rows("silu_mul_quant_i8", "macaq_i8_silu_mul_quant_t256", rows, n, "n", out);
+  if (int rc = describe_rows("silu_mul_quant_i8", "macaq_i8_silu_mul_quant_t256", rows, n, "n", out)) return rc;
+  // the dense form has no row map; the routed form binds both (set_buffer)
+  set_null(out, "row_tok");
+  set_null(out, "meta");
+  return 0;
 }
 
 }  // namespace iu8

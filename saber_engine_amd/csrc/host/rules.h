@@ -42,5 +42,6 @@ int resolve_silu_mul_quant(uint32_t rows, uint32_t n, saber_iu8_desc *out);
 int fill_slots(const std::string &kernel, saber_iu8_desc *d);
 void set_i32(saber_iu8_desc *d, const char *name, int64_t v);
 void set_null(saber_iu8_desc *d, const char *name);
+void set_buffer(saber_iu8_desc *d, const char *name);
 
 }  // namespace iu8

@@ -353,4 +353,106 @@ int saber_iu8_gemm_acc(saber_iu8_ctx *ctx, int wkind, const void *a, const void 
   return launch_gemm(ctx, d, a, (const float *)acc, w, (const float *)acc, acc, nullptr, nullptr, stream);
 }
 
+// ---------------------------------------------------------------------------- routed experts
+
+uint32_t saber_iu8_moe_rows_cap(uint32_t tokens, uint32_t topk, uint32_t experts) {
+  const uint32_t r = tokens * topk;
+  return r + 15u * std::min(r, experts);
+}
+uint32_t saber_iu8_moe_tiles_cap(uint32_t tokens, uint32_t topk, uint32_t experts, uint32_t tile_blocks) {
+  const uint32_t r = tokens * topk;
+  return std::min(r, experts) + r / (16u * std::max(tile_blocks, 1u)) + 1u;
+}
+uint32_t saber_iu8_moe_tile_blocks(uint32_t tokens, uint32_t topk, uint32_t experts) {
+  return (uint64_t)tokens * topk <= 16ull * experts ? 1u : 8u;
+}
+
+static int moe_check(const char *what, uint32_t tokens, uint32_t experts, uint32_t topk, const saber_iu8_moe_tables *t) {
+  if (!t) return fail(SABER_IU8_E_ARG, std::string(what) + ": null tables");
+  if (experts != 128 || topk != 8)
+    return fail(SABER_IU8_E_RULE, fmt("%s: %u experts / top-%u; this object ships the 128-expert top-8 router", what, experts, topk));
+  if (tokens == 0) return fail(SABER_IU8_E_RULE, std::string(what) + ": no tokens; an empty launch is a caller bug");
+  return 0;
+}
+
+static int raw_desc(const char *kernel, uint32_t gx, uint32_t gy, uint32_t block, saber_iu8_desc *d) {
+  const uint32_t grid[3] = {gx, gy, 1};
+  return saber_iu8_describe_raw(kernel, "moe_iu8", grid, block, d);
+}
+
+int saber_iu8_moe_route(saber_iu8_ctx *ctx, const void *logits, uint32_t tokens, uint32_t experts, uint32_t topk,
+                        uint32_t tile_blocks, const saber_iu8_moe_tables *t, void *stream) {
+  if (int rc = moe_check("moe_route", tokens, experts, topk, t)) return rc;
+  if (tile_blocks == 0) return fail(SABER_IU8_E_RULE, "moe_route: tile_blocks 0");
+  saber_iu8_desc d;
+  if (int rc = raw_desc("moe_iu8_route_topk8_sort_e128", (tokens + 31) / 32, 1, 256, &d)) return rc;
+  set_i32(&d, "t", tokens);
+  set_i32(&d, "e_lo", 0);
+  set_i32(&d, "e_loc", experts);
+  set_i32(&d, "tile_blocks", tile_blocks);
+  set_i32(&d, "with_shared", 0);
+  const saber_iu8_binding b[] = {{"logits", (void *)logits},      {"topk_ids", t->topk_ids},   {"topk_w", t->topk_w},
+                                 {"route_pos", t->route_pos},     {"row_tok", t->row_tok},     {"row_route", t->row_route},
+                                 {"tile_expert", t->tile_expert}, {"tile_row0", t->tile_row0}, {"tile_rows", t->tile_rows},
+                                 {"expert_cnt", t->expert_cnt},   {"meta", t->meta},           {"blk_cnt", t->blk_cnt},
+                                 {"rank", t->rank},               {"arrive", t->arrive}};
+  return saber_iu8_launch(ctx, &d, b, sizeof b / sizeof b[0], stream);
+}
+
+int saber_iu8_moe_grouped(saber_iu8_ctx *ctx, const void *a, const float *as, const void *xptr, void *c, uint32_t n,
+                          uint32_t k, int gather, uint32_t tokens, uint32_t experts, uint32_t topk, uint32_t tile_blocks,
+                          const saber_iu8_moe_tables *t, void *stream) {
+  if (int rc = moe_check("moe_grouped", tokens, experts, topk, t)) return rc;
+  if (n == 0 || k == 0 || n % 16 != 0 || k % 128 != 0)
+    return fail(SABER_IU8_E_RULE, fmt("moe_grouped: N=%u must be a multiple of 16 (whole fragments) and K=%u of 128 (the slab)", n, k));
+  if (tile_blocks != 1 && tile_blocks != 8)
+    return fail(SABER_IU8_E_RULE, fmt("moe_grouped: tile_blocks %u; the cells are 1 (16-row) and 8 (128-row)", tile_blocks));
+  const bool dec = tile_blocks == 1;
+  const std::string name = fmt("moe_iu8_grouped_w4_%s_g%d", dec ? "dec" : "pf", gather ? 1 : 0);
+  const uint32_t bn = dec ? 32 : 128, block = dec ? 512 : 256;
+  saber_iu8_desc d;
+  if (int rc = raw_desc(name.c_str(), (n + bn - 1) / bn, saber_iu8_moe_tiles_cap(tokens, topk, experts, tile_blocks), block, &d)) return rc;
+  set_i32(&d, "n", n);
+  set_i32(&d, "k", k);
+  set_i32(&d, "pmax", 0);
+  set_null(&d, "p");
+  set_null(&d, "cnt");
+  const saber_iu8_binding b[] = {{"a", (void *)a},           {"xptr", (void *)xptr},         {"tile_expert", t->tile_expert},
+                                 {"tile_row0", t->tile_row0}, {"tile_rows", t->tile_rows},   {"row_tok", t->row_tok},
+                                 {"meta", t->meta},           {"as", (void *)as},            {"c", c}};
+  return saber_iu8_launch(ctx, &d, b, sizeof b / sizeof b[0], stream);
+}
+
+int saber_iu8_moe_silu_mul_quant(saber_iu8_ctx *ctx, const void *gu, void *q, float *scale, uint32_t n, uint32_t rows_cap,
+                                 const saber_iu8_moe_tables *t, void *stream) {
+  if (!t) return fail(SABER_IU8_E_ARG, "moe_silu_mul_quant: null tables");
+  saber_iu8_desc d;
+  if (int rc = resolve_silu_mul_quant(rows_cap, n, &d)) return rc;
+  set_buffer(&d, "row_tok");
+  set_buffer(&d, "meta");
+  const saber_iu8_binding b[] = {{"gu", (void *)gu}, {"q", q}, {"scale", scale}, {"row_tok", t->row_tok}, {"meta", t->meta}};
+  return saber_iu8_launch(ctx, &d, b, 5, stream);
+}
+
+int saber_iu8_moe_combine(saber_iu8_ctx *ctx, const void *y, const saber_iu8_moe_tables *t, void *out, uint32_t tokens,
+                          uint32_t topk, uint32_t h, void *stream) {
+  if (!t) return fail(SABER_IU8_E_ARG, "moe_combine: null tables");
+  if (topk != 8) return fail(SABER_IU8_E_RULE, fmt("moe_combine: top-%u; this object ships top-8", topk));
+  if (tokens == 0 || h == 0 || h % 8 != 0) return fail(SABER_IU8_E_RULE, fmt("moe_combine: %u tokens of width %u (a multiple of 8)", tokens, h));
+  saber_iu8_desc d;
+  if (int rc = raw_desc("moe_iu8_combine_bf16", tokens, 1, 256, &d)) return rc;
+  set_i32(&d, "h", h);
+  set_null(&d, "sgate");
+  const saber_iu8_binding b[] = {{"y", (void *)y}, {"topk_w", t->topk_w}, {"route_pos", t->route_pos}, {"meta", t->meta}, {"out", out}};
+  return saber_iu8_launch(ctx, &d, b, 5, stream);
+}
+
+int saber_iu8_silu_table(saber_iu8_ctx *ctx, void *out, void *stream) {
+  saber_iu8_desc d;
+  const uint32_t grid[3] = {256, 1, 1};
+  if (int rc = saber_iu8_describe_raw("macaq_silu_bf16_table", "macaq_i8q", grid, 256, &d)) return rc;
+  const saber_iu8_binding b[] = {{"out", out}};
+  return saber_iu8_launch(ctx, &d, b, 1, stream);
+}
+
 }  // extern "C"

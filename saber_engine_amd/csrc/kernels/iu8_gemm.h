@@ -1,0 +1,420 @@
+// The two GEMM bodies of the gfx950 W4A8-iu8 path, shared by the dense code object (`macaq_iu8`)
+// and the grouped, expert-routed one (`moe_iu8`). Operand orders and the contract: iu8_common.h.
+//
+// Both bodies see the rows they work on through an `iu8_rows` map: a dense launch owns rows
+// [0, M) of A / as / C; a grouped launch owns, per tile of the router's tile table, `rows` rows of
+// one expert starting at expert-major row `row0`, whose activations are either those rows of a
+// compact A (down projection) or gathered through `row_tok` from the token-major A (gate+up),
+// the reference's schedule (crates/saber-kernels/hip/moe_grouped.hip:33-120). Rows past the live
+// ones are clamped, never predicated, and never stored.
+#pragma once
+#include "iu8_common.h"
+
+struct iu8_rows {
+  const int *row_tok;  // gather map: expert-major row -> row of A and `as`; nullptr = in place
+  int row0;            // first row (a multiple of 16) of the tile in C and in a compact A
+  int rows;            // live rows from row0
+};
+// The row of A (and of `as`) behind tile-local row m.
+static __device__ __forceinline__ int iu8_arow(const iu8_rows &R, int m) {
+  if (R.row_tok != nullptr) return max(R.row_tok[R.row0 + min(m, R.rows - 1)], 0);
+  return R.row0 + min(m, ((R.rows + 15) & ~15) - 1);
+}
+
+// ============================================================================ decode band
+template <int TM, bool W8, int NT, int KW, int WPB, int D, int ALDS, bool ACC>
+__device__ __forceinline__ void iu8_dec_body(const iu8_u8 *__restrict__ A, const iu8_u8 *__restrict__ W,
+                                             const float *__restrict__ as, const float *__restrict__ ws,
+                                             int *__restrict__ P, int *__restrict__ cnt, void *__restrict__ Cv,
+                                             const iu8_rows R, int N, int K) {
+  const int M = R.rows;
+  static_assert(WPB % KW == 0, "k-waves divide the workgroup");
+  static_assert(ALDS == 0 || TM == 1, "LDS staging of A is the M <= 16 form");
+  constexpr int WN = WPB / KW;
+  constexpr int NTHR = WPB * 64;
+  constexpr int WSTEP = W8 ? 2048 : 1024;  // bytes of one 16-row weight tile per 128-deep K step
+  constexpr int WV = W8 ? 2 : 1;           // 16-byte loads a lane per step per tile
+  constexpr int BN = WN * NT * 16;         // columns a workgroup
+  constexpr int RED = (KW > 1 ? KW - 1 : 1) * WN * TM * NT * 1024;
+  constexpr int ABYTES = ALDS * 1024;
+  // one LDS block: the staged activation rows, re-used for the k-waves' partials at the end
+  __shared__ __attribute__((aligned(16))) iu8_u8 s_mem[ABYTES > RED ? ABYTES : RED];
+  __shared__ int s_last;
+  int *s_red = (int *)s_mem;
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wk = wave % KW, wn = wave / KW;
+  const int ntiles = N >> 4, steps = K >> 7, ktiles = K >> 6;
+  const int Z = gridDim.z, z = blockIdx.z;
+  const int spb = (steps + Z - 1) / Z;
+  const int s_lo = z * spb, s_hi = min(steps, s_lo + spb);
+  const int nt0 = (blockIdx.x * WN + wn) * NT;
+  const int ml = lane & 15, lg = lane >> 4;
+  // this wave's steps: s_lo + wk + t*KW, t in [0, T)
+  const int T = s_lo + wk < s_hi ? (s_hi - s_lo - wk + KW - 1) / KW : 0;
+
+  const iu8_u8 *wp[NT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j) {
+    const int ntj = min(nt0 + j, ntiles - 1);  // a tile past N re-reads the last one and stores nothing
+    wp[j] = W + ((size_t)ntj * steps + s_lo + wk) * WSTEP + lane * 16;
+  }
+
+  iu8_v4i acc[TM][NT];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < NT; ++j) acc[i][j] = iu8_v4i{0, 0, 0, 0};
+
+  // ---- LDS staging of the live activation rows (issued before the weight ring, waited after it)
+  // MR = staged rows (a power of two >= M); piece p = ((kt*4 + g)*MR + r) holds row r's 16 bytes
+  // of k = (2*s_lo + kt)*64 + g*16.
+  bool staged = false;
+  int mr_shift = 0;
+  constexpr int A_PER = ALDS ? (ABYTES / 16 + NTHR - 1) / NTHR : 1;
+  constexpr bool A_INREG = A_PER <= 8;
+  iu8_v4u areg[A_INREG ? A_PER : 1];
+  int a_pieces = 0;
+  if constexpr (ALDS > 0) {
+    while ((1 << mr_shift) < M) ++mr_shift;
+    a_pieces = ((s_hi - s_lo) * 2 * 4) << mr_shift;
+    staged = M <= 16 && a_pieces * 16 <= ABYTES;
+    if (staged) {
+      auto a_src = [&](int piece) {
+        const int r = piece & ((1 << mr_shift) - 1), g = (piece >> mr_shift) & 3, kt = piece >> (mr_shift + 2);
+        const int ar = iu8_arow(R, r);
+        return (const iu8_v4u *)(A + (((size_t)(ar >> 4) * ktiles + 2 * s_lo + kt) * 1024 + ((ar & 15) + 16 * g) * 16));
+      };
+      if constexpr (A_INREG) {  // few pieces a thread: loads now, LDS stores behind the first weight ring
+#pragma unroll
+        for (int p = 0; p < A_PER; ++p)
+          if (p * NTHR + tid < a_pieces) areg[p] = *a_src(p * NTHR + tid);
+      } else {                  // many: copy before the ring starts
+        for (int piece = tid; piece < a_pieces; piece += NTHR) *(iu8_v4u *)&s_mem[piece * 16] = *a_src(piece);
+      }
+    }
+  }
+
+  // ---- the weight ring
+  iu8_v4u ring[D][NT][WV];
+  iu8_v4i ringa[ALDS ? 1 : D][TM][2];  // direct-from-L2 activation operands when not staged
+  bool live[TM];
+#pragma unroll
+  for (int i = 0; i < TM; ++i) live[i] = i * 16 + ml < M;
+  const iu8_u8 *ap[TM];  // this lane's row of every activation tile, at the wave's first K step
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const int ar = iu8_arow(R, i * 16 + ml);
+    ap[i] = A + ((size_t)(ar >> 4) * ktiles + (size_t)(s_lo + wk) * 2) * 1024 + ((ar & 15) + 16 * lg) * 16;
+  }
+  auto issue = [&](int slot, int t) {
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int v = 0; v < WV; ++v) ring[slot][j][v] = iu8_ldg_nt(wp[j] + (size_t)t * (KW * WSTEP) + v * 1024);
+    if (!staged) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          ringa[ALDS ? 0 : slot][i][h] = iu8_v4i{0, 0, 0, 0};
+          if (live[i])
+            ringa[ALDS ? 0 : slot][i][h] =
+                *(const iu8_v4i *)(ap[i] + ((size_t)t * (2 * KW) + h) * 1024);
+        }
+    }
+  };
+  const int a_lane = (((lg << mr_shift) + min(ml, (1 << mr_shift) - 1)) << 4);
+  auto consume = [&](int slot, int t) {
+    iu8_v4i a0[TM], a1[TM];
+    if (ALDS > 0 && staged) {
+      const int kt = 2 * (wk + t * KW);
+      a0[0] = *(const iu8_v4i *)&s_mem[((kt * 4) << (mr_shift + 4)) + a_lane];
+      a1[0] = *(const iu8_v4i *)&s_mem[(((kt + 1) * 4) << (mr_shift + 4)) + a_lane];
+    } else {
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        a0[i] = ringa[ALDS ? 0 : slot][i][0];
+        a1[i] = ringa[ALDS ? 0 : slot][i][1];
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+      iu8_v4i w0, w1;
+      if constexpr (W8) {
+        w0 = (iu8_v4i)ring[slot][j][0];
+        w1 = (iu8_v4i)ring[slot][j][WV - 1];
+      } else {
+        iu8_unpack_w4(ring[slot][j][0], w0, w1);
+      }
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        acc[i][j] = iu8_mfma(w0, a0[i], acc[i][j]);
+        acc[i][j] = iu8_mfma(w1, a1[i], acc[i][j]);
+      }
+    }
+  };
+
+  if constexpr (ALDS > 0) {
+    // staged form: the ring never holds activations, so the not-staged fallback of an ALDS kernel
+    // (shape too large for its LDS) loads them at consume time through the one-slot `ringa`
+    if (!staged) {
+      for (int t = 0; t < T; ++t) {
+        issue(0, t);
+        consume(0, t);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < D; ++i)
+        if (i < T) issue(i, i);
+      if constexpr (A_INREG) {
+#pragma unroll
+        for (int p = 0; p < A_PER; ++p)
+          if (p * NTHR + tid < a_pieces) *(iu8_v4u *)&s_mem[(p * NTHR + tid) * 16] = areg[p];
+      }
+      __syncthreads();
+      int t0 = 0;
+      for (; t0 + 2 * D <= T; t0 += D) {  // steady state: every slot consumed and re-issued
+#pragma unroll
+        for (int i = 0; i < D; ++i) {
+          consume(i, t0 + i);
+          issue(i, t0 + i + D);
+        }
+      }
+      for (; t0 < T; t0 += D) {  // drain
+#pragma unroll
+        for (int i = 0; i < D; ++i)
+          if (t0 + i < T) {
+            consume(i, t0 + i);
+            if (t0 + i + D < T) issue(i, t0 + i + D);
+          }
+      }
+      __syncthreads();  // every wave is done with the staged rows before s_mem holds partials
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < D; ++i)
+      if (i < T) issue(i, i);
+    int t0 = 0;
+    for (; t0 + 2 * D <= T; t0 += D) {
+#pragma unroll
+      for (int i = 0; i < D; ++i) {
+        consume(i, t0 + i);
+        issue(i, t0 + i + D);
+      }
+    }
+    for (; t0 < T; t0 += D) {
+#pragma unroll
+      for (int i = 0; i < D; ++i)
+        if (t0 + i < T) {
+          consume(i, t0 + i);
+          if (t0 + i + D < T) issue(i, t0 + i + D);
+        }
+    }
+  }
+
+  // ---- the k-waves' partials meet in LDS (exact int32 adds)
+  if constexpr (KW > 1) {
+    if (wk > 0) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+          *(iu8_v4i *)&s_red[((((wk - 1) * WN + wn) * TM + i) * NT + j) * 256 + lane * 4] = acc[i][j];
+    }
+    __syncthreads();
+    if (wk == 0) {
+#pragma unroll
+      for (int q = 0; q < KW - 1; ++q)
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < NT; ++j)
+            acc[i][j] += *(const iu8_v4i *)&s_red[(((q * WN + wn) * TM + i) * NT + j) * 256 + lane * 4];
+    }
+  }
+
+  const int nq = lg * 4;
+  if (Z == 1) {
+    if (wk != 0) return;
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+      if (nt0 + j >= ntiles) continue;
+      const int n = (nt0 + j) * 16 + nq;
+      float wsu[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) wsu[r] = iu8_wsu<W8>(ws, n + r);
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        const int m = i * 16 + ml;
+        if (m >= M) continue;
+        const size_t crow = (size_t)(R.row0 + m) * N;
+        if constexpr (ACC) {
+          *(iu8_v4i *)((int *)Cv + crow + n) = acc[i][j];
+        } else {
+          const float am = as[iu8_arow(R, m)];
+          unsigned h[4];
+#pragma unroll
+          for (int r = 0; r < 4; ++r) h[r] = iu8_bf16_bits(iu8_epi(acc[i][j][r], am, wsu[r]));
+          *(iu8_v2u *)((unsigned short *)Cv + crow + n) = iu8_v2u{h[0] | (h[1] << 16), h[2] | (h[3] << 16)};
+        }
+      }
+    }
+    return;
+  }
+
+  // ---- grid-level split: partials to `decode_partial`, the last-arriving workgroup of this
+  // column block sums them and runs the epilogue; the counter is left at zero.
+  if (wk == 0) {
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+      if (nt0 + j >= ntiles) continue;
+      const int n = (nt0 + j) * 16 + nq;
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        const int m = i * 16 + ml;
+        if (m < M) *(iu8_v4i *)&P[((size_t)z * M + m) * N + n] = acc[i][j];
+      }
+    }
+  }
+  __syncthreads();
+  if (tid == 0) {
+    __threadfence();
+    s_last = (atomicAdd(&cnt[blockIdx.x], 1) == Z - 1);
+  }
+  __syncthreads();
+  if (!s_last) return;
+  __threadfence();
+  if (tid == 0) cnt[blockIdx.x] = 0;
+  const int nb = blockIdx.x * BN, nw4 = min(BN, N - nb) >> 2;
+  for (int idx = tid; idx < nw4 * M; idx += NTHR) {
+    const int m = idx / nw4, n = nb + (idx % nw4) * 4;
+    iu8_v4i sum = iu8_v4i{0, 0, 0, 0};
+    for (int q = 0; q < Z; ++q) sum += __builtin_nontemporal_load((const iu8_v4i *)&P[((size_t)q * M + m) * N + n]);
+    const size_t crow = (size_t)(R.row0 + m) * N;
+    if constexpr (ACC) {
+      *(iu8_v4i *)((int *)Cv + crow + n) = sum;
+    } else {
+      const float am = as[iu8_arow(R, m)];
+      unsigned h[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) h[r] = iu8_bf16_bits(iu8_epi(sum[r], am, iu8_wsu<W8>(ws, n + r)));
+      *(iu8_v2u *)((unsigned short *)Cv + crow + n) = iu8_v2u{h[0] | (h[1] << 16), h[2] | (h[3] << 16)};
+    }
+  }
+}
+
+
+// ============================================================================ prefill tile
+template <bool W8, int WMW, int WNW, int TM, int TN, bool ACC>
+__device__ __forceinline__ void iu8_pf_body(const iu8_u8 *__restrict__ A, const iu8_u8 *__restrict__ W,
+                                            const float *__restrict__ as, const float *__restrict__ ws,
+                                            void *__restrict__ Cv, const iu8_rows R, int mbase, int N, int K) {
+  // R: the rows this launch (dense) or this tile (grouped) owns; mbase: the first of them this
+  // workgroup computes
+  constexpr int NTHR = WMW * WNW * 64;
+  constexpr int BMT = WMW * TM, BNT = WNW * TN;  // 16-row tiles a workgroup, both ways
+  constexpr int WSTEP = W8 ? 2048 : 1024;
+  constexpr int A_PIECES = BMT * 128, W_PIECES = BNT * (WSTEP / 16);  // 16-byte pieces a K step
+  constexpr int A_PER = (A_PIECES + NTHR - 1) / NTHR, W_PER = (W_PIECES + NTHR - 1) / NTHR;
+  __shared__ __attribute__((aligned(16))) iu8_u8 sA[BMT * 2048];
+  __shared__ __attribute__((aligned(16))) iu8_u8 sW[BNT * WSTEP];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WNW, wn = wave % WNW;
+  const int M = R.rows, ntiles = N >> 4, steps = K >> 7, ktiles = K >> 6;
+  const int nt0 = blockIdx.x * BNT;
+
+  // the global side of every piece this thread stages (tiles past the edge re-read the last one)
+  const iu8_u8 *ga[A_PER];
+  const iu8_u8 *gw[W_PER];
+#pragma unroll
+  for (int p = 0; p < A_PER; ++p) {
+    const int piece = p * NTHR + tid;
+    const int within = piece % 128, pl = within & 63;
+    const int ar = iu8_arow(R, mbase + (piece / 128) * 16 + (pl & 15));
+    ga[p] = A + ((size_t)(ar >> 4) * ktiles + (within >> 6)) * 1024 + ((ar & 15) + 16 * (pl >> 4)) * 16;
+  }
+#pragma unroll
+  for (int p = 0; p < W_PER; ++p) {
+    const int piece = p * NTHR + tid;
+    const int nt = min(nt0 + piece / (WSTEP / 16), ntiles - 1);
+    gw[p] = W + (size_t)nt * steps * WSTEP + (piece % (WSTEP / 16)) * 16;
+  }
+
+  iu8_v4i acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) acc[i][j] = iu8_v4i{0, 0, 0, 0};
+
+  iu8_v4u ra[A_PER], rw[W_PER];
+  auto gload = [&](int s) {
+#pragma unroll
+    for (int p = 0; p < A_PER; ++p)
+      if (A_PIECES % NTHR == 0 || p * NTHR + tid < A_PIECES) ra[p] = *(const iu8_v4u *)(ga[p] + (size_t)s * 2048);
+#pragma unroll
+    for (int p = 0; p < W_PER; ++p)
+      if (W_PIECES % NTHR == 0 || p * NTHR + tid < W_PIECES) rw[p] = iu8_ldg_nt(gw[p] + (size_t)s * WSTEP);
+  };
+  gload(0);
+  for (int s = 0; s < steps; ++s) {
+    __syncthreads();  // every wave is done reading the previous step's fragments
+#pragma unroll
+    for (int p = 0; p < A_PER; ++p)
+      if (A_PIECES % NTHR == 0 || p * NTHR + tid < A_PIECES) *(iu8_v4u *)&sA[(p * NTHR + tid) * 16] = ra[p];
+#pragma unroll
+    for (int p = 0; p < W_PER; ++p)
+      if (W_PIECES % NTHR == 0 || p * NTHR + tid < W_PIECES) *(iu8_v4u *)&sW[(p * NTHR + tid) * 16] = rw[p];
+    __syncthreads();
+    if (s + 1 < steps) gload(s + 1);
+
+    iu8_v4i wf[TN][2];
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      if constexpr (W8) {
+        wf[j][0] = *(const iu8_v4i *)&sW[((wn * TN + j) * 2 + 0) * 1024 + lane * 16];
+        wf[j][1] = *(const iu8_v4i *)&sW[((wn * TN + j) * 2 + 1) * 1024 + lane * 16];
+      } else {
+        iu8_unpack_w4(*(const iu8_v4u *)&sW[(wn * TN + j) * 1024 + lane * 16], wf[j][0], wf[j][1]);
+      }
+    }
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        const iu8_v4i af = *(const iu8_v4i *)&sA[((wm * TM + i) * 2 + h) * 1024 + lane * 16];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = iu8_mfma(wf[j][h], af, acc[i][j]);
+      }
+  }
+
+  const int ml = lane & 15, nq = (lane >> 4) * 4;
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int nt = nt0 + wn * TN + j;
+    if (nt >= ntiles) continue;
+    const int n = nt * 16 + nq;
+    float wsu[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) wsu[r] = iu8_wsu<W8>(ws, n + r);
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int m = mbase + (wm * TM + i) * 16 + ml;
+      if (m >= M) continue;
+      const size_t crow = (size_t)(R.row0 + m) * N;
+      if constexpr (ACC) {
+        *(iu8_v4i *)((int *)Cv + crow + n) = acc[i][j];
+      } else {
+        const float am = as[iu8_arow(R, m)];
+        unsigned h[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) h[r] = iu8_bf16_bits(iu8_epi(acc[i][j][r], am, wsu[r]));
+        *(iu8_v2u *)((unsigned short *)Cv + crow + n) = iu8_v2u{h[0] | (h[1] << 16), h[2] | (h[3] << 16)};
+      }
+    }
+  }
+}
+

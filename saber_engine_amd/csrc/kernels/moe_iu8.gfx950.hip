@@ -1,0 +1,343 @@
+// The expert-routed (MoE) form of the W4A8-iu8 linear for gfx950: the code object `moe_iu8`.
+// The reference has no iu8 MoE (its grouped GEMM is MXFP4 x e4m3, crates/saber-kernels/hip/
+// moe_grouped.hip); this object composes the reference's routing / tile / combine LAW
+// (crates/saber-kernels/hip/moe_route.hip:1-24,108-329, crates/saber-kernels/src/moe.rs:691-865)
+// with the iu8 GEMM contract (iu8_common.h) at 128 experts, top-8:
+//
+//   moe_iu8_route_topk8_sort_e128   logits bf16 [T,128] -> f32 softmax (IEEE-only exp) -> top-8,
+//        the LOWER expert id wins a tie -> w = p * (1 / (sum > 0 ? sum : 1)), sum in k order ->
+//        expert-major sort of the local experts [e_lo, e_lo + e_loc) into 16-row blocks, cut into
+//        tiles of `tile_blocks` blocks. One launch: a workgroup routes 32 tokens and counts its
+//        routes per expert; the last workgroup to arrive scans and places every route. No atomic
+//        decides an output byte: a route's row = expert offset + earlier workgroups' count + its
+//        rank among this workgroup's earlier tokens, i.e. token order.
+//        Signature: crates/saber-kernels/src/abi.rs:354-374.
+//   moe_iu8_grouped_w4_{dec,pf}_g{0,1}   per tile of the table: one expert's weights through
+//        xptr[2e] (W4 fragments) / xptr[2e+1] (f32 row scales), activation rows gathered through
+//        row_tok (g1: gate+up) or in place (g0: down), C rows at the tile's row0. `dec` streams the
+//        weights for tiles of <= 16 rows (few tokens: HBM-bound), `pf` is the MFMA tile for tiles of
+//        up to 256 rows of one expert. Signature: crates/saber-kernels/src/abi.rs:325-340 (p / cnt /
+//        pmax are the split-K workspaces of the reference's cells; this object does not split).
+//   moe_iu8_combine_bf16   out[t] = bf16(sum_k w[t,k] * f32(Y[pos(t,k)])), f32 adds in top-k order,
+//        one rounding (crates/saber-kernels/hip/moe_route.hip:287-329; abi.rs:377-385).
+#include "iu8_gemm.h"
+
+#define MOE_E 128
+#define MOE_TOPK 8
+#define MOE_TPB 32
+#define MOE_THREADS 256
+
+// e^x for x <= 0 from IEEE-rounded mul/add/rint/ldexp only (the law of
+// crates/saber-kernels/hip/moe_route.hip:43-57: n = rint(x*log2e), two-step Cody-Waite reduction,
+// degree-7 Taylor by Horner, ldexp; x <= -80 or NaN -> 0).
+static __device__ __forceinline__ float moe_exp_nonpos(float x) {
+#pragma clang fp contract(off)
+  if (!(x > -80.f)) return 0.f;
+  const float n = __builtin_rintf(x * __uint_as_float(0x3FB8AA3Bu));
+  float r = x - n * __uint_as_float(0x3F317200u);
+  r = r - n * __uint_as_float(0x35BFBE8Eu);
+  float p = __uint_as_float(0x39500D01u);
+  p = p * r + __uint_as_float(0x3AB60B61u);
+  p = p * r + __uint_as_float(0x3C088889u);
+  p = p * r + __uint_as_float(0x3D2AAAABu);
+  p = p * r + __uint_as_float(0x3E2AAAABu);
+  p = p * r + 0.5f;
+  p = p * r + 1.f;
+  p = p * r + 1.f;
+  return __builtin_ldexpf(p, (int)n);
+}
+
+// exclusive scan of one int a thread over the 256-thread workgroup; *total = the sum
+static __device__ __forceinline__ int moe_exscan(int v, int *s_wave, int *total) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int x = v;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const int y = __shfl_up(x, o, 64);
+    if (lane >= o) x += y;
+  }
+  if (lane == 63) s_wave[wave] = x;
+  __syncthreads();
+  int base = 0, all = 0;
+#pragma unroll
+  for (int w = 0; w < MOE_THREADS / 64; ++w) {
+    const int s = s_wave[w];
+    if (w < wave) base += s;
+    all += s;
+  }
+  __syncthreads();
+  *total = all;
+  return base + x - v;
+}
+
+extern "C" __global__ __launch_bounds__(MOE_THREADS) void moe_iu8_route_topk8_sort_e128(
+    const unsigned short *__restrict__ logits, int T, int e_lo, int e_loc, int tile_blocks, int with_shared,
+    int *__restrict__ topk_ids, float *__restrict__ topk_w, int *__restrict__ route_pos, int *__restrict__ row_tok,
+    int *__restrict__ row_route, int *__restrict__ tile_expert, int *__restrict__ tile_row0,
+    int *__restrict__ tile_rows, int *__restrict__ expert_cnt, int *__restrict__ meta, int *__restrict__ blk_cnt,
+    int *__restrict__ rank, int *__restrict__ arrive) {
+#pragma clang fp contract(off)
+  __shared__ int s_ids[MOE_TPB * MOE_TOPK];
+  __shared__ int s_cnt[MOE_E];
+  __shared__ int s_off[MOE_E], s_toff[MOE_E];
+  __shared__ int s_wave[MOE_THREADS / 64];
+  __shared__ int s_last;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int nblk = gridDim.x, blk = blockIdx.x, t0 = blk * MOE_TPB;
+
+  for (int e = tid; e < MOE_E; e += MOE_THREADS) s_cnt[e] = 0;
+  for (int i = tid; i < MOE_TPB * MOE_TOPK; i += MOE_THREADS) s_ids[i] = -1;
+  __syncthreads();
+
+  // ---- phase 1: 8 lanes a token (a wave = 8 tokens); lane group g owns experts [16g, 16g + 16).
+  // Sum order: a group's 16 in index order, then the xor butterfly 4, 2, 1 over the 8 group sums.
+  {
+    const int g = lane & 7, tl = wave * 8 + (lane >> 3), t = t0 + tl;
+    if (t < T) {
+      float p[16];
+      const iu8_v4u *src = (const iu8_v4u *)(logits + (size_t)t * MOE_E + g * 16);
+      const iu8_v4u v0 = src[0], v1 = src[1];
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        p[2 * w] = __uint_as_float(v0[w] << 16);
+        p[2 * w + 1] = __uint_as_float(v0[w] & 0xFFFF0000u);
+        p[8 + 2 * w] = __uint_as_float(v1[w] << 16);
+        p[8 + 2 * w + 1] = __uint_as_float(v1[w] & 0xFFFF0000u);
+      }
+      float mx = p[0];
+#pragma unroll
+      for (int j = 1; j < 16; ++j) mx = fmaxf(mx, p[j]);
+#pragma unroll
+      for (int o = 4; o; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+      float s = 0.f;
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        p[j] = moe_exp_nonpos(p[j] - mx);
+        s = s + p[j];
+      }
+#pragma unroll
+      for (int o = 4; o; o >>= 1) s = s + __shfl_xor(s, o, 64);
+      const float inv = 1.f / s;
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        float q = p[j] * inv;
+        if (!__builtin_isfinite(q)) q = 0.f;
+        p[j] = q;
+      }
+      float sel = 0.f, mine_w = 0.f;
+      int mine_i = 0;
+#pragma unroll
+      for (int k = 0; k < MOE_TOPK; ++k) {
+        float bv = p[0];
+        int bj = 0;
+#pragma unroll
+        for (int j = 1; j < 16; ++j)
+          if (p[j] > bv) {  // strict: the lower index keeps a tie
+            bv = p[j];
+            bj = j;
+          }
+        int bi = g * 16 + bj;
+#pragma unroll
+        for (int o = 4; o; o >>= 1) {
+          const float ov = __shfl_xor(bv, o, 64);
+          const int oi = __shfl_xor(bi, o, 64);
+          if (ov > bv || (ov == bv && oi < bi)) {
+            bv = ov;
+            bi = oi;
+          }
+        }
+        if ((bi >> 4) == g) {
+#pragma unroll
+          for (int j = 0; j < 16; ++j)
+            if (j == (bi & 15)) p[j] = -1.f;  // probabilities are >= 0
+        }
+        if (k == g) {
+          mine_w = bv;
+          mine_i = bi;
+        }
+        sel = sel + bv;  // k order
+      }
+      const float scale = 1.f / (sel > 0.f ? sel : 1.f);
+      // lane g of the token's group holds route k = g
+      topk_ids[(size_t)t * MOE_TOPK + g] = mine_i;
+      topk_w[(size_t)t * MOE_TOPK + g] = mine_w * scale;
+      s_ids[tl * MOE_TOPK + g] = mine_i;
+    }
+  }
+  __syncthreads();
+
+  // ---- phase 2: this workgroup's per-expert counts and each route's rank among the earlier
+  // tokens of this workgroup routed to the same expert (a token's experts are distinct)
+  for (int i = tid; i < MOE_TPB * MOE_TOPK; i += MOE_THREADS) {
+    const int e = s_ids[i], le = e - e_lo;
+    if (e < 0 || le < 0 || le >= e_loc) continue;
+    atomicAdd(&s_cnt[le], 1);
+    const int before = (i / MOE_TOPK) * MOE_TOPK;
+    int rk = 0;
+    for (int u = 0; u < before; ++u) rk += s_ids[u] == e;
+    rank[(size_t)t0 * MOE_TOPK + i] = rk;
+  }
+  __syncthreads();
+  for (int e = tid; e < e_loc; e += MOE_THREADS) blk_cnt[(size_t)blk * e_loc + e] = s_cnt[e];
+  __syncthreads();
+  if (tid == 0) {
+    __threadfence();
+    s_last = atomicAdd(arrive, 1) == nblk - 1;
+  }
+  __syncthreads();
+  if (!s_last) return;
+  __threadfence();  // acquire: every workgroup's topk_ids, rank and blk_cnt
+  if (tid == 0) *arrive = 0;
+
+  // ---- phase 3 (the last workgroup): totals, each workgroup's base, offsets, tiles, placement
+  for (int e = tid; e < e_loc; e += MOE_THREADS) {
+    int run = 0;
+    for (int b = 0; b < nblk; ++b) {
+      const int c = __builtin_nontemporal_load(&blk_cnt[(size_t)b * e_loc + e]);
+      blk_cnt[(size_t)b * e_loc + e] = run;
+      run += c;
+    }
+    s_cnt[e] = run;
+    expert_cnt[e] = run;
+  }
+  __syncthreads();
+  const int G = tile_blocks, TR = 16 * tile_blocks;
+  int my_rows = 0, my_tiles = 0, my_touched = 0, my_routes = 0;
+  if (tid < e_loc) {
+    const int c = s_cnt[tid], nb = (c + 15) / 16;
+    my_rows = nb * 16;
+    my_tiles = (nb + G - 1) / G;
+    my_touched = c > 0;
+    my_routes = c;
+  }
+  int rows_total, tiles_total, touched_total, routes_total;
+  const int rbase = moe_exscan(my_rows, s_wave, &rows_total);
+  const int tbase = moe_exscan(my_tiles, s_wave, &tiles_total);
+  moe_exscan(my_touched, s_wave, &touched_total);
+  moe_exscan(my_routes, s_wave, &routes_total);
+  if (tid < e_loc) {
+    s_off[tid] = rbase;
+    s_toff[tid] = tbase;
+  }
+  __syncthreads();
+  const int sh_row0 = rows_total;
+  const int sh_blocks = with_shared ? (T + 15) / 16 : 0;
+  const int sh_tiles = (sh_blocks + G - 1) / G;
+  if (tid == 0) {
+    meta[0] = tiles_total + sh_tiles;
+    meta[1] = rows_total + sh_blocks * 16;
+    meta[2] = with_shared ? sh_row0 : -1;
+    meta[3] = routes_total;
+    meta[4] = touched_total;
+    meta[5] = rows_total;
+  }
+  for (int e = tid; e < e_loc; e += MOE_THREADS) {
+    const int c = s_cnt[e], nb = (c + 15) / 16, nt = (nb + G - 1) / G;
+    for (int j = 0; j < nt; ++j) {
+      tile_expert[s_toff[e] + j] = e;
+      tile_row0[s_toff[e] + j] = s_off[e] + j * TR;
+      tile_rows[s_toff[e] + j] = min(TR, c - j * TR);
+    }
+    for (int r = s_off[e] + c; r < s_off[e] + nb * 16; ++r) {
+      row_tok[r] = -1;
+      row_route[r] = -1;
+    }
+  }
+  for (int j = tid; j < sh_tiles; j += MOE_THREADS) {
+    tile_expert[tiles_total + j] = e_loc;
+    tile_row0[tiles_total + j] = sh_row0 + j * TR;
+    tile_rows[tiles_total + j] = min(TR, T - j * TR);
+  }
+  for (int r = tid; r < sh_blocks * 16; r += MOE_THREADS) {
+    row_tok[sh_row0 + r] = r < T ? r : -1;
+    row_route[sh_row0 + r] = -1;
+  }
+  for (int r = tid; r < T * MOE_TOPK; r += MOE_THREADS) {
+    const int e = __builtin_nontemporal_load(&topk_ids[r]), le = e - e_lo;
+    if (le < 0 || le >= e_loc) {
+      route_pos[r] = -1;
+      continue;
+    }
+    const int t = r / MOE_TOPK, b = t / MOE_TPB;
+    const int p = s_off[le] + blk_cnt[(size_t)b * e_loc + le] + __builtin_nontemporal_load(&rank[r]);
+    row_tok[p] = t;
+    row_route[p] = r;
+    route_pos[r] = p;
+  }
+}
+
+// ---------------------------------------------------------------------------- grouped GEMMs
+// grid [ceil(N / BN), tiles_cap, 1]: blockIdx.y is a tile; a workgroup whose tile is past the live
+// count exits whole.
+#define MOE_GROUPED_DEC(name, GATHER, NT, KW, WPB, D, ALDS)                                                      \
+  extern "C" __global__ __launch_bounds__(WPB * 64) void name(                                                    \
+      const unsigned char *__restrict__ a, const unsigned long long *__restrict__ xptr,                           \
+      const int *__restrict__ tile_expert, const int *__restrict__ tile_row0, const int *__restrict__ tile_rows,  \
+      const int *__restrict__ row_tok, const int *__restrict__ meta, const float *__restrict__ as,                \
+      int *__restrict__ p, int *__restrict__ cnt, unsigned short *__restrict__ c, int n, int k, int pmax) {        \
+    const int tile = blockIdx.y;                                                                                   \
+    if (tile >= meta[0]) return;                                                                                   \
+    const int e = tile_expert[tile];                                                                               \
+    const iu8_rows R{GATHER ? row_tok : nullptr, tile_row0[tile], min(tile_rows[tile], 16)};                       \
+    iu8_dec_body<1, false, NT, KW, WPB, D, ALDS, false>(a, (const unsigned char *)xptr[2 * e], as,                 \
+                                                        (const float *)xptr[2 * e + 1], p, cnt, c, R, n, k);       \
+  }
+MOE_GROUPED_DEC(moe_iu8_grouped_w4_dec_g1, true, 1, 4, 8, 8, 20)
+MOE_GROUPED_DEC(moe_iu8_grouped_w4_dec_g0, false, 1, 4, 8, 8, 20)
+#undef MOE_GROUPED_DEC
+
+#define MOE_GROUPED_PF(name, GATHER, WMW, WNW, TM, TN)                                                           \
+  extern "C" __global__ __launch_bounds__(WMW * WNW * 64) void name(                                              \
+      const unsigned char *__restrict__ a, const unsigned long long *__restrict__ xptr,                           \
+      const int *__restrict__ tile_expert, const int *__restrict__ tile_row0, const int *__restrict__ tile_rows,  \
+      const int *__restrict__ row_tok, const int *__restrict__ meta, const float *__restrict__ as,                \
+      int *__restrict__ p, int *__restrict__ cnt, unsigned short *__restrict__ c, int n, int k, int pmax) {        \
+    const int tile = blockIdx.y;                                                                                   \
+    if (tile >= meta[0]) return;                                                                                   \
+    const int e = tile_expert[tile];                                                                               \
+    const iu8_rows R{GATHER ? row_tok : nullptr, tile_row0[tile], min(tile_rows[tile], WMW * TM * 16)};            \
+    iu8_pf_body<false, WMW, WNW, TM, TN, false>(a, (const unsigned char *)xptr[2 * e], as,                         \
+                                                (const float *)xptr[2 * e + 1], c, R, 0, n, k);                    \
+  }
+// tiles of up to 128 rows (tile_blocks 8) on the 128 x 128 tile of 2 x 2 waves
+MOE_GROUPED_PF(moe_iu8_grouped_w4_pf_g1, true, 2, 2, 4, 4)
+MOE_GROUPED_PF(moe_iu8_grouped_w4_pf_g0, false, 2, 2, 4, 4)
+#undef MOE_GROUPED_PF
+
+// ---------------------------------------------------------------------------- combine
+// One workgroup a token, 8 bf16 a thread-step.
+extern "C" __global__ __launch_bounds__(256) void moe_iu8_combine_bf16(
+    const unsigned short *__restrict__ y, const float *__restrict__ topk_w, const int *__restrict__ route_pos,
+    const unsigned short *__restrict__ sgate, const int *__restrict__ meta, unsigned short *__restrict__ out, int h) {
+#pragma clang fp contract(off)
+  const int t = blockIdx.x;
+  __shared__ int s_pos[MOE_TOPK];
+  __shared__ float s_w[MOE_TOPK];
+  if (threadIdx.x < MOE_TOPK) {
+    s_pos[threadIdx.x] = route_pos[(size_t)t * MOE_TOPK + threadIdx.x];
+    s_w[threadIdx.x] = topk_w[(size_t)t * MOE_TOPK + threadIdx.x];
+  }
+  __syncthreads();
+  (void)sgate;  // the shared-expert gate term is not part of this object's layer
+  (void)meta;
+  for (int g = threadIdx.x; g < h / 8; g += 256) {
+    float acc[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j] = 0.f;
+    for (int k = 0; k < MOE_TOPK; ++k) {
+      const int p = s_pos[k];
+      if (p < 0) continue;
+      const float w = s_w[k];
+      const iu8_v4u v = ((const iu8_v4u *)(y + (size_t)p * h))[g];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        acc[2 * q] = acc[2 * q] + w * __uint_as_float(v[q] << 16);
+        acc[2 * q + 1] = acc[2 * q + 1] + w * __uint_as_float(v[q] & 0xFFFF0000u);
+      }
+    }
+    iu8_v4u o;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) o[q] = iu8_bf16_bits(acc[2 * q]) | (iu8_bf16_bits(acc[2 * q + 1]) << 16);
+    ((iu8_v4u *)(out + (size_t)t * h))[g] = o;
+  }
+}

@@ -66,9 +66,12 @@ class Counters(C.Structure):
                 ("refused_wave", C.c_uint32), ("refused_metadata", C.c_uint32), ("launches", C.c_uint32)]
 
 
+MOE_TABLE_FIELDS = ("topk_ids", "topk_w", "route_pos", "row_tok", "row_route", "tile_expert", "tile_row0", "tile_rows",
+                    "expert_cnt", "meta", "blk_cnt", "rank", "arrive")
+
+
 class MoeTables(C.Structure):
-    _fields_ = [(n, C.c_void_p) for n in ("topk_ids", "topk_w", "route_pos", "row_tok", "tile_expert", "tile_row0",
-                                          "tile_rows", "expert_cnt", "meta", "scratch")]
+    _fields_ = [(n, C.c_void_p) for n in MOE_TABLE_FIELDS]
 
 
 class IU8Error(RuntimeError):
@@ -106,6 +109,17 @@ def lib():
         L.saber_iu8_gemm_acc.argtypes = [C.c_void_p, C.c_int] + [C.c_void_p] * 3 + [C.c_uint32] * 3 + [C.c_void_p]
         L.saber_iu8_get_counters.argtypes = [C.c_void_p, C.POINTER(Counters)]
         L.saber_iu8_has_kernel.argtypes = [C.c_void_p, C.c_char_p]
+        for fn in ("saber_iu8_moe_rows_cap", "saber_iu8_moe_tile_blocks"):
+            getattr(L, fn).restype = C.c_uint32
+            getattr(L, fn).argtypes = [C.c_uint32] * 3
+        L.saber_iu8_moe_tiles_cap.restype = C.c_uint32
+        L.saber_iu8_moe_tiles_cap.argtypes = [C.c_uint32] * 4
+        L.saber_iu8_moe_route.argtypes = [C.c_void_p, C.c_void_p] + [C.c_uint32] * 4 + [C.POINTER(MoeTables), C.c_void_p]
+        L.saber_iu8_moe_grouped.argtypes = ([C.c_void_p] * 5 + [C.c_uint32, C.c_uint32, C.c_int] + [C.c_uint32] * 4 +
+                                            [C.POINTER(MoeTables), C.c_void_p])
+        L.saber_iu8_moe_silu_mul_quant.argtypes = [C.c_void_p] * 4 + [C.c_uint32, C.c_uint32, C.POINTER(MoeTables), C.c_void_p]
+        L.saber_iu8_moe_combine.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(MoeTables), C.c_void_p] + [C.c_uint32] * 3 + [C.c_void_p]
+        L.saber_iu8_silu_table.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
         _lib = L
     return _lib
 
@@ -263,6 +277,36 @@ class Context:
 
     def gemm_acc(self, wkind, a, w, acc, m, n, k, stream=0):
         _check(lib().saber_iu8_gemm_acc(self._h, wkind, a, w, acc, m, n, k, stream))
+
+
+    # ---- routed experts
+    def moe_route(self, logits, tokens, experts, topk, tile_blocks, tables, stream=0):
+        _check(lib().saber_iu8_moe_route(self._h, logits, tokens, experts, topk, tile_blocks, C.byref(tables), stream))
+
+    def moe_grouped(self, a, a_scale, xptr, c, n, k, gather, tokens, experts, topk, tile_blocks, tables, stream=0):
+        _check(lib().saber_iu8_moe_grouped(self._h, a, a_scale, xptr, c, n, k, int(gather), tokens, experts, topk,
+                                           tile_blocks, C.byref(tables), stream))
+
+    def moe_silu_mul_quant(self, gu, q, scale, n, rows_cap, tables, stream=0):
+        _check(lib().saber_iu8_moe_silu_mul_quant(self._h, gu, q, scale, n, rows_cap, C.byref(tables), stream))
+
+    def moe_combine(self, y, tables, out, tokens, topk, h, stream=0):
+        _check(lib().saber_iu8_moe_combine(self._h, y, C.byref(tables), out, tokens, topk, h, stream))
+
+    def silu_table(self, out, stream=0):
+        _check(lib().saber_iu8_silu_table(self._h, out, stream))
+
+
+def moe_rows_cap(tokens, topk, experts):
+    return lib().saber_iu8_moe_rows_cap(tokens, topk, experts)
+
+
+def moe_tiles_cap(tokens, topk, experts, tile_blocks):
+    return lib().saber_iu8_moe_tiles_cap(tokens, topk, experts, tile_blocks)
+
+
+def moe_tile_blocks(tokens, topk, experts):
+    return lib().saber_iu8_moe_tile_blocks(tokens, topk, experts)
 
 
 def gemm_workspace(wkind, m, n, k):

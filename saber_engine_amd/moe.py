@@ -1,0 +1,59 @@
+"""The routed-expert layer as a launch train over the C ABI: route+sort -> per-token quant ->
+grouped gate+up (gathered) -> SiLU*up requant -> grouped down -> weighted combine.  The train and
+its buffers follow the reference's MoE block (crates/saber-kernels/src/moe.rs:9-28, 142-171); the
+arithmetic of every GEMM is the iu8 contract.  torch is used for device memory only.
+"""
+import numpy as np
+import torch
+
+from . import iu8
+
+
+class MoeLayerIU8:
+    def __init__(self, ctx, tokens, experts=128, topk=8, hidden=4096, inter=1536, tile_blocks=None, device="cuda"):
+        self.ctx, self.T, self.E, self.topk, self.H, self.I = ctx, tokens, experts, topk, hidden, inter
+        self.tb = tile_blocks or iu8.moe_tile_blocks(tokens, topk, experts)
+        self.rows_cap = iu8.moe_rows_cap(tokens, topk, experts)
+        self.tiles_cap = iu8.moe_tiles_cap(tokens, topk, experts, self.tb)
+        i32 = dict(dtype=torch.int32, device=device)
+        R = tokens * topk
+        self.buf = dict(
+            topk_ids=torch.zeros(R, **i32), topk_w=torch.zeros(R, dtype=torch.float32, device=device),
+            route_pos=torch.zeros(R, **i32), row_tok=torch.full((self.rows_cap,), -1, **i32),
+            row_route=torch.zeros(self.rows_cap, **i32), tile_expert=torch.zeros(self.tiles_cap, **i32),
+            tile_row0=torch.zeros(self.tiles_cap, **i32), tile_rows=torch.zeros(self.tiles_cap, **i32),
+            expert_cnt=torch.zeros(experts, **i32), meta=torch.zeros(8, **i32),
+            blk_cnt=torch.zeros(((tokens + 31) // 32) * experts, **i32), rank=torch.zeros(R, **i32),
+            arrive=torch.zeros(1, **i32))          # persistent: zeroed once, left zero by the kernel
+        self.tables = iu8.MoeTables(*[self.buf[n].data_ptr() for n in iu8.MOE_TABLE_FIELDS])
+        u8 = dict(dtype=torch.uint8, device=device)
+        self.q1 = torch.zeros(iu8.a_bytes(tokens, hidden), **u8)
+        self.s1 = torch.zeros(tokens, dtype=torch.float32, device=device)
+        self.gu = torch.zeros((self.rows_cap, 2 * inter), dtype=torch.int16, device=device)
+        self.q2 = torch.zeros(iu8.a_bytes(self.rows_cap, inter), **u8)
+        self.s2 = torch.zeros(self.rows_cap, dtype=torch.float32, device=device)
+        self.y = torch.zeros((self.rows_cap, hidden), dtype=torch.int16, device=device)
+        self.out = torch.zeros((tokens, hidden), dtype=torch.int16, device=device)
+        self.xptr_gu = self.xptr_dn = None
+
+    def set_weights(self, wgu_frag, wsgu, wdn_frag, wsdn):
+        """Per-expert gfx950 W4 fragments [E, 2I*H/2] / [E, H*I/2] (uint8) and scales [E,2I] / [E,H] (f32) on device."""
+        self._w = (wgu_frag, wsgu, wdn_frag, wsdn)
+        E = self.E
+        gu = [[wgu_frag[e].data_ptr(), wsgu[e].data_ptr()] for e in range(E)]
+        dn = [[wdn_frag[e].data_ptr(), wsdn[e].data_ptr()] for e in range(E)]
+        self.xptr_gu = torch.tensor(np.array(gu, np.int64).ravel(), device=wgu_frag.device)
+        self.xptr_dn = torch.tensor(np.array(dn, np.int64).ravel(), device=wgu_frag.device)
+
+    def forward(self, x, logits, stream=0):
+        """x bf16 bits [T,H] (int16 tensor), logits bf16 bits [T,E]; every launch on `stream`."""
+        c, T, E, k, H, I = self.ctx, self.T, self.E, self.topk, self.H, self.I
+        c.moe_route(logits.data_ptr(), T, E, k, self.tb, self.tables, stream)
+        c.quant(x.data_ptr(), self.q1.data_ptr(), self.s1.data_ptr(), T, H, stream)
+        c.moe_grouped(self.q1.data_ptr(), self.s1.data_ptr(), self.xptr_gu.data_ptr(), self.gu.data_ptr(), 2 * I, H, True,
+                      T, E, k, self.tb, self.tables, stream)
+        c.moe_silu_mul_quant(self.gu.data_ptr(), self.q2.data_ptr(), self.s2.data_ptr(), I, self.rows_cap, self.tables, stream)
+        c.moe_grouped(self.q2.data_ptr(), self.s2.data_ptr(), self.xptr_dn.data_ptr(), self.y.data_ptr(), H, I, False,
+                      T, E, k, self.tb, self.tables, stream)
+        c.moe_combine(self.y.data_ptr(), self.tables, self.out.data_ptr(), T, k, H, stream)
+        return self.out
