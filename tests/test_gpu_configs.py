@@ -1,0 +1,181 @@
+"""GPU parity at the benchmark configurations' own shapes and edge cases: golden vectors, the mixed
+W4/W8 launch sequence, every kernel variant of a regime giving the same bytes, the explicit grid
+split with its workspaces, and size-independent properties at the full sizes."""
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import ref
+from saber_engine_amd import iu8, synth
+from tests.gpu_util import DenseRun, assert_dense_matches, dev_bf16_bits, dev_f32, dev_u8, host_u16, say
+
+pytestmark = pytest.mark.gpu
+GOLD = np.load(os.path.join(os.path.dirname(__file__), "golden", "dense_small.npz"))
+
+
+@pytest.mark.parametrize("i", range(5))
+def test_golden_vectors(ctx, i):
+    M, N, K, w8 = [int(v) for v in GOLD[f"c{i}_meta"]]
+    say(f"golden vector {i}: M={M} N={N} K={K} w8={w8}")
+    case = dict(M=M, N=N, K=K, w8=bool(w8), X=GOLD[f"c{i}_X"], W=GOLD[f"c{i}_W"], ws=GOLD[f"c{i}_ws"])
+    run = DenseRun(ctx, case, want_acc=True)
+    want = dict(q=GOLD[f"c{i}_q"], a_scale=GOLD[f"c{i}_a_scale"], S=GOLD[f"c{i}_S"], C=GOLD[f"c{i}_C"])
+    assert_dense_matches(run, want, bool(w8))
+
+
+def test_config0_single_gemv(ctx):
+    say("config 0: M=1 K=5120 N=5120 seed 0")
+    case = synth.dense_case(1, 5120, 5120, seed=0)
+    r = ref.linear(case["X"], case["W"], case["ws"], False, threads=8)
+    assert_dense_matches(DenseRun(ctx, case), r, False)
+
+
+@pytest.mark.parametrize("M", [1, 4, 8, 16])
+def test_config1_decode_layer_set(ctx, M):
+    for name, n, k in synth.LAYER_LINEARS:
+        say(f"config 1: {name} M={M} N={n} K={k}")
+        case = synth.dense_case(M, n, k, seed=M)
+        r = ref.linear(case["X"], case["W"], case["ws"], False, threads=16)
+        assert_dense_matches(DenseRun(ctx, case), r, False)
+
+
+def all_variants(prefix):
+    text = open(os.path.join(iu8.PKG, "csrc", "kernels", "iu8_variants.def")).read()
+    names = re.findall(r"^IU8_(?:DEC|PF)_VARIANT\((\w+),", text, flags=re.M)
+    return [n for n in names if n.startswith(prefix) and not n.endswith("_acc")]
+
+
+@pytest.mark.parametrize("tag,w8", [("w4", False), ("w8", True)])
+def test_every_decode_variant_gives_the_same_bytes(ctx, tag, w8):
+    case = synth.dense_case(5, 176, 1664, w8=w8, seed=21)     # 11 n-tiles (ragged blocks), 13 K steps
+    r = ref.linear(case["X"], case["W"], case["ws"], w8)
+    names = all_variants(f"macaq_iu8_dec_{tag}_tm")
+    assert len(names) >= 4
+    for name in names:
+        for ks in (1, 2, 3):
+            say(f"variant {name} ks={ks}")
+            run = DenseRun(ctx, case, kernel=name, ks=ks, want_acc=False)
+            np.testing.assert_array_equal(run.C, r["C"])
+            if ks > 1:
+                assert not run.counter.cpu().numpy().any(), "the arrival counters must be left at zero"
+
+
+@pytest.mark.parametrize("tag,w8", [("w4", False), ("w8", True)])
+def test_every_prefill_variant_gives_the_same_bytes(ctx, tag, w8):
+    case = synth.dense_case(200, 272, 640, w8=w8, seed=22)
+    r = ref.linear(case["X"], case["W"], case["ws"], w8)
+    for name in all_variants(f"macaq_iu8_pf_{tag}_"):
+        say(f"variant {name}")
+        run = DenseRun(ctx, case, kernel=name, want_acc=False)
+        np.testing.assert_array_equal(run.C, r["C"])
+
+
+def test_split_counter_is_reusable_across_launches(ctx):
+    say("explicit split, two launches on one counter")
+    case = synth.dense_case(3, 256, 2048, seed=23)
+    r = ref.linear(case["X"], case["W"], case["ws"], False)
+    run = DenseRun(ctx, case, kernel="macaq_iu8_dec_w4_tm1", ks=4, want_acc=False)
+    np.testing.assert_array_equal(run.C, r["C"])
+    d = run.dev
+    d["c"].fill_(0)
+    bufs = dict(a=d["q"].data_ptr(), w=d["wf"].data_ptr(), ws=d["ws"].data_ptr(), c=d["c"].data_ptr(),
+                decode_partial=run.partial.data_ptr(), decode_counter=run.counter.data_ptr())
+    bufs["as"] = d["a_scale"].data_ptr()
+    ctx.launch(run.desc, bufs)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(host_u16(d["c"]), r["C"])
+
+
+def test_config3_mixed_w4_w8_sequence(ctx):
+    """19 int8-row linears among 64, one launch sequence on shared per-token activations, M=16 and
+    (on an N slice of the oracle) M=2048; int32 accumulators bit-exact per linear."""
+    seq = synth.mixed_sequence()
+    assert sum(1 for s in seq if s[3]) == 19
+    shapes = sorted({(n, k, w8) for _, n, k, w8 in seq})
+    for M in (16, 2048):
+        rng = np.random.default_rng(M)
+        acts = {k: synth.activations(rng, M, k) for k in (5120, 17408)}
+        quant = {k: ref.quant_bf16(x) for k, x in acts.items()}
+        dev = {}
+        for k, x in acts.items():
+            xd = dev_bf16_bits(x)
+            q = torch.zeros(iu8.a_bytes(M, k), dtype=torch.uint8, device="cuda")
+            s = torch.zeros(M, dtype=torch.float32, device="cuda")
+            ctx.quant(xd.data_ptr(), q.data_ptr(), s.data_ptr(), M, k)
+            dev[k] = (q, s)
+        for (n, k, w8) in shapes:
+            say(f"config 3: M={M} N={n} K={k} w8={w8}")
+            W, ws = synth.weights(rng, n, k, w8)
+            wk = iu8.W8 if w8 else iu8.W4
+            wf, wsd = dev_u8(iu8.repack_weights(W, w8)), dev_f32(ws)
+            c = torch.zeros((M, n), dtype=torch.int16, device="cuda")
+            q, s = dev[k]
+            ctx.gemm(wk, q.data_ptr(), s.data_ptr(), wf.data_ptr(), wsd.data_ptr(), c.data_ptr(), M, n, k)
+            acc = torch.zeros((M, n), dtype=torch.int32, device="cuda")
+            ctx.gemm_acc(wk, q.data_ptr(), wf.data_ptr(), acc.data_ptr(), M, n, k)
+            torch.cuda.synchronize()
+            qh, sh = quant[k]
+            cols = n if M == 16 else 512                      # the oracle checks an N slice at M=2048
+            Wc = W[:cols]
+            S, _ = ref.gemm_fast(qh, Wc, w8, threads=16)
+            np.testing.assert_array_equal(acc.cpu().numpy()[:, :cols], S if w8 else S * 16)
+            np.testing.assert_array_equal(host_u16(c)[:, :cols], ref.epilogue(S, sh, ws[:cols], w8))
+            # the whole int32 accumulator through a size-independent property: column sums are the
+            # product of the activations' column-summed codes with the weights (exact in int64)
+            colsum = qh.astype(np.int64).sum(0)
+            wfull = W.astype(np.int64) if w8 else synth.unpack_w4(W).astype(np.int64)
+            want = wfull @ colsum * (1 if w8 else 16)
+            np.testing.assert_array_equal(acc.cpu().numpy().astype(np.int64).sum(0), want)
+            del wf, wsd, c, acc
+
+
+@pytest.mark.parametrize("M", [256, 2048, 8192])
+def test_config2_prefill_full_shapes_by_properties(ctx, M):
+    """Full prefill shapes: an oracle slice bit for bit, and the whole accumulator by linearity
+    (sum over rows of A.W^T == (sum over rows of A).W^T, exact in integers)."""
+    rng = np.random.default_rng(M)
+    for name, n, k in synth.LAYER_LINEARS:
+        if M == 8192 and name == "gate_up":
+            n = 8704                                       # a quarter of the columns keeps the int32 tap at 285 MB
+        say(f"config 2: {name} M={M} N={n} K={k}")
+        W, ws = synth.weights(rng, n, k, False)
+        X = synth.activations(rng, M, k)
+        xd, wf, wsd = dev_bf16_bits(X), dev_u8(iu8.repack_w4(W)), dev_f32(ws)
+        q = torch.zeros(iu8.a_bytes(M, k), dtype=torch.uint8, device="cuda")
+        s = torch.zeros(M, dtype=torch.float32, device="cuda")
+        c = torch.zeros((M, n), dtype=torch.int16, device="cuda")
+        acc = torch.zeros((M, n), dtype=torch.int32, device="cuda")
+        ctx.quant(xd.data_ptr(), q.data_ptr(), s.data_ptr(), M, k)
+        ctx.gemm(iu8.W4, q.data_ptr(), s.data_ptr(), wf.data_ptr(), wsd.data_ptr(), c.data_ptr(), M, n, k)
+        ctx.gemm_acc(iu8.W4, q.data_ptr(), wf.data_ptr(), acc.data_ptr(), M, n, k)
+        torch.cuda.synchronize()
+        qh, sh = ref.quant_bf16(X)
+        np.testing.assert_array_equal(iu8.unpack_a(q.cpu().numpy(), M, k), qh)
+        np.testing.assert_array_equal(s.cpu().numpy().view(np.uint32), sh.view(np.uint32))
+        rows = np.unique(np.concatenate([np.arange(0, M, max(1, M // 37)), [M - 1]]))
+        cols = 256
+        S, _ = ref.gemm_fast(qh[rows], W[-cols:], False, threads=16)
+        np.testing.assert_array_equal(acc.cpu().numpy()[rows][:, -cols:], S * 16)
+        np.testing.assert_array_equal(host_u16(c)[rows][:, -cols:], ref.epilogue(S, sh[rows], ws[-cols:], False))
+        want = synth.unpack_w4(W).astype(np.int64) @ qh.astype(np.int64).sum(0) * 16
+        np.testing.assert_array_equal(acc.sum(0, dtype=torch.int64).cpu().numpy(), want)
+        # bf16 outputs of the whole matrix from the device's own accumulators (the epilogue is elementwise)
+        t = (acc.to(torch.float32) * s[:, None]) * (wsd * 0.0625)[None, :]
+        assert torch.equal(t.to(torch.bfloat16).view(torch.int16), c)
+        del xd, wf, wsd, q, s, c, acc, t
+        torch.cuda.empty_cache()
+
+
+def test_config4_moe_prefill_shape(ctx):
+    """T=4096 routed tokens, 128 experts, top-8, H=4096, I=1536 (4 distinct expert weight sets)."""
+    from saber_engine_amd.moe import MoeLayerIU8
+    from tests.test_gpu_moe import check_layer, run_layer
+
+    say("config 4: T=4096 E=128 top-8 H=4096 I=1536")
+    case = synth.moe_case(T=4096, E=128, topk=8, H=4096, I=1536, seed=0, experts=4)
+    layer = run_layer(ctx, case)
+    assert layer.tb == 8
+    check_layer(layer, case, taps=False)
