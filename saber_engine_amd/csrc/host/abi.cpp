@@ -46,7 +46,7 @@ const Signature *signature_for(const std::string &k) {
   if (k == "iu8_probe_read") return &SIG_PROBE_READ;
   if (k == "iu8_probe_copy") return &SIG_PROBE_COPY;
   if (k == "iu8_probe_empty") return &SIG_PROBE_EMPTY;
-  if (k == "iu8_probe_mfma") return &SIG_PROBE_MFMA;
+  if (k == "iu8_probe_mfma" || k == "iu8_probe_mfma32") return &SIG_PROBE_MFMA;
   if (starts(k, "moe_iu8_route_")) return &SIG_MOE_ROUTE;
   if (starts(k, "moe_iu8_grouped_")) return &SIG_MOE_GROUPED;
   if (starts(k, "moe_iu8_combine_")) return &SIG_MOE_COMBINE;

@@ -51,3 +51,24 @@ extern "C" __global__ __launch_bounds__(256) void iu8_probe_mfma(unsigned *__res
   for (int j = 1; j < 8; ++j) s += c[j];
   if ((s.x ^ s.y ^ s.z ^ s.w) == 0x12345679) out[0] = s.x;
 }
+
+// the same with v_mfma_i32_32x32x32_i8 (65,536 int8 ops each), 4 independent chains
+typedef int iu8_v16i __attribute__((ext_vector_type(16)));
+extern "C" __global__ __launch_bounds__(256) void iu8_probe_mfma32(unsigned *__restrict__ out, int n) {
+  iu8_v4i a = iu8_v4i{(int)threadIdx.x, 1, 2, 3}, b = iu8_v4i{4, 5, (int)blockIdx.x, 7};
+  iu8_v16i c[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) c[j][e] = j + e;
+  for (int i = 0; i < n; ++i) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) c[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c[j], 0, 0, 0);
+  }
+  int s = 0;
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) s ^= c[j][e];
+  if (s == 0x12345679) out[0] = s;
+}
