@@ -1,5 +1,6 @@
 #include "rules.h"
 
+#include <cmath>
 #include <cstring>
 
 #include "abi.h"
@@ -9,14 +10,14 @@ namespace iu8 {
 
 static const DecVariant DEC_VARIANTS[] = {
 #define IU8_DEC_VARIANT(name, TM, W8, NT, KW, WPB, D, ALDS, ACC) {#name, TM, W8, NT, KW, WPB, D, ALDS, ACC},
-#define IU8_PF_VARIANT(name, W8, WMW, WNW, TM, TN, ACC)
+#define IU8_PF_VARIANT(name, W8, WMW, WNW, TM, TN, ACC, ST, OCC)
 #include "../kernels/iu8_variants.def"
 #undef IU8_DEC_VARIANT
 #undef IU8_PF_VARIANT
 };
 static const PfVariant PF_VARIANTS[] = {
 #define IU8_DEC_VARIANT(name, TM, W8, NT, KW, WPB, D, ALDS, ACC)
-#define IU8_PF_VARIANT(name, W8, WMW, WNW, TM, TN, ACC) {#name, W8, WMW, WNW, TM, TN, ACC},
+#define IU8_PF_VARIANT(name, W8, WMW, WNW, TM, TN, ACC, ST, OCC) {#name, W8, WMW, WNW, TM, TN, ACC, OCC},
 #include "../kernels/iu8_variants.def"
 #undef IU8_DEC_VARIANT
 #undef IU8_PF_VARIANT
@@ -133,9 +134,10 @@ static int describe_pf(const PfVariant &v, uint32_t m, uint32_t n, uint32_t k, s
   copy_name(d->op, sizeof d->op, op);
   copy_name(d->plugin, sizeof d->plugin, "macaq_iu8");
   copy_name(d->kernel, sizeof d->kernel, v.name);
-  d->grid[0] = (n + v.block_n() - 1) / v.block_n();
-  d->grid[1] = (m + v.block_m() - 1) / v.block_m();
-  d->grid[2] = 1;
+  const uint32_t gx = (n + v.block_n() - 1) / v.block_n(), gy = (m + v.block_m() - 1) / v.block_m();
+  // persistent: OCC workgroups a CU walk the tiles (the kernel derives gx, gy from m, n)
+  const uint64_t tiles = (uint64_t)gx * gy, slots = (uint64_t)CU_COUNT * v.occ;
+  d->grid[0] = (uint32_t)(tiles < slots ? tiles : slots), d->grid[1] = 1, d->grid[2] = 1;
   d->block[0] = v.threads(), d->block[1] = 1, d->block[2] = 1;
   d->n_launches = 1;
   d->ks = 1;
@@ -175,13 +177,30 @@ int resolve(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *out) 
     const uint32_t nblk = (n + v->block_n() - 1) / v->block_n();
     return describe_dec(*v, m, n, k, decode_split(m, n, k, nblk, v->kw), out);
   }
-  // prefill: the 256 x 256 tile once it fills the card, the 128 x 128 tile below
-  const uint64_t big = (uint64_t)((m + 255) / 256) * ((n + 255) / 256);
-  const std::string name =
-      big >= CU_COUNT ? fmt("macaq_iu8_pf_%s_tn4_lbk64", tag) : fmt("macaq_iu8_pf_%s_t4x4w2x2", tag);
-  const PfVariant *v = pf_variant(name);
-  if (!v) return fail(SABER_IU8_E_RULE, name + ": no such variant");
-  return describe_pf(*v, m, n, k, out);
+  return describe_pf(*pf_cell(wkind == SABER_IU8_W8, m, n, k), m, n, k, out);
+}
+
+// The prefill cell of a shape: the tile whose estimated time is least. A cell's time is its tile
+// work over its measured rate (relative to the 256 x 256 cell) times the rounds the card's 256 CUs
+// need; a partly filled last round counts half, because the card is power-bound under MFMA load and
+// the CUs that do run then clock higher. The rates are this card's speed data (M = 256..8192 sweeps
+// of the four 27B-class shapes), as the reference keeps its band tables
+// (crates/saber-kernels/src/macaq_iu8.rs:150-212).
+const PfVariant *pf_cell(bool w8, uint32_t m, uint32_t n, uint32_t k) {
+  (void)k;
+  static const struct { const char *tile; double rate; } CELLS[] = {
+      {"tn4_lbk64", 1.00}, {"t256x224", 0.92}, {"t256x160", 0.88}, {"t128x128", 0.75}, {"t128x64_o2", 0.55}};
+  const PfVariant *best = nullptr;
+  double best_t = 0;
+  for (const auto &c : CELLS) {
+    const PfVariant *v = pf_variant(fmt("macaq_iu8_pf_%s_%s", w8 ? "w8" : "w4", c.tile));
+    if (!v) continue;
+    const double tiles = (double)((n + v->block_n() - 1) / v->block_n()) * ((m + v->block_m() - 1) / v->block_m());
+    const double full = tiles / CU_COUNT, rounds = full + 0.5 * (std::ceil(full) - full);
+    const double t = rounds * v->block_m() * v->block_n() / c.rate;
+    if (!best || t < best_t * 0.97) best = v, best_t = t;  // a later (smaller) cell must win clearly
+  }
+  return best;
 }
 
 static int describe_rows(const char *op, const char *kernel, uint32_t rows, uint32_t width, const char *wname,

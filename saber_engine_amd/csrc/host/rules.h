@@ -17,14 +17,16 @@ struct DecVariant {
 };
 struct PfVariant {
   const char *name;
-  int w8, wmw, wnw, tm, tn, acc;
-  int block_m() const { return wmw * tm * 16; }
-  int block_n() const { return wnw * tn * 16; }
+  int w8, wmw, wnw, tm, tn, acc, occ;  // waves, 32 x 32 MFMA tiles a wave, workgroups a CU
+  int block_m() const { return wmw * tm * 32; }
+  int block_n() const { return wnw * tn * 32; }
   int threads() const { return wmw * wnw * 64; }
 };
 
 const DecVariant *dec_variant(const std::string &name);
 const PfVariant *pf_variant(const std::string &name);
+// The prefill cell (tile shape) the launch law picks for a shape.
+const PfVariant *pf_cell(bool w8, uint32_t m, uint32_t n, uint32_t k);
 
 constexpr uint32_t DECODE_MAX_M = 64;  // the decode band's last row count (macaq_iu8.rs:31)
 constexpr uint32_t KS_MAX = 8;         // the largest grid-level split (macaq_iu8.rs:44)

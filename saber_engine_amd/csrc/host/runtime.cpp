@@ -409,7 +409,7 @@ int saber_iu8_moe_grouped(saber_iu8_ctx *ctx, const void *a, const float *as, co
     return fail(SABER_IU8_E_RULE, fmt("moe_grouped: tile_blocks %u; the cells are 1 (16-row) and 8 (128-row)", tile_blocks));
   const bool dec = tile_blocks == 1;
   const std::string name = fmt("moe_iu8_grouped_w4_%s_g%d", dec ? "dec" : "pf", gather ? 1 : 0);
-  const uint32_t bn = dec ? 32 : 128, block = dec ? 512 : 256;
+  const uint32_t bn = dec ? 32 : 256, block = 512;
   saber_iu8_desc d;
   if (int rc = raw_desc(name.c_str(), (n + bn - 1) / bn, saber_iu8_moe_tiles_cap(tokens, topk, experts, tile_blocks), block, &d)) return rc;
   set_i32(&d, "n", n);

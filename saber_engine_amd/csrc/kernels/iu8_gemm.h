@@ -9,6 +9,7 @@
 // ones are clamped, never predicated, and never stored.
 #pragma once
 #include "iu8_common.h"
+#include <type_traits>
 
 struct iu8_rows {
   const int *row_tok;  // gather map: expert-major row -> row of A and `as`; nullptr = in place
@@ -304,117 +305,3 @@ __device__ __forceinline__ void iu8_dec_body(const iu8_u8 *__restrict__ A, const
     }
   }
 }
-
-
-// ============================================================================ prefill tile
-template <bool W8, int WMW, int WNW, int TM, int TN, bool ACC>
-__device__ __forceinline__ void iu8_pf_body(const iu8_u8 *__restrict__ A, const iu8_u8 *__restrict__ W,
-                                            const float *__restrict__ as, const float *__restrict__ ws,
-                                            void *__restrict__ Cv, const iu8_rows R, int mbase, int N, int K) {
-  // R: the rows this launch (dense) or this tile (grouped) owns; mbase: the first of them this
-  // workgroup computes
-  constexpr int NTHR = WMW * WNW * 64;
-  constexpr int BMT = WMW * TM, BNT = WNW * TN;  // 16-row tiles a workgroup, both ways
-  constexpr int WSTEP = W8 ? 2048 : 1024;
-  constexpr int A_PIECES = BMT * 128, W_PIECES = BNT * (WSTEP / 16);  // 16-byte pieces a K step
-  constexpr int A_PER = (A_PIECES + NTHR - 1) / NTHR, W_PER = (W_PIECES + NTHR - 1) / NTHR;
-  __shared__ __attribute__((aligned(16))) iu8_u8 sA[BMT * 2048];
-  __shared__ __attribute__((aligned(16))) iu8_u8 sW[BNT * WSTEP];
-
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = wave / WNW, wn = wave % WNW;
-  const int M = R.rows, ntiles = N >> 4, steps = K >> 7, ktiles = K >> 6;
-  const int nt0 = blockIdx.x * BNT;
-
-  // the global side of every piece this thread stages (tiles past the edge re-read the last one)
-  const iu8_u8 *ga[A_PER];
-  const iu8_u8 *gw[W_PER];
-#pragma unroll
-  for (int p = 0; p < A_PER; ++p) {
-    const int piece = p * NTHR + tid;
-    const int within = piece % 128, pl = within & 63;
-    const int ar = iu8_arow(R, mbase + (piece / 128) * 16 + (pl & 15));
-    ga[p] = A + ((size_t)(ar >> 4) * ktiles + (within >> 6)) * 1024 + ((ar & 15) + 16 * (pl >> 4)) * 16;
-  }
-#pragma unroll
-  for (int p = 0; p < W_PER; ++p) {
-    const int piece = p * NTHR + tid;
-    const int nt = min(nt0 + piece / (WSTEP / 16), ntiles - 1);
-    gw[p] = W + (size_t)nt * steps * WSTEP + (piece % (WSTEP / 16)) * 16;
-  }
-
-  iu8_v4i acc[TM][TN];
-#pragma unroll
-  for (int i = 0; i < TM; ++i)
-#pragma unroll
-    for (int j = 0; j < TN; ++j) acc[i][j] = iu8_v4i{0, 0, 0, 0};
-
-  iu8_v4u ra[A_PER], rw[W_PER];
-  auto gload = [&](int s) {
-#pragma unroll
-    for (int p = 0; p < A_PER; ++p)
-      if (A_PIECES % NTHR == 0 || p * NTHR + tid < A_PIECES) ra[p] = *(const iu8_v4u *)(ga[p] + (size_t)s * 2048);
-#pragma unroll
-    for (int p = 0; p < W_PER; ++p)
-      if (W_PIECES % NTHR == 0 || p * NTHR + tid < W_PIECES) rw[p] = iu8_ldg_nt(gw[p] + (size_t)s * WSTEP);
-  };
-  gload(0);
-  for (int s = 0; s < steps; ++s) {
-    __syncthreads();  // every wave is done reading the previous step's fragments
-#pragma unroll
-    for (int p = 0; p < A_PER; ++p)
-      if (A_PIECES % NTHR == 0 || p * NTHR + tid < A_PIECES) *(iu8_v4u *)&sA[(p * NTHR + tid) * 16] = ra[p];
-#pragma unroll
-    for (int p = 0; p < W_PER; ++p)
-      if (W_PIECES % NTHR == 0 || p * NTHR + tid < W_PIECES) *(iu8_v4u *)&sW[(p * NTHR + tid) * 16] = rw[p];
-    __syncthreads();
-    if (s + 1 < steps) gload(s + 1);
-
-    iu8_v4i wf[TN][2];
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      if constexpr (W8) {
-        wf[j][0] = *(const iu8_v4i *)&sW[((wn * TN + j) * 2 + 0) * 1024 + lane * 16];
-        wf[j][1] = *(const iu8_v4i *)&sW[((wn * TN + j) * 2 + 1) * 1024 + lane * 16];
-      } else {
-        iu8_unpack_w4(*(const iu8_v4u *)&sW[(wn * TN + j) * 1024 + lane * 16], wf[j][0], wf[j][1]);
-      }
-    }
-#pragma unroll
-    for (int h = 0; h < 2; ++h)
-#pragma unroll
-      for (int i = 0; i < TM; ++i) {
-        const iu8_v4i af = *(const iu8_v4i *)&sA[((wm * TM + i) * 2 + h) * 1024 + lane * 16];
-#pragma unroll
-        for (int j = 0; j < TN; ++j) acc[i][j] = iu8_mfma(wf[j][h], af, acc[i][j]);
-      }
-  }
-
-  const int ml = lane & 15, nq = (lane >> 4) * 4;
-#pragma unroll
-  for (int j = 0; j < TN; ++j) {
-    const int nt = nt0 + wn * TN + j;
-    if (nt >= ntiles) continue;
-    const int n = nt * 16 + nq;
-    float wsu[4];
-#pragma unroll
-    for (int r = 0; r < 4; ++r) wsu[r] = iu8_wsu<W8>(ws, n + r);
-#pragma unroll
-    for (int i = 0; i < TM; ++i) {
-      const int m = mbase + (wm * TM + i) * 16 + ml;
-      if (m >= M) continue;
-      const size_t crow = (size_t)(R.row0 + m) * N;
-      if constexpr (ACC) {
-        *(iu8_v4i *)((int *)Cv + crow + n) = acc[i][j];
-      } else {
-        const float am = as[iu8_arow(R, m)];
-        unsigned h[4];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) h[r] = iu8_bf16_bits(iu8_epi(acc[i][j][r], am, wsu[r]));
-        *(iu8_v2u *)((unsigned short *)Cv + crow + n) = iu8_v2u{h[0] | (h[1] << 16), h[2] | (h[3] << 16)};
-      }
-    }
-  }
-}
-

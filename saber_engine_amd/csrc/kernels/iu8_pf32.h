@@ -1,0 +1,343 @@
+// The MFMA-bound tile GEMM of the gfx950 W4A8-iu8 path on v_mfma_i32_32x32x32_i8, the int8 MFMA
+// shape that sustains the card's matrix rate. Shared by the dense code object (`macaq_iu8`,
+// persistent workgroups walking an XCD-aware tile order) and the grouped, expert-routed one
+// (`moe_iu8`, one tile of the router's table a workgroup). Operand orders and the contract:
+// iu8_common.h; the row map `iu8_rows`: iu8_gemm.h.
+//
+// A workgroup of WMW x WNW waves owns a (WMW*TM*32) x (WNW*TN*32) output tile and runs its tiles
+// one after another. Each 128-deep K step lives in one of NST LDS stages (A fragments, then W
+// fragments, in their HBM fragment order; W4 stays packed). global_load_lds_dwordx4 moves a
+// fragment per wave-load from HBM/L2 into LDS without touching registers, NST-1 steps ahead of the
+// MFMAs, and the stream of steps runs across tile boundaries: the first steps of the next tile are
+// in flight while the current tile finishes and stores its output.
+//
+// Operand K order. An MFMA contracts over 32 k; lanes 0..31 carry one 16-byte k chunk and lanes
+// 32..63 another, and the sum does not care which chunks as long as both operands agree. A step
+// has 8 chunks c = 4*(k64 half) + (16-byte group); sub-step f = 2p + kt2, lane half h use chunk
+// c = 4*kt2 + 2*p + h. A lane's 16-byte W4 piece then holds the operands of sub-steps 2p (dwords
+// 0,1) and 2p+1 (dwords 2,3), so one LDS read serves two sub-steps.
+//
+// D[n][m]: src0 = weight operand (lane: row n = l%32), src1 = activation operand (lane: row
+// m = l%32); lane l, register e holds n = 8*(e/4) + 4*(l/32) + e%4, m = l%32.
+#pragma once
+#include <type_traits>
+
+#include "iu8_gemm.h"
+
+typedef int iu8_v16i __attribute__((ext_vector_type(16)));
+typedef float iu8_v2f __attribute__((ext_vector_type(2)));
+typedef __bf16 iu8_v2bf __attribute__((ext_vector_type(2)));
+
+// two f32 -> packed bf16, round to nearest even (v_cvt_pk_bf16_f32); lo in bits 0..15
+static __device__ __forceinline__ unsigned iu8_bf16_pack(float lo, float hi) {
+  const iu8_v2bf r = __builtin_convertvector(iu8_v2f{lo, hi}, iu8_v2bf);
+  return *(const unsigned *)&r;
+}
+
+// One tile of work: rows [mbase, mbase + BM) of the row map R against the 16-row weight tiles from
+// nt0 of W (with row scales ws).
+struct iu8_tile {
+  iu8_rows R;
+  int mbase, nt0;
+  const iu8_u8 *W;
+  const float *ws;
+};
+
+// Dense tile order of a persistent launch of G workgroups over gx x gy tiles. The hardware deals
+// consecutive workgroup ids round-robin over the 8 XCDs (each with its own L2): in every round an
+// XCD's G/8 workgroups take one run of consecutive tile ids, and ids walk M-fastest in groups of
+// 8 row blocks, so co-resident workgroups share W columns and A rows in their L2.
+static __device__ __forceinline__ bool iu8_dense_tile_at(int r, int gx, int gy, int &bx, int &by) {
+  const int G = gridDim.x, w = blockIdx.x, total = gx * gy;
+  const int id = (G & 7) == 0 ? ((r * 8 + (w & 7)) * (G >> 3) + (w >> 3)) : (w + r * G);
+  if (id >= total) return false;
+  constexpr int GM = 8;
+  const int group = id / (GM * gx), first = group * GM, gm = min(GM, gy - first);
+  const int rr = id - group * (GM * gx);
+  by = first + rr % gm;
+  bx = rr / gm;
+  return true;
+}
+
+template <bool W8, int WMW, int WNW, int TM, int TN, bool ACC, int STMAX, class TileAt>
+__device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const float *__restrict__ as,
+                                             void *__restrict__ Cv, int N, int K, TileAt tile_at) {
+  // tile_at(r, t): fills the workgroup's r-th tile, false when it has none
+  constexpr int NWAVE = WMW * WNW;
+  constexpr int BMT = WMW * TM * 2, BNT = WNW * TN * 2;  // 16-row tiles a workgroup, both ways
+  constexpr int WSTEP = W8 ? 2048 : 1024;                // bytes of a 16-row weight tile per K step
+  constexpr int A_BYTES = BMT * 2048, W_BYTES = BNT * WSTEP, STAGE = A_BYTES + W_BYTES;
+  // a wave moves whole 1-KiB fragments: wave w moves fragments w, w + NWAVE, ... of A and of W
+  constexpr int A_FR = A_BYTES / 1024, W_FR = W_BYTES / 1024;
+  constexpr int A_PER = (A_FR + NWAVE - 1) / NWAVE, W_PER = (W_FR + NWAVE - 1) / NWAVE;
+  constexpr int PER = A_FR / NWAVE + W_FR / NWAVE;  // wave-loads every wave issues a step (some issue one more)
+  constexpr int NST = STMAX >= 3 && 3 * STAGE <= 160 * 1024 ? 3 : 2;
+  __shared__ __attribute__((aligned(1024))) iu8_u8 smem[NST * STAGE];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WNW, wn = wave % WNW;
+  const int ntiles = N >> 4, steps = K >> 7, ktiles = K >> 6;
+
+  // ---- the load stream: (tile L, step ls), NST-1 steps ahead of the MFMAs
+  // Global -> LDS without registers: global_load_lds_dwordx4 writes lane l's 16 bytes at
+  // (wave-uniform LDS base in m0) + 16*l, so one wave-load lands one fragment in fragment order.
+  // Per lane: the 32-bit byte offset of its piece at K step 0 of the load stream's tile.
+  iu8_tile L;
+  if (!tile_at(0, L)) return;
+  int lr = 0, ls = 0;
+  unsigned ga[A_PER], gw[W_PER];
+  auto set_addr = [&]() {
+#pragma unroll
+    for (int p = 0; p < A_PER; ++p) {
+      const int f = min(p * NWAVE + wave, A_FR - 1);  // fragment (mt = f/2, kt2 = f%2) of the step
+      const int ar = iu8_arow(L.R, L.mbase + (f >> 1) * 16 + (lane & 15));  // rows past the edge: the last one
+      ga[p] = (unsigned)(((size_t)(ar >> 4) * ktiles + (f & 1)) * 1024 + ((ar & 15) + 16 * (lane >> 4)) * 16);
+    }
+#pragma unroll
+    for (int p = 0; p < W_PER; ++p) {
+      const int f = min(p * NWAVE + wave, W_FR - 1);
+      const int nt = min(L.nt0 + f / (WSTEP / 1024), ntiles - 1);  // tiles past N: the last one
+      gw[p] = (unsigned)((size_t)nt * steps * WSTEP + (f % (WSTEP / 1024)) * 1024 + lane * 16);
+    }
+  };
+  set_addr();
+  // The load is written as asm: the compiler models an LDS-DMA load as touching both memories and
+  // then drains every counter to zero at each later LDS read, which would serialise the operand
+  // pipeline below. Its completion is tracked by hand (vmcnt, before the step's barrier).
+  // m0 = LDS address of the wave's fragment; one wait state between the m0 write and its use.
+  auto dma = [&](const iu8_u8 *base, unsigned off, unsigned lds) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(lds), "v"(off), "s"(base)
+                 : "memory", "m0");
+  };
+  const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) iu8_u8 *)smem;
+  auto issue = [&](int stage) {  // the load stream's step -> LDS stage
+    const unsigned sA = lds0 + stage * STAGE, sW = sA + A_BYTES;
+    const iu8_u8 *As = A + (size_t)ls * 2048, *Ws = L.W + (size_t)ls * WSTEP;
+#pragma unroll
+    for (int p = 0; p < A_PER; ++p)
+      if (A_FR % NWAVE == 0 || p * NWAVE + wave < A_FR) dma(As, ga[p], sA + (p * NWAVE + wave) * 1024);
+#pragma unroll
+    for (int p = 0; p < W_PER; ++p)
+      if (W_FR % NWAVE == 0 || p * NWAVE + wave < W_FR) dma(Ws, gw[p], sW + (p * NWAVE + wave) * 1024);
+  };
+  auto advance = [&]() {  // next step of the stream; past the last tile it keeps re-loading the last step
+    if (++ls == steps) {
+      iu8_tile T;
+      if (tile_at(lr + 1, T)) {
+        ++lr, ls = 0, L = T;
+        set_addr();
+      } else {
+        ls = steps - 1;
+      }
+    }
+  };
+  // s_waitcnt vmcnt(n) [lgkmcnt(0)] (gfx9 encoding: vmcnt = imm[3:0] | imm[15:14] << 4, expcnt open)
+  auto wait_vm = [&](auto n, bool lgkm0) {
+    constexpr int NN = decltype(n)::value;
+    if (lgkm0) __builtin_amdgcn_s_waitcnt((NN & 15) | ((NN >> 4) << 14) | (7 << 4) | (0 << 8));
+    else __builtin_amdgcn_s_waitcnt((NN & 15) | ((NN >> 4) << 14) | (7 << 4) | (15 << 8));
+  };
+  // Loads that may still fly at a step's barrier: the newest step's. Counted with the fewest a
+  // wave issues, so a wave that issued one more waits for that one too.
+  using InFlight = std::integral_constant<int, (NST - 2) * PER>;
+
+  // this lane's operand addresses inside a stage, at sub-step 0
+  const int r32 = lane & 31, h = lane >> 5;
+  // A: fragment (mt, kt2) at (mt*2 + kt2) KiB; piece (chunk*16 + row%16)
+  const int a_lane = (((wm * TM * 2 + (r32 >> 4)) * 2) * 64 + h * 16 + (r32 & 15)) * 16;
+  // W4: fragment nt at nt KiB; W8: the A form
+  const int w_lane = W8 ? (((wn * TN * 2 + (r32 >> 4)) * 2) * 64 + h * 16 + (r32 & 15)) * 16
+                        : ((wn * TN * 2 + (r32 >> 4)) * 64 + h * 16 + (r32 & 15)) * 16;
+
+  // ---- the pipelined K loop. A step is four phases (sub-steps) f = 2p + kt2. Nothing is consumed
+  // in the phase that fetched it: a phase's MFMAs multiply A operands read from LDS one phase
+  // earlier (register set f&1) with W operands unpacked just in time from packed pieces read at
+  // least one phase earlier (wpk[p]; 16-byte reads of consecutive lanes are free of bank conflicts,
+  // 8-byte reads at this stride are not). The unpack of column tile j+1 issues while the MFMAs of
+  // column tile j run. The step's one barrier sits before the last phase, whose operands are
+  // already in registers: behind it the first operands of the next step are read from the next
+  // stage, and the stage just drained is free for the loads of NST-1 steps ahead.
+  iu8_v16i acc[TM][TN];
+  iu8_v4i af[2][TM] = {};
+  iu8_v4i wf[W8 ? 2 : 1][TN] = {};
+  iu8_v4u wpk[2][W8 ? 1 : TN] = {};
+  auto fetch_a = [&](const iu8_u8 *sA, int buf, int p, int kt2) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i) af[buf][i] = *(const iu8_v4i *)&sA[a_lane + i * 4096 + kt2 * 1024 + p * 512];
+  };
+  auto fetch_w8 = [&](const iu8_u8 *sW, int buf, int p, int kt2) {  // W8: a whole operand a phase
+    if constexpr (W8) {
+#pragma unroll
+      for (int j = 0; j < TN; ++j) wf[buf][j] = *(const iu8_v4i *)&sW[w_lane + j * 4096 + kt2 * 1024 + p * 512];
+    }
+  };
+  auto fetch_w4 = [&](const iu8_u8 *sW, int p) {  // W4: the packed pieces of sub-steps 2p, 2p+1
+    if constexpr (!W8) {
+#pragma unroll
+      for (int j = 0; j < TN; ++j) wpk[p][j] = *(const iu8_v4u *)&sW[w_lane + j * 2048 + p * 512];
+    }
+  };
+  auto mfmas = [&](int buf, int p, int kt2) {
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      if constexpr (!W8) {
+        const unsigned d0 = kt2 ? wpk[p][j].z : wpk[p][j].x, d1 = kt2 ? wpk[p][j].w : wpk[p][j].y;
+        wf[0][j] = iu8_v4i{(int)((d0 << 4) & 0xF0F0F0F0u), (int)(d0 & 0xF0F0F0F0u), (int)((d1 << 4) & 0xF0F0F0F0u),
+                           (int)(d1 & 0xF0F0F0F0u)};
+      }
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[W8 ? buf : 0][j], af[buf][i], acc[i][j], 0, 0, 0);
+    }
+  };
+  // Instruction order inside a phase (the machine scheduler follows these groups): the phase's LDS
+  // reads, the first column tile's unpack, then per column tile its MFMAs with the next one's unpack
+  // issued behind them.
+  constexpr int UNPK = W8 ? 0 : 6;  // VALU ops of one piece-half unpack
+#define IU8_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
+#define IU8_PHASE_ORDER(NDS)                          \
+  IU8_SGB(0x100, NDS);                                \
+  if (UNPK) IU8_SGB(0x002, UNPK);                     \
+  _Pragma("unroll") for (int j_ = 0; j_ < TN; ++j_) { \
+    IU8_SGB(0x008, TM);                               \
+    if (UNPK && j_ + 1 < TN) IU8_SGB(0x002, UNPK);    \
+  }                                                   \
+  __builtin_amdgcn_sched_barrier(0)
+
+  issue(0);
+  advance();
+  if constexpr (NST == 3) {
+    issue(1);
+    advance();
+  }
+  wait_vm(InFlight{}, false);
+  __builtin_amdgcn_s_barrier();
+  fetch_a(smem, 0, 0, 0);
+  fetch_w8(smem + A_BYTES, 0, 0, 0);
+  fetch_w4(smem + A_BYTES, 0);
+  __builtin_amdgcn_sched_barrier(0);
+
+  iu8_tile C = L;
+  tile_at(0, C);
+  int st = 0;  // stage of the MFMAs' step
+  for (int r = 0;; ++r) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
+
+    for (int s = 0; s < steps; ++s) {
+      const int st1 = st == NST - 1 ? 0 : st + 1, stl = st == 0 ? NST - 1 : st - 1;  // next, last
+      const iu8_u8 *sA = smem + st * STAGE, *sW = sA + A_BYTES;
+      const iu8_u8 *nA = smem + st1 * STAGE, *nW = nA + A_BYTES;
+      // phase 0; the load stream's step leaves HBM for the stage drained last
+      fetch_a(sA, 1, 0, 1);
+      fetch_w8(sW, 1, 0, 1);
+      fetch_w4(sW, 1);
+      issue(stl);
+      mfmas(0, 0, 0);
+      IU8_PHASE_ORDER(TM + TN);
+      // phase 1
+      fetch_a(sA, 0, 1, 0);
+      fetch_w8(sW, 0, 1, 0);
+      mfmas(1, 0, 1);
+      IU8_PHASE_ORDER(TM + (W8 ? TN : 0));
+      // phase 2
+      fetch_a(sA, 1, 1, 1);
+      fetch_w8(sW, 1, 1, 1);
+      mfmas(0, 1, 0);
+      IU8_PHASE_ORDER(TM + (W8 ? TN : 0));
+      // phase 3, behind the barrier: every wave's reads of this stage are done and the next step's
+      // fragments have landed
+      wait_vm(InFlight{}, true);
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+      fetch_a(nA, 0, 0, 0);
+      fetch_w8(nW, 0, 0, 0);
+      fetch_w4(nW, 0);
+      mfmas(1, 1, 1);
+      IU8_PHASE_ORDER(TM + TN);
+      advance();
+      st = st1;
+    }
+
+    // ---- epilogue of tile C. The stage the last step drained is free (the barrier of that step's
+    // last phase came after every wave's reads of it); the other stages hold the next tile's first
+    // steps.
+    const int M = C.R.rows;
+    const int nq = h * 4;
+    const int ncol0 = (C.nt0 + wn * TN * 2) * 16;  // first column of the wave tile
+    if constexpr (ACC) {
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int n = ncol0 + j * 32 + g * 8 + nq;
+          if (n >= N) continue;
+#pragma unroll
+          for (int i = 0; i < TM; ++i) {
+            const int m = C.mbase + (wm * TM + i) * 32 + r32;
+            if (m >= M) continue;
+            *(iu8_v4i *)((int *)Cv + (size_t)(C.R.row0 + m) * N + n) =
+                iu8_v4i{acc[i][j][g * 4], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
+          }
+        }
+    } else {
+      // Through LDS: a lane holds 4 consecutive columns of one row, so direct stores would touch 32
+      // rows with 16 bytes each. Each wave turns a block of 32 rows x CB*32 columns at a time into
+      // row-major bf16 in its own LDS region (rows padded by 16 bytes) and stores whole row
+      // segments, 16 bytes a lane.
+      constexpr int CB = TN % 2 == 0 && NWAVE * 32 * (2 * 64 + 16) <= STAGE ? 2 : 1;  // 32-column tiles a block
+      constexpr int ROWB = CB * 64 + 16, LPR = CB * 4, PIECES = 32 * LPR;
+      static_assert(NWAVE * 32 * ROWB <= STAGE, "the epilogue region fits one stage");
+      iu8_u8 *reg = smem + (st == 0 ? NST - 1 : st - 1) * STAGE + wave * (32 * ROWB);
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        const int m = C.mbase + (wm * TM + i) * 32 + r32;
+        const float am = as[iu8_arow(C.R, min(m, M - 1))];
+#pragma unroll
+        for (int jb = 0; jb < TN / CB; ++jb) {
+#pragma unroll
+          for (int jj = 0; jj < CB; ++jj) {
+            const int j = jb * CB + jj;
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+              const int nl = jj * 32 + g * 8 + nq;
+              const int n = min(ncol0 + jb * (CB * 32) + nl, N - 4);
+              const float4 w4 = *(const float4 *)(C.ws + n);
+              const float u = W8 ? 1.f : 0.0625f;  // exact: a power of two
+              const unsigned lo = iu8_bf16_pack(iu8_epi(acc[i][j][g * 4], am, w4.x * u),
+                                                iu8_epi(acc[i][j][g * 4 + 1], am, w4.y * u));
+              const unsigned hi = iu8_bf16_pack(iu8_epi(acc[i][j][g * 4 + 2], am, w4.z * u),
+                                                iu8_epi(acc[i][j][g * 4 + 3], am, w4.w * u));
+              *(iu8_v2u *)&reg[r32 * ROWB + nl * 2] = iu8_v2u{lo, hi};
+            }
+          }
+          __builtin_amdgcn_wave_barrier();
+#pragma unroll
+          for (int q0 = 0; q0 < PIECES; q0 += 64) {
+            const int q = q0 + lane, row = q / LPR, pc = q % LPR;
+            const int mm = C.mbase + (wm * TM + i) * 32 + row, nn = ncol0 + jb * (CB * 32) + pc * 8;
+            if ((PIECES % 64 == 0 || q < PIECES) && mm < M && nn < N)
+              *(iu8_v4u *)((unsigned short *)Cv + (size_t)(C.R.row0 + mm) * N + nn) =
+                  *(const iu8_v4u *)&reg[row * ROWB + pc * 16];
+          }
+          __builtin_amdgcn_wave_barrier();
+        }
+      }
+    }
+    if (!tile_at(r + 1, C)) break;
+    // every wave is done with the epilogue region before the next step's loads land in that stage
+    wait_vm(std::integral_constant<int, 63>{}, true);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+  }
+#undef IU8_PHASE_ORDER
+#undef IU8_SGB
+  wait_vm(std::integral_constant<int, 0>{}, true);
+}

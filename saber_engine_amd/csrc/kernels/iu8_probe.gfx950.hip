@@ -72,3 +72,36 @@ extern "C" __global__ __launch_bounds__(256) void iu8_probe_mfma32(unsigned *__r
     for (int e = 0; e < 16; ++e) s ^= c[j][e];
   if (s == 0x12345679) out[0] = s;
 }
+
+// The matrix rate with real operands: every lane loads 4 + 4 operands from `src` once (random
+// bytes or zeros, the caller's choice) and runs the 4 x 4 tile pattern of the prefill GEMM,
+// 16 v_mfma_i32_32x32x32_i8 an iteration on 16 accumulator tiles. Same code, different data:
+// the difference is what the card's power management takes off the clock.
+extern "C" __global__ __launch_bounds__(256) void iu8_probe_mfma32d(const unsigned char *__restrict__ src,
+                                                                    unsigned *__restrict__ out, int n) {
+  const iu8_v4i *p = (const iu8_v4i *)src + (size_t)(blockIdx.x * 256 + threadIdx.x) * 8;
+  iu8_v4i a[4], b[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) a[i] = p[i], b[i] = p[4 + i];
+  iu8_v16i c[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) c[i][j][e] = 0;
+  for (int it = 0; it < n; ++it) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) c[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(b[j], a[i], c[i][j], 0, 0, 0);
+  }
+  int s = 0;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) s ^= c[i][j][e];
+  if (s == 0x12345679) out[0] = s;
+}

@@ -18,12 +18,13 @@
 //           (gridDim.z) goes through the `decode_partial` / `decode_counter` workspaces with the
 //           last-arriving workgroup summing; it costs device-scope fences across the 8 XCDs' L2s
 //           and the launch law does not use it by default.
-//   prefill (M > 64)   MFMA-bound tile GEMM. A workgroup of WMW x WNW waves owns a
-//           (WMW*TM*16) x (WNW*TN*16) output tile; A and W fragments of one 128-deep K step are
-//           staged in LDS in fragment order (W4 stays packed; the unpack happens after the LDS
-//           read, once per fragment, and is reused across the wave's TM row tiles), with the next
-//           step's global loads in flight during the MFMAs.
+//   prefill (M > 64)   MFMA-bound tile GEMM on v_mfma_i32_32x32x32_i8 (iu8_pf32.h): persistent
+//           workgroups of 8 waves (two a SIMD) walk an XCD-aware tile order; the fragments of a
+//           128-deep K step go from HBM/L2 into one of three LDS stages by LDS-DMA loads, two steps
+//           ahead of the MFMAs and across tile boundaries; W4 stays packed in LDS and is unpacked
+//           in registers just in time; the output tile goes out through LDS as whole row segments.
 #include "iu8_gemm.h"
+#include "iu8_pf32.h"
 
 #define IU8_DEC(name, TM, W8, NT, KW, WPB, D, ALDS, ACC)                                                         \
   extern "C" __global__ __launch_bounds__(WPB * 64) void name(                                                    \
@@ -34,22 +35,31 @@
                                                     iu8_rows{nullptr, 0, m}, n, k);     \
   }
 #define IU8_DEC_VARIANT(name, TM, W8, NT, KW, WPB, D, ALDS, ACC) IU8_DEC(name, TM, W8, NT, KW, WPB, D, ALDS, ACC)
-#define IU8_PF_VARIANT(name, W8, WMW, WNW, TM, TN, ACC)
+#define IU8_PF_VARIANT(name, W8, WMW, WNW, TM, TN, ACC, ST, OCC)
 #include "iu8_variants.def"
 #undef IU8_DEC_VARIANT
 #undef IU8_PF_VARIANT
 #undef IU8_DEC
 
-#define IU8_PF(name, W8, WMW, WNW, TM, TN, ACC)                                                                  \
-  extern "C" __global__ __launch_bounds__(WMW * WNW * 64) void name(                                              \
+// Persistent launch: gridDim.x workgroups (one or OCC a CU) walk the tiles of the m x n output.
+#define IU8_PF32(name, W8, WMW, WNW, TM, TN, ACC, ST, OCC)                                                        \
+  extern "C" __global__ __launch_bounds__(WMW * WNW * 64)                                                         \
+      __attribute__((amdgpu_waves_per_eu(WMW * WNW * OCC / 4, WMW * WNW * OCC / 4))) void name(                    \
       const unsigned char *__restrict__ a, const unsigned char *__restrict__ w, const float *__restrict__ as,     \
       const float *__restrict__ ws, unsigned short *__restrict__ c, int m, int n, int k) {                         \
-    iu8_pf_body<W8, WMW, WNW, TM, TN, ACC>(a, w, as, ws, c, iu8_rows{nullptr, 0, m},                            \
-                                           (int)blockIdx.y * (WMW * TM * 16), n, k);                                              \
+    constexpr int BM = WMW * TM * 32, BN = WNW * TN * 32;                                                          \
+    const int gx = (n + BN - 1) / BN, gy = (m + BM - 1) / BM;                                                      \
+    const iu8_rows R{nullptr, 0, m};                                                                               \
+    iu8_pf32_run<W8, WMW, WNW, TM, TN, ACC, ST>(a, as, c, n, k, [&](int r, iu8_tile &t) {                          \
+      int bx, by;                                                                                                  \
+      if (!iu8_dense_tile_at(r, gx, gy, bx, by)) return false;                                                     \
+      t = iu8_tile{R, by * BM, bx * (BN / 16), w, ws};                                                             \
+      return true;                                                                                                 \
+    });                                                                                                            \
   }
 #define IU8_DEC_VARIANT(name, TM, W8, NT, KW, WPB, D, ALDS, ACC)
-#define IU8_PF_VARIANT(name, W8, WMW, WNW, TM, TN, ACC) IU8_PF(name, W8, WMW, WNW, TM, TN, ACC)
+#define IU8_PF_VARIANT(name, W8, WMW, WNW, TM, TN, ACC, ST, OCC) IU8_PF32(name, W8, WMW, WNW, TM, TN, ACC, ST, OCC)
 #include "iu8_variants.def"
 #undef IU8_DEC_VARIANT
 #undef IU8_PF_VARIANT
-#undef IU8_PF
+#undef IU8_PF32

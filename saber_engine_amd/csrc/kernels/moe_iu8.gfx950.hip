@@ -21,6 +21,7 @@
 //   moe_iu8_combine_bf16   out[t] = bf16(sum_k w[t,k] * f32(Y[pos(t,k)])), f32 adds in top-k order,
 //        one rounding (crates/saber-kernels/hip/moe_route.hip:287-329; abi.rs:377-385).
 #include "iu8_gemm.h"
+#include "iu8_pf32.h"
 
 #define MOE_E 128
 #define MOE_TOPK 8
@@ -295,13 +296,17 @@ MOE_GROUPED_DEC(moe_iu8_grouped_w4_dec_g0, false, 1, 4, 8, 8, 20)
     const int tile = blockIdx.y;                                                                                   \
     if (tile >= meta[0]) return;                                                                                   \
     const int e = tile_expert[tile];                                                                               \
-    const iu8_rows R{GATHER ? row_tok : nullptr, tile_row0[tile], min(tile_rows[tile], WMW * TM * 16)};            \
-    iu8_pf_body<false, WMW, WNW, TM, TN, false>(a, (const unsigned char *)xptr[2 * e], as,                         \
-                                                (const float *)xptr[2 * e + 1], c, R, 0, n, k);                    \
+    const iu8_rows R{GATHER ? row_tok : nullptr, tile_row0[tile], min(tile_rows[tile], WMW * TM * 32)};            \
+    iu8_pf32_run<false, WMW, WNW, TM, TN, false, 3>(a, as, c, n, k, [&](int r, iu8_tile &t) {                      \
+      if (r != 0) return false;                                                                                    \
+      t = iu8_tile{R, 0, (int)blockIdx.x * (WNW * TN * 2), (const unsigned char *)xptr[2 * e],                     \
+                   (const float *)xptr[2 * e + 1]};                                                                \
+      return true;                                                                                                 \
+    });                                                                                                            \
   }
-// tiles of up to 128 rows (tile_blocks 8) on the 128 x 128 tile of 2 x 2 waves
-MOE_GROUPED_PF(moe_iu8_grouped_w4_pf_g1, true, 2, 2, 4, 4)
-MOE_GROUPED_PF(moe_iu8_grouped_w4_pf_g0, false, 2, 2, 4, 4)
+// tiles of up to 128 rows (tile_blocks 8) on the 128 x 256 tile of 4 x 2 waves
+MOE_GROUPED_PF(moe_iu8_grouped_w4_pf_g1, true, 4, 2, 1, 4)
+MOE_GROUPED_PF(moe_iu8_grouped_w4_pf_g0, false, 4, 2, 1, 4)
 #undef MOE_GROUPED_PF
 
 // ---------------------------------------------------------------------------- combine

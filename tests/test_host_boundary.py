@@ -89,12 +89,32 @@ def test_explicit_split_declares_its_workspaces():
     assert d.arg("decode_partial").kind == iu8.ARG_BUFFER
 
 
-def test_prefill_grid_covers_the_output():
-    for (m, n, k) in [(256, 5120, 5120), (2048, 34816, 5120), (300, 304, 640), (8192, 7168, 5120)]:
-        d = iu8.resolve(iu8.W4, m, n, k)
-        name = d.kernel.decode()
-        bm, bn = (256, 256) if name.endswith("tn4_lbk64") else (128, 128)
-        assert d.grid[0] == -(-n // bn) and d.grid[1] == -(-m // bm) and d.grid[2] == 1 and d.block[0] == 256
+PF_CELLS = {  # tile suffix -> (rows, columns, workgroups a CU, threads)
+    "tn4_lbk64": (256, 256, 1, 512), "t256x224": (256, 224, 1, 512), "t256x160": (256, 160, 1, 512),
+    "t128x128": (128, 128, 1, 512), "t128x128_o2": (128, 128, 2, 256), "t128x64_o2": (128, 64, 2, 256)}
+
+
+def test_prefill_launch_is_persistent_and_covers_the_output():
+    for wk, tag in ((iu8.W4, "w4"), (iu8.W8, "w8")):
+        for (m, n, k) in [(256, 5120, 5120), (2048, 34816, 5120), (300, 304, 640), (8192, 7168, 5120), (65, 16, 128)]:
+            d = iu8.resolve(wk, m, n, k)
+            name = d.kernel.decode()
+            assert name.startswith(f"macaq_iu8_pf_{tag}_")
+            bm, bn, occ, thr = PF_CELLS[name[len(f"macaq_iu8_pf_{tag}_"):]]
+            tiles = -(-n // bn) * -(-m // bm)
+            # one workgroup (or two) a CU walks the tiles; the kernel derives the tile grid from m, n
+            assert d.grid[0] == min(tiles, 256 * occ) and d.grid[1] == 1 and d.grid[2] == 1 and d.block[0] == thr
+            assert d.n_workspaces == 0 and d.ks == 1
+
+
+def test_prefill_cells_of_the_benchmark_shapes():
+    # speed data of this card: the cell that was fastest in the sweep of each shape
+    want = {(2048, 34816, 5120): "tn4_lbk64", (2048, 7168, 5120): "tn4_lbk64", (2048, 5120, 17408): "t256x160",
+            (2048, 5120, 5120): "t256x160", (8192, 34816, 5120): "tn4_lbk64", (256, 5120, 17408): "t128x64_o2"}
+    for (m, n, k), tile in want.items():
+        assert iu8.resolve(iu8.W4, m, n, k).kernel.decode() == "macaq_iu8_pf_w4_" + tile, (m, n, k)
+    with pytest.raises(iu8.IU8Error):
+        iu8.describe("macaq_iu8_pf_w4_tn4_lbk64", 256, 5120, 5120, ks=2)   # the prefill tile does not split K
 
 
 # ------------------------------------------------------------------ kernarg ABI
