@@ -73,6 +73,22 @@ def test_every_prefill_variant_gives_the_same_bytes(ctx, tag, w8):
         np.testing.assert_array_equal(run.C, r["C"])
 
 
+@pytest.mark.parametrize("shape", [(65, 16, 128), (97, 48, 256), (129, 304, 384), (4160, 1088, 256)])
+def test_prefill_edges_on_every_tile(ctx, shape):
+    """One K step, two K steps (fewer than the LDS stages), ragged rows and columns, a tile count
+    above the persistent grid (several tiles a workgroup, the load stream running across tiles)."""
+    M, N, K = shape
+    for tag, w8 in (("w4", False), ("w8", True)):
+        case = synth.dense_case(M, N, K, w8=w8, seed=31 + M)
+        r = ref.linear(case["X"], case["W"], case["ws"], w8, threads=8)
+        for name in all_variants(f"macaq_iu8_pf_{tag}_"):
+            say(f"prefill edge {shape} {name}")
+            run = DenseRun(ctx, case, kernel=name, want_acc=False)
+            np.testing.assert_array_equal(run.C, r["C"])
+        run = DenseRun(ctx, case, want_acc=True)            # the launch law's cell and the int32 tap
+        assert_dense_matches(run, r, w8)
+
+
 def test_split_counter_is_reusable_across_launches(ctx):
     say("explicit split, two launches on one counter")
     case = synth.dense_case(3, 256, 2048, seed=23)
