@@ -27,6 +27,10 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0      # MI355X published HBM3E bandwidth
 INT8_PEAK_TOPS = 5000.0     # MI355X published dense int8 MFMA peak
 LAYERS = 6                  # distinct weight copies walked by successive steps (6 x 165 MB)
+# HBM-side bytes of one launch of the dominant kernel, mean over the four layer shapes, from
+# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this very command (profiles/*hbm_counters*.txt), each
+# counter scaled by what it reads for the 256 MiB copy probe. Keyed by (kernel, M); None = not measured.
+TRAFFIC = {}
 
 
 def alg_bytes(m, n, k, w8=False):
@@ -79,6 +83,9 @@ def main():
         dev_as[name] = torch.zeros(M, dtype=torch.float32, device=dev)
         dev_c[name] = torch.zeros((M, n), dtype=torch.int16, device=dev)
     descs = {name: iu8.resolve(iu8.W4, M, n, k) for name, n, k in linears}
+    # one launch a linear (quantisation fused into the GEMV's activation staging) where every shape allows
+    fused = all(iu8.fused_holds(M, k) for _, _, k in linears)
+    fdescs = {name: iu8.resolve_fused(iu8.W4, M, n, k) for name, n, k in linears} if fused else {}
     qdescs = {name: iu8.resolve_quant(M, k) for name, n, k in linears}
     pbytes = max([d.workspace("decode_partial").bytes for d in descs.values() if d.ks > 1] + [4])
     cbytes = max([d.workspace("decode_counter").bytes for d in descs.values() if d.ks > 1] + [4])
@@ -106,17 +113,31 @@ def main():
         b["as"] = dev_as[name].data_ptr()
         ctx.launch(descs[name], b, sh)
 
-    def step(i, gemm_only=False):
+    def launch_fused(name, layer):
+        # the optional code / scale outputs stay unbound: the step needs the bf16 output only
+        d = fdescs[name]
+        for i in range(d.n_args):
+            if d.args[i].name in (b"q", b"scale"):
+                d.args[i].kind = iu8.ARG_NULL_BUFFER
+        ctx.launch(d, dict(x=dev_x[name].data_ptr(), w=dev_w[name][layer].data_ptr(), ws=dev_ws[name].data_ptr(),
+                           c=dev_c[name].data_ptr()), sh)
+
+    def step(i, mode="hot"):
+        """hot: the path as a caller runs it (fused launch where the shapes allow, else producer +
+        GEMM); two: always producer + GEMM; gemm: the GEMM launches alone."""
         for name, _, _ in linears:
-            if not gemm_only:
+            if mode == "hot" and fused:
+                launch_fused(name, i % LAYERS)
+                continue
+            if mode != "gemm":
                 launch_quant(name)
             launch_gemm(name, i % LAYERS)
 
-    def capture(nsteps, gemm_only=False):
+    def capture(nsteps, mode="hot"):
         g = torch.cuda.CUDAGraph()
         with torch.cuda.graph(g, stream=stream):
             for i in range(nsteps):
-                step(i, gemm_only)
+                step(i, mode)
         return g
 
     with torch.cuda.stream(stream):
@@ -124,9 +145,11 @@ def main():
             step(i)
     stream.synchronize()
     g_all = capture(K_steps)
-    g_gemm = capture(K_steps, gemm_only=True)
+    g_two = capture(K_steps, "two")
+    g_gemm = capture(K_steps, "hot" if fused else "gemm")
     with torch.cuda.stream(stream):
         g_all.replay()
+        g_two.replay()
         g_gemm.replay()
     torch.cuda.synchronize()
 
@@ -141,7 +164,15 @@ def main():
     step_bytes = sum(alg_bytes(M, n, k) for _, n, k in linears)
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
 
-    # ---- the dominant kernel alone (decode GEMM, 4 launches a step), HIP events on its stream
+    # ---- the same K steps as producer + GEMM launches (what the fused launch replaces)
+    torch.cuda.synchronize()
+    t2 = time.perf_counter()
+    with torch.cuda.stream(stream):
+        g_two.replay()
+    torch.cuda.synchronize()
+    two_ms = (time.perf_counter() - t2) * 1e3 / K_steps
+
+    # ---- the dominant kernel alone (the decode GEMV, 4 launches a step), HIP events on its stream
     ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     with torch.cuda.stream(stream):
         ev0.record(stream)
@@ -149,12 +180,18 @@ def main():
         ev1.record(stream)
     torch.cuda.synchronize()
     gemm_us = ev0.elapsed_time(ev1) * 1e3 / (K_steps * len(linears))
-    gemm_bytes = sum(alg_bytes(M, n, k) - 2 * M * k + M * k + 4 * M for _, n, k in linears) / len(linears)
+    if fused:   # reads the bf16 rows itself
+        gemm_bytes = sum(alg_bytes(M, n, k) for _, n, k in linears) / len(linears)
+        kname = fdescs["down"].kernel.decode()
+    else:       # reads the int8 codes and the row scales
+        gemm_bytes = sum(alg_bytes(M, n, k) - 2 * M * k + M * k + 4 * M for _, n, k in linears) / len(linears)
+        kname = descs["down"].kernel.decode()
     achieved = gemm_bytes / (gemm_us * 1e-6) / 1e9
-    roofline = dict(bound="hbm", kernel=descs["down"].kernel.decode(), achieved=round(achieved, 1), peak=HBM_PEAK_GBPS,
-                    unit="GB/s", frac=round(achieved / HBM_PEAK_GBPS, 4), traffic=None,
+    roofline = dict(bound="hbm", kernel=kname, achieved=round(achieved, 1), peak=HBM_PEAK_GBPS,
+                    unit="GB/s", frac=round(achieved / HBM_PEAK_GBPS, 4), traffic=TRAFFIC.get((kname, M)),
                     avg_launch_us=round(gemm_us, 3), bytes_per_launch=gemm_bytes,
-                    note="mean over the four layer shapes, cold weights (rotating %d copies), graph replay" % LAYERS)
+                    note="mean over the four layer shapes, cold weights (rotating %d copies), graph replay; traffic = "
+                         "FETCH_SIZE + WRITE_SIZE per launch (rocprofv3 --pmc, scaled by the copy probe), see profiles/" % LAYERS)
 
     # ---- parity spot check against the CPU oracle, and the CPU baseline beside it
     out = dict(metric="W4A8 GEMM GB/s (%HBM) at M=1; int8 TOPS (%MFMA peak) at M=2048", value=round(value, 1), unit="GB/s",
@@ -162,7 +199,9 @@ def main():
                scaling="weak", vs_baseline=None, dtype="int4 x int8 -> int32 -> bf16", data="synthetic (seed 0)",
                config=dict(workload="configs[1]: decode-batch W4A8 linear set of one 27B-class layer (QKV, O, gate+up, down), "
                                     "hidden 5120, TP=1", m=M, layers_rotated=LAYERS, cold=True,
-                           launches_per_step=2 * len(linears), hbm_frac=round(value / HBM_PEAK_GBPS, 4)),
+                           launches_per_step=(1 if fused else 2) * len(linears), fused_quant=fused,
+                           hbm_frac=round(value / HBM_PEAK_GBPS, 4),
+                           two_launch_gbps=round(step_bytes / (two_ms * 1e-3) / 1e9, 1)),
                roofline=roofline)
 
     if not args.no_cpu:

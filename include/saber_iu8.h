@@ -206,6 +206,18 @@ int saber_iu8_launch(saber_iu8_ctx *ctx, const saber_iu8_desc *desc, const saber
 /* Per-token int8 quantisation: x bf16 [m,k] -> q (A edge, saber_iu8_a_bytes) + scale f32 [m]. */
 int saber_iu8_quant(saber_iu8_ctx *ctx, const void *x_bf16, void *q, float *scale, uint32_t m, uint32_t k, void *stream);
 
+/* The whole decode linear in one launch where the shape allows (at most 4 rows whose codes fit the
+ * kernel's 20 KiB staging area; saber_iu8_fused_holds): per-token quantisation fused into the
+ * GEMV's activation staging. x bf16 [m,k]; q (A edge) and scale f32 [m] are optional outputs (NULL:
+ * not stored) with the bytes saber_iu8_quant would write. Other shapes are refused
+ * (SABER_IU8_E_RULE): run saber_iu8_quant + saber_iu8_gemm. No counterpart among the reference's
+ * iu8 symbols (its fusions put the quantisation behind norm/activation producers,
+ * crates/saber-kernels/src/macaq_iu8.rs:864-875); the law and the bytes are the same. */
+int saber_iu8_fused_holds(uint32_t m, uint32_t k);
+int saber_iu8_resolve_fused(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *out);
+int saber_iu8_linear_fused(saber_iu8_ctx *ctx, int wkind, const void *x_bf16, const void *w, const float *ws,
+                           void *c_bf16, void *q, float *scale, uint32_t m, uint32_t n, uint32_t k, void *stream);
+
 /* Workspace bytes the resolved GEMM needs (both 0 when it does not split). */
 int saber_iu8_gemm_workspace(int wkind, uint32_t m, uint32_t n, uint32_t k, uint64_t *partial_bytes,
                              uint64_t *counter_bytes);

@@ -9,6 +9,9 @@ static const Signature SIG_DEC = {{"a", K::Buffer},  {"w", K::Buffer},
                                   {"decode_partial", K::Buffer}, {"decode_counter", K::Buffer},
                                   {"c", K::Buffer},  {"m", K::I32},
                                   {"n", K::I32},     {"k", K::I32}};
+static const Signature SIG_DECQ = {{"x", K::Buffer},     {"w", K::Buffer}, {"ws", K::Buffer}, {"q", K::Buffer},
+                                   {"scale", K::Buffer}, {"c", K::Buffer}, {"m", K::I32},     {"n", K::I32},
+                                   {"k", K::I32}};
 static const Signature SIG_PF = {{"a", K::Buffer}, {"w", K::Buffer}, {"as", K::Buffer}, {"ws", K::Buffer},
                                  {"c", K::Buffer}, {"m", K::I32},    {"n", K::I32},     {"k", K::I32}};
 static const Signature SIG_QUANT = {{"x", K::Buffer}, {"q", K::Buffer}, {"scale", K::Buffer}, {"k", K::I32}};
@@ -39,6 +42,7 @@ static bool starts(const std::string &s, const char *p) { return s.rfind(p, 0) =
 
 const Signature *signature_for(const std::string &k) {
   if (starts(k, "macaq_iu8_dec_")) return &SIG_DEC;
+  if (starts(k, "macaq_iu8_decq_")) return &SIG_DECQ;
   if (starts(k, "macaq_iu8_pf_")) return &SIG_PF;
   if (starts(k, "macaq_i8_quant_")) return &SIG_QUANT;
   if (starts(k, "macaq_i8_silu_mul_quant_")) return &SIG_SILU;

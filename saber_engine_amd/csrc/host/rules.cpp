@@ -221,6 +221,37 @@ static int describe_rows(const char *op, const char *kernel, uint32_t rows, uint
   return 0;
 }
 
+// The fused form quantises up to 4 rows whose int8 codes (rows rounded up to a power of two) fit
+// the kernel's 20 KiB staging area.
+bool fused_holds(uint32_t m, uint32_t k) {
+  if (m == 0 || m > 4) return false;
+  uint32_t mr = 1;
+  while (mr < m) mr *= 2;
+  return (uint64_t)mr * k <= 20 * 1024;
+}
+
+int resolve_fused(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *d) {
+  if (wkind != SABER_IU8_W4 && wkind != SABER_IU8_W8) return fail(SABER_IU8_E_ARG, "unknown weight kind");
+  const char *op = wkind == SABER_IU8_W8 ? "linear_i8a8_fused" : "linear_i4a8_fused";
+  if (int rc = check_shape(op, m, n, k)) return rc;
+  if (!fused_holds(m, k))
+    return fail(SABER_IU8_E_RULE, fmt("%s: %u rows of %u do not fit the fused form (at most 4 rows, 20 KiB of codes)", op, m, k));
+  const std::string name = fmt("macaq_iu8_decq_%s_tm1", wkind == SABER_IU8_W8 ? "w8" : "w4");
+  memset(d, 0, sizeof *d);
+  copy_name(d->op, sizeof d->op, op);
+  copy_name(d->plugin, sizeof d->plugin, "macaq_iu8");
+  copy_name(d->kernel, sizeof d->kernel, name);
+  d->grid[0] = (n + 31) / 32, d->grid[1] = 1, d->grid[2] = 1;  // 8 waves: 4 k-waves x 2 weight tiles
+  d->block[0] = 512, d->block[1] = 1, d->block[2] = 1;
+  d->n_launches = 1;
+  d->ks = 1;
+  if (int rc = fill_slots(name, d)) return rc;
+  set_i32(d, "m", m);
+  set_i32(d, "n", n);
+  set_i32(d, "k", k);
+  return 0;
+}
+
 int resolve_quant(uint32_t m, uint32_t k, saber_iu8_desc *out) {
   return describe_rows("quant_i8", "macaq_i8_quant_t256", m, k, "k", out);
 }

@@ -38,6 +38,9 @@ uint32_t decode_split(uint32_t m, uint32_t n, uint32_t k, uint32_t nblk, uint32_
 int resolve(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *out);
 int describe(const std::string &kernel, uint32_t m, uint32_t n, uint32_t k, uint32_t ks, saber_iu8_desc *out);
 int resolve_quant(uint32_t m, uint32_t k, saber_iu8_desc *out);
+// The fused quant + GEMV of a decode linear; refuses (by name) shapes it does not hold.
+bool fused_holds(uint32_t m, uint32_t k);
+int resolve_fused(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *out);
 int resolve_silu_mul_quant(uint32_t rows, uint32_t n, saber_iu8_desc *out);
 
 // Fills name/offset/size of every slot from the kernel's signature; kinds default to BUFFER.

@@ -84,6 +84,11 @@ int saber_iu8_resolve_quant(uint32_t m, uint32_t k, saber_iu8_desc *out) {
   if (!out) return fail(SABER_IU8_E_ARG, "resolve_quant: null descriptor");
   return resolve_quant(m, k, out);
 }
+int saber_iu8_fused_holds(uint32_t m, uint32_t k) { return fused_holds(m, k) ? 1 : 0; }
+int saber_iu8_resolve_fused(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *out) {
+  if (!out) return fail(SABER_IU8_E_ARG, "resolve_fused: null descriptor");
+  return resolve_fused(wkind, m, n, k, out);
+}
 int saber_iu8_resolve_silu_mul_quant(uint32_t rows, uint32_t n, saber_iu8_desc *out) {
   if (!out) return fail(SABER_IU8_E_ARG, "resolve_silu_mul_quant: null descriptor");
   return resolve_silu_mul_quant(rows, n, out);
@@ -313,6 +318,17 @@ int saber_iu8_quant(saber_iu8_ctx *ctx, const void *x, void *q, float *scale, ui
   if (int rc = resolve_quant(m, k, &d)) return rc;
   const saber_iu8_binding b[] = {{"x", (void *)x}, {"q", q}, {"scale", scale}};
   return saber_iu8_launch(ctx, &d, b, 3, stream);
+}
+
+int saber_iu8_linear_fused(saber_iu8_ctx *ctx, int wkind, const void *x, const void *w, const float *ws, void *c, void *q,
+                           float *scale, uint32_t m, uint32_t n, uint32_t k, void *stream) {
+  saber_iu8_desc d;
+  if (int rc = resolve_fused(wkind, m, n, k, &d)) return rc;
+  // the optional outputs are named-null when absent: the kernel tests the pointers
+  if (!q) set_null(&d, "q");
+  if (!scale) set_null(&d, "scale");
+  const saber_iu8_binding b[] = {{"x", (void *)x}, {"w", (void *)w}, {"ws", (void *)ws}, {"c", c}, {"q", q}, {"scale", scale}};
+  return saber_iu8_launch(ctx, &d, b, 6, stream);
 }
 
 int saber_iu8_gemm_workspace(int wkind, uint32_t m, uint32_t n, uint32_t k, uint64_t *partial_bytes, uint64_t *counter_bytes) {

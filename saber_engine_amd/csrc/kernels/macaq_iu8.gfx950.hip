@@ -41,6 +41,25 @@
 #undef IU8_PF_VARIANT
 #undef IU8_DEC
 
+// The decode linear with the per-token quantisation fused into the activation staging (M <= 4 rows
+// that fit the staged form): x is the bf16 activation matrix; `q` / `scale` (optional, may be null)
+// receive the int8 codes in A fragment order and the row scales, written by workgroup 0. One launch
+// instead of producer + GEMM; the bytes of c, q and scale are those of the two-launch path. The
+// reference fuses producers the other way round (norm/activation + quant in front of an int8 GEMM,
+// crates/saber-kernels/hip/mxfp4_hadi8.hip); this is the same law inside the GEMV's prologue, where
+// it hides behind the first weight loads.
+#define IU8_DECQ(name, W8, D)                                                                                      \
+  extern "C" __global__ __launch_bounds__(512) void name(                                                          \
+      const unsigned short *__restrict__ x, const unsigned char *__restrict__ w, const float *__restrict__ ws,     \
+      unsigned char *__restrict__ q, float *__restrict__ scale, unsigned short *__restrict__ c, int m, int n,      \
+      int k) {                                                                                                     \
+    iu8_dec_body<1, W8, 1, 4, 8, D, 20, false, true>((const unsigned char *)x, w, nullptr, ws, nullptr, nullptr, c, \
+                                                     iu8_rows{nullptr, 0, m}, n, k, q, scale);                     \
+  }
+IU8_DECQ(macaq_iu8_decq_w4_tm1, false, 8)
+IU8_DECQ(macaq_iu8_decq_w8_tm1, true, 4)
+#undef IU8_DECQ
+
 // Persistent launch: gridDim.x workgroups (one or OCC a CU) walk the tiles of the m x n output.
 #define IU8_PF32(name, W8, WMW, WNW, TM, TN, ACC, ST, OCC)                                                        \
   extern "C" __global__ __launch_bounds__(WMW * WNW * 64)                                                         \

@@ -107,6 +107,8 @@ def lib():
         L.saber_iu8_quant.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32, C.c_uint32, C.c_void_p]
         L.saber_iu8_gemm.argtypes = [C.c_void_p, C.c_int] + [C.c_void_p] * 5 + [C.c_uint32] * 3 + [C.c_void_p] * 3
         L.saber_iu8_gemm_acc.argtypes = [C.c_void_p, C.c_int] + [C.c_void_p] * 3 + [C.c_uint32] * 3 + [C.c_void_p]
+        L.saber_iu8_fused_holds.argtypes = [C.c_uint32, C.c_uint32]
+        L.saber_iu8_linear_fused.argtypes = [C.c_void_p, C.c_int] + [C.c_void_p] * 6 + [C.c_uint32] * 3 + [C.c_void_p]
         L.saber_iu8_get_counters.argtypes = [C.c_void_p, C.POINTER(Counters)]
         L.saber_iu8_has_kernel.argtypes = [C.c_void_p, C.c_char_p]
         for fn in ("saber_iu8_moe_rows_cap", "saber_iu8_moe_tile_blocks"):
@@ -140,6 +142,16 @@ def resolve(wkind, m, n, k):
 def describe(kernel, m, n, k, ks=1):
     d = Desc()
     _check(lib().saber_iu8_describe(kernel.encode(), m, n, k, ks, C.byref(d)))
+    return d
+
+
+def fused_holds(m, k):
+    return bool(lib().saber_iu8_fused_holds(m, k))
+
+
+def resolve_fused(wkind, m, n, k):
+    d = Desc()
+    _check(lib().saber_iu8_resolve_fused(wkind, m, n, k, C.byref(d)))
     return d
 
 
@@ -274,6 +286,9 @@ class Context:
 
     def gemm(self, wkind, a, a_scale, w, w_scale, c, m, n, k, partial=None, counter=None, stream=0):
         _check(lib().saber_iu8_gemm(self._h, wkind, a, a_scale, w, w_scale, c, m, n, k, partial, counter, stream))
+
+    def linear_fused(self, wkind, x, w, w_scale, c, m, n, k, q=None, scale=None, stream=0):
+        _check(lib().saber_iu8_linear_fused(self._h, wkind, x, w, w_scale, c, q, scale, m, n, k, stream))
 
     def gemm_acc(self, wkind, a, w, acc, m, n, k, stream=0):
         _check(lib().saber_iu8_gemm_acc(self._h, wkind, a, w, acc, m, n, k, stream))
