@@ -277,6 +277,15 @@ int saber_iu8_moe_grouped(saber_iu8_ctx *ctx, const void *a, const float *as, co
                           uint32_t k, int gather, uint32_t tokens, uint32_t experts, uint32_t topk, uint32_t tile_blocks,
                           const saber_iu8_moe_tables *t, void *stream);
 
+/* The routed layer's activations gathered and quantised in one pass: output row r (expert-major,
+ * rows_cap rows, A edge) = the int8 codes of token row row_tok[r], scale[r] its scale; pad rows and
+ * rows past meta[1] are left alone. With it the grouped gate+up GEMM runs on compact rows (gather 0)
+ * and reads whole fragments; the reference gathers inside its grouped GEMM from row-major rows
+ * (crates/saber-kernels/hip/moe_grouped.hip:67-74), which this object's tiled A order would turn
+ * into 16-byte reads. */
+int saber_iu8_moe_quant_rows(saber_iu8_ctx *ctx, const void *x_bf16, void *q, float *scale, uint32_t k, uint32_t rows_cap,
+                             const saber_iu8_moe_tables *tables, void *stream);
+
 /* SiLU(gate)*up + requant over the live expert-major rows: gu bf16 [rows_cap, 2n] -> q (A edge of
  * rows_cap rows), scale f32 [rows_cap]. Pad rows are skipped. */
 int saber_iu8_moe_silu_mul_quant(saber_iu8_ctx *ctx, const void *gu_bf16, void *q, float *scale, uint32_t n,

@@ -15,6 +15,8 @@ static const Signature SIG_DECQ = {{"x", K::Buffer},     {"w", K::Buffer}, {"ws"
 static const Signature SIG_PF = {{"a", K::Buffer}, {"w", K::Buffer}, {"as", K::Buffer}, {"ws", K::Buffer},
                                  {"c", K::Buffer}, {"m", K::I32},    {"n", K::I32},     {"k", K::I32}};
 static const Signature SIG_QUANT = {{"x", K::Buffer}, {"q", K::Buffer}, {"scale", K::Buffer}, {"k", K::I32}};
+static const Signature SIG_QUANT_ROWS = {{"x", K::Buffer}, {"q", K::Buffer},       {"scale", K::Buffer},
+                                         {"k", K::I32},    {"row_tok", K::Buffer}, {"meta", K::Buffer}};
 static const Signature SIG_SILU = {{"gu", K::Buffer}, {"q", K::Buffer},       {"scale", K::Buffer},
                                    {"n", K::I32},     {"row_tok", K::Buffer}, {"meta", K::Buffer}};
 static const Signature SIG_TABLE = {{"out", K::Buffer}};
@@ -44,6 +46,7 @@ const Signature *signature_for(const std::string &k) {
   if (starts(k, "macaq_iu8_dec_")) return &SIG_DEC;
   if (starts(k, "macaq_iu8_decq_")) return &SIG_DECQ;
   if (starts(k, "macaq_iu8_pf_")) return &SIG_PF;
+  if (starts(k, "macaq_i8_quant_rows_")) return &SIG_QUANT_ROWS;
   if (starts(k, "macaq_i8_quant_")) return &SIG_QUANT;
   if (starts(k, "macaq_i8_silu_mul_quant_")) return &SIG_SILU;
   if (k == "macaq_silu_bf16_table") return &SIG_TABLE;

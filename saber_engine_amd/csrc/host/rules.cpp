@@ -212,7 +212,11 @@ static int describe_rows(const char *op, const char *kernel, uint32_t rows, uint
   copy_name(d->op, sizeof d->op, op);
   copy_name(d->plugin, sizeof d->plugin, "macaq_i8q");
   copy_name(d->kernel, sizeof d->kernel, kernel);
-  d->grid[0] = rows, d->grid[1] = 1, d->grid[2] = 1;
+  // the wave-a-row forms take four rows a workgroup
+  const bool w64 = strlen(kernel) > 4 && !strcmp(kernel + strlen(kernel) - 4, "_w64");
+  if (w64 && (rows % 4 != 0 || width > 4096))
+    return fail(SABER_IU8_E_RULE, fmt("%s: %s takes a multiple of 4 rows of at most 4096, got %u of %u", op, kernel, rows, width));
+  d->grid[0] = w64 ? rows / 4 : rows, d->grid[1] = 1, d->grid[2] = 1;
   d->block[0] = 256, d->block[1] = 1, d->block[2] = 1;
   d->n_launches = 1;
   d->ks = 1;
@@ -252,12 +256,26 @@ int resolve_fused(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc 
   return 0;
 }
 
+// The row kernels' register forms: the narrowest that holds the row (4,096 elements a group slot).
+// Many narrow rows go a wave a row (`base`_w64), the rest a workgroup a row (`base`_t256...).
+static std::string row_form(const char *base, uint32_t rows, uint32_t width) {
+  if (width <= 2048 && rows % 4 == 0 && rows >= 64) return std::string(base) + "_w64";  // up to two groups a lane
+  const uint32_t slots = (width + 4095) / 4096;
+  return std::string(base) + "_t256" + (slots <= 1 ? "_g1" : slots <= 2 ? "_g2" : slots <= 5 ? "_g5" : "");
+}
+
 int resolve_quant(uint32_t m, uint32_t k, saber_iu8_desc *out) {
-  return describe_rows("quant_i8", "macaq_i8_quant_t256", m, k, "k", out);
+  return describe_rows("quant_i8", row_form("macaq_i8_quant", m, k).c_str(), m, k, "k", out);
+}
+
+int resolve_quant_rows(uint32_t rows, uint32_t k, saber_iu8_desc *out) {
+  const uint32_t slots = (k + 4095) / 4096;
+  const std::string name = std::string("macaq_i8_quant_rows_t256") + (slots <= 1 ? "_g1" : slots <= 2 ? "_g2" : "");
+  return describe_rows("quant_rows_i8", name.c_str(), rows, k, "k", out);
 }
 
 int resolve_silu_mul_quant(uint32_t rows, uint32_t n, saber_iu8_desc *out) {
-  if (int rc = describe_rows("silu_mul_quant_i8", "macaq_i8_silu_mul_quant_t256", rows, n, "n", out)) return rc;
+  if (int rc = describe_rows("silu_mul_quant_i8", row_form("macaq_i8_silu_mul_quant", rows, n).c_str(), rows, n, "n", out)) return rc;
   // the dense form has no row map; the routed form binds both (set_buffer)
   set_null(out, "row_tok");
   set_null(out, "meta");

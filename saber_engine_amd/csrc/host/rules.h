@@ -42,6 +42,8 @@ int resolve_quant(uint32_t m, uint32_t k, saber_iu8_desc *out);
 bool fused_holds(uint32_t m, uint32_t k);
 int resolve_fused(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *out);
 int resolve_silu_mul_quant(uint32_t rows, uint32_t n, saber_iu8_desc *out);
+// Quantisation through a row map (output row r = input row row_tok[r]).
+int resolve_quant_rows(uint32_t rows, uint32_t k, saber_iu8_desc *out);
 
 // Fills name/offset/size of every slot from the kernel's signature; kinds default to BUFFER.
 int fill_slots(const std::string &kernel, saber_iu8_desc *d);

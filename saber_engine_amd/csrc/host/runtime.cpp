@@ -427,7 +427,13 @@ int saber_iu8_moe_grouped(saber_iu8_ctx *ctx, const void *a, const float *as, co
   const std::string name = fmt("moe_iu8_grouped_w4_%s_g%d", dec ? "dec" : "pf", gather ? 1 : 0);
   const uint32_t bn = dec ? 32 : 256, block = 512;
   saber_iu8_desc d;
-  if (int rc = raw_desc(name.c_str(), (n + bn - 1) / bn, saber_iu8_moe_tiles_cap(tokens, topk, experts, tile_blocks), block, &d)) return rc;
+  // the streaming cell: a workgroup a (column block, tile), static worst-case grid; the MFMA cell:
+  // persistent, one workgroup a CU over the live work items
+  const uint32_t tiles_cap = saber_iu8_moe_tiles_cap(tokens, topk, experts, tile_blocks), gx = (n + bn - 1) / bn;
+  const uint64_t items = (uint64_t)gx * tiles_cap;
+  if (int rc = dec ? raw_desc(name.c_str(), gx, tiles_cap, block, &d)
+                   : raw_desc(name.c_str(), (uint32_t)(items < CU_COUNT ? items : CU_COUNT), 1, block, &d))
+    return rc;
   set_i32(&d, "n", n);
   set_i32(&d, "k", k);
   set_i32(&d, "pmax", 0);
@@ -437,6 +443,15 @@ int saber_iu8_moe_grouped(saber_iu8_ctx *ctx, const void *a, const float *as, co
                                  {"tile_row0", t->tile_row0}, {"tile_rows", t->tile_rows},   {"row_tok", t->row_tok},
                                  {"meta", t->meta},           {"as", (void *)as},            {"c", c}};
   return saber_iu8_launch(ctx, &d, b, sizeof b / sizeof b[0], stream);
+}
+
+int saber_iu8_moe_quant_rows(saber_iu8_ctx *ctx, const void *x, void *q, float *scale, uint32_t k, uint32_t rows_cap,
+                             const saber_iu8_moe_tables *t, void *stream) {
+  if (!t) return fail(SABER_IU8_E_ARG, "moe_quant_rows: null tables");
+  saber_iu8_desc d;
+  if (int rc = resolve_quant_rows(rows_cap, k, &d)) return rc;
+  const saber_iu8_binding b[] = {{"x", (void *)x}, {"q", q}, {"scale", scale}, {"row_tok", t->row_tok}, {"meta", t->meta}};
+  return saber_iu8_launch(ctx, &d, b, 5, stream);
 }
 
 int saber_iu8_moe_silu_mul_quant(saber_iu8_ctx *ctx, const void *gu, void *q, float *scale, uint32_t n, uint32_t rows_cap,

@@ -69,6 +69,21 @@ static __device__ __forceinline__ unsigned iu8_code(float x, float sc) {
   return ((unsigned)(int)__builtin_rintf(y)) & 0xffu;
 }
 
+// The same code without a divide per element: rcp = __fdiv_rn(1, sc) once a row, t = x * rcp is
+// within 1.6e-5 of x / sc for |x / sc| <= 127 (two roundings of 2^-24 relative), the IEEE quotient
+// within 7.6e-6. If t sits at least 1e-4 inside its rounding interval, the IEEE quotient rounds to
+// the same integer; otherwise (a tie or next to one, rare) the divide decides. NaN and infinite
+// rows come out as through the divide: NaN clamps to -127 on both paths.
+static __device__ __forceinline__ unsigned iu8_code_rcp(float x, float sc, float rcp) {
+  float y = fminf(fmaxf(x * rcp, -127.f), 127.f);
+  float q = __builtin_rintf(y);
+  if (__builtin_expect(fabsf(y - q) > 0.4999f, 0)) {
+    y = fminf(fmaxf(__fdiv_rn(x, sc), -127.f), 127.f);
+    q = __builtin_rintf(y);
+  }
+  return ((unsigned)(int)q) & 0xffu;
+}
+
 static __device__ __forceinline__ iu8_v4u iu8_ldg_nt(const iu8_u8 *p) {
   return __builtin_nontemporal_load((const iu8_v4u *)p);
 }

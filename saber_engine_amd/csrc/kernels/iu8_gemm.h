@@ -232,13 +232,14 @@ __device__ __forceinline__ void iu8_dec_body(const iu8_u8 *__restrict__ A, const
           if (piece >= x_pieces) continue;
           const int row = piece / k8, k = (piece - row * k8) << 3;
           const float sc = row == 0 ? qsc[0] : row == 1 ? qsc[1] : row == 2 ? qsc[2] : qsc[3];
+          const float rcp = __fdiv_rn(1.f, sc);
           unsigned d0 = 0, d1 = 0;
 #pragma unroll
           for (int w = 0; w < 2; ++w) {
-            d0 |= iu8_code(__uint_as_float(xreg[p][w] << 16), sc) << (16 * w);
-            d0 |= iu8_code(__uint_as_float(xreg[p][w] & 0xFFFF0000u), sc) << (16 * w + 8);
-            d1 |= iu8_code(__uint_as_float(xreg[p][2 + w] << 16), sc) << (16 * w);
-            d1 |= iu8_code(__uint_as_float(xreg[p][2 + w] & 0xFFFF0000u), sc) << (16 * w + 8);
+            d0 |= iu8_code_rcp(__uint_as_float(xreg[p][w] << 16), sc, rcp) << (16 * w);
+            d0 |= iu8_code_rcp(__uint_as_float(xreg[p][w] & 0xFFFF0000u), sc, rcp) << (16 * w + 8);
+            d1 |= iu8_code_rcp(__uint_as_float(xreg[p][2 + w] << 16), sc, rcp) << (16 * w);
+            d1 |= iu8_code_rcp(__uint_as_float(xreg[p][2 + w] & 0xFFFF0000u), sc, rcp) << (16 * w + 8);
           }
           const int kt = k >> 6, g = (k >> 4) & 3, half = (k >> 3) & 1;
           *(iu8_v2u *)&s_mem[((((kt * 4 + g) << mr_shift) + row) << 4) + half * 8] = iu8_v2u{d0, d1};

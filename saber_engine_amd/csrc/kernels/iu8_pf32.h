@@ -83,25 +83,29 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
   // Global -> LDS without registers: global_load_lds_dwordx4 writes lane l's 16 bytes at
   // (wave-uniform LDS base in m0) + 16*l, so one wave-load lands one fragment in fragment order.
   // Per lane: the 32-bit byte offset of its piece at K step 0 of the load stream's tile.
-  iu8_tile L;
+  iu8_tile L, Nx;  // the stream's tile and the one after it
   if (!tile_at(0, L)) return;
   int lr = 0, ls = 0;
-  unsigned ga[A_PER], gw[W_PER];
-  auto set_addr = [&]() {
+  unsigned ga[A_PER], gw[W_PER], gaN[A_PER], gwN[W_PER];
+  auto addr_of = [&](const iu8_tile &t, unsigned (&oa)[A_PER], unsigned (&ow)[W_PER]) {
 #pragma unroll
     for (int p = 0; p < A_PER; ++p) {
       const int f = min(p * NWAVE + wave, A_FR - 1);  // fragment (mt = f/2, kt2 = f%2) of the step
-      const int ar = iu8_arow(L.R, L.mbase + (f >> 1) * 16 + (lane & 15));  // rows past the edge: the last one
-      ga[p] = (unsigned)(((size_t)(ar >> 4) * ktiles + (f & 1)) * 1024 + ((ar & 15) + 16 * (lane >> 4)) * 16);
+      const int ar = iu8_arow(t.R, t.mbase + (f >> 1) * 16 + (lane & 15));  // rows past the edge: the last one
+      oa[p] = (unsigned)(((size_t)(ar >> 4) * ktiles + (f & 1)) * 1024 + ((ar & 15) + 16 * (lane >> 4)) * 16);
     }
 #pragma unroll
     for (int p = 0; p < W_PER; ++p) {
       const int f = min(p * NWAVE + wave, W_FR - 1);
-      const int nt = min(L.nt0 + f / (WSTEP / 1024), ntiles - 1);  // tiles past N: the last one
-      gw[p] = (unsigned)((size_t)nt * steps * WSTEP + (f % (WSTEP / 1024)) * 1024 + lane * 16);
+      const int nt = min(t.nt0 + f / (WSTEP / 1024), ntiles - 1);  // tiles past N: the last one
+      ow[p] = (unsigned)((size_t)nt * steps * WSTEP + (f % (WSTEP / 1024)) * 1024 + lane * 16);
     }
   };
-  set_addr();
+  addr_of(L, ga, gw);
+  // The next tile's descriptor and addresses (a gathered tile reads its row map for them) are
+  // fetched a whole tile ahead, so the stream never waits for them when it crosses into that tile.
+  bool haveN = tile_at(1, Nx);
+  if (haveN) addr_of(Nx, gaN, gwN);
   // The load is written as asm: the compiler models an LDS-DMA load as touching both memories and
   // then drains every counter to zero at each later LDS read, which would serialise the operand
   // pipeline below. Its completion is tracked by hand (vmcnt, before the step's barrier).
@@ -125,10 +129,14 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
   };
   auto advance = [&]() {  // next step of the stream; past the last tile it keeps re-loading the last step
     if (++ls == steps) {
-      iu8_tile T;
-      if (tile_at(lr + 1, T)) {
-        ++lr, ls = 0, L = T;
-        set_addr();
+      if (haveN) {
+        ++lr, ls = 0, L = Nx;
+#pragma unroll
+        for (int p = 0; p < A_PER; ++p) ga[p] = gaN[p];
+#pragma unroll
+        for (int p = 0; p < W_PER; ++p) gw[p] = gwN[p];
+        haveN = tile_at(lr + 1, Nx);
+        if (haveN) addr_of(Nx, gaN, gwN);
       } else {
         ls = steps - 1;
       }

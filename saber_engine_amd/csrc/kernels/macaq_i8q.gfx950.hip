@@ -5,17 +5,33 @@
 // A fragment order (iu8_common.h), scale f32 per row.
 //
 //   macaq_i8_quant_t256           x bf16 [M,K] -> q, scale                 (grid M, block 256)
+//   macaq_i8_quant_rows_t256      the same through a row map: output row r = input row row_tok[r]
+//                                 (the gathered, expert-major activations of a routed layer)
 //   macaq_i8_silu_mul_quant_t256  gu bf16 [M, 2N] (gate | up) -> p = bf16(bf16(silu(g)) * u)
 //                                 -> q, scale over N                       (grid M, block 256)
 //                                 (crates/saber-kernels/hip/mxfp4_hadi8.hip:118-146 without the
 //                                 Hadamard; signature crates/saber-kernels/src/abi.rs:315-320)
+//   macaq_i8_quant_w64, macaq_i8_silu_mul_quant_w64   the same two for rows of up to 4,096 elements,
+//                                 a wave a row, four rows a workgroup (grid M/4, block 256)
 //   macaq_silu_bf16_table         the bf16 silu of all 65,536 bf16 inputs (a checker's tap)
 //
 // One workgroup a row; a thread owns 16-element groups g = tid + i*256 (one 16-byte store each).
+// A kernel holds its row in registers, so each comes in forms for rows of up to 4,096 (_g1), 8,192
+// (_g2), 20,480 (_g5) and 32,768 (no suffix) elements: the narrow forms keep the register count low
+// enough for eight waves a SIMD, which is what hides the load latency of a one-pass row kernel.
 #include "iu8_common.h"
 
 #define I8Q_T 256
-#define I8Q_MAXG 8  // K <= 16 * 256 * 8 = 32,768
+
+// The row of workgroup b. The hardware deals consecutive workgroups round-robin over the 8 XCDs, and
+// the 16 rows of an A tile interleave their 16-byte pieces inside 256-byte runs: so the 8 tiles of
+// every full group of 128 rows go one to an XCD, and an XCD's L2 sees whole lines before it writes
+// them back. Rows past the last full group keep their order.
+static __device__ __forceinline__ int i8q_row() {
+  const int b = blockIdx.x, full = (int)gridDim.x & ~127;
+  if (b >= full) return b;
+  return (b & ~127) + (b & 7) * 16 + ((b & 127) >> 3);
+}
 
 static __device__ __forceinline__ float i8q_block_max(float v) {
   __shared__ float s_w[I8Q_T / 64];
@@ -30,45 +46,58 @@ static __device__ __forceinline__ float i8q_block_max(float v) {
 }
 
 // codes of one row from v[g][16] (f32 values), written in A fragment order
+template <int I8Q_MAXG>
 static __device__ __forceinline__ void i8q_tail(float (&v)[I8Q_MAXG][16], int G, iu8_u8 *__restrict__ q,
                                                 float *__restrict__ scale, int row, int K) {
   const int tid = threadIdx.x;
   float amax = 0.f;
 #pragma unroll
   for (int i = 0; i < I8Q_MAXG; ++i) {
-    if (tid + i * I8Q_T >= G) break;
+    if (tid + i * I8Q_T >= G) continue;
 #pragma unroll
     for (int j = 0; j < 16; ++j) amax = fmaxf(amax, fabsf(v[i][j]));
   }
   amax = i8q_block_max(amax);
   const float sc = fmaxf(__fdiv_rn(amax, 127.f), 1e-30f);
+  const float rcp = __fdiv_rn(1.f, sc);
   if (tid == 0) scale[row] = sc;
   iu8_u8 *qrow = q + (size_t)(row >> 4) * (K >> 6) * 1024 + (row & 15) * 16;
 #pragma unroll
   for (int i = 0; i < I8Q_MAXG; ++i) {
     const int g = tid + i * I8Q_T;
-    if (g >= G) break;
+    if (g >= G) continue;
     unsigned d[4];
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
       d[w] = 0;
 #pragma unroll
-      for (int b = 0; b < 4; ++b) d[w] |= iu8_code(v[i][w * 4 + b], sc) << (8 * b);
+      for (int b = 0; b < 4; ++b) d[w] |= iu8_code_rcp(v[i][w * 4 + b], sc, rcp) << (8 * b);
     }
     *(iu8_v4u *)(qrow + (size_t)(g >> 2) * 1024 + (g & 3) * 256) = iu8_v4u{d[0], d[1], d[2], d[3]};
   }
 }
 
-extern "C" __global__ __launch_bounds__(I8Q_T) void macaq_i8_quant_t256(const unsigned short *__restrict__ x,
-                                                                        unsigned char *__restrict__ q,
-                                                                        float *__restrict__ scale, int k) {
-  const int row = blockIdx.x, G = k >> 4;
-  const unsigned short *xr = x + (size_t)row * k;
+// `row_tok` / `meta` (optional, may be null): with them output row r is the quantised input row
+// row_tok[r] (the expert-major rows of a routed layer, gathered here once so that the grouped GEMM
+// reads whole fragments); pad rows (row_tok < 0) and rows past meta[1] are skipped.
+template <int I8Q_MAXG>
+static __device__ __forceinline__ void i8q_quant_body(const unsigned short *__restrict__ x, unsigned char *__restrict__ q,
+                                                      float *__restrict__ scale, int k,
+                                                      const int *__restrict__ row_tok = nullptr,
+                                                      const int *__restrict__ meta = nullptr) {
+  const int row = i8q_row(), G = k >> 4;
+  if (meta != nullptr && row >= meta[1]) return;
+  int src = row;
+  if (row_tok != nullptr) {
+    src = row_tok[row];
+    if (src < 0) return;
+  }
+  const unsigned short *xr = x + (size_t)src * k;
   float v[I8Q_MAXG][16];
 #pragma unroll
   for (int i = 0; i < I8Q_MAXG; ++i) {
     const int g = threadIdx.x + i * I8Q_T;
-    if (g >= G) break;
+    if (g >= G) continue;
     const iu8_v4u lo = *(const iu8_v4u *)(xr + g * 16), hi = *(const iu8_v4u *)(xr + g * 16 + 8);
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
@@ -78,8 +107,29 @@ extern "C" __global__ __launch_bounds__(I8Q_T) void macaq_i8_quant_t256(const un
       v[i][8 + 2 * w + 1] = __uint_as_float(hi[w] & 0xFFFF0000u);
     }
   }
-  i8q_tail(v, G, q, scale, row, k);
+  i8q_tail<I8Q_MAXG>(v, G, q, scale, row, k);
 }
+#define I8Q_QUANT(name, MAXG)                                                                                   \
+  extern "C" __global__ __launch_bounds__(I8Q_T) void name(const unsigned short *__restrict__ x,                \
+                                                           unsigned char *__restrict__ q, float *__restrict__ scale, \
+                                                           int k) {                                             \
+    i8q_quant_body<MAXG>(x, q, scale, k);                                                                       \
+  }
+I8Q_QUANT(macaq_i8_quant_t256, 8)
+I8Q_QUANT(macaq_i8_quant_t256_g5, 5)
+I8Q_QUANT(macaq_i8_quant_t256_g2, 2)
+I8Q_QUANT(macaq_i8_quant_t256_g1, 1)
+#undef I8Q_QUANT
+#define I8Q_QUANT_ROWS(name, MAXG)                                                                               \
+  extern "C" __global__ __launch_bounds__(I8Q_T) void name(                                                      \
+      const unsigned short *__restrict__ x, unsigned char *__restrict__ q, float *__restrict__ scale, int k,     \
+      const int *__restrict__ row_tok, const int *__restrict__ meta) {                                           \
+    i8q_quant_body<MAXG>(x, q, scale, k, row_tok, meta);                                                         \
+  }
+I8Q_QUANT_ROWS(macaq_i8_quant_rows_t256, 8)
+I8Q_QUANT_ROWS(macaq_i8_quant_rows_t256_g2, 2)
+I8Q_QUANT_ROWS(macaq_i8_quant_rows_t256_g1, 1)
+#undef I8Q_QUANT_ROWS
 
 static __device__ __forceinline__ float i8q_silu_bf16(float x) {
 #pragma clang fp contract(off)
@@ -89,11 +139,12 @@ static __device__ __forceinline__ float i8q_silu_bf16(float x) {
 // `row_tok` / `meta` are optional (may be null): with them the kernel runs on the expert-major
 // rows of a routed layer and skips pad rows (row_tok < 0) and rows past meta[1]
 // (signature crates/saber-kernels/src/abi.rs:344-351).
-extern "C" __global__ __launch_bounds__(I8Q_T) void macaq_i8_silu_mul_quant_t256(
-    const unsigned short *__restrict__ gu, unsigned char *__restrict__ q, float *__restrict__ scale, int n,
-    const int *__restrict__ row_tok, const int *__restrict__ meta) {
+template <int I8Q_MAXG>
+static __device__ __forceinline__ void i8q_silu_body(const unsigned short *__restrict__ gu, unsigned char *__restrict__ q,
+                                                     float *__restrict__ scale, int n, const int *__restrict__ row_tok,
+                                                     const int *__restrict__ meta) {
 #pragma clang fp contract(off)
-  const int row = blockIdx.x, G = n >> 4;
+  const int row = i8q_row(), G = n >> 4;
   if (meta != nullptr && row >= meta[1]) return;
   if (row_tok != nullptr && row_tok[row] < 0) return;
   const unsigned short *gr = gu + (size_t)row * 2 * n;
@@ -101,7 +152,7 @@ extern "C" __global__ __launch_bounds__(I8Q_T) void macaq_i8_silu_mul_quant_t256
 #pragma unroll
   for (int i = 0; i < I8Q_MAXG; ++i) {
     const int g = threadIdx.x + i * I8Q_T;
-    if (g >= G) break;
+    if (g >= G) continue;
     union { iu8_v4u u[2]; unsigned short h[16]; } vg, vu;
     vg.u[0] = *(const iu8_v4u *)(gr + g * 16);
     vg.u[1] = *(const iu8_v4u *)(gr + g * 16 + 8);
@@ -113,7 +164,108 @@ extern "C" __global__ __launch_bounds__(I8Q_T) void macaq_i8_silu_mul_quant_t256
       v[i][j] = iu8_bf16_f32((unsigned short)iu8_bf16_bits(t * iu8_bf16_f32(vu.h[j])));
     }
   }
-  i8q_tail(v, G, q, scale, row, n);
+  i8q_tail<I8Q_MAXG>(v, G, q, scale, row, n);
+}
+#define I8Q_SILU(name, MAXG)                                                                                     \
+  extern "C" __global__ __launch_bounds__(I8Q_T) void name(                                                      \
+      const unsigned short *__restrict__ gu, unsigned char *__restrict__ q, float *__restrict__ scale, int n,    \
+      const int *__restrict__ row_tok, const int *__restrict__ meta) {                                           \
+    i8q_silu_body<MAXG>(gu, q, scale, n, row_tok, meta);                                                         \
+  }
+I8Q_SILU(macaq_i8_silu_mul_quant_t256, 8)
+I8Q_SILU(macaq_i8_silu_mul_quant_t256_g5, 5)
+I8Q_SILU(macaq_i8_silu_mul_quant_t256_g2, 2)
+I8Q_SILU(macaq_i8_silu_mul_quant_t256_g1, 1)
+#undef I8Q_SILU
+
+// ---------------------------------------------------------------------------- a wave a row
+// Rows of up to 4,096 elements: four rows a workgroup, one wave each, a lane owns groups
+// g = lane + i*64. No LDS and no barrier: the row maximum is a wave butterfly. The launch covers
+// 4 * gridDim.x rows (the caller's row count is a multiple of 4).
+#define I8Q_WG 4  // groups a lane
+static __device__ __forceinline__ int i8q_row4() {
+  const int b = blockIdx.x, full = (int)gridDim.x & ~31;  // 32 workgroups = 128 rows = 8 tiles, one an XCD
+  const int u = b >= full ? b : (b & ~31) + (b & 7) * 4 + ((b & 31) >> 3);
+  return u * 4 + (threadIdx.x >> 6);
+}
+static __device__ __forceinline__ void i8q_tail_w64(float (&v)[I8Q_WG][16], int G, iu8_u8 *__restrict__ q,
+                                                    float *__restrict__ scale, int row, int K) {
+  const int lane = threadIdx.x & 63;
+  float amax = 0.f;
+#pragma unroll
+  for (int i = 0; i < I8Q_WG; ++i) {
+    if (lane + i * 64 >= G) continue;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) amax = fmaxf(amax, fabsf(v[i][j]));
+  }
+#pragma unroll
+  for (int o = 32; o; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
+  const float sc = fmaxf(__fdiv_rn(amax, 127.f), 1e-30f);
+  const float rcp = __fdiv_rn(1.f, sc);
+  if (lane == 0) scale[row] = sc;
+  iu8_u8 *qrow = q + (size_t)(row >> 4) * (K >> 6) * 1024 + (row & 15) * 16;
+#pragma unroll
+  for (int i = 0; i < I8Q_WG; ++i) {
+    const int g = lane + i * 64;
+    if (g >= G) continue;
+    unsigned d[4];
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      d[w] = 0;
+#pragma unroll
+      for (int b = 0; b < 4; ++b) d[w] |= iu8_code_rcp(v[i][w * 4 + b], sc, rcp) << (8 * b);
+    }
+    *(iu8_v4u *)(qrow + (size_t)(g >> 2) * 1024 + (g & 3) * 256) = iu8_v4u{d[0], d[1], d[2], d[3]};
+  }
+}
+
+extern "C" __global__ __launch_bounds__(256) void macaq_i8_quant_w64(const unsigned short *__restrict__ x,
+                                                                     unsigned char *__restrict__ q,
+                                                                     float *__restrict__ scale, int k) {
+  const int row = i8q_row4(), G = k >> 4, lane = threadIdx.x & 63;
+  const unsigned short *xr = x + (size_t)row * k;
+  float v[I8Q_WG][16];
+#pragma unroll
+  for (int i = 0; i < I8Q_WG; ++i) {
+    const int g = lane + i * 64;
+    if (g >= G) continue;
+    const iu8_v4u lo = *(const iu8_v4u *)(xr + g * 16), hi = *(const iu8_v4u *)(xr + g * 16 + 8);
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      v[i][2 * w] = __uint_as_float(lo[w] << 16);
+      v[i][2 * w + 1] = __uint_as_float(lo[w] & 0xFFFF0000u);
+      v[i][8 + 2 * w] = __uint_as_float(hi[w] << 16);
+      v[i][8 + 2 * w + 1] = __uint_as_float(hi[w] & 0xFFFF0000u);
+    }
+  }
+  i8q_tail_w64(v, G, q, scale, row, k);
+}
+
+extern "C" __global__ __launch_bounds__(256) void macaq_i8_silu_mul_quant_w64(
+    const unsigned short *__restrict__ gu, unsigned char *__restrict__ q, float *__restrict__ scale, int n,
+    const int *__restrict__ row_tok, const int *__restrict__ meta) {
+#pragma clang fp contract(off)
+  const int row = i8q_row4(), G = n >> 4, lane = threadIdx.x & 63;
+  if (meta != nullptr && row >= meta[1]) return;
+  if (row_tok != nullptr && row_tok[row] < 0) return;
+  const unsigned short *gr = gu + (size_t)row * 2 * n;
+  float v[I8Q_WG][16];
+#pragma unroll
+  for (int i = 0; i < I8Q_WG; ++i) {
+    const int g = lane + i * 64;
+    if (g >= G) continue;
+    union { iu8_v4u u[2]; unsigned short h[16]; } vg, vu;
+    vg.u[0] = *(const iu8_v4u *)(gr + g * 16);
+    vg.u[1] = *(const iu8_v4u *)(gr + g * 16 + 8);
+    vu.u[0] = *(const iu8_v4u *)(gr + n + g * 16);
+    vu.u[1] = *(const iu8_v4u *)(gr + n + g * 16 + 8);
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      const float t = i8q_silu_bf16(iu8_bf16_f32(vg.h[j]));
+      v[i][j] = iu8_bf16_f32((unsigned short)iu8_bf16_bits(t * iu8_bf16_f32(vu.h[j])));
+    }
+  }
+  i8q_tail_w64(v, G, q, scale, row, n);
 }
 
 extern "C" __global__ __launch_bounds__(256) void macaq_silu_bf16_table(unsigned short *__restrict__ out) {

@@ -191,12 +191,20 @@ extern "C" __global__ __launch_bounds__(MOE_THREADS) void moe_iu8_route_topk8_so
   if (tid == 0) *arrive = 0;
 
   // ---- phase 3 (the last workgroup): totals, each workgroup's base, offsets, tiles, placement
+  // (loads in batches of 8: the last workgroup works alone, so its time is load latency)
   for (int e = tid; e < e_loc; e += MOE_THREADS) {
     int run = 0;
-    for (int b = 0; b < nblk; ++b) {
-      const int c = __builtin_nontemporal_load(&blk_cnt[(size_t)b * e_loc + e]);
-      blk_cnt[(size_t)b * e_loc + e] = run;
-      run += c;
+    for (int b0 = 0; b0 < nblk; b0 += 8) {
+      int c[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        c[u] = b0 + u < nblk ? __builtin_nontemporal_load(&blk_cnt[(size_t)(b0 + u) * e_loc + e]) : 0;
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (b0 + u < nblk) {
+          blk_cnt[(size_t)(b0 + u) * e_loc + e] = run;
+          run += c[u];
+        }
     }
     s_cnt[e] = run;
     expert_cnt[e] = run;
@@ -253,17 +261,33 @@ extern "C" __global__ __launch_bounds__(MOE_THREADS) void moe_iu8_route_topk8_so
     row_tok[sh_row0 + r] = r < T ? r : -1;
     row_route[sh_row0 + r] = -1;
   }
-  for (int r = tid; r < T * MOE_TOPK; r += MOE_THREADS) {
-    const int e = __builtin_nontemporal_load(&topk_ids[r]), le = e - e_lo;
-    if (le < 0 || le >= e_loc) {
-      route_pos[r] = -1;
-      continue;
+  __syncthreads();  // every expert's blk_cnt bases are written
+  for (int r0 = tid; r0 < T * MOE_TOPK; r0 += 8 * MOE_THREADS) {
+    int e[8], rk[8], base[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int r = r0 + u * MOE_THREADS;
+      e[u] = r < T * MOE_TOPK ? __builtin_nontemporal_load(&topk_ids[r]) : -1;
+      rk[u] = r < T * MOE_TOPK ? __builtin_nontemporal_load(&rank[r]) : 0;
     }
-    const int t = r / MOE_TOPK, b = t / MOE_TPB;
-    const int p = s_off[le] + blk_cnt[(size_t)b * e_loc + le] + __builtin_nontemporal_load(&rank[r]);
-    row_tok[p] = t;
-    row_route[p] = r;
-    route_pos[r] = p;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int r = r0 + u * MOE_THREADS, le = e[u] - e_lo;
+      base[u] = (r < T * MOE_TOPK && le >= 0 && le < e_loc) ? blk_cnt[(size_t)(r / MOE_TOPK / MOE_TPB) * e_loc + le] : 0;
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int r = r0 + u * MOE_THREADS, le = e[u] - e_lo;
+      if (r >= T * MOE_TOPK) continue;
+      if (le < 0 || le >= e_loc) {
+        route_pos[r] = -1;
+        continue;
+      }
+      const int p = s_off[le] + base[u] + rk[u];
+      row_tok[p] = r / MOE_TOPK;
+      row_route[p] = r;
+      route_pos[r] = p;
+    }
   }
 }
 
@@ -287,26 +311,29 @@ MOE_GROUPED_DEC(moe_iu8_grouped_w4_dec_g1, true, 1, 4, 8, 8, 20)
 MOE_GROUPED_DEC(moe_iu8_grouped_w4_dec_g0, false, 1, 4, 8, 8, 20)
 #undef MOE_GROUPED_DEC
 
+// The MFMA-bound cell: a persistent launch of one workgroup a CU walks the work items
+// (tile, column block) of the live tiles, column blocks of one tile on neighbouring workgroups, the
+// load stream running across items (iu8_pf32.h). grid [256, 1, 1].
 #define MOE_GROUPED_PF(name, GATHER, WMW, WNW, TM, TN)                                                           \
   extern "C" __global__ __launch_bounds__(WMW * WNW * 64) void name(                                              \
       const unsigned char *__restrict__ a, const unsigned long long *__restrict__ xptr,                           \
       const int *__restrict__ tile_expert, const int *__restrict__ tile_row0, const int *__restrict__ tile_rows,  \
       const int *__restrict__ row_tok, const int *__restrict__ meta, const float *__restrict__ as,                \
       int *__restrict__ p, int *__restrict__ cnt, unsigned short *__restrict__ c, int n, int k, int pmax) {        \
-    const int tile = blockIdx.y;                                                                                   \
-    if (tile >= meta[0]) return;                                                                                   \
-    const int e = tile_expert[tile];                                                                               \
-    const iu8_rows R{GATHER ? row_tok : nullptr, tile_row0[tile], min(tile_rows[tile], WMW * TM * 32)};            \
+    constexpr int BN = WNW * TN * 32;                                                                              \
+    const int gx = (n + BN - 1) / BN, total = meta[0] * gx;                                                        \
     iu8_pf32_run<false, WMW, WNW, TM, TN, false, 3>(a, as, c, n, k, [&](int r, iu8_tile &t) {                      \
-      if (r != 0) return false;                                                                                    \
-      t = iu8_tile{R, 0, (int)blockIdx.x * (WNW * TN * 2), (const unsigned char *)xptr[2 * e],                     \
-                   (const float *)xptr[2 * e + 1]};                                                                \
+      const int id = (int)blockIdx.x + r * (int)gridDim.x;                                                         \
+      if (id >= total) return false;                                                                               \
+      const int tile = id / gx, bx = id - tile * gx, e = tile_expert[tile];                                        \
+      t = iu8_tile{iu8_rows{GATHER ? row_tok : nullptr, tile_row0[tile], min(tile_rows[tile], WMW * TM * 32)}, 0,  \
+                   bx * (BN / 16), (const unsigned char *)xptr[2 * e], (const float *)xptr[2 * e + 1]};            \
       return true;                                                                                                 \
     });                                                                                                            \
   }
-// tiles of up to 128 rows (tile_blocks 8) on the 128 x 256 tile of 4 x 2 waves
-MOE_GROUPED_PF(moe_iu8_grouped_w4_pf_g1, true, 4, 2, 1, 4)
-MOE_GROUPED_PF(moe_iu8_grouped_w4_pf_g0, false, 4, 2, 1, 4)
+// tiles of up to 128 rows (tile_blocks 8) on the 128 x 256 tile of 2 x 4 waves
+MOE_GROUPED_PF(moe_iu8_grouped_w4_pf_g1, true, 2, 4, 2, 2)
+MOE_GROUPED_PF(moe_iu8_grouped_w4_pf_g0, false, 2, 4, 2, 2)
 #undef MOE_GROUPED_PF
 
 // ---------------------------------------------------------------------------- combine

@@ -119,6 +119,7 @@ def lib():
         L.saber_iu8_moe_route.argtypes = [C.c_void_p, C.c_void_p] + [C.c_uint32] * 4 + [C.POINTER(MoeTables), C.c_void_p]
         L.saber_iu8_moe_grouped.argtypes = ([C.c_void_p] * 5 + [C.c_uint32, C.c_uint32, C.c_int] + [C.c_uint32] * 4 +
                                             [C.POINTER(MoeTables), C.c_void_p])
+        L.saber_iu8_moe_quant_rows.argtypes = [C.c_void_p] * 4 + [C.c_uint32, C.c_uint32, C.POINTER(MoeTables), C.c_void_p]
         L.saber_iu8_moe_silu_mul_quant.argtypes = [C.c_void_p] * 4 + [C.c_uint32, C.c_uint32, C.POINTER(MoeTables), C.c_void_p]
         L.saber_iu8_moe_combine.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(MoeTables), C.c_void_p] + [C.c_uint32] * 3 + [C.c_void_p]
         L.saber_iu8_silu_table.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
@@ -301,6 +302,9 @@ class Context:
     def moe_grouped(self, a, a_scale, xptr, c, n, k, gather, tokens, experts, topk, tile_blocks, tables, stream=0):
         _check(lib().saber_iu8_moe_grouped(self._h, a, a_scale, xptr, c, n, k, int(gather), tokens, experts, topk,
                                            tile_blocks, C.byref(tables), stream))
+
+    def moe_quant_rows(self, x, q, scale, k, rows_cap, tables, stream=0):
+        _check(lib().saber_iu8_moe_quant_rows(self._h, x, q, scale, k, rows_cap, C.byref(tables), stream))
 
     def moe_silu_mul_quant(self, gu, q, scale, n, rows_cap, tables, stream=0):
         _check(lib().saber_iu8_moe_silu_mul_quant(self._h, gu, q, scale, n, rows_cap, C.byref(tables), stream))

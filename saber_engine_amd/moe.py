@@ -27,8 +27,12 @@ class MoeLayerIU8:
             arrive=torch.zeros(1, **i32))          # persistent: zeroed once, left zero by the kernel
         self.tables = iu8.MoeTables(*[self.buf[n].data_ptr() for n in iu8.MOE_TABLE_FIELDS])
         u8 = dict(dtype=torch.uint8, device=device)
-        self.q1 = torch.zeros(iu8.a_bytes(tokens, hidden), **u8)
-        self.s1 = torch.zeros(tokens, dtype=torch.float32, device=device)
+        # the streaming cell (16-row tiles) gathers token rows inside the grouped GEMM; the MFMA cell
+        # runs on rows gathered and quantised once into expert-major order
+        self.gather_in_gemm = self.tb == 1
+        rows1 = tokens if self.gather_in_gemm else self.rows_cap
+        self.q1 = torch.zeros(iu8.a_bytes(rows1, hidden), **u8)
+        self.s1 = torch.zeros(rows1, dtype=torch.float32, device=device)
         self.gu = torch.zeros((self.rows_cap, 2 * inter), dtype=torch.int16, device=device)
         self.q2 = torch.zeros(iu8.a_bytes(self.rows_cap, inter), **u8)
         self.s2 = torch.zeros(self.rows_cap, dtype=torch.float32, device=device)
@@ -49,9 +53,12 @@ class MoeLayerIU8:
         """x bf16 bits [T,H] (int16 tensor), logits bf16 bits [T,E]; every launch on `stream`."""
         c, T, E, k, H, I = self.ctx, self.T, self.E, self.topk, self.H, self.I
         c.moe_route(logits.data_ptr(), T, E, k, self.tb, self.tables, stream)
-        c.quant(x.data_ptr(), self.q1.data_ptr(), self.s1.data_ptr(), T, H, stream)
-        c.moe_grouped(self.q1.data_ptr(), self.s1.data_ptr(), self.xptr_gu.data_ptr(), self.gu.data_ptr(), 2 * I, H, True,
-                      T, E, k, self.tb, self.tables, stream)
+        if self.gather_in_gemm:
+            c.quant(x.data_ptr(), self.q1.data_ptr(), self.s1.data_ptr(), T, H, stream)
+        else:
+            c.moe_quant_rows(x.data_ptr(), self.q1.data_ptr(), self.s1.data_ptr(), H, self.rows_cap, self.tables, stream)
+        c.moe_grouped(self.q1.data_ptr(), self.s1.data_ptr(), self.xptr_gu.data_ptr(), self.gu.data_ptr(), 2 * I, H,
+                      self.gather_in_gemm, T, E, k, self.tb, self.tables, stream)
         c.moe_silu_mul_quant(self.gu.data_ptr(), self.q2.data_ptr(), self.s2.data_ptr(), I, self.rows_cap, self.tables, stream)
         c.moe_grouped(self.q2.data_ptr(), self.s2.data_ptr(), self.xptr_dn.data_ptr(), self.y.data_ptr(), H, I, False,
                       T, E, k, self.tb, self.tables, stream)

@@ -64,3 +64,42 @@ def test_fused_form_refuses_what_it_does_not_hold(ctx):
     assert e.value.code == iu8.E_RULE
     with pytest.raises(iu8.IU8Error):
         iu8.resolve_fused(iu8.W4, 1, 250, 1024)
+
+
+def test_quant_ties_and_near_ties_round_like_the_ieee_divide(ctx):
+    """Rows built so that x / scale lands on half-integers (exact ties, half to even) and one bf16
+    step beside them: the producer's reciprocal fast path must hand these to the divide."""
+    say("quant ties")
+    K = 1024
+    rows = []
+    for amax in (127.0, 254.0, 63.5, 1.984375, 3.96875e-3, 508.0):
+        sc = np.float32(amax) / np.float32(127.0)
+        ks = np.arange(K, dtype=np.float32) % 126          # below the row maximum, which x[0] sets
+        x = (ks + np.float32(0.5)) * sc * np.where(np.arange(K) % 2 == 0, 1, -1).astype(np.float32)
+        x[0] = amax
+        rows.append(x)
+        b = synth.f32_to_bf16_bits(x).astype(np.uint16)
+        for step in (1, -1):                      # the neighbouring bf16 values of every tie
+            rows.append(synth.bf16_bits_to_f32((b.astype(np.int32) + step).astype(np.uint16)))
+            rows[-1][0] = amax
+    X = synth.f32_to_bf16_bits(np.stack(rows).astype(np.float32))
+    M = X.shape[0]
+    want_q, want_s = ref.quant_bf16(X)
+    x = dev_bf16_bits(X)
+    q = torch.zeros(iu8.a_bytes(M, K), dtype=torch.uint8, device="cuda")
+    s = torch.zeros(M, dtype=torch.float32, device="cuda")
+    ctx.quant(x.data_ptr(), q.data_ptr(), s.data_ptr(), M, K)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(s.cpu().numpy().view(np.uint32), want_s.view(np.uint32))
+    np.testing.assert_array_equal(iu8.unpack_a(q.cpu().numpy(), M, K), want_q)
+    # ... and through the fused decode linear, which quantises in its prologue
+    W, ws = synth.weights(np.random.default_rng(3), 64, K, False)
+    wf, wsd = dev_u8(iu8.repack_w4(W)), dev_f32(ws)
+    for r0 in range(0, M - M % 4, 4):
+        xs = dev_bf16_bits(X[r0:r0 + 4])
+        q4 = torch.zeros(iu8.a_bytes(4, K), dtype=torch.uint8, device="cuda")
+        s4 = torch.zeros(4, dtype=torch.float32, device="cuda")
+        c = torch.zeros((4, 64), dtype=torch.int16, device="cuda")
+        ctx.linear_fused(iu8.W4, xs.data_ptr(), wf.data_ptr(), wsd.data_ptr(), c.data_ptr(), 4, 64, K, q=q4.data_ptr(), scale=s4.data_ptr())
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(iu8.unpack_a(q4.cpu().numpy(), 4, K), want_q[r0:r0 + 4])
