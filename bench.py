@@ -28,9 +28,9 @@ HBM_PEAK_GBPS = 8000.0      # MI355X published HBM3E bandwidth
 INT8_PEAK_TOPS = 5000.0     # MI355X published dense int8 MFMA peak
 LAYERS = 6                  # distinct weight copies walked by successive steps (6 x 165 MB)
 # HBM-side bytes of one launch of the dominant kernel, mean over the four layer shapes, from
-# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this very command (profiles/*hbm_counters*.txt), each
+# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this very command (profiles/macaq_iu8_decq_w4_tm1__layer_set_m1.txt), each
 # counter scaled by what it reads for the 256 MiB copy probe. Keyed by (kernel, M); None = not measured.
-TRAFFIC = {}
+TRAFFIC = {("macaq_iu8_decq_w4_tm1", 1): 41714330.0, ("macaq_iu8_dec_w4_tm1", 1): 41993502.0}
 
 
 def alg_bytes(m, n, k, w8=False):
@@ -46,6 +46,7 @@ def main():
     ap.add_argument("--m", type=int, default=1, help="tokens per step (decode band, 1..16)")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-moe", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--probe-copy", action="store_true",
                     help="also launch the 256 MiB copy probe (scale factor of the HBM byte counters under rocprofv3 --pmc)")
@@ -300,6 +301,45 @@ def main():
                                                   unit="POP/s", frac=round(tops / INT8_PEAK_TOPS, 4), traffic=None,
                                                   note="GEMM launches alone over the four shapes (ops = 2*M*N*K); "
                                                        "with_quant adds the int8 producer launches"))
+    # ---- the routed-expert layer of configs[4] (128 experts, top-8, hidden 4096, expert intermediate
+    # 1536) as its launch train, T = 16 (weight streaming) and T = 4096 (MFMA); weights are random
+    # nibbles generated on the device (parity of this path is the GPU tests' business)
+    if not args.no_moe:
+        from saber_engine_amd.moe import MoeLayerIU8
+
+        E, topk, H, I = 128, 8, 4096, 1536
+        g = torch.Generator(device=dev)
+        g.manual_seed(0)
+        wgu = torch.randint(0, 256, (E, 2 * I * H // 2), dtype=torch.uint8, device=dev, generator=g)
+        wdn = torch.randint(0, 256, (E, H * I // 2), dtype=torch.uint8, device=dev, generator=g)
+        wsgu = torch.rand((E, 2 * I), device=dev, generator=g) * 0.02 + 1e-4
+        wsdn = torch.rand((E, H), device=dev, generator=g) * 0.02 + 1e-4
+        moe = {}
+        for T in (16, 4096):
+            layer = MoeLayerIU8(ctx, T, E, topk, H, I)
+            layer.set_weights(wgu, wsgu, wdn, wsdn)
+            x = torch.randn((T, H), device=dev, generator=g).to(torch.bfloat16).view(torch.int16)
+            lg = torch.randn((T, E), device=dev, generator=g).to(torch.bfloat16).view(torch.int16)
+            reps = 20 if T == 16 else 5
+            with torch.cuda.stream(stream):
+                for _ in range(3):
+                    layer.forward(x, lg, sh)
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record(stream)
+                for _ in range(reps):
+                    layer.forward(x, lg, sh)
+                e1.record(stream)
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) * 1e3 / reps
+            live = int((layer.buf["expert_cnt"] > 0).sum().item())
+            wbytes = live * (2 * I * H // 2 + H * I // 2 + 4 * (2 * I + H))
+            ops = 2.0 * T * topk * (2 * I * H + H * I)
+            moe["t%d" % T] = dict(layer_us=round(us, 1), launches=6, tile_rows=16 * layer.tb, experts_touched=live,
+                                  weight_gbps=round(wbytes / us / 1e3, 1), tops=round(ops / us / 1e6, 1),
+                                  bound="hbm" if T == 16 else "mfma",
+                                  frac=round((wbytes / us / 1e3) / HBM_PEAK_GBPS if T == 16 else (ops / us / 1e6) / INT8_PEAK_TOPS, 4))
+            del layer, x, lg
+        out["moe_e128_top8_h4096_i1536"] = moe
     print(json.dumps(out), flush=True)
     ctx.close()
 
