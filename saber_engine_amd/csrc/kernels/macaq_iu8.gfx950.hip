@@ -48,17 +48,19 @@
 // reference fuses producers the other way round (norm/activation + quant in front of an int8 GEMM,
 // crates/saber-kernels/hip/mxfp4_hadi8.hip); this is the same law inside the GEMV's prologue, where
 // it hides behind the first weight loads.
-#define IU8_DECQ(name, W8, D)                                                                                      \
-  extern "C" __global__ __launch_bounds__(512) void name(                                                          \
+#define IU8_DECQ(name, W8, D) IU8_DECQX(name, W8, 1, 4, 8, D)  /* the default decode cell's geometry */
+#define IU8_DECQX(name, W8, NT, KW, WPB, D)                                                                            \
+  extern "C" __global__ __launch_bounds__(WPB * 64) void name(                                                          \
       const unsigned short *__restrict__ x, const unsigned char *__restrict__ w, const float *__restrict__ ws,     \
       unsigned char *__restrict__ q, float *__restrict__ scale, unsigned short *__restrict__ c, int m, int n,      \
       int k) {                                                                                                     \
-    iu8_dec_body<1, W8, 1, 4, 8, D, 20, false, true>((const unsigned char *)x, w, nullptr, ws, nullptr, nullptr, c, \
+    iu8_dec_body<1, W8, NT, KW, WPB, D, 20, false, true>((const unsigned char *)x, w, nullptr, ws, nullptr, nullptr, c, \
                                                      iu8_rows{nullptr, 0, m}, n, k, q, scale);                     \
   }
 IU8_DECQ(macaq_iu8_decq_w4_tm1, false, 8)
 IU8_DECQ(macaq_iu8_decq_w8_tm1, true, 4)
 #undef IU8_DECQ
+#undef IU8_DECQX
 
 // Persistent launch: gridDim.x workgroups (one or OCC a CU) walk the tiles of the m x n output.
 #define IU8_PF32(name, W8, WMW, WNW, TM, TN, ACC, ST, OCC)                                                        \
