@@ -206,6 +206,23 @@ int saber_iu8_launch(saber_iu8_ctx *ctx, const saber_iu8_desc *desc, const saber
 /* Per-token int8 quantisation: x bf16 [m,k] -> q (A edge, saber_iu8_a_bytes) + scale f32 [m]. */
 int saber_iu8_quant(saber_iu8_ctx *ctx, const void *x_bf16, void *q, float *scale, uint32_t m, uint32_t k, void *stream);
 
+/* The Hadamard-basis producers in front of a MACaQ-W4A8 GEMM (crates/saber-kernels/hip/mxfp4_hadi8.hip,
+ * hip/macaq_had.h): the producer's bf16-rounded values times `had_t` (f32 [width]), a 32-point
+ * Hadamard transform per 32-block, times 1/sqrt(32), then the per-token int8 law; codes in the A edge
+ * order. Row widths: multiples of 64, at most 20,480.
+ *   quant_had           x bf16 [m,k]                                 (the transform + the law alone)
+ *   silu_mul_quant_had  gu bf16 [m, 2n] (gate | up) -> bf16(bf16(silu(gate)) * up)
+ *   add_rms_quant_had   y, res bf16 [m,k], w bf16 [k]: v = y + res (stored to res_out as bf16),
+ *                       bf16(v * inv * (w + 1)) with inv = 1/sqrt(mean(v^2) + eps)
+ * The square-root reciprocal is IEEE here where the reference calls the device's approximate rsqrtf. */
+int saber_iu8_quant_had(saber_iu8_ctx *ctx, const void *x_bf16, void *q, float *scale, uint32_t m, uint32_t k,
+                        const float *had_t, void *stream);
+int saber_iu8_silu_mul_quant_had(saber_iu8_ctx *ctx, const void *gu_bf16, void *q, float *scale, uint32_t m, uint32_t n,
+                                 const float *had_t, void *stream);
+int saber_iu8_add_rms_quant_had(saber_iu8_ctx *ctx, const void *y_bf16, const void *res_bf16, const void *w_bf16, void *q,
+                                float *scale, void *res_out_bf16, uint32_t m, uint32_t k, float eps, const float *had_t,
+                                void *stream);
+
 /* The whole decode linear in one launch where the shape allows (at most 4 rows whose codes fit the
  * kernel's 20 KiB staging area; saber_iu8_fused_holds): per-token quantisation fused into the
  * GEMV's activation staging. x bf16 [m,k]; q (A edge) and scale f32 [m] are optional outputs (NULL:

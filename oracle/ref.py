@@ -222,3 +222,44 @@ def moe_layer(x_bits, topk_w, lay, Wgu, wsgu, Wdn, wsdn, I, threads=1, taps=Fals
                          _p(_c(Wdn, np.uint8)), _p(_c(wsdn, np.float32)), _p(Y), _p(out), _p(gu), _p(q2), _p(s2),
                          C.c_int(threads))
     return dict(Y=Y, out=out, gu=gu, q2=q2, s2=s2)
+
+
+# ---------------------------------------------------------------------------- Hadamard-basis producers
+
+def had32_rows(v, t):
+    """f32 rows [M,K] (K % 32 == 0) -> rows transformed per 32-block."""
+    v = np.array(v, dtype=np.float32, copy=True, order="C")
+    M, K = v.shape
+    lib().w4a8_had32_rows(_p(v), _p(_c(t, np.float32)), C.c_int(M), C.c_int(K))
+    return v
+
+
+def quant_had(x_bits, t):
+    x = _c(x_bits, np.uint16)
+    M, K = x.shape
+    t = _c(t, np.float32)
+    q, s = np.empty((M, K), np.int8), np.empty(M, np.float32)
+    for m in range(M):
+        lib().w4a8_quant_had_row(_p(x[m]), _p(t), C.c_int(K), _p(q[m]), _p(s[m:m + 1]))
+    return q, s
+
+
+def silu_mul_quant_had(gu_bits, t):
+    gu = _c(gu_bits, np.uint16)
+    M, I = gu.shape[0], gu.shape[1] // 2
+    t = _c(t, np.float32)
+    q, s = np.empty((M, I), np.int8), np.empty(M, np.float32)
+    for m in range(M):
+        lib().w4a8_silu_mul_quant_had_row(_p(gu[m]), _p(t), C.c_int(I), _p(q[m]), _p(s[m:m + 1]))
+    return q, s
+
+
+def add_rms_quant_had(y_bits, res_bits, w_bits, t, eps, threads_per_row=256):
+    y, res, w = _c(y_bits, np.uint16), _c(res_bits, np.uint16), _c(w_bits, np.uint16)
+    M, K = y.shape
+    t = _c(t, np.float32)
+    q, s, ro = np.empty((M, K), np.int8), np.empty(M, np.float32), np.empty((M, K), np.uint16)
+    for m in range(M):
+        lib().w4a8_add_rms_quant_had_row(_p(y[m]), _p(res[m]), _p(w), _p(t), C.c_int(K), C.c_float(eps),
+                                         C.c_int(threads_per_row), _p(q[m]), _p(s[m:m + 1]), _p(ro[m]))
+    return q, s, ro

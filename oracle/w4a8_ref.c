@@ -536,3 +536,112 @@ void w4a8_moe_layer(const uint16_t *x, int T, int H, int I, int E, int topk, con
   w4a8_combine(Y, topk_w, route_pos, T, topk, H, out);
   free(q1); free(s1); free(qa); free(sa); free(S1); free(S2); free(gu); free(q2); free(s2);
 }
+
+/* ------------------------------------------------------------------ Q3: Hadamard-basis producers */
+
+/* The activation transform of the `*_hadi8_*` producers (hip/macaq_had.h:1-19, 47-83), on one
+ * 32-block: u = v * t (one f32 multiply each), the unnormalised Sylvester butterfly over element
+ * bits 0, 1, 2, 3, 4 in that order, each stage (lo, hi) -> (lo + hi, lo - hi) in f32, then one f32
+ * multiply by (float)(1/sqrt(32)) = 0x3E3504F3. In place. */
+void w4a8_had32_block(float *v, const float *t) {
+  for (int e = 0; e < 32; ++e) {
+    volatile float u = v[e] * t[e];
+    v[e] = u;
+  }
+  for (int s = 1; s < 32; s <<= 1)
+    for (int e = 0; e < 32; ++e) {
+      if (e & s) continue;
+      volatile float lo = v[e], hi = v[e | s];
+      volatile float a = lo + hi, b = lo - hi;
+      v[e] = a;
+      v[e | s] = b;
+    }
+  const float inv = bits_f32(0x3E3504F3u);
+  for (int e = 0; e < 32; ++e) {
+    volatile float r = v[e] * inv;
+    v[e] = r;
+  }
+}
+
+/* Rows of f32 values (K a multiple of 32) -> transformed rows. */
+void w4a8_had32_rows(float *v, const float *t, int M, int K) {
+  for (int m = 0; m < M; ++m)
+    for (int b = 0; b < K; b += 32) w4a8_had32_block(v + (size_t)m * K + b, t + b);
+}
+
+/* quant_hadi8: bf16 row -> had32 -> Q1. */
+void w4a8_quant_had_row(const uint16_t *x, const float *t, int K, int8_t *q, float *scale) {
+  float *v = (float *)malloc(sizeof(float) * (size_t)K);
+  for (int k = 0; k < K; ++k) v[k] = w4a8_bf16_f32(x[k]);
+  w4a8_had32_rows(v, t, 1, K);
+  w4a8_quant_row(v, K, q, scale);
+  free(v);
+}
+
+/* silu_mul_quant_hadi8 (hip/mxfp4_hadi8.hip:117-146): p = bf16(bf16(silu(g)) * u), had32, Q1. */
+void w4a8_silu_mul_quant_had_row(const uint16_t *gu, const float *t, int I, int8_t *q, float *scale) {
+  float *p = (float *)malloc(sizeof(float) * (size_t)I);
+  for (int i = 0; i < I; ++i) {
+    const float s = w4a8_bf16_f32(w4a8_silu_bf16(gu[i]));
+    volatile float m = s * w4a8_bf16_f32(gu[I + i]);
+    p[i] = w4a8_bf16_f32(w4a8_bf16_rne(m));
+  }
+  w4a8_had32_rows(p, t, 1, I);
+  w4a8_quant_row(p, I, q, scale);
+  free(p);
+}
+
+/* add_rms_quant_hadi8 (hip/mxfp4_hadi8.hip:60-115), one row, as a workgroup of T threads computes
+ * it: v = f32(y) + f32(res); res_out = bf16(v); the sum of squares accumulates per thread with fma
+ * over its 8-element groups g = tid + i*T in order, then the reference's trees: shfl_down 16, 8, 4, 2,
+ * 1 inside each 32 lanes, then shfl_down T/64 ... 1 over the T/32 partials. inv = 1 / sqrt(ssq / K +
+ * eps) with IEEE sqrt and divide (the reference calls the device's approximate rsqrtf, which no
+ * host can restate: parity unpinned against the reference's hardware for this one function).
+ * out = bf16((v * inv) * (f32(w) + 1)), had32, Q1. */
+void w4a8_add_rms_quant_had_row(const uint16_t *y, const uint16_t *res, const uint16_t *w, const float *t, int K,
+                                float eps, int T, int8_t *q, float *scale, uint16_t *res_out) {
+  float *v = (float *)malloc(sizeof(float) * (size_t)K);
+  float *part = (float *)calloc((size_t)T, sizeof(float));
+  const int KV = K >> 3;
+  for (int k = 0; k < K; ++k) {
+    volatile float s = w4a8_bf16_f32(y[k]) + w4a8_bf16_f32(res[k]);
+    v[k] = s;
+    res_out[k] = w4a8_bf16_rne(s);
+  }
+  for (int tid = 0; tid < T; ++tid) {
+    float ssq = 0.f;
+    for (int g = tid; g < KV; g += T)
+      for (int j = 0; j < 8; ++j) ssq = fmaf(v[g * 8 + j], v[g * 8 + j], ssq);
+    part[tid] = ssq;
+  }
+  float wave[64];
+  for (int wv = 0; wv < T / 32; ++wv) {
+    float l[32];
+    memcpy(l, part + wv * 32, sizeof l);
+    for (int o = 16; o; o >>= 1)
+      for (int i = 0; i < o; ++i) {
+        volatile float s = l[i] + l[i + o];
+        l[i] = s;
+      }
+    wave[wv] = l[0];
+  }
+  for (int o = T / 64; o; o >>= 1)
+    for (int i = 0; i < o; ++i) {
+      volatile float s = wave[i] + wave[i + o];
+      wave[i] = s;
+    }
+  volatile float mean = wave[0] / (float)K;
+  volatile float me = mean + eps;
+  volatile float rt = sqrtf(me);
+  volatile float inv = 1.f / rt;
+  for (int k = 0; k < K; ++k) {
+    volatile float a = v[k] * inv;
+    volatile float wp = w4a8_bf16_f32(w[k]) + 1.f;
+    volatile float b = a * wp;
+    v[k] = w4a8_bf16_f32(w4a8_bf16_rne(b));
+  }
+  w4a8_had32_rows(v, t, 1, K);
+  w4a8_quant_row(v, K, q, scale);
+  free(part);
+  free(v);
+}

@@ -17,6 +17,13 @@ static const Signature SIG_PF = {{"a", K::Buffer}, {"w", K::Buffer}, {"as", K::B
 static const Signature SIG_QUANT = {{"x", K::Buffer}, {"q", K::Buffer}, {"scale", K::Buffer}, {"k", K::I32}};
 static const Signature SIG_QUANT_ROWS = {{"x", K::Buffer}, {"q", K::Buffer},       {"scale", K::Buffer},
                                          {"k", K::I32},    {"row_tok", K::Buffer}, {"meta", K::Buffer}};
+// the Hadamard-basis producers: the reference's lists, `had_t` last
+// (prebuilt/gfx1201/mxfp4_hadi8.manifest.toml: 64 and 40 bytes)
+static const Signature SIG_HAD_ARQ = {{"y", K::Buffer},     {"res", K::Buffer},     {"w", K::Buffer},
+                                      {"q", K::Buffer},     {"scale", K::Buffer},   {"res_out", K::Buffer},
+                                      {"K", K::I32},        {"eps", K::F32},        {"had_t", K::Buffer}};
+static const Signature SIG_HAD_SMQ = {{"gu", K::Buffer}, {"q", K::Buffer}, {"scale", K::Buffer}, {"N", K::I32}, {"had_t", K::Buffer}};
+static const Signature SIG_HAD_Q = {{"x", K::Buffer}, {"q", K::Buffer}, {"scale", K::Buffer}, {"k", K::I32}, {"had_t", K::Buffer}};
 static const Signature SIG_SILU = {{"gu", K::Buffer}, {"q", K::Buffer},       {"scale", K::Buffer},
                                    {"n", K::I32},     {"row_tok", K::Buffer}, {"meta", K::Buffer}};
 static const Signature SIG_TABLE = {{"out", K::Buffer}};
@@ -46,6 +53,9 @@ const Signature *signature_for(const std::string &k) {
   if (starts(k, "macaq_iu8_dec_")) return &SIG_DEC;
   if (starts(k, "macaq_iu8_decq_")) return &SIG_DECQ;
   if (starts(k, "macaq_iu8_pf_")) return &SIG_PF;
+  if (starts(k, "add_rms_quant_hadi8_")) return &SIG_HAD_ARQ;
+  if (starts(k, "silu_mul_quant_hadi8_")) return &SIG_HAD_SMQ;
+  if (starts(k, "quant_hadi8_")) return &SIG_HAD_Q;
   if (starts(k, "macaq_i8_quant_rows_")) return &SIG_QUANT_ROWS;
   if (starts(k, "macaq_i8_quant_")) return &SIG_QUANT;
   if (starts(k, "macaq_i8_silu_mul_quant_")) return &SIG_SILU;

@@ -369,6 +369,59 @@ int saber_iu8_gemm_acc(saber_iu8_ctx *ctx, int wkind, const void *a, const void 
   return launch_gemm(ctx, d, a, (const float *)acc, w, (const float *)acc, acc, nullptr, nullptr, stream);
 }
 
+// ---------------------------------------------------------------------------- Hadamard-basis producers
+
+// One workgroup a row, T = 256 threads for rows of up to 10,240 elements (5 groups of 8 a thread),
+// 512 up to 20,480 (the reference's t256 / t512 pair, crates/saber-kernels/src/macaq_iu8.rs:864-875).
+static int had_desc(const char *op, const char *stem, uint32_t rows, uint32_t width, saber_iu8_desc *d) {
+  if (rows == 0 || width == 0) return fail(SABER_IU8_E_RULE, fmt("%s: %u rows of %u has nothing to do", op, rows, width));
+  if (width % 64 != 0 || width > 20480)
+    return fail(SABER_IU8_E_RULE,
+                fmt("%s: row width %u must be a multiple of 64 (whole A fragments, whole 32-blocks), at most 20480", op, width));
+  const uint32_t t = width <= 10240 ? 256 : 512;
+  const std::string name = fmt("%s_hadi8_t%u_tiled1", stem, t);
+  const uint32_t grid[3] = {rows, 1, 1};
+  if (int rc = saber_iu8_describe_raw(name.c_str(), "mxfp4_hadi8", grid, t, d)) return rc;
+  snprintf(d->op, sizeof d->op, "%s", op);
+  return 0;
+}
+static void set_f32(saber_iu8_desc *d, const char *name, float v) {
+  for (uint32_t i = 0; i < d->n_args; ++i)
+    if (!strcmp(d->args[i].name, name)) {
+      d->args[i].kind = SABER_IU8_ARG_F32;
+      d->args[i].fval = v;
+    }
+}
+
+int saber_iu8_quant_had(saber_iu8_ctx *ctx, const void *x, void *q, float *scale, uint32_t m, uint32_t k,
+                        const float *had_t, void *stream) {
+  saber_iu8_desc d;
+  if (int rc = had_desc("quant_had_i8", "quant", m, k, &d)) return rc;
+  set_i32(&d, "k", k);
+  const saber_iu8_binding b[] = {{"x", (void *)x}, {"q", q}, {"scale", scale}, {"had_t", (void *)had_t}};
+  return saber_iu8_launch(ctx, &d, b, 4, stream);
+}
+
+int saber_iu8_silu_mul_quant_had(saber_iu8_ctx *ctx, const void *gu, void *q, float *scale, uint32_t m, uint32_t n,
+                                 const float *had_t, void *stream) {
+  saber_iu8_desc d;
+  if (int rc = had_desc("silu_mul_quant_had_i8", "silu_mul_quant", m, n, &d)) return rc;
+  set_i32(&d, "N", n);
+  const saber_iu8_binding b[] = {{"gu", (void *)gu}, {"q", q}, {"scale", scale}, {"had_t", (void *)had_t}};
+  return saber_iu8_launch(ctx, &d, b, 4, stream);
+}
+
+int saber_iu8_add_rms_quant_had(saber_iu8_ctx *ctx, const void *y, const void *res, const void *w, void *q, float *scale,
+                                void *res_out, uint32_t m, uint32_t k, float eps, const float *had_t, void *stream) {
+  saber_iu8_desc d;
+  if (int rc = had_desc("add_rms_quant_had_i8", "add_rms_quant", m, k, &d)) return rc;
+  set_i32(&d, "K", k);
+  set_f32(&d, "eps", eps);
+  const saber_iu8_binding b[] = {{"y", (void *)y}, {"res", (void *)res}, {"w", (void *)w}, {"q", q},
+                                 {"scale", scale}, {"res_out", res_out}, {"had_t", (void *)had_t}};
+  return saber_iu8_launch(ctx, &d, b, 7, stream);
+}
+
 // ---------------------------------------------------------------------------- routed experts
 
 uint32_t saber_iu8_moe_rows_cap(uint32_t tokens, uint32_t topk, uint32_t experts) {

@@ -109,6 +109,9 @@ def lib():
         L.saber_iu8_gemm_acc.argtypes = [C.c_void_p, C.c_int] + [C.c_void_p] * 3 + [C.c_uint32] * 3 + [C.c_void_p]
         L.saber_iu8_fused_holds.argtypes = [C.c_uint32, C.c_uint32]
         L.saber_iu8_linear_fused.argtypes = [C.c_void_p, C.c_int] + [C.c_void_p] * 6 + [C.c_uint32] * 3 + [C.c_void_p]
+        L.saber_iu8_quant_had.argtypes = [C.c_void_p] * 4 + [C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p]
+        L.saber_iu8_silu_mul_quant_had.argtypes = [C.c_void_p] * 4 + [C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p]
+        L.saber_iu8_add_rms_quant_had.argtypes = [C.c_void_p] * 7 + [C.c_uint32, C.c_uint32, C.c_float, C.c_void_p, C.c_void_p]
         L.saber_iu8_get_counters.argtypes = [C.c_void_p, C.POINTER(Counters)]
         L.saber_iu8_has_kernel.argtypes = [C.c_void_p, C.c_char_p]
         for fn in ("saber_iu8_moe_rows_cap", "saber_iu8_moe_tile_blocks"):
@@ -290,6 +293,15 @@ class Context:
 
     def linear_fused(self, wkind, x, w, w_scale, c, m, n, k, q=None, scale=None, stream=0):
         _check(lib().saber_iu8_linear_fused(self._h, wkind, x, w, w_scale, c, q, scale, m, n, k, stream))
+
+    def quant_had(self, x, q, scale, m, k, had_t, stream=0):
+        _check(lib().saber_iu8_quant_had(self._h, x, q, scale, m, k, had_t, stream))
+
+    def silu_mul_quant_had(self, gu, q, scale, m, n, had_t, stream=0):
+        _check(lib().saber_iu8_silu_mul_quant_had(self._h, gu, q, scale, m, n, had_t, stream))
+
+    def add_rms_quant_had(self, y, res, w, q, scale, res_out, m, k, eps, had_t, stream=0):
+        _check(lib().saber_iu8_add_rms_quant_had(self._h, y, res, w, q, scale, res_out, m, k, eps, had_t, stream))
 
     def gemm_acc(self, wkind, a, w, acc, m, n, k, stream=0):
         _check(lib().saber_iu8_gemm_acc(self._h, wkind, a, w, acc, m, n, k, stream))
