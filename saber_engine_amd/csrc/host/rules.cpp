@@ -165,12 +165,11 @@ int resolve(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *out) 
     const uint32_t tm = (m + 15) / 16;
     std::string name = fmt("macaq_iu8_dec_%s_tm%u", tag, tm);
     if (tm == 1) {
-      // live rows staged in LDS when they fit the 20 KiB or the 80 KiB form, else read from L2
+      // live rows staged in LDS when they fit the 20 KiB form, else streamed from L2 beside the
+      // weights (the 80 KiB staged form stays loadable by name; it measured slower on every shape)
       uint32_t mr = 1;
       while (mr < m) mr *= 2;
-      const uint64_t need = (uint64_t)mr * k;
-      if (need > 80 * 1024) name += "_a0";
-      else if (need > 20 * 1024) name += "_a80";
+      if ((uint64_t)mr * k > 20 * 1024) name += "_a0";
     }
     const DecVariant *v = dec_variant(name);
     if (!v) return fail(SABER_IU8_E_RULE, name + ": no such variant");

@@ -76,7 +76,7 @@ def test_decode_band_routing(wk, tag):
 def test_activation_rows_are_staged_when_they_fit():
     assert iu8.resolve(iu8.W4, 1, 5120, 17408).kernel == b"macaq_iu8_dec_w4_tm1"        # 17 KiB
     assert iu8.resolve(iu8.W4, 4, 5120, 5120).kernel == b"macaq_iu8_dec_w4_tm1"         # 20 KiB
-    assert iu8.resolve(iu8.W4, 16, 5120, 5120).kernel == b"macaq_iu8_dec_w4_tm1_a80"    # 80 KiB
+    assert iu8.resolve(iu8.W4, 16, 5120, 5120).kernel == b"macaq_iu8_dec_w4_tm1_a0"     # past 20 KiB: streamed
     assert iu8.resolve(iu8.W4, 8, 5120, 17408).kernel == b"macaq_iu8_dec_w4_tm1_a0"     # does not fit
 
 
