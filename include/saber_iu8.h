@@ -80,6 +80,7 @@ int saber_iu8_repack_w8_from_gfx12(const uint8_t *frag12, uint32_t n, uint32_t k
 #define SABER_IU8_ARG_NULL_BUFFER 1 /* a named buffer passed as NULL (workspaces at ks == 1) */
 #define SABER_IU8_ARG_I32 2
 #define SABER_IU8_ARG_F32 3
+#define SABER_IU8_ARG_I64 4 /* an 8-byte by-value integer (a row stride in elements) */
 
 typedef struct {
   char name[24];
@@ -214,6 +215,14 @@ int saber_iu8_quant(saber_iu8_ctx *ctx, const void *x_bf16, void *q, float *scal
  *   silu_mul_quant_had  gu bf16 [m, 2n] (gate | up) -> bf16(bf16(silu(gate)) * up)
  *   add_rms_quant_had   y, res bf16 [m,k], w bf16 [k]: v = y + res (stored to res_out as bf16),
  *                       bf16(v * inv * (w + 1)) with inv = 1/sqrt(mean(v^2) + eps)
+ *   gdn_norm_quant_had  x bf16 [m,n] of 128-element heads, z bf16 rows `z_stride` elements apart,
+ *                       w bf16 [128]: bf16(((x * inv_head) * w) * silu(z)), silu in f32, inv_head =
+ *                       1/sqrt(mean_head(x^2) + eps); n a multiple of 128, at most 10,240
+ *                       (hip/mxfp4_hadi8.hip:148-186, symbol gdn_norm_quant_hadi8_t256_tiled1)
+ *   attn_gate_quant_had core bf16 [m,n]; gate = the projection's [q | gate] block, rows `gate_stride`
+ *                       elements apart, head h's gate at h*2*head_dim + head_dim:
+ *                       bf16(core * bf16(sigmoid(gate))); n at most 6,144
+ *                       (hip/attn_glue_hadi8.hip:23-79, symbol attn_gate_quant_hadi8_t256_tiled1)
  * The square-root reciprocal is IEEE here where the reference calls the device's approximate rsqrtf. */
 int saber_iu8_quant_had(saber_iu8_ctx *ctx, const void *x_bf16, void *q, float *scale, uint32_t m, uint32_t k,
                         const float *had_t, void *stream);
@@ -222,6 +231,12 @@ int saber_iu8_silu_mul_quant_had(saber_iu8_ctx *ctx, const void *gu_bf16, void *
 int saber_iu8_add_rms_quant_had(saber_iu8_ctx *ctx, const void *y_bf16, const void *res_bf16, const void *w_bf16, void *q,
                                 float *scale, void *res_out_bf16, uint32_t m, uint32_t k, float eps, const float *had_t,
                                 void *stream);
+int saber_iu8_gdn_norm_quant_had(saber_iu8_ctx *ctx, const void *x_bf16, const void *z_bf16, int64_t z_stride,
+                                 const void *w_bf16, void *q, float *scale, uint32_t m, uint32_t n, float eps,
+                                 const float *had_t, void *stream);
+int saber_iu8_attn_gate_quant_had(saber_iu8_ctx *ctx, const void *core_bf16, const void *gate_bf16, void *q, float *scale,
+                                  uint32_t m, uint32_t n, uint32_t head_dim, uint32_t gate_stride, const float *had_t,
+                                  void *stream);
 
 /* The whole decode linear in one launch where the shape allows (at most 4 rows whose codes fit the
  * kernel's 20 KiB staging area; saber_iu8_fused_holds): per-token quantisation fused into the

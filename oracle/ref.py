@@ -263,3 +263,43 @@ def add_rms_quant_had(y_bits, res_bits, w_bits, t, eps, threads_per_row=256):
         lib().w4a8_add_rms_quant_had_row(_p(y[m]), _p(res[m]), _p(w), _p(t), C.c_int(K), C.c_float(eps),
                                          C.c_int(threads_per_row), _p(q[m]), _p(s[m:m + 1]), _p(ro[m]))
     return q, s, ro
+
+
+def silu_f32_table():
+    """f32 z / (1 + expf(-z)) of all 65,536 bf16 inputs, by the host's libm."""
+    out = np.empty(65536, np.float32)
+    lib().w4a8_silu_f32_table(_p(out))
+    return out
+
+
+def sigmoid_bf16_table():
+    """bf16(1 / (1 + expf(-g))) of all 65,536 bf16 inputs."""
+    f = lib().w4a8_sigmoid_bf16
+    f.restype, f.argtypes = C.c_uint16, [C.c_uint16]
+    return np.array([f(i) for i in range(65536)], dtype=np.uint16)
+
+
+def gdn_norm_quant_had(x_bits, z_bits, w_bits, t, eps, silu_tab=None):
+    """x [M,N] bf16 bits, z [M,N] (the rows the stride selects), w [128]; `silu_tab`: a card's own
+    table of the f32 gate, or None for the host's libm."""
+    x, z, w = _c(x_bits, np.uint16), _c(z_bits, np.uint16), _c(w_bits, np.uint16)
+    M, N = x.shape
+    t = _c(t, np.float32)
+    tab = None if silu_tab is None else _c(silu_tab, np.float32)
+    q, s = np.empty((M, N), np.int8), np.empty(M, np.float32)
+    for m in range(M):
+        lib().w4a8_gdn_norm_quant_had_row(_p(x[m]), _p(z[m]), _p(w), _p(t), _p(tab) if tab is not None else None,
+                                          C.c_int(N), C.c_float(eps), _p(q[m]), _p(s[m:m + 1]))
+    return q, s
+
+
+def attn_gate_quant_had(core_bits, gate_bits, t, head_dim):
+    """core [M,n]; gate [M, >= 2n]: the [q | gate] block rows."""
+    core, gate = _c(core_bits, np.uint16), _c(gate_bits, np.uint16)
+    M, n = core.shape
+    t = _c(t, np.float32)
+    q, s = np.empty((M, n), np.int8), np.empty(M, np.float32)
+    for m in range(M):
+        lib().w4a8_attn_gate_quant_had_row(_p(core[m]), _p(gate[m]), _p(t), C.c_int(n), C.c_int(head_dim),
+                                           _p(q[m]), _p(s[m:m + 1]))
+    return q, s

@@ -23,7 +23,10 @@
  * IEEE identities recomputed in float64, int64 matrix products, exhaustive bf16
  * sweeps against torch's rounding, brute-force sorts.  M4 calls libm expf(), the
  * one function that is not IEEE-specified: "parity unpinned" beyond the exhaustive
- * on-device comparison of all 65,536 bf16 inputs.
+ * on-device comparison of all 65,536 bf16 inputs.  The same holds for the bf16
+ * sigmoid of the attention gate; gdn_norm's f32 silu gate is "parity unpinned"
+ * beyond a 2-ulp bound against the card's own table, and the two norms' rsqrtf
+ * (an approximate device instruction) is restated as IEEE 1/sqrt.
  *
  * Structure follows saber-cpux: a scalar law (gemm_*_ref), a vectorised multi-thread
  * body (gemm_fast: 16-column tiles as the work unit, lib.rs:280-303; threads pinned
@@ -643,5 +646,90 @@ void w4a8_add_rms_quant_had_row(const uint16_t *y, const uint16_t *res, const ui
   w4a8_had32_rows(v, t, 1, K);
   w4a8_quant_row(v, K, q, scale);
   free(part);
+  free(v);
+}
+
+/* f32 silu of a bf16 input, z / (1 + expf(-z)), left unrounded: gdn_norm's gate
+ * (hip/mxfp4_hadi8.hip:180-182). expf is the host's libm here and the device's own on a card, so a
+ * checker that wants bit parity passes the device's table of all 65,536 values instead. */
+float w4a8_silu_f32(uint16_t zb) {
+  const float z = w4a8_bf16_f32(zb);
+  volatile float e = expf(-z);
+  volatile float d = 1.f + e;
+  volatile float s = z / d;
+  return s;
+}
+void w4a8_silu_f32_table(float *out) {
+  for (int i = 0; i < 65536; ++i) out[i] = w4a8_silu_f32((uint16_t)i);
+}
+
+/* bf16( 1 / (1 + expf(-g)) ) for one bf16 input (hip/attn_glue_hadi8.hip:49). */
+uint16_t w4a8_sigmoid_bf16(uint16_t gb) {
+  const float g = w4a8_bf16_f32(gb);
+  volatile float e = expf(-g);
+  volatile float d = 1.f + e;
+  volatile float s = 1.f / d;
+  return w4a8_bf16_rne(s);
+}
+
+/* gdn_norm_quant_hadi8 (hip/mxfp4_hadi8.hip:148-186), one row of N = heads * 128 elements. Per
+ * 128-element head, as its 16 lanes compute it: each lane's 8 elements give ssq = x1*x1, then
+ * fma(x0, x0, ssq), then fma over x2..x7; the 16 lane sums meet in the xor butterfly 8, 4, 2, 1
+ * (every lane ends with the same bits, additions being commutative). inv = 1 / sqrt(ssq * (1/128)
+ * + eps) with IEEE sqrt and divide (the reference calls the device's approximate rsqrtf: parity
+ * unpinned against the reference's hardware for that one function). out = bf16(((x * inv) * w[j])
+ * * silu_f32(z)), had32, Q1. `silu_tab`: 65,536 f32 indexed by z's bits, or NULL for libm. */
+void w4a8_gdn_norm_quant_had_row(const uint16_t *x, const uint16_t *z, const uint16_t *w, const float *t,
+                                 const float *silu_tab, int N, float eps, int8_t *q, float *scale) {
+  float *v = (float *)malloc(sizeof(float) * (size_t)N);
+  for (int h = 0; h < N; h += 128) {
+    float lane[16];
+    for (int l = 0; l < 16; ++l) {
+      const uint16_t *xl = x + h + l * 8;
+      const float x0 = w4a8_bf16_f32(xl[0]), x1 = w4a8_bf16_f32(xl[1]);
+      volatile float s = x1 * x1;
+      float ssq = fmaf(x0, x0, s);
+      for (int j = 2; j < 8; ++j) ssq = fmaf(w4a8_bf16_f32(xl[j]), w4a8_bf16_f32(xl[j]), ssq);
+      lane[l] = ssq;
+    }
+    for (int o = 8; o; o >>= 1) {
+      float nx[16];
+      for (int l = 0; l < 16; ++l) {
+        volatile float s = lane[l] + lane[l ^ o];
+        nx[l] = s;
+      }
+      memcpy(lane, nx, sizeof nx);
+    }
+    volatile float mean = lane[0] * (1.f / 128.f);
+    volatile float me = mean + eps;
+    volatile float rt = sqrtf(me);
+    volatile float inv = 1.f / rt;
+    for (int j = 0; j < 128; ++j) {
+      const float sg = silu_tab ? silu_tab[z[h + j]] : w4a8_silu_f32(z[h + j]);
+      volatile float a = w4a8_bf16_f32(x[h + j]) * inv;
+      volatile float b = a * w4a8_bf16_f32(w[j]);
+      volatile float c = b * sg;
+      v[h + j] = w4a8_bf16_f32(w4a8_bf16_rne(c));
+    }
+  }
+  w4a8_had32_rows(v, t, 1, N);
+  w4a8_quant_row(v, N, q, scale);
+  free(v);
+}
+
+/* attn_gate_quant_hadi8 (hip/attn_glue_hadi8.hip:23-79), one row: `gate` is the row of the
+ * projection's [q | gate] block, head h's gate values at h*2*hd + hd; p = bf16(core * bf16(sigmoid
+ * (gate))), had32, Q1. */
+void w4a8_attn_gate_quant_had_row(const uint16_t *core, const uint16_t *gate, const float *t, int n, int hd,
+                                  int8_t *q, float *scale) {
+  float *v = (float *)malloc(sizeof(float) * (size_t)n);
+  for (int e = 0; e < n; ++e) {
+    const int h = e / hd, o = e - h * hd;
+    const float sig = w4a8_bf16_f32(w4a8_sigmoid_bf16(gate[(size_t)h * 2 * hd + hd + o]));
+    volatile float p = w4a8_bf16_f32(core[e]) * sig;
+    v[e] = w4a8_bf16_f32(w4a8_bf16_rne(p));
+  }
+  w4a8_had32_rows(v, t, 1, n);
+  w4a8_quant_row(v, n, q, scale);
   free(v);
 }

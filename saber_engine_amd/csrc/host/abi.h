@@ -8,12 +8,12 @@
 
 namespace iu8 {
 
-enum class ArgKind { Buffer, I32, F32 };
+enum class ArgKind { Buffer, I32, F32, I64 };
 
 struct SigArg {
   const char *name;
   ArgKind kind;
-  uint32_t size() const { return kind == ArgKind::Buffer ? 8 : 4; }
+  uint32_t size() const { return kind == ArgKind::Buffer || kind == ArgKind::I64 ? 8 : 4; }
   uint32_t align() const { return size(); }
   const char *value_kind() const { return kind == ArgKind::Buffer ? "global_buffer" : "by_value"; }
 };

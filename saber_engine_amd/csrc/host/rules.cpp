@@ -53,6 +53,7 @@ int fill_slots(const std::string &kernel, saber_iu8_desc *d) {
     s.size = packed[i].second;
     s.kind = (*sig)[i].kind == ArgKind::Buffer ? SABER_IU8_ARG_BUFFER
              : (*sig)[i].kind == ArgKind::F32  ? SABER_IU8_ARG_F32
+             : (*sig)[i].kind == ArgKind::I64  ? SABER_IU8_ARG_I64
                                                : SABER_IU8_ARG_I32;
   }
   return 0;
@@ -61,7 +62,7 @@ int fill_slots(const std::string &kernel, saber_iu8_desc *d) {
 void set_i32(saber_iu8_desc *d, const char *name, int64_t v) {
   for (uint32_t i = 0; i < d->n_args; ++i)
     if (!strcmp(d->args[i].name, name)) {
-      d->args[i].kind = SABER_IU8_ARG_I32;
+      d->args[i].kind = d->args[i].size == 8 ? SABER_IU8_ARG_I64 : SABER_IU8_ARG_I32;
       d->args[i].ival = v;
     }
 }

@@ -115,7 +115,7 @@ int saber_iu8_desc_set_i32(saber_iu8_desc *desc, const char *name, int64_t value
     if (!strcmp(desc->args[i].name, name)) {
       if (desc->args[i].kind == SABER_IU8_ARG_BUFFER || desc->args[i].kind == SABER_IU8_ARG_NULL_BUFFER)
         return fail(SABER_IU8_E_ARG, std::string(name) + ": a buffer slot, not a scalar");
-      desc->args[i].kind = SABER_IU8_ARG_I32;
+      desc->args[i].kind = desc->args[i].size == 8 ? SABER_IU8_ARG_I64 : SABER_IU8_ARG_I32;
       desc->args[i].ival = value;
       return 0;
     }
@@ -158,6 +158,9 @@ int saber_iu8_pack_kernarg(const saber_iu8_desc *d, const saber_iu8_binding *buf
         memcpy(image + s.offset, &v, 4);
         break;
       }
+      case SABER_IU8_ARG_I64:
+        memcpy(image + s.offset, &s.ival, 8);
+        break;
       case SABER_IU8_ARG_F32:
         memcpy(image + s.offset, &s.fval, 4);
         break;
@@ -420,6 +423,47 @@ int saber_iu8_add_rms_quant_had(saber_iu8_ctx *ctx, const void *y, const void *r
   const saber_iu8_binding b[] = {{"y", (void *)y}, {"res", (void *)res}, {"w", (void *)w}, {"q", q},
                                  {"scale", scale}, {"res_out", res_out}, {"had_t", (void *)had_t}};
   return saber_iu8_launch(ctx, &d, b, 7, stream);
+}
+
+// gdn_norm: rows of whole 128-element heads, one 256-thread workgroup a row (at most 10,240 wide).
+int saber_iu8_gdn_norm_quant_had(saber_iu8_ctx *ctx, const void *x, const void *z, int64_t z_stride, const void *w, void *q,
+                                 float *scale, uint32_t m, uint32_t n, float eps, const float *had_t, void *stream) {
+  if (m == 0 || n == 0) return fail(SABER_IU8_E_RULE, fmt("gdn_norm_quant_had_i8: %u rows of %u has nothing to do", m, n));
+  if (n % 128 != 0 || n > 10240)
+    return fail(SABER_IU8_E_RULE, fmt("gdn_norm_quant_had_i8: row width %u must be whole 128-element heads, at most 10240", n));
+  if (z_stride < (int64_t)n || z_stride % 8 != 0)
+    return fail(SABER_IU8_E_RULE, fmt("gdn_norm_quant_had_i8: z stride %lld must cover the row width %u in whole 16-byte pieces", (long long)z_stride, n));
+  saber_iu8_desc d;
+  const uint32_t grid[3] = {m, 1, 1};
+  if (int rc = saber_iu8_describe_raw("gdn_norm_quant_hadi8_t256_tiled1", "mxfp4_hadi8", grid, 256, &d)) return rc;
+  snprintf(d.op, sizeof d.op, "gdn_norm_quant_had_i8");
+  set_i32(&d, "N", n);
+  set_i32(&d, "zs", z_stride);
+  set_f32(&d, "eps", eps);
+  const saber_iu8_binding b[] = {{"x", (void *)x}, {"z", (void *)z}, {"w", (void *)w}, {"q", q}, {"scale", scale}, {"had_t", (void *)had_t}};
+  return saber_iu8_launch(ctx, &d, b, 6, stream);
+}
+
+// attn_gate: the reference's t256 form holds rows of at most 6,144 elements (3 groups of 8 a thread,
+// crates/saber-kernels/hip/attn_glue_hadi8.hip:33); heads of `hd` elements, a multiple of 8.
+int saber_iu8_attn_gate_quant_had(saber_iu8_ctx *ctx, const void *core, const void *gate, void *q, float *scale, uint32_t m,
+                                  uint32_t n, uint32_t head_dim, uint32_t gate_stride, const float *had_t, void *stream) {
+  if (m == 0 || n == 0) return fail(SABER_IU8_E_RULE, fmt("attn_gate_quant_had_i8: %u rows of %u has nothing to do", m, n));
+  if (n % 64 != 0 || n > 6144)
+    return fail(SABER_IU8_E_RULE, fmt("attn_gate_quant_had_i8: row width %u must be a multiple of 64, at most 6144", n));
+  if (head_dim == 0 || head_dim % 8 != 0 || n % head_dim != 0)
+    return fail(SABER_IU8_E_RULE, fmt("attn_gate_quant_had_i8: head width %u must be a multiple of 8 dividing %u", head_dim, n));
+  if (gate_stride < 2 * n || gate_stride % 8 != 0)
+    return fail(SABER_IU8_E_RULE, fmt("attn_gate_quant_had_i8: gate stride %u must cover the [q | gate] block of %u in whole 16-byte pieces", gate_stride, 2 * n));
+  saber_iu8_desc d;
+  const uint32_t grid[3] = {m, 1, 1};
+  if (int rc = saber_iu8_describe_raw("attn_gate_quant_hadi8_t256_tiled1", "attn_glue_hadi8", grid, 256, &d)) return rc;
+  snprintf(d.op, sizeof d.op, "attn_gate_quant_had_i8");
+  set_i32(&d, "n", n);
+  set_i32(&d, "hd", head_dim);
+  set_i32(&d, "gs", gate_stride);
+  const saber_iu8_binding b[] = {{"core", (void *)core}, {"gate", (void *)gate}, {"q", q}, {"scale", scale}, {"had_t", (void *)had_t}};
+  return saber_iu8_launch(ctx, &d, b, 5, stream);
 }
 
 // ---------------------------------------------------------------------------- routed experts

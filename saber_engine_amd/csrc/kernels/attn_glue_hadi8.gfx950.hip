@@ -1,0 +1,48 @@
+// The attention output gate's Hadamard-basis int8 producer for gfx950: the code object
+// `attn_glue_hadi8`, standing in for the reference's object of the same name
+// (crates/saber-kernels/hip/attn_glue_hadi8.hip, symbol crates/saber-kernels/src/macaq_iu8.rs:870)
+// with the same kernel symbol and kernarg layout (`had_t` last).
+//
+//   attn_gate_quant_hadi8_t256_tiled1   v = bf16(core * bf16(sigmoid(gate))), the o_proj's A producer.
+//       core bf16 [rows, n]; gate is the projection's [q | gate] block, row stride `gs`, head stride
+//       2*hd, the gate half at +hd (crates/saber-kernels/src/abi.rs:2683-2694); n <= 6144.
+//   attn_glue_hadi8_sigmoid_bf16_table  a checker's tap: bf16(sigmoid) of all 65,536 bf16 inputs
+//
+// Then u = v * t, x = H32 u per 32-block, x * (1/sqrt(32)), and the per-token int8 law on x; codes
+// in the gfx950 A fragment order. sigmoid = 1 / (1 + expf(-g)) is rounded to bf16 before use, so the
+// device's expf shows only through a bf16 -> bf16 function, which the tap kernel tables.
+#include "iu8_had.h"
+
+static __device__ __forceinline__ float glue_sigmoid_bf16(float g) {
+#pragma clang fp contract(off)
+  return iu8_bf16_f32((unsigned short)iu8_bf16_bits(1.f / (1.f + expf(-g))));
+}
+
+extern "C" __global__ __launch_bounds__(256) void attn_gate_quant_hadi8_t256_tiled1(
+    const unsigned short *__restrict__ core, const unsigned short *__restrict__ gate, unsigned char *__restrict__ q,
+    float *__restrict__ scale, int n, int hd, int gs, const float *__restrict__ had_t) {
+#pragma clang fp contract(off)
+  constexpr int T = 256;
+  const int row = had_row(), tid = threadIdx.x, NV = n >> 3;
+  core += (size_t)row * n, gate += (size_t)row * gs;
+  float sv[HAD_MAXG][8];
+#pragma unroll
+  for (int i = 0; i < HAD_MAXG; ++i) {
+    const int g = tid + i * T;
+    if (g >= NV) continue;
+    const int e = g << 3, h = e / hd, o = e - h * hd;
+    float vc[8], vg[8];
+    had_load8(core + e, vc);
+    had_load8(gate + (size_t)h * 2 * hd + hd + o, vg);
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      sv[i][j] = iu8_bf16_f32((unsigned short)iu8_bf16_bits(vc[j] * glue_sigmoid_bf16(vg[j])));
+    had32(sv[i], had_t + 8 * g, tid);
+  }
+  had_tail<T>(sv, NV, q, scale, row, n);
+}
+
+extern "C" __global__ __launch_bounds__(256) void attn_glue_hadi8_sigmoid_bf16_table(unsigned short *__restrict__ out) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  out[i] = (unsigned short)iu8_bf16_bits(glue_sigmoid_bf16(iu8_bf16_f32((unsigned short)i)));
+}

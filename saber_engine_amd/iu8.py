@@ -19,7 +19,7 @@ LIB_PATH = os.path.join(PKG, "libsaber_iu8.so")
 PREBUILT = os.path.join(ROOT, "prebuilt", "gfx950")
 
 W4, W8 = 0, 1
-ARG_BUFFER, ARG_NULL_BUFFER, ARG_I32, ARG_F32 = 0, 1, 2, 3
+ARG_BUFFER, ARG_NULL_BUFFER, ARG_I32, ARG_F32, ARG_I64 = 0, 1, 2, 3, 4
 WS_SCRATCH, WS_PERSISTENT = 0, 1
 E_RULE, E_PARSE, E_VALIDATE, E_HIP, E_ARG, E_IO, E_NOTLOADED = -1, -2, -3, -4, -5, -6, -7
 REFUSED_KERNARG, REFUSED_WAVE, REFUSED_METADATA = 1, 2, 3
@@ -112,6 +112,9 @@ def lib():
         L.saber_iu8_quant_had.argtypes = [C.c_void_p] * 4 + [C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p]
         L.saber_iu8_silu_mul_quant_had.argtypes = [C.c_void_p] * 4 + [C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p]
         L.saber_iu8_add_rms_quant_had.argtypes = [C.c_void_p] * 7 + [C.c_uint32, C.c_uint32, C.c_float, C.c_void_p, C.c_void_p]
+        L.saber_iu8_gdn_norm_quant_had.argtypes = [C.c_void_p] * 3 + [C.c_int64] + [C.c_void_p] * 3 + [
+            C.c_uint32, C.c_uint32, C.c_float, C.c_void_p, C.c_void_p]
+        L.saber_iu8_attn_gate_quant_had.argtypes = [C.c_void_p] * 5 + [C.c_uint32] * 4 + [C.c_void_p, C.c_void_p]
         L.saber_iu8_get_counters.argtypes = [C.c_void_p, C.POINTER(Counters)]
         L.saber_iu8_has_kernel.argtypes = [C.c_void_p, C.c_char_p]
         for fn in ("saber_iu8_moe_rows_cap", "saber_iu8_moe_tile_blocks"):
@@ -302,6 +305,12 @@ class Context:
 
     def add_rms_quant_had(self, y, res, w, q, scale, res_out, m, k, eps, had_t, stream=0):
         _check(lib().saber_iu8_add_rms_quant_had(self._h, y, res, w, q, scale, res_out, m, k, eps, had_t, stream))
+
+    def gdn_norm_quant_had(self, x, z, z_stride, w, q, scale, m, n, eps, had_t, stream=0):
+        _check(lib().saber_iu8_gdn_norm_quant_had(self._h, x, z, z_stride, w, q, scale, m, n, eps, had_t, stream))
+
+    def attn_gate_quant_had(self, core, gate, q, scale, m, n, head_dim, gate_stride, had_t, stream=0):
+        _check(lib().saber_iu8_attn_gate_quant_had(self._h, core, gate, q, scale, m, n, head_dim, gate_stride, had_t, stream))
 
     def gemm_acc(self, wkind, a, w, acc, m, n, k, stream=0):
         _check(lib().saber_iu8_gemm_acc(self._h, wkind, a, w, acc, m, n, k, stream))

@@ -1,4 +1,4 @@
-"""GPU parity of the Hadamard-basis int8 producers (code object `mxfp4_hadi8`), through the C ABI,
+"""GPU parity of the Hadamard-basis int8 producers (code objects `mxfp4_hadi8`, `attn_glue_hadi8`), through the C ABI,
 against the CPU oracle: codes, scales and the residual output, bit for bit."""
 import numpy as np
 import pytest
@@ -66,6 +66,77 @@ def test_add_rms_quant_had(ctx, M, K):
     np.testing.assert_array_equal(iu8.unpack_a(q.cpu().numpy(), M, K), wq)
 
 
+def tap(ctx, kernel, plugin, dtype):
+    """A checker's tap kernel: one value for each of the 65,536 bf16 inputs."""
+    out = torch.zeros(65536, dtype=dtype, device="cuda")
+    ctx.launch(iu8.describe_raw(kernel, (256, 1, 1), 256, plugin=plugin), dict(out=out.data_ptr()))
+    torch.cuda.synchronize()
+    return out.cpu().numpy()
+
+
+def test_device_sigmoid_equals_host_formula_on_all_65536_inputs(ctx):
+    say("sigmoid table, all bf16 inputs")
+    got = tap(ctx, "attn_glue_hadi8_sigmoid_bf16_table", "attn_glue_hadi8", torch.int16).view(np.uint16)
+    want = ref.sigmoid_bf16_table()
+    fin = np.isfinite(synth.bf16_bits_to_f32(np.arange(65536, dtype=np.uint16)))
+    bad = np.flatnonzero(fin & (got != want))
+    assert bad.size == 0, [(hex(i), hex(got[i]), hex(want[i])) for i in bad[:8]]
+
+
+def device_silu_f32_table(ctx):
+    return tap(ctx, "mxfp4_hadi8_silu_f32_table", "mxfp4_hadi8", torch.float32)
+
+
+def test_device_silu_f32_is_within_an_ulp_of_the_host_formula(ctx):
+    """The f32 gate of gdn_norm carries the device's expf: held against the host's libm value to
+    2 units in the last place over every finite bf16 input (and reported: how many differ)."""
+    say("silu f32 table, all bf16 inputs")
+    got, want = device_silu_f32_table(ctx), ref.silu_f32_table()
+    x = synth.bf16_bits_to_f32(np.arange(65536, dtype=np.uint16))
+    fin = np.isfinite(x) & np.isfinite(want)
+    gi, wi = got.view(np.int32).astype(np.int64), want.view(np.int32).astype(np.int64)
+    d = np.abs(gi - wi)[fin]
+    say(f"silu f32: {int((d != 0).sum())} of {int(fin.sum())} inputs differ from libm, max {int(d.max())} ulp")
+    assert d.max() <= 2
+
+
+@pytest.mark.parametrize("M,H,zs_pad", [(1, 1, 0), (7, 48, 64), (130, 16, 0), (3, 80, 8)])
+def test_gdn_norm_quant_had(ctx, M, H, zs_pad):
+    N = H * 128
+    say(f"gdn_norm_quant_had M={M} N={N} z stride {N + zs_pad}")
+    rng = np.random.default_rng(M + N)
+    x = synth.f32_to_bf16_bits((rng.standard_normal((M, N)) * 2).astype(np.float32))
+    zfull = synth.f32_to_bf16_bits((rng.standard_normal((M, N + zs_pad)) * 3).astype(np.float32))
+    w = synth.f32_to_bf16_bits((1 + rng.standard_normal(128) * 0.1).astype(np.float32))
+    t = rng.choice([-1.0, 1.0], size=N).astype(np.float32)
+    q, s = outs(M, N)
+    xd, zd, wd, td = dev_bf16_bits(x), dev_bf16_bits(zfull), dev_bf16_bits(w), dev_f32(t)
+    ctx.gdn_norm_quant_had(xd.data_ptr(), zd.data_ptr(), N + zs_pad, wd.data_ptr(), q.data_ptr(), s.data_ptr(), M, N, 1e-6,
+                           td.data_ptr())
+    torch.cuda.synchronize()
+    # the gate's f32 values are the card's own (its expf), tabled by the tap kernel
+    wq, wsc = ref.gdn_norm_quant_had(x, zfull[:, :N], w, t, 1e-6, silu_tab=device_silu_f32_table(ctx))
+    np.testing.assert_array_equal(s.cpu().numpy().view(np.uint32), wsc.view(np.uint32))
+    np.testing.assert_array_equal(iu8.unpack_a(q.cpu().numpy(), M, N), wq)
+
+
+@pytest.mark.parametrize("M,H,hd,pad", [(1, 1, 64, 0), (9, 24, 256, 0), (140, 16, 128, 96), (2, 48, 128, 0)])
+def test_attn_gate_quant_had(ctx, M, H, hd, pad):
+    n = H * hd
+    say(f"attn_gate_quant_had M={M} n={n} hd={hd} gate stride {2 * n + pad}")
+    rng = np.random.default_rng(M + n + hd)
+    core = synth.f32_to_bf16_bits(rng.standard_normal((M, n)).astype(np.float32))
+    block = synth.f32_to_bf16_bits((rng.standard_normal((M, 2 * n + pad)) * 3).astype(np.float32))
+    t = rng.choice([-1.0, 1.0], size=n).astype(np.float32)
+    q, s = outs(M, n)
+    cd, gd, td = dev_bf16_bits(core), dev_bf16_bits(block), dev_f32(t)
+    ctx.attn_gate_quant_had(cd.data_ptr(), gd.data_ptr(), q.data_ptr(), s.data_ptr(), M, n, hd, 2 * n + pad, td.data_ptr())
+    torch.cuda.synchronize()
+    wq, wsc = ref.attn_gate_quant_had(core, block, t, hd)
+    np.testing.assert_array_equal(s.cpu().numpy().view(np.uint32), wsc.view(np.uint32))
+    np.testing.assert_array_equal(iu8.unpack_a(q.cpu().numpy(), M, n), wq)
+
+
 def test_had_producers_feed_the_gemm(ctx):
     """The transformed codes are ordinary A operands: producer + GEMM equals the oracle's GEMM on them."""
     say("quant_had -> gemm")
@@ -89,4 +160,17 @@ def test_had_refusals(ctx):
     for (m, k) in [(0, 64), (1, 96), (1, 20544)]:       # nothing to do, not whole fragments, too wide
         with pytest.raises(iu8.IU8Error) as e:
             ctx.quant_had(q.data_ptr(), q.data_ptr(), s.data_ptr(), m, k, s.data_ptr())
+        assert e.value.code == iu8.E_RULE
+    p = q.data_ptr()
+    for args in [(p, p, 128, p, p, s.data_ptr(), 1, 192, 1e-6, p),          # not whole heads
+                 (p, p, 64, p, p, s.data_ptr(), 1, 128, 1e-6, p),           # z stride under the row
+                 (p, p, 10368, p, p, s.data_ptr(), 1, 10368, 1e-6, p)]:     # too wide
+        with pytest.raises(iu8.IU8Error) as e:
+            ctx.gdn_norm_quant_had(*args)
+        assert e.value.code == iu8.E_RULE
+    for args in [(p, p, p, s.data_ptr(), 1, 6208, 64, 12416, p),            # past the t256 form
+                 (p, p, p, s.data_ptr(), 1, 256, 96, 512, p),               # heads do not divide the row
+                 (p, p, p, s.data_ptr(), 1, 256, 64, 256, p)]:              # stride under the [q | gate] block
+        with pytest.raises(iu8.IU8Error) as e:
+            ctx.attn_gate_quant_had(*args)
         assert e.value.code == iu8.E_RULE

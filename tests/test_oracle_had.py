@@ -119,3 +119,87 @@ def test_add_rms_quant_had_against_float64(threads):
     # never by more
     q2, s2, _ = ref.add_rms_quant_had(y, r, w, t, eps, 768 - threads)
     np.testing.assert_allclose(s, s2, rtol=1e-6)
+
+
+def _bf16(x):
+    return synth.bf16_bits_to_f32(synth.f32_to_bf16_bits(np.asarray(x, np.float32)))
+
+
+def test_sigmoid_and_silu_tables_against_float64():
+    bits = np.arange(65536, dtype=np.uint16)
+    g = synth.bf16_bits_to_f32(bits).astype(np.float64)
+    ok = np.isfinite(g)
+    sig = synth.bf16_bits_to_f32(ref.sigmoid_bf16_table()).astype(np.float64)
+    with np.errstate(over="ignore"):
+        want = 1 / (1 + np.exp(-g[ok]))
+    assert np.abs(sig[ok] - want).max() <= 2.0 ** -9            # one bf16 rounding of a value in [0, 1]
+    assert (np.diff(sig[:0x7F80]) >= 0).all()                   # monotone over the non-negative inputs
+    assert sig[0] == 0.5 and sig[0x7F80] == 1.0 and sig[0xFF80] == 0.0
+    silu = ref.silu_f32_table().astype(np.float64)
+    with np.errstate(over="ignore", invalid="ignore"):
+        want = g[ok] / (1 + np.exp(-g[ok]))
+    fin = np.isfinite(want) & (g[ok] > -88)                     # below, expf(-z) overflows f32 and the law gives -0
+    err = np.abs(silu[ok][fin] - want[fin])
+    assert (err <= np.maximum(np.abs(want[fin]) * 2.0 ** -22, 1e-44)).all()   # f32 roundings of exp, add, divide
+    assert (silu[ok][g[ok] < -89] == 0).all()
+
+
+def test_attn_gate_quant_had_composes_the_pinned_pieces():
+    rng = np.random.default_rng(6)
+    M, H, hd = 3, 4, 64
+    n = H * hd
+    core = synth.f32_to_bf16_bits(rng.standard_normal((M, n)).astype(np.float32))
+    block = synth.f32_to_bf16_bits((rng.standard_normal((M, 2 * n + 32)) * 3).astype(np.float32))   # a padded row stride
+    t = rng.choice([-1.0, 1.0], size=n).astype(np.float32)
+    q, s = ref.attn_gate_quant_had(core, block, t, hd)
+    gate = block[:, :2 * n].reshape(M, H, 2, hd)[:, :, 1, :].reshape(M, n)      # head h: [q(hd) | gate(hd)]
+    sig = synth.bf16_bits_to_f32(ref.sigmoid_bf16_table()[gate])
+    p = _bf16(synth.bf16_bits_to_f32(core) * sig)
+    x = ref.had32_rows(p, t)
+    for m in range(M):
+        qq, ss = ref.quant_row_f32(x[m])
+        np.testing.assert_array_equal(q[m], qq)
+        assert s[m] == ss
+    # taking the q half of the block instead gives another result
+    wrong = synth.bf16_bits_to_f32(ref.sigmoid_bf16_table()[block[:, :2 * n].reshape(M, H, 2, hd)[:, :, 0, :].reshape(M, n)])
+    assert (ref.quant_row_f32(ref.had32_rows(_bf16(synth.bf16_bits_to_f32(core) * wrong), t)[0])[0] != q[0]).any()
+
+
+def test_gdn_norm_quant_had_against_a_numpy_float32_restatement():
+    rng = np.random.default_rng(7)
+    M, H, eps = 4, 3, 1e-6
+    N = H * 128
+    xb = synth.f32_to_bf16_bits((rng.standard_normal((M, N)) * 2).astype(np.float32))
+    zb = synth.f32_to_bf16_bits((rng.standard_normal((M, N)) * 2).astype(np.float32))
+    wb = synth.f32_to_bf16_bits((1 + rng.standard_normal(128) * 0.1).astype(np.float32))
+    t = rng.choice([-1.0, 1.0], size=N).astype(np.float32)
+    q, s = ref.gdn_norm_quant_had(xb, zb, wb, t, eps)
+    x = synth.bf16_bits_to_f32(xb).reshape(M, H, 16, 8)
+    f64 = np.float64
+
+    def fma(a, b, c):       # products of two f32 are exact in f64; the one f64 rounding before the f32
+        return (a.astype(f64) * b.astype(f64) + c.astype(f64)).astype(np.float32)    # one is harmless here
+    ssq = x[..., 1] * x[..., 1]
+    ssq = fma(x[..., 0], x[..., 0], ssq)
+    for j in range(2, 8):
+        ssq = fma(x[..., j], x[..., j], ssq)
+    lanes = np.arange(16)
+    for o in (8, 4, 2, 1):
+        ssq = ssq + ssq[..., lanes ^ o]
+    assert (ssq == ssq[..., :1]).all()                                # every lane holds the same bits
+    inv = np.float32(1) / np.sqrt(ssq[..., 0] * np.float32(1 / 128) + np.float32(eps))       # [M, H]
+    sg = ref.silu_f32_table()[zb].reshape(M, H, 128)
+    w = synth.bf16_bits_to_f32(wb)
+    pre = _bf16(((x.reshape(M, H, 128) * inv[..., None]) * w) * sg).reshape(M, N)
+    xt = ref.had32_rows(pre, t)
+    for m in range(M):
+        qq, ss = ref.quant_row_f32(xt[m])
+        np.testing.assert_array_equal(q[m], qq)
+        assert s[m] == ss
+    # and the mathematics: per-head RMS norm times the weight times silu(z), in float64
+    x64, z64 = x.reshape(M, H, 128).astype(f64), synth.bf16_bits_to_f32(zb).reshape(M, H, 128).astype(f64)
+    want = x64 / np.sqrt((x64 ** 2).mean(-1, keepdims=True) + eps) * w * (z64 / (1 + np.exp(-z64)))
+    np.testing.assert_allclose(pre.reshape(M, H, 128), want, rtol=2.0 ** -7, atol=1e-6)
+    # a table handed in replaces the host's libm
+    q2, s2 = ref.gdn_norm_quant_had(xb, zb, wb, t, eps, silu_tab=np.zeros(65536, np.float32))
+    assert not q2.any() and (s2 == np.float32(1e-30)).all()
