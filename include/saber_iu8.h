@@ -238,6 +238,17 @@ int saber_iu8_attn_gate_quant_had(saber_iu8_ctx *ctx, const void *core_bf16, con
                                   uint32_t m, uint32_t n, uint32_t head_dim, uint32_t gate_stride, const float *had_t,
                                   void *stream);
 
+/* macaq_iu8::pair(first, second) (crates/saber-kernels/src/macaq_iu8.rs:632-704): two W4 decode
+ * GEMMs that read one A operand, one dispatch of the fused object's `macaq_iu8f_pair_w4_tm*`
+ * (kernarg list abi.rs:3411-3432). Each half is the descriptor saber_iu8_resolve / _describe gave
+ * it alone; the grids go end to end, the second half's buffers and workspaces take the suffix `_b`.
+ * Refused (SABER_IU8_E_RULE) unless both halves are W4 decode cells of one kernel, M and K. */
+int saber_iu8_pair(const saber_iu8_desc *first, const saber_iu8_desc *second, saber_iu8_desc *out);
+/* resolve x 2 + pair + launch for the unsplit decode law: c [m,n] and c_b [m,n_b] from one a / a_scale. */
+int saber_iu8_gemm_pair(saber_iu8_ctx *ctx, const void *a, const float *a_scale, const void *w, const float *w_scale, void *c,
+                        uint32_t n, const void *w_b, const float *w_scale_b, void *c_b, uint32_t n_b, uint32_t m, uint32_t k,
+                        void *stream);
+
 /* The whole decode linear in one launch where the shape allows (at most 4 rows whose codes fit the
  * kernel's 20 KiB staging area; saber_iu8_fused_holds): per-token quantisation fused into the
  * GEMV's activation staging. x bf16 [m,k]; q (A edge) and scale f32 [m] are optional outputs (NULL:

@@ -12,6 +12,14 @@ static const Signature SIG_DEC = {{"a", K::Buffer},  {"w", K::Buffer},
 static const Signature SIG_DECQ = {{"x", K::Buffer},     {"w", K::Buffer}, {"ws", K::Buffer}, {"q", K::Buffer},
                                    {"scale", K::Buffer}, {"c", K::Buffer}, {"m", K::I32},     {"n", K::I32},
                                    {"k", K::I32}};
+// the decode pair (crates/saber-kernels/src/abi.rs:3411-3432)
+static const Signature SIG_PAIR = {{"a", K::Buffer},  {"as", K::Buffer}, {"w", K::Buffer},  {"ws", K::Buffer},
+                                   {"decode_partial", K::Buffer},   {"decode_counter", K::Buffer},
+                                   {"c", K::Buffer},  {"w_b", K::Buffer}, {"ws_b", K::Buffer},
+                                   {"decode_partial_b", K::Buffer}, {"decode_counter_b", K::Buffer},
+                                   {"c_b", K::Buffer}, {"m", K::I32},    {"k", K::I32},     {"n", K::I32},
+                                   {"ks", K::I32},    {"nb", K::I32},    {"n_b", K::I32},   {"ks_b", K::I32},
+                                   {"nb_b", K::I32}};
 static const Signature SIG_PF = {{"a", K::Buffer}, {"w", K::Buffer}, {"as", K::Buffer}, {"ws", K::Buffer},
                                  {"c", K::Buffer}, {"m", K::I32},    {"n", K::I32},     {"k", K::I32}};
 static const Signature SIG_QUANT = {{"x", K::Buffer}, {"q", K::Buffer}, {"scale", K::Buffer}, {"k", K::I32}};
@@ -21,12 +29,12 @@ static const Signature SIG_QUANT_ROWS = {{"x", K::Buffer}, {"q", K::Buffer},    
 // (prebuilt/gfx1201/mxfp4_hadi8.manifest.toml: 64 and 40 bytes)
 static const Signature SIG_HAD_ARQ = {{"y", K::Buffer},     {"res", K::Buffer},     {"w", K::Buffer},
                                       {"q", K::Buffer},     {"scale", K::Buffer},   {"res_out", K::Buffer},
-                                      {"K", K::I32},        {"eps", K::F32},        {"had_t", K::Buffer}};
-static const Signature SIG_HAD_SMQ = {{"gu", K::Buffer}, {"q", K::Buffer}, {"scale", K::Buffer}, {"N", K::I32}, {"had_t", K::Buffer}};
+                                      {"k", K::I32},        {"eps", K::F32},        {"had_t", K::Buffer}};
+static const Signature SIG_HAD_SMQ = {{"gu", K::Buffer}, {"q", K::Buffer}, {"scale", K::Buffer}, {"n", K::I32}, {"had_t", K::Buffer}};
 static const Signature SIG_HAD_Q = {{"x", K::Buffer}, {"q", K::Buffer}, {"scale", K::Buffer}, {"k", K::I32}, {"had_t", K::Buffer}};
 // crates/saber-kernels/src/abi.rs:652-662 and :2683-2694, `had_t` appended last
 static const Signature SIG_HAD_GNQ = {{"x", K::Buffer}, {"z", K::Buffer},     {"zs", K::I64}, {"w", K::Buffer},
-                                      {"q", K::Buffer}, {"scale", K::Buffer}, {"N", K::I32},  {"eps", K::F32},
+                                      {"q", K::Buffer}, {"scale", K::Buffer}, {"n", K::I32},  {"eps", K::F32},
                                       {"had_t", K::Buffer}};
 static const Signature SIG_HAD_AGQ = {{"core", K::Buffer}, {"gate", K::Buffer}, {"q", K::Buffer}, {"scale", K::Buffer},
                                       {"n", K::I32},       {"hd", K::I32},      {"gs", K::I32},   {"had_t", K::Buffer}};
@@ -59,6 +67,7 @@ const Signature *signature_for(const std::string &k) {
   if (starts(k, "macaq_iu8_dec_")) return &SIG_DEC;
   if (starts(k, "macaq_iu8_decq_")) return &SIG_DECQ;
   if (starts(k, "macaq_iu8_pf_")) return &SIG_PF;
+  if (starts(k, "macaq_iu8f_pair_")) return &SIG_PAIR;
   if (starts(k, "add_rms_quant_hadi8_")) return &SIG_HAD_ARQ;
   if (starts(k, "silu_mul_quant_hadi8_")) return &SIG_HAD_SMQ;
   if (starts(k, "quant_hadi8_")) return &SIG_HAD_Q;

@@ -11,20 +11,38 @@ namespace iu8 {
 static const DecVariant DEC_VARIANTS[] = {
 #define IU8_DEC_VARIANT(name, TM, W8, NT, KW, WPB, D, ALDS, ACC) {#name, TM, W8, NT, KW, WPB, D, ALDS, ACC},
 #define IU8_PF_VARIANT(name, W8, WMW, WNW, TM, TN, ACC, ST, OCC)
+#define IU8_PAIR_VARIANT(name, TM, NT, KW, WPB, D, ALDS)
 #include "../kernels/iu8_variants.def"
 #undef IU8_DEC_VARIANT
 #undef IU8_PF_VARIANT
+#undef IU8_PAIR_VARIANT
 };
 static const PfVariant PF_VARIANTS[] = {
 #define IU8_DEC_VARIANT(name, TM, W8, NT, KW, WPB, D, ALDS, ACC)
 #define IU8_PF_VARIANT(name, W8, WMW, WNW, TM, TN, ACC, ST, OCC) {#name, W8, WMW, WNW, TM, TN, ACC, OCC},
+#define IU8_PAIR_VARIANT(name, TM, NT, KW, WPB, D, ALDS)
 #include "../kernels/iu8_variants.def"
 #undef IU8_DEC_VARIANT
 #undef IU8_PF_VARIANT
+#undef IU8_PAIR_VARIANT
+};
+static const DecVariant PAIR_VARIANTS[] = {
+#define IU8_DEC_VARIANT(name, TM, W8, NT, KW, WPB, D, ALDS, ACC)
+#define IU8_PF_VARIANT(name, W8, WMW, WNW, TM, TN, ACC, ST, OCC)
+#define IU8_PAIR_VARIANT(name, TM, NT, KW, WPB, D, ALDS) {#name, TM, false, NT, KW, WPB, D, ALDS, false},
+#include "../kernels/iu8_variants.def"
+#undef IU8_DEC_VARIANT
+#undef IU8_PF_VARIANT
+#undef IU8_PAIR_VARIANT
 };
 
 const DecVariant *dec_variant(const std::string &name) {
   for (const DecVariant &v : DEC_VARIANTS)
+    if (name == v.name) return &v;
+  return nullptr;
+}
+const DecVariant *pair_variant(const std::string &name) {
+  for (const DecVariant &v : PAIR_VARIANTS)
     if (name == v.name) return &v;
   return nullptr;
 }
@@ -156,6 +174,61 @@ int describe(const std::string &kernel, uint32_t m, uint32_t n, uint32_t k, uint
     return describe_pf(*v, m, n, k, out);
   }
   return fail(SABER_IU8_E_RULE, kernel + ": not a kernel of the macaq_iu8 object");
+}
+
+static bool int_arg(const saber_iu8_desc &d, const char *name, int64_t *v) {
+  for (uint32_t i = 0; i < d.n_args; ++i)
+    if (!strcmp(d.args[i].name, name) && (d.args[i].kind == SABER_IU8_ARG_I32 || d.args[i].kind == SABER_IU8_ARG_I64)) {
+      *v = d.args[i].ival;
+      return true;
+    }
+  return false;
+}
+
+// The decode pair: each half is exactly the descriptor `resolve` / `describe` gave it alone (its
+// split count, its partial slab and counters), the two grids end to end, problem 0 first
+// (macaq_iu8.rs:632-704). Refused unless both halves are W4 decode cells of one kernel (so one row
+// tiling and one staging form), M and K.
+int pair(const saber_iu8_desc &first, const saber_iu8_desc &second, saber_iu8_desc *out) {
+  static const char PREFIX[] = "macaq_iu8_dec_w4_";
+  const std::string k0 = first.kernel, k1 = second.kernel;
+  const DecVariant *v0 = dec_variant(k0), *v1 = dec_variant(k1);
+  int64_t m0 = 0, kk0 = 0, n0 = 0, m1 = 0, kk1 = 0, n1 = 0;
+  const bool ints = int_arg(first, "m", &m0) && int_arg(first, "k", &kk0) && int_arg(first, "n", &n0) &&
+                    int_arg(second, "m", &m1) && int_arg(second, "k", &kk1) && int_arg(second, "n", &n1);
+  if (!v0 || !v1 || !ints || v0->w8 || v1->w8 || v0->acc || v1->acc || k0 != k1 || m0 != m1 || kk0 != kk1)
+    return fail(SABER_IU8_E_RULE, fmt("macaq iu8 pair: halves `%s` M %lld K %lld and `%s` M %lld K %lld are not two W4 cells of one M, K",
+                                      k0.c_str(), (long long)m0, (long long)kk0, k1.c_str(), (long long)m1, (long long)kk1));
+  const std::string name = "macaq_iu8f_pair_w4_" + k0.substr(sizeof PREFIX - 1);
+  const DecVariant *pv = pair_variant(name);
+  if (!pv) return fail(SABER_IU8_E_RULE, name + ": the fused object carries no such pair");
+  const uint32_t nb0 = first.grid[0], nb1 = second.grid[0], ks0 = first.ks, ks1 = second.ks;
+  memset(out, 0, sizeof *out);
+  copy_name(out->op, sizeof out->op, "gemm_i4a8_pair");
+  copy_name(out->plugin, sizeof out->plugin, "macaq_iu8f");
+  copy_name(out->kernel, sizeof out->kernel, name);
+  out->grid[0] = nb0 * ks0 + nb1 * ks1, out->grid[1] = 1, out->grid[2] = 1;
+  out->block[0] = pv->threads(), out->block[1] = 1, out->block[2] = 1;
+  out->n_launches = 1;
+  out->ks = 1;
+  if (int rc = fill_slots(name, out)) return rc;
+  set_i32(out, "m", m0), set_i32(out, "k", kk0);
+  set_i32(out, "n", n0), set_i32(out, "ks", ks0), set_i32(out, "nb", nb0);
+  set_i32(out, "n_b", n1), set_i32(out, "ks_b", ks1), set_i32(out, "nb_b", nb1);
+  const saber_iu8_desc *half[2] = {&first, &second};
+  for (int h = 0; h < 2; ++h) {
+    const char *sfx = h ? "_b" : "";
+    const std::string p = std::string("decode_partial") + sfx, c = std::string("decode_counter") + sfx;
+    if (half[h]->ks == 1) {
+      set_null(out, p.c_str()), set_null(out, c.c_str());
+    } else {
+      for (uint32_t i = 0; i < half[h]->n_workspaces; ++i) {
+        const saber_iu8_workspace &w = half[h]->workspaces[i];
+        add_ws(out, (std::string(w.name) + sfx).c_str(), w.kind, w.bytes, w.zero_once);
+      }
+    }
+  }
+  return 0;
 }
 
 int resolve(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *out) {

@@ -37,6 +37,9 @@ uint32_t decode_split(uint32_t m, uint32_t n, uint32_t k, uint32_t nblk, uint32_
 
 int resolve(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *out);
 int describe(const std::string &kernel, uint32_t m, uint32_t n, uint32_t k, uint32_t ks, saber_iu8_desc *out);
+// Two W4 decode descriptors of one M, K and kernel -> the one-dispatch pair (macaq_iu8.rs:632-704).
+int pair(const saber_iu8_desc &first, const saber_iu8_desc &second, saber_iu8_desc *out);
+const DecVariant *pair_variant(const std::string &name);
 int resolve_quant(uint32_t m, uint32_t k, saber_iu8_desc *out);
 // The fused quant + GEMV of a decode linear; refuses (by name) shapes it does not hold.
 bool fused_holds(uint32_t m, uint32_t k);

@@ -84,6 +84,10 @@ int saber_iu8_resolve_quant(uint32_t m, uint32_t k, saber_iu8_desc *out) {
   if (!out) return fail(SABER_IU8_E_ARG, "resolve_quant: null descriptor");
   return resolve_quant(m, k, out);
 }
+int saber_iu8_pair(const saber_iu8_desc *first, const saber_iu8_desc *second, saber_iu8_desc *out) {
+  if (!first || !second || !out) return fail(SABER_IU8_E_ARG, "pair: null descriptor");
+  return pair(*first, *second, out);
+}
 int saber_iu8_fused_holds(uint32_t m, uint32_t k) { return fused_holds(m, k) ? 1 : 0; }
 int saber_iu8_resolve_fused(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *out) {
   if (!out) return fail(SABER_IU8_E_ARG, "resolve_fused: null descriptor");
@@ -361,6 +365,20 @@ int saber_iu8_gemm(saber_iu8_ctx *ctx, int wkind, const void *a, const float *as
   return launch_gemm(ctx, d, a, as, w, ws, c, partial, counter, stream);
 }
 
+// Two W4 linears on one activation operand in one dispatch (decode band; the launch law's own
+// descriptors, which do not split K, so no workspace is bound).
+int saber_iu8_gemm_pair(saber_iu8_ctx *ctx, const void *a, const float *as, const void *w, const float *ws, void *c, uint32_t n,
+                        const void *w_b, const float *ws_b, void *c_b, uint32_t n_b, uint32_t m, uint32_t k, void *stream) {
+  saber_iu8_desc d0, d1, d;
+  if (int rc = resolve(SABER_IU8_W4, m, n, k, &d0)) return rc;
+  if (int rc = resolve(SABER_IU8_W4, m, n_b, k, &d1)) return rc;
+  if (int rc = pair(d0, d1, &d)) return rc;
+  if (d.n_workspaces) return fail(SABER_IU8_E_RULE, "gemm_pair: a half splits K; bind its workspaces through saber_iu8_pair + saber_iu8_launch");
+  const saber_iu8_binding b[] = {{"a", (void *)a},     {"as", (void *)as},     {"w", (void *)w}, {"ws", (void *)ws}, {"c", c},
+                                 {"w_b", (void *)w_b}, {"ws_b", (void *)ws_b}, {"c_b", c_b}};
+  return saber_iu8_launch(ctx, &d, b, 8, stream);
+}
+
 int saber_iu8_gemm_acc(saber_iu8_ctx *ctx, int wkind, const void *a, const void *w, int32_t *acc, uint32_t m, uint32_t n,
                        uint32_t k, void *stream) {
   if (wkind != SABER_IU8_W4 && wkind != SABER_IU8_W8) return fail(SABER_IU8_E_ARG, "unknown weight kind");
@@ -409,7 +427,7 @@ int saber_iu8_silu_mul_quant_had(saber_iu8_ctx *ctx, const void *gu, void *q, fl
                                  const float *had_t, void *stream) {
   saber_iu8_desc d;
   if (int rc = had_desc("silu_mul_quant_had_i8", "silu_mul_quant", m, n, &d)) return rc;
-  set_i32(&d, "N", n);
+  set_i32(&d, "n", n);
   const saber_iu8_binding b[] = {{"gu", (void *)gu}, {"q", q}, {"scale", scale}, {"had_t", (void *)had_t}};
   return saber_iu8_launch(ctx, &d, b, 4, stream);
 }
@@ -418,7 +436,7 @@ int saber_iu8_add_rms_quant_had(saber_iu8_ctx *ctx, const void *y, const void *r
                                 void *res_out, uint32_t m, uint32_t k, float eps, const float *had_t, void *stream) {
   saber_iu8_desc d;
   if (int rc = had_desc("add_rms_quant_had_i8", "add_rms_quant", m, k, &d)) return rc;
-  set_i32(&d, "K", k);
+  set_i32(&d, "k", k);
   set_f32(&d, "eps", eps);
   const saber_iu8_binding b[] = {{"y", (void *)y}, {"res", (void *)res}, {"w", (void *)w}, {"q", q},
                                  {"scale", scale}, {"res_out", res_out}, {"had_t", (void *)had_t}};
@@ -437,7 +455,7 @@ int saber_iu8_gdn_norm_quant_had(saber_iu8_ctx *ctx, const void *x, const void *
   const uint32_t grid[3] = {m, 1, 1};
   if (int rc = saber_iu8_describe_raw("gdn_norm_quant_hadi8_t256_tiled1", "mxfp4_hadi8", grid, 256, &d)) return rc;
   snprintf(d.op, sizeof d.op, "gdn_norm_quant_had_i8");
-  set_i32(&d, "N", n);
+  set_i32(&d, "n", n);
   set_i32(&d, "zs", z_stride);
   set_f32(&d, "eps", eps);
   const saber_iu8_binding b[] = {{"x", (void *)x}, {"z", (void *)z}, {"w", (void *)w}, {"q", q}, {"scale", scale}, {"had_t", (void *)had_t}};

@@ -22,6 +22,16 @@ static __device__ __forceinline__ int iu8_arow(const iu8_rows &R, int m) {
   return R.row0 + min(m, ((R.rows + 15) & ~15) - 1);
 }
 
+// Where a workgroup stands in a decode launch: its column block, its share of a grid-level split
+// of K and the number of shares. A plain launch reads them off the grid; a launch that lays
+// several problems' grids end to end hands each workgroup its own.
+struct iu8_blk {
+  int bx, z, Z;
+};
+static __device__ __forceinline__ iu8_blk iu8_blk_of_grid() {
+  return iu8_blk{(int)blockIdx.x, (int)blockIdx.z, (int)gridDim.z};
+}
+
 // ============================================================================ decode band
 // QF ("quant fused", M <= 4, dense rows, no grid split): `A` is the bf16 activation matrix [M, K]
 // itself. Every workgroup quantises the rows on its way into LDS (the per-token int8 law of
@@ -33,7 +43,7 @@ __device__ __forceinline__ void iu8_dec_body(const iu8_u8 *__restrict__ A, const
                                              const float *__restrict__ as, const float *__restrict__ ws,
                                              int *__restrict__ P, int *__restrict__ cnt, void *__restrict__ Cv,
                                              const iu8_rows R, int N, int K, iu8_u8 *__restrict__ qout = nullptr,
-                                             float *__restrict__ sout = nullptr) {
+                                             float *__restrict__ sout = nullptr, const iu8_blk B = iu8_blk_of_grid()) {
   const int M = R.rows;
   static_assert(!QF || (ALDS > 0 && TM == 1 && !ACC), "the fused form stages its rows in LDS");
   static_assert(WPB % KW == 0, "k-waves divide the workgroup");
@@ -54,10 +64,10 @@ __device__ __forceinline__ void iu8_dec_body(const iu8_u8 *__restrict__ A, const
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wk = wave % KW, wn = wave / KW;
   const int ntiles = N >> 4, steps = K >> 7, ktiles = K >> 6;
-  const int Z = gridDim.z, z = blockIdx.z;
+  const int Z = B.Z, z = B.z;
   const int spb = (steps + Z - 1) / Z;
   const int s_lo = z * spb, s_hi = min(steps, s_lo + spb);
-  const int nt0 = (blockIdx.x * WN + wn) * NT;
+  const int nt0 = (B.bx * WN + wn) * NT;
   const int ml = lane & 15, lg = lane >> 4;
   // this wave's steps: s_lo + wk + t*KW, t in [0, T)
   const int T = s_lo + wk < s_hi ? (s_hi - s_lo - wk + KW - 1) / KW : 0;
@@ -223,8 +233,8 @@ __device__ __forceinline__ void iu8_dec_body(const iu8_u8 *__restrict__ A, const
           for (int w = 1; w < WPB; ++w) a = fmaxf(a, s_amax[w][r]);
           qsc[r] = fmaxf(__fdiv_rn(a, 127.f), 1e-30f);
         }
-        const bool out0 = blockIdx.x == 0 && qout != nullptr;
-        if (blockIdx.x == 0 && sout != nullptr && tid < M)
+        const bool out0 = B.bx == 0 && qout != nullptr;
+        if (B.bx == 0 && sout != nullptr && tid < M)
           sout[tid] = tid == 0 ? qsc[0] : tid == 1 ? qsc[1] : tid == 2 ? qsc[2] : qsc[3];
 #pragma unroll
         for (int p = 0; p < X_PER; ++p) {
@@ -360,13 +370,13 @@ __device__ __forceinline__ void iu8_dec_body(const iu8_u8 *__restrict__ A, const
   __syncthreads();
   if (tid == 0) {
     __threadfence();
-    s_last = (atomicAdd(&cnt[blockIdx.x], 1) == Z - 1);
+    s_last = (atomicAdd(&cnt[B.bx], 1) == Z - 1);
   }
   __syncthreads();
   if (!s_last) return;
   __threadfence();
-  if (tid == 0) cnt[blockIdx.x] = 0;
-  const int nb = blockIdx.x * BN, nw4 = min(BN, N - nb) >> 2;
+  if (tid == 0) cnt[B.bx] = 0;
+  const int nb = B.bx * BN, nw4 = min(BN, N - nb) >> 2;
   for (int idx = tid; idx < nw4 * M; idx += NTHR) {
     const int m = idx / nw4, n = nb + (idx % nw4) * 4;
     iu8_v4i sum = iu8_v4i{0, 0, 0, 0};

@@ -36,9 +36,11 @@
   }
 #define IU8_DEC_VARIANT(name, TM, W8, NT, KW, WPB, D, ALDS, ACC) IU8_DEC(name, TM, W8, NT, KW, WPB, D, ALDS, ACC)
 #define IU8_PF_VARIANT(name, W8, WMW, WNW, TM, TN, ACC, ST, OCC)
+#define IU8_PAIR_VARIANT(name, TM, NT, KW, WPB, D, ALDS)
 #include "iu8_variants.def"
 #undef IU8_DEC_VARIANT
 #undef IU8_PF_VARIANT
+#undef IU8_PAIR_VARIANT
 #undef IU8_DEC
 
 // The decode linear with the per-token quantisation fused into the activation staging (M <= 4 rows
@@ -80,7 +82,9 @@ IU8_DECQ(macaq_iu8_decq_w8_tm1, true, 4)
   }
 #define IU8_DEC_VARIANT(name, TM, W8, NT, KW, WPB, D, ALDS, ACC)
 #define IU8_PF_VARIANT(name, W8, WMW, WNW, TM, TN, ACC, ST, OCC) IU8_PF32(name, W8, WMW, WNW, TM, TN, ACC, ST, OCC)
+#define IU8_PAIR_VARIANT(name, TM, NT, KW, WPB, D, ALDS)
 #include "iu8_variants.def"
 #undef IU8_DEC_VARIANT
 #undef IU8_PF_VARIANT
+#undef IU8_PAIR_VARIANT
 #undef IU8_PF32

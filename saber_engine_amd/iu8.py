@@ -108,6 +108,8 @@ def lib():
         L.saber_iu8_gemm.argtypes = [C.c_void_p, C.c_int] + [C.c_void_p] * 5 + [C.c_uint32] * 3 + [C.c_void_p] * 3
         L.saber_iu8_gemm_acc.argtypes = [C.c_void_p, C.c_int] + [C.c_void_p] * 3 + [C.c_uint32] * 3 + [C.c_void_p]
         L.saber_iu8_fused_holds.argtypes = [C.c_uint32, C.c_uint32]
+        L.saber_iu8_pair.argtypes = [C.POINTER(Desc)] * 3
+        L.saber_iu8_gemm_pair.argtypes = [C.c_void_p] * 6 + [C.c_uint32] + [C.c_void_p] * 3 + [C.c_uint32] * 3 + [C.c_void_p]
         L.saber_iu8_linear_fused.argtypes = [C.c_void_p, C.c_int] + [C.c_void_p] * 6 + [C.c_uint32] * 3 + [C.c_void_p]
         L.saber_iu8_quant_had.argtypes = [C.c_void_p] * 4 + [C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p]
         L.saber_iu8_silu_mul_quant_had.argtypes = [C.c_void_p] * 4 + [C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p]
@@ -149,6 +151,13 @@ def resolve(wkind, m, n, k):
 def describe(kernel, m, n, k, ks=1):
     d = Desc()
     _check(lib().saber_iu8_describe(kernel.encode(), m, n, k, ks, C.byref(d)))
+    return d
+
+
+def pair(first, second):
+    """Two W4 decode descriptors of one M, K -> the one-dispatch pair (macaq_iu8.rs:632-704)."""
+    d = Desc()
+    _check(lib().saber_iu8_pair(C.byref(first), C.byref(second), C.byref(d)))
     return d
 
 
@@ -293,6 +302,9 @@ class Context:
 
     def gemm(self, wkind, a, a_scale, w, w_scale, c, m, n, k, partial=None, counter=None, stream=0):
         _check(lib().saber_iu8_gemm(self._h, wkind, a, a_scale, w, w_scale, c, m, n, k, partial, counter, stream))
+
+    def gemm_pair(self, a, a_scale, w, w_scale, c, n, w_b, w_scale_b, c_b, n_b, m, k, stream=0):
+        _check(lib().saber_iu8_gemm_pair(self._h, a, a_scale, w, w_scale, c, n, w_b, w_scale_b, c_b, n_b, m, k, stream))
 
     def linear_fused(self, wkind, x, w, w_scale, c, m, n, k, q=None, scale=None, stream=0):
         _check(lib().saber_iu8_linear_fused(self._h, wkind, x, w, w_scale, c, q, scale, m, n, k, stream))

@@ -29,7 +29,7 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # -ffp-contract=off: every product and sum rounds where the source says (the epilogue contract);
 # the packed-fp32 feature is switched off for every device compile of this tree.
 FLAGS = f"--genco --offload-arch={ARCH} -O3 -ffp-contract=off -Xclang -target-feature -Xclang -packed-fp32-ops"
-PLUGINS = ("macaq_iu8", "macaq_i8q", "mxfp4_hadi8", "attn_glue_hadi8", "moe_iu8", "iu8_probe")
+PLUGINS = ("macaq_iu8", "macaq_iu8f", "macaq_i8q", "mxfp4_hadi8", "attn_glue_hadi8", "moe_iu8", "iu8_probe")
 
 
 def candidates(stem, arch):

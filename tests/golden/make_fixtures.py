@@ -57,17 +57,34 @@ def main():
         out[f"c{i}_meta"] = np.array([M, N, K, int(w8)], np.int32)
     np.savez_compressed(os.path.join(HERE, "dense_small.npz"), **out)
 
-    ref_manifest = "/root/reference/prebuilt/gfx1201/macaq_iu8.manifest.toml"
-    if os.path.exists(ref_manifest):
-        import re
+    write_kernarg_table()
 
-        text = open(ref_manifest).read()
-        table = {}
+
+# The reference's committed manifests hold the explicit kernarg offsets/sizes its host packs; the
+# symbols this build also ships are kept (every macaq_iu8 kernel, the decode pair, the int8 twins).
+KERNARG_SOURCES = {
+    "macaq_iu8": None,
+    "macaq_iu8f": ("macaq_iu8f_pair_w4_tm",),
+    "mxfp4_hadi8": ("add_rms_quant_hadi8_", "silu_mul_quant_hadi8_", "gdn_norm_quant_hadi8_"),
+    "attn_glue_hadi8": ("attn_gate_quant_hadi8_",),
+}
+
+
+def write_kernarg_table(ref_dir="/root/reference/prebuilt/gfx1201"):
+    import re
+
+    if not os.path.isdir(ref_dir):
+        return
+    table = {}
+    for plugin, prefixes in KERNARG_SOURCES.items():
+        text = open(os.path.join(ref_dir, plugin + ".manifest.toml")).read()
         for blk in text.split("[[kernel]]")[1:]:
             name = re.search(r'name = "(\w+)"', blk).group(1)
+            if prefixes is not None and not name.startswith(prefixes):
+                continue
             args = re.findall(r'offset = (\d+)\nsize = (\d+)\nvalue_kind = "(\w+)"\nname = "(\w+)"', blk)
             table[name] = [dict(name=a[3], offset=int(a[0]), size=int(a[1]), value_kind=a[2]) for a in args]
-        json.dump(table, open(os.path.join(HERE, "kernarg_gfx1201.json"), "w"), indent=1, sort_keys=True)
+    json.dump(table, open(os.path.join(HERE, "kernarg_gfx1201.json"), "w"), indent=1, sort_keys=True)
 
 
 if __name__ == "__main__":

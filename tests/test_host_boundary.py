@@ -80,6 +80,47 @@ def test_activation_rows_are_staged_when_they_fit():
     assert iu8.resolve(iu8.W4, 8, 5120, 17408).kernel == b"macaq_iu8_dec_w4_tm1_a0"     # does not fit
 
 
+def test_pair_lays_two_decode_grids_end_to_end():
+    """macaq_iu8::pair (crates/saber-kernels/src/macaq_iu8.rs:632-704): each half keeps its own descriptor's
+    split and workspaces; refusals by name."""
+    a, b = iu8.resolve(iu8.W4, 4, 12288, 5120), iu8.resolve(iu8.W4, 4, 96, 5120)
+    d = iu8.pair(a, b)
+    assert d.kernel == b"macaq_iu8f_pair_w4_tm1" and d.plugin == b"macaq_iu8f" and d.op == b"gemm_i4a8_pair"
+    assert tuple(d.grid) == (a.grid[0] + b.grid[0], 1, 1) and d.block[0] == a.block[0] and d.n_launches == 1
+    vals = {n: d.arg(n).ival for n in ("m", "k", "n", "ks", "nb", "n_b", "ks_b", "nb_b")}
+    assert vals == dict(m=4, k=5120, n=12288, ks=1, nb=a.grid[0], n_b=96, ks_b=1, nb_b=b.grid[0])
+    for n in ("decode_partial", "decode_counter", "decode_partial_b", "decode_counter_b"):
+        assert d.arg(n).kind == iu8.ARG_NULL_BUFFER
+    assert d.n_workspaces == 0 and d.kernarg_bytes == 128
+    # rows that stream from L2 pair on the streamed form
+    assert iu8.pair(iu8.resolve(iu8.W4, 16, 5120, 5120), iu8.resolve(iu8.W4, 16, 64, 5120)).kernel == b"macaq_iu8f_pair_w4_tm1_a0"
+    assert iu8.pair(iu8.resolve(iu8.W4, 40, 5120, 5120), iu8.resolve(iu8.W4, 40, 64, 5120)).kernel == b"macaq_iu8f_pair_w4_tm3"
+    # explicit splits: the grids multiply, the second half's workspaces take the suffix
+    a2, b2 = iu8.describe("macaq_iu8_dec_w4_tm1", 4, 256, 5120, ks=2), iu8.describe("macaq_iu8_dec_w4_tm1", 4, 64, 5120, ks=4)
+    d2 = iu8.pair(a2, b2)
+    assert d2.grid[0] == a2.grid[0] * 2 + b2.grid[0] * 4 and d2.n_workspaces == 4
+    assert d2.workspace("decode_partial").bytes == 2 * 4 * 256 * 4 and d2.workspace("decode_partial_b").bytes == 4 * 4 * 64 * 4
+    assert d2.workspace("decode_counter_b").kind == iu8.WS_PERSISTENT and d2.workspace("decode_counter_b").zero_once
+    assert d2.arg("decode_partial_b").kind == iu8.ARG_BUFFER and d2.arg("ks_b").ival == 4
+    for x, y in [(iu8.resolve(iu8.W4, 4, 256, 5120), iu8.resolve(iu8.W4, 4, 256, 17408)),      # another K
+                 (iu8.resolve(iu8.W4, 4, 256, 5120), iu8.resolve(iu8.W4, 5, 256, 5120)),       # another M
+                 (iu8.resolve(iu8.W4, 4, 256, 5120), iu8.resolve(iu8.W8, 4, 256, 5120)),       # an int8-row half
+                 (iu8.resolve(iu8.W4, 100, 256, 5120), iu8.resolve(iu8.W4, 100, 256, 5120))]:  # prefill cells
+        with pytest.raises(iu8.IU8Error) as e:
+            iu8.pair(x, y)
+        assert e.value.code == iu8.E_RULE and "pair" in str(e.value)
+
+
+def test_pair_variants_share_their_decode_twin_geometry():
+    text = open(os.path.join(iu8.PKG, "csrc", "kernels", "iu8_variants.def")).read()
+    dec = {m[0]: m[1:] for m in re.findall(r"^IU8_DEC_VARIANT\((\w+), (\d+), (\w+), (\d+), (\d+), (\d+), (\d+), (\d+), (\w+)\)", text, flags=re.M)}
+    pairs = re.findall(r"^IU8_PAIR_VARIANT\((\w+), (\d+), (\d+), (\d+), (\d+), (\d+), (\d+)\)", text, flags=re.M)
+    assert len(pairs) == 5
+    for name, tm, nt, kw, wpb, d, alds in pairs:
+        twin = dec[name.replace("macaq_iu8f_pair_", "macaq_iu8_dec_")]
+        assert twin == (tm, "false", nt, kw, wpb, d, alds, "false"), name
+
+
 def test_explicit_split_declares_its_workspaces():
     d = iu8.describe("macaq_iu8_dec_w4_tm1", 4, 5120, 17408, ks=4)
     assert d.ks == 4 and d.grid[2] == 4
@@ -128,7 +169,7 @@ def test_signatures_pack_exactly_like_the_reference_manifest():
         assert [("global_buffer" if s[3] == iu8.ARG_BUFFER else "by_value") for s in slots] == [a["value_kind"] for a in args]
         assert nbytes == max(a["offset"] + a["size"] for a in args)
         checked += 1
-    assert checked == 10
+    assert checked == 20
 
 
 def test_kernarg_image_built_two_ways_is_byte_identical():
@@ -174,7 +215,8 @@ def test_every_built_manifest_validates_against_its_code_object():
 
 
 def test_reference_symbols_and_lds_budget():
-    text = open(os.path.join(iu8.PREBUILT, "macaq_iu8.manifest.toml")).read()
+    stems = ("macaq_iu8", "macaq_iu8f", "mxfp4_hadi8", "attn_glue_hadi8")
+    text = "".join(open(os.path.join(iu8.PREBUILT, f"{s}.manifest.toml")).read() for s in stems)
     for name in json.load(open(os.path.join(GOLD, "kernarg_gfx1201.json"))):
         assert f'name = "{name}"' in text and f'symbol = "{name}.kd"' in text
     assert max(int(v) for v in re.findall(r"group_segment_fixed_size = (\d+)", text)) <= 160 * 1024
