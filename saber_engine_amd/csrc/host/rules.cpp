@@ -318,7 +318,12 @@ int resolve_fused(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc 
   copy_name(d->op, sizeof d->op, op);
   copy_name(d->plugin, sizeof d->plugin, "macaq_iu8");
   copy_name(d->kernel, sizeof d->kernel, name);
-  d->grid[0] = (n + 31) / 32, d->grid[1] = 1, d->grid[2] = 1;  // 8 waves: 4 k-waves x 2 weight tiles
+  // 8 waves: 4 k-waves x 2 weight tiles = 32 columns a block. Persistent past two workgroups a CU
+  // (what its registers let reside): the workgroups walk the blocks, at most 8 each.
+  const uint32_t nblk = (n + 31) / 32, resident = 2 * CU_COUNT;
+  uint32_t grid = nblk;
+  if (nblk > resident) grid = std::max(resident, ((nblk + 7) / 8 + CU_COUNT - 1) / CU_COUNT * CU_COUNT);
+  d->grid[0] = grid, d->grid[1] = 1, d->grid[2] = 1;
   d->block[0] = 512, d->block[1] = 1, d->block[2] = 1;
   d->n_launches = 1;
   d->ks = 1;

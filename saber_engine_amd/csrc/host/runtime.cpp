@@ -301,6 +301,26 @@ int saber_iu8_has_kernel(const saber_iu8_ctx *ctx, const char *kernel) {
   return ctx && kernel && ctx->fn.count(kernel) ? 1 : 0;
 }
 
+// What a hand-edited descriptor could get wrong for a kernel whose bounds depend on its grid: the
+// fused decode linear keeps at most 8 column blocks' weight scales a workgroup and 20 KiB of codes.
+static int launch_guard(const saber_iu8_desc *d) {
+  if (strncmp(d->kernel, "macaq_iu8_decq_", 15) != 0) return 0;
+  int64_t m = 0, n = 0, k = 0;
+  for (uint32_t i = 0; i < d->n_args; ++i) {
+    if (d->args[i].kind != SABER_IU8_ARG_I32) continue;
+    if (!strcmp(d->args[i].name, "m")) m = d->args[i].ival;
+    if (!strcmp(d->args[i].name, "n")) n = d->args[i].ival;
+    if (!strcmp(d->args[i].name, "k")) k = d->args[i].ival;
+  }
+  if (m <= 0 || n <= 0 || k <= 0 || !fused_holds((uint32_t)m, (uint32_t)k))
+    return fail(SABER_IU8_E_RULE, fmt("%s: %lld rows of %lld do not fit the fused form", d->kernel, (long long)m, (long long)k));
+  const int64_t nblk = (n + 31) / 32;
+  if ((int64_t)d->grid[0] * 8 < nblk || d->grid[1] != 1 || d->grid[2] != 1 || d->block[0] != 512)
+    return fail(SABER_IU8_E_RULE, fmt("%s: grid %u x %u x %u of %u threads cannot walk %lld column blocks (at most 8 a workgroup)",
+                                      d->kernel, d->grid[0], d->grid[1], d->grid[2], d->block[0], (long long)nblk));
+  return 0;
+}
+
 int saber_iu8_launch(saber_iu8_ctx *ctx, const saber_iu8_desc *d, const saber_iu8_binding *bufs, uint32_t n_bufs,
                      void *stream) {
   if (!ctx || !d) return fail(SABER_IU8_E_ARG, "launch: null argument");
@@ -308,6 +328,7 @@ int saber_iu8_launch(saber_iu8_ctx *ctx, const saber_iu8_desc *d, const saber_iu
   if (it == ctx->fn.end()) return fail(SABER_IU8_E_NOTLOADED, std::string(d->kernel) + ": not in the loaded plugin set");
   if (d->shared_bytes != 0) return fail(SABER_IU8_E_RULE, std::string(d->kernel) + ": dynamic LDS is not part of this ABI");
   if (!d->grid[0] || !d->grid[1] || !d->grid[2] || !d->block[0]) return fail(SABER_IU8_E_RULE, std::string(d->kernel) + ": empty grid");
+  if (int rc = launch_guard(d)) return rc;
   alignas(16) uint8_t image[256];
   uint32_t bytes = 0;
   if (int rc = saber_iu8_pack_kernarg(d, bufs, n_bufs, image, sizeof image, &bytes)) return rc;

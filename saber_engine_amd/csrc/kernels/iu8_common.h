@@ -69,19 +69,33 @@ static __device__ __forceinline__ unsigned iu8_code(float x, float sc) {
   return ((unsigned)(int)__builtin_rintf(y)) & 0xffu;
 }
 
-// The same code without a divide per element: rcp = __fdiv_rn(1, sc) once a row, t = x * rcp is
+// The same codes without a divide per element: rcp = __fdiv_rn(1, sc) once a row, t = x * rcp is
 // within 1.6e-5 of x / sc for |x / sc| <= 127 (two roundings of 2^-24 relative), the IEEE quotient
 // within 7.6e-6. If t sits at least 1e-4 inside its rounding interval, the IEEE quotient rounds to
 // the same integer; otherwise (a tie or next to one, rare) the divide decides. NaN and infinite
 // rows come out as through the divide: NaN clamps to -127 on both paths.
-static __device__ __forceinline__ unsigned iu8_code_rcp(float x, float sc, float rcp) {
-  float y = fminf(fmaxf(x * rcp, -127.f), 127.f);
-  float q = __builtin_rintf(y);
-  if (__builtin_expect(fabsf(y - q) > 0.4999f, 0)) {
-    y = fminf(fmaxf(__fdiv_rn(x, sc), -127.f), 127.f);
-    q = __builtin_rintf(y);
-  }
-  return ((unsigned)(int)q) & 0xffu;
+//
+// Four codes at once, packed little-endian into a dword, by the same law. The fast path rounds by
+// adding 1.5 * 2^23: for |t| <= 127 the sum's unit in the last place is 1, so the IEEE addition itself
+// rounds t to the nearest integer, ties to even, and leaves that integer's two's-complement low byte
+// in the low byte of the sum's bit pattern; subtracting the constant again (exact) gives the rounded
+// value for the tie test. v_med3_f32 returns the minimum of its operands when one is NaN, which is
+// the -127 of fminf(fmaxf(NaN, -127), 127). Any element next to a tie sends its four to the divide.
+static __device__ __forceinline__ unsigned iu8_code4_rcp(float x0, float x1, float x2, float x3, float sc, float rcp) {
+#pragma clang fp contract(off)
+  const float MAGIC = 12582912.f;
+  const float t0 = __builtin_amdgcn_fmed3f(x0 * rcp, -127.f, 127.f), t1 = __builtin_amdgcn_fmed3f(x1 * rcp, -127.f, 127.f);
+  const float t2 = __builtin_amdgcn_fmed3f(x2 * rcp, -127.f, 127.f), t3 = __builtin_amdgcn_fmed3f(x3 * rcp, -127.f, 127.f);
+  const float u0 = t0 + MAGIC, u1 = t1 + MAGIC, u2 = t2 + MAGIC, u3 = t3 + MAGIC;
+  // one test for the four: the largest distance of a t from its rounded value
+  const float off = fmaxf(fmaxf(fabsf(t0 - (u0 - MAGIC)), fabsf(t1 - (u1 - MAGIC))),
+                          fmaxf(fabsf(t2 - (u2 - MAGIC)), fabsf(t3 - (u3 - MAGIC))));
+  const bool near_tie = !(off <= 0.4999f);  // NaN goes to the divide as well
+  if (__builtin_expect(near_tie, 0))
+    return iu8_code(x0, sc) | (iu8_code(x1, sc) << 8) | (iu8_code(x2, sc) << 16) | (iu8_code(x3, sc) << 24);
+  // bytes 0,1 from (u0, u1), bytes 2,3 from (u2, u3); selector 0x0c yields a zero byte
+  return __builtin_amdgcn_perm(__float_as_uint(u1), __float_as_uint(u0), 0x0c0c0400u) |
+         __builtin_amdgcn_perm(__float_as_uint(u3), __float_as_uint(u2), 0x04000c0cu);
 }
 
 static __device__ __forceinline__ iu8_v4u iu8_ldg_nt(const iu8_u8 *p) {

@@ -1,0 +1,240 @@
+// The fused decode linear of the gfx950 W4A8-iu8 path: per-token int8 quantisation of at most 4 bf16
+// rows + the GEMV against them, one persistent launch. Operand orders and the contract: iu8_common.h.
+//
+// A workgroup (WPB waves: WN column groups x KW k-waves, as in the plain decode body) owns the
+// column blocks blockIdx.x, blockIdx.x + gridDim.x, ... of WN*NT*16 columns each. It quantises the
+// rows once (row amax, IEEE divide law, codes into LDS in staged order) while its first weight loads
+// are in flight, then streams its blocks' weights against the staged codes. The weight ring (D
+// 128-deep K steps of 128-bit nontemporal loads a wave) runs ACROSS block boundaries: when a wave
+// consumes the last step of a block its loads for the next block are already in flight, so the
+// memory pipe never drains inside the launch. A block ends with the k-waves' partials meeting in
+// LDS (exact int32, two alternating areas so one barrier a block suffices) and the bf16 epilogue,
+// whose weight scales were put in LDS at the start: loads return in order, so a scale load issued
+// at a block's end would only come back behind the whole ring. A launch gives a workgroup at most
+// IU8_DECQ_MAXB blocks (the host's grid law).
+#pragma once
+#include "iu8_common.h"
+
+#define IU8_DECQ_MAXB 8  // column blocks a workgroup: gridDim.x >= ceil(blocks / 8)
+
+template <bool W8, int NT, int KW, int WPB, int D>
+__device__ __forceinline__ void iu8_decq_body(const unsigned short *__restrict__ X, const iu8_u8 *__restrict__ W,
+                                              const float *__restrict__ ws, iu8_u8 *__restrict__ qout,
+                                              float *__restrict__ sout, unsigned short *__restrict__ C, int M, int N,
+                                              int K) {
+  static_assert(KW > 1 && WPB % KW == 0, "k-waves divide the workgroup");
+  constexpr int WN = WPB / KW;
+  constexpr int NTHR = WPB * 64;
+  constexpr int WSTEP = W8 ? 2048 : 1024;  // bytes of one 16-row weight tile per 128-deep K step
+  constexpr int WV = W8 ? 2 : 1;           // 16-byte loads a lane per step per tile
+  constexpr int ABYTES = 20 * 1024;        // staged codes: pow2(M) * K bytes
+  constexpr int RED = (KW - 1) * WN * NT * 256;  // ints of one partial area
+  __shared__ __attribute__((aligned(16))) iu8_u8 s_a[ABYTES];
+  __shared__ __attribute__((aligned(16))) int s_red[2][RED];
+  __shared__ float s_amax[WPB][4];
+  __shared__ float s_ws[IU8_DECQ_MAXB][WN * NT * 16];  // the epilogue's weight scales (W4: already / 16)
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wk = wave % KW, wn = wave / KW;
+  const int ntiles = N >> 4, steps = K >> 7;
+  const int ml = lane & 15, lg = lane >> 4;
+  const int T = wk < steps ? (steps - wk + KW - 1) / KW : 0;  // this wave's steps of a block: wk + t*KW
+  const int nblk = (ntiles + WN * NT - 1) / (WN * NT);
+  const int G = gridDim.x;
+  const int nb = (int)blockIdx.x < nblk ? (nblk - (int)blockIdx.x + G - 1) / G : 0;  // this workgroup's blocks
+  const int TT = nb * T;
+
+  // ---- the rows' bf16 pieces (8 elements = 16 bytes; piece p = row * K/8 + k/8), loaded first
+  int mr_shift = 0;
+  while ((1 << mr_shift) < M) ++mr_shift;
+  constexpr int X_PER = (ABYTES / 8 + NTHR - 1) / NTHR;
+  iu8_v4u xreg[X_PER];
+  const int k8 = K >> 3, x_pieces = M * k8;
+#pragma unroll
+  for (int p = 0; p < X_PER; ++p)
+    if (p * NTHR + tid < x_pieces) xreg[p] = *((const iu8_v4u *)X + p * NTHR + tid);
+
+  // ---- this workgroup's weight scales, all blocks
+  for (int i = tid; i < min(nb, IU8_DECQ_MAXB) * (WN * NT * 16); i += NTHR) {
+    const int b = i / (WN * NT * 16), c = i - b * (WN * NT * 16);
+    const int n = ((int)blockIdx.x + b * G) * (WN * NT * 16) + c;
+    s_ws[b][c] = n < N ? iu8_wsu<W8>(ws, n) : 0.f;
+  }
+
+  // ---- the issue side of the ring: block ib, step it, this lane's address in every tile
+  int ib = 0, it = 0;
+  const iu8_u8 *ip[NT];
+  auto set_ip = [&](int b) {
+    const int nt0 = (((int)blockIdx.x + b * G) * WN + wn) * NT;
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+      const int ntj = min(nt0 + j, ntiles - 1);  // a tile past N re-reads the last one and stores nothing
+      ip[j] = W + ((size_t)ntj * steps + wk) * WSTEP + lane * 16;
+    }
+  };
+  set_ip(0);
+  iu8_v4u ring[D][NT][WV];
+  auto issue = [&](int slot) {
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int v = 0; v < WV; ++v) ring[slot][j][v] = iu8_ldg_nt(ip[j] + v * 1024);
+    if (++it == T) {
+      it = 0;
+      if (++ib < nb) set_ip(ib);
+    } else {
+#pragma unroll
+      for (int j = 0; j < NT; ++j) ip[j] += KW * WSTEP;
+    }
+  };
+#pragma unroll
+  for (int i = 0; i < D; ++i)
+    if (i < TT) issue(i);
+
+  // ---- quantise the rows behind the first loads: amax lane -> wave (butterfly) -> workgroup (LDS),
+  // all order-free maxima; sc = max(amax / 127, 1e-30); codes by the exact reciprocal path
+  float qsc[4] = {1.f, 1.f, 1.f, 1.f};
+  {
+    float am[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int p = 0; p < X_PER; ++p) {
+      const int piece = p * NTHR + tid;
+      if (piece >= x_pieces) continue;
+      const int row = (piece >= k8) + (piece >= 2 * k8) + (piece >= 3 * k8);  // M <= 4: no divide
+      float m8 = 0.f;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        m8 = fmaxf(m8, fabsf(__uint_as_float(xreg[p][w] << 16)));
+        m8 = fmaxf(m8, fabsf(__uint_as_float(xreg[p][w] & 0xFFFF0000u)));
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r) am[r] = r == row ? fmaxf(am[r], m8) : am[r];
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+#pragma unroll
+      for (int o = 32; o; o >>= 1) am[r] = fmaxf(am[r], __shfl_xor(am[r], o, 64));
+    }
+    if (lane == 0) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) s_amax[wave][r] = am[r];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      float a = s_amax[0][r];
+#pragma unroll
+      for (int w = 1; w < WPB; ++w) a = fmaxf(a, s_amax[w][r]);
+      qsc[r] = fmaxf(__fdiv_rn(a, 127.f), 1e-30f);
+    }
+    const bool out0 = blockIdx.x == 0 && qout != nullptr;
+    if (blockIdx.x == 0 && sout != nullptr && tid < M)
+      sout[tid] = tid == 0 ? qsc[0] : tid == 1 ? qsc[1] : tid == 2 ? qsc[2] : qsc[3];
+#pragma unroll
+    for (int p = 0; p < X_PER; ++p) {
+      const int piece = p * NTHR + tid;
+      if (piece >= x_pieces) continue;
+      const int row = (piece >= k8) + (piece >= 2 * k8) + (piece >= 3 * k8), k = (piece - row * k8) << 3;
+      const float sc = row == 0 ? qsc[0] : row == 1 ? qsc[1] : row == 2 ? qsc[2] : qsc[3];
+      const float rcp = __fdiv_rn(1.f, sc);
+      float f[8];
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        f[2 * w] = __uint_as_float(xreg[p][w] << 16);
+        f[2 * w + 1] = __uint_as_float(xreg[p][w] & 0xFFFF0000u);
+      }
+      const unsigned d0 = iu8_code4_rcp(f[0], f[1], f[2], f[3], sc, rcp);
+      const unsigned d1 = iu8_code4_rcp(f[4], f[5], f[6], f[7], sc, rcp);
+      // staged order: piece ((kt*4 + g) * MR + row) holds the row's 16 bytes of k = kt*64 + g*16
+      const int kt = k >> 6, g = (k >> 4) & 3, half = (k >> 3) & 1;
+      *(iu8_v2u *)&s_a[((((kt * 4 + g) << mr_shift) + row) << 4) + half * 8] = iu8_v2u{d0, d1};
+      if (out0) *(iu8_v2u *)(qout + (size_t)kt * 1024 + (row + 16 * g) * 16 + half * 8) = iu8_v2u{d0, d1};
+    }
+    __syncthreads();
+  }
+
+  // ---- the consume side: block cb, step ct
+  iu8_v4i acc[NT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j) acc[j] = iu8_v4i{0, 0, 0, 0};
+  int cb = 0, ct = 0;
+  const int a_lane = (((lg << mr_shift) + min(ml, (1 << mr_shift) - 1)) << 4);
+  // LDS writes of this wave are done, then the workgroup meets; loads in flight stay in flight
+  auto meet = [&]() {
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+  };
+  auto block_end = [&]() {
+    int *red = s_red[cb & 1];
+    if (wk > 0) {
+#pragma unroll
+      for (int j = 0; j < NT; ++j) *(iu8_v4i *)&red[(((wk - 1) * WN + wn) * NT + j) * 256 + lane * 4] = acc[j];
+    }
+    meet();
+    if (wk == 0) {
+#pragma unroll
+      for (int q = 0; q < KW - 1; ++q)
+#pragma unroll
+        for (int j = 0; j < NT; ++j) acc[j] += *(const iu8_v4i *)&red[((q * WN + wn) * NT + j) * 256 + lane * 4];
+      const int nt0 = (((int)blockIdx.x + cb * G) * WN + wn) * NT;
+#pragma unroll
+      for (int j = 0; j < NT; ++j) {
+        if (nt0 + j >= ntiles || ml >= M) continue;
+        const int n = (nt0 + j) * 16 + lg * 4;
+        const float *wsu = &s_ws[min(cb, IU8_DECQ_MAXB - 1)][(wn * NT + j) * 16 + lg * 4];
+        const float am = ml == 0 ? qsc[0] : ml == 1 ? qsc[1] : ml == 2 ? qsc[2] : qsc[3];
+        unsigned h[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) h[r] = iu8_bf16_bits(iu8_epi(acc[j][r], am, wsu[r]));
+        *(iu8_v2u *)(C + (size_t)ml * N + n) = iu8_v2u{h[0] | (h[1] << 16), h[2] | (h[3] << 16)};
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < NT; ++j) acc[j] = iu8_v4i{0, 0, 0, 0};
+    ++cb;
+  };
+  auto consume = [&](int slot) {
+    const int kt = 2 * (wk + ct * KW);
+    const iu8_v4i a0 = *(const iu8_v4i *)&s_a[((kt * 4) << (mr_shift + 4)) + a_lane];
+    const iu8_v4i a1 = *(const iu8_v4i *)&s_a[(((kt + 1) * 4) << (mr_shift + 4)) + a_lane];
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+      iu8_v4i w0, w1;
+      if constexpr (W8) {
+        w0 = (iu8_v4i)ring[slot][j][0];
+        w1 = (iu8_v4i)ring[slot][j][WV - 1];
+      } else {
+        iu8_unpack_w4(ring[slot][j][0], w0, w1);
+      }
+      acc[j] = iu8_mfma(w0, a0, acc[j]);
+      acc[j] = iu8_mfma(w1, a1, acc[j]);
+    }
+    if (++ct == T) {
+      ct = 0;
+      block_end();
+    }
+  };
+
+  if (T == 0) {  // a k-wave past a short K: no steps, but it meets the others once a block
+    for (int b = 0; b < nb; ++b) block_end();
+    return;
+  }
+  int L0 = 0;
+  for (; L0 + 2 * D <= TT; L0 += D) {  // steady state: every slot consumed and re-issued
+#pragma unroll
+    for (int i = 0; i < D; ++i) {
+      consume(i);
+      issue(i);
+    }
+  }
+  for (; L0 < TT; L0 += D) {  // drain
+#pragma unroll
+    for (int i = 0; i < D; ++i) {
+      if (L0 + i < TT) {
+        consume(i);
+        if (L0 + i + D < TT) issue(i);
+      }
+    }
+  }
+}

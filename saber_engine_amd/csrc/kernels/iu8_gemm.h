@@ -33,19 +33,12 @@ static __device__ __forceinline__ iu8_blk iu8_blk_of_grid() {
 }
 
 // ============================================================================ decode band
-// QF ("quant fused", M <= 4, dense rows, no grid split): `A` is the bf16 activation matrix [M, K]
-// itself. Every workgroup quantises the rows on its way into LDS (the per-token int8 law of
-// iu8_common.h: row amax, IEEE divide, round half to even) while its first weight loads are in
-// flight, and keeps the row scales in registers; workgroup 0 also stores the codes (A fragment
-// order) and scales to `qout` / `sout` when those are not null.
-template <int TM, bool W8, int NT, int KW, int WPB, int D, int ALDS, bool ACC, bool QF = false>
+template <int TM, bool W8, int NT, int KW, int WPB, int D, int ALDS, bool ACC>
 __device__ __forceinline__ void iu8_dec_body(const iu8_u8 *__restrict__ A, const iu8_u8 *__restrict__ W,
                                              const float *__restrict__ as, const float *__restrict__ ws,
                                              int *__restrict__ P, int *__restrict__ cnt, void *__restrict__ Cv,
-                                             const iu8_rows R, int N, int K, iu8_u8 *__restrict__ qout = nullptr,
-                                             float *__restrict__ sout = nullptr, const iu8_blk B = iu8_blk_of_grid()) {
+                                             const iu8_rows R, int N, int K, const iu8_blk B = iu8_blk_of_grid()) {
   const int M = R.rows;
-  static_assert(!QF || (ALDS > 0 && TM == 1 && !ACC), "the fused form stages its rows in LDS");
   static_assert(WPB % KW == 0, "k-waves divide the workgroup");
   static_assert(ALDS == 0 || TM == 1, "LDS staging of A is the M <= 16 form");
   constexpr int WN = WPB / KW;
@@ -94,18 +87,7 @@ __device__ __forceinline__ void iu8_dec_body(const iu8_u8 *__restrict__ A, const
   constexpr bool A_INREG = A_PER <= 8;
   iu8_v4u areg[A_INREG ? A_PER : 1];
   int a_pieces = 0;
-  // fused form: pieces of 8 bf16 (16 bytes) of x, row-major; piece p = row * K/8 + k/8
-  constexpr int X_PER = QF ? (ABYTES / 8 + NTHR - 1) / NTHR : 1;
-  iu8_v4u xreg[X_PER];
-  float qsc[4] = {1.f, 1.f, 1.f, 1.f};
-  const int x_pieces = QF ? M * (K >> 3) : 0;
-  if constexpr (QF) {
-    while ((1 << mr_shift) < M) ++mr_shift;
-    staged = true;
-#pragma unroll
-    for (int p = 0; p < X_PER; ++p)
-      if (p * NTHR + tid < x_pieces) xreg[p] = *((const iu8_v4u *)A + p * NTHR + tid);
-  } else if constexpr (ALDS > 0) {
+  if constexpr (ALDS > 0) {
     while ((1 << mr_shift) < M) ++mr_shift;
     a_pieces = ((s_hi - s_lo) * 2 * 4) << mr_shift;
     staged = M <= 16 && a_pieces * 16 <= ABYTES;
@@ -197,65 +179,7 @@ __device__ __forceinline__ void iu8_dec_body(const iu8_u8 *__restrict__ A, const
 #pragma unroll
       for (int i = 0; i < D; ++i)
         if (i < T) issue(i, i);
-      if constexpr (QF) {
-        // row amax: lane -> wave (butterfly) -> workgroup (LDS), all order-free maxima
-        __shared__ float s_amax[WPB][4];
-        const int k8 = K >> 3;
-        float am[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int p = 0; p < X_PER; ++p) {
-          const int piece = p * NTHR + tid;
-          if (piece >= x_pieces) continue;
-          const int row = piece / k8;
-          float m8 = 0.f;
-#pragma unroll
-          for (int w = 0; w < 4; ++w) {
-            m8 = fmaxf(m8, fabsf(__uint_as_float(xreg[p][w] << 16)));
-            m8 = fmaxf(m8, fabsf(__uint_as_float(xreg[p][w] & 0xFFFF0000u)));
-          }
-#pragma unroll
-          for (int r = 0; r < 4; ++r) am[r] = r == row ? fmaxf(am[r], m8) : am[r];
-        }
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-#pragma unroll
-          for (int o = 32; o; o >>= 1) am[r] = fmaxf(am[r], __shfl_xor(am[r], o, 64));
-        }
-        if (lane == 0) {
-#pragma unroll
-          for (int r = 0; r < 4; ++r) s_amax[wave][r] = am[r];
-        }
-        __syncthreads();
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          float a = s_amax[0][r];
-#pragma unroll
-          for (int w = 1; w < WPB; ++w) a = fmaxf(a, s_amax[w][r]);
-          qsc[r] = fmaxf(__fdiv_rn(a, 127.f), 1e-30f);
-        }
-        const bool out0 = B.bx == 0 && qout != nullptr;
-        if (B.bx == 0 && sout != nullptr && tid < M)
-          sout[tid] = tid == 0 ? qsc[0] : tid == 1 ? qsc[1] : tid == 2 ? qsc[2] : qsc[3];
-#pragma unroll
-        for (int p = 0; p < X_PER; ++p) {
-          const int piece = p * NTHR + tid;
-          if (piece >= x_pieces) continue;
-          const int row = piece / k8, k = (piece - row * k8) << 3;
-          const float sc = row == 0 ? qsc[0] : row == 1 ? qsc[1] : row == 2 ? qsc[2] : qsc[3];
-          const float rcp = __fdiv_rn(1.f, sc);
-          unsigned d0 = 0, d1 = 0;
-#pragma unroll
-          for (int w = 0; w < 2; ++w) {
-            d0 |= iu8_code_rcp(__uint_as_float(xreg[p][w] << 16), sc, rcp) << (16 * w);
-            d0 |= iu8_code_rcp(__uint_as_float(xreg[p][w] & 0xFFFF0000u), sc, rcp) << (16 * w + 8);
-            d1 |= iu8_code_rcp(__uint_as_float(xreg[p][2 + w] << 16), sc, rcp) << (16 * w);
-            d1 |= iu8_code_rcp(__uint_as_float(xreg[p][2 + w] & 0xFFFF0000u), sc, rcp) << (16 * w + 8);
-          }
-          const int kt = k >> 6, g = (k >> 4) & 3, half = (k >> 3) & 1;
-          *(iu8_v2u *)&s_mem[((((kt * 4 + g) << mr_shift) + row) << 4) + half * 8] = iu8_v2u{d0, d1};
-          if (out0) *(iu8_v2u *)(qout + (size_t)kt * 1024 + (row + 16 * g) * 16 + half * 8) = iu8_v2u{d0, d1};
-        }
-      } else if constexpr (A_INREG) {
+      if constexpr (A_INREG) {
 #pragma unroll
         for (int p = 0; p < A_PER; ++p)
           if (p * NTHR + tid < a_pieces) *(iu8_v4u *)&s_mem[(p * NTHR + tid) * 16] = areg[p];
@@ -340,9 +264,7 @@ __device__ __forceinline__ void iu8_dec_body(const iu8_u8 *__restrict__ A, const
         if constexpr (ACC) {
           *(iu8_v4i *)((int *)Cv + crow + n) = acc[i][j];
         } else {
-          float am;
-          if constexpr (QF) am = m == 0 ? qsc[0] : m == 1 ? qsc[1] : m == 2 ? qsc[2] : qsc[3];
-          else am = as[iu8_arow(R, m)];
+          const float am = as[iu8_arow(R, m)];
           unsigned h[4];
 #pragma unroll
           for (int r = 0; r < 4; ++r) h[r] = iu8_bf16_bits(iu8_epi(acc[i][j][r], am, wsu[r]));

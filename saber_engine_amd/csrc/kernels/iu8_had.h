@@ -85,12 +85,8 @@ static __device__ __forceinline__ void had_tail(float (&sv)[HAD_MAXG][8], int NV
   for (int i = 0; i < HAD_MAXG; ++i) {
     const int g = tid + i * T;
     if (g >= NV) continue;
-    unsigned lo = 0, hi = 0;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      lo |= iu8_code_rcp(sv[i][j], sc, rcp) << (8 * j);
-      hi |= iu8_code_rcp(sv[i][4 + j], sc, rcp) << (8 * j);
-    }
+    const unsigned lo = iu8_code4_rcp(sv[i][0], sv[i][1], sv[i][2], sv[i][3], sc, rcp);
+    const unsigned hi = iu8_code4_rcp(sv[i][4], sv[i][5], sv[i][6], sv[i][7], sc, rcp);
     // group g = elements 8g..8g+7: fragment kt = g/8, 16-byte piece (g/2)%4 of the row, half g%2
     *(iu8_v2u *)(qrow + (size_t)(g >> 3) * 1024 + ((g >> 1) & 3) * 256 + (g & 1) * 8) = iu8_v2u{lo, hi};
   }

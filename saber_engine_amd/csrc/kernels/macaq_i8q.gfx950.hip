@@ -69,9 +69,7 @@ static __device__ __forceinline__ void i8q_tail(float (&v)[I8Q_MAXG][16], int G,
     unsigned d[4];
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
-      d[w] = 0;
-#pragma unroll
-      for (int b = 0; b < 4; ++b) d[w] |= iu8_code_rcp(v[i][w * 4 + b], sc, rcp) << (8 * b);
+      d[w] = iu8_code4_rcp(v[i][w * 4], v[i][w * 4 + 1], v[i][w * 4 + 2], v[i][w * 4 + 3], sc, rcp);
     }
     *(iu8_v4u *)(qrow + (size_t)(g >> 2) * 1024 + (g & 3) * 256) = iu8_v4u{d[0], d[1], d[2], d[3]};
   }
@@ -211,9 +209,7 @@ static __device__ __forceinline__ void i8q_tail_w64(float (&v)[I8Q_WG][16], int 
     unsigned d[4];
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
-      d[w] = 0;
-#pragma unroll
-      for (int b = 0; b < 4; ++b) d[w] |= iu8_code_rcp(v[i][w * 4 + b], sc, rcp) << (8 * b);
+      d[w] = iu8_code4_rcp(v[i][w * 4], v[i][w * 4 + 1], v[i][w * 4 + 2], v[i][w * 4 + 3], sc, rcp);
     }
     *(iu8_v4u *)(qrow + (size_t)(g >> 2) * 1024 + (g & 3) * 256) = iu8_v4u{d[0], d[1], d[2], d[3]};
   }

@@ -24,6 +24,7 @@
 //           ahead of the MFMAs and across tile boundaries; W4 stays packed in LDS and is unpacked
 //           in registers just in time; the output tile goes out through LDS as whole row segments.
 #include "iu8_gemm.h"
+#include "iu8_decq.h"
 #include "iu8_pf32.h"
 
 #define IU8_DEC(name, TM, W8, NT, KW, WPB, D, ALDS, ACC)                                                         \
@@ -52,12 +53,11 @@
 // it hides behind the first weight loads.
 #define IU8_DECQ(name, W8, D) IU8_DECQX(name, W8, 1, 4, 8, D)  /* the default decode cell's geometry */
 #define IU8_DECQX(name, W8, NT, KW, WPB, D)                                                                            \
-  extern "C" __global__ __launch_bounds__(WPB * 64) void name(                                                          \
+  extern "C" __global__ __launch_bounds__(WPB * 64) __attribute__((amdgpu_waves_per_eu(4, 4))) void name(              \
       const unsigned short *__restrict__ x, const unsigned char *__restrict__ w, const float *__restrict__ ws,     \
       unsigned char *__restrict__ q, float *__restrict__ scale, unsigned short *__restrict__ c, int m, int n,      \
       int k) {                                                                                                     \
-    iu8_dec_body<1, W8, NT, KW, WPB, D, 20, false, true>((const unsigned char *)x, w, nullptr, ws, nullptr, nullptr, c, \
-                                                     iu8_rows{nullptr, 0, m}, n, k, q, scale);                     \
+    iu8_decq_body<W8, NT, KW, WPB, D>(x, w, ws, q, scale, c, m, n, k);                                             \
   }
 IU8_DECQ(macaq_iu8_decq_w4_tm1, false, 8)
 IU8_DECQ(macaq_iu8_decq_w8_tm1, true, 4)

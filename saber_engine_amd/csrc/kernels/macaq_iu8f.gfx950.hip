@@ -23,8 +23,8 @@
     const int bl = p1 ? (int)blockIdx.x - b0 : (int)blockIdx.x, nbp = p1 ? nb_b : nb;                              \
     iu8_dec_body<TM, false, NT, KW, WPB, D, ALDS, false>(                                                           \
         a, p1 ? w_b : w, as, p1 ? ws_b : ws, p1 ? decode_partial_b : decode_partial,                                \
-        p1 ? decode_counter_b : decode_counter, p1 ? c_b : c, iu8_rows{nullptr, 0, m}, p1 ? n_b : n, k, nullptr,    \
-        nullptr, iu8_blk{bl % nbp, bl / nbp, p1 ? ks_b : ks});                                                      \
+        p1 ? decode_counter_b : decode_counter, p1 ? c_b : c, iu8_rows{nullptr, 0, m}, p1 ? n_b : n, k,             \
+        iu8_blk{bl % nbp, bl / nbp, p1 ? ks_b : ks});                                                               \
   }
 #define IU8_DEC_VARIANT(name, TM, W8, NT, KW, WPB, D, ALDS, ACC)
 #define IU8_PF_VARIANT(name, W8, WMW, WNW, TM, TN, ACC, ST, OCC)

@@ -56,6 +56,37 @@ def test_fused_quant_decode_linear_gives_the_bytes_of_the_two_launch_path(ctx, M
         np.testing.assert_array_equal(s.cpu().numpy().view(np.uint32), r["a_scale"].view(np.uint32))
 
 
+@pytest.mark.parametrize("M,N,K,grid", [(2, 16400, 640, None),     # 513 blocks > the persistent grid; k-waves of 2, 1, 1, 1 steps
+                                          (3, 688, 384, 3),         # up to 8 blocks a workgroup; a k-wave with no step
+                                          (1, 1040, 128, 5),        # one K step: three idle k-waves
+                                          (4, 2080, 5120, 17)])     # the ring crossing block ends in its steady state
+def test_fused_linear_walks_column_blocks(ctx, M, N, K, grid):
+    """The fused form is persistent: a workgroup streams several column blocks against rows it
+    quantised once, its load ring running across the block ends."""
+    for w8 in (False, True):
+        say(f"fused decode linear, blocks walked: M={M} N={N} K={K} grid={grid} w8={w8}")
+        case = synth.dense_case(M, N, K, w8=w8, seed=77 + M)
+        r = ref.linear(case["X"], case["W"], case["ws"], w8, threads=8)
+        wk = iu8.W8 if w8 else iu8.W4
+        x, wf, ws = dev_bf16_bits(case["X"]), dev_u8(iu8.repack_weights(case["W"], w8)), dev_f32(case["ws"])
+        c = torch.full((M, N), 0x7FC0, dtype=torch.int16, device="cuda")
+        d = iu8.resolve_fused(wk, M, N, K)
+        if grid is None:
+            assert d.grid[0] == 512 < (N + 31) // 32
+        else:
+            d.grid[0] = grid
+        for name in ("q", "scale"):
+            d.arg(name).kind = iu8.ARG_NULL_BUFFER
+        ctx.launch(d, dict(x=x.data_ptr(), w=wf.data_ptr(), ws=ws.data_ptr(), c=c.data_ptr()))
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(host_u16(c), r["C"])
+    d.grid[0] = 1                                  # more than 8 blocks a workgroup: refused on the host
+    if (N + 31) // 32 > 8:
+        with pytest.raises(iu8.IU8Error) as e:
+            ctx.launch(d, dict(x=x.data_ptr(), w=wf.data_ptr(), ws=ws.data_ptr(), c=c.data_ptr()))
+        assert e.value.code == iu8.E_RULE
+
+
 def test_fused_form_refuses_what_it_does_not_hold(ctx):
     assert not iu8.fused_holds(5, 1024) and not iu8.fused_holds(2, 17408) and not iu8.fused_holds(4, 5248)
     assert iu8.fused_holds(1, 17408) and iu8.fused_holds(4, 5120) and iu8.fused_holds(2, 10240)
