@@ -342,6 +342,53 @@ int saber_iu8_moe_combine(saber_iu8_ctx *ctx, const void *y_bf16, const saber_iu
  * parity suite compares it with the host formula for all 65,536 inputs. */
 int saber_iu8_silu_table(saber_iu8_ctx *ctx, void *out_u16, void *stream);
 
+/* ---- tier packs ("SBRPACK1"): reading the iu8 records of a built pack ------------------------------
+ * The byte layout of include/saber_abi.h:541-944 and the open-time rules of
+ * crates/saber-mem/src/pack/{format,reader}.rs (PackReader::open_with / open_expecting): magic,
+ * format version 1..2, 256-byte header, 160-byte records sorted by 4096-aligned data_off, lengths
+ * implied by shape and dtype, name prefixes, the chunk-digest blob, the table hash last, and the plan
+ * hash when one is expected. Refusals: SABER_IU8_E_PARSE (malformed), SABER_IU8_E_VALIDATE (a hash
+ * does not match), SABER_IU8_E_IO. */
+typedef struct saber_iu8_pack saber_iu8_pack;
+typedef struct {
+  uint32_t format_version, record_count, tp_size, rank, chunk_bytes;
+  uint64_t data_off, file_bytes, build_unix_seconds;
+  uint8_t plan_hash[32], tier_id[32];
+} saber_iu8_pack_header;
+typedef struct {
+  char name[128];       /* the checkpoint's tensor name, NUL-terminated here */
+  uint32_t rank, layout_id, flags;
+  uint16_t dtype;       /* saber_pack_dtype tag */
+  uint8_t ndim, shard_kind;
+  uint64_t data_off, length, shape[8];
+  uint8_t sha256[32];
+} saber_iu8_pack_record;
+typedef struct {
+  int wkind;            /* SABER_IU8_W4: `<op>.wi4` layout 17; SABER_IU8_W8: `<op>.wi8` layout 18 */
+  uint32_t n, k, w_record, s_record;
+  uint64_t w_bytes;     /* N*K/2 or N*K */
+  uint8_t shard_kind;
+} saber_iu8_pack_linear_info;
+
+/* expected_plan_hash: 32 bytes, or NULL to open without the plan check. */
+int saber_iu8_pack_open(const char *path, const uint8_t *expected_plan_hash, saber_iu8_pack **out);
+void saber_iu8_pack_close(saber_iu8_pack *pack);
+int saber_iu8_pack_info(const saber_iu8_pack *pack, saber_iu8_pack_header *out);
+int saber_iu8_pack_record_at(const saber_iu8_pack *pack, uint32_t index, saber_iu8_pack_record *out);
+/* Index of the record of that name, or -1. */
+int saber_iu8_pack_find(const saber_iu8_pack *pack, const char *name);
+/* One record's payload (exactly `length` bytes) into dst, verified against its sha256 and its chunk
+ * digests where the pack carries them: a bad record is a load error, not a garbage weight. */
+int saber_iu8_pack_read(saber_iu8_pack *pack, uint32_t index, void *dst, uint64_t cap);
+/* The two records of an iu8 GEMM op (crates/saber-model/src/graph.rs:3848-3914): codes in the gfx12
+ * W-fragment order (`<op>.wi4` layout 17 U8 [N/16, K*8] or `<op>.wi8` layout 18 U8 [N/16, K*16]) and
+ * the f32 row scale (`<op>.wi4s` / `<op>.wi8s`, layout 19 [N]). */
+int saber_iu8_pack_linear(const saber_iu8_pack *pack, const char *op, saber_iu8_pack_linear_info *out);
+/* Read + verify + repack offline into the gfx950 fragment order (layout ids 33 / 34): w_gfx950 host
+ * memory of w_bytes, w_scale of n floats. */
+int saber_iu8_pack_load_linear(saber_iu8_pack *pack, const char *op, uint8_t *w_gfx950, uint64_t w_cap, float *w_scale,
+                               uint64_t ws_cap);
+
 #ifdef __cplusplus
 }
 #endif

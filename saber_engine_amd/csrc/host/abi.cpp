@@ -78,7 +78,7 @@ const Signature *signature_for(const std::string &k) {
   if (starts(k, "macaq_i8_quant_")) return &SIG_QUANT;
   if (starts(k, "macaq_i8_silu_mul_quant_")) return &SIG_SILU;
   if (k == "macaq_silu_bf16_table") return &SIG_TABLE;
-  if (k == "iu8_probe_read" || k == "iu8_probe_mfma32d") return &SIG_PROBE_READ;
+  if (k == "iu8_probe_read" || k == "iu8_probe_mfma32d" || k == "iu8_probe_first") return &SIG_PROBE_READ;
   if (k == "iu8_probe_copy") return &SIG_PROBE_COPY;
   if (k == "iu8_probe_empty") return &SIG_PROBE_EMPTY;
   if (k == "iu8_probe_mfma" || k == "iu8_probe_mfma32") return &SIG_PROBE_MFMA;

@@ -73,8 +73,26 @@ void sha_block(uint32_t h[8], const uint8_t *p) {
 }
 }  // namespace
 
+static void sha256_words(const uint8_t *data, size_t len, uint32_t h[8]);
+
+void sha256(const uint8_t *data, size_t len, uint8_t out[32]) {
+  uint32_t h[8];
+  sha256_words(data, len, h);
+  for (int k = 0; k < 8; ++k)
+    for (int b = 0; b < 4; ++b) out[4 * k + b] = (uint8_t)(h[k] >> (24 - 8 * b));
+}
+
 std::string sha256_hex(const uint8_t *data, size_t len) {
-  uint32_t h[8] = {0x6a09e667, 0xbb67ae85, 0x3c6ef372, 0xa54ff53a, 0x510e527f, 0x9b05688c, 0x1f83d9ab, 0x5be0cd19};
+  uint32_t h[8];
+  sha256_words(data, len, h);
+  char out[65];
+  for (int k = 0; k < 8; ++k) snprintf(out + 8 * k, 9, "%08x", h[k]);
+  return out;
+}
+
+static void sha256_words(const uint8_t *data, size_t len, uint32_t h[8]) {
+  static const uint32_t H0[8] = {0x6a09e667, 0xbb67ae85, 0x3c6ef372, 0xa54ff53a, 0x510e527f, 0x9b05688c, 0x1f83d9ab, 0x5be0cd19};
+  memcpy(h, H0, sizeof H0);
   size_t i = 0;
   for (; i + 64 <= len; i += 64) sha_block(h, data + i);
   uint8_t tail[128] = {0};
@@ -86,9 +104,6 @@ std::string sha256_hex(const uint8_t *data, size_t len) {
   for (int b = 0; b < 8; ++b) tail[tl - 1 - b] = (uint8_t)(bits >> (8 * b));
   sha_block(h, tail);
   if (tl == 128) sha_block(h, tail + 64);
-  char out[65];
-  for (int k = 0; k < 8; ++k) snprintf(out + 8 * k, 9, "%08x", h[k]);
-  return out;
 }
 
 }  // namespace iu8

@@ -17,6 +17,7 @@ bool read_file(const std::string &path, std::vector<uint8_t> &out);
 bool write_file(const std::string &path, const std::string &text);
 
 std::string sha256_hex(const uint8_t *data, size_t len);
+void sha256(const uint8_t *data, size_t len, uint8_t out[32]);
 
 std::string fmt(const char *f, ...) __attribute__((format(printf, 1, 2)));
 

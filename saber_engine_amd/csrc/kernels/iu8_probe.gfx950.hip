@@ -105,3 +105,25 @@ extern "C" __global__ __launch_bounds__(256) void iu8_probe_mfma32d(const unsign
       for (int e = 0; e < 16; ++e) s ^= c[i][j][e];
   if (s == 0x12345679) out[0] = s;
 }
+
+// What a launch pays before its first bytes: every wave stamps the 100 MHz constant clock at its
+// start and after each of n dependent 1 KiB wave-loads (16 bytes a lane, nontemporal, one in flight
+// at a time) of its own region of src; lane 0 stores the n + 1 stamps to out[(wave id) * (n + 1) ...]
+// as 64-bit values. The first interval holds the start-of-kernel cost on top of the memory latency
+// the later intervals show.
+extern "C" __global__ __launch_bounds__(512) void iu8_probe_first(const unsigned char *__restrict__ src,
+                                                                  unsigned *__restrict__ out, int n) {
+  const int wave = (int)blockIdx.x * 8 + (int)(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  unsigned long long *o = (unsigned long long *)out + (size_t)wave * (n + 1);
+  unsigned long long t = __builtin_amdgcn_s_memrealtime();
+  if (lane == 0) o[0] = t;
+  const unsigned char *p = src + ((size_t)wave * n) * 1024 + lane * 16;
+  for (int r = 0; r < n; ++r) {
+    iu8_v4u v;
+    const unsigned char *q = p + (size_t)r * 1024;
+    // load and wait in one volatile statement, so the stamp that follows is taken after the data
+    asm volatile("global_load_dwordx4 %0, %1, off nt\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(q) : "memory");
+    t = __builtin_amdgcn_s_memrealtime() + (v.x == 0x9E3779B9u && v.y == 1u);
+    if (lane == 0) o[r + 1] = t;
+  }
+}
