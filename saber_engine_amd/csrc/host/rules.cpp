@@ -10,7 +10,7 @@ namespace iu8 {
 
 static const DecVariant DEC_VARIANTS[] = {
 #define IU8_DEC_VARIANT(name, TM, W8, NT, KW, WPB, D, ALDS, ACC) {#name, TM, W8, NT, KW, WPB, D, ALDS, ACC},
-#define IU8_PF_VARIANT(name, W8, WMW, WNW, TM, TN, ACC, ST, OCC)
+#define IU8_PF_VARIANT(name, W8, WMW, WNW, TM, TN, ACC, ST, OCC, DEEP)
 #define IU8_PAIR_VARIANT(name, TM, NT, KW, WPB, D, ALDS)
 #include "../kernels/iu8_variants.def"
 #undef IU8_DEC_VARIANT
@@ -19,7 +19,7 @@ static const DecVariant DEC_VARIANTS[] = {
 };
 static const PfVariant PF_VARIANTS[] = {
 #define IU8_DEC_VARIANT(name, TM, W8, NT, KW, WPB, D, ALDS, ACC)
-#define IU8_PF_VARIANT(name, W8, WMW, WNW, TM, TN, ACC, ST, OCC) {#name, W8, WMW, WNW, TM, TN, ACC, OCC},
+#define IU8_PF_VARIANT(name, W8, WMW, WNW, TM, TN, ACC, ST, OCC, DEEP) {#name, W8, WMW, WNW, TM, TN, ACC, OCC},
 #define IU8_PAIR_VARIANT(name, TM, NT, KW, WPB, D, ALDS)
 #include "../kernels/iu8_variants.def"
 #undef IU8_DEC_VARIANT
@@ -28,7 +28,7 @@ static const PfVariant PF_VARIANTS[] = {
 };
 static const DecVariant PAIR_VARIANTS[] = {
 #define IU8_DEC_VARIANT(name, TM, W8, NT, KW, WPB, D, ALDS, ACC)
-#define IU8_PF_VARIANT(name, W8, WMW, WNW, TM, TN, ACC, ST, OCC)
+#define IU8_PF_VARIANT(name, W8, WMW, WNW, TM, TN, ACC, ST, OCC, DEEP)
 #define IU8_PAIR_VARIANT(name, TM, NT, KW, WPB, D, ALDS) {#name, TM, false, NT, KW, WPB, D, ALDS, false},
 #include "../kernels/iu8_variants.def"
 #undef IU8_DEC_VARIANT
@@ -235,7 +235,11 @@ int resolve(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *out) 
   if (wkind != SABER_IU8_W4 && wkind != SABER_IU8_W8) return fail(SABER_IU8_E_ARG, "unknown weight kind");
   const char *tag = wkind == SABER_IU8_W8 ? "w8" : "w4";
   if (int rc = check_shape(wkind == SABER_IU8_W8 ? "gemm_i8a8" : "gemm_i4a8", m, n, k)) return rc;
-  if (m <= DECODE_MAX_M) {
+  // The decode band ends where the tile GEMM's small cells overtake the streaming form (speed data of
+  // this card: 17..32 rows stream unless the output is very wide, 33..48 unless it is wide, from 49
+  // rows the tiles win on every shape measured).
+  const bool stream = m <= 16 || (m <= 32 && n <= 16384) || (m <= 48 && n <= 8192);
+  if (m <= DECODE_MAX_M && stream) {
     const uint32_t tm = (m + 15) / 16;
     std::string name = fmt("macaq_iu8_dec_%s_tm%u", tag, tm);
     if (tm == 1) {
@@ -253,25 +257,37 @@ int resolve(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *out) 
   return describe_pf(*pf_cell(wkind == SABER_IU8_W8, m, n, k), m, n, k, out);
 }
 
-// The prefill cell of a shape: the tile whose estimated time is least. A cell's time is its tile
-// work over its measured rate (relative to the 256 x 256 cell) times the rounds the card's 256 CUs
-// need; a partly filled last round counts half, because the card is power-bound under MFMA load and
-// the CUs that do run then clock higher. The rates are this card's speed data (M = 256..8192 sweeps
-// of the four 27B-class shapes), as the reference keeps its band tables
-// (crates/saber-kernels/src/macaq_iu8.rs:150-212).
+// The prefill cell of a shape: the tile whose estimated time is least. A launch's time is a fixed
+// cost plus the largest of three: the matrix work of the busiest CU over the cell's measured rate
+// (co-resident workgroups of a two-a-CU cell share the CU's matrix units), the bytes that CU pulls in
+// (its tiles' A rows and W columns, K deep) over what one CU takes from L2, and all tiles' bytes over
+// what the L2s deliver together -- the last two are what bind for M up to about 512, where the A rows
+// are re-read once a column block, so small tiles that put every CU to work win there and the large
+// ones take over as the matrix work grows. The constants are this card's speed data (least-squares fit
+// of 520 timings: the four 27B-class shapes x M = 65..8192 x ten cells; the picked cell is within 2 %
+// of the best measured one on 47 of the 52 shapes and within 13 % on all), as the reference keeps its
+// band tables (crates/saber-kernels/src/macaq_iu8.rs:150-212).
 const PfVariant *pf_cell(bool w8, uint32_t m, uint32_t n, uint32_t k) {
-  (void)k;
-  static const struct { const char *tile; double rate; } CELLS[] = {
-      {"tn4_lbk64", 1.00}, {"t256x224", 0.92}, {"t256x160", 0.88}, {"t128x128", 0.75}, {"t128x64_o2", 0.55}};
+  static const struct { const char *tile; double tops_per_cu; } CELLS[] = {
+      {"tn4_lbk64", 13.27}, {"t256x224", 11.27}, {"t256x160", 9.98}, {"t128x128", 7.85},
+      {"t128x128_o2", 8.68}, {"t128x64_s", 6.21}, {"t64x128_s", 7.24}, {"t64x64_s", 5.96}};
+  constexpr double FIXED_US = 2.78, CU_GBPS = 90.0, L2_TBPS = 17.7;
   const PfVariant *best = nullptr;
   double best_t = 0;
   for (const auto &c : CELLS) {
     const PfVariant *v = pf_variant(fmt("macaq_iu8_pf_%s_%s", w8 ? "w8" : "w4", c.tile));
     if (!v) continue;
-    const double tiles = (double)((n + v->block_n() - 1) / v->block_n()) * ((m + v->block_m() - 1) / v->block_m());
-    const double full = tiles / CU_COUNT, rounds = full + 0.5 * (std::ceil(full) - full);
-    const double t = rounds * v->block_m() * v->block_n() / c.rate;
-    if (!best || t < best_t * 0.97) best = v, best_t = t;  // a later (smaller) cell must win clearly
+    const double bm = v->block_m(), bn = v->block_n();
+    const uint64_t tiles = (uint64_t)((n + v->block_n() - 1) / v->block_n()) * ((m + v->block_m() - 1) / v->block_m());
+    const uint64_t grid = std::min<uint64_t>(tiles, (uint64_t)CU_COUNT * v->occ);
+    const uint64_t per_wg = (tiles + grid - 1) / grid;
+    const double cu_tiles = (double)per_wg * std::min<uint64_t>(v->occ, (grid + CU_COUNT - 1) / CU_COUNT);
+    const double tile_bytes = bm * k + bn * k * (w8 ? 1.0 : 0.5);
+    const double t_mfma = cu_tiles * bm * bn * k * 2.0 / (c.tops_per_cu * 1e6);
+    const double t_cu = cu_tiles * tile_bytes / (CU_GBPS * 1e3);
+    const double t_l2 = (double)tiles * tile_bytes / (L2_TBPS * 1e6);
+    const double t = FIXED_US + std::max(t_mfma, std::max(t_cu, t_l2));
+    if (!best || t < best_t) best = v, best_t = t;
   }
   return best;
 }

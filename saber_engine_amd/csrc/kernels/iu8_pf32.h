@@ -17,6 +17,13 @@
 // c = 4*kt2 + 2*p + h. A lane's 16-byte W4 piece then holds the operands of sub-steps 2p (dwords
 // 0,1) and 2p+1 (dwords 2,3), so one LDS read serves two sub-steps.
 //
+// DEEP (small wave tiles). With TM*TN MFMAs a sub-step there is too little matrix work between an
+// LDS read and its use to hide the read, and a lone workgroup a CU has no other wave to run. The
+// deep form reads the operands of a whole K step (all four sub-steps) into registers one step
+// ahead of its MFMAs, double-buffered a step: one barrier a step at its top, behind it the loads
+// for NST-1 steps ahead leave, the next step's operands are read from its stage and this step's
+// MFMAs run from registers filled a step ago.
+//
 // D[n][m]: src0 = weight operand (lane: row n = l%32), src1 = activation operand (lane: row
 // m = l%32); lane l, register e holds n = 8*(e/4) + 4*(l/32) + e%4, m = l%32.
 #pragma once
@@ -59,7 +66,7 @@ static __device__ __forceinline__ bool iu8_dense_tile_at(int r, int gx, int gy, 
   return true;
 }
 
-template <bool W8, int WMW, int WNW, int TM, int TN, bool ACC, int STMAX, class TileAt>
+template <bool W8, int WMW, int WNW, int TM, int TN, bool ACC, int STMAX, bool DEEP = false, class TileAt>
 __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const float *__restrict__ as,
                                              void *__restrict__ Cv, int N, int K, TileAt tile_at) {
   // tile_at(r, t): fills the workgroup's r-th tile, false when it has none
@@ -71,7 +78,11 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
   constexpr int A_FR = A_BYTES / 1024, W_FR = W_BYTES / 1024;
   constexpr int A_PER = (A_FR + NWAVE - 1) / NWAVE, W_PER = (W_FR + NWAVE - 1) / NWAVE;
   constexpr int PER = A_FR / NWAVE + W_FR / NWAVE;  // wave-loads every wave issues a step (some issue one more)
-  constexpr int NST = STMAX >= 3 && 3 * STAGE <= 160 * 1024 ? 3 : 2;
+  // as many stages as asked for and as fit the 160 KiB of LDS, at least two
+  constexpr int NFIT = 160 * 1024 / STAGE;
+  constexpr int NST = STMAX < 2 ? 2 : (STMAX < NFIT ? STMAX : (NFIT < 2 ? 2 : NFIT));
+  static_assert((NST - 2) * (A_FR / NWAVE + W_FR / NWAVE) <= 63, "the in-flight count fits s_waitcnt's vmcnt field");
+  static_assert(!DEEP || NST >= 3, "the deep form reads a stage a step ahead of its MFMAs");
   __shared__ __attribute__((aligned(1024))) iu8_u8 smem[NST * STAGE];
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -215,17 +226,45 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
   }                                                   \
   __builtin_amdgcn_sched_barrier(0)
 
-  issue(0);
-  advance();
-  if constexpr (NST == 3) {
-    issue(1);
+#pragma unroll
+  for (int s0 = 0; s0 < NST - 1; ++s0) {
+    issue(s0);
     advance();
   }
   wait_vm(InFlight{}, false);
   __builtin_amdgcn_s_barrier();
-  fetch_a(smem, 0, 0, 0);
-  fetch_w8(smem + A_BYTES, 0, 0, 0);
-  fetch_w4(smem + A_BYTES, 0);
+  // deep form: register sets of one whole step, [set][sub-step f = 2p + kt2]
+  iu8_v4i afd[DEEP ? 2 : 1][DEEP ? 4 : 1][TM] = {};
+  iu8_v4i wfd[DEEP && W8 ? 2 : 1][DEEP && W8 ? 4 : 1][TN] = {};
+  iu8_v4u wpd[DEEP && !W8 ? 2 : 1][DEEP && !W8 ? 2 : 1][TN] = {};
+  auto fetch_step = [&](const iu8_u8 *sA, int set) {  // all operands of the step in stage sA
+    const iu8_u8 *sW = sA + A_BYTES;
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {
+#pragma unroll
+      for (int kt2 = 0; kt2 < 2; ++kt2) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+          afd[set][2 * p + kt2][i] = *(const iu8_v4i *)&sA[a_lane + i * 4096 + kt2 * 1024 + p * 512];
+        if constexpr (W8) {
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+            wfd[set][2 * p + kt2][j] = *(const iu8_v4i *)&sW[w_lane + j * 4096 + kt2 * 1024 + p * 512];
+        }
+      }
+      if constexpr (!W8) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) wpd[set][p][j] = *(const iu8_v4u *)&sW[w_lane + j * 2048 + p * 512];
+      }
+    }
+  };
+  if constexpr (DEEP) {
+    fetch_step(smem, 0);
+  } else {
+    fetch_a(smem, 0, 0, 0);
+    fetch_w8(smem + A_BYTES, 0, 0, 0);
+    fetch_w4(smem + A_BYTES, 0);
+  }
   __builtin_amdgcn_sched_barrier(0);
 
   iu8_tile C = L;
@@ -239,6 +278,65 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
 
+    if constexpr (DEEP) {
+      auto mfma_step = [&](int set) {
+#pragma unroll
+        for (int p = 0; p < 2; ++p)
+#pragma unroll
+          for (int kt2 = 0; kt2 < 2; ++kt2)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+              iu8_v4i wv;
+              if constexpr (W8) {
+                wv = wfd[set][2 * p + kt2][j];
+              } else {
+                const unsigned d0 = kt2 ? wpd[set][p][j].z : wpd[set][p][j].x, d1 = kt2 ? wpd[set][p][j].w : wpd[set][p][j].y;
+                wv = iu8_v4i{(int)((d0 << 4) & 0xF0F0F0F0u), (int)(d0 & 0xF0F0F0F0u), (int)((d1 << 4) & 0xF0F0F0F0u),
+                             (int)(d1 & 0xF0F0F0F0u)};
+              }
+#pragma unroll
+              for (int i = 0; i < TM; ++i)
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wv, afd[set][2 * p + kt2][i], acc[i][j], 0, 0, 0);
+            }
+      };
+      auto deep_step = [&](int set) {  // the MFMAs of the step in register set `set`; the next step's into the other
+        const int st1 = st == NST - 1 ? 0 : st + 1, stl = st == 0 ? NST - 1 : st - 1;
+        // The stage of the step before this one was read two steps ago (the last barrier vouches for
+        // every wave), so the loads for NST-1 steps ahead leave first; then the next step's fragments
+        // must have landed: all but the newest NST-2 steps' loads.
+        issue(stl);
+        advance();
+        wait_vm(InFlight{}, true);
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        fetch_step(smem + st1 * STAGE, set ^ 1);
+        mfma_step(set);
+        st = st1;
+      };
+      int s = 0;
+      for (; s + 2 <= steps; s += 2) {
+        deep_step(0);
+        deep_step(1);
+      }
+      if (s < steps) {  // an odd step count: one more step, then the sets are renamed back
+        deep_step(0);
+#pragma unroll
+        for (int f = 0; f < 4; ++f) {
+#pragma unroll
+          for (int i = 0; i < TM; ++i) afd[0][f][i] = afd[1][f][i];
+          if constexpr (W8) {
+#pragma unroll
+            for (int j = 0; j < TN; ++j) wfd[0][f][j] = wfd[1][f][j];
+          }
+        }
+        if constexpr (!W8) {
+#pragma unroll
+          for (int p = 0; p < 2; ++p)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) wpd[0][p][j] = wpd[1][p][j];
+        }
+      }
+    } else
     for (int s = 0; s < steps; ++s) {
       const int st1 = st == NST - 1 ? 0 : st + 1, stl = st == 0 ? NST - 1 : st - 1;  // next, last
       const iu8_u8 *sA = smem + st * STAGE, *sW = sA + A_BYTES;

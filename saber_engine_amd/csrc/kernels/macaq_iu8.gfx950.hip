@@ -36,7 +36,7 @@
                                                     iu8_rows{nullptr, 0, m}, n, k);     \
   }
 #define IU8_DEC_VARIANT(name, TM, W8, NT, KW, WPB, D, ALDS, ACC) IU8_DEC(name, TM, W8, NT, KW, WPB, D, ALDS, ACC)
-#define IU8_PF_VARIANT(name, W8, WMW, WNW, TM, TN, ACC, ST, OCC)
+#define IU8_PF_VARIANT(name, W8, WMW, WNW, TM, TN, ACC, ST, OCC, DEEP)
 #define IU8_PAIR_VARIANT(name, TM, NT, KW, WPB, D, ALDS)
 #include "iu8_variants.def"
 #undef IU8_DEC_VARIANT
@@ -65,7 +65,7 @@ IU8_DECQ(macaq_iu8_decq_w8_tm1, true, 4)
 #undef IU8_DECQX
 
 // Persistent launch: gridDim.x workgroups (one or OCC a CU) walk the tiles of the m x n output.
-#define IU8_PF32(name, W8, WMW, WNW, TM, TN, ACC, ST, OCC)                                                        \
+#define IU8_PF32(name, W8, WMW, WNW, TM, TN, ACC, ST, OCC, DEEP)                                                        \
   extern "C" __global__ __launch_bounds__(WMW * WNW * 64)                                                         \
       __attribute__((amdgpu_waves_per_eu(WMW * WNW * OCC / 4, WMW * WNW * OCC / 4))) void name(                    \
       const unsigned char *__restrict__ a, const unsigned char *__restrict__ w, const float *__restrict__ as,     \
@@ -73,7 +73,7 @@ IU8_DECQ(macaq_iu8_decq_w8_tm1, true, 4)
     constexpr int BM = WMW * TM * 32, BN = WNW * TN * 32;                                                          \
     const int gx = (n + BN - 1) / BN, gy = (m + BM - 1) / BM;                                                      \
     const iu8_rows R{nullptr, 0, m};                                                                               \
-    iu8_pf32_run<W8, WMW, WNW, TM, TN, ACC, ST>(a, as, c, n, k, [&](int r, iu8_tile &t) {                          \
+    iu8_pf32_run<W8, WMW, WNW, TM, TN, ACC, ST, DEEP>(a, as, c, n, k, [&](int r, iu8_tile &t) {                          \
       int bx, by;                                                                                                  \
       if (!iu8_dense_tile_at(r, gx, gy, bx, by)) return false;                                                     \
       t = iu8_tile{R, by * BM, bx * (BN / 16), w, ws};                                                             \
@@ -81,7 +81,7 @@ IU8_DECQ(macaq_iu8_decq_w8_tm1, true, 4)
     });                                                                                                            \
   }
 #define IU8_DEC_VARIANT(name, TM, W8, NT, KW, WPB, D, ALDS, ACC)
-#define IU8_PF_VARIANT(name, W8, WMW, WNW, TM, TN, ACC, ST, OCC) IU8_PF32(name, W8, WMW, WNW, TM, TN, ACC, ST, OCC)
+#define IU8_PF_VARIANT(name, W8, WMW, WNW, TM, TN, ACC, ST, OCC, DEEP) IU8_PF32(name, W8, WMW, WNW, TM, TN, ACC, ST, OCC, DEEP)
 #define IU8_PAIR_VARIANT(name, TM, NT, KW, WPB, D, ALDS)
 #include "iu8_variants.def"
 #undef IU8_DEC_VARIANT

@@ -27,7 +27,7 @@
         iu8_blk{bl % nbp, bl / nbp, p1 ? ks_b : ks});                                                               \
   }
 #define IU8_DEC_VARIANT(name, TM, W8, NT, KW, WPB, D, ALDS, ACC)
-#define IU8_PF_VARIANT(name, W8, WMW, WNW, TM, TN, ACC, ST, OCC)
+#define IU8_PF_VARIANT(name, W8, WMW, WNW, TM, TN, ACC, ST, OCC, DEEP)
 #define IU8_PAIR_VARIANT(name, TM, NT, KW, WPB, D, ALDS) IU8F_PAIR(name, TM, NT, KW, WPB, D, ALDS)
 #include "iu8_variants.def"
 #undef IU8_DEC_VARIANT

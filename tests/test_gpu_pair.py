@@ -21,7 +21,7 @@ def halves(rng, M, K, n0, n1):
 # GDN's in_proj_qkvz + in_proj_ba at hidden 5120 (the reference's pair), ragged column blocks, each
 # row tiling (tm1 staged and streamed, tm2..tm4), a long K
 @pytest.mark.parametrize("M,K,n0,n1", [(1, 5120, 12288, 96), (4, 5120, 1040, 48), (16, 5120, 272, 528), (8, 17408, 320, 64),
-                                       (20, 1024, 144, 32), (40, 640, 80, 304), (64, 512, 64, 64)])
+                                       (20, 1024, 144, 32), (40, 640, 80, 304), (48, 512, 64, 64)])
 def test_pair_matches_the_oracle_and_two_launches(ctx, M, K, n0, n1):
     say(f"pair M={M} K={K} N={n0}+{n1}")
     rng = np.random.default_rng(M * 7 + n0)
@@ -44,6 +44,35 @@ def test_pair_matches_the_oracle_and_two_launches(ctx, M, K, n0, n1):
     r1 = ref.linear(X, W1, ws1, False, threads=8)
     np.testing.assert_array_equal(host_u16(c0), r0["C"])
     np.testing.assert_array_equal(host_u16(c1), r1["C"])
+
+
+def test_pair_of_named_cells_past_the_streaming_band(ctx):
+    """From 49 rows the launch law hands a linear to the tile GEMM, which does not pair (refused by name);
+    the four-tile streaming cell still pairs when it is named."""
+    say("pair of named tm4 cells, M=64")
+    M, K, n0, n1 = 64, 512, 80, 48
+    rng = np.random.default_rng(64)
+    X, (W0, ws0), (W1, ws1) = halves(rng, M, K, n0, n1)
+    xd = dev_bf16_bits(X)
+    q = torch.zeros(iu8.a_bytes(M, K), dtype=torch.uint8, device="cuda")
+    s = torch.zeros(M, dtype=torch.float32, device="cuda")
+    ctx.quant(xd.data_ptr(), q.data_ptr(), s.data_ptr(), M, K)
+    w0, w1, s0, s1 = dev_u8(iu8.repack_w4(W0)), dev_u8(iu8.repack_w4(W1)), dev_f32(ws0), dev_f32(ws1)
+    c0 = torch.full((M, n0), 0x7FC0, dtype=torch.int16, device="cuda")
+    c1 = torch.full((M, n1), 0x7FC0, dtype=torch.int16, device="cuda")
+    with pytest.raises(iu8.IU8Error) as e:
+        ctx.gemm_pair(q.data_ptr(), s.data_ptr(), w0.data_ptr(), s0.data_ptr(), c0.data_ptr(), n0,
+                      w1.data_ptr(), s1.data_ptr(), c1.data_ptr(), n1, M, K)
+    assert e.value.code == iu8.E_RULE
+    d = iu8.pair(iu8.describe("macaq_iu8_dec_w4_tm4", M, n0, K), iu8.describe("macaq_iu8_dec_w4_tm4", M, n1, K))
+    assert d.kernel == b"macaq_iu8f_pair_w4_tm4"
+    bufs = dict(a=q.data_ptr(), w=w0.data_ptr(), ws=s0.data_ptr(), c=c0.data_ptr(), w_b=w1.data_ptr(), ws_b=s1.data_ptr(),
+                c_b=c1.data_ptr())
+    bufs["as"] = s.data_ptr()
+    ctx.launch(d, bufs)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(host_u16(c0), ref.linear(X, W0, ws0, False)["C"])
+    np.testing.assert_array_equal(host_u16(c1), ref.linear(X, W1, ws1, False)["C"])
 
 
 def test_pair_with_explicitly_split_halves(ctx):

@@ -63,14 +63,19 @@ def test_resolve_refuses_by_name():
 
 @pytest.mark.parametrize("wk,tag", [(iu8.W4, "w4"), (iu8.W8, "w8")])
 def test_decode_band_routing(wk, tag):
-    for m in (1, 4, 8, 16, 17, 32, 33, 48, 49, 64):
+    for m in (1, 4, 8, 16, 17, 32, 33, 48):
         d = iu8.resolve(wk, m, 5120, 5120)
         tm = (m + 15) // 16
         assert d.kernel.decode().startswith(f"macaq_iu8_dec_{tag}_tm{tm}")
         assert d.ks == 1 and d.grid[2] == 1 and d.n_workspaces == 0
         assert d.arg("decode_partial").kind == iu8.ARG_NULL_BUFFER and d.arg("decode_counter").kind == iu8.ARG_NULL_BUFFER
         assert d.grid[0] * (d.block[0] // 64) >= 5120 // 16 // 4       # the grid covers every 16-column tile
-    assert iu8.resolve(wk, 65, 5120, 5120).kernel.decode().startswith(f"macaq_iu8_pf_{tag}")
+    # the tile GEMM's small cells take over from 49 rows, earlier on wide outputs; the streaming forms
+    # stay reachable by name up to 64 rows
+    for (m, n) in [(49, 5120), (64, 5120), (65, 5120), (33, 34816), (17, 34816)]:
+        assert iu8.resolve(wk, m, n, 5120).kernel.decode().startswith(f"macaq_iu8_pf_{tag}"), (m, n)
+    assert iu8.resolve(wk, 16, 34816, 5120).kernel.decode().startswith(f"macaq_iu8_dec_{tag}_tm1")
+    assert iu8.describe(f"macaq_iu8_dec_{tag}_tm4", 64, 5120, 5120).grid[0] > 0
 
 
 def test_activation_rows_are_staged_when_they_fit():
@@ -132,7 +137,8 @@ def test_explicit_split_declares_its_workspaces():
 
 PF_CELLS = {  # tile suffix -> (rows, columns, workgroups a CU, threads)
     "tn4_lbk64": (256, 256, 1, 512), "t256x224": (256, 224, 1, 512), "t256x160": (256, 160, 1, 512),
-    "t128x128": (128, 128, 1, 512), "t128x128_o2": (128, 128, 2, 256), "t128x64_o2": (128, 64, 2, 256)}
+    "t128x128": (128, 128, 1, 512), "t128x128_o2": (128, 128, 2, 256), "t128x64_o2": (128, 64, 2, 256),
+    "t128x64_s": (128, 64, 1, 256), "t64x128_s": (64, 128, 2, 256), "t64x64_s": (64, 64, 2, 256)}
 
 
 def test_prefill_launch_is_persistent_and_covers_the_output():
@@ -151,7 +157,10 @@ def test_prefill_launch_is_persistent_and_covers_the_output():
 def test_prefill_cells_of_the_benchmark_shapes():
     # speed data of this card: the cell that was fastest in the sweep of each shape
     want = {(2048, 34816, 5120): "tn4_lbk64", (2048, 7168, 5120): "tn4_lbk64", (2048, 5120, 17408): "t256x160",
-            (2048, 5120, 5120): "t256x160", (8192, 34816, 5120): "tn4_lbk64", (256, 5120, 17408): "t128x64_o2"}
+            (2048, 5120, 5120): "t256x160", (8192, 34816, 5120): "tn4_lbk64",
+            # up to M of about 512 the launch is bound by what the CUs pull from L2: small tiles on every CU
+            (256, 5120, 17408): "t64x128_s", (128, 5120, 17408): "t64x64_s", (256, 34816, 5120): "t256x160",
+            (1024, 5120, 5120): "t128x128_o2", (1024, 7168, 5120): "t128x128_o2"}
     for (m, n, k), tile in want.items():
         assert iu8.resolve(iu8.W4, m, n, k).kernel.decode() == "macaq_iu8_pf_w4_" + tile, (m, n, k)
     with pytest.raises(iu8.IU8Error):
