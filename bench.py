@@ -229,8 +229,7 @@ def main():
     # ---- the second half of the metric: int8 TOPS at M=2048 on the same four shapes. Activations are
     # the configuration's (bf16 N(0,1), 0.5 % of the channels x20), quantised by the producer kernel:
     # the operand values set the card's clock under MFMA load, so uniform random codes would misstate it.
-    if not args.no_prefill:
-        PM = 2048
+    def prefill_at(PM, warm, reps):
         pf = {}
         tot_ops, tot_us, tot_q_us = 0.0, 0.0, 0.0
         for name, n, k in linears:
@@ -241,21 +240,23 @@ def main():
             c = torch.zeros((PM, n), dtype=torch.int16, device=dev)
             qd = iu8.resolve_quant(PM, k)
             qb = dict(x=x.data_ptr(), q=q.data_ptr(), scale=a_s.data_ptr())
-            b = dict(a=q.data_ptr(), w=dev_w[name][0].data_ptr(), ws=dev_ws[name].data_ptr(), c=c.data_ptr())
-            b["as"] = a_s.data_ptr()
-            reps = 20
+            bs = []
+            for layer in range(LAYERS):     # successive launches walk the weight copies: cold weights here too
+                b = dict(a=q.data_ptr(), w=dev_w[name][layer].data_ptr(), ws=dev_ws[name].data_ptr(), c=c.data_ptr())
+                b["as"] = a_s.data_ptr()
+                bs.append(b)
             with torch.cuda.stream(stream):
                 for _ in range(3):
                     ctx.launch(qd, qb, sh)
-                for _ in range(40):  # tens of ms of MFMA load: the clock settles where it stays under this kernel
-                    ctx.launch(d, b, sh)
+                for i in range(warm):  # tens of ms of MFMA load: the clock settles where it stays under this kernel
+                    ctx.launch(d, bs[i % LAYERS], sh)
                 e0, e1, e2 = (torch.cuda.Event(enable_timing=True) for _ in range(3))
                 e0.record(stream)
                 for _ in range(reps):
                     ctx.launch(qd, qb, sh)
                 e1.record(stream)
-                for _ in range(reps):
-                    ctx.launch(d, b, sh)
+                for i in range(reps):
+                    ctx.launch(d, bs[i % LAYERS], sh)
                 e2.record(stream)
             torch.cuda.synchronize()
             q_us = e0.elapsed_time(e1) * 1e3 / reps
@@ -267,6 +268,10 @@ def main():
             tot_us += us
             tot_q_us += q_us
             del x, q, a_s, c
+        return pf, tot_ops, tot_us, tot_q_us
+
+    if not args.no_prefill:
+        pf, tot_ops, tot_us, tot_q_us = prefill_at(2048, 40, 20)
         tops = tot_ops / tot_us / 1e6
         # what the matrix cores sustain on this card with such operands: the register-resident MFMA
         # loop of the probe object, fed zeros, codes like this workload's (small activations, 16*w
@@ -301,6 +306,17 @@ def main():
                                                   unit="POP/s", frac=round(tops / INT8_PEAK_TOPS, 4), traffic=None,
                                                   note="GEMM launches alone over the four shapes (ops = 2*M*N*K); "
                                                        "with_quant adds the int8 producer launches"))
+        # the other row counts of configs[2]: M = 256 sits near the ridge (both roofs reported: the weights'
+        # GB/s beside the TOPS), M = 8192 is the matrix-bound end
+        other = {}
+        for PM, warm, reps in ((256, 20, 20), (8192, 6, 6)):
+            pfm, ops_m, us_m, q_us_m = prefill_at(PM, warm, reps)
+            wbytes = sum(n * k // 2 for _, n, k in linears)
+            other["m%d" % PM] = dict(tops=round(ops_m / us_m / 1e6, 1), with_quant=round(ops_m / (us_m + q_us_m) / 1e6, 1),
+                                     weight_gbps=round(wbytes / us_m / 1e3, 1), mfma_frac=round(ops_m / us_m / 1e6 / INT8_PEAK_TOPS, 4),
+                                     hbm_frac=round(wbytes / us_m / 1e3 / HBM_PEAK_GBPS, 4),
+                                     per_linear={k_: dict(kernel=v["kernel"], us=v["us"], tops=v["tops"]) for k_, v in pfm.items()})
+        out["prefill_other_m"] = other
     # ---- the routed-expert layer of configs[4] (128 experts, top-8, hidden 4096, expert intermediate
     # 1536) as its launch train, T = 16 (weight streaming) and T = 4096 (MFMA); weights are random
     # nibbles generated on the device (parity of this path is the GPU tests' business)
