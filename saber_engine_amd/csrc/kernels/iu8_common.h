@@ -98,6 +98,22 @@ static __device__ __forceinline__ unsigned iu8_code4_rcp(float x0, float x1, flo
          __builtin_amdgcn_perm(__float_as_uint(u3), __float_as_uint(u2), 0x04000c0cu);
 }
 
+// Cross-workgroup hand-over without a cache flush. The card has one L2 per XCD, so a device-scope
+// release fence writes back and invalidates a whole L2 -- costly when every workgroup of a launch does
+// it. Data written with both scope bits set goes straight through to memory, and a load with both
+// set comes from there, so a producer that stores its data this way, waits for the stores' completion
+// (vmcnt) and then bumps a device-scope atomic, and a consumer that reads the atomic and then loads
+// this way, need no fence at all.
+static __device__ __forceinline__ void iu8_store_through(int *p, iu8_v4i v) {
+  asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" ::"v"(p), "v"(v) : "memory");
+}
+static __device__ __forceinline__ iu8_v4i iu8_load_through(const int *p) {
+  iu8_v4i v;
+  asm volatile("global_load_dwordx4 %0, %1, off sc0 sc1\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(p) : "memory");
+  return v;
+}
+static __device__ __forceinline__ void iu8_stores_done() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
 static __device__ __forceinline__ iu8_v4u iu8_ldg_nt(const iu8_u8 *p) {
   return __builtin_nontemporal_load((const iu8_v4u *)p);
 }

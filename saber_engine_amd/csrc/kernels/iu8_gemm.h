@@ -285,24 +285,21 @@ __device__ __forceinline__ void iu8_dec_body(const iu8_u8 *__restrict__ A, const
 #pragma unroll
       for (int i = 0; i < TM; ++i) {
         const int m = i * 16 + ml;
-        if (m < M) *(iu8_v4i *)&P[((size_t)z * M + m) * N + n] = acc[i][j];
+        if (m < M) iu8_store_through(&P[((size_t)z * M + m) * N + n], acc[i][j]);
       }
     }
+    iu8_stores_done();
   }
   __syncthreads();
-  if (tid == 0) {
-    __threadfence();
-    s_last = (atomicAdd(&cnt[B.bx], 1) == Z - 1);
-  }
+  if (tid == 0) s_last = (__hip_atomic_fetch_add(&cnt[B.bx], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == Z - 1);
   __syncthreads();
   if (!s_last) return;
-  __threadfence();
-  if (tid == 0) cnt[B.bx] = 0;
+  if (tid == 0) __hip_atomic_store(&cnt[B.bx], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   const int nb = B.bx * BN, nw4 = min(BN, N - nb) >> 2;
   for (int idx = tid; idx < nw4 * M; idx += NTHR) {
     const int m = idx / nw4, n = nb + (idx % nw4) * 4;
     iu8_v4i sum = iu8_v4i{0, 0, 0, 0};
-    for (int q = 0; q < Z; ++q) sum += __builtin_nontemporal_load((const iu8_v4i *)&P[((size_t)q * M + m) * N + n]);
+    for (int q = 0; q < Z; ++q) sum += iu8_load_through(&P[((size_t)q * M + m) * N + n]);
     const size_t crow = (size_t)(R.row0 + m) * N;
     if constexpr (ACC) {
       *(iu8_v4i *)((int *)Cv + crow + n) = sum;
