@@ -66,7 +66,7 @@ static bool starts(const std::string &s, const char *p) { return s.rfind(p, 0) =
 const Signature *signature_for(const std::string &k) {
   if (starts(k, "macaq_iu8_dec_")) return &SIG_DEC;
   if (starts(k, "macaq_iu8_decq_")) return &SIG_DECQ;
-  if (starts(k, "macaq_iu8_pf_")) return &SIG_PF;
+  if (starts(k, "macaq_iu8_pf_")) return k.size() > 3 && k.compare(k.size() - 3, 3, "_ks") == 0 ? &SIG_DEC : &SIG_PF;
   if (starts(k, "macaq_iu8f_pair_")) return &SIG_PAIR;
   if (starts(k, "add_rms_quant_hadi8_")) return &SIG_HAD_ARQ;
   if (starts(k, "silu_mul_quant_hadi8_")) return &SIG_HAD_SMQ;

@@ -112,9 +112,10 @@ static int check_shape(const char *op, uint32_t m, uint32_t n, uint32_t k) {
   return 0;
 }
 
-// The grid-level split of a decode GEMM. On this card a split costs device-scope fences across
-// the 8 XCDs' L2s (measured: 3-7x the unsplit kernel), and the k-waves of a workgroup already
-// split K through LDS, so the law does not split; `describe` still takes an explicit count.
+// The grid-level split of a decode GEMM. The k-waves of a workgroup already split K through LDS, and
+// a split across workgroups adds 1.5-2 us of hand-over (partials through memory, a device-scope
+// counter) to launches whose fixed cost dominates: measured on the 27B-class shapes it never wins
+// by more than the noise, so the law does not split; `describe` still takes an explicit count.
 uint32_t decode_split(uint32_t, uint32_t, uint32_t, uint32_t, uint32_t) { return 1; }
 
 static int describe_dec(const DecVariant &v, uint32_t m, uint32_t n, uint32_t k, uint32_t ks, saber_iu8_desc *d) {
@@ -146,33 +147,53 @@ static int describe_dec(const DecVariant &v, uint32_t m, uint32_t n, uint32_t k,
   return 0;
 }
 
-static int describe_pf(const PfVariant &v, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *d) {
+// `ks` > 0 names the cell's split form (`<cell>_ks`, the decode kernarg list): gridDim.z shares of the
+// K steps, none of them empty, `grid[0]` persistent workgroups a share.
+static int describe_pf(const PfVariant &v, uint32_t m, uint32_t n, uint32_t k, uint32_t ks, saber_iu8_desc *d) {
   const char *op = v.w8 ? "gemm_i8a8" : "gemm_i4a8";
   if (int rc = check_shape(op, m, n, k)) return rc;
+  const std::string name = std::string(v.name) + (ks ? "_ks" : "");
+  if (ks) {
+    const uint32_t steps = k / 128, spb = (steps + ks - 1) / ks;
+    if (ks > steps || (uint64_t)spb * (ks - 1) >= steps)
+      return fail(SABER_IU8_E_RULE, fmt("%s: %u shares of %u K steps would leave one empty", op, ks, steps));
+  }
   memset(d, 0, sizeof *d);
   copy_name(d->op, sizeof d->op, op);
   copy_name(d->plugin, sizeof d->plugin, "macaq_iu8");
-  copy_name(d->kernel, sizeof d->kernel, v.name);
+  copy_name(d->kernel, sizeof d->kernel, name);
   const uint32_t gx = (n + v.block_n() - 1) / v.block_n(), gy = (m + v.block_m() - 1) / v.block_m();
   // persistent: OCC workgroups a CU walk the tiles (the kernel derives gx, gy from m, n)
-  const uint64_t tiles = (uint64_t)gx * gy, slots = (uint64_t)CU_COUNT * v.occ;
-  d->grid[0] = (uint32_t)(tiles < slots ? tiles : slots), d->grid[1] = 1, d->grid[2] = 1;
+  const uint64_t tiles = (uint64_t)gx * gy, slots = std::max<uint64_t>(1, (uint64_t)CU_COUNT * v.occ / std::max(ks, 1u));
+  d->grid[0] = (uint32_t)(tiles < slots ? tiles : slots), d->grid[1] = 1, d->grid[2] = std::max(ks, 1u);
   d->block[0] = v.threads(), d->block[1] = 1, d->block[2] = 1;
   d->n_launches = 1;
-  d->ks = 1;
-  if (int rc = fill_slots(v.name, d)) return rc;
+  d->ks = std::max(ks, 1u);
+  if (int rc = fill_slots(name, d)) return rc;
   set_i32(d, "m", m);
   set_i32(d, "n", n);
   set_i32(d, "k", k);
+  if (ks == 1) {
+    set_null(d, "decode_partial");
+    set_null(d, "decode_counter");
+  } else if (ks > 1) {
+    add_ws(d, "decode_partial", SABER_IU8_WS_SCRATCH, (uint64_t)ks * m * n * 4, 0);
+    add_ws(d, "decode_counter", SABER_IU8_WS_PERSISTENT, tiles * 4, 1);
+  }
   return 0;
 }
 
 int describe(const std::string &kernel, uint32_t m, uint32_t n, uint32_t k, uint32_t ks, saber_iu8_desc *out) {
   if (const DecVariant *v = dec_variant(kernel)) return describe_dec(*v, m, n, k, ks, out);
   if (const PfVariant *v = pf_variant(kernel)) {
-    if (ks != 1) return fail(SABER_IU8_E_RULE, kernel + ": the prefill tile does not split K");
-    return describe_pf(*v, m, n, k, out);
+    if (ks != 1) return fail(SABER_IU8_E_RULE, kernel + ": the prefill tile does not split K (its `_ks` form does)");
+    return describe_pf(*v, m, n, k, 0, out);
   }
+  if (kernel.size() > 3 && kernel.compare(kernel.size() - 3, 3, "_ks") == 0)
+    if (const PfVariant *v = pf_variant(kernel.substr(0, kernel.size() - 3))) {
+      if (!signature_for(kernel)) return fail(SABER_IU8_E_RULE, kernel + ": no such split form");
+      return describe_pf(*v, m, n, k, ks, out);
+    }
   return fail(SABER_IU8_E_RULE, kernel + ": not a kernel of the macaq_iu8 object");
 }
 
@@ -254,7 +275,27 @@ int resolve(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *out) 
     const uint32_t nblk = (n + v->block_n() - 1) / v->block_n();
     return describe_dec(*v, m, n, k, decode_split(m, n, k, nblk, v->kw), out);
   }
-  return describe_pf(*pf_cell(wkind == SABER_IU8_W8, m, n, k), m, n, k, out);
+  const PfVariant *split_cell = nullptr;
+  if (const uint32_t ks = pf_split(wkind == SABER_IU8_W8, m, n, k, &split_cell))
+    return describe_pf(*split_cell, m, n, k, ks, out);
+  return describe_pf(*pf_cell(wkind == SABER_IU8_W8, m, n, k), m, n, k, 0, out);
+}
+
+// K shares of a tile launch (0: none). A deep, narrow linear at a few dozen rows gives the unsplit
+// law so few tiles that two thirds of the CUs idle through hundreds of K steps; there, 3-4 workgroups
+// a tile of the 64x128 cell, each on a share of K, measured 9-19 % faster although the partials
+// travel through memory (5120 x 17408: M=64 34.1 -> 28.6 us, M=128 33.6 -> 30.7 us). On every other
+// shape timed (K <= 6144 at any M, more than 80 tiles at any K) the unsplit cell won by 1.3-3x --
+// the partials cost ks*M*N*4 bytes each way and the last arriver sums alone -- so the rule is this
+// narrow. The launch then needs the `decode_partial` / `decode_counter` workspaces the descriptor lists.
+uint32_t pf_split(bool w8, uint32_t m, uint32_t n, uint32_t k, const PfVariant **cell) {
+  if (w8 || k < 16384) return 0;
+  const PfVariant *v = pf_variant("macaq_iu8_pf_w4_t64x128_s");
+  if (!v || !signature_for(std::string(v->name) + "_ks")) return 0;
+  const uint64_t tiles = (uint64_t)((n + v->block_n() - 1) / v->block_n()) * ((m + v->block_m() - 1) / v->block_m());
+  if (tiles > 80) return 0;
+  *cell = v;
+  return (uint32_t)std::min<uint64_t>(4, CU_COUNT / tiles);
 }
 
 // The prefill cell of a shape: the tile whose estimated time is least. A launch's time is a fixed

@@ -27,6 +27,7 @@ const DecVariant *dec_variant(const std::string &name);
 const PfVariant *pf_variant(const std::string &name);
 // The prefill cell (tile shape) the launch law picks for a shape.
 const PfVariant *pf_cell(bool w8, uint32_t m, uint32_t n, uint32_t k);
+uint32_t pf_split(bool w8, uint32_t m, uint32_t n, uint32_t k, const PfVariant **cell);
 
 constexpr uint32_t DECODE_MAX_M = 64;  // the decode band's last row count (macaq_iu8.rs:31)
 constexpr uint32_t KS_MAX = 8;         // the largest grid-level split (macaq_iu8.rs:44)

@@ -99,13 +99,18 @@ static __device__ __forceinline__ unsigned iu8_code4_rcp(float x0, float x1, flo
 }
 
 // Cross-workgroup hand-over without a cache flush. The card has one L2 per XCD, so a device-scope
-// release fence writes back and invalidates a whole L2 -- costly when every workgroup of a launch does
-// it. Data written with both scope bits set goes straight through to memory, and a load with both
-// set comes from there, so a producer that stores its data this way, waits for the stores' completion
-// (vmcnt) and then bumps a device-scope atomic, and a consumer that reads the atomic and then loads
-// this way, need no fence at all.
+// release fence writes an L2's dirty lines back and an acquire fence invalidates it; with hundreds of
+// workgroups doing that the fences alone cost 15-60 us a launch (measured with and without dirty
+// data). Accesses with both scope bits set are coherent by themselves: such a store goes through to
+// memory and its completion (vmcnt) means it is visible there, such a load comes from there. So a
+// producer stores its partials this way, waits for their completion, meets its workgroup and bumps a
+// device-scope atomic counter; the consumer that finds the counter full loads the partials this way.
+// The order is the hardware's in-order completion count, not a language-level fence: these helpers
+// are asm for that reason.
 static __device__ __forceinline__ void iu8_store_through(int *p, iu8_v4i v) {
-  asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" ::"v"(p), "v"(v) : "memory");
+  // the wait states behind it: a store of more than 8 bytes reads its data registers for two more
+  // cycles, and the compiler's hazard recognizer does not look inside an asm statement
+  asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1\n\ts_nop 2" ::"v"(p), "v"(v) : "memory");
 }
 static __device__ __forceinline__ iu8_v4i iu8_load_through(const int *p) {
   iu8_v4i v;
@@ -113,6 +118,10 @@ static __device__ __forceinline__ iu8_v4i iu8_load_through(const int *p) {
   return v;
 }
 static __device__ __forceinline__ void iu8_stores_done() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+// one lane, after the workgroup met behind its completed stores: count the arrival
+static __device__ __forceinline__ int iu8_arrive(int *counter) {
+  return __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 
 static __device__ __forceinline__ iu8_v4u iu8_ldg_nt(const iu8_u8 *p) {
   return __builtin_nontemporal_load((const iu8_v4u *)p);

@@ -291,7 +291,7 @@ __device__ __forceinline__ void iu8_dec_body(const iu8_u8 *__restrict__ A, const
     iu8_stores_done();
   }
   __syncthreads();
-  if (tid == 0) s_last = (__hip_atomic_fetch_add(&cnt[B.bx], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == Z - 1);
+  if (tid == 0) s_last = (iu8_arrive(&cnt[B.bx]) == Z - 1);
   __syncthreads();
   if (!s_last) return;
   if (tid == 0) __hip_atomic_store(&cnt[B.bx], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -48,6 +48,7 @@ struct iu8_tile {
   int mbase, nt0;
   const iu8_u8 *W;
   const float *ws;
+  int id;  // the tile's index in the launch (its arrival counter under a split of K)
 };
 
 // Dense tile order of a persistent launch of G workgroups over gx x gy tiles. The hardware deals
@@ -66,9 +67,14 @@ static __device__ __forceinline__ bool iu8_dense_tile_at(int r, int gx, int gy, 
   return true;
 }
 
+// A split of K over gridDim.z (P, cnt not null): the workgroups of share z run steps [z*spb, (z+1)*spb)
+// of every tile and hand their int32 partials over through memory, the last to arrive at a tile's
+// counter sums the shares and runs the epilogue (the flush-free hand-over of iu8_common.h; the counter
+// is left at zero).
 template <bool W8, int WMW, int WNW, int TM, int TN, bool ACC, int STMAX, bool DEEP = false, class TileAt>
 __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const float *__restrict__ as,
-                                             void *__restrict__ Cv, int N, int K, TileAt tile_at) {
+                                             void *__restrict__ Cv, int N, int K, TileAt tile_at,
+                                             int *__restrict__ P = nullptr, int *__restrict__ cnt = nullptr) {
   // tile_at(r, t): fills the workgroup's r-th tile, false when it has none
   constexpr int NWAVE = WMW * WNW;
   constexpr int BMT = WMW * TM * 2, BNT = WNW * TN * 2;  // 16-row tiles a workgroup, both ways
@@ -88,7 +94,14 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WNW, wn = wave % WNW;
-  const int ntiles = N >> 4, steps = K >> 7, ktiles = K >> 6;
+  const int ntiles = N >> 4, ksteps = K >> 7, ktiles = K >> 6;
+  // this workgroup's share of the K steps
+  const int Z = P != nullptr ? (int)gridDim.z : 1, z = P != nullptr ? (int)blockIdx.z : 0;
+  const int spb = (ksteps + Z - 1) / Z;
+  const int s_lo = min(z * spb, ksteps - 1), s_hi = max(min(ksteps, z * spb + spb), s_lo + 1);
+  const bool share_empty = z * spb >= ksteps;  // more shares than steps: this one re-runs a step and adds nothing
+  const int steps = s_hi - s_lo;
+  __shared__ int s_last;
 
   // ---- the load stream: (tile L, step ls), NST-1 steps ahead of the MFMAs
   // Global -> LDS without registers: global_load_lds_dwordx4 writes lane l's 16 bytes at
@@ -96,7 +109,7 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
   // Per lane: the 32-bit byte offset of its piece at K step 0 of the load stream's tile.
   iu8_tile L, Nx;  // the stream's tile and the one after it
   if (!tile_at(0, L)) return;
-  int lr = 0, ls = 0;
+  int lr = 0, ls = s_lo;
   unsigned ga[A_PER], gw[W_PER], gaN[A_PER], gwN[W_PER];
   auto addr_of = [&](const iu8_tile &t, unsigned (&oa)[A_PER], unsigned (&ow)[W_PER]) {
 #pragma unroll
@@ -109,7 +122,7 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
     for (int p = 0; p < W_PER; ++p) {
       const int f = min(p * NWAVE + wave, W_FR - 1);
       const int nt = min(t.nt0 + f / (WSTEP / 1024), ntiles - 1);  // tiles past N: the last one
-      ow[p] = (unsigned)((size_t)nt * steps * WSTEP + (f % (WSTEP / 1024)) * 1024 + lane * 16);
+      ow[p] = (unsigned)((size_t)nt * ksteps * WSTEP + (f % (WSTEP / 1024)) * 1024 + lane * 16);
     }
   };
   addr_of(L, ga, gw);
@@ -139,9 +152,9 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
       if (W_FR % NWAVE == 0 || p * NWAVE + wave < W_FR) dma(Ws, gw[p], sW + (p * NWAVE + wave) * 1024);
   };
   auto advance = [&]() {  // next step of the stream; past the last tile it keeps re-loading the last step
-    if (++ls == steps) {
+    if (++ls == s_hi) {
       if (haveN) {
-        ++lr, ls = 0, L = Nx;
+        ++lr, ls = s_lo, L = Nx;
 #pragma unroll
         for (int p = 0; p < A_PER; ++p) ga[p] = gaN[p];
 #pragma unroll
@@ -149,7 +162,7 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
         haveN = tile_at(lr + 1, Nx);
         if (haveN) addr_of(Nx, gaN, gwN);
       } else {
-        ls = steps - 1;
+        ls = s_hi - 1;
       }
     }
   };
@@ -378,7 +391,50 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
     const int M = C.R.rows;
     const int nq = h * 4;
     const int ncol0 = (C.nt0 + wn * TN * 2) * 16;  // first column of the wave tile
-    if constexpr (ACC) {
+    if (Z > 1) {
+      // ---- a share of K: the partial goes out straight through memory, the last share to arrive at
+      // the tile's counter sums all of them in share order (exact in int32) and runs the epilogue
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        const int m = C.mbase + (wm * TM + i) * 32 + r32;
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const int n = ncol0 + j * 32 + g * 8 + nq;
+            if (m >= M || n >= N) continue;
+            const iu8_v4i v = share_empty ? iu8_v4i{0, 0, 0, 0}
+                                          : iu8_v4i{acc[i][j][g * 4], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
+            iu8_store_through(&P[((size_t)z * M + C.R.row0 + m) * N + n], v);
+          }
+      }
+      iu8_stores_done();
+      __builtin_amdgcn_s_barrier();
+      if (tid == 0) s_last = (iu8_arrive(&cnt[C.id]) == Z - 1);
+      wait_vm(std::integral_constant<int, 63>{}, true);
+      __builtin_amdgcn_s_barrier();
+      if (s_last) {
+              if (tid == 0) __hip_atomic_store(&cnt[C.id], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        constexpr int BM = WMW * TM * 32, BN = WNW * TN * 32;
+        const int nb = C.nt0 * 16, rows = min(BM, M - C.mbase), cols4 = min(BN, N - nb) >> 2;
+        for (int idx = tid; idx < rows * cols4; idx += NWAVE * 64) {
+          const int r = idx / cols4, m = C.mbase + r, n = nb + (idx - r * cols4) * 4;
+          iu8_v4i sum = iu8_v4i{0, 0, 0, 0};
+          for (int q = 0; q < Z; ++q) sum += iu8_load_through(&P[((size_t)q * M + C.R.row0 + m) * N + n]);
+          const size_t crow = (size_t)(C.R.row0 + m) * N;
+          if constexpr (ACC) {
+            *(iu8_v4i *)((int *)Cv + crow + n) = sum;
+          } else {
+            const float am = as[iu8_arow(C.R, m)];
+            const float4 w4 = *(const float4 *)(C.ws + n);
+            const float u = W8 ? 1.f : 0.0625f;
+            const unsigned lo = iu8_bf16_pack(iu8_epi(sum[0], am, w4.x * u), iu8_epi(sum[1], am, w4.y * u));
+            const unsigned hi = iu8_bf16_pack(iu8_epi(sum[2], am, w4.z * u), iu8_epi(sum[3], am, w4.w * u));
+            *(iu8_v2u *)((unsigned short *)Cv + crow + n) = iu8_v2u{lo, hi};
+          }
+        }
+      }
+    } else if constexpr (ACC) {
 #pragma unroll
       for (int j = 0; j < TN; ++j)
 #pragma unroll

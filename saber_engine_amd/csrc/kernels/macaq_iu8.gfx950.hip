@@ -16,8 +16,8 @@
 //           row of A only reaches its own row of C, and dead rows are never stored. The k-waves'
 //           partials are reduced through LDS (exact int32). An optional grid-level split
 //           (gridDim.z) goes through the `decode_partial` / `decode_counter` workspaces with the
-//           last-arriving workgroup summing; it costs device-scope fences across the 8 XCDs' L2s
-//           and the launch law does not use it by default.
+//           last-arriving workgroup summing (partials handed over straight through memory, no
+//           cache flush); the launch law does not use it by default.
 //   prefill (M > 64)   MFMA-bound tile GEMM on v_mfma_i32_32x32x32_i8 (iu8_pf32.h): persistent
 //           workgroups of 8 waves (two a SIMD) walk an XCD-aware tile order; the fragments of a
 //           128-deep K step go from HBM/L2 into one of three LDS stages by LDS-DMA loads, two steps
@@ -76,10 +76,39 @@ IU8_DECQ(macaq_iu8_decq_w8_tm1, true, 4)
     iu8_pf32_run<W8, WMW, WNW, TM, TN, ACC, ST, DEEP>(a, as, c, n, k, [&](int r, iu8_tile &t) {                          \
       int bx, by;                                                                                                  \
       if (!iu8_dense_tile_at(r, gx, gy, bx, by)) return false;                                                     \
-      t = iu8_tile{R, by * BM, bx * (BN / 16), w, ws};                                                             \
+      t = iu8_tile{R, by * BM, bx * (BN / 16), w, ws, by * gx + bx};                                               \
       return true;                                                                                                 \
     });                                                                                                            \
   }
+// Cells with K split over gridDim.z (symbol suffix `_ks`, the decode kernarg list: the two workspaces
+// in front of c), for the rows between the regimes, where few tiles leave CUs idle. Measured, the
+// partials' way through memory (ks * M * N * 4 bytes out and back) costs more than the idle CUs: the
+// launch law does not pick these; they are kept, tested and reachable by name like the decode split.
+#define IU8_PF32K(name, W8, WMW, WNW, TM, TN, ST, OCC, DEEP)                                                       \
+  extern "C" __global__ __launch_bounds__(WMW * WNW * 64)                                                         \
+      __attribute__((amdgpu_waves_per_eu(WMW * WNW * OCC / 4, WMW * WNW * OCC / 4))) void name(                    \
+      const unsigned char *__restrict__ a, const unsigned char *__restrict__ w, const float *__restrict__ as,     \
+      const float *__restrict__ ws, int *__restrict__ decode_partial, int *__restrict__ decode_counter,           \
+      unsigned short *__restrict__ c, int m, int n, int k) {                                                       \
+    constexpr int BM = WMW * TM * 32, BN = WNW * TN * 32;                                                          \
+    const int gx = (n + BN - 1) / BN, gy = (m + BM - 1) / BM;                                                      \
+    const iu8_rows R{nullptr, 0, m};                                                                               \
+    iu8_pf32_run<W8, WMW, WNW, TM, TN, false, ST, DEEP>(                                                           \
+        a, as, c, n, k,                                                                                            \
+        [&](int r, iu8_tile &t) {                                                                                  \
+          int bx, by;                                                                                              \
+          if (!iu8_dense_tile_at(r, gx, gy, bx, by)) return false;                                                 \
+          t = iu8_tile{R, by * BM, bx * (BN / 16), w, ws, by * gx + bx};                                           \
+          return true;                                                                                             \
+        },                                                                                                         \
+        gridDim.z > 1 ? decode_partial : nullptr, decode_counter);                                                 \
+  }
+IU8_PF32K(macaq_iu8_pf_w4_t128x128_ks, false, 4, 2, 1, 2, 3, 1, false)
+IU8_PF32K(macaq_iu8_pf_w8_t128x128_ks, true, 4, 2, 1, 2, 3, 1, false)
+IU8_PF32K(macaq_iu8_pf_w4_t256x160_ks, false, 8, 1, 1, 5, 3, 1, false)
+IU8_PF32K(macaq_iu8_pf_w8_t256x160_ks, true, 8, 1, 1, 5, 3, 1, false)
+IU8_PF32K(macaq_iu8_pf_w4_t64x128_s_ks, false, 2, 2, 1, 2, 5, 2, true)
+#undef IU8_PF32K
 #define IU8_DEC_VARIANT(name, TM, W8, NT, KW, WPB, D, ALDS, ACC)
 #define IU8_PF_VARIANT(name, W8, WMW, WNW, TM, TN, ACC, ST, OCC, DEEP) IU8_PF32(name, W8, WMW, WNW, TM, TN, ACC, ST, OCC, DEEP)
 #define IU8_PAIR_VARIANT(name, TM, NT, KW, WPB, D, ALDS)

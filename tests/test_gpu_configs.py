@@ -89,6 +89,60 @@ def test_prefill_edges_on_every_tile(ctx, shape):
         assert_dense_matches(run, r, w8)
 
 
+SPLIT_CELLS = {"w4": ("t128x128", "t256x160", "t64x128_s"), "w8": ("t128x128", "t256x160")}
+
+
+@pytest.mark.parametrize("shape,splits", [((200, 272, 640), (1, 2, 3, 5)), ((129, 304, 384), (2, 3)), ((300, 1040, 2048), (4, 8)),
+                                          ((520, 528, 1280), (2, 5))])
+def test_tile_gemm_with_k_split_over_workgroups(ctx, shape, splits):
+    """The `_ks` forms: shares of the K steps on gridDim.z, partials handed over through memory, the
+    last share to arrive sums and stores. Same bytes as the oracle for every cell and share count,
+    ragged edges, more tiles than workgroups a share, counters left at zero and re-usable."""
+    M, N, K = shape
+    for tag, w8 in (("w4", False), ("w8", True)):
+        case = synth.dense_case(M, N, K, w8=w8, seed=51 + M)
+        r = ref.linear(case["X"], case["W"], case["ws"], w8, threads=8)
+        for cell in SPLIT_CELLS[tag]:
+            for ks in splits:
+                name = f"macaq_iu8_pf_{tag}_{cell}_ks"
+                say(f"split tile GEMM {shape} {name} ks={ks}")
+                run = DenseRun(ctx, case, kernel=name, ks=ks, want_acc=False)
+                assert run.desc.grid[2] == ks
+                np.testing.assert_array_equal(run.C, r["C"])
+                if ks > 1:
+                    assert not run.counter.cpu().numpy().any(), "the arrival counters must be left at zero"
+                    d = run.dev
+                    d["c"].fill_(0)
+                    bufs = dict(a=d["q"].data_ptr(), w=d["wf"].data_ptr(), ws=d["ws"].data_ptr(), c=d["c"].data_ptr(),
+                                decode_partial=run.partial.data_ptr(), decode_counter=run.counter.data_ptr())
+                    bufs["as"] = d["a_scale"].data_ptr()
+                    ctx.launch(run.desc, bufs)
+                    torch.cuda.synchronize()
+                    np.testing.assert_array_equal(host_u16(d["c"]), r["C"])
+    with pytest.raises(iu8.IU8Error):
+        iu8.describe("macaq_iu8_pf_w4_t128x128_ks", 200, 272, 640, ks=4)          # 5 steps in 4 shares: the last is empty
+    with pytest.raises(iu8.IU8Error):
+        iu8.describe("macaq_iu8_pf_w4_t128x128", 200, 272, 640, ks=2)             # the plain cell does not split
+
+
+@pytest.mark.parametrize("shape,ks", [((64, 384, 16384), 4), ((100, 640, 17408), 4), ((128, 5120, 17408), 3)])
+def test_launch_law_splits_deep_narrow_tile_gemm(ctx, shape, ks):
+    """Where the law shares K over workgroups (K >= 16384, at most 80 tiles of the 64x128 cell) the
+    descriptor lists the workspaces and the launch through it gives the oracle's bytes."""
+    M, N, K = shape
+    say(f"law-split tile GEMM {shape}")
+    case = synth.dense_case(M, N, K, seed=77 + M)
+    run = DenseRun(ctx, case, want_acc=False)
+    assert run.desc.kernel.decode() == "macaq_iu8_pf_w4_t64x128_s_ks" and run.desc.ks == ks
+    cols = min(N, 512)
+    qh, sh = ref.quant_bf16(case["X"])
+    S, _ = ref.gemm_fast(qh, case["W"][:cols], False, threads=16)
+    np.testing.assert_array_equal(run.C[:, :cols], ref.epilogue(S, sh, case["ws"][:cols], False))
+    S, _ = ref.gemm_fast(qh, case["W"][-cols:], False, threads=16)
+    np.testing.assert_array_equal(run.C[:, -cols:], ref.epilogue(S, sh, case["ws"][-cols:], False))
+    assert not run.counter.cpu().numpy().any()
+
+
 def test_split_counter_is_reusable_across_launches(ctx):
     say("explicit split, two launches on one counter")
     case = synth.dense_case(3, 256, 2048, seed=23)

@@ -126,6 +126,23 @@ def test_pair_variants_share_their_decode_twin_geometry():
         assert twin == (tm, "false", nt, kw, wpb, d, alds, "false"), name
 
 
+def test_launch_law_shares_k_only_on_deep_narrow_tile_gemms():
+    """The one band where the law splits the tile GEMM: K >= 16384 and at most 80 tiles of the
+    64x128 cell; the descriptor then names the `_ks` form, its z grid and both workspaces."""
+    for m, ks, tiles in ((49, 4, 40), (64, 4, 40), (65, 3, 80), (128, 3, 80)):
+        d = iu8.resolve(iu8.W4, m, 5120, 17408)
+        assert d.kernel == b"macaq_iu8_pf_w4_t64x128_s_ks" and d.ks == ks and tuple(d.grid) == (tiles, 1, ks)
+        assert d.workspace("decode_partial").bytes == ks * m * 5120 * 4 and d.workspace("decode_partial").kind == iu8.WS_SCRATCH
+        c = d.workspace("decode_counter")
+        assert c.bytes == tiles * 4 and c.kind == iu8.WS_PERSISTENT and c.zero_once
+        assert iu8.gemm_workspace(iu8.W4, m, 5120, 17408) == (ks * m * 5120 * 4, tiles * 4)
+    for wk, m, n, k in ((iu8.W4, 129, 5120, 17408), (iu8.W4, 64, 5120, 16256), (iu8.W4, 64, 12288, 17408),
+                        (iu8.W8, 64, 5120, 17408), (iu8.W4, 2048, 5120, 17408), (iu8.W4, 64, 5120, 5120)):
+        d = iu8.resolve(wk, m, n, k)
+        assert d.ks == 1 and d.n_workspaces == 0 and not d.kernel.endswith(b"_ks"), (m, n, k)
+        assert iu8.gemm_workspace(wk, m, n, k) == (0, 0)
+
+
 def test_explicit_split_declares_its_workspaces():
     d = iu8.describe("macaq_iu8_dec_w4_tm1", 4, 5120, 17408, ks=4)
     assert d.ks == 4 and d.grid[2] == 4
@@ -159,7 +176,7 @@ def test_prefill_cells_of_the_benchmark_shapes():
     want = {(2048, 34816, 5120): "tn4_lbk64", (2048, 7168, 5120): "tn4_lbk64", (2048, 5120, 17408): "t256x160",
             (2048, 5120, 5120): "t256x160", (8192, 34816, 5120): "tn4_lbk64",
             # up to M of about 512 the launch is bound by what the CUs pull from L2: small tiles on every CU
-            (256, 5120, 17408): "t64x128_s", (128, 5120, 17408): "t64x64_s", (256, 34816, 5120): "t256x160",
+            (256, 5120, 17408): "t64x128_s", (128, 5120, 17408): "t64x128_s_ks", (128, 5120, 5120): "t64x64_s", (256, 34816, 5120): "t256x160",
             (1024, 5120, 5120): "t128x128_o2", (1024, 7168, 5120): "t128x128_o2"}
     for (m, n, k), tile in want.items():
         assert iu8.resolve(iu8.W4, m, n, k).kernel.decode() == "macaq_iu8_pf_w4_" + tile, (m, n, k)
