@@ -207,6 +207,12 @@ int saber_iu8_launch(saber_iu8_ctx *ctx, const saber_iu8_desc *desc, const saber
 /* Per-token int8 quantisation: x bf16 [m,k] -> q (A edge, saber_iu8_a_bytes) + scale f32 [m]. */
 int saber_iu8_quant(saber_iu8_ctx *ctx, const void *x_bf16, void *q, float *scale, uint32_t m, uint32_t k, void *stream);
 
+/* The same law with the codes row-major, q[row * k + col] (m * k bytes): the operand the grouped GEMM
+ * of a routed layer gathers whole token rows from (gather 2), as the reference's grouped GEMM does
+ * (crates/saber-kernels/hip/moe_grouped.hip:67-74). */
+int saber_iu8_quant_rowmajor(saber_iu8_ctx *ctx, const void *x_bf16, void *q, float *scale, uint32_t m, uint32_t k,
+                             void *stream);
+
 /* The Hadamard-basis producers in front of a MACaQ-W4A8 GEMM (crates/saber-kernels/hip/mxfp4_hadi8.hip,
  * hip/macaq_had.h): the producer's bf16-rounded values times `had_t` (f32 [width]), a 32-point
  * Hadamard transform per 32-block, times 1/sqrt(32), then the per-token int8 law; codes in the A edge
@@ -287,7 +293,7 @@ int saber_iu8_gemm_acc(saber_iu8_ctx *ctx, int wkind, const void *a, const void 
 uint32_t saber_iu8_moe_rows_cap(uint32_t tokens, uint32_t topk, uint32_t experts);
 uint32_t saber_iu8_moe_tiles_cap(uint32_t tokens, uint32_t topk, uint32_t experts, uint32_t tile_blocks);
 /* tile_blocks the grouped law picks for `tokens`: 1 (16-row tiles, weight-streaming cells) while an
- * expert averages <= 16 routes, 8 (128-row MFMA tiles) above. */
+ * expert averages <= 16 routes, 8 (128-row MFMA tiles) up to 96 routes an expert, 16 (256-row) from there. */
 uint32_t saber_iu8_moe_tile_blocks(uint32_t tokens, uint32_t topk, uint32_t experts);
 
 /* Device buffers of one routed layer, named as the router kernel's arguments
@@ -303,9 +309,11 @@ typedef struct {
   int32_t *tile_rows;   /* [tiles_cap] */
   int32_t *expert_cnt;  /* [experts] */
   int32_t *meta;        /* [8]: [0] tiles, [1] rows, [3] routes, [4] experts touched */
-  int32_t *blk_cnt;     /* [ceil(T / 32) * experts]  scratch */
+  int32_t *blk_cnt;     /* [ceil(T / 32) * experts]  scratch (the router uses the first ceil(T / 128) * experts) */
   int32_t *rank;        /* [T * topk]                scratch */
   int32_t *arrive;      /* [1]  persistent: zeroed once by the caller, left zero */
+  const uint16_t *silu_lut; /* optional (may be NULL): [65536] as saber_iu8_silu_table wrote it; with it
+                             * saber_iu8_moe_silu_mul_quant reads the bf16 silu from the table on large row counts */
 } saber_iu8_moe_tables;
 
 /* Router + expert-major sort + tile table, one launch. logits bf16 [T, experts]. */
@@ -314,8 +322,9 @@ int saber_iu8_moe_route(saber_iu8_ctx *ctx, const void *logits_bf16, uint32_t to
 
 /* Grouped W4 GEMM over the tile table: per tile the expert's weights (gfx950 W4 fragments) at
  * xptr[2e] and f32 row scales at xptr[2e + 1] (device array of 2 * experts addresses); A rows
- * gathered through row_tok (gather != 0: a / as are token-major) or in place (a / as are
- * expert-major); C bf16 [rows_cap, n]. tile_blocks as given to the router. */
+ * gathered through row_tok (gather 1: a is the token-major A edge; gather 2, MFMA cells only: a is
+ * token-major row-major codes from saber_iu8_quant_rowmajor; as token-major) or in place (gather 0:
+ * a / as are expert-major); C bf16 [rows_cap, n]. tile_blocks as given to the router (1, 8 or 16). */
 int saber_iu8_moe_grouped(saber_iu8_ctx *ctx, const void *a, const float *as, const void *xptr, void *c_bf16, uint32_t n,
                           uint32_t k, int gather, uint32_t tokens, uint32_t experts, uint32_t topk, uint32_t tile_blocks,
                           const saber_iu8_moe_tables *t, void *stream);

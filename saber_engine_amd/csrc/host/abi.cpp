@@ -40,6 +40,8 @@ static const Signature SIG_HAD_AGQ = {{"core", K::Buffer}, {"gate", K::Buffer}, 
                                       {"n", K::I32},       {"hd", K::I32},      {"gs", K::I32},   {"had_t", K::Buffer}};
 static const Signature SIG_SILU = {{"gu", K::Buffer}, {"q", K::Buffer},       {"scale", K::Buffer},
                                    {"n", K::I32},     {"row_tok", K::Buffer}, {"meta", K::Buffer}};
+static const Signature SIG_SILU_LUT = {{"gu", K::Buffer}, {"q", K::Buffer},       {"scale", K::Buffer}, {"n", K::I32},
+                                       {"row_tok", K::Buffer}, {"meta", K::Buffer}, {"lut", K::Buffer}};
 static const Signature SIG_TABLE = {{"out", K::Buffer}};
 static const Signature SIG_MOE_ROUTE = {
     {"logits", K::Buffer},      {"t", K::I32},           {"e_lo", K::I32},        {"e_loc", K::I32},
@@ -76,6 +78,7 @@ const Signature *signature_for(const std::string &k) {
   if (k == "mxfp4_hadi8_silu_f32_table" || k == "attn_glue_hadi8_sigmoid_bf16_table") return &SIG_TABLE;
   if (starts(k, "macaq_i8_quant_rows_")) return &SIG_QUANT_ROWS;
   if (starts(k, "macaq_i8_quant_")) return &SIG_QUANT;
+  if (starts(k, "macaq_i8_silu_mul_quant_lut_")) return &SIG_SILU_LUT;
   if (starts(k, "macaq_i8_silu_mul_quant_")) return &SIG_SILU;
   if (k == "macaq_silu_bf16_table") return &SIG_TABLE;
   if (k == "iu8_probe_read" || k == "iu8_probe_mfma32d" || k == "iu8_probe_first") return &SIG_PROBE_READ;

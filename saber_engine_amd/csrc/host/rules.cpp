@@ -403,6 +403,12 @@ int resolve_quant(uint32_t m, uint32_t k, saber_iu8_desc *out) {
   return describe_rows("quant_i8", row_form("macaq_i8_quant", m, k).c_str(), m, k, "k", out);
 }
 
+int resolve_quant_rowmajor(uint32_t m, uint32_t k, saber_iu8_desc *out) {
+  const uint32_t slots = (k + 4095) / 4096;
+  const std::string name = std::string("macaq_i8_quant_rm_t256") + (slots <= 1 ? "_g1" : slots <= 2 ? "_g2" : "");
+  return describe_rows("quant_i8_rowmajor", name.c_str(), m, k, "k", out);
+}
+
 int resolve_quant_rows(uint32_t rows, uint32_t k, saber_iu8_desc *out) {
   const uint32_t slots = (k + 4095) / 4096;
   const std::string name = std::string("macaq_i8_quant_rows_t256") + (slots <= 1 ? "_g1" : slots <= 2 ? "_g2" : "");

@@ -46,6 +46,8 @@ int resolve_quant(uint32_t m, uint32_t k, saber_iu8_desc *out);
 bool fused_holds(uint32_t m, uint32_t k);
 int resolve_fused(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *out);
 int resolve_silu_mul_quant(uint32_t rows, uint32_t n, saber_iu8_desc *out);
+// Quantisation to row-major codes (q[row * k + col]).
+int resolve_quant_rowmajor(uint32_t m, uint32_t k, saber_iu8_desc *out);
 // Quantisation through a row map (output row r = input row row_tok[r]).
 int resolve_quant_rows(uint32_t rows, uint32_t k, saber_iu8_desc *out);
 

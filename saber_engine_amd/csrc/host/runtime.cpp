@@ -348,6 +348,13 @@ int saber_iu8_quant(saber_iu8_ctx *ctx, const void *x, void *q, float *scale, ui
   return saber_iu8_launch(ctx, &d, b, 3, stream);
 }
 
+int saber_iu8_quant_rowmajor(saber_iu8_ctx *ctx, const void *x, void *q, float *scale, uint32_t m, uint32_t k, void *stream) {
+  saber_iu8_desc d;
+  if (int rc = resolve_quant_rowmajor(m, k, &d)) return rc;
+  const saber_iu8_binding b[] = {{"x", (void *)x}, {"q", q}, {"scale", scale}};
+  return saber_iu8_launch(ctx, &d, b, 3, stream);
+}
+
 int saber_iu8_linear_fused(saber_iu8_ctx *ctx, int wkind, const void *x, const void *w, const float *ws, void *c, void *q,
                            float *scale, uint32_t m, uint32_t n, uint32_t k, void *stream) {
   saber_iu8_desc d;
@@ -515,8 +522,14 @@ uint32_t saber_iu8_moe_tiles_cap(uint32_t tokens, uint32_t topk, uint32_t expert
   const uint32_t r = tokens * topk;
   return std::min(r, experts) + r / (16u * std::max(tile_blocks, 1u)) + 1u;
 }
+// Rows a tile (x16): 16-row tiles on the streaming cell while a tile a route's expert is the common
+// case; from about 96 routes an expert the 256-row MFMA cell (one tile an expert more often than
+// not, and the dense GEMM's fastest shape), between them the 128-row one. Speed data of this card:
+// 128 experts, top-8, 4096 x 1536: T=1024 400 vs 431 us a layer (8 vs 16), T=2048 592 vs 531.
 uint32_t saber_iu8_moe_tile_blocks(uint32_t tokens, uint32_t topk, uint32_t experts) {
-  return (uint64_t)tokens * topk <= 16ull * experts ? 1u : 8u;
+  const uint64_t routes = (uint64_t)tokens * topk;
+  if (routes <= 16ull * experts) return 1u;
+  return routes >= 96ull * experts ? 16u : 8u;
 }
 
 static int moe_check(const char *what, uint32_t tokens, uint32_t experts, uint32_t topk, const saber_iu8_moe_tables *t) {
@@ -537,7 +550,7 @@ int saber_iu8_moe_route(saber_iu8_ctx *ctx, const void *logits, uint32_t tokens,
   if (int rc = moe_check("moe_route", tokens, experts, topk, t)) return rc;
   if (tile_blocks == 0) return fail(SABER_IU8_E_RULE, "moe_route: tile_blocks 0");
   saber_iu8_desc d;
-  if (int rc = raw_desc("moe_iu8_route_topk8_sort_e128", (tokens + 31) / 32, 1, 256, &d)) return rc;
+  if (int rc = raw_desc("moe_iu8_route_topk8_sort_e128", (tokens + 127) / 128, 1, 1024, &d)) return rc;
   set_i32(&d, "t", tokens);
   set_i32(&d, "e_lo", 0);
   set_i32(&d, "e_loc", experts);
@@ -557,10 +570,12 @@ int saber_iu8_moe_grouped(saber_iu8_ctx *ctx, const void *a, const float *as, co
   if (int rc = moe_check("moe_grouped", tokens, experts, topk, t)) return rc;
   if (n == 0 || k == 0 || n % 16 != 0 || k % 128 != 0)
     return fail(SABER_IU8_E_RULE, fmt("moe_grouped: N=%u must be a multiple of 16 (whole fragments) and K=%u of 128 (the slab)", n, k));
-  if (tile_blocks != 1 && tile_blocks != 8)
-    return fail(SABER_IU8_E_RULE, fmt("moe_grouped: tile_blocks %u; the cells are 1 (16-row) and 8 (128-row)", tile_blocks));
+  if (tile_blocks != 1 && tile_blocks != 8 && tile_blocks != 16)
+    return fail(SABER_IU8_E_RULE, fmt("moe_grouped: tile_blocks %u; the cells are 1 (16-row), 8 (128-row) and 16 (256-row)", tile_blocks));
   const bool dec = tile_blocks == 1;
-  const std::string name = fmt("moe_iu8_grouped_w4_%s_g%d", dec ? "dec" : "pf", gather ? 1 : 0);
+  if (gather < 0 || gather > 2 || (gather == 2 && dec))
+    return fail(SABER_IU8_E_RULE, fmt("moe_grouped: gather %d; 0 in place, 1 from A fragments, 2 from row-major codes (MFMA cells only)", gather));
+  const std::string name = fmt("moe_iu8_grouped_w4_%s_g%d", dec ? "dec" : tile_blocks == 8 ? "pf" : "pf16", gather);
   const uint32_t bn = dec ? 32 : 256, block = 512;
   saber_iu8_desc d;
   // the streaming cell: a workgroup a (column block, tile), static worst-case grid; the MFMA cell:
@@ -594,6 +609,17 @@ int saber_iu8_moe_silu_mul_quant(saber_iu8_ctx *ctx, const void *gu, void *q, fl
                                  const saber_iu8_moe_tables *t, void *stream) {
   if (!t) return fail(SABER_IU8_E_ARG, "moe_silu_mul_quant: null tables");
   saber_iu8_desc d;
+  // From a few thousand rows the table form (memory-bound) overtakes the computed one (bound by the
+  // exp and divide of every element); below, copying the table into LDS costs more than it saves.
+  if (t->silu_lut && rows_cap >= 4096 && n % 16 == 0 && n <= 4096) {
+    const uint32_t tiles = (rows_cap + 15) / 16;
+    const uint32_t grid[3] = {tiles < CU_COUNT ? tiles : CU_COUNT, 1, 1};
+    if (int rc = saber_iu8_describe_raw("macaq_i8_silu_mul_quant_lut_w64", "macaq_i8q", grid, 1024, &d)) return rc;
+    set_i32(&d, "n", n);
+    const saber_iu8_binding b[] = {{"gu", (void *)gu}, {"q", q}, {"scale", scale}, {"row_tok", t->row_tok}, {"meta", t->meta},
+                                   {"lut", (void *)t->silu_lut}};
+    return saber_iu8_launch(ctx, &d, b, 6, stream);
+  }
   if (int rc = resolve_silu_mul_quant(rows_cap, n, &d)) return rc;
   set_buffer(&d, "row_tok");
   set_buffer(&d, "meta");

@@ -71,7 +71,16 @@ static __device__ __forceinline__ bool iu8_dense_tile_at(int r, int gx, int gy, 
 // of every tile and hand their int32 partials over through memory, the last to arrive at a tile's
 // counter sums the shares and runs the epilogue (the flush-free hand-over of iu8_common.h; the counter
 // is left at zero).
-template <bool W8, int WMW, int WNW, int TM, int TN, bool ACC, int STMAX, bool DEEP = false, class TileAt>
+//
+// ARM (the A operand row-major, K bytes a row, rows through the tile's row map): a wave-load still
+// lands one fragment in LDS in fragment order -- lane l fetches the 16 bytes of row l % 16, k chunk
+// l / 16 -- from 16 rows' 64-byte runs instead of one contiguous KiB.
+//
+// SPARSE (tiles of a routed layer, often nearly empty): a wave whose 32-row blocks of the tile are
+// all past the tile's rows, or all but the first, runs the K loop in a form with none, or one, of
+// its TM row blocks -- the same loads, barriers and stage walk, a fraction of the MFMAs and LDS reads
+// -- so such a tile costs its operand traffic instead of a full tile's matrix work.
+template <bool W8, int WMW, int WNW, int TM, int TN, bool ACC, int STMAX, bool DEEP = false, bool SPARSE = false, bool ARM = false, class TileAt>
 __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const float *__restrict__ as,
                                              void *__restrict__ Cv, int N, int K, TileAt tile_at,
                                              int *__restrict__ P = nullptr, int *__restrict__ cnt = nullptr) {
@@ -89,6 +98,7 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
   constexpr int NST = STMAX < 2 ? 2 : (STMAX < NFIT ? STMAX : (NFIT < 2 ? 2 : NFIT));
   static_assert((NST - 2) * (A_FR / NWAVE + W_FR / NWAVE) <= 63, "the in-flight count fits s_waitcnt's vmcnt field");
   static_assert(!DEEP || NST >= 3, "the deep form reads a stage a step ahead of its MFMAs");
+  static_assert(!(DEEP && SPARSE), "the sparse forms exist for the phased loop only");
   __shared__ __attribute__((aligned(1024))) iu8_u8 smem[NST * STAGE];
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -116,7 +126,8 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
     for (int p = 0; p < A_PER; ++p) {
       const int f = min(p * NWAVE + wave, A_FR - 1);  // fragment (mt = f/2, kt2 = f%2) of the step
       const int ar = iu8_arow(t.R, t.mbase + (f >> 1) * 16 + (lane & 15));  // rows past the edge: the last one
-      oa[p] = (unsigned)(((size_t)(ar >> 4) * ktiles + (f & 1)) * 1024 + ((ar & 15) + 16 * (lane >> 4)) * 16);
+      if constexpr (ARM) oa[p] = (unsigned)((size_t)ar * K + (f & 1) * 64 + (lane >> 4) * 16);
+      else oa[p] = (unsigned)(((size_t)(ar >> 4) * ktiles + (f & 1)) * 1024 + ((ar & 15) + 16 * (lane >> 4)) * 16);
     }
 #pragma unroll
     for (int p = 0; p < W_PER; ++p) {
@@ -143,7 +154,7 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
   const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) iu8_u8 *)smem;
   auto issue = [&](int stage) {  // the load stream's step -> LDS stage
     const unsigned sA = lds0 + stage * STAGE, sW = sA + A_BYTES;
-    const iu8_u8 *As = A + (size_t)ls * 2048, *Ws = L.W + (size_t)ls * WSTEP;
+    const iu8_u8 *As = A + (size_t)ls * (ARM ? 128 : 2048), *Ws = L.W + (size_t)ls * WSTEP;
 #pragma unroll
     for (int p = 0; p < A_PER; ++p)
       if (A_FR % NWAVE == 0 || p * NWAVE + wave < A_FR) dma(As, ga[p], sA + (p * NWAVE + wave) * 1024);
@@ -196,9 +207,10 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
   iu8_v4i af[2][TM] = {};
   iu8_v4i wf[W8 ? 2 : 1][TN] = {};
   iu8_v4u wpk[2][W8 ? 1 : TN] = {};
-  auto fetch_a = [&](const iu8_u8 *sA, int buf, int p, int kt2) {
+  using Full = std::integral_constant<int, TM>;
+  auto fetch_a = [&](const iu8_u8 *sA, int buf, int p, int kt2, auto nl) {  // the first nl row blocks
 #pragma unroll
-    for (int i = 0; i < TM; ++i) af[buf][i] = *(const iu8_v4i *)&sA[a_lane + i * 4096 + kt2 * 1024 + p * 512];
+    for (int i = 0; i < decltype(nl)::value; ++i) af[buf][i] = *(const iu8_v4i *)&sA[a_lane + i * 4096 + kt2 * 1024 + p * 512];
   };
   auto fetch_w8 = [&](const iu8_u8 *sW, int buf, int p, int kt2) {  // W8: a whole operand a phase
     if constexpr (W8) {
@@ -212,7 +224,8 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
       for (int j = 0; j < TN; ++j) wpk[p][j] = *(const iu8_v4u *)&sW[w_lane + j * 2048 + p * 512];
     }
   };
-  auto mfmas = [&](int buf, int p, int kt2) {
+  auto mfmas = [&](int buf, int p, int kt2, auto nl) {
+    if constexpr (decltype(nl)::value > 0)
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       if constexpr (!W8) {
@@ -221,7 +234,7 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
                            (int)(d1 & 0xF0F0F0F0u)};
       }
 #pragma unroll
-      for (int i = 0; i < TM; ++i)
+      for (int i = 0; i < decltype(nl)::value; ++i)
         acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[W8 ? buf : 0][j], af[buf][i], acc[i][j], 0, 0, 0);
     }
   };
@@ -230,13 +243,15 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
   // issued behind them.
   constexpr int UNPK = W8 ? 0 : 6;  // VALU ops of one piece-half unpack
 #define IU8_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
-#define IU8_PHASE_ORDER(NDS)                          \
-  IU8_SGB(0x100, NDS);                                \
-  if (UNPK) IU8_SGB(0x002, UNPK);                     \
-  _Pragma("unroll") for (int j_ = 0; j_ < TN; ++j_) { \
-    IU8_SGB(0x008, TM);                               \
-    if (UNPK && j_ + 1 < TN) IU8_SGB(0x002, UNPK);    \
-  }                                                   \
+#define IU8_PHASE_ORDER(NDS, NM)                        \
+  if constexpr ((NDS) > 0) IU8_SGB(0x100, NDS);         \
+  if constexpr ((NM) > 0) {                             \
+    if (UNPK) IU8_SGB(0x002, UNPK);                     \
+    _Pragma("unroll") for (int j_ = 0; j_ < TN; ++j_) { \
+      IU8_SGB(0x008, NM);                               \
+      if (UNPK && j_ + 1 < TN) IU8_SGB(0x002, UNPK);    \
+    }                                                   \
+  }                                                     \
   __builtin_amdgcn_sched_barrier(0)
 
 #pragma unroll
@@ -274,7 +289,7 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
   if constexpr (DEEP) {
     fetch_step(smem, 0);
   } else {
-    fetch_a(smem, 0, 0, 0);
+    fetch_a(smem, 0, 0, 0, Full{});
     fetch_w8(smem + A_BYTES, 0, 0, 0);
     fetch_w4(smem + A_BYTES, 0);
   }
@@ -349,40 +364,57 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
             for (int j = 0; j < TN; ++j) wpd[0][p][j] = wpd[1][p][j];
         }
       }
-    } else
-    for (int s = 0; s < steps; ++s) {
-      const int st1 = st == NST - 1 ? 0 : st + 1, stl = st == 0 ? NST - 1 : st - 1;  // next, last
-      const iu8_u8 *sA = smem + st * STAGE, *sW = sA + A_BYTES;
-      const iu8_u8 *nA = smem + st1 * STAGE, *nW = nA + A_BYTES;
-      // phase 0; the load stream's step leaves HBM for the stage drained last
-      fetch_a(sA, 1, 0, 1);
-      fetch_w8(sW, 1, 0, 1);
-      fetch_w4(sW, 1);
-      issue(stl);
-      mfmas(0, 0, 0);
-      IU8_PHASE_ORDER(TM + TN);
-      // phase 1
-      fetch_a(sA, 0, 1, 0);
-      fetch_w8(sW, 0, 1, 0);
-      mfmas(1, 0, 1);
-      IU8_PHASE_ORDER(TM + (W8 ? TN : 0));
-      // phase 2
-      fetch_a(sA, 1, 1, 1);
-      fetch_w8(sW, 1, 1, 1);
-      mfmas(0, 1, 0);
-      IU8_PHASE_ORDER(TM + (W8 ? TN : 0));
-      // phase 3, behind the barrier: every wave's reads of this stage are done and the next step's
-      // fragments have landed
-      wait_vm(InFlight{}, true);
-      __builtin_amdgcn_s_barrier();
-      __builtin_amdgcn_sched_barrier(0);
-      fetch_a(nA, 0, 0, 0);
-      fetch_w8(nW, 0, 0, 0);
-      fetch_w4(nW, 0);
-      mfmas(1, 1, 1);
-      IU8_PHASE_ORDER(TM + TN);
-      advance();
-      st = st1;
+    } else {
+      // the phased loop with the first `nl` of this wave's TM row blocks live
+      auto run_steps = [&](auto nl) {
+        constexpr int NL = decltype(nl)::value;
+        constexpr int NW = NL > 0 ? TN : 0;  // weight reads a phase that has MFMAs
+        for (int s = 0; s < steps; ++s) {
+          const int st1 = st == NST - 1 ? 0 : st + 1, stl = st == 0 ? NST - 1 : st - 1;  // next, last
+          const iu8_u8 *sA = smem + st * STAGE, *sW = sA + A_BYTES;
+          const iu8_u8 *nA = smem + st1 * STAGE, *nW = nA + A_BYTES;
+          // phase 0; the load stream's step leaves HBM for the stage drained last
+          fetch_a(sA, 1, 0, 1, nl);
+          if constexpr (NL > 0) {
+            fetch_w8(sW, 1, 0, 1);
+            fetch_w4(sW, 1);
+          }
+          issue(stl);
+          mfmas(0, 0, 0, nl);
+          IU8_PHASE_ORDER(NL + NW, NL);
+          // phase 1
+          fetch_a(sA, 0, 1, 0, nl);
+          if constexpr (NL > 0) fetch_w8(sW, 0, 1, 0);
+          mfmas(1, 0, 1, nl);
+          IU8_PHASE_ORDER(NL + (W8 ? NW : 0), NL);
+          // phase 2
+          fetch_a(sA, 1, 1, 1, nl);
+          if constexpr (NL > 0) fetch_w8(sW, 1, 1, 1);
+          mfmas(0, 1, 0, nl);
+          IU8_PHASE_ORDER(NL + (W8 ? NW : 0), NL);
+          // phase 3, behind the barrier: every wave's reads of this stage are done and the next step's
+          // fragments have landed. The next step may be another tile's first, with every row block
+          // live: its first operands are read in full whatever this tile's form.
+          wait_vm(InFlight{}, true);
+          __builtin_amdgcn_s_barrier();
+          __builtin_amdgcn_sched_barrier(0);
+          fetch_a(nA, 0, 0, 0, Full{});
+          fetch_w8(nW, 0, 0, 0);
+          fetch_w4(nW, 0);
+          mfmas(1, 1, 1, nl);
+          IU8_PHASE_ORDER(TM + TN, NL);
+          advance();
+          st = st1;
+        }
+      };
+      int nlw = TM;
+      if constexpr (SPARSE) {
+        const int blocks = (min(C.R.rows - C.mbase, WMW * TM * 32) + 31) >> 5;
+        nlw = max(0, min(TM, blocks - wm * TM));
+      }
+      if (!SPARSE || nlw >= 2 || TM == 1) run_steps(Full{});
+      else if (nlw == 1) run_steps(std::integral_constant<int, 1>{});
+      else run_steps(std::integral_constant<int, 0>{});
     }
 
     // ---- epilogue of tile C. The stage the last step drained is free (the barrier of that step's
@@ -460,6 +492,7 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
       iu8_u8 *reg = smem + (st == 0 ? NST - 1 : st - 1) * STAGE + wave * (32 * ROWB);
 #pragma unroll
       for (int i = 0; i < TM; ++i) {
+        if (C.mbase + (wm * TM + i) * 32 >= M) continue;  // a row block past the tile's rows (the whole wave)
         const int m = C.mbase + (wm * TM + i) * 32 + r32;
         const float am = as[iu8_arow(C.R, min(m, M - 1))];
 #pragma unroll

@@ -5,7 +5,9 @@
 // A fragment order (iu8_common.h), scale f32 per row.
 //
 //   macaq_i8_quant_t256           x bf16 [M,K] -> q, scale                 (grid M, block 256)
-//   macaq_i8_quant_rows_t256      the same through a row map: output row r = input row row_tok[r]
+//   macaq_i8_quant_rm_t256        the same with the codes row-major, q[row * K + col] (the operand a
+//                                 grouped GEMM gathers whole token rows from)
+//   macaq_i8_quant_rows_t256      the first through a row map: output row r = input row row_tok[r]
 //                                 (the gathered, expert-major activations of a routed layer)
 //   macaq_i8_silu_mul_quant_t256  gu bf16 [M, 2N] (gate | up) -> p = bf16(bf16(silu(g)) * u)
 //                                 -> q, scale over N                       (grid M, block 256)
@@ -13,6 +15,8 @@
 //                                 Hadamard; signature crates/saber-kernels/src/abi.rs:315-320)
 //   macaq_i8_quant_w64, macaq_i8_silu_mul_quant_w64   the same two for rows of up to 4,096 elements,
 //                                 a wave a row, four rows a workgroup (grid M/4, block 256)
+//   macaq_i8_silu_mul_quant_lut_w64   the second with the bf16 silu read from a 65,536-entry table in
+//                                 LDS: persistent, 16 waves, a wave a row (grid <= 256, block 1024)
 //   macaq_silu_bf16_table         the bf16 silu of all 65,536 bf16 inputs (a checker's tap)
 //
 // One workgroup a row; a thread owns 16-element groups g = tid + i*256 (one 16-byte store each).
@@ -45,8 +49,8 @@ static __device__ __forceinline__ float i8q_block_max(float v) {
   return r;
 }
 
-// codes of one row from v[g][16] (f32 values), written in A fragment order
-template <int I8Q_MAXG>
+// codes of one row from v[g][16] (f32 values), written in A fragment order (RM: row-major, K bytes a row)
+template <int I8Q_MAXG, bool RM = false>
 static __device__ __forceinline__ void i8q_tail(float (&v)[I8Q_MAXG][16], int G, iu8_u8 *__restrict__ q,
                                                 float *__restrict__ scale, int row, int K) {
   const int tid = threadIdx.x;
@@ -71,14 +75,15 @@ static __device__ __forceinline__ void i8q_tail(float (&v)[I8Q_MAXG][16], int G,
     for (int w = 0; w < 4; ++w) {
       d[w] = iu8_code4_rcp(v[i][w * 4], v[i][w * 4 + 1], v[i][w * 4 + 2], v[i][w * 4 + 3], sc, rcp);
     }
-    *(iu8_v4u *)(qrow + (size_t)(g >> 2) * 1024 + (g & 3) * 256) = iu8_v4u{d[0], d[1], d[2], d[3]};
+    if constexpr (RM) *(iu8_v4u *)(q + (size_t)row * K + g * 16) = iu8_v4u{d[0], d[1], d[2], d[3]};
+    else *(iu8_v4u *)(qrow + (size_t)(g >> 2) * 1024 + (g & 3) * 256) = iu8_v4u{d[0], d[1], d[2], d[3]};
   }
 }
 
 // `row_tok` / `meta` (optional, may be null): with them output row r is the quantised input row
 // row_tok[r] (the expert-major rows of a routed layer, gathered here once so that the grouped GEMM
 // reads whole fragments); pad rows (row_tok < 0) and rows past meta[1] are skipped.
-template <int I8Q_MAXG>
+template <int I8Q_MAXG, bool RM = false>
 static __device__ __forceinline__ void i8q_quant_body(const unsigned short *__restrict__ x, unsigned char *__restrict__ q,
                                                       float *__restrict__ scale, int k,
                                                       const int *__restrict__ row_tok = nullptr,
@@ -105,7 +110,7 @@ static __device__ __forceinline__ void i8q_quant_body(const unsigned short *__re
       v[i][8 + 2 * w + 1] = __uint_as_float(hi[w] & 0xFFFF0000u);
     }
   }
-  i8q_tail<I8Q_MAXG>(v, G, q, scale, row, k);
+  i8q_tail<I8Q_MAXG, RM>(v, G, q, scale, row, k);
 }
 #define I8Q_QUANT(name, MAXG)                                                                                   \
   extern "C" __global__ __launch_bounds__(I8Q_T) void name(const unsigned short *__restrict__ x,                \
@@ -118,6 +123,17 @@ I8Q_QUANT(macaq_i8_quant_t256_g5, 5)
 I8Q_QUANT(macaq_i8_quant_t256_g2, 2)
 I8Q_QUANT(macaq_i8_quant_t256_g1, 1)
 #undef I8Q_QUANT
+// row-major codes (q[row * k + col]): the operand a routed layer's grouped GEMM gathers token rows from
+#define I8Q_QUANT_RM(name, MAXG)                                                                                \
+  extern "C" __global__ __launch_bounds__(I8Q_T) void name(const unsigned short *__restrict__ x,                \
+                                                           unsigned char *__restrict__ q, float *__restrict__ scale, \
+                                                           int k) {                                             \
+    i8q_quant_body<MAXG, true>(x, q, scale, k);                                                                 \
+  }
+I8Q_QUANT_RM(macaq_i8_quant_rm_t256, 8)
+I8Q_QUANT_RM(macaq_i8_quant_rm_t256_g2, 2)
+I8Q_QUANT_RM(macaq_i8_quant_rm_t256_g1, 1)
+#undef I8Q_QUANT_RM
 #define I8Q_QUANT_ROWS(name, MAXG)                                                                               \
   extern "C" __global__ __launch_bounds__(I8Q_T) void name(                                                      \
       const unsigned short *__restrict__ x, unsigned char *__restrict__ q, float *__restrict__ scale, int k,     \
@@ -262,6 +278,46 @@ extern "C" __global__ __launch_bounds__(256) void macaq_i8_silu_mul_quant_w64(
     }
   }
   i8q_tail_w64(v, G, q, scale, row, n);
+}
+
+// The same op for many rows, with the bf16 silu read from a table: `lut` holds the silu of every
+// bf16 bit pattern as macaq_silu_bf16_table wrote it (128 KiB), each workgroup copies it into LDS
+// once and its 16 waves then walk the rows, a wave a row, the 16 rows of an A tile on one workgroup
+// (tile = blockIdx.x + r * gridDim.x) so that the tile's 256-byte runs fill in one L2. The computed
+// form spends about 60 VALU operations an element on exp and the IEEE divide and is bound by them;
+// this one is bound by memory. Same bytes: the table is that form's own output.
+extern "C" __global__ __launch_bounds__(1024) void macaq_i8_silu_mul_quant_lut_w64(
+    const unsigned short *__restrict__ gu, unsigned char *__restrict__ q, float *__restrict__ scale, int n,
+    const int *__restrict__ row_tok, const int *__restrict__ meta, const unsigned short *__restrict__ lut) {
+#pragma clang fp contract(off)
+  __shared__ __attribute__((aligned(16))) unsigned short s_lut[65536];
+  for (int i = threadIdx.x; i < 65536 / 8; i += 1024) ((iu8_v4u *)s_lut)[i] = ((const iu8_v4u *)lut)[i];
+  __syncthreads();
+  const int G = n >> 4, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int rows = meta != nullptr ? meta[1] : 0x7FFFFFFF;
+  for (int tile = blockIdx.x;; tile += gridDim.x) {
+    const int row = tile * 16 + wave;
+    if (tile * 16 >= rows) break;
+    if (row >= rows || (row_tok != nullptr && row_tok[row] < 0)) continue;
+    const unsigned short *gr = gu + (size_t)row * 2 * n;
+    float v[I8Q_WG][16];
+#pragma unroll
+    for (int i = 0; i < I8Q_WG; ++i) {
+      const int g = lane + i * 64;
+      if (g >= G) continue;
+      union { iu8_v4u u[2]; unsigned short h[16]; } vg, vu;
+      vg.u[0] = *(const iu8_v4u *)(gr + g * 16);
+      vg.u[1] = *(const iu8_v4u *)(gr + g * 16 + 8);
+      vu.u[0] = *(const iu8_v4u *)(gr + n + g * 16);
+      vu.u[1] = *(const iu8_v4u *)(gr + n + g * 16 + 8);
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        const float t = iu8_bf16_f32(s_lut[vg.h[j]]);
+        v[i][j] = iu8_bf16_f32((unsigned short)iu8_bf16_bits(t * iu8_bf16_f32(vu.h[j])));
+      }
+    }
+    i8q_tail_w64(v, G, q, scale, row, n);
+  }
 }
 
 extern "C" __global__ __launch_bounds__(256) void macaq_silu_bf16_table(unsigned short *__restrict__ out) {

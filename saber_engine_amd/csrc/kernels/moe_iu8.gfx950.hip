@@ -7,14 +7,15 @@
 //   moe_iu8_route_topk8_sort_e128   logits bf16 [T,128] -> f32 softmax (IEEE-only exp) -> top-8,
 //        the LOWER expert id wins a tie -> w = p * (1 / (sum > 0 ? sum : 1)), sum in k order ->
 //        expert-major sort of the local experts [e_lo, e_lo + e_loc) into 16-row blocks, cut into
-//        tiles of `tile_blocks` blocks. One launch: a workgroup routes 32 tokens and counts its
+//        tiles of `tile_blocks` blocks. One launch: a workgroup routes 128 tokens and counts its
 //        routes per expert; the last workgroup to arrive scans and places every route. No atomic
 //        decides an output byte: a route's row = expert offset + earlier workgroups' count + its
 //        rank among this workgroup's earlier tokens, i.e. token order.
 //        Signature: crates/saber-kernels/src/abi.rs:354-374.
 //   moe_iu8_grouped_w4_{dec,pf}_g{0,1}   per tile of the table: one expert's weights through
 //        xptr[2e] (W4 fragments) / xptr[2e+1] (f32 row scales), activation rows gathered through
-//        row_tok (g1: gate+up) or in place (g0: down), C rows at the tile's row0. `dec` streams the
+//        row_tok (g1: from token-major A fragments; g2: from row-major codes, the reference's form,
+//        crates/saber-kernels/hip/moe_grouped.hip:67-74) or in place (g0: down), C rows at the tile's row0. `dec` streams the
 //        weights for tiles of <= 16 rows (few tokens: HBM-bound), `pf` is the MFMA tile for tiles of
 //        up to 256 rows of one expert. Signature: crates/saber-kernels/src/abi.rs:325-340 (p / cnt /
 //        pmax are the split-K workspaces of the reference's cells; this object does not split).
@@ -25,8 +26,9 @@
 
 #define MOE_E 128
 #define MOE_TOPK 8
-#define MOE_TPB 32
-#define MOE_THREADS 256
+#define MOE_TPB 128
+#define MOE_THREADS 1024
+#define MOE_CHUNK 36864  // rows of the placement tables held in LDS at a time (144 KiB)
 
 // e^x for x <= 0 from IEEE-rounded mul/add/rint/ldexp only (the law of
 // crates/saber-kernels/hip/moe_route.hip:43-57: n = rint(x*log2e), two-step Cody-Waite reduction,
@@ -46,6 +48,21 @@ static __device__ __forceinline__ float moe_exp_nonpos(float x) {
   p = p * r + 1.f;
   p = p * r + 1.f;
   return __builtin_ldexpf(p, (int)n);
+}
+
+// Lane exchanges inside a token's 8 lanes without the LDS crossbar's latency: DPP quad permutes for
+// the partners xor 1 and xor 2, and the half-row mirror (lane i <-> 7 - i), which after those two
+// brings in the other quad. Only for order-free reductions (max, arg-max under a total order).
+#define MOE_DPP_XOR1 0xB1    // quad_perm [1,0,3,2]
+#define MOE_DPP_XOR2 0x4E    // quad_perm [2,3,0,1]
+#define MOE_DPP_MIRROR8 0x141  // row_half_mirror
+template <int CTRL>
+static __device__ __forceinline__ int moe_dpp(int v) {
+  return __builtin_amdgcn_update_dpp(v, v, CTRL, 0xF, 0xF, false);
+}
+template <int CTRL>
+static __device__ __forceinline__ float moe_dppf(float v) {
+  return __int_as_float(moe_dpp<CTRL>(__float_as_int(v)));
 }
 
 // exclusive scan of one int a thread over the 256-thread workgroup; *total = the sum
@@ -78,7 +95,10 @@ extern "C" __global__ __launch_bounds__(MOE_THREADS) void moe_iu8_route_topk8_so
     int *__restrict__ tile_rows, int *__restrict__ expert_cnt, int *__restrict__ meta, int *__restrict__ blk_cnt,
     int *__restrict__ rank, int *__restrict__ arrive) {
 #pragma clang fp contract(off)
-  __shared__ int s_ids[MOE_TPB * MOE_TOPK];
+  __shared__ __attribute__((aligned(16))) int s_ids[MOE_TPB * MOE_TOPK];
+  __shared__ int s_part[MOE_THREADS / MOE_E][MOE_E];
+  __shared__ int s_rows[MOE_CHUNK];
+  __shared__ unsigned s_mask[MOE_E][MOE_TPB / 32];
   __shared__ int s_cnt[MOE_E];
   __shared__ int s_off[MOE_E], s_toff[MOE_E];
   __shared__ int s_wave[MOE_THREADS / 64];
@@ -87,6 +107,7 @@ extern "C" __global__ __launch_bounds__(MOE_THREADS) void moe_iu8_route_topk8_so
   const int nblk = gridDim.x, blk = blockIdx.x, t0 = blk * MOE_TPB;
 
   for (int e = tid; e < MOE_E; e += MOE_THREADS) s_cnt[e] = 0;
+  for (int i = tid; i < MOE_E * (MOE_TPB / 32); i += MOE_THREADS) s_mask[i / (MOE_TPB / 32)][i % (MOE_TPB / 32)] = 0u;
   for (int i = tid; i < MOE_TPB * MOE_TOPK; i += MOE_THREADS) s_ids[i] = -1;
   __syncthreads();
 
@@ -108,16 +129,19 @@ extern "C" __global__ __launch_bounds__(MOE_THREADS) void moe_iu8_route_topk8_so
       float mx = p[0];
 #pragma unroll
       for (int j = 1; j < 16; ++j) mx = fmaxf(mx, p[j]);
-#pragma unroll
-      for (int o = 4; o; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+      mx = fmaxf(mx, moe_dppf<MOE_DPP_XOR1>(mx));
+      mx = fmaxf(mx, moe_dppf<MOE_DPP_XOR2>(mx));
+      mx = fmaxf(mx, moe_dppf<MOE_DPP_MIRROR8>(mx));
       float s = 0.f;
 #pragma unroll
       for (int j = 0; j < 16; ++j) {
         p[j] = moe_exp_nonpos(p[j] - mx);
         s = s + p[j];
       }
-#pragma unroll
-      for (int o = 4; o; o >>= 1) s = s + __shfl_xor(s, o, 64);
+      // the sum's order is part of the law: partner xor 4 (a swizzle), then xor 2, then xor 1
+      s = s + __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(s), 0x101F));
+      s = s + moe_dppf<MOE_DPP_XOR2>(s);
+      s = s + moe_dppf<MOE_DPP_XOR1>(s);
       const float inv = 1.f / s;
 #pragma unroll
       for (int j = 0; j < 16; ++j) {
@@ -138,15 +162,15 @@ extern "C" __global__ __launch_bounds__(MOE_THREADS) void moe_iu8_route_topk8_so
             bj = j;
           }
         int bi = g * 16 + bj;
-#pragma unroll
-        for (int o = 4; o; o >>= 1) {
-          const float ov = __shfl_xor(bv, o, 64);
-          const int oi = __shfl_xor(bi, o, 64);
+        auto take = [&](float ov, int oi) {
           if (ov > bv || (ov == bv && oi < bi)) {
             bv = ov;
             bi = oi;
           }
-        }
+        };
+        take(moe_dppf<MOE_DPP_XOR1>(bv), moe_dpp<MOE_DPP_XOR1>(bi));
+        take(moe_dppf<MOE_DPP_XOR2>(bv), moe_dpp<MOE_DPP_XOR2>(bi));
+        take(moe_dppf<MOE_DPP_MIRROR8>(bv), moe_dpp<MOE_DPP_MIRROR8>(bi));
         if ((bi >> 4) == g) {
 #pragma unroll
           for (int j = 0; j < 16; ++j)
@@ -168,15 +192,29 @@ extern "C" __global__ __launch_bounds__(MOE_THREADS) void moe_iu8_route_topk8_so
   __syncthreads();
 
   // ---- phase 2: this workgroup's per-expert counts and each route's rank among the earlier
-  // tokens of this workgroup routed to the same expert (a token's experts are distinct)
+  // tokens of this workgroup routed to the same expert (a token's experts are distinct): a bit a
+  // token in the expert's 128-bit mask, the rank is the count of the bits below the token's
   for (int i = tid; i < MOE_TPB * MOE_TOPK; i += MOE_THREADS) {
-    const int e = s_ids[i], le = e - e_lo;
+    const int e = s_ids[i], le = e - e_lo, tl = i / MOE_TOPK;
+    if (e >= 0 && le >= 0 && le < e_loc) atomicOr(&s_mask[le][tl >> 5], 1u << (tl & 31));
+  }
+  __syncthreads();
+  for (int i = tid; i < MOE_TPB * MOE_TOPK; i += MOE_THREADS) {
+    const int e = s_ids[i], le = e - e_lo, tl = i / MOE_TOPK;
     if (e < 0 || le < 0 || le >= e_loc) continue;
-    atomicAdd(&s_cnt[le], 1);
-    const int before = (i / MOE_TOPK) * MOE_TOPK;
     int rk = 0;
-    for (int u = 0; u < before; ++u) rk += s_ids[u] == e;
+#pragma unroll
+    for (int w = 0; w < MOE_TPB / 32; ++w) {
+      const unsigned m = s_mask[le][w];
+      rk += __popc(w < (tl >> 5) ? m : w == (tl >> 5) ? m & ((1u << (tl & 31)) - 1u) : 0u);
+    }
     rank[(size_t)t0 * MOE_TOPK + i] = rk;
+  }
+  for (int e = tid; e < e_loc; e += MOE_THREADS) {
+    int c = 0;
+#pragma unroll
+    for (int w = 0; w < MOE_TPB / 32; ++w) c += __popc(s_mask[e][w]);
+    s_cnt[e] = c;
   }
   __syncthreads();
   for (int e = tid; e < e_loc; e += MOE_THREADS) blk_cnt[(size_t)blk * e_loc + e] = s_cnt[e];
@@ -190,24 +228,48 @@ extern "C" __global__ __launch_bounds__(MOE_THREADS) void moe_iu8_route_topk8_so
   __threadfence();  // acquire: every workgroup's topk_ids, rank and blk_cnt
   if (tid == 0) *arrive = 0;
 
-  // ---- phase 3 (the last workgroup): totals, each workgroup's base, offsets, tiles, placement
-  // (loads in batches of 8: the last workgroup works alone, so its time is load latency)
-  for (int e = tid; e < e_loc; e += MOE_THREADS) {
-    int run = 0;
-    for (int b0 = 0; b0 < nblk; b0 += 8) {
-      int c[8];
+  // ---- phase 3 (the last workgroup): totals, each workgroup's base, offsets, tiles, placement.
+  // It works alone, so its time is load latency: eight threads an expert scan an eighth of the
+  // workgroups' counts each, loads in batches of 8.
+  {
+    constexpr int PARTS = MOE_THREADS / MOE_E;
+    const int e = tid % MOE_E, part = tid / MOE_E;
+    const int chunk = (nblk + PARTS - 1) / PARTS, b_lo = min(part * chunk, nblk), b_hi = min(b_lo + chunk, nblk);
+    int sum = 0;
+    if (e < e_loc)
+      for (int b0 = b_lo; b0 < b_hi; b0 += 8) {
+        int c[8];
 #pragma unroll
-      for (int u = 0; u < 8; ++u)
-        c[u] = b0 + u < nblk ? __builtin_nontemporal_load(&blk_cnt[(size_t)(b0 + u) * e_loc + e]) : 0;
+        for (int u = 0; u < 8; ++u) c[u] = b0 + u < b_hi ? __builtin_nontemporal_load(&blk_cnt[(size_t)(b0 + u) * e_loc + e]) : 0;
 #pragma unroll
-      for (int u = 0; u < 8; ++u)
-        if (b0 + u < nblk) {
-          blk_cnt[(size_t)(b0 + u) * e_loc + e] = run;
-          run += c[u];
-        }
+        for (int u = 0; u < 8; ++u) sum += c[u];
+      }
+    s_part[part][e] = sum;
+    __syncthreads();
+    int run = 0, all = 0;
+#pragma unroll
+    for (int q = 0; q < PARTS; ++q) {
+      const int v = s_part[q][e];
+      run += q < part ? v : 0;
+      all += v;
     }
-    s_cnt[e] = run;
-    expert_cnt[e] = run;
+    if (e < e_loc) {
+      for (int b0 = b_lo; b0 < b_hi; b0 += 8) {
+        int c[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) c[u] = b0 + u < b_hi ? __builtin_nontemporal_load(&blk_cnt[(size_t)(b0 + u) * e_loc + e]) : 0;
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          if (b0 + u < b_hi) {
+            blk_cnt[(size_t)(b0 + u) * e_loc + e] = run;
+            run += c[u];
+          }
+      }
+      if (part == 0) {
+        s_cnt[e] = all;
+        expert_cnt[e] = all;
+      }
+    }
   }
   __syncthreads();
   const int G = tile_blocks, TR = 16 * tile_blocks;
@@ -247,10 +309,6 @@ extern "C" __global__ __launch_bounds__(MOE_THREADS) void moe_iu8_route_topk8_so
       tile_row0[s_toff[e] + j] = s_off[e] + j * TR;
       tile_rows[s_toff[e] + j] = min(TR, c - j * TR);
     }
-    for (int r = s_off[e] + c; r < s_off[e] + nb * 16; ++r) {
-      row_tok[r] = -1;
-      row_route[r] = -1;
-    }
   }
   for (int j = tid; j < sh_tiles; j += MOE_THREADS) {
     tile_expert[tiles_total + j] = e_loc;
@@ -262,33 +320,48 @@ extern "C" __global__ __launch_bounds__(MOE_THREADS) void moe_iu8_route_topk8_so
     row_route[sh_row0 + r] = -1;
   }
   __syncthreads();  // every expert's blk_cnt bases are written
-  for (int r0 = tid; r0 < T * MOE_TOPK; r0 += 8 * MOE_THREADS) {
-    int e[8], rk[8], base[8];
+  // Placement. A route's row is a scattered 4-byte store, and one workgroup scattering every route
+  // straight to memory is bound by that (about 3 ns a route). So the row tables are built in LDS, a
+  // chunk of MOE_CHUNK rows at a time (every slot starts as a pad, -1; each pass walks all routes
+  // and keeps those that land in the chunk), and go out in whole lines.
+  const int R = T * MOE_TOPK;
+  for (int c0 = 0; c0 < rows_total; c0 += MOE_CHUNK) {
+    const int cn = min(MOE_CHUNK, rows_total - c0);
+    for (int i = tid; i < cn; i += MOE_THREADS) s_rows[i] = -1;
+    __syncthreads();
+    for (int r0 = tid; r0 < R; r0 += 16 * MOE_THREADS) {
+      int e[16], rk[16], base[16];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      const int r = r0 + u * MOE_THREADS;
-      e[u] = r < T * MOE_TOPK ? __builtin_nontemporal_load(&topk_ids[r]) : -1;
-      rk[u] = r < T * MOE_TOPK ? __builtin_nontemporal_load(&rank[r]) : 0;
-    }
-#pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      const int r = r0 + u * MOE_THREADS, le = e[u] - e_lo;
-      base[u] = (r < T * MOE_TOPK && le >= 0 && le < e_loc) ? blk_cnt[(size_t)(r / MOE_TOPK / MOE_TPB) * e_loc + le] : 0;
-    }
-#pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      const int r = r0 + u * MOE_THREADS, le = e[u] - e_lo;
-      if (r >= T * MOE_TOPK) continue;
-      if (le < 0 || le >= e_loc) {
-        route_pos[r] = -1;
-        continue;
+      for (int u = 0; u < 16; ++u) {
+        const int r = r0 + u * MOE_THREADS;
+        e[u] = r < R ? __builtin_nontemporal_load(&topk_ids[r]) : -1;
+        rk[u] = r < R ? __builtin_nontemporal_load(&rank[r]) : 0;
       }
-      const int p = s_off[le] + base[u] + rk[u];
-      row_tok[p] = r / MOE_TOPK;
-      row_route[p] = r;
-      route_pos[r] = p;
+#pragma unroll
+      for (int u = 0; u < 16; ++u) {
+        const int r = r0 + u * MOE_THREADS, le = e[u] - e_lo;
+        base[u] = (r < R && le >= 0 && le < e_loc) ? blk_cnt[(size_t)(r / MOE_TOPK / MOE_TPB) * e_loc + le] : 0;
+      }
+#pragma unroll
+      for (int u = 0; u < 16; ++u) {
+        const int r = r0 + u * MOE_THREADS, le = e[u] - e_lo;
+        if (r >= R) continue;
+        const bool local = le >= 0 && le < e_loc;
+        const int p = local ? s_off[le] + base[u] + rk[u] : -1;
+        if (c0 == 0) route_pos[r] = p;
+        if (local && p >= c0 && p < c0 + cn) s_rows[p - c0] = r;
+      }
     }
+    __syncthreads();
+    for (int i = tid; i < cn; i += MOE_THREADS) {
+      const int r = s_rows[i];
+      row_route[c0 + i] = r;
+      row_tok[c0 + i] = r < 0 ? -1 : r / MOE_TOPK;
+    }
+    __syncthreads();
   }
+  if (rows_total == 0)  // no local route at all: the positions still have to be written
+    for (int r = tid; r < R; r += MOE_THREADS) route_pos[r] = -1;
 }
 
 // ---------------------------------------------------------------------------- grouped GEMMs
@@ -314,6 +387,48 @@ MOE_GROUPED_DEC(moe_iu8_grouped_w4_dec_g0, false, 1, 4, 8, 8, 20)
 // The MFMA-bound cell: a persistent launch of one workgroup a CU walks the work items
 // (tile, column block) of the live tiles, column blocks of one tile on neighbouring workgroups, the
 // load stream running across items (iu8_pf32.h). grid [256, 1, 1].
+// The walk is static (item = blockIdx.x + r * gridDim.x), and an expert's last tile is often nearly
+// empty and then cheap (the sparse forms of iu8_pf32.h); in table order some workgroups would draw
+// mostly full tiles and set the launch's time. So every workgroup first sorts the tiles the same
+// way -- those with more than one live 32-row block first, in table order, the light ones after
+// them -- and the round-robin deals each kind evenly.
+#define MOE_ORDER_CAP 4096  // tiles the ordering holds in LDS; beyond, table order
+template <int NTHR>
+static __device__ __forceinline__ void moe_tile_order(const int *__restrict__ tile_rows, int nt, unsigned short *s_order) {
+  __shared__ int s_w[NTHR / 64];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  auto block_sum = [&](int v, int &before) {  // sum over the workgroup; `before` = the waves ahead of this one
+    if (lane == 0) s_w[wave] = v;
+    __syncthreads();
+    int all = 0;
+    before = 0;
+#pragma unroll
+    for (int w = 0; w < NTHR / 64; ++w) {
+      const int x = s_w[w];
+      before += w < wave ? x : 0;
+      all += x;
+    }
+    __syncthreads();
+    return all;
+  };
+  int mine = 0, unused;
+  for (int t = tid; t < nt; t += NTHR) mine += tile_rows[t] > 32;
+#pragma unroll
+  for (int o = 32; o; o >>= 1) mine += __shfl_xor(mine, o, 64);
+  const int heavy_total = block_sum(mine, unused);
+  int run = 0;  // heavy tiles before this chunk
+  for (int base = 0; base < nt; base += NTHR) {
+    const int t = base + tid;
+    const bool h = t < nt && tile_rows[t] > 32;
+    const unsigned long long b = __ballot(h);
+    int wave_before;
+    const int chunk = block_sum(__popcll(b), wave_before);
+    const int hb = run + wave_before + __popcll(b & ((1ull << lane) - 1ull));  // heavy tiles before t
+    if (t < nt) s_order[h ? hb : heavy_total + (t - hb)] = (unsigned short)t;
+    run += chunk;
+  }
+  __syncthreads();
+}
 #define MOE_GROUPED_PF(name, GATHER, WMW, WNW, TM, TN)                                                           \
   extern "C" __global__ __launch_bounds__(WMW * WNW * 64) void name(                                              \
       const unsigned char *__restrict__ a, const unsigned long long *__restrict__ xptr,                           \
@@ -321,19 +436,28 @@ MOE_GROUPED_DEC(moe_iu8_grouped_w4_dec_g0, false, 1, 4, 8, 8, 20)
       const int *__restrict__ row_tok, const int *__restrict__ meta, const float *__restrict__ as,                \
       int *__restrict__ p, int *__restrict__ cnt, unsigned short *__restrict__ c, int n, int k, int pmax) {        \
     constexpr int BN = WNW * TN * 32;                                                                              \
-    const int gx = (n + BN - 1) / BN, total = meta[0] * gx;                                                        \
-    iu8_pf32_run<false, WMW, WNW, TM, TN, false, 3>(a, as, c, n, k, [&](int r, iu8_tile &t) {                      \
+    __shared__ unsigned short s_order[MOE_ORDER_CAP];                                                              \
+    const int nt = meta[0], gx = (n + BN - 1) / BN, total = nt * gx;                                               \
+    const bool ordered = nt <= MOE_ORDER_CAP;                                                                      \
+    if (ordered) moe_tile_order<WMW * WNW * 64>(tile_rows, nt, s_order);                                           \
+    iu8_pf32_run<false, WMW, WNW, TM, TN, false, 3, false, true, GATHER == 2>(a, as, c, n, k, [&](int r, iu8_tile &t) { \
       const int id = (int)blockIdx.x + r * (int)gridDim.x;                                                         \
       if (id >= total) return false;                                                                               \
-      const int tile = id / gx, bx = id - tile * gx, e = tile_expert[tile];                                        \
+      const int slot = id / gx, bx = id - slot * gx, tile = ordered ? (int)s_order[slot] : slot;                   \
+      const int e = tile_expert[tile];                                                                             \
       t = iu8_tile{iu8_rows{GATHER ? row_tok : nullptr, tile_row0[tile], min(tile_rows[tile], WMW * TM * 32)}, 0,  \
                    bx * (BN / 16), (const unsigned char *)xptr[2 * e], (const float *)xptr[2 * e + 1]};            \
       return true;                                                                                                 \
     });                                                                                                            \
   }
 // tiles of up to 128 rows (tile_blocks 8) on the 128 x 256 tile of 2 x 4 waves
-MOE_GROUPED_PF(moe_iu8_grouped_w4_pf_g1, true, 2, 4, 2, 2)
-MOE_GROUPED_PF(moe_iu8_grouped_w4_pf_g0, false, 2, 4, 2, 2)
+MOE_GROUPED_PF(moe_iu8_grouped_w4_pf_g2, 2, 2, 4, 2, 2)
+MOE_GROUPED_PF(moe_iu8_grouped_w4_pf_g1, 1, 2, 4, 2, 2)
+MOE_GROUPED_PF(moe_iu8_grouped_w4_pf_g0, 0, 2, 4, 2, 2)
+// tiles of up to 256 rows (tile_blocks 16) on the 256 x 256 tile, the dense GEMM's fastest cell
+MOE_GROUPED_PF(moe_iu8_grouped_w4_pf16_g2, 2, 2, 4, 4, 2)
+MOE_GROUPED_PF(moe_iu8_grouped_w4_pf16_g1, 1, 2, 4, 4, 2)
+MOE_GROUPED_PF(moe_iu8_grouped_w4_pf16_g0, 0, 2, 4, 4, 2)
 #undef MOE_GROUPED_PF
 
 // ---------------------------------------------------------------------------- combine

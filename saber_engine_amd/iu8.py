@@ -67,7 +67,7 @@ class Counters(C.Structure):
 
 
 MOE_TABLE_FIELDS = ("topk_ids", "topk_w", "route_pos", "row_tok", "row_route", "tile_expert", "tile_row0", "tile_rows",
-                    "expert_cnt", "meta", "blk_cnt", "rank", "arrive")
+                    "expert_cnt", "meta", "blk_cnt", "rank", "arrive", "silu_lut")
 
 
 class MoeTables(C.Structure):
@@ -105,6 +105,7 @@ def lib():
         L.saber_iu8_close.argtypes = [C.c_void_p]
         L.saber_iu8_launch.argtypes = [C.c_void_p, C.POINTER(Desc), C.POINTER(Binding), C.c_uint32, C.c_void_p]
         L.saber_iu8_quant.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32, C.c_uint32, C.c_void_p]
+        L.saber_iu8_quant_rowmajor.argtypes = L.saber_iu8_quant.argtypes
         L.saber_iu8_gemm.argtypes = [C.c_void_p, C.c_int] + [C.c_void_p] * 5 + [C.c_uint32] * 3 + [C.c_void_p] * 3
         L.saber_iu8_gemm_acc.argtypes = [C.c_void_p, C.c_int] + [C.c_void_p] * 3 + [C.c_uint32] * 3 + [C.c_void_p]
         L.saber_iu8_fused_holds.argtypes = [C.c_uint32, C.c_uint32]
@@ -299,6 +300,9 @@ class Context:
 
     def quant(self, x, q, scale, m, k, stream=0):
         _check(lib().saber_iu8_quant(self._h, x, q, scale, m, k, stream))
+
+    def quant_rowmajor(self, x, q, scale, m, k, stream=0):
+        _check(lib().saber_iu8_quant_rowmajor(self._h, x, q, scale, m, k, stream))
 
     def gemm(self, wkind, a, a_scale, w, w_scale, c, m, n, k, partial=None, counter=None, stream=0):
         _check(lib().saber_iu8_gemm(self._h, wkind, a, a_scale, w, w_scale, c, m, n, k, partial, counter, stream))

@@ -1,5 +1,5 @@
 """The routed-expert layer as a launch train over the C ABI: route+sort -> per-token quant ->
-grouped gate+up (gathered) -> SiLU*up requant -> grouped down -> weighted combine.  The train and
+grouped gate+up (token rows gathered) -> SiLU*up requant -> grouped down -> weighted combine.  The train and
 its buffers follow the reference's MoE block (crates/saber-kernels/src/moe.rs:9-28, 142-171); the
 arithmetic of every GEMM is the iu8 contract.  torch is used for device memory only.
 """
@@ -25,14 +25,17 @@ class MoeLayerIU8:
             expert_cnt=torch.zeros(experts, **i32), meta=torch.zeros(8, **i32),
             blk_cnt=torch.zeros(((tokens + 31) // 32) * experts, **i32), rank=torch.zeros(R, **i32),
             arrive=torch.zeros(1, **i32))          # persistent: zeroed once, left zero by the kernel
+        # the bf16 silu of every bf16 input as the device computes it, for the table form of SiLU*up
+        self.buf["silu_lut"] = torch.zeros(65536, dtype=torch.int16, device=device)
+        ctx.silu_table(self.buf["silu_lut"].data_ptr())
+        torch.cuda.synchronize()
         self.tables = iu8.MoeTables(*[self.buf[n].data_ptr() for n in iu8.MOE_TABLE_FIELDS])
         u8 = dict(dtype=torch.uint8, device=device)
-        # the streaming cell (16-row tiles) gathers token rows inside the grouped GEMM; the MFMA cell
-        # runs on rows gathered and quantised once into expert-major order
-        self.gather_in_gemm = self.tb == 1
-        rows1 = tokens if self.gather_in_gemm else self.rows_cap
-        self.q1 = torch.zeros(iu8.a_bytes(rows1, hidden), **u8)
-        self.s1 = torch.zeros(rows1, dtype=torch.float32, device=device)
+        # tokens are quantised once and the grouped gate+up GEMM gathers their rows: the streaming cell
+        # (16-row tiles) from the A edge, the MFMA cells from row-major codes (whole 64-byte runs a row)
+        self.gather = 1 if self.tb == 1 else 2
+        self.q1 = torch.zeros(max(iu8.a_bytes(tokens, hidden), tokens * hidden), **u8)
+        self.s1 = torch.zeros(tokens, dtype=torch.float32, device=device)
         self.gu = torch.zeros((self.rows_cap, 2 * inter), dtype=torch.int16, device=device)
         self.q2 = torch.zeros(iu8.a_bytes(self.rows_cap, inter), **u8)
         self.s2 = torch.zeros(self.rows_cap, dtype=torch.float32, device=device)
@@ -53,12 +56,12 @@ class MoeLayerIU8:
         """x bf16 bits [T,H] (int16 tensor), logits bf16 bits [T,E]; every launch on `stream`."""
         c, T, E, k, H, I = self.ctx, self.T, self.E, self.topk, self.H, self.I
         c.moe_route(logits.data_ptr(), T, E, k, self.tb, self.tables, stream)
-        if self.gather_in_gemm:
+        if self.gather == 1:
             c.quant(x.data_ptr(), self.q1.data_ptr(), self.s1.data_ptr(), T, H, stream)
         else:
-            c.moe_quant_rows(x.data_ptr(), self.q1.data_ptr(), self.s1.data_ptr(), H, self.rows_cap, self.tables, stream)
+            c.quant_rowmajor(x.data_ptr(), self.q1.data_ptr(), self.s1.data_ptr(), T, H, stream)
         c.moe_grouped(self.q1.data_ptr(), self.s1.data_ptr(), self.xptr_gu.data_ptr(), self.gu.data_ptr(), 2 * I, H,
-                      self.gather_in_gemm, T, E, k, self.tb, self.tables, stream)
+                      self.gather, T, E, k, self.tb, self.tables, stream)
         c.moe_silu_mul_quant(self.gu.data_ptr(), self.q2.data_ptr(), self.s2.data_ptr(), I, self.rows_cap, self.tables, stream)
         c.moe_grouped(self.q2.data_ptr(), self.s2.data_ptr(), self.xptr_dn.data_ptr(), self.y.data_ptr(), H, I, False,
                       T, E, k, self.tb, self.tables, stream)

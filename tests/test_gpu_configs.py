@@ -247,5 +247,5 @@ def test_config4_moe_prefill_shape(ctx):
     say("config 4: T=4096 E=128 top-8 H=4096 I=1536")
     case = synth.moe_case(T=4096, E=128, topk=8, H=4096, I=1536, seed=0, experts=4)
     layer = run_layer(ctx, case)
-    assert layer.tb == 8
+    assert layer.tb == 16 and layer.gather == 2
     check_layer(layer, case, taps=False)

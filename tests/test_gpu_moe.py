@@ -69,7 +69,7 @@ def check_layer(layer, case, taps=True):
     np.testing.assert_array_equal(host_u16(layer.out), r["out"])
 
 
-@pytest.mark.parametrize("T,tb", [(1, None), (16, None), (16, 8), (100, None), (300, None)])
+@pytest.mark.parametrize("T,tb", [(1, None), (16, None), (16, 8), (100, None), (300, None), (40, 16), (300, 16), (700, 16)])
 def test_moe_layer_small_experts(ctx, T, tb):
     say(f"moe layer T={T} tile_blocks={tb} E=128 top-8 H=512 I=256")
     case = synth.moe_case(T=T, E=128, topk=8, H=512, I=256, seed=T, experts=8)
@@ -88,8 +88,121 @@ def test_moe_router_ties_and_skew(ctx):
     check_layer(layer, case)
 
 
+@pytest.mark.parametrize("T", [129, 1000, 4096, 5001])
+def test_moe_router_many_workgroups(ctx, T):
+    """The router alone at token counts that take several workgroups (128 tokens each): ids, weights
+    and the whole sort / tile table against the oracle, twice on the same tables."""
+    say(f"moe router T={T}")
+    E, k = 128, 8
+    rng = np.random.default_rng(T)
+    logits = synth.f32_to_bf16_bits(rng.standard_normal((T, E)).astype(np.float32))
+    layer = MoeLayerIU8(ctx, T, E, k, 512, 256)
+    lg = dev_bf16_bits(logits)
+    for _ in range(2):
+        ctx.moe_route(lg.data_ptr(), T, E, k, layer.tb, layer.tables)
+    torch.cuda.synchronize()
+    ids, w = ref.route(logits, k)
+    lay = ref.sort_layout(ids, E, layer.tb)
+    b = {n: t.cpu().numpy() for n, t in layer.buf.items()}
+    np.testing.assert_array_equal(b["topk_ids"].reshape(T, k), ids)
+    np.testing.assert_array_equal(b["topk_w"].reshape(T, k).view(np.uint32), w.view(np.uint32))
+    assert int(b["meta"][0]) == lay["tiles"] and int(b["meta"][1]) == lay["rows"] and int(b["meta"][3]) == T * k
+    assert int(b["arrive"][0]) == 0
+    np.testing.assert_array_equal(b["expert_cnt"], lay["expert_cnt"])
+    np.testing.assert_array_equal(b["route_pos"].reshape(T, k), lay["route_pos"])
+    np.testing.assert_array_equal(b["row_tok"][:lay["rows"]], lay["row_tok"])
+    nt = lay["tiles"]
+    np.testing.assert_array_equal(b["tile_expert"][:nt], lay["tile_expert"])
+    np.testing.assert_array_equal(b["tile_row0"][:nt], lay["tile_row0"])
+    np.testing.assert_array_equal(b["tile_rows"][:nt], lay["tile_rows"])
+
+
 def test_moe_layer_config4_decode_shape(ctx):
     say("moe layer config 4: T=16 E=128 top-8 H=4096 I=1536")
     case = synth.moe_case(T=16, E=128, topk=8, H=4096, I=1536, seed=0, experts=6)
     layer = run_layer(ctx, case)
     check_layer(layer, case, taps=True)
+
+
+def test_quant_rowmajor_matches_the_oracle_codes(ctx):
+    say("row-major per-token quantisation")
+    rng = np.random.default_rng(3)
+    for M, K in ((5, 512), (33, 4096), (7, 5120)):
+        X = synth.activations(rng, M, K)
+        q = torch.full((M * K,), 0x55, dtype=torch.uint8, device="cuda")
+        s = torch.zeros(M, dtype=torch.float32, device="cuda")
+        ctx.quant_rowmajor(dev_bf16_bits(X).data_ptr(), q.data_ptr(), s.data_ptr(), M, K)
+        torch.cuda.synchronize()
+        qh, sh = ref.quant_bf16(X)
+        np.testing.assert_array_equal(q.cpu().numpy().view(np.int8).reshape(M, K), qh)
+        np.testing.assert_array_equal(s.cpu().numpy().view(np.uint32), sh.view(np.uint32))
+
+
+def test_moe_layer_config4_prefill_shape(ctx):
+    """T=4096 at the full expert shape: the tables against the oracle, every route of a sample of
+    tokens (those that land in an expert's nearly empty last tile among them) through both GEMMs
+    and the combine against the oracle, and the whole output against the same layer run on 128-row
+    tiles over rows gathered by the quantiser -- other cells, other operand orders, same bytes."""
+    T, E, k, H, I = 4096, 128, 8, 4096, 1536
+    say(f"moe layer config 4: T={T} E=128 top-8 H=4096 I=1536")
+    case = synth.moe_case(T=T, E=E, topk=k, H=H, I=I, seed=1, experts=3)
+    ne = 3
+    fgu = torch.from_numpy(np.stack([iu8.repack_w4(case["Wgu"][e]) for e in range(ne)])).cuda()
+    fdn = torch.from_numpy(np.stack([iu8.repack_w4(case["Wdn"][e]) for e in range(ne)])).cuda()
+    idx = torch.arange(E, device="cuda") % ne
+    wgu, wdn = fgu[idx].contiguous(), fdn[idx].contiguous()
+    wsgu, wsdn = torch.from_numpy(case["wsgu"]).cuda(), torch.from_numpy(case["wsdn"]).cuda()
+    x, lg = dev_bf16_bits(case["X"]), dev_bf16_bits(case["logits"])
+    layer = MoeLayerIU8(ctx, T, E, k, H, I)
+    assert layer.tb == 16 and layer.gather == 2
+    layer.set_weights(wgu, wsgu, wdn, wsdn)
+    layer.gu.fill_(0x7FC0)
+    layer.y.fill_(0x7FC0)
+    layer.forward(x, lg)
+    layer.forward(x, lg)
+    torch.cuda.synchronize()
+    ids, w = ref.route(case["logits"], k)
+    lay = ref.sort_layout(ids, E, layer.tb)
+    b = {n: t.cpu().numpy() for n, t in layer.buf.items()}
+    np.testing.assert_array_equal(b["topk_ids"].reshape(T, k), ids)
+    np.testing.assert_array_equal(b["route_pos"].reshape(T, k), lay["route_pos"])
+    np.testing.assert_array_equal(b["row_tok"][:lay["rows"]], lay["row_tok"])
+    nt = lay["tiles"]
+    assert int(b["meta"][0]) == nt
+    np.testing.assert_array_equal(b["tile_rows"][:nt], lay["tile_rows"])
+    # sample: the token of the last route of every expert whose last tile holds at most 32 rows, and a few others
+    cnt = lay["expert_cnt"]
+    off = np.concatenate([[0], np.cumsum((cnt + 15) // 16 * 16)])
+    tail = [int(lay["row_tok"][off[e] + cnt[e] - 1]) for e in range(E) if 0 < cnt[e] % 256 <= 32][:10]
+    assert tail, "the draw has no expert with a nearly empty last tile"
+    toks = sorted(set(tail + [0, 1, 2047, 4095] + list(np.random.default_rng(0).integers(0, T, 6))))
+    gu_d, y_d, out_d = host_u16(layer.gu), host_u16(layer.y), host_u16(layer.out)
+    for t in toks:
+        rows = []
+        for j in range(k):
+            e, p = int(ids[t, j]), int(lay["route_pos"][t, j])
+            r1 = ref.linear(case["X"][t:t + 1], case["Wgu"][e], case["wsgu"][e], False)
+            np.testing.assert_array_equal(gu_d[p], r1["C"][0], err_msg=f"gate+up token {t} route {j}")
+            q2, s2, _ = ref.silu_mul_quant(r1["C"])
+            S, _ = ref.gemm_fast(q2, case["Wdn"][e], False)
+            yrow = ref.epilogue(S, s2, case["wsdn"][e], False)
+            np.testing.assert_array_equal(y_d[p], yrow[0], err_msg=f"down token {t} route {j}")
+            rows.append(yrow[0])
+        want = ref.combine(np.stack(rows), w[t:t + 1], np.arange(k, dtype=np.int32)[None], H)
+        np.testing.assert_array_equal(out_d[t], want[0], err_msg=f"combine token {t}")
+    # the same layer through the 128-row cells on rows the quantiser gathered
+    tb = 8
+    other = MoeLayerIU8(ctx, T, E, k, H, I, tile_blocks=tb)
+    other.set_weights(wgu, wsgu, wdn, wsdn)
+    q1 = torch.zeros(iu8.a_bytes(other.rows_cap, H), dtype=torch.uint8, device="cuda")
+    s1 = torch.zeros(other.rows_cap, dtype=torch.float32, device="cuda")
+    ctx.moe_route(lg.data_ptr(), T, E, k, tb, other.tables)
+    ctx.moe_quant_rows(x.data_ptr(), q1.data_ptr(), s1.data_ptr(), H, other.rows_cap, other.tables)
+    ctx.moe_grouped(q1.data_ptr(), s1.data_ptr(), other.xptr_gu.data_ptr(), other.gu.data_ptr(), 2 * I, H, 0, T, E, k, tb, other.tables)
+    ctx.moe_silu_mul_quant(other.gu.data_ptr(), other.q2.data_ptr(), other.s2.data_ptr(), I, other.rows_cap, other.tables)
+    ctx.moe_grouped(other.q2.data_ptr(), other.s2.data_ptr(), other.xptr_dn.data_ptr(), other.y.data_ptr(), H, I, 0, T, E, k, tb, other.tables)
+    ctx.moe_combine(other.y.data_ptr(), other.tables, other.out.data_ptr(), T, k, H)
+    torch.cuda.synchronize()
+    live = lay["row_tok"] >= 0
+    np.testing.assert_array_equal(host_u16(other.y)[:lay["rows"]][live], y_d[:lay["rows"]][live])
+    np.testing.assert_array_equal(host_u16(other.out), out_d)
