@@ -522,13 +522,17 @@ uint32_t saber_iu8_moe_tiles_cap(uint32_t tokens, uint32_t topk, uint32_t expert
   const uint32_t r = tokens * topk;
   return std::min(r, experts) + r / (16u * std::max(tile_blocks, 1u)) + 1u;
 }
-// Rows a tile (x16): 16-row tiles on the streaming cell while a tile a route's expert is the common
-// case; from about 96 routes an expert the 256-row MFMA cell (one tile an expert more often than
-// not, and the dense GEMM's fastest shape), between them the 128-row one. Speed data of this card:
-// 128 experts, top-8, 4096 x 1536: T=1024 400 vs 431 us a layer (8 vs 16), T=2048 592 vs 531.
+// Rows a tile (x16). 16-row tiles on the streaming cell while routes are so few that most tiles hold
+// a route or two (up to 5 routes an expert on average); above, the MFMA cells, whose sparse forms make
+// a thinly filled tile cost about its weight traffic and which stream an expert's weights once
+// instead of once a 16-row tile: 128-row tiles up to 96 routes an expert, 256-row tiles (one tile an
+// expert more often than not, on the dense GEMM's fastest shape) from there. Speed data of this card,
+// 128 experts, top-8, 4096 x 1536, us a layer at tile_blocks 1 / 8 / 16: T=32 256 / 316 / 328,
+// T=64 324 / 341 / 347, T=128 477 / 362 / 362, T=256 730 / 376 / 379, T=512 1282 / 370 / 396,
+// T=1024 2349 / 430 / 469, T=2048 - / 650 / 597, T=4096 - / 982 / 952.
 uint32_t saber_iu8_moe_tile_blocks(uint32_t tokens, uint32_t topk, uint32_t experts) {
   const uint64_t routes = (uint64_t)tokens * topk;
-  if (routes <= 16ull * experts) return 1u;
+  if (routes <= 5ull * experts) return 1u;
   return routes >= 96ull * experts ? 16u : 8u;
 }
 

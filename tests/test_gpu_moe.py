@@ -69,7 +69,7 @@ def check_layer(layer, case, taps=True):
     np.testing.assert_array_equal(host_u16(layer.out), r["out"])
 
 
-@pytest.mark.parametrize("T,tb", [(1, None), (16, None), (16, 8), (100, None), (300, None), (40, 16), (300, 16), (700, 16)])
+@pytest.mark.parametrize("T,tb", [(1, None), (16, None), (16, 8), (100, None), (100, 1), (300, None), (300, 1), (40, 16), (300, 16), (700, 16)])
 def test_moe_layer_small_experts(ctx, T, tb):
     say(f"moe layer T={T} tile_blocks={tb} E=128 top-8 H=512 I=256")
     case = synth.moe_case(T=T, E=128, topk=8, H=512, I=256, seed=T, experts=8)

@@ -143,6 +143,13 @@ def test_launch_law_shares_k_only_on_deep_narrow_tile_gemms():
         assert iu8.gemm_workspace(wk, m, n, k) == (0, 0)
 
 
+def test_moe_tile_law_thresholds():
+    """16-row streaming tiles up to 5 routes an expert, 128-row MFMA tiles up to 96, 256-row above."""
+    got = {t: iu8.moe_tile_blocks(t, 8, 128) for t in (1, 16, 80, 81, 256, 1535, 1536, 4096)}
+    assert got == {1: 1, 16: 1, 80: 1, 81: 8, 256: 8, 1535: 8, 1536: 16, 4096: 16}
+    assert iu8.moe_tiles_cap(4096, 8, 128, 16) == 128 + 128 + 1 and iu8.moe_rows_cap(4096, 8, 128) == 32768 + 15 * 128
+
+
 def test_explicit_split_declares_its_workspaces():
     d = iu8.describe("macaq_iu8_dec_w4_tm1", 4, 5120, 17408, ks=4)
     assert d.ks == 4 and d.grid[2] == 4
