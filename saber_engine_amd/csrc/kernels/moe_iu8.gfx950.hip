@@ -429,7 +429,7 @@ static __device__ __forceinline__ void moe_tile_order(const int *__restrict__ ti
   }
   __syncthreads();
 }
-#define MOE_GROUPED_PF(name, GATHER, WMW, WNW, TM, TN)                                                           \
+#define MOE_GROUPED_PF(name, GATHER, WMW, WNW, TM, TN, ST)                                                           \
   extern "C" __global__ __launch_bounds__(WMW * WNW * 64) void name(                                              \
       const unsigned char *__restrict__ a, const unsigned long long *__restrict__ xptr,                           \
       const int *__restrict__ tile_expert, const int *__restrict__ tile_row0, const int *__restrict__ tile_rows,  \
@@ -440,7 +440,7 @@ static __device__ __forceinline__ void moe_tile_order(const int *__restrict__ ti
     const int nt = meta[0], gx = (n + BN - 1) / BN, total = nt * gx;                                               \
     const bool ordered = nt <= MOE_ORDER_CAP;                                                                      \
     if (ordered) moe_tile_order<WMW * WNW * 64>(tile_rows, nt, s_order);                                           \
-    iu8_pf32_run<false, WMW, WNW, TM, TN, false, 3, false, true, GATHER == 2>(a, as, c, n, k, [&](int r, iu8_tile &t) { \
+    iu8_pf32_run<false, WMW, WNW, TM, TN, false, ST, false, true, GATHER == 2>(a, as, c, n, k, [&](int r, iu8_tile &t) { \
       const int id = (int)blockIdx.x + r * (int)gridDim.x;                                                         \
       if (id >= total) return false;                                                                               \
       const int slot = id / gx, bx = id - slot * gx, tile = ordered ? (int)s_order[slot] : slot;                   \
@@ -451,13 +451,13 @@ static __device__ __forceinline__ void moe_tile_order(const int *__restrict__ ti
     });                                                                                                            \
   }
 // tiles of up to 128 rows (tile_blocks 8) on the 128 x 256 tile of 2 x 4 waves
-MOE_GROUPED_PF(moe_iu8_grouped_w4_pf_g2, 2, 2, 4, 2, 2)
-MOE_GROUPED_PF(moe_iu8_grouped_w4_pf_g1, 1, 2, 4, 2, 2)
-MOE_GROUPED_PF(moe_iu8_grouped_w4_pf_g0, 0, 2, 4, 2, 2)
+MOE_GROUPED_PF(moe_iu8_grouped_w4_pf_g2, 2, 2, 4, 2, 2, 4)
+MOE_GROUPED_PF(moe_iu8_grouped_w4_pf_g1, 1, 2, 4, 2, 2, 4)
+MOE_GROUPED_PF(moe_iu8_grouped_w4_pf_g0, 0, 2, 4, 2, 2, 4)
 // tiles of up to 256 rows (tile_blocks 16) on the 256 x 256 tile, the dense GEMM's fastest cell
-MOE_GROUPED_PF(moe_iu8_grouped_w4_pf16_g2, 2, 2, 4, 4, 2)
-MOE_GROUPED_PF(moe_iu8_grouped_w4_pf16_g1, 1, 2, 4, 4, 2)
-MOE_GROUPED_PF(moe_iu8_grouped_w4_pf16_g0, 0, 2, 4, 4, 2)
+MOE_GROUPED_PF(moe_iu8_grouped_w4_pf16_g2, 2, 2, 4, 4, 2, 3)
+MOE_GROUPED_PF(moe_iu8_grouped_w4_pf16_g1, 1, 2, 4, 4, 2, 3)
+MOE_GROUPED_PF(moe_iu8_grouped_w4_pf16_g0, 0, 2, 4, 4, 2, 3)
 #undef MOE_GROUPED_PF
 
 // ---------------------------------------------------------------------------- combine
