@@ -322,12 +322,20 @@ const PfVariant *pf_cell(bool w8, uint32_t m, uint32_t n, uint32_t k) {
     const uint64_t tiles = (uint64_t)((n + v->block_n() - 1) / v->block_n()) * ((m + v->block_m() - 1) / v->block_m());
     const uint64_t grid = std::min<uint64_t>(tiles, (uint64_t)CU_COUNT * v->occ);
     const uint64_t per_wg = (tiles + grid - 1) / grid;
-    const double cu_tiles = (double)per_wg * std::min<uint64_t>(v->occ, (grid + CU_COUNT - 1) / CU_COUNT);
+    double cu_tiles = (double)per_wg * std::min<uint64_t>(v->occ, (grid + CU_COUNT - 1) / CU_COUNT);
+    // the 256 x 256 cell runs a thin last round (at most half the workgroups) as quarter tiles on the
+    // 128 x 128 cell, each a quarter of the work at that cell's rate
+    const uint64_t q = tiles / grid, rem = tiles - q * grid;
+    if (!strcmp(c.tile, "tn4_lbk64") && q >= 1 && rem > 0 && 2 * rem <= grid)
+      cu_tiles = (double)q + (double)((4 * rem + grid - 1) / grid) * 0.25 * (13.27 / 7.85);
     const double tile_bytes = bm * k + bn * k * (w8 ? 1.0 : 0.5);
     const double t_mfma = cu_tiles * bm * bn * k * 2.0 / (c.tops_per_cu * 1e6);
     const double t_cu = cu_tiles * tile_bytes / (CU_GBPS * 1e3);
     const double t_l2 = (double)tiles * tile_bytes / (L2_TBPS * 1e6);
-    const double t = FIXED_US + std::max(t_mfma, std::max(t_cu, t_l2));
+    // the two-a-CU 128 x 128 cell alone on a CU (no more workgroups than CUs) has four waves to hide
+    // its latencies with and measured 9-12 % behind the eight-wave 128 x 128 cell there
+    const double lone = (!strcmp(c.tile, "t128x128_o2") && grid <= CU_COUNT) ? 1.15 : 1.0;
+    const double t = FIXED_US + lone * std::max(t_mfma, std::max(t_cu, t_l2));
     if (!best || t < best_t) best = v, best_t = t;
   }
   return best;

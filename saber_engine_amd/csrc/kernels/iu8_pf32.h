@@ -55,16 +55,28 @@ struct iu8_tile {
 // consecutive workgroup ids round-robin over the 8 XCDs (each with its own L2): in every round an
 // XCD's G/8 workgroups take one run of consecutive tile ids, and ids walk M-fastest in groups of
 // 8 row blocks, so co-resident workgroups share W columns and A rows in their L2.
-static __device__ __forceinline__ bool iu8_dense_tile_at(int r, int gx, int gy, int &bx, int &by) {
-  const int G = gridDim.x, w = blockIdx.x, total = gx * gy;
-  const int id = (G & 7) == 0 ? ((r * 8 + (w & 7)) * (G >> 3) + (w >> 3)) : (w + r * G);
-  if (id >= total) return false;
+static __device__ __forceinline__ void iu8_dense_tile_of(int id, int gx, int gy, int &bx, int &by) {
   constexpr int GM = 8;
   const int group = id / (GM * gx), first = group * GM, gm = min(GM, gy - first);
   const int rr = id - group * (GM * gx);
   by = first + rr % gm;
   bx = rr / gm;
+}
+static __device__ __forceinline__ bool iu8_dense_tile_at(int r, int gx, int gy, int &bx, int &by) {
+  const int G = gridDim.x, w = blockIdx.x, total = gx * gy;
+  const int id = (G & 7) == 0 ? ((r * 8 + (w & 7)) * (G >> 3) + (w >> 3)) : (w + r * G);
+  if (id >= total) return false;
+  iu8_dense_tile_of(id, gx, gy, bx, by);
   return true;
+}
+
+// LDS bytes of a cell's stages (what iu8_pf32_run declares, or expects from its caller).
+template <bool W8, int WMW, int WNW, int TM, int TN, int STMAX>
+constexpr int iu8_pf32_lds_bytes() {
+  constexpr int STAGE = WMW * TM * 2 * 2048 + WNW * TN * 2 * (W8 ? 2048 : 1024);
+  constexpr int NFIT = 160 * 1024 / STAGE;
+  constexpr int NST = STMAX < 2 ? 2 : (STMAX < NFIT ? STMAX : (NFIT < 2 ? 2 : NFIT));
+  return NST * STAGE;
 }
 
 // A split of K over gridDim.z (P, cnt not null): the workgroups of share z run steps [z*spb, (z+1)*spb)
@@ -80,10 +92,11 @@ static __device__ __forceinline__ bool iu8_dense_tile_at(int r, int gx, int gy, 
 // all past the tile's rows, or all but the first, runs the K loop in a form with none, or one, of
 // its TM row blocks -- the same loads, barriers and stage walk, a fraction of the MFMAs and LDS reads
 // -- so such a tile costs its operand traffic instead of a full tile's matrix work.
-template <bool W8, int WMW, int WNW, int TM, int TN, bool ACC, int STMAX, bool DEEP = false, bool SPARSE = false, bool ARM = false, class TileAt>
+template <bool W8, int WMW, int WNW, int TM, int TN, bool ACC, int STMAX, bool DEEP = false, bool SPARSE = false, bool ARM = false, bool EXT_LDS = false, class TileAt>
 __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const float *__restrict__ as,
                                              void *__restrict__ Cv, int N, int K, TileAt tile_at,
-                                             int *__restrict__ P = nullptr, int *__restrict__ cnt = nullptr) {
+                                             int *__restrict__ P = nullptr, int *__restrict__ cnt = nullptr,
+                                             iu8_u8 *ext_lds = nullptr) {
   // tile_at(r, t): fills the workgroup's r-th tile, false when it has none
   constexpr int NWAVE = WMW * WNW;
   constexpr int BMT = WMW * TM * 2, BNT = WNW * TN * 2;  // 16-row tiles a workgroup, both ways
@@ -99,7 +112,15 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
   static_assert((NST - 2) * (A_FR / NWAVE + W_FR / NWAVE) <= 63, "the in-flight count fits s_waitcnt's vmcnt field");
   static_assert(!DEEP || NST >= 3, "the deep form reads a stage a step ahead of its MFMAs");
   static_assert(!(DEEP && SPARSE), "the sparse forms exist for the phased loop only");
-  __shared__ __attribute__((aligned(1024))) iu8_u8 smem[NST * STAGE];
+  // EXT_LDS: the stages live in the caller's LDS block (1-KiB aligned, iu8_pf32_lds_bytes of this cell),
+  // for a kernel that runs two cells one after the other in the same memory
+  iu8_u8 *smem;
+  if constexpr (EXT_LDS) {
+    smem = ext_lds;
+  } else {
+    __shared__ __attribute__((aligned(1024))) iu8_u8 own_lds[NST * STAGE];
+    smem = own_lds;
+  }
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);

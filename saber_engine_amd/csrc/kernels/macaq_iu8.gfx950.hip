@@ -65,20 +65,58 @@ IU8_DECQ(macaq_iu8_decq_w8_tm1, true, 4)
 #undef IU8_DECQX
 
 // Persistent launch: gridDim.x workgroups (one or OCC a CU) walk the tiles of the m x n output.
+//
+// The 256 x 256 cell's last round. With G workgroups and q * G + rem tiles, the last round keeps rem
+// workgroups busy and the others idle for a whole tile (a fifth of the launch at 1,088 tiles on 256
+// workgroups). When rem <= G / 2 those rem tiles are cut into quarters and run on the 128 x 128 cell
+// instead: 4 * rem quarter tiles over all G workgroups take 0.42 (one round) or 0.84 (two) of a big
+// tile's time. Same bytes: every output element is one exact integer sum and one epilogue, whichever
+// cell computes it.
 #define IU8_PF32(name, W8, WMW, WNW, TM, TN, ACC, ST, OCC, DEEP)                                                        \
   extern "C" __global__ __launch_bounds__(WMW * WNW * 64)                                                         \
       __attribute__((amdgpu_waves_per_eu(WMW * WNW * OCC / 4, WMW * WNW * OCC / 4))) void name(                    \
       const unsigned char *__restrict__ a, const unsigned char *__restrict__ w, const float *__restrict__ as,     \
       const float *__restrict__ ws, unsigned short *__restrict__ c, int m, int n, int k) {                         \
     constexpr int BM = WMW * TM * 32, BN = WNW * TN * 32;                                                          \
+    constexpr bool TAIL = WMW == 2 && WNW == 4 && TM == 4 && TN == 2 && !ACC && !DEEP;                             \
     const int gx = (n + BN - 1) / BN, gy = (m + BM - 1) / BM;                                                      \
     const iu8_rows R{nullptr, 0, m};                                                                               \
-    iu8_pf32_run<W8, WMW, WNW, TM, TN, ACC, ST, DEEP>(a, as, c, n, k, [&](int r, iu8_tile &t) {                          \
-      int bx, by;                                                                                                  \
-      if (!iu8_dense_tile_at(r, gx, gy, bx, by)) return false;                                                     \
-      t = iu8_tile{R, by * BM, bx * (BN / 16), w, ws, by * gx + bx};                                               \
-      return true;                                                                                                 \
-    });                                                                                                            \
+    if constexpr (TAIL) {                                                                                          \
+      constexpr int LB = iu8_pf32_lds_bytes<W8, WMW, WNW, TM, TN, ST>(), LS = iu8_pf32_lds_bytes<W8, 4, 2, 1, 2, 3>(); \
+      __shared__ __attribute__((aligned(1024))) iu8_u8 lds[LB > LS ? LB : LS];                                     \
+      const int G = gridDim.x, total = gx * gy, q = total / G, rem = total - q * G;                                \
+      const bool tail = q >= 1 && rem > 0 && 2 * rem <= G;                                                         \
+      iu8_pf32_run<W8, WMW, WNW, TM, TN, ACC, ST, DEEP, false, false, true>(                                       \
+          a, as, c, n, k,                                                                                          \
+          [&](int r, iu8_tile &t) {                                                                                \
+            int bx, by;                                                                                            \
+            if ((tail && r >= q) || !iu8_dense_tile_at(r, gx, gy, bx, by)) return false;                           \
+            t = iu8_tile{R, by * BM, bx * (BN / 16), w, ws, by * gx + bx};                                         \
+            return true;                                                                                           \
+          },                                                                                                       \
+          nullptr, nullptr, lds);                                                                                  \
+      if (tail) {                                                                                                  \
+        __syncthreads();                                                                                           \
+        iu8_pf32_run<W8, 4, 2, 1, 2, ACC, 3, false, false, false, true>(                                           \
+            a, as, c, n, k,                                                                                        \
+            [&](int r, iu8_tile &t) {                                                                              \
+              const int j = (int)blockIdx.x + r * G;                                                               \
+              if (j >= 4 * rem) return false;                                                                      \
+              int bx, by;                                                                                          \
+              iu8_dense_tile_of(q * G + (j >> 2), gx, gy, bx, by);                                                 \
+              t = iu8_tile{R, by * BM + ((j >> 1) & 1) * 128, (bx * BN + (j & 1) * 128) / 16, w, ws, 0};           \
+              return true;                                                                                         \
+            },                                                                                                     \
+            nullptr, nullptr, lds);                                                                                \
+      }                                                                                                            \
+    } else {                                                                                                       \
+      iu8_pf32_run<W8, WMW, WNW, TM, TN, ACC, ST, DEEP>(a, as, c, n, k, [&](int r, iu8_tile &t) {                  \
+        int bx, by;                                                                                                \
+        if (!iu8_dense_tile_at(r, gx, gy, bx, by)) return false;                                                   \
+        t = iu8_tile{R, by * BM, bx * (BN / 16), w, ws, by * gx + bx};                                             \
+        return true;                                                                                               \
+      });                                                                                                          \
+    }                                                                                                              \
   }
 // Cells with K split over gridDim.z (symbol suffix `_ks`, the decode kernarg list: the two workspaces
 // in front of c), for the rows between the regimes, where few tiles leave CUs idle. Measured, the

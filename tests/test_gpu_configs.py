@@ -143,6 +143,27 @@ def test_launch_law_splits_deep_narrow_tile_gemm(ctx, shape, ks):
     assert not run.counter.cpu().numpy().any()
 
 
+@pytest.mark.parametrize("grid", [8, 10, 11])
+@pytest.mark.parametrize("tag,w8", [("w4", False), ("w8", True)])
+def test_last_round_of_the_256x256_cell_runs_as_quarter_tiles(ctx, grid, tag, w8):
+    """12 tiles of the 256 x 256 cell (ragged both ways) on 8, 10 or 11 persistent workgroups: one full
+    round, then the 4 / 2 / 1 remaining tiles as quarter tiles on the 128 x 128 cell; same bytes as the oracle."""
+    M, N, K = 700, 1008, 640
+    say(f"256x256 cell, last round as quarter tiles: grid {grid} {tag}")
+    case = synth.dense_case(M, N, K, w8=w8, seed=grid)
+    r = ref.linear(case["X"], case["W"], case["ws"], w8, threads=8)
+    q, s = ref.quant_bf16(case["X"])
+    qd = dev_u8(iu8.repack_a(q))
+    sd, wf, wsd = dev_f32(s), dev_u8(iu8.repack_weights(case["W"], w8)), dev_f32(case["ws"])
+    c = torch.full((M, N), 0x7FC0, dtype=torch.int16, device="cuda")
+    d = iu8.describe_raw(f"macaq_iu8_pf_{tag}_tn4_lbk64", (grid, 1, 1), 512, plugin="macaq_iu8", m=M, n=N, k=K)
+    bufs = dict(a=qd.data_ptr(), w=wf.data_ptr(), ws=wsd.data_ptr(), c=c.data_ptr())
+    bufs["as"] = sd.data_ptr()
+    ctx.launch(d, bufs)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(host_u16(c), r["C"])
+
+
 def test_split_counter_is_reusable_across_launches(ctx):
     say("explicit split, two launches on one counter")
     case = synth.dense_case(3, 256, 2048, seed=23)
