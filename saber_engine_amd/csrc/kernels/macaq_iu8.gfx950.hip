@@ -120,8 +120,9 @@ IU8_DECQ(macaq_iu8_decq_w8_tm1, true, 4)
   }
 // Cells with K split over gridDim.z (symbol suffix `_ks`, the decode kernarg list: the two workspaces
 // in front of c), for the rows between the regimes, where few tiles leave CUs idle. Measured, the
-// partials' way through memory (ks * M * N * 4 bytes out and back) costs more than the idle CUs: the
-// launch law does not pick these; they are kept, tested and reachable by name like the decode split.
+// partials' way through memory (ks * M * N * 4 bytes out and back) costs more than the idle CUs on
+// every shape but deep, narrow linears at 49-128 rows, the one band where the launch law picks a
+// split form (the 64 x 128 cell); the others are kept, tested and reachable by name like the decode split.
 #define IU8_PF32K(name, W8, WMW, WNW, TM, TN, ST, OCC, DEEP)                                                       \
   extern "C" __global__ __launch_bounds__(WMW * WNW * 64)                                                         \
       __attribute__((amdgpu_waves_per_eu(WMW * WNW * OCC / 4, WMW * WNW * OCC / 4))) void name(                    \

@@ -217,21 +217,28 @@ extern "C" __global__ __launch_bounds__(MOE_THREADS) void moe_iu8_route_topk8_so
     s_cnt[e] = c;
   }
   __syncthreads();
-  for (int e = tid; e < e_loc; e += MOE_THREADS) blk_cnt[(size_t)blk * e_loc + e] = s_cnt[e];
-  __syncthreads();
-  if (tid == 0) {
-    __threadfence();
-    s_last = atomicAdd(arrive, 1) == nblk - 1;
+  // A lone workgroup (up to 128 tokens) is its own last arriver: its counts are the totals, its
+  // routes' bases are zero, and no hand-over through memory is needed.
+  const bool solo = nblk == 1;
+  if (!solo) {
+    for (int e = tid; e < e_loc; e += MOE_THREADS) blk_cnt[(size_t)blk * e_loc + e] = s_cnt[e];
+    __syncthreads();
+    if (tid == 0) {
+      __threadfence();
+      s_last = atomicAdd(arrive, 1) == nblk - 1;
+    }
+    __syncthreads();
+    if (!s_last) return;
+    __threadfence();  // acquire: every workgroup's topk_ids, rank and blk_cnt
+    if (tid == 0) *arrive = 0;
   }
-  __syncthreads();
-  if (!s_last) return;
-  __threadfence();  // acquire: every workgroup's topk_ids, rank and blk_cnt
-  if (tid == 0) *arrive = 0;
 
   // ---- phase 3 (the last workgroup): totals, each workgroup's base, offsets, tiles, placement.
   // It works alone, so its time is load latency: eight threads an expert scan an eighth of the
   // workgroups' counts each, loads in batches of 8.
-  {
+  if (solo) {
+    for (int e = tid; e < e_loc; e += MOE_THREADS) expert_cnt[e] = s_cnt[e];
+  } else {
     constexpr int PARTS = MOE_THREADS / MOE_E;
     const int e = tid % MOE_E, part = tid / MOE_E;
     const int chunk = (nblk + PARTS - 1) / PARTS, b_lo = min(part * chunk, nblk), b_hi = min(b_lo + chunk, nblk);
@@ -340,7 +347,7 @@ extern "C" __global__ __launch_bounds__(MOE_THREADS) void moe_iu8_route_topk8_so
 #pragma unroll
       for (int u = 0; u < 16; ++u) {
         const int r = r0 + u * MOE_THREADS, le = e[u] - e_lo;
-        base[u] = (r < R && le >= 0 && le < e_loc) ? blk_cnt[(size_t)(r / MOE_TOPK / MOE_TPB) * e_loc + le] : 0;
+        base[u] = (!solo && r < R && le >= 0 && le < e_loc) ? blk_cnt[(size_t)(r / MOE_TOPK / MOE_TPB) * e_loc + le] : 0;
       }
 #pragma unroll
       for (int u = 0; u < 16; ++u) {
