@@ -522,17 +522,17 @@ uint32_t saber_iu8_moe_tiles_cap(uint32_t tokens, uint32_t topk, uint32_t expert
   const uint32_t r = tokens * topk;
   return std::min(r, experts) + r / (16u * std::max(tile_blocks, 1u)) + 1u;
 }
-// Rows a tile (x16). 16-row tiles on the streaming cell while routes are so few that most tiles hold
-// a route or two (up to 5 routes an expert on average); above, the MFMA cells, whose sparse forms make
-// a thinly filled tile cost about its weight traffic and which stream an expert's weights once
-// instead of once a 16-row tile: 128-row tiles up to 96 routes an expert, 256-row tiles (one tile an
-// expert more often than not, on the dense GEMM's fastest shape) from there. Speed data of this card,
-// 128 experts, top-8, 4096 x 1536, us a layer at tile_blocks 1 / 8 / 16: T=32 256 / 316 / 328,
-// T=64 324 / 341 / 347, T=128 477 / 362 / 362, T=256 730 / 376 / 379, T=512 1282 / 370 / 396,
+// Rows a tile (x16). 16-row tiles on the streaming cell while routes are few (up to 7 routes an
+// expert on average); above, the MFMA cells, whose sparse forms make a thinly filled tile cost about
+// its weight traffic and which stream an expert's weights once instead of once a 16-row tile:
+// 128-row tiles up to 96 routes an expert, 256-row tiles (one tile an expert more often than not, on
+// the dense GEMM's fastest shape) from there. Speed data of this card, 128 experts, top-8,
+// 4096 x 1536, us a layer at tile_blocks 1 / 8 / 16: T=32 255 / 309 / 328, T=64 296 / 335 / 347,
+// T=80 318 / 340, T=128 363 / 347 / 362, T=256 730 / 376 / 379, T=512 1282 / 370 / 396,
 // T=1024 2349 / 430 / 469, T=2048 - / 650 / 597, T=4096 - / 982 / 952.
 uint32_t saber_iu8_moe_tile_blocks(uint32_t tokens, uint32_t topk, uint32_t experts) {
   const uint64_t routes = (uint64_t)tokens * topk;
-  if (routes <= 5ull * experts) return 1u;
+  if (routes <= 7ull * experts) return 1u;
   return routes >= 96ull * experts ? 16u : 8u;
 }
 
@@ -579,7 +579,11 @@ int saber_iu8_moe_grouped(saber_iu8_ctx *ctx, const void *a, const float *as, co
   const bool dec = tile_blocks == 1;
   if (gather < 0 || gather > 2 || (gather == 2 && dec))
     return fail(SABER_IU8_E_RULE, fmt("moe_grouped: gather %d; 0 in place, 1 from A fragments, 2 from row-major codes (MFMA cells only)", gather));
-  const std::string name = fmt("moe_iu8_grouped_w4_%s_g%d", dec ? "dec" : tile_blocks == 8 ? "pf" : "pf16", gather);
+  // the streaming cell stages a tile's rows in LDS while they are few (pow2(rows) * K <= 20 KiB);
+  // from about two routes an expert most launches have tiles that do not fit, and the form that
+  // streams the rows beside the weights is the faster one
+  const bool stream_rows = (uint64_t)tokens * topk > 2ull * experts || (uint64_t)k * 4 > 20 * 1024;
+  const std::string name = fmt("moe_iu8_grouped_w4_%s_g%d", dec ? (stream_rows ? "deca" : "dec") : tile_blocks == 8 ? "pf" : "pf16", gather);
   const uint32_t bn = dec ? 32 : 256, block = 512;
   saber_iu8_desc d;
   // the streaming cell: a workgroup a (column block, tile), static worst-case grid; the MFMA cell:

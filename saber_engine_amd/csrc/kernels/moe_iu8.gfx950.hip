@@ -389,6 +389,11 @@ extern "C" __global__ __launch_bounds__(MOE_THREADS) void moe_iu8_route_topk8_so
   }
 MOE_GROUPED_DEC(moe_iu8_grouped_w4_dec_g1, true, 1, 4, 8, 8, 20)
 MOE_GROUPED_DEC(moe_iu8_grouped_w4_dec_g0, false, 1, 4, 8, 8, 20)
+// The same cell with the activation rows streamed from L2 beside the weights instead of staged in
+// LDS: the staged form holds pow2(rows) * K <= 20 KiB (4 rows at K = 4096) and runs a tile that
+// does not fit without its load ring; this one keeps the ring for any tile.
+MOE_GROUPED_DEC(moe_iu8_grouped_w4_deca_g1, true, 2, 8, 8, 2, 0)
+MOE_GROUPED_DEC(moe_iu8_grouped_w4_deca_g0, false, 2, 8, 8, 2, 0)
 #undef MOE_GROUPED_DEC
 
 // The MFMA-bound cell: a persistent launch of one workgroup a CU walks the work items
