@@ -30,7 +30,7 @@ LAYERS = 6                  # distinct weight copies walked by successive steps 
 # HBM-side bytes of one launch of the dominant kernel, mean over the four layer shapes, from
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this very command (profiles/macaq_iu8_decq_w4_tm1__layer_set_m1.txt), each
 # counter scaled by what it reads for the 256 MiB copy probe. Keyed by (kernel, M); None = not measured.
-TRAFFIC = {("macaq_iu8_decq_w4_tm1", 1): 41898738.0, ("macaq_iu8_dec_w4_tm1", 1): 41992603.0}
+TRAFFIC = {("macaq_iu8_decq_w4_tm1", 1): 41897033.0, ("macaq_iu8_dec_w4_tm1", 1): 41992603.0}
 
 
 def alg_bytes(m, n, k, w8=False):
@@ -47,6 +47,7 @@ def main():
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-moe", action="store_true")
+    ap.add_argument("--no-other-m", action="store_true", help="prefill at M = 2048 only (a profiler run that wants one M a kernel)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--probe-copy", action="store_true",
                     help="also launch the 256 MiB copy probe (scale factor of the HBM byte counters under rocprofv3 --pmc)")
@@ -309,7 +310,7 @@ def main():
         # the other row counts of configs[2]: M = 256 sits near the ridge (both roofs reported: the weights'
         # GB/s beside the TOPS), M = 8192 is the matrix-bound end
         other = {}
-        for PM, warm, reps in ((256, 20, 20), (8192, 6, 6)):
+        for PM, warm, reps in (() if args.no_other_m else ((256, 20, 20), (8192, 6, 6))):
             pfm, ops_m, us_m, q_us_m = prefill_at(PM, warm, reps)
             wbytes = sum(n * k // 2 for _, n, k in linears)
             other["m%d" % PM] = dict(tops=round(ops_m / us_m / 1e6, 1), with_quant=round(ops_m / (us_m + q_us_m) / 1e6, 1),
