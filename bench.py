@@ -227,6 +227,58 @@ def main():
                                           "threads pinned one per core, 16-column tiles" % (n_cpu, M, isa))
         out["parity_vs_oracle"] = ok
 
+    # ---- the other batch sizes of configs[1] (M = 4, 8, 16) through the same step: a linear is one fused
+    # launch while its rows fit the fused form (M <= 4 and pow2(M) * K <= 20 KiB), else producer + GEMV;
+    # graph replay, cold weights
+    def decode_at(DM, nsteps=60):
+        xs, qs, ss, cs = {}, {}, {}, {}
+        for name, n, k in linears:
+            xs[name] = torch.from_numpy(synth.activations(np.random.default_rng(2), DM, k).view(np.int16)).to(dev)
+            qs[name] = torch.zeros(iu8.a_bytes(DM, k), dtype=torch.uint8, device=dev)
+            ss[name] = torch.zeros(DM, dtype=torch.float32, device=dev)
+            cs[name] = torch.zeros((DM, n), dtype=torch.int16, device=dev)
+        nlaunch = sum(1 if iu8.fused_holds(DM, k) else 2 for _, _, k in linears)
+
+        def one(i):
+            for name, n, k in linears:
+                w, wsd = dev_w[name][i % LAYERS].data_ptr(), dev_ws[name].data_ptr()
+                if iu8.fused_holds(DM, k):
+                    d = iu8.resolve_fused(iu8.W4, DM, n, k)
+                    for j in range(d.n_args):
+                        if d.args[j].name in (b"q", b"scale"):
+                            d.args[j].kind = iu8.ARG_NULL_BUFFER
+                    ctx.launch(d, dict(x=xs[name].data_ptr(), w=w, ws=wsd, c=cs[name].data_ptr()), sh)
+                else:
+                    ctx.launch(iu8.resolve_quant(DM, k), dict(x=xs[name].data_ptr(), q=qs[name].data_ptr(), scale=ss[name].data_ptr()), sh)
+                    d = iu8.resolve(iu8.W4, DM, n, k)
+                    assert d.ks == 1
+                    b = dict(a=qs[name].data_ptr(), w=w, ws=wsd, c=cs[name].data_ptr())
+                    b["as"] = ss[name].data_ptr()
+                    ctx.launch(d, b, sh)
+
+        with torch.cuda.stream(stream):
+            for i in range(6):
+                one(i)
+        stream.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=stream):
+            for i in range(nsteps):
+                one(i)
+        with torch.cuda.stream(stream):
+            g.replay()
+        torch.cuda.synchronize()
+        c0 = time.perf_counter()
+        with torch.cuda.stream(stream):
+            g.replay()
+        torch.cuda.synchronize()
+        us = (time.perf_counter() - c0) * 1e6 / nsteps
+        nbytes = sum(alg_bytes(DM, n, k) for _, n, k in linears)
+        return dict(us_per_step=round(us, 2), gbps=round(nbytes / us / 1e3, 1), hbm_frac=round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4),
+                    launches_per_step=nlaunch)
+
+    if M == 1 and not args.no_other_m:
+        out["decode_other_m"] = {"m%d" % DM: decode_at(DM) for DM in (4, 8, 16)}
+
     # ---- the second half of the metric: int8 TOPS at M=2048 on the same four shapes. Activations are
     # the configuration's (bf16 N(0,1), 0.5 % of the channels x20), quantised by the producer kernel:
     # the operand values set the card's clock under MFMA load, so uniform random codes would misstate it.
