@@ -370,6 +370,59 @@ def main():
                                      hbm_frac=round(wbytes / us_m / 1e3 / HBM_PEAK_GBPS, 4),
                                      per_linear={k_: dict(kernel=v["kernel"], us=v["us"], tops=v["tops"]) for k_, v in pfm.items()})
         out["prefill_other_m"] = other
+    # ---- configs[3]: the 64-entry launch sequence with 19 int8-row linears among the int4 ones (output-side
+    # projections), one HIP graph a sequence on shared per-token activations, every entry its own weights
+    # (random codes generated on the device: parity of this sequence is the GPU tests' business)
+    if not args.no_other_m:
+        seq = synth.mixed_sequence()
+        gen = torch.Generator(device=dev)
+        gen.manual_seed(3)
+        seq_w = []
+        for _, n, k, w8 in seq:
+            seq_w.append(torch.randint(0, 256, (n * k if w8 else n * k // 2,), dtype=torch.uint8, device=dev, generator=gen))
+        mixed = {}
+        for SM in (16, 2048):
+            acts = {}
+            for k in (5120, 17408):
+                x = torch.from_numpy(synth.activations(np.random.default_rng(4), SM, k).view(np.int16)).to(dev)
+                q = torch.zeros(iu8.a_bytes(SM, k), dtype=torch.uint8, device=dev)
+                a_s = torch.zeros(SM, dtype=torch.float32, device=dev)
+                ctx.quant(x.data_ptr(), q.data_ptr(), a_s.data_ptr(), SM, k, sh)
+                acts[k] = (q, a_s)
+            cbuf = {n: torch.zeros((SM, n), dtype=torch.int16, device=dev) for n in {e[1] for e in seq}}
+
+            def run_seq():
+                for (name, n, k, w8), w in zip(seq, seq_w):
+                    d = iu8.resolve(iu8.W8 if w8 else iu8.W4, SM, n, k)
+                    assert d.ks == 1
+                    b = dict(a=acts[k][0].data_ptr(), w=w.data_ptr(), ws=dev_ws[name].data_ptr(), c=cbuf[n].data_ptr())
+                    b["as"] = acts[k][1].data_ptr()
+                    ctx.launch(d, b, sh)
+
+            with torch.cuda.stream(stream):
+                run_seq()
+            stream.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, stream=stream):
+                run_seq()
+            reps = 6 if SM == 16 else 3
+            with torch.cuda.stream(stream):
+                g.replay()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record(stream)
+                for _ in range(reps):
+                    g.replay()
+                e1.record(stream)
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) * 1e3 / reps
+            wbytes = sum(n * k if w8 else n * k // 2 for _, n, k, w8 in seq)
+            ops = sum(2.0 * SM * n * k for _, n, k, _ in seq)
+            mixed["m%d" % SM] = dict(sequence_us=round(us, 1), launches=len(seq), w8_entries=sum(1 for e in seq if e[3]),
+                                     weight_gbps=round(wbytes / us / 1e3, 1), tops=round(ops / us / 1e6, 1))
+            del acts, cbuf, g
+        out["mixed_w4_w8_sequence"] = mixed
+        del seq_w
+
     # ---- the routed-expert layer of configs[4] (128 experts, top-8, hidden 4096, expert intermediate
     # 1536) as its launch train, T = 16 (weight streaming) and T = 4096 (MFMA); weights are random
     # nibbles generated on the device (parity of this path is the GPU tests' business)
