@@ -198,9 +198,9 @@ def main():
     # ---- parity spot check against the CPU oracle, and the CPU baseline beside it
     out = dict(metric="W4A8 GEMM GB/s (%HBM) at M=1; int8 TOPS (%MFMA peak) at M=2048", value=round(value, 1), unit="GB/s",
                n_gpus=1, steps=K_steps, warmup=W_steps, ms_per_step=round(ms_per_step, 5), higher_is_better=True,
-               scaling="weak", vs_baseline=None, dtype="int4 x int8 -> int32 -> bf16", data="synthetic (seed 0)",
+               scaling="weak", vs_baseline=None, dtype="int8", data="synthetic (seed 0)",
                config=dict(workload="configs[1]: decode-batch W4A8 linear set of one 27B-class layer (QKV, O, gate+up, down), "
-                                    "hidden 5120, TP=1", m=M, layers_rotated=LAYERS, cold=True,
+                                    "hidden 5120, TP=1", arithmetic="int4 weights x int8 activations -> int32 accumulators -> bf16 outputs", m=M, layers_rotated=LAYERS, cold=True,
                            launches_per_step=(1 if fused else 2) * len(linears), fused_quant=fused,
                            hbm_frac=round(value / HBM_PEAK_GBPS, 4),
                            two_launch_gbps=round(step_bytes / (two_ms * 1e-3) / 1e9, 1)),
