@@ -579,12 +579,17 @@ int saber_iu8_moe_grouped(saber_iu8_ctx *ctx, const void *a, const float *as, co
   const bool dec = tile_blocks == 1;
   if (gather < 0 || gather > 2 || (gather == 2 && dec))
     return fail(SABER_IU8_E_RULE, fmt("moe_grouped: gather %d; 0 in place, 1 from A fragments, 2 from row-major codes (MFMA cells only)", gather));
-  // the streaming cell stages a tile's rows in LDS while they are few (pow2(rows) * K <= 20 KiB);
-  // from about two routes an expert most launches have tiles that do not fit, and the form that
-  // streams the rows beside the weights is the faster one
-  const bool stream_rows = (uint64_t)tokens * topk > 2ull * experts || (uint64_t)k * 4 > 20 * 1024;
-  const std::string name = fmt("moe_iu8_grouped_w4_%s_g%d", dec ? (stream_rows ? "deca" : "dec") : tile_blocks == 8 ? "pf" : "pf16", gather);
-  const uint32_t bn = dec ? 32 : 256, block = 512;
+  // The streaming cell. Short K (an expert's down projection) takes the two-k-wave form with 64 columns a
+  // workgroup (K = 1536: 64 vs 72 us at 48 tokens, 75 vs 86 at 112). Else a tile's rows are staged in LDS
+  // while they fit (pow2(rows) * K <= 20 KiB, 4 rows at K = 4096); where a launch's tiles mostly would
+  // not (more than two routes an expert on average at that K), the form that streams the rows beside
+  // the weights is the faster one.
+  const bool short_k = k <= 2048;
+  uint32_t cap = 1;
+  while ((uint64_t)cap * 2 * k <= 20 * 1024 && cap < 16) cap *= 2;
+  const bool stream_rows = !short_k && (uint64_t)tokens * topk * 2 > (uint64_t)cap * experts;
+  const std::string name = fmt("moe_iu8_grouped_w4_%s_g%d", dec ? (short_k ? "deck" : stream_rows ? "deca" : "dec") : tile_blocks == 8 ? "pf" : "pf16", gather);
+  const uint32_t bn = dec ? (short_k ? 64 : 32) : 256, block = 512;
   saber_iu8_desc d;
   // the streaming cell: a workgroup a (column block, tile), static worst-case grid; the MFMA cell:
   // persistent, one workgroup a CU over the live work items

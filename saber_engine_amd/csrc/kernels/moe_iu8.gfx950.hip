@@ -392,6 +392,10 @@ MOE_GROUPED_DEC(moe_iu8_grouped_w4_dec_g0, false, 1, 4, 8, 8, 20)
 // The same cell with the activation rows streamed from L2 beside the weights instead of staged in
 // LDS: the staged form holds pow2(rows) * K <= 20 KiB (4 rows at K = 4096) and runs a tile that
 // does not fit without its load ring; this one keeps the ring for any tile.
+// Short K (up to 16 steps): two k-waves a tile instead of four, so a workgroup covers 64 columns and a
+// wave's ring holds its whole share (an expert's down projection, K = 1536: 50 -> 45 us at 16 tokens)
+MOE_GROUPED_DEC(moe_iu8_grouped_w4_deck_g1, true, 1, 2, 8, 6, 20)
+MOE_GROUPED_DEC(moe_iu8_grouped_w4_deck_g0, false, 1, 2, 8, 6, 20)
 MOE_GROUPED_DEC(moe_iu8_grouped_w4_deca_g1, true, 2, 8, 8, 2, 0)
 MOE_GROUPED_DEC(moe_iu8_grouped_w4_deca_g0, false, 2, 8, 8, 2, 0)
 #undef MOE_GROUPED_DEC

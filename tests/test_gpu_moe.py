@@ -77,6 +77,16 @@ def test_moe_layer_small_experts(ctx, T, tb):
     check_layer(layer, case)
 
 
+def test_moe_layer_streamed_rows_cell(ctx):
+    """K past the short-K form and more routes than the LDS staging is sized for: the streaming cell
+    that reads the rows beside the weights (gate+up), the short-K cell (down)."""
+    say("moe layer T=100 tile_blocks=1 E=128 top-8 H=2560 I=256")
+    case = synth.moe_case(T=100, E=128, topk=8, H=2560, I=256, seed=21, experts=4)
+    layer = run_layer(ctx, case)
+    assert layer.tb == 1
+    check_layer(layer, case)
+
+
 def test_moe_router_ties_and_skew(ctx):
     say("moe router: ties and one hot expert")
     case = synth.moe_case(T=40, E=128, topk=8, H=512, I=256, seed=5, experts=4)
