@@ -55,11 +55,15 @@ __device__ __forceinline__ void iu8_decq_body(const unsigned short *__restrict__
   for (int p = 0; p < X_PER; ++p)
     if (p * NTHR + tid < x_pieces) xreg[p] = *((const iu8_v4u *)X + p * NTHR + tid);
 
-  // ---- this workgroup's weight scales, all blocks
-  for (int i = tid; i < min(nb, IU8_DECQ_MAXB) * (WN * NT * 16); i += NTHR) {
-    const int b = i / (WN * NT * 16), c = i - b * (WN * NT * 16);
+  // ---- this workgroup's weight scales, all blocks: loaded now, put in LDS behind the ring's issue
+  // (a store here would wait out the load's whole latency in front of the weight loads)
+  constexpr int WS_ALL = IU8_DECQ_MAXB * (WN * NT * 16), WS_PER = (WS_ALL + NTHR - 1) / NTHR;
+  float wsreg[WS_PER];
+#pragma unroll
+  for (int p = 0; p < WS_PER; ++p) {
+    const int i = p * NTHR + tid, b = i / (WN * NT * 16), c = i - b * (WN * NT * 16);
     const int n = ((int)blockIdx.x + b * G) * (WN * NT * 16) + c;
-    s_ws[b][c] = n < N ? iu8_wsu<W8>(ws, n) : 0.f;
+    wsreg[p] = (i < min(nb, IU8_DECQ_MAXB) * (WN * NT * 16) && n < N) ? iu8_wsu<W8>(ws, n) : 0.f;
   }
 
   // ---- the issue side of the ring: block ib, step it, this lane's address in every tile
@@ -111,22 +115,40 @@ __device__ __forceinline__ void iu8_decq_body(const unsigned short *__restrict__
 #pragma unroll
       for (int r = 0; r < 4; ++r) am[r] = r == row ? fmaxf(am[r], m8) : am[r];
     }
+    // wave maximum of the live rows: DPP inside each 16-lane row, then the four rows' values through
+    // scalar registers (they are non-negative and never NaN, so the unsigned order of their bit
+    // patterns is their order); a butterfly through the LDS crossbar costs a microsecond here
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-#pragma unroll
-      for (int o = 32; o; o >>= 1) am[r] = fmaxf(am[r], __shfl_xor(am[r], o, 64));
+      if (r >= M) break;
+      float v = am[r];
+      v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, false)));   // xor 1
+      v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, false)));   // xor 2
+      v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, false)));  // half-row mirror
+      v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xF, 0xF, false)));  // row mirror
+      const unsigned u = __float_as_uint(v);
+      const unsigned m01 = max(__builtin_amdgcn_readlane(u, 0), __builtin_amdgcn_readlane(u, 16));
+      const unsigned m23 = max(__builtin_amdgcn_readlane(u, 32), __builtin_amdgcn_readlane(u, 48));
+      am[r] = __uint_as_float(max(m01, m23));
     }
     if (lane == 0) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) s_amax[wave][r] = am[r];
     }
+    // the weight scales have long arrived behind the rows' loads
+#pragma unroll
+    for (int p = 0; p < WS_PER; ++p)
+      if (p * NTHR + tid < WS_ALL) (&s_ws[0][0])[p * NTHR + tid] = wsreg[p];
     __syncthreads();
+    float qrcp[4] = {1.f, 1.f, 1.f, 1.f};
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
+      if (r >= M) break;
       float a = s_amax[0][r];
 #pragma unroll
       for (int w = 1; w < WPB; ++w) a = fmaxf(a, s_amax[w][r]);
       qsc[r] = fmaxf(__fdiv_rn(a, 127.f), 1e-30f);
+      qrcp[r] = __fdiv_rn(1.f, qsc[r]);
     }
     const bool out0 = blockIdx.x == 0 && qout != nullptr;
     if (blockIdx.x == 0 && sout != nullptr && tid < M)
@@ -137,7 +159,7 @@ __device__ __forceinline__ void iu8_decq_body(const unsigned short *__restrict__
       if (piece >= x_pieces) continue;
       const int row = (piece >= k8) + (piece >= 2 * k8) + (piece >= 3 * k8), k = (piece - row * k8) << 3;
       const float sc = row == 0 ? qsc[0] : row == 1 ? qsc[1] : row == 2 ? qsc[2] : qsc[3];
-      const float rcp = __fdiv_rn(1.f, sc);
+      const float rcp = row == 0 ? qrcp[0] : row == 1 ? qrcp[1] : row == 2 ? qrcp[2] : qrcp[3];
       float f[8];
 #pragma unroll
       for (int w = 0; w < 4; ++w) {
