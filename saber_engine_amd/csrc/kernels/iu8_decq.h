@@ -2,9 +2,10 @@
 // rows + the GEMV against them, one persistent launch. Operand orders and the contract: iu8_common.h.
 //
 // A workgroup (WPB waves: WN column groups x KW k-waves, as in the plain decode body) owns the
-// column blocks blockIdx.x, blockIdx.x + gridDim.x, ... of WN*NT*16 columns each. It quantises the
-// rows once (row amax, IEEE divide law, codes into LDS in staged order) while its first weight loads
-// are in flight, then streams its blocks' weights against the staged codes. The weight ring (D
+// column blocks blockIdx.x, blockIdx.x + gridDim.x, ... of WN*NT*16 columns each. It loads the rows,
+// starts its weight loads as soon as they are in, quantises the rows once (row amax, IEEE divide law,
+// codes into LDS in staged order) while those loads fly, then streams its blocks' weights against the
+// staged codes. The weight ring (D
 // 128-deep K steps of 128-bit nontemporal loads a wave) runs ACROSS block boundaries: when a wave
 // consumes the last step of a block its loads for the next block are already in flight, so the
 // memory pipe never drains inside the launch. A block ends with the k-waves' partials meeting in
@@ -92,11 +93,8 @@ __device__ __forceinline__ void iu8_decq_body(const unsigned short *__restrict__
       for (int j = 0; j < NT; ++j) ip[j] += KW * WSTEP;
     }
   };
-#pragma unroll
-  for (int i = 0; i < D; ++i)
-    if (i < TT) issue(i);
 
-  // ---- quantise the rows behind the first loads: amax lane -> wave (butterfly) -> workgroup (LDS),
+  // ---- quantise the rows: amax lane -> wave (butterfly) -> workgroup (LDS),
   // all order-free maxima; sc = max(amax / 127, 1e-30); codes by the exact reciprocal path
   float qsc[4] = {1.f, 1.f, 1.f, 1.f};
   {
@@ -115,6 +113,14 @@ __device__ __forceinline__ void iu8_decq_body(const unsigned short *__restrict__
 #pragma unroll
       for (int r = 0; r < 4; ++r) am[r] = r == row ? fmaxf(am[r], m8) : am[r];
     }
+    // The weight ring starts here, behind the first use of the rows, not at the kernel's top: every
+    // workgroup of the launch fires its ring at once, and rows requested in front of that burst took
+    // 2.5 us to arrive instead of one -- the whole quantisation chain waited on them, while the
+    // weights are not needed before the codes exist (QKV 7.7 -> 6.4 us, O 6.8 -> 5.9, down 13.7 -> 12.5;
+    // gate+up, bound by its bytes, unchanged).
+#pragma unroll
+    for (int i = 0; i < D; ++i)
+      if (i < TT) issue(i);
     // wave maximum of the live rows: DPP inside each 16-lane row, then the four rows' values through
     // scalar registers (they are non-negative and never NaN, so the unsigned order of their bit
     // patterns is their order); a butterfly through the LDS crossbar costs a microsecond here
