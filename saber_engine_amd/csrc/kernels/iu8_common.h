@@ -98,6 +98,22 @@ static __device__ __forceinline__ unsigned iu8_code4_rcp(float x0, float x1, flo
          __builtin_amdgcn_perm(__float_as_uint(u3), __float_as_uint(u2), 0x04000c0cu);
 }
 
+// Maximum over the 64 lanes of a wave of values that are non-negative and never NaN (row maxima of
+// |x|): DPP inside each 16-lane row (partners xor 1, xor 2, the half-row and the row mirror), then the
+// four rows' values through scalar registers, where the unsigned order of the bit patterns is the
+// values' order. The result is wave-uniform. A butterfly of six exchanges through the LDS crossbar
+// costs most of a microsecond in a kernel that is a latency chain.
+static __device__ __forceinline__ float iu8_wave_max_nonneg(float v) {
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, false)));
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, false)));
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, false)));
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xF, 0xF, false)));
+  const int u = __float_as_int(v);
+  const unsigned m01 = max((unsigned)__builtin_amdgcn_readlane(u, 0), (unsigned)__builtin_amdgcn_readlane(u, 16));
+  const unsigned m23 = max((unsigned)__builtin_amdgcn_readlane(u, 32), (unsigned)__builtin_amdgcn_readlane(u, 48));
+  return __uint_as_float(max(m01, m23));
+}
+
 // Cross-workgroup hand-over without a cache flush. The card has one L2 per XCD, so a device-scope
 // release fence writes an L2's dirty lines back and an acquire fence invalidates it; with hundreds of
 // workgroups doing that the fences alone cost 15-60 us a launch (measured with and without dirty

@@ -121,21 +121,11 @@ __device__ __forceinline__ void iu8_decq_body(const unsigned short *__restrict__
 #pragma unroll
     for (int i = 0; i < D; ++i)
       if (i < TT) issue(i);
-    // wave maximum of the live rows: DPP inside each 16-lane row, then the four rows' values through
-    // scalar registers (they are non-negative and never NaN, so the unsigned order of their bit
-    // patterns is their order); a butterfly through the LDS crossbar costs a microsecond here
+    // wave maximum of the live rows
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       if (r >= M) break;
-      float v = am[r];
-      v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, false)));   // xor 1
-      v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, false)));   // xor 2
-      v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, false)));  // half-row mirror
-      v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xF, 0xF, false)));  // row mirror
-      const unsigned u = __float_as_uint(v);
-      const unsigned m01 = max(__builtin_amdgcn_readlane(u, 0), __builtin_amdgcn_readlane(u, 16));
-      const unsigned m23 = max(__builtin_amdgcn_readlane(u, 32), __builtin_amdgcn_readlane(u, 48));
-      am[r] = __uint_as_float(max(m01, m23));
+      am[r] = iu8_wave_max_nonneg(am[r]);
     }
     if (lane == 0) {
 #pragma unroll

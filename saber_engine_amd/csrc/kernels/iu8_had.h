@@ -70,8 +70,7 @@ static __device__ __forceinline__ void had_tail(float (&sv)[HAD_MAXG][8], int NV
 #pragma unroll
     for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(sv[i][j]));
   }
-#pragma unroll
-  for (int o = 32; o; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
+  amax = iu8_wave_max_nonneg(amax);
   if ((tid & 63) == 0) s_max[tid >> 6] = amax;
   __syncthreads();
   amax = s_max[0];

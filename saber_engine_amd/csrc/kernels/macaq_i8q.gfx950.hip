@@ -39,8 +39,7 @@ static __device__ __forceinline__ int i8q_row() {
 
 static __device__ __forceinline__ float i8q_block_max(float v) {
   __shared__ float s_w[I8Q_T / 64];
-#pragma unroll
-  for (int o = 32; o; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  v = iu8_wave_max_nonneg(v);
   if ((threadIdx.x & 63) == 0) s_w[threadIdx.x >> 6] = v;
   __syncthreads();
   float r = s_w[0];
@@ -212,8 +211,7 @@ static __device__ __forceinline__ void i8q_tail_w64(float (&v)[I8Q_WG][16], int 
 #pragma unroll
     for (int j = 0; j < 16; ++j) amax = fmaxf(amax, fabsf(v[i][j]));
   }
-#pragma unroll
-  for (int o = 32; o; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
+  amax = iu8_wave_max_nonneg(amax);
   const float sc = fmaxf(__fdiv_rn(amax, 127.f), 1e-30f);
   const float rcp = __fdiv_rn(1.f, sc);
   if (lane == 0) scale[row] = sc;
