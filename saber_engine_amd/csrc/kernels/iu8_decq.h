@@ -5,14 +5,14 @@
 // column blocks blockIdx.x, blockIdx.x + gridDim.x, ... of WN*NT*16 columns each. It loads the rows,
 // starts its weight loads as soon as they are in, quantises the rows once (row amax, IEEE divide law,
 // codes into LDS in staged order) while those loads fly, then streams its blocks' weights against the
-// staged codes. The weight ring (D
-// 128-deep K steps of 128-bit nontemporal loads a wave) runs ACROSS block boundaries: when a wave
-// consumes the last step of a block its loads for the next block are already in flight, so the
-// memory pipe never drains inside the launch. A block ends with the k-waves' partials meeting in
-// LDS (exact int32, two alternating areas so one barrier a block suffices) and the bf16 epilogue,
-// whose weight scales were put in LDS at the start: loads return in order, so a scale load issued
-// at a block's end would only come back behind the whole ring. A launch gives a workgroup at most
-// IU8_DECQ_MAXB blocks (the host's grid law).
+// staged codes. The weight ring (D 128-deep K steps of 128-bit nontemporal loads a wave) runs ACROSS
+// block boundaries: when a wave consumes the last step of a block its loads for the next block are
+// already in flight, so the memory pipe never drains inside the launch. A block ends with the
+// k-waves' partials meeting in LDS (exact int32, two alternating areas so one barrier a block
+// suffices) and the bf16 epilogue, whose weight scales were requested at the start and put in LDS
+// behind the ring's issue: loads return in order, so a scale load issued at a block's end would only
+// come back behind the whole ring. A launch gives a workgroup at most IU8_DECQ_MAXB blocks (the
+// host's grid law).
 #pragma once
 #include "iu8_common.h"
 
