@@ -49,6 +49,10 @@ struct iu8_tile {
   const iu8_u8 *W;
   const float *ws;
   int id;  // the tile's index in the launch (its arrival counter under a split of K)
+  // The tile's K steps run from step `rot` of the workgroup's share round to rot - 1 (0 <= rot < steps of
+  // the share). The int32 sum does not depend on the order; tiles that start at different depths do
+  // not all ask the same memory channels for the same K at the same time.
+  int rot = 0;
 };
 
 // Dense tile order of a persistent launch of G workgroups over gx x gy tiles. The hardware deals
@@ -109,7 +113,9 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
   // as many stages as asked for and as fit the 160 KiB of LDS, at least two
   constexpr int NFIT = 160 * 1024 / STAGE;
   constexpr int NST = STMAX < 2 ? 2 : (STMAX < NFIT ? STMAX : (NFIT < 2 ? 2 : NFIT));
-  static_assert((NST - 2) * (A_FR / NWAVE + W_FR / NWAVE) <= 63, "the in-flight count fits s_waitcnt's vmcnt field");
+  // waves below these issue one more wave-load a step (a cell whose fragments do not divide by its waves)
+  constexpr int A_X = A_FR % NWAVE, W_X = W_FR % NWAVE;
+  static_assert((NST - 2) * (PER + (A_X > 0) + (W_X > 0)) <= 63, "the in-flight count fits s_waitcnt's vmcnt field");
   static_assert(!DEEP || NST >= 3, "the deep form reads a stage a step ahead of its MFMAs");
   static_assert(!(DEEP && SPARSE), "the sparse forms exist for the phased loop only");
   // EXT_LDS: the stages live in the caller's LDS block (1-KiB aligned, iu8_pf32_lds_bytes of this cell),
@@ -122,7 +128,11 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
     smem = own_lds;
   }
 
-  const int tid = threadIdx.x, lane = tid & 63;
+  // Opaque to the optimiser: a kernel that runs cells in a loop must not carry one cell's per-lane
+  // addresses in registers through the other cell's K loop.
+  int tid = threadIdx.x;
+  asm volatile("" : "+v"(tid));
+  const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WNW, wn = wave % WNW;
   const int ntiles = N >> 4, ksteps = K >> 7, ktiles = K >> 6;
@@ -175,7 +185,9 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
   const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) iu8_u8 *)smem;
   auto issue = [&](int stage) {  // the load stream's step -> LDS stage
     const unsigned sA = lds0 + stage * STAGE, sW = sA + A_BYTES;
-    const iu8_u8 *As = A + (size_t)ls * (ARM ? 128 : 2048), *Ws = L.W + (size_t)ls * WSTEP;
+    int kk = ls + L.rot;
+    if (kk >= s_hi) kk -= s_hi - s_lo;
+    const iu8_u8 *As = A + (size_t)kk * (ARM ? 128 : 2048), *Ws = L.W + (size_t)kk * WSTEP;
 #pragma unroll
     for (int p = 0; p < A_PER; ++p)
       if (A_FR % NWAVE == 0 || p * NWAVE + wave < A_FR) dma(As, ga[p], sA + (p * NWAVE + wave) * 1024);
@@ -204,9 +216,18 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
     if (lgkm0) __builtin_amdgcn_s_waitcnt((NN & 15) | ((NN >> 4) << 14) | (7 << 4) | (0 << 8));
     else __builtin_amdgcn_s_waitcnt((NN & 15) | ((NN >> 4) << 14) | (7 << 4) | (15 << 8));
   };
-  // Loads that may still fly at a step's barrier: the newest step's. Counted with the fewest a
-  // wave issues, so a wave that issued one more waits for that one too.
-  using InFlight = std::integral_constant<int, (NST - 2) * PER>;
+  // Loads that may still fly at a step's barrier: those of the newest NST-2 steps, counted with what
+  // this wave issues a step.
+  const int xtra = (wave < A_X) + (wave < W_X);
+  auto wait_step = [&](bool lgkm0) {
+    if constexpr (A_X == 0 && W_X == 0) {
+      wait_vm(std::integral_constant<int, (NST - 2) * PER>{}, lgkm0);
+    } else {
+      if (xtra == 0) wait_vm(std::integral_constant<int, (NST - 2) * PER>{}, lgkm0);
+      else if (xtra == 1) wait_vm(std::integral_constant<int, (NST - 2) * (PER + 1)>{}, lgkm0);
+      else wait_vm(std::integral_constant<int, (NST - 2) * (PER + (A_X > 0) + (W_X > 0))>{}, lgkm0);
+    }
+  };
 
   // this lane's operand addresses inside a stage, at sub-step 0
   const int r32 = lane & 31, h = lane >> 5;
@@ -280,7 +301,7 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
     issue(s0);
     advance();
   }
-  wait_vm(InFlight{}, false);
+  wait_step(false);
   __builtin_amdgcn_s_barrier();
   // deep form: register sets of one whole step, [set][sub-step f = 2p + kt2]
   iu8_v4i afd[DEEP ? 2 : 1][DEEP ? 4 : 1][TM] = {};
@@ -355,7 +376,7 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
         // must have landed: all but the newest NST-2 steps' loads.
         issue(stl);
         advance();
-        wait_vm(InFlight{}, true);
+        wait_step(true);
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
         fetch_step(smem + st1 * STAGE, set ^ 1);
@@ -416,7 +437,7 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
           // phase 3, behind the barrier: every wave's reads of this stage are done and the next step's
           // fragments have landed. The next step may be another tile's first, with every row block
           // live: its first operands are read in full whatever this tile's form.
-          wait_vm(InFlight{}, true);
+          wait_step(true);
           __builtin_amdgcn_s_barrier();
           __builtin_amdgcn_sched_barrier(0);
           fetch_a(nA, 0, 0, 0, Full{});
@@ -502,6 +523,26 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
                 iu8_v4i{acc[i][j][g * 4], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
           }
         }
+    } else if constexpr (NWAVE * 32 * (64 + 16) > STAGE) {
+      // A cell of few rows, whose stage is too small for the transposing form below: every lane stores
+      // its 4 consecutive columns of a row (8 bytes; lane halves side by side) -- such a tile's output
+      // is small.
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        const int m = C.mbase + (wm * TM + i) * 32 + r32;
+        const float am = as[iu8_arow(C.R, min(m, M - 1))];
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const int n = ncol0 + j * 32 + g * 8 + nq;
+            const float4 w4 = *(const float4 *)(C.ws + min(n, N - 4));
+            const float u = W8 ? 1.f : 0.0625f;  // exact: a power of two
+            const unsigned lo = iu8_bf16_pack(iu8_epi(acc[i][j][g * 4], am, w4.x * u), iu8_epi(acc[i][j][g * 4 + 1], am, w4.y * u));
+            const unsigned hi = iu8_bf16_pack(iu8_epi(acc[i][j][g * 4 + 2], am, w4.z * u), iu8_epi(acc[i][j][g * 4 + 3], am, w4.w * u));
+            if (m < M && n < N) *(iu8_v2u *)((unsigned short *)Cv + (size_t)(C.R.row0 + m) * N + n) = iu8_v2u{lo, hi};
+          }
+      }
     } else {
       // Through LDS: a lane holds 4 consecutive columns of one row, so direct stores would touch 32
       // rows with 16 bytes each. Each wave turns a block of 32 rows x CB*32 columns at a time into

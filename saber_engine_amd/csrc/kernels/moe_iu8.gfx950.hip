@@ -400,17 +400,42 @@ MOE_GROUPED_DEC(moe_iu8_grouped_w4_deca_g1, true, 2, 8, 8, 2, 0)
 MOE_GROUPED_DEC(moe_iu8_grouped_w4_deca_g0, false, 2, 8, 8, 2, 0)
 #undef MOE_GROUPED_DEC
 
-// The MFMA-bound cell: a persistent launch of one workgroup a CU walks the work items
+// The MFMA-bound cells: a persistent launch of one workgroup a CU walks the work items
 // (tile, column block) of the live tiles, column blocks of one tile on neighbouring workgroups, the
-// load stream running across items (iu8_pf32.h). grid [256, 1, 1].
-// The walk is static (item = blockIdx.x + r * gridDim.x), and an expert's last tile is often nearly
-// empty and then cheap (the sparse forms of iu8_pf32.h); in table order some workgroups would draw
-// mostly full tiles and set the launch's time. So every workgroup first sorts the tiles the same
-// way -- those with more than one live 32-row block first, in table order, the light ones after
-// them -- and the round-robin deals each kind evenly.
-#define MOE_ORDER_CAP 4096  // tiles the ordering holds in LDS; beyond, table order
+// load stream running across items (iu8_pf32.h). grid [256, 1, 1]. Every workgroup first sorts the
+// tiles the same way, those of more than MOE_LIGHT_ROWS rows first in table order, the light ones
+// after them; the walk is static (item = workgroup + r * gridDim.x), so each kind is dealt evenly.
+//
+// An expert's last tile is often nearly empty. On the tile cell such a tile still moves whole stages
+// of mostly dead rows behind a barrier a step: measured, some 70 % of a full tile's time for a
+// twentieth of its work. The two-cell form (LIGHT) runs the light tiles on a second cell in the same
+// LDS, 64 rows x 256 columns (2 x 4 waves, the deep form of iu8_pf32.h), whose small stages keep five
+// steps of loads in flight and move no dead rows; its K steps start at a depth that differs from
+// item to item (iu8_tile::rot), which spreads the weight streams of the light items over the memory
+// channels (512 tokens, gate+up: 187 -> 160 us). Light tiles together are bound by the memory rate,
+// the heavy ones by the matrix pipes, so a workgroup runs its light items between two parts of its
+// heavy ones, after (workgroup / 8) mod (rounds + 1) rounds, the light walk dealt from the last
+// workgroup down: at any time a slice of every XCD's CUs streams light tiles under the others'
+// matrix work (2,048 tokens on 128-row tiles: 633 -> 577 us a layer against 639 with the light items
+// last). An item's descriptor hangs on a chain of dependent loads (order -> tile table -> expert
+// pointers), so a workgroup resolves its items up front, one lane an item, into a table in LDS.
+// The 128-row kernels are two-cell (256 to 2,048 tokens: 3 to 9 % a layer). The 256-row kernels are
+// not: at 4,096 tokens the light tiles' weights come from memory a second time whichever cell asks
+// (timestamps: a light item takes 20-28 us there against 4 with its weights cached, a heavy round
+// 62-82 us with light items beside it against 63 without), the layer gained 2 %, and launches with no
+// light tile (1,536 to 2,048 tokens) lost 2 to 4 % to the two-cell kernel's heavier item switch.
+#define MOE_ORDER_CAP 4096  // tiles the ordering holds in LDS; beyond, table order on the big cell
+#define MOE_LIGHT_ROWS 64
+#define MOE_LIGHT_ST 6
+#define MOE_HEAVY_ROUNDS 8  // rounds of items a workgroup resolves at a time: the item table in LDS
+#define MOE_LIGHT_ROUNDS 8
+struct moe_item {
+  int row0, rows, nt0, rot;  // rows < 0: no item
+  const unsigned char *W;
+  const float *ws;
+};
 template <int NTHR>
-static __device__ __forceinline__ void moe_tile_order(const int *__restrict__ tile_rows, int nt, unsigned short *s_order) {
+static __device__ __forceinline__ int moe_tile_order(const int *__restrict__ tile_rows, int nt, unsigned short *s_order) {
   __shared__ int s_w[NTHR / 64];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   auto block_sum = [&](int v, int &before) {  // sum over the workgroup; `before` = the waves ahead of this one
@@ -428,14 +453,14 @@ static __device__ __forceinline__ void moe_tile_order(const int *__restrict__ ti
     return all;
   };
   int mine = 0, unused;
-  for (int t = tid; t < nt; t += NTHR) mine += tile_rows[t] > 32;
+  for (int t = tid; t < nt; t += NTHR) mine += tile_rows[t] > MOE_LIGHT_ROWS;
 #pragma unroll
   for (int o = 32; o; o >>= 1) mine += __shfl_xor(mine, o, 64);
   const int heavy_total = block_sum(mine, unused);
   int run = 0;  // heavy tiles before this chunk
   for (int base = 0; base < nt; base += NTHR) {
     const int t = base + tid;
-    const bool h = t < nt && tile_rows[t] > 32;
+    const bool h = t < nt && tile_rows[t] > MOE_LIGHT_ROWS;
     const unsigned long long b = __ballot(h);
     int wave_before;
     const int chunk = block_sum(__popcll(b), wave_before);
@@ -444,36 +469,109 @@ static __device__ __forceinline__ void moe_tile_order(const int *__restrict__ ti
     run += chunk;
   }
   __syncthreads();
+  return heavy_total;
 }
-#define MOE_GROUPED_PF(name, GATHER, WMW, WNW, TM, TN, ST)                                                           \
+#define MOE_GROUPED_PF(name, GATHER, WMW, WNW, TM, TN, ST, LIGHT)                                                        \
   extern "C" __global__ __launch_bounds__(WMW * WNW * 64) void name(                                              \
       const unsigned char *__restrict__ a, const unsigned long long *__restrict__ xptr,                           \
       const int *__restrict__ tile_expert, const int *__restrict__ tile_row0, const int *__restrict__ tile_rows,  \
       const int *__restrict__ row_tok, const int *__restrict__ meta, const float *__restrict__ as,                \
       int *__restrict__ p, int *__restrict__ cnt, unsigned short *__restrict__ c, int n, int k, int pmax) {        \
     constexpr int BN = WNW * TN * 32;                                                                              \
+    static_assert(BN == 256 && WMW * WNW == 8, "both cells are 8 waves and 256 columns wide");                     \
+    if constexpr (!LIGHT) {                                                                                        \
+      /* one cell, items in table order */                                                                        \
+      __shared__ unsigned short s_order[MOE_ORDER_CAP];                                                            \
+      const int nt = meta[0], gx = (n + BN - 1) / BN, total = nt * gx;                                             \
+      const bool ordered = nt <= MOE_ORDER_CAP;                                                                    \
+      if (ordered) moe_tile_order<WMW * WNW * 64>(tile_rows, nt, s_order);                                         \
+      iu8_pf32_run<false, WMW, WNW, TM, TN, false, ST, false, true, GATHER == 2>(a, as, c, n, k, [&](int r, iu8_tile &t) { \
+        const int id = (int)blockIdx.x + r * (int)gridDim.x;                                                       \
+        if (id >= total) return false;                                                                             \
+        const int slot = id / gx, bx = id - slot * gx, tile = ordered ? (int)s_order[slot] : slot;                 \
+        const int e = tile_expert[tile];                                                                           \
+        t = iu8_tile{iu8_rows{GATHER ? row_tok : nullptr, tile_row0[tile], min(tile_rows[tile], WMW * TM * 32)}, 0, \
+                     bx * (BN / 16), (const unsigned char *)xptr[2 * e], (const float *)xptr[2 * e + 1]};          \
+        return true;                                                                                               \
+      });                                                                                                          \
+      return;                                                                                                      \
+    }                                                                                                              \
+    constexpr int LB = iu8_pf32_lds_bytes<false, WMW, WNW, TM, TN, ST>();                                          \
+    constexpr int LL = iu8_pf32_lds_bytes<false, 2, 4, 1, 2, MOE_LIGHT_ST>();                                      \
+    __shared__ __attribute__((aligned(1024))) iu8_u8 lds[LB > LL ? LB : LL];                                       \
     __shared__ unsigned short s_order[MOE_ORDER_CAP];                                                              \
-    const int nt = meta[0], gx = (n + BN - 1) / BN, total = nt * gx;                                               \
-    const bool ordered = nt <= MOE_ORDER_CAP;                                                                      \
-    if (ordered) moe_tile_order<WMW * WNW * 64>(tile_rows, nt, s_order);                                           \
-    iu8_pf32_run<false, WMW, WNW, TM, TN, false, ST, false, true, GATHER == 2>(a, as, c, n, k, [&](int r, iu8_tile &t) { \
-      const int id = (int)blockIdx.x + r * (int)gridDim.x;                                                         \
-      if (id >= total) return false;                                                                               \
-      const int slot = id / gx, bx = id - slot * gx, tile = ordered ? (int)s_order[slot] : slot;                   \
-      const int e = tile_expert[tile];                                                                             \
-      t = iu8_tile{iu8_rows{GATHER ? row_tok : nullptr, tile_row0[tile], min(tile_rows[tile], WMW * TM * 32)}, 0,  \
-                   bx * (BN / 16), (const unsigned char *)xptr[2 * e], (const float *)xptr[2 * e + 1]};            \
+    /* the walk's numbers and this workgroup's resolved items live in LDS */                                      \
+    __shared__ int s_par[4];                                                                                       \
+    __shared__ moe_item s_item[MOE_HEAVY_ROUNDS + MOE_LIGHT_ROUNDS];                                               \
+    auto par = [&](int i) { return __builtin_amdgcn_readfirstlane(((volatile int *)s_par)[i]); };                  \
+    auto item = [&](int q, iu8_tile &t) {                                                                          \
+      const volatile int *p32 = (const volatile int *)&s_item[q];                                                  \
+      auto u = [&](int i) { return __builtin_amdgcn_readfirstlane(p32[i]); };                                      \
+      if (u(1) < 0) return false;                                                                                  \
+      const unsigned long long wp = (unsigned)u(4) | ((unsigned long long)(unsigned)u(5) << 32);                   \
+      const unsigned long long sp = (unsigned)u(6) | ((unsigned long long)(unsigned)u(7) << 32);                   \
+      t = iu8_tile{iu8_rows{GATHER ? row_tok : nullptr, u(0), u(1)}, 0, u(2), (const unsigned char *)wp, (const float *)sp, 0, u(3)}; \
       return true;                                                                                                 \
-    });                                                                                                            \
+    };                                                                                                             \
+    const int nt = meta[0];                                                                                        \
+    const bool ordered = nt <= MOE_ORDER_CAP;                                                                      \
+    const int heavy = ordered ? moe_tile_order<WMW * WNW * 64>(tile_rows, nt, s_order) : nt;                       \
+    /* a launch of more rounds than the item table holds runs in epochs of that many */                           \
+    for (int ep = 0;; ++ep) {                                                                                      \
+      {                                                                                                            \
+        const int gx = (n + BN - 1) / BN, G = gridDim.x, w = blockIdx.x;                                           \
+        const int hi = heavy * gx, li = (nt - heavy) * gx;                                                         \
+        const int h0 = ep * MOE_HEAVY_ROUNDS, l0 = ep * MOE_LIGHT_ROUNDS;                                          \
+        const int rounds = max(0, min((hi + G - 1) / G - h0, MOE_HEAVY_ROUNDS));                                   \
+        const int lrounds = max(0, min((li + G - 1) / G - l0, MOE_LIGHT_ROUNDS));                                  \
+        if (rounds + lrounds == 0) break;                                                                          \
+        /* a workgroup's heavy items run in two parts, its light items between them, after `first` rounds */      \
+        if (threadIdx.x == 0) {                                                                                    \
+          s_par[0] = rounds, s_par[1] = lrounds;                                                                   \
+          s_par[2] = lrounds > 0 ? (w >> 3) % (rounds + 1) : rounds;                                               \
+        }                                                                                                          \
+        const int q = threadIdx.x;                                                                                 \
+        if (q < rounds + lrounds) {                                                                                \
+          const bool light = q >= rounds;                                                                          \
+          const int id = light ? G - 1 - w + (l0 + q - rounds) * G : w + (h0 + q) * G;                             \
+          moe_item it{0, -1, 0, 0, nullptr, nullptr};                                                              \
+          if (id < (light ? li : hi)) {                                                                            \
+            const int slot = (light ? heavy : 0) + id / gx, tile = ordered ? (int)s_order[slot] : slot;            \
+            const int e = tile_expert[tile];                                                                       \
+            it = moe_item{tile_row0[tile], min(tile_rows[tile], light ? MOE_LIGHT_ROWS : WMW * TM * 32),           \
+                          id % gx * (BN / 16), light ? (int)(((unsigned)id * 2654435761u >> 10) % (unsigned)(k >> 7)) : 0, \
+                          (const unsigned char *)xptr[2 * e], (const float *)xptr[2 * e + 1]};                     \
+          }                                                                                                        \
+          s_item[q] = it;                                                                                          \
+        }                                                                                                          \
+        __syncthreads();                                                                                           \
+      }                                                                                                            \
+      for (int part = 0; part < 2; ++part) {                                                                       \
+        if (part == 1) {                                                                                           \
+          if (par(1) == 0) break;                                                                                  \
+          iu8_pf32_run<false, 2, 4, 1, 2, false, MOE_LIGHT_ST, true, false, GATHER == 2, true>(                    \
+              a, as, c, n, k, [&](int r, iu8_tile &t) { return r < par(1) && item(par(0) + r, t); }, nullptr, nullptr, lds); \
+          __syncthreads();                                                                                         \
+        }                                                                                                          \
+        iu8_pf32_run<false, WMW, WNW, TM, TN, false, ST, false, true, GATHER == 2, true>(                          \
+            a, as, c, n, k,                                                                                        \
+            [&](int r, iu8_tile &t) {                                                                              \
+              const int first = par(2), rr = part ? first + r : r;                                                 \
+              return rr < (part ? par(0) : first) && item(rr, t);                                                  \
+            },                                                                                                     \
+            nullptr, nullptr, lds);                                                                                \
+        __syncthreads();                                                                                           \
+      }                                                                                                            \
+    }                                                                                                              \
   }
 // tiles of up to 128 rows (tile_blocks 8) on the 128 x 256 tile of 2 x 4 waves
-MOE_GROUPED_PF(moe_iu8_grouped_w4_pf_g2, 2, 2, 4, 2, 2, 4)
-MOE_GROUPED_PF(moe_iu8_grouped_w4_pf_g1, 1, 2, 4, 2, 2, 4)
-MOE_GROUPED_PF(moe_iu8_grouped_w4_pf_g0, 0, 2, 4, 2, 2, 4)
+MOE_GROUPED_PF(moe_iu8_grouped_w4_pf_g2, 2, 2, 4, 2, 2, 4, true)
+MOE_GROUPED_PF(moe_iu8_grouped_w4_pf_g1, 1, 2, 4, 2, 2, 4, true)
+MOE_GROUPED_PF(moe_iu8_grouped_w4_pf_g0, 0, 2, 4, 2, 2, 4, true)
 // tiles of up to 256 rows (tile_blocks 16) on the 256 x 256 tile, the dense GEMM's fastest cell
-MOE_GROUPED_PF(moe_iu8_grouped_w4_pf16_g2, 2, 2, 4, 4, 2, 3)
-MOE_GROUPED_PF(moe_iu8_grouped_w4_pf16_g1, 1, 2, 4, 4, 2, 3)
-MOE_GROUPED_PF(moe_iu8_grouped_w4_pf16_g0, 0, 2, 4, 4, 2, 3)
+MOE_GROUPED_PF(moe_iu8_grouped_w4_pf16_g2, 2, 2, 4, 4, 2, 3, false)
+MOE_GROUPED_PF(moe_iu8_grouped_w4_pf16_g1, 1, 2, 4, 4, 2, 3, false)
+MOE_GROUPED_PF(moe_iu8_grouped_w4_pf16_g0, 0, 2, 4, 4, 2, 3, false)
 #undef MOE_GROUPED_PF
 
 // ---------------------------------------------------------------------------- combine

@@ -87,6 +87,32 @@ def test_moe_layer_streamed_rows_cell(ctx):
     check_layer(layer, case)
 
 
+@pytest.mark.parametrize("T,I,hot,boost", [(512, 2560, 0, 0.0), (2048, 4352, 8, 6.0), (1024, 256, 4, 1.5)])
+def test_moe_layer_two_cell_walk(ctx, T, I, hot, boost):
+    """The 128-row tile cell runs tiles of up to 64 rows on a second, smaller cell between two parts of
+    its heavy items, and resolves a workgroup's items eight heavy and eight light rounds at a time: ten
+    rounds of light items (512 tokens over 128 experts, 20 column blocks), seventeen of heavy ones
+    (2,048 tokens on 8 experts, 34 column blocks), and a skewed routing with both kinds in one launch."""
+    say(f"moe layer T={T} tile_blocks=8 E=128 top-8 H=256 I={I} hot experts={hot} (+{boost})")
+    case = synth.moe_case(T=T, E=128, topk=8, H=256, I=I, seed=T + 3, experts=2)
+    if hot:
+        lg = synth.bf16_bits_to_f32(case["logits"])
+        if boost > 3:
+            lg = lg * np.float32(0.25) - np.float32(3.0)
+        lg[:, :hot] += np.float32(boost)
+        case["logits"] = synth.f32_to_bf16_bits(lg)
+    layer = run_layer(ctx, case, tile_blocks=8)
+    tr = layer.buf["tile_rows"][:int(layer.buf["meta"][0].item())].cpu().numpy()
+    light, heavy, gx = int((tr <= 64).sum()), int((tr > 64).sum()), (2 * I + 255) // 256
+    if hot == 0:
+        assert light * gx > 8 * 256
+    elif boost > 3:
+        assert heavy * gx > 8 * 256
+    else:
+        assert light >= 32 and heavy >= 8
+    check_layer(layer, case)
+
+
 def test_moe_router_ties_and_skew(ctx):
     say("moe router: ties and one hot expert")
     case = synth.moe_case(T=40, E=128, topk=8, H=512, I=256, seed=5, experts=4)
