@@ -471,107 +471,120 @@ static __device__ __forceinline__ int moe_tile_order(const int *__restrict__ til
   __syncthreads();
   return heavy_total;
 }
-#define MOE_GROUPED_PF(name, GATHER, WMW, WNW, TM, TN, ST, LIGHT)                                                        \
+// one cell, items in the sorted order
+template <int GATHER, int WMW, int WNW, int TM, int TN, int ST>
+static __device__ __forceinline__ void moe_grouped_pf_one(
+    const unsigned char *__restrict__ a, const unsigned long long *__restrict__ xptr, const int *__restrict__ tile_expert,
+    const int *__restrict__ tile_row0, const int *__restrict__ tile_rows, const int *__restrict__ row_tok,
+    const int *__restrict__ meta, const float *__restrict__ as, unsigned short *__restrict__ c, int n, int k) {
+  constexpr int BN = WNW * TN * 32;
+  static_assert(BN == 256 && WMW * WNW == 8, "both cells are 8 waves and 256 columns wide");
+  __shared__ unsigned short s_order[MOE_ORDER_CAP];
+  const int nt = meta[0], gx = (n + BN - 1) / BN, total = nt * gx;
+  const bool ordered = nt <= MOE_ORDER_CAP;
+  if (ordered) moe_tile_order<WMW * WNW * 64>(tile_rows, nt, s_order);
+  iu8_pf32_run<false, WMW, WNW, TM, TN, false, ST, false, true, GATHER == 2>(a, as, c, n, k, [&](int r, iu8_tile &t) {
+    const int id = (int)blockIdx.x + r * (int)gridDim.x;
+    if (id >= total) return false;
+    const int slot = id / gx, bx = id - slot * gx, tile = ordered ? (int)s_order[slot] : slot;
+    const int e = tile_expert[tile];
+    t = iu8_tile{iu8_rows{GATHER ? row_tok : nullptr, tile_row0[tile], min(tile_rows[tile], WMW * TM * 32)}, 0,
+                 bx * (BN / 16), (const unsigned char *)xptr[2 * e], (const float *)xptr[2 * e + 1]};
+    return true;
+  });
+}
+// two cells: heavy items on the tile cell, light ones on the small cell between two parts of them
+template <int GATHER, int WMW, int WNW, int TM, int TN, int ST>
+static __device__ __forceinline__ void moe_grouped_pf_two(
+    const unsigned char *__restrict__ a, const unsigned long long *__restrict__ xptr, const int *__restrict__ tile_expert,
+    const int *__restrict__ tile_row0, const int *__restrict__ tile_rows, const int *__restrict__ row_tok,
+    const int *__restrict__ meta, const float *__restrict__ as, unsigned short *__restrict__ c, int n, int k) {
+  constexpr int BN = WNW * TN * 32;
+  static_assert(BN == 256 && WMW * WNW == 8, "both cells are 8 waves and 256 columns wide");
+  constexpr int LB = iu8_pf32_lds_bytes<false, WMW, WNW, TM, TN, ST>();
+  constexpr int LL = iu8_pf32_lds_bytes<false, 2, 4, 1, 2, MOE_LIGHT_ST>();
+  __shared__ __attribute__((aligned(1024))) iu8_u8 lds[LB > LL ? LB : LL];
+  __shared__ unsigned short s_order[MOE_ORDER_CAP];
+  /* the walk's numbers and this workgroup's resolved items live in LDS */
+  __shared__ int s_par[4];
+  __shared__ moe_item s_item[MOE_HEAVY_ROUNDS + MOE_LIGHT_ROUNDS];
+  auto par = [&](int i) { return __builtin_amdgcn_readfirstlane(((volatile int *)s_par)[i]); };
+  auto item = [&](int q, iu8_tile &t) {
+    const volatile int *p32 = (const volatile int *)&s_item[q];
+    auto u = [&](int i) { return __builtin_amdgcn_readfirstlane(p32[i]); };
+    if (u(1) < 0) return false;
+    const unsigned long long wp = (unsigned)u(4) | ((unsigned long long)(unsigned)u(5) << 32);
+    const unsigned long long sp = (unsigned)u(6) | ((unsigned long long)(unsigned)u(7) << 32);
+    t = iu8_tile{iu8_rows{GATHER ? row_tok : nullptr, u(0), u(1)}, 0, u(2), (const unsigned char *)wp, (const float *)sp, 0, u(3)};
+    return true;
+  };
+  const int nt = meta[0];
+  const bool ordered = nt <= MOE_ORDER_CAP;
+  const int heavy = ordered ? moe_tile_order<WMW * WNW * 64>(tile_rows, nt, s_order) : nt;
+  /* a launch of more rounds than the item table holds runs in epochs of that many */
+  for (int ep = 0;; ++ep) {
+    {
+      const int gx = (n + BN - 1) / BN, G = gridDim.x, w = blockIdx.x;
+      const int hi = heavy * gx, li = (nt - heavy) * gx;
+      const int h0 = ep * MOE_HEAVY_ROUNDS, l0 = ep * MOE_LIGHT_ROUNDS;
+      const int rounds = max(0, min((hi + G - 1) / G - h0, MOE_HEAVY_ROUNDS));
+      const int lrounds = max(0, min((li + G - 1) / G - l0, MOE_LIGHT_ROUNDS));
+      if (rounds + lrounds == 0) break;
+      /* a workgroup's heavy items run in two parts, its light items between them, after `first` rounds */
+      if (threadIdx.x == 0) {
+        s_par[0] = rounds, s_par[1] = lrounds;
+        s_par[2] = lrounds > 0 ? (w >> 3) % (rounds + 1) : rounds;
+      }
+      const int q = threadIdx.x;
+      if (q < rounds + lrounds) {
+        const bool light = q >= rounds;
+        const int id = light ? G - 1 - w + (l0 + q - rounds) * G : w + (h0 + q) * G;
+        moe_item it{0, -1, 0, 0, nullptr, nullptr};
+        if (id < (light ? li : hi)) {
+          const int slot = (light ? heavy : 0) + id / gx, tile = ordered ? (int)s_order[slot] : slot;
+          const int e = tile_expert[tile];
+          it = moe_item{tile_row0[tile], min(tile_rows[tile], light ? MOE_LIGHT_ROWS : WMW * TM * 32),
+                        id % gx * (BN / 16), light ? (int)(((unsigned)id * 2654435761u >> 10) % (unsigned)(k >> 7)) : 0,
+                        (const unsigned char *)xptr[2 * e], (const float *)xptr[2 * e + 1]};
+        }
+        s_item[q] = it;
+      }
+      __syncthreads();
+    }
+    for (int part = 0; part < 2; ++part) {
+      if (part == 1) {
+        if (par(1) == 0) break;
+        iu8_pf32_run<false, 2, 4, 1, 2, false, MOE_LIGHT_ST, true, false, GATHER == 2, true>(
+            a, as, c, n, k, [&](int r, iu8_tile &t) { return r < par(1) && item(par(0) + r, t); }, nullptr, nullptr, lds);
+        __syncthreads();
+      }
+      iu8_pf32_run<false, WMW, WNW, TM, TN, false, ST, false, true, GATHER == 2, true>(
+          a, as, c, n, k,
+          [&](int r, iu8_tile &t) {
+            const int first = par(2), rr = part ? first + r : r;
+            return rr < (part ? par(0) : first) && item(rr, t);
+          },
+          nullptr, nullptr, lds);
+      __syncthreads();
+    }
+  }
+}
+#define MOE_GROUPED_PF(name, BODY, GATHER, WMW, WNW, TM, TN, ST)                                                     \
   extern "C" __global__ __launch_bounds__(WMW * WNW * 64) void name(                                              \
       const unsigned char *__restrict__ a, const unsigned long long *__restrict__ xptr,                           \
       const int *__restrict__ tile_expert, const int *__restrict__ tile_row0, const int *__restrict__ tile_rows,  \
       const int *__restrict__ row_tok, const int *__restrict__ meta, const float *__restrict__ as,                \
       int *__restrict__ p, int *__restrict__ cnt, unsigned short *__restrict__ c, int n, int k, int pmax) {        \
-    constexpr int BN = WNW * TN * 32;                                                                              \
-    static_assert(BN == 256 && WMW * WNW == 8, "both cells are 8 waves and 256 columns wide");                     \
-    if constexpr (!LIGHT) {                                                                                        \
-      /* one cell, items in table order */                                                                        \
-      __shared__ unsigned short s_order[MOE_ORDER_CAP];                                                            \
-      const int nt = meta[0], gx = (n + BN - 1) / BN, total = nt * gx;                                             \
-      const bool ordered = nt <= MOE_ORDER_CAP;                                                                    \
-      if (ordered) moe_tile_order<WMW * WNW * 64>(tile_rows, nt, s_order);                                         \
-      iu8_pf32_run<false, WMW, WNW, TM, TN, false, ST, false, true, GATHER == 2>(a, as, c, n, k, [&](int r, iu8_tile &t) { \
-        const int id = (int)blockIdx.x + r * (int)gridDim.x;                                                       \
-        if (id >= total) return false;                                                                             \
-        const int slot = id / gx, bx = id - slot * gx, tile = ordered ? (int)s_order[slot] : slot;                 \
-        const int e = tile_expert[tile];                                                                           \
-        t = iu8_tile{iu8_rows{GATHER ? row_tok : nullptr, tile_row0[tile], min(tile_rows[tile], WMW * TM * 32)}, 0, \
-                     bx * (BN / 16), (const unsigned char *)xptr[2 * e], (const float *)xptr[2 * e + 1]};          \
-        return true;                                                                                               \
-      });                                                                                                          \
-      return;                                                                                                      \
-    }                                                                                                              \
-    constexpr int LB = iu8_pf32_lds_bytes<false, WMW, WNW, TM, TN, ST>();                                          \
-    constexpr int LL = iu8_pf32_lds_bytes<false, 2, 4, 1, 2, MOE_LIGHT_ST>();                                      \
-    __shared__ __attribute__((aligned(1024))) iu8_u8 lds[LB > LL ? LB : LL];                                       \
-    __shared__ unsigned short s_order[MOE_ORDER_CAP];                                                              \
-    /* the walk's numbers and this workgroup's resolved items live in LDS */                                      \
-    __shared__ int s_par[4];                                                                                       \
-    __shared__ moe_item s_item[MOE_HEAVY_ROUNDS + MOE_LIGHT_ROUNDS];                                               \
-    auto par = [&](int i) { return __builtin_amdgcn_readfirstlane(((volatile int *)s_par)[i]); };                  \
-    auto item = [&](int q, iu8_tile &t) {                                                                          \
-      const volatile int *p32 = (const volatile int *)&s_item[q];                                                  \
-      auto u = [&](int i) { return __builtin_amdgcn_readfirstlane(p32[i]); };                                      \
-      if (u(1) < 0) return false;                                                                                  \
-      const unsigned long long wp = (unsigned)u(4) | ((unsigned long long)(unsigned)u(5) << 32);                   \
-      const unsigned long long sp = (unsigned)u(6) | ((unsigned long long)(unsigned)u(7) << 32);                   \
-      t = iu8_tile{iu8_rows{GATHER ? row_tok : nullptr, u(0), u(1)}, 0, u(2), (const unsigned char *)wp, (const float *)sp, 0, u(3)}; \
-      return true;                                                                                                 \
-    };                                                                                                             \
-    const int nt = meta[0];                                                                                        \
-    const bool ordered = nt <= MOE_ORDER_CAP;                                                                      \
-    const int heavy = ordered ? moe_tile_order<WMW * WNW * 64>(tile_rows, nt, s_order) : nt;                       \
-    /* a launch of more rounds than the item table holds runs in epochs of that many */                           \
-    for (int ep = 0;; ++ep) {                                                                                      \
-      {                                                                                                            \
-        const int gx = (n + BN - 1) / BN, G = gridDim.x, w = blockIdx.x;                                           \
-        const int hi = heavy * gx, li = (nt - heavy) * gx;                                                         \
-        const int h0 = ep * MOE_HEAVY_ROUNDS, l0 = ep * MOE_LIGHT_ROUNDS;                                          \
-        const int rounds = max(0, min((hi + G - 1) / G - h0, MOE_HEAVY_ROUNDS));                                   \
-        const int lrounds = max(0, min((li + G - 1) / G - l0, MOE_LIGHT_ROUNDS));                                  \
-        if (rounds + lrounds == 0) break;                                                                          \
-        /* a workgroup's heavy items run in two parts, its light items between them, after `first` rounds */      \
-        if (threadIdx.x == 0) {                                                                                    \
-          s_par[0] = rounds, s_par[1] = lrounds;                                                                   \
-          s_par[2] = lrounds > 0 ? (w >> 3) % (rounds + 1) : rounds;                                               \
-        }                                                                                                          \
-        const int q = threadIdx.x;                                                                                 \
-        if (q < rounds + lrounds) {                                                                                \
-          const bool light = q >= rounds;                                                                          \
-          const int id = light ? G - 1 - w + (l0 + q - rounds) * G : w + (h0 + q) * G;                             \
-          moe_item it{0, -1, 0, 0, nullptr, nullptr};                                                              \
-          if (id < (light ? li : hi)) {                                                                            \
-            const int slot = (light ? heavy : 0) + id / gx, tile = ordered ? (int)s_order[slot] : slot;            \
-            const int e = tile_expert[tile];                                                                       \
-            it = moe_item{tile_row0[tile], min(tile_rows[tile], light ? MOE_LIGHT_ROWS : WMW * TM * 32),           \
-                          id % gx * (BN / 16), light ? (int)(((unsigned)id * 2654435761u >> 10) % (unsigned)(k >> 7)) : 0, \
-                          (const unsigned char *)xptr[2 * e], (const float *)xptr[2 * e + 1]};                     \
-          }                                                                                                        \
-          s_item[q] = it;                                                                                          \
-        }                                                                                                          \
-        __syncthreads();                                                                                           \
-      }                                                                                                            \
-      for (int part = 0; part < 2; ++part) {                                                                       \
-        if (part == 1) {                                                                                           \
-          if (par(1) == 0) break;                                                                                  \
-          iu8_pf32_run<false, 2, 4, 1, 2, false, MOE_LIGHT_ST, true, false, GATHER == 2, true>(                    \
-              a, as, c, n, k, [&](int r, iu8_tile &t) { return r < par(1) && item(par(0) + r, t); }, nullptr, nullptr, lds); \
-          __syncthreads();                                                                                         \
-        }                                                                                                          \
-        iu8_pf32_run<false, WMW, WNW, TM, TN, false, ST, false, true, GATHER == 2, true>(                          \
-            a, as, c, n, k,                                                                                        \
-            [&](int r, iu8_tile &t) {                                                                              \
-              const int first = par(2), rr = part ? first + r : r;                                                 \
-              return rr < (part ? par(0) : first) && item(rr, t);                                                  \
-            },                                                                                                     \
-            nullptr, nullptr, lds);                                                                                \
-        __syncthreads();                                                                                           \
-      }                                                                                                            \
-    }                                                                                                              \
+    BODY<GATHER, WMW, WNW, TM, TN, ST>(a, xptr, tile_expert, tile_row0, tile_rows, row_tok, meta, as, c, n, k);    \
   }
 // tiles of up to 128 rows (tile_blocks 8) on the 128 x 256 tile of 2 x 4 waves
-MOE_GROUPED_PF(moe_iu8_grouped_w4_pf_g2, 2, 2, 4, 2, 2, 4, true)
-MOE_GROUPED_PF(moe_iu8_grouped_w4_pf_g1, 1, 2, 4, 2, 2, 4, true)
-MOE_GROUPED_PF(moe_iu8_grouped_w4_pf_g0, 0, 2, 4, 2, 2, 4, true)
+MOE_GROUPED_PF(moe_iu8_grouped_w4_pf_g2, moe_grouped_pf_two, 2, 2, 4, 2, 2, 4)
+MOE_GROUPED_PF(moe_iu8_grouped_w4_pf_g1, moe_grouped_pf_two, 1, 2, 4, 2, 2, 4)
+MOE_GROUPED_PF(moe_iu8_grouped_w4_pf_g0, moe_grouped_pf_two, 0, 2, 4, 2, 2, 4)
 // tiles of up to 256 rows (tile_blocks 16) on the 256 x 256 tile, the dense GEMM's fastest cell
-MOE_GROUPED_PF(moe_iu8_grouped_w4_pf16_g2, 2, 2, 4, 4, 2, 3, false)
-MOE_GROUPED_PF(moe_iu8_grouped_w4_pf16_g1, 1, 2, 4, 4, 2, 3, false)
-MOE_GROUPED_PF(moe_iu8_grouped_w4_pf16_g0, 0, 2, 4, 4, 2, 3, false)
+MOE_GROUPED_PF(moe_iu8_grouped_w4_pf16_g2, moe_grouped_pf_one, 2, 2, 4, 4, 2, 3)
+MOE_GROUPED_PF(moe_iu8_grouped_w4_pf16_g1, moe_grouped_pf_one, 1, 2, 4, 4, 2, 3)
+MOE_GROUPED_PF(moe_iu8_grouped_w4_pf16_g0, moe_grouped_pf_one, 0, 2, 4, 4, 2, 3)
 #undef MOE_GROUPED_PF
 
 // ---------------------------------------------------------------------------- combine
