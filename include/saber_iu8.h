@@ -111,7 +111,7 @@ typedef struct {
   uint32_t shared_bytes;  /* always 0: LDS is static */
   uint32_t kernarg_bytes; /* explicit arguments only */
   uint32_t n_args;
-  saber_iu8_slot args[20];
+  saber_iu8_slot args[24];
   uint32_t n_workspaces;
   saber_iu8_workspace workspaces[4];
   uint32_t n_launches; /* 1: split-K reduce is fused */
@@ -319,6 +319,15 @@ typedef struct {
 /* Router + expert-major sort + tile table, one launch. logits bf16 [T, experts]. */
 int saber_iu8_moe_route(saber_iu8_ctx *ctx, const void *logits_bf16, uint32_t tokens, uint32_t experts, uint32_t topk,
                         uint32_t tile_blocks, const saber_iu8_moe_tables *t, void *stream);
+
+/* The router and the per-token quantisation of the layer's input in one launch (the two are
+ * independent; in the reference they are two operators, moe_route.hip:108-284 and the int8 producer
+ * mxfp4_hadi8.hip:22-58): what saber_iu8_moe_route and saber_iu8_quant(x, q, scale, tokens, k) would
+ * write, for the few-token regime where a layer's time is its launches. x bf16 [tokens, k], q in the
+ * A fragment order ([ceil(tokens/16)*16, k] bytes), scale f32 [tokens]; K % 128 == 0, K <= 16384. */
+int saber_iu8_moe_route_quant(saber_iu8_ctx *ctx, const void *logits_bf16, const void *x_bf16, void *q, float *scale,
+                              uint32_t tokens, uint32_t experts, uint32_t topk, uint32_t k, uint32_t tile_blocks,
+                              const saber_iu8_moe_tables *t, void *stream);
 
 /* Grouped W4 GEMM over the tile table: per tile the expert's weights (gfx950 W4 fragments) at
  * xptr[2e] and f32 row scales at xptr[2e + 1] (device array of 2 * experts addresses); A rows

@@ -49,6 +49,13 @@ static const Signature SIG_MOE_ROUTE = {
     {"route_pos", K::Buffer},   {"row_tok", K::Buffer},  {"row_route", K::Buffer}, {"tile_expert", K::Buffer},
     {"tile_row0", K::Buffer},   {"tile_rows", K::Buffer}, {"expert_cnt", K::Buffer}, {"meta", K::Buffer},
     {"blk_cnt", K::Buffer},     {"rank", K::Buffer},     {"arrive", K::Buffer}};
+static const Signature SIG_MOE_ROUTEQ = {
+    {"logits", K::Buffer},      {"t", K::I32},           {"e_lo", K::I32},        {"e_loc", K::I32},
+    {"tile_blocks", K::I32},    {"with_shared", K::I32}, {"topk_ids", K::Buffer}, {"topk_w", K::Buffer},
+    {"route_pos", K::Buffer},   {"row_tok", K::Buffer},  {"row_route", K::Buffer}, {"tile_expert", K::Buffer},
+    {"tile_row0", K::Buffer},   {"tile_rows", K::Buffer}, {"expert_cnt", K::Buffer}, {"meta", K::Buffer},
+    {"blk_cnt", K::Buffer},     {"rank", K::Buffer},     {"arrive", K::Buffer},   {"x", K::Buffer},
+    {"q", K::Buffer},           {"scale", K::Buffer},    {"k", K::I32}};
 static const Signature SIG_MOE_GROUPED = {
     {"a", K::Buffer},       {"xptr", K::Buffer}, {"tile_expert", K::Buffer}, {"tile_row0", K::Buffer},
     {"tile_rows", K::Buffer}, {"row_tok", K::Buffer}, {"meta", K::Buffer},   {"as", K::Buffer},
@@ -86,6 +93,7 @@ const Signature *signature_for(const std::string &k) {
   if (k == "iu8_probe_empty") return &SIG_PROBE_EMPTY;
   if (k == "iu8_probe_mfma" || k == "iu8_probe_mfma32") return &SIG_PROBE_MFMA;
   if (starts(k, "moe_iu8_route_")) return &SIG_MOE_ROUTE;
+  if (starts(k, "moe_iu8_routeq_")) return &SIG_MOE_ROUTEQ;
   if (starts(k, "moe_iu8_grouped_")) return &SIG_MOE_GROUPED;
   if (starts(k, "moe_iu8_combine_")) return &SIG_MOE_COMBINE;
   return nullptr;

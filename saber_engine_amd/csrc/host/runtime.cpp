@@ -568,6 +568,30 @@ int saber_iu8_moe_route(saber_iu8_ctx *ctx, const void *logits, uint32_t tokens,
   return saber_iu8_launch(ctx, &d, b, sizeof b / sizeof b[0], stream);
 }
 
+int saber_iu8_moe_route_quant(saber_iu8_ctx *ctx, const void *logits, const void *x, void *q, float *scale, uint32_t tokens,
+                              uint32_t experts, uint32_t topk, uint32_t k, uint32_t tile_blocks,
+                              const saber_iu8_moe_tables *t, void *stream) {
+  if (int rc = moe_check("moe_route_quant", tokens, experts, topk, t)) return rc;
+  if (tile_blocks == 0) return fail(SABER_IU8_E_RULE, "moe_route_quant: tile_blocks 0");
+  if (k == 0 || k % 128 != 0 || k > 16384)
+    return fail(SABER_IU8_E_RULE, fmt("moe_route_quant: K=%u must be a multiple of 128 (the slab) up to 16384 (a 16-element group a thread)", k));
+  saber_iu8_desc d;
+  if (int rc = raw_desc("moe_iu8_routeq_topk8_sort_e128", (tokens + 127) / 128 + tokens, 1, 1024, &d)) return rc;
+  set_i32(&d, "t", tokens);
+  set_i32(&d, "e_lo", 0);
+  set_i32(&d, "e_loc", experts);
+  set_i32(&d, "tile_blocks", tile_blocks);
+  set_i32(&d, "with_shared", 0);
+  set_i32(&d, "k", k);
+  const saber_iu8_binding b[] = {{"logits", (void *)logits},      {"topk_ids", t->topk_ids},   {"topk_w", t->topk_w},
+                                 {"route_pos", t->route_pos},     {"row_tok", t->row_tok},     {"row_route", t->row_route},
+                                 {"tile_expert", t->tile_expert}, {"tile_row0", t->tile_row0}, {"tile_rows", t->tile_rows},
+                                 {"expert_cnt", t->expert_cnt},   {"meta", t->meta},           {"blk_cnt", t->blk_cnt},
+                                 {"rank", t->rank},               {"arrive", t->arrive},       {"x", (void *)x},
+                                 {"q", q},                        {"scale", scale}};
+  return saber_iu8_launch(ctx, &d, b, sizeof b / sizeof b[0], stream);
+}
+
 int saber_iu8_moe_grouped(saber_iu8_ctx *ctx, const void *a, const float *as, const void *xptr, void *c, uint32_t n,
                           uint32_t k, int gather, uint32_t tokens, uint32_t experts, uint32_t topk, uint32_t tile_blocks,
                           const saber_iu8_moe_tables *t, void *stream) {

@@ -88,12 +88,13 @@ static __device__ __forceinline__ int moe_exscan(int v, int *s_wave, int *total)
   return base + x - v;
 }
 
-extern "C" __global__ __launch_bounds__(MOE_THREADS) void moe_iu8_route_topk8_sort_e128(
+// The router's workgroup `blk` of `nblk` (128 tokens each).
+static __device__ __forceinline__ void moe_route_body(
     const unsigned short *__restrict__ logits, int T, int e_lo, int e_loc, int tile_blocks, int with_shared,
     int *__restrict__ topk_ids, float *__restrict__ topk_w, int *__restrict__ route_pos, int *__restrict__ row_tok,
     int *__restrict__ row_route, int *__restrict__ tile_expert, int *__restrict__ tile_row0,
     int *__restrict__ tile_rows, int *__restrict__ expert_cnt, int *__restrict__ meta, int *__restrict__ blk_cnt,
-    int *__restrict__ rank, int *__restrict__ arrive) {
+    int *__restrict__ rank, int *__restrict__ arrive, const int nblk, const int blk) {
 #pragma clang fp contract(off)
   __shared__ __attribute__((aligned(16))) int s_ids[MOE_TPB * MOE_TOPK];
   __shared__ int s_part[MOE_THREADS / MOE_E][MOE_E];
@@ -104,7 +105,7 @@ extern "C" __global__ __launch_bounds__(MOE_THREADS) void moe_iu8_route_topk8_so
   __shared__ int s_wave[MOE_THREADS / 64];
   __shared__ int s_last;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int nblk = gridDim.x, blk = blockIdx.x, t0 = blk * MOE_TPB;
+  const int t0 = blk * MOE_TPB;
 
   for (int e = tid; e < MOE_E; e += MOE_THREADS) s_cnt[e] = 0;
   for (int i = tid; i < MOE_E * (MOE_TPB / 32); i += MOE_THREADS) s_mask[i / (MOE_TPB / 32)][i % (MOE_TPB / 32)] = 0u;
@@ -369,6 +370,69 @@ extern "C" __global__ __launch_bounds__(MOE_THREADS) void moe_iu8_route_topk8_so
   }
   if (rows_total == 0)  // no local route at all: the positions still have to be written
     for (int r = tid; r < R; r += MOE_THREADS) route_pos[r] = -1;
+}
+extern "C" __global__ __launch_bounds__(MOE_THREADS) void moe_iu8_route_topk8_sort_e128(
+    const unsigned short *__restrict__ logits, int T, int e_lo, int e_loc, int tile_blocks, int with_shared,
+    int *__restrict__ topk_ids, float *__restrict__ topk_w, int *__restrict__ route_pos, int *__restrict__ row_tok,
+    int *__restrict__ row_route, int *__restrict__ tile_expert, int *__restrict__ tile_row0,
+    int *__restrict__ tile_rows, int *__restrict__ expert_cnt, int *__restrict__ meta, int *__restrict__ blk_cnt,
+    int *__restrict__ rank, int *__restrict__ arrive) {
+  moe_route_body(logits, T, e_lo, e_loc, tile_blocks, with_shared, topk_ids, topk_w, route_pos, row_tok, row_route,
+                 tile_expert, tile_row0, tile_rows, expert_cnt, meta, blk_cnt, rank, arrive, gridDim.x, blockIdx.x);
+}
+
+// The router and the tokens' quantisation in one launch, for the few-token regime where a layer's time
+// is its launches: the two do not depend on each other, so the first ceil(T / 128) workgroups route and
+// workgroup ceil(T / 128) + t quantises token t (x bf16 [T, k] -> codes in the A fragment order +
+// scale[t]; macaq_i8.h:10-13, one 16-element group a thread, k <= 16,384). grid [ceil(T/128) + T, 1, 1].
+extern "C" __global__ __launch_bounds__(MOE_THREADS) void moe_iu8_routeq_topk8_sort_e128(
+    const unsigned short *__restrict__ logits, int T, int e_lo, int e_loc, int tile_blocks, int with_shared,
+    int *__restrict__ topk_ids, float *__restrict__ topk_w, int *__restrict__ route_pos, int *__restrict__ row_tok,
+    int *__restrict__ row_route, int *__restrict__ tile_expert, int *__restrict__ tile_row0,
+    int *__restrict__ tile_rows, int *__restrict__ expert_cnt, int *__restrict__ meta, int *__restrict__ blk_cnt,
+    int *__restrict__ rank, int *__restrict__ arrive, const unsigned short *__restrict__ x,
+    unsigned char *__restrict__ q, float *__restrict__ scale, int k) {
+#pragma clang fp contract(off)
+  const int nblk = (T + MOE_TPB - 1) / MOE_TPB;
+  if ((int)blockIdx.x < nblk) {
+    moe_route_body(logits, T, e_lo, e_loc, tile_blocks, with_shared, topk_ids, topk_w, route_pos, row_tok, row_route,
+                   tile_expert, tile_row0, tile_rows, expert_cnt, meta, blk_cnt, rank, arrive, nblk, blockIdx.x);
+    return;
+  }
+  __shared__ float s_max[MOE_THREADS / 64];
+  const int row = blockIdx.x - nblk, g = threadIdx.x, G = k >> 4;
+  float v[16];
+#pragma unroll
+  for (int j = 0; j < 16; ++j) v[j] = 0.f;
+  if (g < G) {
+    const unsigned short *xr = x + (size_t)row * k + g * 16;
+    const iu8_v4u lo = *(const iu8_v4u *)xr, hi = *(const iu8_v4u *)(xr + 8);
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      v[2 * w] = __uint_as_float(lo[w] << 16);
+      v[2 * w + 1] = __uint_as_float(lo[w] & 0xFFFF0000u);
+      v[8 + 2 * w] = __uint_as_float(hi[w] << 16);
+      v[8 + 2 * w + 1] = __uint_as_float(hi[w] & 0xFFFF0000u);
+    }
+  }
+  float amax = 0.f;
+#pragma unroll
+  for (int j = 0; j < 16; ++j) amax = fmaxf(amax, fabsf(v[j]));
+  amax = iu8_wave_max_nonneg(amax);
+  if ((threadIdx.x & 63) == 0) s_max[threadIdx.x >> 6] = amax;
+  __syncthreads();
+#pragma unroll
+  for (int w = 0; w < MOE_THREADS / 64; ++w) amax = fmaxf(amax, s_max[w]);
+  const float sc = fmaxf(__fdiv_rn(amax, 127.f), 1e-30f), rcp = __fdiv_rn(1.f, sc);
+  if (threadIdx.x == 0) scale[row] = sc;
+  if (g < G) {
+    unsigned d[4];
+#pragma unroll
+    for (int w = 0; w < 4; ++w) d[w] = iu8_code4_rcp(v[w * 4], v[w * 4 + 1], v[w * 4 + 2], v[w * 4 + 3], sc, rcp);
+    // fragment (row / 16, k / 64): 1 KiB; the 16 bytes of (row % 16, k chunk (g & 3)) at (row % 16 + 16 * chunk) * 16
+    *(iu8_v4u *)(q + ((size_t)(row >> 4) * (k >> 6) + (g >> 2)) * 1024 + (g & 3) * 256 + (row & 15) * 16) =
+        iu8_v4u{d[0], d[1], d[2], d[3]};
+  }
 }
 
 // ---------------------------------------------------------------------------- grouped GEMMs

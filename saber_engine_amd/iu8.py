@@ -37,7 +37,7 @@ class Workspace(C.Structure):
 class Desc(C.Structure):
     _fields_ = [("op", C.c_char * 24), ("plugin", C.c_char * 24), ("kernel", C.c_char * 64), ("grid", C.c_uint32 * 3),
                 ("block", C.c_uint32 * 3), ("shared_bytes", C.c_uint32), ("kernarg_bytes", C.c_uint32),
-                ("n_args", C.c_uint32), ("args", Slot * 20), ("n_workspaces", C.c_uint32), ("workspaces", Workspace * 4),
+                ("n_args", C.c_uint32), ("args", Slot * 24), ("n_workspaces", C.c_uint32), ("workspaces", Workspace * 4),
                 ("n_launches", C.c_uint32), ("ks", C.c_uint32)]
 
     def summary(self):
@@ -126,6 +126,7 @@ def lib():
         L.saber_iu8_moe_tiles_cap.restype = C.c_uint32
         L.saber_iu8_moe_tiles_cap.argtypes = [C.c_uint32] * 4
         L.saber_iu8_moe_route.argtypes = [C.c_void_p, C.c_void_p] + [C.c_uint32] * 4 + [C.POINTER(MoeTables), C.c_void_p]
+        L.saber_iu8_moe_route_quant.argtypes = [C.c_void_p] * 5 + [C.c_uint32] * 5 + [C.POINTER(MoeTables), C.c_void_p]
         L.saber_iu8_moe_grouped.argtypes = ([C.c_void_p] * 5 + [C.c_uint32, C.c_uint32, C.c_int] + [C.c_uint32] * 4 +
                                             [C.POINTER(MoeTables), C.c_void_p])
         L.saber_iu8_moe_quant_rows.argtypes = [C.c_void_p] * 4 + [C.c_uint32, C.c_uint32, C.POINTER(MoeTables), C.c_void_p]
@@ -335,6 +336,10 @@ class Context:
     # ---- routed experts
     def moe_route(self, logits, tokens, experts, topk, tile_blocks, tables, stream=0):
         _check(lib().saber_iu8_moe_route(self._h, logits, tokens, experts, topk, tile_blocks, C.byref(tables), stream))
+
+    def moe_route_quant(self, logits, x, q, scale, tokens, experts, topk, k, tile_blocks, tables, stream=0):
+        _check(lib().saber_iu8_moe_route_quant(self._h, logits, x, q, scale, tokens, experts, topk, k, tile_blocks,
+                                               C.byref(tables), stream))
 
     def moe_grouped(self, a, a_scale, xptr, c, n, k, gather, tokens, experts, topk, tile_blocks, tables, stream=0):
         _check(lib().saber_iu8_moe_grouped(self._h, a, a_scale, xptr, c, n, k, int(gather), tokens, experts, topk,

@@ -55,11 +55,15 @@ class MoeLayerIU8:
     def forward(self, x, logits, stream=0):
         """x bf16 bits [T,H] (int16 tensor), logits bf16 bits [T,E]; every launch on `stream`."""
         c, T, E, k, H, I = self.ctx, self.T, self.E, self.topk, self.H, self.I
-        c.moe_route(logits.data_ptr(), T, E, k, self.tb, self.tables, stream)
-        if self.gather == 1:
-            c.quant(x.data_ptr(), self.q1.data_ptr(), self.s1.data_ptr(), T, H, stream)
+        if self.gather == 1 and H <= 16384:   # few tokens: the router and the quantisation in one launch
+            c.moe_route_quant(logits.data_ptr(), x.data_ptr(), self.q1.data_ptr(), self.s1.data_ptr(), T, E, k, H, self.tb,
+                              self.tables, stream)
         else:
-            c.quant_rowmajor(x.data_ptr(), self.q1.data_ptr(), self.s1.data_ptr(), T, H, stream)
+            c.moe_route(logits.data_ptr(), T, E, k, self.tb, self.tables, stream)
+            if self.gather == 1:
+                c.quant(x.data_ptr(), self.q1.data_ptr(), self.s1.data_ptr(), T, H, stream)
+            else:
+                c.quant_rowmajor(x.data_ptr(), self.q1.data_ptr(), self.s1.data_ptr(), T, H, stream)
         c.moe_grouped(self.q1.data_ptr(), self.s1.data_ptr(), self.xptr_gu.data_ptr(), self.gu.data_ptr(), 2 * I, H,
                       self.gather, T, E, k, self.tb, self.tables, stream)
         c.moe_silu_mul_quant(self.gu.data_ptr(), self.q2.data_ptr(), self.s2.data_ptr(), I, self.rows_cap, self.tables, stream)

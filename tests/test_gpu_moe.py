@@ -113,6 +113,42 @@ def test_moe_layer_two_cell_walk(ctx, T, I, hot, boost):
     check_layer(layer, case)
 
 
+@pytest.mark.parametrize("T,H", [(1, 128), (16, 4096), (37, 640), (112, 16384), (300, 512)])
+def test_route_and_quant_in_one_launch(ctx, T, H):
+    """The merged launch writes what the router and the int8 producer write on their own: tables,
+    codes (A fragment order) and scales, byte for byte; twice in a row (the arrival counter)."""
+    say(f"moe route + quant in one launch: T={T} H={H}")
+    E, k = 128, 8
+    rng = np.random.default_rng(T * 31 + H)
+    X = synth.activations(rng, T, H)
+    if T > 2:
+        X[1] = 0                                            # an all-zero row: scale 1e-30, codes 0
+    logits = synth.f32_to_bf16_bits(rng.standard_normal(size=(T, E), dtype=np.float32))
+    x, lg = dev_bf16_bits(X), dev_bf16_bits(logits)
+    a, b = MoeLayerIU8(ctx, T, E, k, H, 256), MoeLayerIU8(ctx, T, E, k, H, 256)
+    qa = torch.full((iu8.a_bytes(T, H),), 0x55, dtype=torch.uint8, device="cuda")
+    sa = torch.zeros(T, dtype=torch.float32, device="cuda")
+    for _ in range(2):
+        ctx.moe_route_quant(lg.data_ptr(), x.data_ptr(), qa.data_ptr(), sa.data_ptr(), T, E, k, H, a.tb, a.tables)
+    ctx.moe_route(lg.data_ptr(), T, E, k, b.tb, b.tables)
+    torch.cuda.synchronize()
+    want_q, want_s = ref.quant_bf16(X)
+    np.testing.assert_array_equal(sa.cpu().numpy().view(np.uint32), want_s.view(np.uint32))
+    np.testing.assert_array_equal(iu8.unpack_a(qa.cpu().numpy(), T, H), want_q)
+    nt, rows = int(a.buf["meta"][0].item()), int(a.buf["meta"][1].item())
+    for name in ("topk_ids", "topk_w", "route_pos", "expert_cnt", "meta", "arrive"):
+        assert torch.equal(a.buf[name], b.buf[name]), name
+    for name in ("tile_expert", "tile_row0", "tile_rows"):
+        assert torch.equal(a.buf[name][:nt], b.buf[name][:nt]), name
+    for name in ("row_tok", "row_route"):
+        assert torch.equal(a.buf[name][:rows], b.buf[name][:rows]), name
+    ids, _ = ref.route(logits, k)
+    np.testing.assert_array_equal(a.buf["topk_ids"].cpu().numpy().reshape(T, k), ids)
+    with pytest.raises(iu8.IU8Error) as e:
+        ctx.moe_route_quant(lg.data_ptr(), x.data_ptr(), qa.data_ptr(), sa.data_ptr(), T, E, k, 16512, a.tb, a.tables)
+    assert e.value.code == iu8.E_RULE
+
+
 def test_moe_router_ties_and_skew(ctx):
     say("moe router: ties and one hot expert")
     case = synth.moe_case(T=40, E=128, topk=8, H=512, I=256, seed=5, experts=4)
