@@ -30,7 +30,7 @@ LAYERS = 6                  # distinct weight copies walked by successive steps 
 # HBM-side bytes of one launch of the dominant kernel, mean over the four layer shapes, from
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this very command (profiles/macaq_iu8_decq_w4_tm1__layer_set_m1.txt), each
 # counter scaled by what it reads for the 256 MiB copy probe. Keyed by (kernel, M); None = not measured.
-TRAFFIC = {("macaq_iu8_decq_w4_tm1", 1): 41894217.0, ("macaq_iu8_dec_w4_tm1", 1): 41992603.0}
+TRAFFIC = {("macaq_iu8_decq_w4_tm1", 1): 41893449.0, ("macaq_iu8_dec_w4_tm1", 1): 41992603.0}
 
 
 def alg_bytes(m, n, k, w8=False):
