@@ -442,9 +442,13 @@ def main():
             layer.set_weights(wgu, wsgu, wdn, wsdn)
             x = torch.randn((T, H), device=dev, generator=g).to(torch.bfloat16).view(torch.int16)
             lg = torch.randn((T, E), device=dev, generator=g).to(torch.bfloat16).view(torch.int16)
-            reps = 20 if T == 16 else 5
+            # a run long enough (0.2 s at T = 4096) to show the layer's own sustained rate, from an idle
+            # card: straight after the dense prefill sections a short burst ran 15-20 % slower
+            reps = 200
+            torch.cuda.synchronize()
+            time.sleep(1.0)
             with torch.cuda.stream(stream):
-                for _ in range(3):
+                for _ in range(20):
                     layer.forward(x, lg, sh)
                 e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                 e0.record(stream)
