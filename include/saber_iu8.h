@@ -293,7 +293,7 @@ int saber_iu8_gemm_acc(saber_iu8_ctx *ctx, int wkind, const void *a, const void 
 uint32_t saber_iu8_moe_rows_cap(uint32_t tokens, uint32_t topk, uint32_t experts);
 uint32_t saber_iu8_moe_tiles_cap(uint32_t tokens, uint32_t topk, uint32_t experts, uint32_t tile_blocks);
 /* tile_blocks the grouped law picks for `tokens`: 1 (16-row tiles, weight-streaming cells) while an
- * expert averages <= 7 routes, 8 (128-row MFMA tiles) up to 96 routes an expert, 16 (256-row) from there. */
+ * expert averages <= 7 routes, 8 (128-row MFMA tiles) below 128 routes an expert, 16 (256-row) from there. */
 uint32_t saber_iu8_moe_tile_blocks(uint32_t tokens, uint32_t topk, uint32_t experts);
 
 /* Device buffers of one routed layer, named as the router kernel's arguments

@@ -525,15 +525,17 @@ uint32_t saber_iu8_moe_tiles_cap(uint32_t tokens, uint32_t topk, uint32_t expert
 // Rows a tile (x16). 16-row tiles on the streaming cell while routes are few (up to 7 routes an
 // expert on average); above, the MFMA cells, whose sparse forms make a thinly filled tile cost about
 // its weight traffic and which stream an expert's weights once instead of once a 16-row tile:
-// 128-row tiles up to 96 routes an expert, 256-row tiles (one tile an expert more often than not, on
-// the dense GEMM's fastest shape) from there. Speed data of this card, 128 experts, top-8,
+// 128-row tiles while an expert's routes on average do not fill one (the two-cell kernels, which run
+// the thin tiles on a small cell), 256-row tiles (one tile an expert more often than not, on the
+// dense GEMM's fastest shape) from 128 routes an expert. Speed data of this card, 128 experts, top-8,
 // 4096 x 1536, us a layer at tile_blocks 1 / 8 / 16: T=32 255 / 309 / 328, T=64 296 / 335 / 347,
-// T=80 318 / 340, T=128 363 / 347 / 362, T=256 730 / 376 / 379, T=512 1282 / 370 / 396,
-// T=1024 2349 / 430 / 469, T=2048 - / 650 / 597, T=4096 - / 982 / 952.
+// T=80 318 / 340, T=128 363 / 347 / 362, T=256 730 / 293 / 298, T=512 1282 / 315 / 319,
+// T=1024 2349 / 377 / 402, T=1280 - / 425 / 458, T=1536 - / 472 / 528, T=1792 - / 493 / 516,
+// T=1920 - / 526 / 532, T=2048 - / 586 / 544, T=4096 - / 960 / 916.
 uint32_t saber_iu8_moe_tile_blocks(uint32_t tokens, uint32_t topk, uint32_t experts) {
   const uint64_t routes = (uint64_t)tokens * topk;
   if (routes <= 7ull * experts) return 1u;
-  return routes >= 96ull * experts ? 16u : 8u;
+  return routes >= 128ull * experts ? 16u : 8u;
 }
 
 static int moe_check(const char *what, uint32_t tokens, uint32_t experts, uint32_t topk, const saber_iu8_moe_tables *t) {

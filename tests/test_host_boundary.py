@@ -145,8 +145,8 @@ def test_launch_law_shares_k_only_on_deep_narrow_tile_gemms():
 
 def test_moe_tile_law_thresholds():
     """16-row streaming tiles up to 7 routes an expert, 128-row MFMA tiles up to 96, 256-row above."""
-    got = {t: iu8.moe_tile_blocks(t, 8, 128) for t in (1, 16, 112, 113, 256, 1535, 1536, 4096)}
-    assert got == {1: 1, 16: 1, 112: 1, 113: 8, 256: 8, 1535: 8, 1536: 16, 4096: 16}
+    got = {t: iu8.moe_tile_blocks(t, 8, 128) for t in (1, 16, 112, 113, 256, 1536, 2047, 2048, 4096)}
+    assert got == {1: 1, 16: 1, 112: 1, 113: 8, 256: 8, 1536: 8, 2047: 8, 2048: 16, 4096: 16}
     assert iu8.moe_tiles_cap(4096, 8, 128, 16) == 128 + 128 + 1 and iu8.moe_rows_cap(4096, 8, 128) == 32768 + 15 * 128
 
 
