@@ -536,6 +536,7 @@ static __device__ __forceinline__ int moe_tile_order(const int *__restrict__ til
   return heavy_total;
 }
 // one cell, items in the sorted order
+#define MOE_ONE_ITEMS 64  // items a workgroup resolves up front (16,384 items a launch of 256 workgroups)
 template <int GATHER, int WMW, int WNW, int TM, int TN, int ST>
 static __device__ __forceinline__ void moe_grouped_pf_one(
     const unsigned char *__restrict__ a, const unsigned long long *__restrict__ xptr, const int *__restrict__ tile_expert,
@@ -544,18 +545,50 @@ static __device__ __forceinline__ void moe_grouped_pf_one(
   constexpr int BN = WNW * TN * 32;
   static_assert(BN == 256 && WMW * WNW == 8, "both cells are 8 waves and 256 columns wide");
   __shared__ unsigned short s_order[MOE_ORDER_CAP];
+  __shared__ moe_item s_item[MOE_ONE_ITEMS];
+  __shared__ __attribute__((aligned(1024))) iu8_u8 lds[iu8_pf32_lds_bytes<false, WMW, WNW, TM, TN, ST>()];  // one block for both walks below
   const int nt = meta[0], gx = (n + BN - 1) / BN, total = nt * gx;
   const bool ordered = nt <= MOE_ORDER_CAP;
   if (ordered) moe_tile_order<WMW * WNW * 64>(tile_rows, nt, s_order);
-  iu8_pf32_run<false, WMW, WNW, TM, TN, false, ST, false, true, GATHER == 2>(a, as, c, n, k, [&](int r, iu8_tile &t) {
-    const int id = (int)blockIdx.x + r * (int)gridDim.x;
-    if (id >= total) return false;
+  auto resolve = [&](int id, moe_item &it) {
     const int slot = id / gx, bx = id - slot * gx, tile = ordered ? (int)s_order[slot] : slot;
     const int e = tile_expert[tile];
-    t = iu8_tile{iu8_rows{GATHER ? row_tok : nullptr, tile_row0[tile], min(tile_rows[tile], WMW * TM * 32)}, 0,
-                 bx * (BN / 16), (const unsigned char *)xptr[2 * e], (const float *)xptr[2 * e + 1]};
+    it = moe_item{tile_row0[tile], min(tile_rows[tile], WMW * TM * 32), bx * (BN / 16), 0,
+                  (const unsigned char *)xptr[2 * e], (const float *)xptr[2 * e + 1]};
+  };
+  const int G = gridDim.x, rounds = (total + G - 1) / G;
+  if (rounds <= MOE_ONE_ITEMS) {
+    // An item's descriptor hangs on a chain of dependent loads (order -> tile table -> expert pointers);
+    // fetched where the load stream crosses into the item, every link drains the stream. The
+    // workgroup's items are resolved here instead, one lane an item, into a table in LDS.
+    const int q = threadIdx.x;
+    if (q < rounds) {
+      moe_item it{0, -1, 0, 0, nullptr, nullptr};
+      const int id = (int)blockIdx.x + q * G;
+      if (id < total) resolve(id, it);
+      s_item[q] = it;
+    }
+    __syncthreads();
+    iu8_pf32_run<false, WMW, WNW, TM, TN, false, ST, false, true, GATHER == 2, true>(a, as, c, n, k, [&](int r, iu8_tile &t) {
+      if (r >= rounds) return false;
+      const volatile int *p32 = (const volatile int *)&s_item[r];
+      auto u = [&](int i) { return __builtin_amdgcn_readfirstlane(p32[i]); };
+      if (u(1) < 0) return false;
+      const unsigned long long wp = (unsigned)u(4) | ((unsigned long long)(unsigned)u(5) << 32);
+      const unsigned long long sp = (unsigned)u(6) | ((unsigned long long)(unsigned)u(7) << 32);
+      t = iu8_tile{iu8_rows{GATHER ? row_tok : nullptr, u(0), u(1)}, 0, u(2), (const unsigned char *)wp, (const float *)sp};
+      return true;
+    }, nullptr, nullptr, lds);
+    return;
+  }
+  iu8_pf32_run<false, WMW, WNW, TM, TN, false, ST, false, true, GATHER == 2, true>(a, as, c, n, k, [&](int r, iu8_tile &t) {
+    const int id = (int)blockIdx.x + r * G;
+    if (id >= total) return false;
+    moe_item it;
+    resolve(id, it);
+    t = iu8_tile{iu8_rows{GATHER ? row_tok : nullptr, it.row0, it.rows}, 0, it.nt0, it.W, it.ws};
     return true;
-  });
+  }, nullptr, nullptr, lds);
 }
 // two cells: heavy items on the tile cell, light ones on the small cell between two parts of them
 template <int GATHER, int WMW, int WNW, int TM, int TN, int ST>
