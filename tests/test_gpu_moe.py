@@ -149,6 +149,31 @@ def test_route_and_quant_in_one_launch(ctx, T, H):
     assert e.value.code == iu8.E_RULE
 
 
+def test_grouped_tile_kernels_on_a_tiny_grid(ctx):
+    """The tile kernels are persistent: on 3 workgroups instead of one a CU every workgroup walks more
+    items than its item table holds (the 256-row kernel then resolves items as it goes, the 128-row
+    one runs several passes over its table) and writes the same bytes."""
+    T, E, k, H, I = 300, 128, 8, 512, 256
+    case = synth.moe_case(T=T, E=E, topk=k, H=H, I=I, seed=9, experts=4)
+    for tb, kern in ((16, "moe_iu8_grouped_w4_pf16_g2"), (8, "moe_iu8_grouped_w4_pf_g2")):
+        say(f"grouped gate+up on 3 workgroups: {kern}")
+        layer = run_layer(ctx, case, tile_blocks=tb)
+        want = layer.gu.clone()
+        nt, rows = int(layer.buf["meta"][0].item()), int(layer.buf["meta"][1].item())
+        assert nt * ((2 * I + 255) // 256) > 3 * 64
+        d = iu8.describe_raw(kern, (3, 1, 1), 512, plugin="moe_iu8", n=2 * I, k=H, pmax=0)
+        for name in ("p", "cnt"):
+            d.arg(name).kind = iu8.ARG_NULL_BUFFER
+        layer.gu.fill_(0x7FC0)
+        bufs = dict(a=layer.q1.data_ptr(), xptr=layer.xptr_gu.data_ptr(), c=layer.gu.data_ptr(),
+                    **{n_: layer.buf[n_].data_ptr() for n_ in ("tile_expert", "tile_row0", "tile_rows", "row_tok", "meta")})
+        bufs["as"] = layer.s1.data_ptr()
+        ctx.launch(d, bufs)
+        torch.cuda.synchronize()
+        live = layer.buf["row_tok"][:rows] >= 0
+        assert torch.equal(layer.gu[:rows][live], want[:rows][live])
+
+
 def test_moe_router_ties_and_skew(ctx):
     say("moe router: ties and one hot expert")
     case = synth.moe_case(T=40, E=128, topk=8, H=512, I=256, seed=5, experts=4)
