@@ -221,10 +221,19 @@ def main():
                     got = dev_c[name].cpu().numpy().view(np.uint16)
                     ok = ok and bool(np.array_equal(got, r["C"]))
             n_cpu += 1
+        # ... and on one core (a quarter of the time budget again)
+        t_one, n_one = 0.0, 0
+        while t_one < args.cpu_seconds / 4:
+            for name, n, k in linears:
+                c0 = time.perf_counter()
+                ref.linear(host[name]["X"][:M], host[name]["W"], host[name]["ws"], False, threads=1, pin=1)
+                t_one += time.perf_counter() - c0
+            n_one += 1
         isa = {0: "scalar", 1: "avx2", 2: "avx512-vnni"}[ref.lib().w4a8_isa()]
         out["cpu_baseline"] = dict(value=round(step_bytes * n_cpu / t_cpu / 1e9, 2), unit="GB/s", cores=threads, kind="port",
                                    sample="%d steps (quant + GEMM + epilogue of the same four linears, M=%d), %s body, "
-                                          "threads pinned one per core, 16-column tiles" % (n_cpu, M, isa))
+                                          "threads pinned one per core, 16-column tiles" % (n_cpu, M, isa),
+                                   single_core_gbps=round(step_bytes * n_one / t_one / 1e9, 2), single_core_steps=n_one)
         out["parity_vs_oracle"] = ok
 
     # ---- the other batch sizes of configs[1] (M = 4, 8, 16) through the same step: a linear is one fused
