@@ -42,7 +42,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=120)
-    ap.add_argument("--warmup", type=int, default=12)
+    ap.add_argument("--warmup", type=int, default=600)   # 24 ms of the step: the card's clock settles over tens of ms
     ap.add_argument("--m", type=int, default=1, help="tokens per step (decode band, 1..16)")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
@@ -326,7 +326,7 @@ def main():
             with torch.cuda.stream(stream):
                 for _ in range(3):
                     ctx.launch(qd, qb, sh)
-                for i in range(warm):  # tens of ms of MFMA load: the clock settles where it stays under this kernel
+                for i in range(warm):  # 40-300 ms of this kernel: the card's clock takes tens of ms to settle where it stays under it
                     ctx.launch(d, bs[i % LAYERS], sh)
                 e0, e1, e2 = (torch.cuda.Event(enable_timing=True) for _ in range(3))
                 e0.record(stream)
@@ -349,7 +349,7 @@ def main():
         return pf, tot_ops, tot_us, tot_q_us
 
     if not args.no_prefill:
-        pf, tot_ops, tot_us, tot_q_us = prefill_at(2048, 40, 20)
+        pf, tot_ops, tot_us, tot_q_us = prefill_at(2048, 600, 60)
         tops = tot_ops / tot_us / 1e6
         # what the matrix cores sustain on this card with such operands: the register-resident MFMA
         # loop of the probe object, fed zeros, codes like this workload's (small activations, 16*w
@@ -387,7 +387,7 @@ def main():
         # the other row counts of configs[2]: M = 256 sits near the ridge (both roofs reported: the weights'
         # GB/s beside the TOPS), M = 8192 is the matrix-bound end
         other = {}
-        for PM, warm, reps in (() if args.no_other_m else ((256, 20, 20), (8192, 6, 6))):
+        for PM, warm, reps in (() if args.no_other_m else ((256, 600, 60), (8192, 80, 12))):
             pfm, ops_m, us_m, q_us_m = prefill_at(PM, warm, reps)
             wbytes = sum(n * k // 2 for _, n, k in linears)
             other["m%d" % PM] = dict(tops=round(ops_m / us_m / 1e6, 1), with_quant=round(ops_m / (us_m + q_us_m) / 1e6, 1),
@@ -430,9 +430,10 @@ def main():
             g = torch.cuda.CUDAGraph()
             with torch.cuda.graph(g, stream=stream):
                 run_seq()
-            reps = 6 if SM == 16 else 3
+            reps = 60 if SM == 16 else 12
             with torch.cuda.stream(stream):
-                g.replay()
+                for _ in range(reps // 2):   # sustained: tens of ms of the sequence before the timed replays
+                    g.replay()
                 e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                 e0.record(stream)
                 for _ in range(reps):
