@@ -27,9 +27,11 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0      # MI355X published HBM3E bandwidth
 INT8_PEAK_TOPS = 5000.0     # MI355X published dense int8 MFMA peak
 LAYERS = 6                  # distinct weight copies walked by successive steps (6 x 165 MB)
-# HBM-side bytes of one launch of the dominant kernel, mean over the four layer shapes, from
-# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this very command (profiles/macaq_iu8_decq_w4_tm1__layer_set_m1.txt), each
-# counter scaled by what it reads for the 256 MiB copy probe. Keyed by (kernel, M); None = not measured.
+# HBM-side bytes of one launch of the dominant kernel, mean over the four layer shapes. A counter
+# figure cannot be read inside this process: it comes from two rocprofv3 --pmc runs of this very
+# command (FETCH_SIZE, then WRITE_SIZE), each counter scaled by what it reads for the 256 MiB copy
+# probe, and is kept in the profile summary named below. Keyed by (kernel, M); None = not measured.
+TRAFFIC_SOURCE = "profiles/macaq_iu8_decq_w4_tm1__layer_set_m1.txt"
 TRAFFIC = {("macaq_iu8_decq_w4_tm1", 1): 41893449.0, ("macaq_iu8_dec_w4_tm1", 1): 41992603.0}
 
 
@@ -206,9 +208,60 @@ def main():
     achieved = gemm_bytes / (gemm_us * 1e-6) / 1e9
     roofline = dict(bound="hbm", kernel=kname, achieved=round(achieved, 1), peak=HBM_PEAK_GBPS,
                     unit="GB/s", frac=round(achieved / HBM_PEAK_GBPS, 4), traffic=TRAFFIC.get((kname, M)),
+                    traffic_source="not of this run: FETCH_SIZE + WRITE_SIZE per launch from rocprofv3 --pmc runs of this command, "
+                                   "scaled by the copy probe, " + TRAFFIC_SOURCE,
                     avg_launch_us=round(gemm_us, 3), bytes_per_launch=gemm_bytes,
-                    note="mean over the four layer shapes, cold weights (rotating %d copies), graph replay; traffic = "
-                         "FETCH_SIZE + WRITE_SIZE per launch (rocprofv3 --pmc, scaled by the copy probe), see profiles/" % LAYERS)
+                    note="mean over the four layer shapes, cold weights (rotating %d copies), graph replay" % LAYERS)
+
+    # ---- the measured HBM ceiling beside the nominal one: the streaming-read probe over 1 GiB (four times the
+    # 256 MB Infinity Cache, so every launch reads from memory), best of three grids, HIP events on its stream
+    def probe_read_us(ptr, nbytes, grid, reps):
+        pd = iu8.describe_raw("iu8_probe_read", (grid, 1, 1), 256, n=nbytes // 16)
+        pb = dict(src=ptr, out=probe_out.data_ptr())
+        with torch.cuda.stream(stream):
+            ctx.launch(pd, pb, sh)
+            p0, p1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            p0.record(stream)
+            for _ in range(reps):
+                ctx.launch(pd, pb, sh)
+            p1.record(stream)
+        torch.cuda.synchronize()
+        return p0.elapsed_time(p1) * 1e3 / reps
+
+    probe_out = torch.zeros(16, dtype=torch.int32, device=dev)
+    big = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+    big.random_(0, 255)
+    hbm_probe = max((1 << 30) / probe_read_us(big.data_ptr(), 1 << 30, g, 8) / 1e3 for g in (1024, 2048, 4096))
+    del big
+    roofline["hbm_probe_gbps"] = round(hbm_probe, 1)
+    roofline["frac_of_probe"] = round(achieved / hbm_probe, 4)
+
+    # ---- every linear of the step by itself: the fused launch alone (graph of K launches walking the weight
+    # copies), and the read probe on the same weight bytes, cold the same way. down = the 5120 x 17408 GEMV.
+    per_linear = {}
+    for name, n, k in linears:
+        gl = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gl, stream=stream):
+            for i in range(K_steps):
+                if fused:
+                    launch_fused(name, i % LAYERS)
+                else:
+                    launch_gemm(name, i % LAYERS)
+        with torch.cuda.stream(stream):
+            gl.replay()
+            l0, l1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            l0.record(stream)
+            gl.replay()
+            l1.record(stream)
+        torch.cuda.synchronize()
+        us = l0.elapsed_time(l1) * 1e3 / K_steps
+        nb = alg_bytes(M, n, k) if fused else alg_bytes(M, n, k) - M * k + 4 * M
+        wbytes = n * k // 2
+        pus = min(sum(probe_read_us(dev_w[name][layer].data_ptr(), wbytes, g, 1) for layer in range(LAYERS)) / LAYERS for g in (512, 1024, 2048))
+        per_linear[name] = dict(n=n, k=k, kernel=(fdescs if fused else descs)[name].kernel.decode(), us=round(us, 2), bytes=nb,
+                                gbps=round(nb / us / 1e3, 1), hbm_frac=round(nb / us / 1e3 / HBM_PEAK_GBPS, 4),
+                                frac_of_probe=round(nb / us / 1e3 / hbm_probe, 4), read_probe_us=round(pus, 2))
+        del gl
 
     # ---- parity spot check against the CPU oracle, and the CPU baseline beside it
     out = dict(metric="W4A8 GEMM GB/s (%HBM) at M=1; int8 TOPS (%MFMA peak) at M=2048", value=round(value, 1), unit="GB/s",
@@ -219,8 +272,11 @@ def main():
                            launches_per_step=(1 if fused else 2) * len(linears), fused_quant=fused,
                            hbm_frac=round(value / HBM_PEAK_GBPS, 4),
                            two_launch_gbps=round(step_bytes / (two_ms * 1e-3) / 1e9, 1),
-                           warm_cache_gbps=round(step_bytes / (warm_ms * 1e-3) / 1e9, 1)),
+                           warm_cache_gbps=round(step_bytes / (warm_ms * 1e-3) / 1e9, 1),
+                           hbm_frac_of_probe=round(value / hbm_probe, 4)),
                roofline=roofline)
+    out["decode_m%d" % M] = dict(per_linear=per_linear, note="one launch a linear, cold weights, graph replay; read_probe_us = a plain "
+                                 "streaming read of the same weight bytes, cold the same way; down is the 5120x17408 GEMV")
 
     if not args.no_cpu:
         from oracle import ref
@@ -246,10 +302,19 @@ def main():
                 t_one += time.perf_counter() - c0
             n_one += 1
         isa = {0: "scalar", 1: "avx2", 2: "avx512-vnni"}[ref.lib().w4a8_isa()]
+        try:    # the host's last-level cache against the step's 165 MB of weights, read again every step
+            txt = open("/sys/devices/system/cpu/cpu0/cache/index3/size").read().strip()
+            llc = int(txt[:-1]) * {"K": 1 << 10, "M": 1 << 20, "G": 1 << 30}[txt[-1]]
+        except Exception:
+            llc = None
+        wbytes_step = sum(n * k // 2 for _, n, k in linears)
         out["cpu_baseline"] = dict(value=round(step_bytes * n_cpu / t_cpu / 1e9, 2), unit="GB/s", cores=threads, kind="port",
                                    sample="%d steps (quant + GEMM + epilogue of the same four linears, M=%d), %s body, "
                                           "threads pinned one per core, 16-column tiles" % (n_cpu, M, isa),
-                                   single_core_gbps=round(step_bytes * n_one / t_one / 1e9, 2), single_core_steps=n_one)
+                                   single_core_gbps=round(step_bytes * n_one / t_one / 1e9, 2), single_core_steps=n_one,
+                                   weight_bytes_per_step=wbytes_step, llc_bytes=llc,
+                                   weights="unknown" if llc is None else ("DRAM-cold: the step's weights exceed the LLC and every step "
+                                           "re-reads all of them" if wbytes_step > llc else "LLC-warm: the step's weights fit the LLC"))
         out["parity_vs_oracle"] = ok
 
     # ---- the other batch sizes of configs[1] (M = 4, 8, 16) through the same step: a linear is one fused

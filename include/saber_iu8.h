@@ -124,6 +124,25 @@ int saber_iu8_resolve(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_d
 /* The same descriptor for an explicitly named kernel of the object and split count (the
  * autotuner's and the parity tests' entry: every variant of one regime gives the same bytes). */
 int saber_iu8_describe(const char *kernel, uint32_t m, uint32_t n, uint32_t k, uint32_t ks, saber_iu8_desc *out);
+/* A name of the reference's symbol set that these objects do not carry (its gfx1201 tile shapes:
+ * macaq_iu8f_dec_*_tm{5..8}, macaq_iu8f_pf_*_bm{128,64}, macaq_iu8f_pf_*_t..., macaq_iu8.rs:520-546)
+ * is taken by saber_iu8_describe as a request for the op at that shape and answered with the cell
+ * the gfx950 law picks; the all-reduce forms (macaq_iu8f_arnq_*) are refused by name.
+ *
+ * LAUNCH LAW. The ten names of the reference's `macaq_iu8` object and the pair names are kept, with
+ * their kernarg bytes, but NOT the reference's grid/block law or operand byte order: the gfx950
+ * kernels are 256-, 512- or 1024-thread workgroups, mostly persistent, over the layouts 33/34/35.
+ * A host must take grid and block from saber_iu8_resolve / _describe or from the band table
+ * (saber_iu8_band_toml, committed as prebuilt/gfx950/macaq_iu8.band.toml); saber_iu8_launch refuses
+ * a descriptor whose block is not the kernel's max_flat_workgroup_size. */
+
+/* The launch law as data (TOML text, NUL-terminated): the cells' geometry, the (op, n, k, rows) ->
+ * kernel bands over the 27B-class linears for M = 1..8192, the reference's symbol set and what
+ * answers each name, the routed layer's tile thresholds, the pair's block order. The gfx950
+ * counterpart of the reference's band tables (macaq_iu8.rs:150-212) for a host that cannot link
+ * this library. *need (optional) receives the bytes required; buf may be NULL to ask for it. */
+int saber_iu8_band_toml(char *buf, size_t cap, size_t *need);
+
 /* The activation producer's descriptor (i8_twin's role, macaq_iu8.rs:881-916): bf16 [m,k] rows
  * -> int8 A edge + f32 scales. */
 int saber_iu8_resolve_quant(uint32_t m, uint32_t k, saber_iu8_desc *out);
@@ -190,6 +209,11 @@ typedef struct {
  * pass with hipModuleLoadData on `device`. A refused plugin is skipped and counted, as in the
  * reference; no plugin at all is SABER_IU8_E_NOTLOADED. */
 int saber_iu8_open(const char *prebuilt_dir, int device, saber_iu8_ctx **out);
+/* PluginSet's single-manifest path (crates/saber-exec/src/loader.rs:249-290): validates one
+ * `<plugin>.manifest.toml` + code object outside the plugin directory and adds its kernels to the
+ * context; a refusal moves the counter it names. The parity suite adds its test-only object
+ * (`taps/iu8_taps.manifest.toml`: accumulator and table taps) this way. */
+int saber_iu8_load_plugin(saber_iu8_ctx *ctx, const char *manifest_path);
 void saber_iu8_close(saber_iu8_ctx *ctx);
 int saber_iu8_get_counters(const saber_iu8_ctx *ctx, saber_iu8_counters *out);
 /* 1 if `kernel` was loaded. */
@@ -250,6 +274,11 @@ int saber_iu8_attn_gate_quant_had(saber_iu8_ctx *ctx, const void *core_bf16, con
  * it alone; the grids go end to end, the second half's buffers and workspaces take the suffix `_b`.
  * Refused (SABER_IU8_E_RULE) unless both halves are W4 decode cells of one kernel, M and K. */
 int saber_iu8_pair(const saber_iu8_desc *first, const saber_iu8_desc *second, saber_iu8_desc *out);
+/* The same with the block order named instead of taken from the law (PAIR_BA_FIRST,
+ * macaq_iu8.rs:549-553): second_first = 1 lays the second problem's workgroups first
+ * (macaq_iu8f_pairb_w4_tm*), 0 problem 0's (macaq_iu8f_pair_w4_tm*). Same bytes either way. */
+int saber_iu8_pair_ordered(const saber_iu8_desc *first, const saber_iu8_desc *second, int second_first,
+                           saber_iu8_desc *out);
 /* resolve x 2 + pair + launch for the unsplit decode law: c [m,n] and c_b [m,n_b] from one a / a_scale. */
 int saber_iu8_gemm_pair(saber_iu8_ctx *ctx, const void *a, const float *a_scale, const void *w, const float *w_scale, void *c,
                         uint32_t n, const void *w_b, const float *w_scale_b, void *c_b, uint32_t n_b, uint32_t m, uint32_t k,
@@ -267,7 +296,9 @@ int saber_iu8_resolve_fused(int wkind, uint32_t m, uint32_t n, uint32_t k, saber
 int saber_iu8_linear_fused(saber_iu8_ctx *ctx, int wkind, const void *x_bf16, const void *w, const float *ws,
                            void *c_bf16, void *q, float *scale, uint32_t m, uint32_t n, uint32_t k, void *stream);
 
-/* Workspace bytes the resolved GEMM needs (both 0 when it does not split). */
+/* Workspace bytes the resolved GEMM needs (both 0 when it does not split). Ask before every
+ * saber_iu8_gemm of a new shape: the law splits K in one band (K >= 16384, 49..128 rows, few tiles),
+ * and such a launch with `partial` / `counter` NULL is refused (SABER_IU8_E_ARG). */
 int saber_iu8_gemm_workspace(int wkind, uint32_t m, uint32_t n, uint32_t k, uint64_t *partial_bytes,
                              uint64_t *counter_bytes);
 
@@ -279,7 +310,9 @@ int saber_iu8_gemm(saber_iu8_ctx *ctx, int wkind, const void *a, const float *as
 
 /* The raw int32 accumulators of the same GEMM (16 * sum(a*w) for W4, sum(a*w) for W8), int32
  * [m,n]: the parity tap. No counterpart in the reference's shipped object (its tests replay
- * captured bytes, crates/saber-kernels/hip/harness/run_hsaco.cpp:1-15). */
+ * captured bytes, crates/saber-kernels/hip/harness/run_hsaco.cpp:1-15). The tap kernels are not in
+ * the plugin directory: SABER_IU8_E_NOTLOADED until the test-only object `iu8_taps` was added with
+ * saber_iu8_load_plugin. */
 int saber_iu8_gemm_acc(saber_iu8_ctx *ctx, int wkind, const void *a, const void *w, int32_t *acc, uint32_t m,
                        uint32_t n, uint32_t k, void *stream);
 

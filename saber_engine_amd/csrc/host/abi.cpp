@@ -67,8 +67,6 @@ static const Signature SIG_MOE_COMBINE = {{"y", K::Buffer},    {"topk_w", K::Buf
 
 static const Signature SIG_PROBE_READ = {{"src", K::Buffer}, {"out", K::Buffer}, {"n", K::I32}};
 static const Signature SIG_PROBE_COPY = {{"src", K::Buffer}, {"dst", K::Buffer}, {"n", K::I32}};
-static const Signature SIG_PROBE_EMPTY = {{"out", K::Buffer}};
-static const Signature SIG_PROBE_MFMA = {{"out", K::Buffer}, {"n", K::I32}};
 
 static bool starts(const std::string &s, const char *p) { return s.rfind(p, 0) == 0; }
 
@@ -76,7 +74,7 @@ const Signature *signature_for(const std::string &k) {
   if (starts(k, "macaq_iu8_dec_")) return &SIG_DEC;
   if (starts(k, "macaq_iu8_decq_")) return &SIG_DECQ;
   if (starts(k, "macaq_iu8_pf_")) return k.size() > 3 && k.compare(k.size() - 3, 3, "_ks") == 0 ? &SIG_DEC : &SIG_PF;
-  if (starts(k, "macaq_iu8f_pair_")) return &SIG_PAIR;
+  if (starts(k, "macaq_iu8f_pair_") || starts(k, "macaq_iu8f_pairb_")) return &SIG_PAIR;
   if (starts(k, "add_rms_quant_hadi8_")) return &SIG_HAD_ARQ;
   if (starts(k, "silu_mul_quant_hadi8_")) return &SIG_HAD_SMQ;
   if (starts(k, "quant_hadi8_")) return &SIG_HAD_Q;
@@ -88,10 +86,8 @@ const Signature *signature_for(const std::string &k) {
   if (starts(k, "macaq_i8_silu_mul_quant_lut_")) return &SIG_SILU_LUT;
   if (starts(k, "macaq_i8_silu_mul_quant_")) return &SIG_SILU;
   if (k == "macaq_silu_bf16_table") return &SIG_TABLE;
-  if (k == "iu8_probe_read" || k == "iu8_probe_mfma32d" || k == "iu8_probe_first") return &SIG_PROBE_READ;
+  if (k == "iu8_probe_read" || k == "iu8_probe_mfma32d") return &SIG_PROBE_READ;
   if (k == "iu8_probe_copy") return &SIG_PROBE_COPY;
-  if (k == "iu8_probe_empty") return &SIG_PROBE_EMPTY;
-  if (k == "iu8_probe_mfma" || k == "iu8_probe_mfma32") return &SIG_PROBE_MFMA;
   if (starts(k, "moe_iu8_route_")) return &SIG_MOE_ROUTE;
   if (starts(k, "moe_iu8_routeq_")) return &SIG_MOE_ROUTEQ;
   if (starts(k, "moe_iu8_grouped_")) return &SIG_MOE_GROUPED;

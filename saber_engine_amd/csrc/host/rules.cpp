@@ -10,30 +10,17 @@ namespace iu8 {
 
 static const DecVariant DEC_VARIANTS[] = {
 #define IU8_DEC_VARIANT(name, TM, W8, NT, KW, WPB, D, ALDS, ACC) {#name, TM, W8, NT, KW, WPB, D, ALDS, ACC},
-#define IU8_PF_VARIANT(name, W8, WMW, WNW, TM, TN, ACC, ST, OCC, DEEP)
-#define IU8_PAIR_VARIANT(name, TM, NT, KW, WPB, D, ALDS)
+#define IU8_DEC_TAP(name, TM, W8, NT, KW, WPB, D, ALDS, ACC) {#name, TM, W8, NT, KW, WPB, D, ALDS, ACC},
 #include "../kernels/iu8_variants.def"
-#undef IU8_DEC_VARIANT
-#undef IU8_PF_VARIANT
-#undef IU8_PAIR_VARIANT
 };
 static const PfVariant PF_VARIANTS[] = {
-#define IU8_DEC_VARIANT(name, TM, W8, NT, KW, WPB, D, ALDS, ACC)
 #define IU8_PF_VARIANT(name, W8, WMW, WNW, TM, TN, ACC, ST, OCC, DEEP) {#name, W8, WMW, WNW, TM, TN, ACC, OCC},
-#define IU8_PAIR_VARIANT(name, TM, NT, KW, WPB, D, ALDS)
+#define IU8_PF_TAP(name, W8, WMW, WNW, TM, TN, ACC, ST, OCC, DEEP) {#name, W8, WMW, WNW, TM, TN, ACC, OCC},
 #include "../kernels/iu8_variants.def"
-#undef IU8_DEC_VARIANT
-#undef IU8_PF_VARIANT
-#undef IU8_PAIR_VARIANT
 };
 static const DecVariant PAIR_VARIANTS[] = {
-#define IU8_DEC_VARIANT(name, TM, W8, NT, KW, WPB, D, ALDS, ACC)
-#define IU8_PF_VARIANT(name, W8, WMW, WNW, TM, TN, ACC, ST, OCC, DEEP)
-#define IU8_PAIR_VARIANT(name, TM, NT, KW, WPB, D, ALDS) {#name, TM, false, NT, KW, WPB, D, ALDS, false},
+#define IU8_PAIR_VARIANT(name, TM, NT, KW, WPB, D, ALDS, BFIRST) {#name, TM, false, NT, KW, WPB, D, ALDS, false},
 #include "../kernels/iu8_variants.def"
-#undef IU8_DEC_VARIANT
-#undef IU8_PF_VARIANT
-#undef IU8_PAIR_VARIANT
 };
 
 const DecVariant *dec_variant(const std::string &name) {
@@ -152,6 +139,11 @@ static int describe_dec(const DecVariant &v, uint32_t m, uint32_t n, uint32_t k,
 static int describe_pf(const PfVariant &v, uint32_t m, uint32_t n, uint32_t k, uint32_t ks, saber_iu8_desc *d) {
   const char *op = v.w8 ? "gemm_i8a8" : "gemm_i4a8";
   if (int rc = check_shape(op, m, n, k)) return rc;
+  // the tile GEMM addresses its operands with 32-bit byte offsets from a per-step base
+  const uint64_t a_bytes = (uint64_t)((m + 15) / 16 * 16) * k, w_bytes = (uint64_t)n * k / (v.w8 ? 1 : 2);
+  if (a_bytes > 0xFFFFFFFFull || w_bytes > 0xFFFFFFFFull)
+    return fail(SABER_IU8_E_RULE, fmt("%s: %u x %u x %u puts an operand past 4 GiB (A %llu B, W %llu B), more than the tile GEMM addresses",
+                                      op, m, n, k, (unsigned long long)a_bytes, (unsigned long long)w_bytes));
   const std::string name = std::string(v.name) + (ks ? "_ks" : "");
   if (ks) {
     const uint32_t steps = k / 128, spb = (steps + ks - 1) / ks;
@@ -194,6 +186,16 @@ int describe(const std::string &kernel, uint32_t m, uint32_t n, uint32_t k, uint
       if (!signature_for(kernel)) return fail(SABER_IU8_E_RULE, kernel + ": no such split form");
       return describe_pf(*v, m, n, k, ks, out);
     }
+  // a name of the reference's symbol set that this object does not carry (gfx1201 tile shapes): the
+  // request is for the op at this shape, and the gfx950 law picks the cell
+  int w8 = 0;
+  const char *note = "";
+  const int r = ref_symbol_by_law(kernel, &w8, &note);
+  if (r > 0) {
+    if (ks != 1) return fail(SABER_IU8_E_RULE, kernel + ": answered by the launch law, which picks the split itself");
+    return resolve(w8 ? SABER_IU8_W8 : SABER_IU8_W4, m, n, k, out);
+  }
+  if (r < 0) return fail(SABER_IU8_E_RULE, kernel + ": " + note);
   return fail(SABER_IU8_E_RULE, kernel + ": not a kernel of the macaq_iu8 object");
 }
 
@@ -210,7 +212,7 @@ static bool int_arg(const saber_iu8_desc &d, const char *name, int64_t *v) {
 // split count, its partial slab and counters), the two grids end to end, problem 0 first
 // (macaq_iu8.rs:632-704). Refused unless both halves are W4 decode cells of one kernel (so one row
 // tiling and one staging form), M and K.
-int pair(const saber_iu8_desc &first, const saber_iu8_desc &second, saber_iu8_desc *out) {
+int pair(const saber_iu8_desc &first, const saber_iu8_desc &second, saber_iu8_desc *out, int order) {
   static const char PREFIX[] = "macaq_iu8_dec_w4_";
   const std::string k0 = first.kernel, k1 = second.kernel;
   const DecVariant *v0 = dec_variant(k0), *v1 = dec_variant(k1);
@@ -220,7 +222,13 @@ int pair(const saber_iu8_desc &first, const saber_iu8_desc &second, saber_iu8_de
   if (!v0 || !v1 || !ints || v0->w8 || v1->w8 || v0->acc || v1->acc || k0 != k1 || m0 != m1 || kk0 != kk1)
     return fail(SABER_IU8_E_RULE, fmt("macaq iu8 pair: halves `%s` M %lld K %lld and `%s` M %lld K %lld are not two W4 cells of one M, K",
                                       k0.c_str(), (long long)m0, (long long)kk0, k1.c_str(), (long long)m1, (long long)kk1));
-  const std::string name = "macaq_iu8f_pair_w4_" + k0.substr(sizeof PREFIX - 1);
+  // The block order by tm (speed data; both orders give the same bytes): the second problem's
+  // workgroups first (`pairb`), as the reference's PAIR_BA_FIRST has it at every tm
+  // (macaq_iu8.rs:549-553) -- the small half then does not sit in the launch's tail.
+  static const bool PAIR_B_FIRST[4] = {true, true, true, true};
+  const bool b_first = order < 0 ? PAIR_B_FIRST[std::min(std::max(v0->tm, 1), 4) - 1] : order > 0;
+  const char *form = b_first ? "pairb" : "pair";
+  const std::string name = std::string("macaq_iu8f_") + form + "_w4_" + k0.substr(sizeof PREFIX - 1);
   const DecVariant *pv = pair_variant(name);
   if (!pv) return fail(SABER_IU8_E_RULE, name + ": the fused object carries no such pair");
   const uint32_t nb0 = first.grid[0], nb1 = second.grid[0], ks0 = first.ks, ks1 = second.ks;
@@ -289,7 +297,8 @@ int resolve(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *out) 
 // the partials cost ks*M*N*4 bytes each way and the last arriver sums alone -- so the rule is this
 // narrow. The launch then needs the `decode_partial` / `decode_counter` workspaces the descriptor lists.
 uint32_t pf_split(bool w8, uint32_t m, uint32_t n, uint32_t k, const PfVariant **cell) {
-  if (w8 || k < 16384) return 0;
+  // measured at 49..128 rows only; above, the partials (ks * M * N * 4 bytes each way) grow with M
+  if (w8 || k < 16384 || m > 128) return 0;
   const PfVariant *v = pf_variant("macaq_iu8_pf_w4_t64x128_s");
   if (!v || !signature_for(std::string(v->name) + "_ks")) return 0;
   const uint64_t tiles = (uint64_t)((n + v->block_n() - 1) / v->block_n()) * ((m + v->block_m() - 1) / v->block_m());

@@ -39,7 +39,8 @@ uint32_t decode_split(uint32_t m, uint32_t n, uint32_t k, uint32_t nblk, uint32_
 int resolve(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *out);
 int describe(const std::string &kernel, uint32_t m, uint32_t n, uint32_t k, uint32_t ks, saber_iu8_desc *out);
 // Two W4 decode descriptors of one M, K and kernel -> the one-dispatch pair (macaq_iu8.rs:632-704).
-int pair(const saber_iu8_desc &first, const saber_iu8_desc &second, saber_iu8_desc *out);
+// order: -1 the law's block order, 0 problem 0 first (`pair`), 1 the second problem first (`pairb`).
+int pair(const saber_iu8_desc &first, const saber_iu8_desc &second, saber_iu8_desc *out, int order = -1);
 const DecVariant *pair_variant(const std::string &name);
 int resolve_quant(uint32_t m, uint32_t k, saber_iu8_desc *out);
 // The fused quant + GEMV of a decode linear; refuses (by name) shapes it does not hold.
@@ -50,6 +51,10 @@ int resolve_silu_mul_quant(uint32_t rows, uint32_t n, saber_iu8_desc *out);
 int resolve_quant_rowmajor(uint32_t m, uint32_t k, saber_iu8_desc *out);
 // Quantisation through a row map (output row r = input row row_tok[r]).
 int resolve_quant_rows(uint32_t rows, uint32_t k, saber_iu8_desc *out);
+
+// The reference's symbol names this object answers through its launch law (band.cpp).
+int ref_symbol_by_law(const std::string &kernel, int *w8, const char **note);
+std::string band_toml();
 
 // Fills name/offset/size of every slot from the kernel's signature; kinds default to BUFFER.
 int fill_slots(const std::string &kernel, saber_iu8_desc *d);

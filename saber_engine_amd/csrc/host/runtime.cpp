@@ -18,10 +18,15 @@
 
 using namespace iu8;
 
+struct LoadedKernel {
+  hipFunction_t fn;
+  uint32_t max_threads;  // the code object's max_flat_workgroup_size: the block its indexing is written for
+};
 struct saber_iu8_ctx {
   int device = 0;
+  std::string arch;
   std::vector<hipModule_t> modules;
-  std::map<std::string, hipFunction_t> fn;
+  std::map<std::string, LoadedKernel> fn;
   saber_iu8_counters counters{};
 };
 
@@ -67,6 +72,34 @@ static const void *find_binding(const saber_iu8_binding *bufs, uint32_t n, const
   return nullptr;
 }
 
+// Validates one manifest + code object and adds its kernels to the context. A refusal moves the
+// counter it names and leaves the context as it was (the plugin is skipped, loader.rs:249-270); a HIP
+// failure is returned as such.
+static int load_one(saber_iu8_ctx *ctx, const std::string &manifest_path) {
+  Manifest m;
+  std::vector<uint8_t> blob;
+  int refusal = 0;
+  const int rc = load_and_validate(manifest_path, ctx->arch, m, blob, &refusal);
+  if (rc != 0) {
+    if (refusal == SABER_IU8_REFUSED_KERNARG) ctx->counters.refused_kernarg++;
+    else if (refusal == SABER_IU8_REFUSED_WAVE) ctx->counters.refused_wave++;
+    else ctx->counters.refused_metadata++;
+    return rc;
+  }
+  hipModule_t mod;
+  hipError_t e;
+  if ((e = hipModuleLoadData(&mod, blob.data())) != hipSuccess) return hip_fail(("hipModuleLoadData " + m.hsaco).c_str(), e);
+  ctx->modules.push_back(mod);
+  ctx->counters.plugins_loaded++;
+  for (const KernelDecl &k : m.kernel) {
+    hipFunction_t fn;
+    if ((e = hipModuleGetFunction(&fn, mod, k.name.c_str())) != hipSuccess) return hip_fail(("hipModuleGetFunction " + k.name).c_str(), e);
+    ctx->fn[k.name] = LoadedKernel{fn, k.max_flat_workgroup_size};
+    ctx->counters.kernels_loaded++;
+  }
+  return 0;
+}
+
 extern "C" {
 
 const char *saber_iu8_last_error(void) { return last_error(); }
@@ -87,6 +120,10 @@ int saber_iu8_resolve_quant(uint32_t m, uint32_t k, saber_iu8_desc *out) {
 int saber_iu8_pair(const saber_iu8_desc *first, const saber_iu8_desc *second, saber_iu8_desc *out) {
   if (!first || !second || !out) return fail(SABER_IU8_E_ARG, "pair: null descriptor");
   return pair(*first, *second, out);
+}
+int saber_iu8_pair_ordered(const saber_iu8_desc *first, const saber_iu8_desc *second, int second_first, saber_iu8_desc *out) {
+  if (!first || !second || !out) return fail(SABER_IU8_E_ARG, "pair: null descriptor");
+  return pair(*first, *second, out, second_first ? 1 : 0);
 }
 int saber_iu8_fused_holds(uint32_t m, uint32_t k) { return fused_holds(m, k) ? 1 : 0; }
 int saber_iu8_resolve_fused(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *out) {
@@ -245,35 +282,15 @@ int saber_iu8_open(const char *prebuilt_dir, int device, saber_iu8_ctx **out) {
   std::sort(manifests.begin(), manifests.end());
   saber_iu8_ctx *ctx = new saber_iu8_ctx();
   ctx->device = device;
+  ctx->arch = arch;
   std::string first_refusal;
   for (const std::string &f : manifests) {
-    Manifest m;
-    std::vector<uint8_t> blob;
-    int refusal = 0;
-    const int rc = load_and_validate(std::string(prebuilt_dir) + "/" + f, arch, m, blob, &refusal);
-    if (rc != 0) {
-      if (refusal == SABER_IU8_REFUSED_KERNARG) ctx->counters.refused_kernarg++;
-      else if (refusal == SABER_IU8_REFUSED_WAVE) ctx->counters.refused_wave++;
-      else ctx->counters.refused_metadata++;
-      if (first_refusal.empty()) first_refusal = f + ": " + last_error();
-      continue;
-    }
-    hipModule_t mod;
-    if ((e = hipModuleLoadData(&mod, blob.data())) != hipSuccess) {
+    const int rc = load_one(ctx, std::string(prebuilt_dir) + "/" + f);
+    if (rc == SABER_IU8_E_HIP) {
       saber_iu8_close(ctx);
-      return hip_fail(("hipModuleLoadData " + m.hsaco).c_str(), e);
+      return rc;
     }
-    ctx->modules.push_back(mod);
-    ctx->counters.plugins_loaded++;
-    for (const KernelDecl &k : m.kernel) {
-      hipFunction_t fn;
-      if ((e = hipModuleGetFunction(&fn, mod, k.name.c_str())) != hipSuccess) {
-        saber_iu8_close(ctx);
-        return hip_fail(("hipModuleGetFunction " + k.name).c_str(), e);
-      }
-      ctx->fn[k.name] = fn;
-      ctx->counters.kernels_loaded++;
-    }
+    if (rc != 0 && first_refusal.empty()) first_refusal = f + ": " + last_error();
   }
   if (ctx->modules.empty()) {
     const std::string msg = std::string(prebuilt_dir) + ": no plugin loaded for " + arch +
@@ -283,6 +300,13 @@ int saber_iu8_open(const char *prebuilt_dir, int device, saber_iu8_ctx **out) {
   }
   *out = ctx;
   return 0;
+}
+
+int saber_iu8_load_plugin(saber_iu8_ctx *ctx, const char *manifest_path) {
+  if (!ctx || !manifest_path) return fail(SABER_IU8_E_ARG, "load_plugin: null argument");
+  hipError_t e;
+  if ((e = hipSetDevice(ctx->device)) != hipSuccess) return hip_fail("hipSetDevice", e);
+  return load_one(ctx, manifest_path);
 }
 
 void saber_iu8_close(saber_iu8_ctx *ctx) {
@@ -328,13 +352,20 @@ int saber_iu8_launch(saber_iu8_ctx *ctx, const saber_iu8_desc *d, const saber_iu
   if (it == ctx->fn.end()) return fail(SABER_IU8_E_NOTLOADED, std::string(d->kernel) + ": not in the loaded plugin set");
   if (d->shared_bytes != 0) return fail(SABER_IU8_E_RULE, std::string(d->kernel) + ": dynamic LDS is not part of this ABI");
   if (!d->grid[0] || !d->grid[1] || !d->grid[2] || !d->block[0]) return fail(SABER_IU8_E_RULE, std::string(d->kernel) + ": empty grid");
+  // Every kernel of these objects indexes by the workgroup size it was compiled for (its
+  // max_flat_workgroup_size): a descriptor from another launch law -- the reference's 256-thread
+  // blocks under its own names -- would run and give wrong bytes, so it is refused here by name.
+  const uint64_t threads = (uint64_t)d->block[0] * std::max(d->block[1], 1u) * std::max(d->block[2], 1u);
+  if (threads != it->second.max_threads)
+    return fail(SABER_IU8_E_RULE, fmt("%s: a block of %llu threads; the gfx950 kernel is written for %u (use this object's launch law)",
+                                      d->kernel, (unsigned long long)threads, it->second.max_threads));
   if (int rc = launch_guard(d)) return rc;
   alignas(16) uint8_t image[256];
   uint32_t bytes = 0;
   if (int rc = saber_iu8_pack_kernarg(d, bufs, n_bufs, image, sizeof image, &bytes)) return rc;
   size_t sz = bytes;
   void *extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, image, HIP_LAUNCH_PARAM_BUFFER_SIZE, &sz, HIP_LAUNCH_PARAM_END};
-  const hipError_t e = hipModuleLaunchKernel(it->second, d->grid[0], d->grid[1], d->grid[2], d->block[0], d->block[1],
+  const hipError_t e = hipModuleLaunchKernel(it->second.fn, d->grid[0], d->grid[1], d->grid[2], d->block[0], d->block[1],
                                              d->block[2], 0, (hipStream_t)stream, nullptr, extra);
   if (e != hipSuccess) return hip_fail(d->kernel, e);
   ctx->counters.launches++;
@@ -414,6 +445,8 @@ int saber_iu8_gemm_acc(saber_iu8_ctx *ctx, int wkind, const void *a, const void 
   saber_iu8_desc d;
   const std::string name = m <= 16 ? fmt("macaq_iu8_dec_%s_tm1_acc", tag) : fmt("macaq_iu8_pf_%s_acc", tag);
   if (int rc = describe(name, m, n, k, 1, &d)) return rc;
+  if (ctx && !ctx->fn.count(name))
+    return fail(SABER_IU8_E_NOTLOADED, name + ": the accumulator taps live in the test-only object `iu8_taps`; add it with saber_iu8_load_plugin");
   // the taps read no scales; bind the accumulator buffer where a pointer is required
   return launch_gemm(ctx, d, a, (const float *)acc, w, (const float *)acc, acc, nullptr, nullptr, stream);
 }
@@ -603,6 +636,13 @@ int saber_iu8_moe_grouped(saber_iu8_ctx *ctx, const void *a, const float *as, co
   if (tile_blocks != 1 && tile_blocks != 8 && tile_blocks != 16)
     return fail(SABER_IU8_E_RULE, fmt("moe_grouped: tile_blocks %u; the cells are 1 (16-row), 8 (128-row) and 16 (256-row)", tile_blocks));
   const bool dec = tile_blocks == 1;
+  // the MFMA cells address A with 32-bit byte offsets: token-major codes (gather 1, 2) or rows_cap rows
+  if (!dec) {
+    const uint64_t a_rows = gather ? (uint64_t)(tokens + 15) / 16 * 16 : saber_iu8_moe_rows_cap(tokens, topk, experts);
+    if (a_rows * k > 0xFFFFFFFFull || (uint64_t)n * k / 2 > 0xFFFFFFFFull)
+      return fail(SABER_IU8_E_RULE, fmt("moe_grouped: %llu rows of K=%u (or an expert's %u x %u weights) pass 4 GiB, more than the tile GEMM addresses",
+                                        (unsigned long long)a_rows, k, n, k));
+  }
   if (gather < 0 || gather > 2 || (gather == 2 && dec))
     return fail(SABER_IU8_E_RULE, fmt("moe_grouped: gather %d; 0 in place, 1 from A fragments, 2 from row-major codes (MFMA cells only)", gather));
   // The streaming cell. Short K (an expert's down projection) takes the two-k-wave form with 64 columns a

@@ -6,17 +6,12 @@
 //   attn_gate_quant_hadi8_t256_tiled1   v = bf16(core * bf16(sigmoid(gate))), the o_proj's A producer.
 //       core bf16 [rows, n]; gate is the projection's [q | gate] block, row stride `gs`, head stride
 //       2*hd, the gate half at +hd (crates/saber-kernels/src/abi.rs:2683-2694); n <= 6144.
-//   attn_glue_hadi8_sigmoid_bf16_table  a checker's tap: bf16(sigmoid) of all 65,536 bf16 inputs
 //
 // Then u = v * t, x = H32 u per 32-block, x * (1/sqrt(32)), and the per-token int8 law on x; codes
 // in the gfx950 A fragment order. sigmoid = 1 / (1 + expf(-g)) is rounded to bf16 before use, so the
-// device's expf shows only through a bf16 -> bf16 function, which the tap kernel tables.
+// device's expf shows only through a bf16 -> bf16 function (glue_sigmoid_bf16, iu8_had.h), which a
+// tap kernel of the test-only object `iu8_taps` tables.
 #include "iu8_had.h"
-
-static __device__ __forceinline__ float glue_sigmoid_bf16(float g) {
-#pragma clang fp contract(off)
-  return iu8_bf16_f32((unsigned short)iu8_bf16_bits(1.f / (1.f + expf(-g))));
-}
 
 extern "C" __global__ __launch_bounds__(256) void attn_gate_quant_hadi8_t256_tiled1(
     const unsigned short *__restrict__ core, const unsigned short *__restrict__ gate, unsigned char *__restrict__ q,
@@ -40,9 +35,4 @@ extern "C" __global__ __launch_bounds__(256) void attn_gate_quant_hadi8_t256_til
     had32(sv[i], had_t + 8 * g, tid);
   }
   had_tail<T>(sv, NV, q, scale, row, n);
-}
-
-extern "C" __global__ __launch_bounds__(256) void attn_glue_hadi8_sigmoid_bf16_table(unsigned short *__restrict__ out) {
-  const int i = blockIdx.x * 256 + threadIdx.x;
-  out[i] = (unsigned short)iu8_bf16_bits(glue_sigmoid_bf16(iu8_bf16_f32((unsigned short)i)));
 }

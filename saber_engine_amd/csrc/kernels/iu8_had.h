@@ -100,3 +100,15 @@ static __device__ __forceinline__ void had_load8(const unsigned short *p, float 
   }
 }
 
+// The two gates of the producers above that carry the device's expf. Both are functions of a bf16
+// input, so a checker can table them over all 65,536 inputs (the tap kernels of `iu8_taps`).
+// silu in f32 (the GDN norm's gate, crates/saber-kernels/hip/mxfp4_hadi8.hip:148-186):
+static __device__ __forceinline__ float had_silu_f32(float z) {
+#pragma clang fp contract(off)
+  return z / (1.f + expf(-z));
+}
+// sigmoid rounded to bf16 (the attention output gate, crates/saber-kernels/hip/attn_glue_hadi8.hip:23-79):
+static __device__ __forceinline__ float glue_sigmoid_bf16(float g) {
+#pragma clang fp contract(off)
+  return iu8_bf16_f32((unsigned short)iu8_bf16_bits(1.f / (1.f + expf(-g))));
+}

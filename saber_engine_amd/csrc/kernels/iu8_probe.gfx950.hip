@@ -1,7 +1,7 @@
 // Roofline denominators measured on the card, next to the published ones: the code object
-// `iu8_probe`. A streaming read, a plain copy of known size (the scale factor of the HBM byte
-// counters), an empty launch (the per-launch floor of back-to-back timing) and a register-resident
-// int8 MFMA loop (the matrix peak the clocks actually sustain).
+// `iu8_probe`. A streaming read (the HBM bandwidth a kernel can reach), a plain copy of known size
+// (the scale factor of the HBM byte counters) and a register-resident int8 MFMA loop on operands read
+// from memory once (the matrix rate the clocks sustain for given operand values).
 #include "iu8_common.h"
 
 // reads n16 16-byte pieces once; grid-stride, 8 loads in flight a lane; the xor lands in out[0]
@@ -31,47 +31,7 @@ extern "C" __global__ __launch_bounds__(256) void iu8_probe_copy(const unsigned 
   for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n16; i += stride) q[i] = p[i];
 }
 
-extern "C" __global__ __launch_bounds__(256) void iu8_probe_empty(unsigned *__restrict__ out) {
-  if (out == nullptr && threadIdx.x == 1023) __builtin_trap();
-}
-
-// n = iterations; every wave runs 8 independent accumulator chains of v_mfma_i32_16x16x64_i8
-// (32,768 int8 ops each) per iteration
-extern "C" __global__ __launch_bounds__(256) void iu8_probe_mfma(unsigned *__restrict__ out, int n) {
-  iu8_v4i a = iu8_v4i{(int)threadIdx.x, 1, 2, 3}, b = iu8_v4i{4, 5, (int)blockIdx.x, 7};
-  iu8_v4i c[8];
-#pragma unroll
-  for (int j = 0; j < 8; ++j) c[j] = iu8_v4i{j, 0, 0, 0};
-  for (int i = 0; i < n; ++i) {
-#pragma unroll
-    for (int j = 0; j < 8; ++j) c[j] = iu8_mfma(a, b, c[j]);
-  }
-  iu8_v4i s = c[0];
-#pragma unroll
-  for (int j = 1; j < 8; ++j) s += c[j];
-  if ((s.x ^ s.y ^ s.z ^ s.w) == 0x12345679) out[0] = s.x;
-}
-
-// the same with v_mfma_i32_32x32x32_i8 (65,536 int8 ops each), 4 independent chains
 typedef int iu8_v16i __attribute__((ext_vector_type(16)));
-extern "C" __global__ __launch_bounds__(256) void iu8_probe_mfma32(unsigned *__restrict__ out, int n) {
-  iu8_v4i a = iu8_v4i{(int)threadIdx.x, 1, 2, 3}, b = iu8_v4i{4, 5, (int)blockIdx.x, 7};
-  iu8_v16i c[4];
-#pragma unroll
-  for (int j = 0; j < 4; ++j)
-#pragma unroll
-    for (int e = 0; e < 16; ++e) c[j][e] = j + e;
-  for (int i = 0; i < n; ++i) {
-#pragma unroll
-    for (int j = 0; j < 4; ++j) c[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c[j], 0, 0, 0);
-  }
-  int s = 0;
-#pragma unroll
-  for (int j = 0; j < 4; ++j)
-#pragma unroll
-    for (int e = 0; e < 16; ++e) s ^= c[j][e];
-  if (s == 0x12345679) out[0] = s;
-}
 
 // The matrix rate with real operands: every lane loads 4 + 4 operands from `src` once (random
 // bytes or zeros, the caller's choice) and runs the 4 x 4 tile pattern of the prefill GEMM,
@@ -104,26 +64,4 @@ extern "C" __global__ __launch_bounds__(256) void iu8_probe_mfma32d(const unsign
 #pragma unroll
       for (int e = 0; e < 16; ++e) s ^= c[i][j][e];
   if (s == 0x12345679) out[0] = s;
-}
-
-// What a launch pays before its first bytes: every wave stamps the 100 MHz constant clock at its
-// start and after each of n dependent 1 KiB wave-loads (16 bytes a lane, nontemporal, one in flight
-// at a time) of its own region of src; lane 0 stores the n + 1 stamps to out[(wave id) * (n + 1) ...]
-// as 64-bit values. The first interval holds the start-of-kernel cost on top of the memory latency
-// the later intervals show.
-extern "C" __global__ __launch_bounds__(512) void iu8_probe_first(const unsigned char *__restrict__ src,
-                                                                  unsigned *__restrict__ out, int n) {
-  const int wave = (int)blockIdx.x * 8 + (int)(threadIdx.x >> 6), lane = threadIdx.x & 63;
-  unsigned long long *o = (unsigned long long *)out + (size_t)wave * (n + 1);
-  unsigned long long t = __builtin_amdgcn_s_memrealtime();
-  if (lane == 0) o[0] = t;
-  const unsigned char *p = src + ((size_t)wave * n) * 1024 + lane * 16;
-  for (int r = 0; r < n; ++r) {
-    iu8_v4u v;
-    const unsigned char *q = p + (size_t)r * 1024;
-    // load and wait in one volatile statement, so the stamp that follows is taken after the data
-    asm volatile("global_load_dwordx4 %0, %1, off nt\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(q) : "memory");
-    t = __builtin_amdgcn_s_memrealtime() + (v.x == 0x9E3779B9u && v.y == 1u);
-    if (lane == 0) o[r + 1] = t;
-  }
 }

@@ -8,29 +8,26 @@
 // column block fastest -- then problem 1's, end to end in gridDim.x; each workgroup runs the plain
 // decode body (iu8_gemm.h) on its problem's operands, so the bytes of c and c_b are those of two
 // separate launches. What it saves is a launch: on this card a decode GEMV launch costs several
-// microseconds of start and drain beside its streaming time.
+// microseconds of start and drain beside its streaming time. The `pairb` symbols lay the second
+// problem's workgroups in front of problem 0's (the reference's ba-first order,
+// crates/saber-kernels/src/macaq_iu8.rs:549-553): the same bytes, the small half not in the tail.
 #include "iu8_gemm.h"
 
-#define IU8F_PAIR(name, TM, NT, KW, WPB, D, ALDS)                                                                  \
+#define IU8F_PAIR(name, TM, NT, KW, WPB, D, ALDS, BFIRST)                                                                \
   extern "C" __global__ __launch_bounds__(WPB * 64) void name(                                                      \
       const unsigned char *__restrict__ a, const float *__restrict__ as, const unsigned char *__restrict__ w,       \
       const float *__restrict__ ws, int *__restrict__ decode_partial, int *__restrict__ decode_counter,             \
       unsigned short *__restrict__ c, const unsigned char *__restrict__ w_b, const float *__restrict__ ws_b,        \
       int *__restrict__ decode_partial_b, int *__restrict__ decode_counter_b, unsigned short *__restrict__ c_b,     \
       int m, int k, int n, int ks, int nb, int n_b, int ks_b, int nb_b) {                                           \
-    const int b0 = nb * ks;                                                                                         \
-    const bool p1 = (int)blockIdx.x >= b0;                                                                          \
-    const int bl = p1 ? (int)blockIdx.x - b0 : (int)blockIdx.x, nbp = p1 ? nb_b : nb;                              \
+    const int b0 = nb * ks, b1 = nb_b * ks_b, bx = (int)blockIdx.x;                                                 \
+    const bool p1 = BFIRST ? bx < b1 : bx >= b0;                                                                    \
+    const int bl = BFIRST ? (p1 ? bx : bx - b1) : (p1 ? bx - b0 : bx), nbp = p1 ? nb_b : nb;                        \
     iu8_dec_body<TM, false, NT, KW, WPB, D, ALDS, false>(                                                           \
         a, p1 ? w_b : w, as, p1 ? ws_b : ws, p1 ? decode_partial_b : decode_partial,                                \
         p1 ? decode_counter_b : decode_counter, p1 ? c_b : c, iu8_rows{nullptr, 0, m}, p1 ? n_b : n, k,             \
         iu8_blk{bl % nbp, bl / nbp, p1 ? ks_b : ks});                                                               \
   }
-#define IU8_DEC_VARIANT(name, TM, W8, NT, KW, WPB, D, ALDS, ACC)
-#define IU8_PF_VARIANT(name, W8, WMW, WNW, TM, TN, ACC, ST, OCC, DEEP)
-#define IU8_PAIR_VARIANT(name, TM, NT, KW, WPB, D, ALDS) IU8F_PAIR(name, TM, NT, KW, WPB, D, ALDS)
+#define IU8_PAIR_VARIANT(name, TM, NT, KW, WPB, D, ALDS, BFIRST) IU8F_PAIR(name, TM, NT, KW, WPB, D, ALDS, BFIRST)
 #include "iu8_variants.def"
-#undef IU8_DEC_VARIANT
-#undef IU8_PF_VARIANT
-#undef IU8_PAIR_VARIANT
 #undef IU8F_PAIR

@@ -10,7 +10,6 @@
 //   quant_hadi8_t{256,512}_tiled1           v = x (no counterpart among the reference's symbols: the
 //                                           transform in front of the plain producer)
 //   gdn_norm_quant_hadi8_t256_tiled1        v = bf16(((x * inv_head) * w) * silu_f32(z)), per 128-element head
-//   mxfp4_hadi8_silu_f32_table              a checker's tap: silu_f32 of all 65,536 bf16 inputs
 //
 // The sums of squares keep the reference's order: add_rms per-thread fma over its groups, then
 // shfl_down 16..1 inside each 32 lanes, then over the T/32 partials; gdn_norm per group
@@ -18,7 +17,8 @@
 // `rsqrtf` is the one thing not taken over: the device's approximate reciprocal square root cannot be
 // restated on a host, so inv = 1 / sqrt(x) here uses the IEEE square root and divide. gdn_norm's
 // gate silu_f32(z) = z / (1 + expf(-z)) stays in f32 and so carries the device's expf: a function of
-// a bf16 input, it is tabled by the tap kernel for a checker to hold against a host's.
+// a bf16 input, it is tabled by a tap kernel of the test-only object `iu8_taps` (had_silu_f32 lives
+// in iu8_had.h for both) for a checker to hold against a host's.
 #include "iu8_had.h"
 
 template <int T>
@@ -151,11 +151,6 @@ HAD_Q(quant_hadi8_t256_tiled1, 256)
 HAD_Q(quant_hadi8_t512_tiled1, 512)
 #undef HAD_Q
 
-static __device__ __forceinline__ float had_silu_f32(float z) {
-#pragma clang fp contract(off)
-  return z / (1.f + expf(-z));
-}
-
 // One workgroup a row of N = heads * 128 elements; z rows `zs` elements apart; w the head's 128 weights.
 template <int T>
 static __device__ __forceinline__ void had_gdn_norm_body(const unsigned short *__restrict__ x,
@@ -198,9 +193,4 @@ extern "C" __global__ __launch_bounds__(256) void gdn_norm_quant_hadi8_t256_tile
     const unsigned short *__restrict__ w, unsigned char *__restrict__ q, float *__restrict__ scale, int N, float eps,
     const float *__restrict__ had_t) {
   had_gdn_norm_body<256>(x, z, zs, w, q, scale, N, eps, had_t);
-}
-
-extern "C" __global__ __launch_bounds__(256) void mxfp4_hadi8_silu_f32_table(float *__restrict__ out) {
-  const int i = blockIdx.x * 256 + threadIdx.x;
-  out[i] = had_silu_f32(iu8_bf16_f32((unsigned short)i));
 }

@@ -17,6 +17,9 @@ PKG = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(PKG)
 LIB_PATH = os.path.join(PKG, "libsaber_iu8.so")
 PREBUILT = os.path.join(ROOT, "prebuilt", "gfx950")
+# the parity suite's test-only object (accumulator and table taps), outside the plugin directory
+TAPS_MANIFEST = os.path.join(PREBUILT, "taps", "iu8_taps.manifest.toml")
+BAND_TABLE = os.path.join(PREBUILT, "macaq_iu8.band.toml")
 
 W4, W8 = 0, 1
 ARG_BUFFER, ARG_NULL_BUFFER, ARG_I32, ARG_F32, ARG_I64 = 0, 1, 2, 3, 4
@@ -110,6 +113,9 @@ def lib():
         L.saber_iu8_gemm_acc.argtypes = [C.c_void_p, C.c_int] + [C.c_void_p] * 3 + [C.c_uint32] * 3 + [C.c_void_p]
         L.saber_iu8_fused_holds.argtypes = [C.c_uint32, C.c_uint32]
         L.saber_iu8_pair.argtypes = [C.POINTER(Desc)] * 3
+        L.saber_iu8_pair_ordered.argtypes = [C.POINTER(Desc)] * 2 + [C.c_int, C.POINTER(Desc)]
+        L.saber_iu8_load_plugin.argtypes = [C.c_void_p, C.c_char_p]
+        L.saber_iu8_band_toml.argtypes = [C.c_char_p, C.c_size_t, C.POINTER(C.c_size_t)]
         L.saber_iu8_gemm_pair.argtypes = [C.c_void_p] * 6 + [C.c_uint32] + [C.c_void_p] * 3 + [C.c_uint32] * 3 + [C.c_void_p]
         L.saber_iu8_linear_fused.argtypes = [C.c_void_p, C.c_int] + [C.c_void_p] * 6 + [C.c_uint32] * 3 + [C.c_void_p]
         L.saber_iu8_quant_had.argtypes = [C.c_void_p] * 4 + [C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p]
@@ -161,6 +167,22 @@ def pair(first, second):
     d = Desc()
     _check(lib().saber_iu8_pair(C.byref(first), C.byref(second), C.byref(d)))
     return d
+
+
+def pair_ordered(first, second, second_first):
+    """The pair with its block order named: the second problem's workgroups first (`pairb`) or last."""
+    d = Desc()
+    _check(lib().saber_iu8_pair_ordered(C.byref(first), C.byref(second), int(bool(second_first)), C.byref(d)))
+    return d
+
+
+def band_toml():
+    """The launch law as TOML text (what the build step writes to BAND_TABLE)."""
+    need = C.c_size_t(0)
+    lib().saber_iu8_band_toml(None, 0, C.byref(need))
+    buf = C.create_string_buffer(need.value)
+    _check(lib().saber_iu8_band_toml(buf, need.value, None))
+    return buf.value.decode()
 
 
 def fused_holds(m, k):
@@ -287,6 +309,13 @@ class Context:
             self.close()
         except Exception:
             pass
+
+    def load_plugin(self, manifest_path):
+        """Add one plugin from outside the plugin directory (the parity suite's taps)."""
+        _check(lib().saber_iu8_load_plugin(self._h, manifest_path.encode()))
+
+    def load_taps(self):
+        self.load_plugin(TAPS_MANIFEST)
 
     def counters(self):
         c = Counters()

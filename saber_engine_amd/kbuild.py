@@ -5,7 +5,9 @@
 For every kernel stem: resolve `<k>.gfx950.hip -> <k>.gfx95.hip -> <k>.hip`, compile with
 `hipcc --genco --offload-arch=gfx950 -O3 ...`, hash sha256(preprocessed source ++ flags), and
 write `prebuilt/gfx950/<k>.hsaco` + `<k>.manifest.toml` (schema 1, every number read back from
-the code object that was just built). Also builds the host library `libsaber_iu8.so`.
+the code object that was just built). Also builds the host library `libsaber_iu8.so`, the
+test-only tap object under `prebuilt/gfx950/taps/`, and writes the launch law as data to
+`prebuilt/gfx950/macaq_iu8.band.toml`.
 
     python -m saber_engine_amd.kbuild            # everything
     python -m saber_engine_amd.kbuild macaq_iu8  # one plugin
@@ -30,6 +32,11 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # the packed-fp32 feature is switched off for every device compile of this tree.
 FLAGS = f"--genco --offload-arch={ARCH} -O3 -ffp-contract=off -Xclang -target-feature -Xclang -packed-fp32-ops"
 PLUGINS = ("macaq_iu8", "macaq_iu8f", "macaq_i8q", "mxfp4_hadi8", "attn_glue_hadi8", "moe_iu8", "iu8_probe")
+# test infrastructure (accumulator and table taps of the parity suite): built beside the plugin
+# directory, where opening the plugin set does not see it
+TAPS = ("iu8_taps",)
+TAPS_DIR = os.path.join(PREBUILT, "taps")
+BAND = os.path.join(PREBUILT, "macaq_iu8.band.toml")
 
 
 def candidates(stem, arch):
@@ -96,13 +103,33 @@ def build_plugin(stem, out_dir=PREBUILT):
     return hsaco, manifest
 
 
+def band_text():
+    """The launch law as TOML text, straight from the host library."""
+    L = _lib()
+    need = ctypes.c_size_t(0)
+    L.saber_iu8_band_toml(None, ctypes.c_size_t(0), ctypes.byref(need))
+    buf = ctypes.create_string_buffer(need.value)
+    if L.saber_iu8_band_toml(buf, ctypes.c_size_t(need.value), None) != 0:
+        raise RuntimeError("band table: " + L.saber_iu8_last_error().decode())
+    return buf.value.decode()
+
+
+def write_band(path=BAND):
+    os.makedirs(os.path.dirname(path), exist_ok=True)
+    with open(path, "w") as f:
+        f.write(band_text())
+    return path
+
+
 def build_all(stems=None):
     build_lib()
     built = []
-    for stem in stems or PLUGINS:
+    for stem in stems or PLUGINS + TAPS:
         if resolve_source(stem) is None:
             continue
-        built.append(build_plugin(stem))
+        built.append(build_plugin(stem, TAPS_DIR if stem in TAPS else PREBUILT))
+    if not stems:
+        write_band()
     return built
 
 

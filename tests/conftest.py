@@ -21,6 +21,7 @@ def ctx():
     from saber_engine_amd import iu8
 
     c = iu8.Context()
+    c.load_taps()   # accumulator and table taps: test infrastructure, not in the plugin directory
     yield c
     torch.cuda.synchronize()
     c.close()

@@ -8,8 +8,11 @@ int64 matrix product for the accumulators, float64 products rounded once to floa
 epilogue multiplies (exact: a product of two float32 fits float64), the bit trick for bf16 -- and
 NOT by the C oracle. The oracle and the HIP path are both checked against them.
 
-kernarg_gfx1201.json holds data read off the reference's committed manifest
-(prebuilt/gfx1201/macaq_iu8.manifest.toml): the explicit kernarg offsets/sizes the host packs.
+kernarg_gfx1201.json holds data read off the reference's committed manifests
+(prebuilt/gfx1201/macaq_iu8.manifest.toml and those of the pair and the int8 producers): the explicit
+kernarg offsets/sizes the host packs; kernarg_gfx1201_moe.json the same for the routed layer's
+kernels (prebuilt/gfx1201/moe_route.manifest.toml, moe_grouped.manifest.toml), each with the gfx950
+kernels that keep its list.
 """
 import json
 import os
@@ -64,10 +67,53 @@ def main():
 # symbols this build also ships are kept (every macaq_iu8 kernel, the decode pair, the int8 twins).
 KERNARG_SOURCES = {
     "macaq_iu8": None,
-    "macaq_iu8f": ("macaq_iu8f_pair_w4_tm",),
+    "macaq_iu8f": ("macaq_iu8f_pair_w4_tm", "macaq_iu8f_pairb_w4_tm"),
     "mxfp4_hadi8": ("add_rms_quant_hadi8_", "silu_mul_quant_hadi8_", "gdn_norm_quant_hadi8_"),
     "attn_glue_hadi8": ("attn_gate_quant_hadi8_",),
 }
+
+
+# The routed layer: the reference's kernels carry other names (its router is 512 experts / top-10, its
+# grouped GEMM MXFP4 x e4m3) but the argument lists are the launch contract this build keeps; each
+# reference kernel is listed with the gfx950 kernels that take the same list.
+MOE_KERNARG_SOURCES = {
+    "moe_route": {
+        "moe_route_topk10_sort_e512": ["moe_iu8_route_topk8_sort_e128"],
+        "moe_combine_bf16": ["moe_iu8_combine_bf16"],
+    },
+    "moe_grouped": {
+        "moe_grouped_w4a8_bk128_ks1_tm1_g0": ["moe_iu8_grouped_w4_dec_g0", "moe_iu8_grouped_w4_deca_g0", "moe_iu8_grouped_w4_deck_g0"],
+        "moe_grouped_w4a8_bk128_ks1_tm1_g1": ["moe_iu8_grouped_w4_dec_g1", "moe_iu8_grouped_w4_deca_g1", "moe_iu8_grouped_w4_deck_g1"],
+        "moe_grouped_w4a8_pf_tm8_g0": ["moe_iu8_grouped_w4_pf_g0"],
+        "moe_grouped_w4a8_pf_tm8_g1": ["moe_iu8_grouped_w4_pf_g1", "moe_iu8_grouped_w4_pf_g2"],
+        "moe_grouped_w4a8_pf_tm16_g0": ["moe_iu8_grouped_w4_pf16_g0"],
+        "moe_grouped_w4a8_pf_tm16_g1": ["moe_iu8_grouped_w4_pf16_g1", "moe_iu8_grouped_w4_pf16_g2"],
+        "moe_silu_mul_quant_t256": ["macaq_i8_silu_mul_quant_t256", "macaq_i8_silu_mul_quant_t256_g1", "macaq_i8_silu_mul_quant_w64"],
+    },
+}
+
+
+def _manifest_args(ref_dir, plugin):
+    import re
+
+    text = open(os.path.join(ref_dir, plugin + ".manifest.toml")).read()
+    out = {}
+    for blk in text.split("[[kernel]]")[1:]:
+        name = re.search(r'name = "(\w+)"', blk).group(1)
+        args = re.findall(r'offset = (\d+)\nsize = (\d+)\nvalue_kind = "(\w+)"\nname = "(\w+)"', blk)
+        out[name] = [dict(name=a[3], offset=int(a[0]), size=int(a[1]), value_kind=a[2]) for a in args]
+    return out
+
+
+def write_moe_kernarg_table(ref_dir="/root/reference/prebuilt/gfx1201"):
+    if not os.path.isdir(ref_dir):
+        return
+    table = {}
+    for plugin, names in MOE_KERNARG_SOURCES.items():
+        args = _manifest_args(ref_dir, plugin)
+        for ref_name, ours in names.items():
+            table[ref_name] = dict(args=args[ref_name], gfx950=ours)
+    json.dump(table, open(os.path.join(HERE, "kernarg_gfx1201_moe.json"), "w"), indent=1, sort_keys=True)
 
 
 def write_kernarg_table(ref_dir="/root/reference/prebuilt/gfx1201"):
@@ -75,6 +121,7 @@ def write_kernarg_table(ref_dir="/root/reference/prebuilt/gfx1201"):
 
     if not os.path.isdir(ref_dir):
         return
+    write_moe_kernarg_table(ref_dir)
     table = {}
     for plugin, prefixes in KERNARG_SOURCES.items():
         text = open(os.path.join(ref_dir, plugin + ".manifest.toml")).read()

@@ -42,6 +42,44 @@ def test_config1_decode_layer_set(ctx, M):
         assert_dense_matches(DenseRun(ctx, case), r, False)
 
 
+@pytest.mark.parametrize("M", [1, 4])
+def test_config1_decode_layer_set_as_the_fused_launches_the_benchmark_times(ctx, M):
+    """The hot path as bench.py launches it: one fused quant + GEMV launch a linear
+    (macaq_iu8_decq_w4_tm1), on the four full layer shapes, against the oracle."""
+    for name, n, k in synth.LAYER_LINEARS:
+        if not iu8.fused_holds(M, k):          # down at M = 4: 4 x 17408 codes do not fit the staged form
+            assert (name, M) == ("down", 4)
+            continue
+        say(f"config 1, fused launch: {name} M={M} N={n} K={k}")
+        case = synth.dense_case(M, n, k, seed=M)
+        r = ref.linear(case["X"], case["W"], case["ws"], False, threads=16)
+        x, wf, ws = dev_bf16_bits(case["X"]), dev_u8(iu8.repack_w4(case["W"])), dev_f32(case["ws"])
+        c = torch.full((M, n), 0x7FC0, dtype=torch.int16, device="cuda")
+        d = iu8.resolve_fused(iu8.W4, M, n, k)
+        assert d.kernel == b"macaq_iu8_decq_w4_tm1"
+        for a in ("q", "scale"):                # as the benchmark launches it: no optional outputs
+            d.arg(a).kind = iu8.ARG_NULL_BUFFER
+        ctx.launch(d, dict(x=x.data_ptr(), w=wf.data_ptr(), ws=ws.data_ptr(), c=c.data_ptr()))
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(host_u16(c), r["C"])
+
+
+def test_launch_refuses_a_block_the_kernel_is_not_written_for(ctx):
+    """A descriptor under another launch law (the reference's 256-thread blocks under its own names,
+    crates/saber-kernels/src/macaq_iu8.rs:429-489) is refused by name before anything is launched."""
+    x = torch.zeros(4096, dtype=torch.uint8, device="cuda")
+    for kernel, m in (("macaq_iu8_pf_w4_tn4_lbk64", 256), ("macaq_iu8_dec_w4_tm1", 1)):
+        d = iu8.describe(kernel, m, 128, 256)
+        d.block[0] = 256                         # the reference's block
+        bufs = dict(a=x.data_ptr(), w=x.data_ptr(), ws=x.data_ptr(), c=x.data_ptr())
+        bufs["as"] = x.data_ptr()
+        before = ctx.counters().launches
+        with pytest.raises(iu8.IU8Error) as e:
+            ctx.launch(d, bufs)
+        assert e.value.code == iu8.E_RULE and "threads" in str(e.value)
+        assert ctx.counters().launches == before
+
+
 def all_variants(prefix):
     text = open(os.path.join(iu8.PKG, "csrc", "kernels", "iu8_variants.def")).read()
     names = re.findall(r"^IU8_(?:DEC|PF)_VARIANT\((\w+),", text, flags=re.M)
@@ -230,7 +268,7 @@ def test_config2_prefill_full_shapes_by_properties(ctx, M):
     rng = np.random.default_rng(M)
     for name, n, k in synth.LAYER_LINEARS:
         if M == 8192 and name == "gate_up":
-            n = 8704                                       # a quarter of the columns keeps the int32 tap at 285 MB
+            continue                                       # its int32 tap would be 1.1 GB: the test below, by column quarters
         say(f"config 2: {name} M={M} N={n} K={k}")
         W, ws = synth.weights(rng, n, k, False)
         X = synth.activations(rng, M, k)
@@ -258,6 +296,74 @@ def test_config2_prefill_full_shapes_by_properties(ctx, M):
         assert torch.equal(t.to(torch.bfloat16).view(torch.int16), c)
         del xd, wf, wsd, q, s, c, acc, t
         torch.cuda.empty_cache()
+
+
+def test_config2_gate_up_at_8192_rows_full_width(ctx):
+    """gate+up 34816 x 5120 at M = 8192, the largest cell of configs[2], at its full width: the bf16
+    output of ONE launch over all 34,816 columns; the int32 tap on column quarters (the rows of W are
+    16-row fragments, so a quarter of the columns is a contiguous quarter of the weight bytes), every
+    quarter by linearity and by the device-side epilogue identity, an oracle slice bit for bit."""
+    M, n, k = 8192, 34816, 5120
+    say(f"config 2: gate_up M={M} N={n} K={k}, full width")
+    rng = np.random.default_rng(8192)
+    W, ws = synth.weights(rng, n, k, False)
+    X = synth.activations(rng, M, k)
+    xd, wf, wsd = dev_bf16_bits(X), dev_u8(iu8.repack_w4(W)), dev_f32(ws)
+    q = torch.zeros(iu8.a_bytes(M, k), dtype=torch.uint8, device="cuda")
+    s = torch.zeros(M, dtype=torch.float32, device="cuda")
+    c = torch.zeros((M, n), dtype=torch.int16, device="cuda")
+    ctx.quant(xd.data_ptr(), q.data_ptr(), s.data_ptr(), M, k)
+    ctx.gemm(iu8.W4, q.data_ptr(), s.data_ptr(), wf.data_ptr(), wsd.data_ptr(), c.data_ptr(), M, n, k)
+    torch.cuda.synchronize()
+    qh, sh = ref.quant_bf16(X)
+    np.testing.assert_array_equal(iu8.unpack_a(q.cpu().numpy(), M, k), qh)
+    colsum = qh.astype(np.int64).sum(0)
+    rows = np.unique(np.concatenate([np.arange(0, M, 331), [M - 1]]))
+    nq = n // 4
+    acc = torch.zeros((M, nq), dtype=torch.int32, device="cuda")
+    for part in range(4):
+        say(f"config 2: gate_up M={M}, int32 tap on columns {part * nq}..{(part + 1) * nq}")
+        c0 = part * nq
+        ctx.gemm_acc(iu8.W4, q.data_ptr(), wf.data_ptr() + c0 * k // 2, acc.data_ptr(), M, nq, k)
+        torch.cuda.synchronize()
+        want = synth.unpack_w4(W[c0:c0 + nq]).astype(np.int64) @ colsum * 16
+        np.testing.assert_array_equal(acc.sum(0, dtype=torch.int64).cpu().numpy(), want)
+        t = (acc.to(torch.float32) * s[:, None]) * (wsd[c0:c0 + nq] * 0.0625)[None, :]
+        assert torch.equal(t.to(torch.bfloat16).view(torch.int16), c[:, c0:c0 + nq])
+        S, _ = ref.gemm_fast(qh[rows], W[c0 + nq - 128:c0 + nq], False, threads=16)
+        np.testing.assert_array_equal(acc.cpu().numpy()[rows][:, -128:], S * 16)
+        np.testing.assert_array_equal(host_u16(c)[rows][:, c0 + nq - 128:c0 + nq], ref.epilogue(S, sh[rows], ws[c0 + nq - 128:c0 + nq], False))
+        del t
+
+
+def test_split_k_hand_over_repeats_on_full_size_shapes(ctx):
+    """A bounded soak of the cross-workgroup hand-over of the split forms (partials straight through
+    memory, a relaxed device-scope arrival counter, no fences) at the sizes the launch law and the
+    explicit splits run at: every repeat must give the first launch's bytes, which are the oracle's on
+    a column slice; the counters stay zero. Stops at its first mismatch."""
+    for kernel, (M, N, K), ks, reps in (("macaq_iu8_pf_w4_t64x128_s_ks", (128, 5120, 17408), 3, 40),
+                                        ("macaq_iu8_pf_w4_t64x128_s_ks", (64, 5120, 17408), 4, 40),
+                                        ("macaq_iu8_dec_w4_tm1", (1, 5120, 17408), 4, 60),
+                                        ("macaq_iu8_dec_w4_tm1_a0", (16, 7168, 5120), 2, 60),
+                                        ("macaq_iu8_dec_w4_tm2", (32, 5120, 5120), 3, 40)):
+        say(f"split hand-over soak {kernel} {M}x{N}x{K} ks={ks} x{reps}")
+        case = synth.dense_case(M, N, K, seed=ks * 100 + M)
+        run = DenseRun(ctx, case, kernel=kernel, ks=ks, want_acc=False)
+        qh, sh = ref.quant_bf16(case["X"])
+        S, _ = ref.gemm_fast(qh, case["W"][:512], False, threads=16)
+        np.testing.assert_array_equal(run.C[:, :512], ref.epilogue(S, sh, case["ws"][:512], False))
+        d = run.dev
+        first = d["c"].clone()
+        bufs = dict(a=d["q"].data_ptr(), w=d["wf"].data_ptr(), ws=d["ws"].data_ptr(), c=d["c"].data_ptr(),
+                    decode_partial=run.partial.data_ptr(), decode_counter=run.counter.data_ptr())
+        bufs["as"] = d["a_scale"].data_ptr()
+        for rep in range(reps):
+            d["c"].fill_(0x7FC0)
+            run.partial.fill_(0x5A5A5A5A + rep)           # scratch: undefined at entry
+            ctx.launch(run.desc, bufs)
+            torch.cuda.synchronize()
+            assert torch.equal(d["c"], first), f"repeat {rep} of {kernel} differs"
+            assert not run.counter.any().item(), "the arrival counters must be left at zero"
 
 
 def test_config4_moe_prefill_shape(ctx):

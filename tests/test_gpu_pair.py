@@ -65,7 +65,7 @@ def test_pair_of_named_cells_past_the_streaming_band(ctx):
                       w1.data_ptr(), s1.data_ptr(), c1.data_ptr(), n1, M, K)
     assert e.value.code == iu8.E_RULE
     d = iu8.pair(iu8.describe("macaq_iu8_dec_w4_tm4", M, n0, K), iu8.describe("macaq_iu8_dec_w4_tm4", M, n1, K))
-    assert d.kernel == b"macaq_iu8f_pair_w4_tm4"
+    assert d.kernel == b"macaq_iu8f_pairb_w4_tm4"
     bufs = dict(a=q.data_ptr(), w=w0.data_ptr(), ws=s0.data_ptr(), c=c0.data_ptr(), w_b=w1.data_ptr(), ws_b=s1.data_ptr(),
                 c_b=c1.data_ptr())
     bufs["as"] = s.data_ptr()
@@ -105,3 +105,31 @@ def test_pair_with_explicitly_split_halves(ctx):
         np.testing.assert_array_equal(host_u16(c0), r0["C"])
         np.testing.assert_array_equal(host_u16(c1), r1["C"])
         assert not ws_bufs["decode_counter"].cpu().numpy().any() and not ws_bufs["decode_counter_b"].cpu().numpy().any()
+
+
+@pytest.mark.parametrize("M,K,n0,n1", [(1, 5120, 12288, 96), (16, 1024, 272, 528), (40, 640, 80, 304)])
+def test_both_block_orders_give_the_same_bytes(ctx, M, K, n0, n1):
+    """`pair` (problem 0's workgroups first) and `pairb` (the second problem's first, the law's pick as
+    in the reference, crates/saber-kernels/src/macaq_iu8.rs:549-553): one kernarg list, the oracle's bytes."""
+    rng = np.random.default_rng(M + n1)
+    X, (W0, ws0), (W1, ws1) = halves(rng, M, K, n0, n1)
+    xd = dev_bf16_bits(X)
+    q = torch.zeros(iu8.a_bytes(M, K), dtype=torch.uint8, device="cuda")
+    s = torch.zeros(M, dtype=torch.float32, device="cuda")
+    ctx.quant(xd.data_ptr(), q.data_ptr(), s.data_ptr(), M, K)
+    w0, w1, s0, s1 = dev_u8(iu8.repack_w4(W0)), dev_u8(iu8.repack_w4(W1)), dev_f32(ws0), dev_f32(ws1)
+    r0, r1 = ref.linear(X, W0, ws0, False, threads=8), ref.linear(X, W1, ws1, False, threads=8)
+    a, b = iu8.resolve(iu8.W4, M, n0, K), iu8.resolve(iu8.W4, M, n1, K)
+    for second_first in (False, True):
+        d = iu8.pair_ordered(a, b, second_first)
+        say(f"pair order {d.kernel.decode()} M={M} K={K} N={n0}+{n1}")
+        assert (b"_pairb_" in d.kernel) == second_first
+        c0 = torch.full((M, n0), 0x7FC0, dtype=torch.int16, device="cuda")
+        c1 = torch.full((M, n1), 0x7FC0, dtype=torch.int16, device="cuda")
+        bufs = dict(a=q.data_ptr(), w=w0.data_ptr(), ws=s0.data_ptr(), c=c0.data_ptr(), w_b=w1.data_ptr(), ws_b=s1.data_ptr(),
+                    c_b=c1.data_ptr())
+        bufs["as"] = s.data_ptr()
+        ctx.launch(d, bufs)
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(host_u16(c0), r0["C"])
+        np.testing.assert_array_equal(host_u16(c1), r1["C"])

@@ -90,7 +90,12 @@ def test_pair_lays_two_decode_grids_end_to_end():
     split and workspaces; refusals by name."""
     a, b = iu8.resolve(iu8.W4, 4, 12288, 5120), iu8.resolve(iu8.W4, 4, 96, 5120)
     d = iu8.pair(a, b)
-    assert d.kernel == b"macaq_iu8f_pair_w4_tm1" and d.plugin == b"macaq_iu8f" and d.op == b"gemm_i4a8_pair"
+    # the law's block order is the reference's: the second ("ba") half's workgroups first at every tm
+    # (PAIR_BA_FIRST, crates/saber-kernels/src/macaq_iu8.rs:549-553)
+    assert d.kernel == b"macaq_iu8f_pairb_w4_tm1" and d.plugin == b"macaq_iu8f" and d.op == b"gemm_i4a8_pair"
+    assert iu8.pair_ordered(a, b, False).kernel == b"macaq_iu8f_pair_w4_tm1"
+    assert iu8.pair_ordered(a, b, True).kernel == b"macaq_iu8f_pairb_w4_tm1"
+    assert bytes(iu8.pair_ordered(a, b, False).args) == bytes(d.args)          # one kernarg list for both orders
     assert tuple(d.grid) == (a.grid[0] + b.grid[0], 1, 1) and d.block[0] == a.block[0] and d.n_launches == 1
     vals = {n: d.arg(n).ival for n in ("m", "k", "n", "ks", "nb", "n_b", "ks_b", "nb_b")}
     assert vals == dict(m=4, k=5120, n=12288, ks=1, nb=a.grid[0], n_b=96, ks_b=1, nb_b=b.grid[0])
@@ -98,8 +103,8 @@ def test_pair_lays_two_decode_grids_end_to_end():
         assert d.arg(n).kind == iu8.ARG_NULL_BUFFER
     assert d.n_workspaces == 0 and d.kernarg_bytes == 128
     # rows that stream from L2 pair on the streamed form
-    assert iu8.pair(iu8.resolve(iu8.W4, 16, 5120, 5120), iu8.resolve(iu8.W4, 16, 64, 5120)).kernel == b"macaq_iu8f_pair_w4_tm1_a0"
-    assert iu8.pair(iu8.resolve(iu8.W4, 40, 5120, 5120), iu8.resolve(iu8.W4, 40, 64, 5120)).kernel == b"macaq_iu8f_pair_w4_tm3"
+    assert iu8.pair(iu8.resolve(iu8.W4, 16, 5120, 5120), iu8.resolve(iu8.W4, 16, 64, 5120)).kernel == b"macaq_iu8f_pairb_w4_tm1_a0"
+    assert iu8.pair(iu8.resolve(iu8.W4, 40, 5120, 5120), iu8.resolve(iu8.W4, 40, 64, 5120)).kernel == b"macaq_iu8f_pairb_w4_tm3"
     # explicit splits: the grids multiply, the second half's workspaces take the suffix
     a2, b2 = iu8.describe("macaq_iu8_dec_w4_tm1", 4, 256, 5120, ks=2), iu8.describe("macaq_iu8_dec_w4_tm1", 4, 64, 5120, ks=4)
     d2 = iu8.pair(a2, b2)
@@ -119,11 +124,72 @@ def test_pair_lays_two_decode_grids_end_to_end():
 def test_pair_variants_share_their_decode_twin_geometry():
     text = open(os.path.join(iu8.PKG, "csrc", "kernels", "iu8_variants.def")).read()
     dec = {m[0]: m[1:] for m in re.findall(r"^IU8_DEC_VARIANT\((\w+), (\d+), (\w+), (\d+), (\d+), (\d+), (\d+), (\d+), (\w+)\)", text, flags=re.M)}
-    pairs = re.findall(r"^IU8_PAIR_VARIANT\((\w+), (\d+), (\d+), (\d+), (\d+), (\d+), (\d+)\)", text, flags=re.M)
-    assert len(pairs) == 5
-    for name, tm, nt, kw, wpb, d, alds in pairs:
-        twin = dec[name.replace("macaq_iu8f_pair_", "macaq_iu8_dec_")]
+    pairs = re.findall(r"^IU8_PAIR_VARIANT\((\w+), (\d+), (\d+), (\d+), (\d+), (\d+), (\d+), (\w+)\)", text, flags=re.M)
+    assert len(pairs) == 10
+    for name, tm, nt, kw, wpb, d, alds, bfirst in pairs:
+        assert (bfirst == "true") == ("_pairb_" in name)
+        twin = dec[name.replace("macaq_iu8f_pairb_", "macaq_iu8_dec_").replace("macaq_iu8f_pair_", "macaq_iu8_dec_")]
         assert twin == (tm, "false", nt, kw, wpb, d, alds, "false"), name
+
+
+def test_reference_symbol_names_are_answered_by_the_law():
+    """Names of the reference's fused object that encode gfx1201 tiles (macaq_iu8.rs:520-546) are
+    requests for the op at the shape: the descriptor is the gfx950 law's; the all-reduce forms are
+    refused by name."""
+    for name, wk, shape in (("macaq_iu8f_dec_w4_tm5", iu8.W4, (80, 5120, 5120)), ("macaq_iu8f_pf_w4_bm128", iu8.W4, (400, 5120, 17408)),
+                            ("macaq_iu8f_pf_w8_bm64", iu8.W8, (200, 5120, 5120)), ("macaq_iu8f_pf_w4_t3w8n4k128p", iu8.W4, (384, 34816, 5120)),
+                            ("macaq_iu8f_pf_w8_t1w4n2k128", iu8.W8, (300, 5120, 6144))):
+        d, law = iu8.describe(name, *shape), iu8.resolve(wk, *shape)
+        assert bytes(d) == bytes(law) and d.kernel.decode().startswith("macaq_iu8_pf_"), name
+    with pytest.raises(iu8.IU8Error) as e:
+        iu8.describe("macaq_iu8f_arnq_hadi8_w4_tm1", 1, 5120, 5120)
+    assert e.value.code == iu8.E_RULE and "all-reduce" in str(e.value)
+    with pytest.raises(iu8.IU8Error):
+        iu8.describe("macaq_iu8f_pf_w4_bm128", 400, 5120, 17408, ks=2)
+
+
+def test_band_table_is_the_launch_law():
+    """prebuilt/gfx950/macaq_iu8.band.toml (the law as data, the gfx950 counterpart of the reference's
+    PF_BAND / PF_TILES tables, macaq_iu8.rs:150-212) is what the library writes today, and every row
+    re-derives from saber_iu8_resolve at both ends and the middle of its run."""
+    import tomli
+
+    text = open(iu8.BAND_TABLE).read()
+    assert text == iu8.band_toml(), "stale band table: run python -m saber_engine_amd.kbuild"
+    t = tomli.loads(text)
+    assert t["arch"] == "gfx950" and t["cu_count"] == 256 and t["decode_split"] == 1
+    cells = {c["kernel"]: c for c in t["cell"]}
+    runs = {}
+    for b in t["band"]:
+        wk = iu8.W8 if b["w8"] else iu8.W4
+        for m in sorted({b["first_m"], (b["first_m"] + b["last_m"]) // 2, b["last_m"]}):
+            d = iu8.resolve(wk, m, b["n"], b["k"])
+            assert d.kernel.decode() == b["kernel"] and d.ks == b["ks"] and d.block[0] == b["block"], (b, m)
+        assert list(iu8.resolve(wk, b["first_m"], b["n"], b["k"]).grid) == b["grid_first"]
+        assert list(iu8.resolve(wk, b["last_m"], b["n"], b["k"]).grid) == b["grid_last"]
+        c = cells[b["kernel"]]
+        assert c["threads"] == b["block"] and c["w8"] == b["w8"]
+        if c["regime"] == "prefill" and b["ks"] == 1:     # the persistent grid law the cell row states
+            tiles = -(-b["last_m"] // c["block_m"]) * -(-b["n"] // c["block_n"])
+            assert b["grid_last"] == [min(tiles, 256 * c["workgroups_per_cu"]), 1, 1]
+        runs.setdefault((b["op"], b["w8"]), []).append((b["first_m"], b["last_m"]))
+    for key, rr in runs.items():       # the runs of a shape tile 1..band_last_m without gap or overlap
+        rr.sort()
+        assert rr[0][0] == 1 and rr[-1][1] == t["band_last_m"] and all(x[1] + 1 == y[0] for x, y in zip(rr, rr[1:])), key
+    # the reference's whole symbol set is listed, with an answer each
+    names = {r["name"]: r["answer"] for r in t["reference_symbol"]}
+    assert len(names) == 45 and names["macaq_iu8_pf_w4_tn4_lbk64"].startswith("same name") and names["macaq_iu8f_arnq_hadi8_w4_tm1"] == "none"
+    assert t["moe"]["tile_blocks_1_last_tokens"] == 112 and t["moe"]["tile_blocks_8_last_tokens"] == 2047
+    assert t["pair"]["second_first"] == [True] * 4
+
+
+def test_operands_past_4_gib_are_refused_by_the_tile_gemm():
+    with pytest.raises(iu8.IU8Error) as e:
+        iu8.resolve(iu8.W4, 300000, 5120, 17408)            # A: 300,000 x 17,408 bytes
+    assert e.value.code == iu8.E_RULE and "4 GiB" in str(e.value)
+    with pytest.raises(iu8.IU8Error):
+        iu8.resolve(iu8.W8, 256, 262144, 16384)             # W8: 4 GiB of weights
+    assert iu8.resolve(iu8.W4, 8192, 34816, 5120).ks == 1
 
 
 def test_launch_law_shares_k_only_on_deep_narrow_tile_gemms():
@@ -137,7 +203,8 @@ def test_launch_law_shares_k_only_on_deep_narrow_tile_gemms():
         assert c.bytes == tiles * 4 and c.kind == iu8.WS_PERSISTENT and c.zero_once
         assert iu8.gemm_workspace(iu8.W4, m, 5120, 17408) == (ks * m * 5120 * 4, tiles * 4)
     for wk, m, n, k in ((iu8.W4, 129, 5120, 17408), (iu8.W4, 64, 5120, 16256), (iu8.W4, 64, 12288, 17408),
-                        (iu8.W8, 64, 5120, 17408), (iu8.W4, 2048, 5120, 17408), (iu8.W4, 64, 5120, 5120)):
+                        (iu8.W8, 64, 5120, 17408), (iu8.W4, 2048, 5120, 17408), (iu8.W4, 64, 5120, 5120),
+                        (iu8.W4, 4096, 128, 17408), (iu8.W4, 4096, 16, 16384)):       # many rows of a narrow output: few tiles, no split
         d = iu8.resolve(wk, m, n, k)
         assert d.ks == 1 and d.n_workspaces == 0 and not d.kernel.endswith(b"_ks"), (m, n, k)
         assert iu8.gemm_workspace(wk, m, n, k) == (0, 0)
@@ -202,7 +269,27 @@ def test_signatures_pack_exactly_like_the_reference_manifest():
         assert [("global_buffer" if s[3] == iu8.ARG_BUFFER else "by_value") for s in slots] == [a["value_kind"] for a in args]
         assert nbytes == max(a["offset"] + a["size"] for a in args)
         checked += 1
-    assert checked == 20
+    assert checked == 24
+
+
+def test_routed_layer_signatures_keep_the_reference_lists():
+    """The router, the grouped GEMM, the SiLU*up requant and the combine pack their kernargs as the
+    reference's kernels of the same role do (prebuilt/gfx1201/moe_route.manifest.toml,
+    moe_grouped.manifest.toml): names, offsets, sizes, value kinds."""
+    table = json.load(open(os.path.join(GOLD, "kernarg_gfx1201_moe.json")))
+    checked = 0
+    for ref_name, row in table.items():
+        for ours in row["gfx950"]:
+            slots, nbytes = iu8.signature(ours)
+            assert [(s[0], s[1], s[2]) for s in slots] == [(a["name"], a["offset"], a["size"]) for a in row["args"]], (ref_name, ours)
+            assert [("global_buffer" if s[3] == iu8.ARG_BUFFER else "by_value") for s in slots] == [a["value_kind"] for a in row["args"]]
+            assert nbytes == max(a["offset"] + a["size"] for a in row["args"])
+            checked += 1
+    assert checked == 17 and len(table) == 9
+    text = open(os.path.join(iu8.PREBUILT, "moe_iu8.manifest.toml")).read() + open(os.path.join(iu8.PREBUILT, "macaq_i8q.manifest.toml")).read()
+    for row in table.values():
+        for ours in row["gfx950"]:
+            assert f'name = "{ours}"' in text, ours
 
 
 def test_kernarg_image_built_two_ways_is_byte_identical():
