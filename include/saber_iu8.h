@@ -308,6 +308,20 @@ int saber_iu8_gemm_workspace(int wkind, uint32_t m, uint32_t n, uint32_t k, uint
 int saber_iu8_gemm(saber_iu8_ctx *ctx, int wkind, const void *a, const float *as, const void *w, const float *ws,
                    void *c_bf16, uint32_t m, uint32_t n, uint32_t k, void *partial, void *counter, void *stream);
 
+/* saber_iu8_gemm for callers that cannot allocate: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc between launches. No counterpart in the reference, whose host owns
+ * every allocation (include/saber_abi.h:163-174). The split-K workspaces of the launch (`partial`,
+ * `counter`) are not arguments: they live in one static device array of the library, 8 MiB of
+ * partials + 64 KiB of counters (saber_iu8_static_workspace_bytes), present once on every GPU a context
+ * was opened on and held until the process ends. Same kernels, same bytes as saber_iu8_gemm. Allocates,
+ * clears and synchronises nothing: the counters are zero from set-up and every kernel leaves them
+ * zero. A shape whose split needs more than the array holds is refused (SABER_IU8_E_RULE): use
+ * saber_iu8_gemm with caller-owned workspaces. All calls on one GPU share that GPU's array: calls
+ * that overlap in time on one GPU (different streams, no event between them) race on it. */
+int saber_iu8_gemm_static(saber_iu8_ctx *ctx, int wkind, const void *a, const float *as, const void *w, const float *ws,
+                          void *c_bf16, uint32_t m, uint32_t n, uint32_t k, void *stream);
+uint64_t saber_iu8_static_workspace_bytes(void);
+
 /* The raw int32 accumulators of the same GEMM (16 * sum(a*w) for W4, sum(a*w) for W8), int32
  * [m,n]: the parity tap. No counterpart in the reference's shipped object (its tests replay
  * captured bytes, crates/saber-kernels/hip/harness/run_hsaco.cpp:1-15). The tap kernels are not in

@@ -14,6 +14,7 @@
 #include "abi.h"
 #include "manifest.h"
 #include "rules.h"
+#include "static_ws.h"
 #include "util.h"
 
 using namespace iu8;
@@ -280,6 +281,9 @@ int saber_iu8_open(const char *prebuilt_dir, int device, saber_iu8_ctx **out) {
   }
   closedir(dp);
   std::sort(manifests.begin(), manifests.end());
+  // the library's static split-K workspace on this device (saber_iu8_gemm_static): its address is
+  // taken here, once a device, with the device current
+  if (int rc = static_ws_init(device)) return rc;
   saber_iu8_ctx *ctx = new saber_iu8_ctx();
   ctx->device = device;
   ctx->arch = arch;
@@ -423,6 +427,31 @@ int saber_iu8_gemm(saber_iu8_ctx *ctx, int wkind, const void *a, const float *as
   if (int rc = resolve(wkind, m, n, k, &d)) return rc;
   return launch_gemm(ctx, d, a, as, w, ws, c, partial, counter, stream);
 }
+
+// saber_iu8_gemm with the split-K workspaces in the library's static device array: nothing is
+// allocated, cleared or synchronised here (the counters are zero from set-up and left zero by every
+// kernel that uses them; the partials are written before they are read).
+int saber_iu8_gemm_static(saber_iu8_ctx *ctx, int wkind, const void *a, const float *as, const void *w, const float *ws,
+                          void *c, uint32_t m, uint32_t n, uint32_t k, void *stream) {
+  if (!ctx) return fail(SABER_IU8_E_ARG, "gemm_static: null context");
+  saber_iu8_desc d;
+  if (int rc = resolve(wkind, m, n, k, &d)) return rc;
+  void *partial = nullptr, *counter = nullptr;
+  for (uint32_t i = 0; i < d.n_workspaces; ++i) {
+    const saber_iu8_workspace &wsp = d.workspaces[i];
+    const bool is_partial = !strcmp(wsp.name, "decode_partial");
+    const uint64_t cap = is_partial ? STATIC_WS_PARTIAL_BYTES : STATIC_WS_COUNTER_BYTES;
+    if (wsp.bytes > cap)
+      return fail(SABER_IU8_E_RULE, fmt("gemm_static: %u x %u x %u needs %llu B of `%s`, the static workspace holds %llu; use saber_iu8_gemm "
+                                        "with caller-owned workspaces", m, n, k, (unsigned long long)wsp.bytes, wsp.name, (unsigned long long)cap));
+    (is_partial ? partial : counter) = is_partial ? static_ws_partial(ctx->device) : static_ws_counter(ctx->device);
+  }
+  if (d.n_workspaces && (!partial || !counter))
+    return fail(SABER_IU8_E_NOTLOADED, fmt("gemm_static: the static workspace of device %d was not set up", ctx->device));
+  return launch_gemm(ctx, d, a, as, w, ws, c, partial, counter, stream);
+}
+
+uint64_t saber_iu8_static_workspace_bytes(void) { return STATIC_WS_BYTES; }
 
 // Two W4 linears on one activation operand in one dispatch (decode band; the launch law's own
 // descriptors, which do not split K, so no workspace is bound).

@@ -67,8 +67,22 @@ def _run(cmd):
 
 
 def build_lib():
-    srcs = sorted(glob.glob(os.path.join(HOST, "*.cpp")))
-    _run([HIPCC, "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-o", LIB] + srcs + ["-I" + os.path.join(ROOT, "include")])
+    """Host sources as plain C++; the one file with device code (the static workspace array and its
+    fill kernel) as HIP for gfx950, its fat binary linked into the library."""
+    inc = "-I" + os.path.join(ROOT, "include")
+    objs = []
+    odir = os.path.join(PKG, "build")
+    os.makedirs(odir, exist_ok=True)
+    for src in sorted(glob.glob(os.path.join(HOST, "*.cpp"))):
+        obj = os.path.join(odir, os.path.basename(src) + ".o")
+        _run([HIPCC, "-x", "c++", "-O2", "-std=c++17", "-fPIC", "-Wall", "-D__HIP_PLATFORM_AMD__", "-I/opt/rocm/include", inc, "-c", src, "-o", obj])
+        objs.append(obj)
+    for src in sorted(glob.glob(os.path.join(HOST, "*.hip"))):
+        obj = os.path.join(odir, os.path.basename(src) + ".o")
+        _run([HIPCC, "-x", "hip", f"--offload-arch={ARCH}", "-O2", "-std=c++17", "-fPIC", "-Wall", "-Xclang", "-target-feature", "-Xclang",
+              "-packed-fp32-ops", inc, "-c", src, "-o", obj])
+        objs.append(obj)
+    _run([HIPCC, "-shared", "-fPIC", "-o", LIB] + objs)
     return LIB
 
 
