@@ -372,7 +372,7 @@ def main():
     # ---- the second half of the metric: int8 TOPS at M=2048 on the same four shapes. Activations are
     # the configuration's (bf16 N(0,1), 0.5 % of the channels x20), quantised by the producer kernel:
     # the operand values set the card's clock under MFMA load, so uniform random codes would misstate it.
-    def prefill_at(PM, warm, reps):
+    def prefill_at(PM, warm, reps, fused_too=False):
         pf = {}
         tot_ops, tot_us, tot_q_us = 0.0, 0.0, 0.0
         for name, n, k in linears:
@@ -407,6 +407,29 @@ def main():
             ops = 2.0 * PM * n * k
             pf[name] = dict(kernel=d.kernel.decode(), grid=list(d.grid), us=round(us, 2), tops=round(ops / us / 1e6, 1),
                             quant_us=round(q_us, 2))
+            if fused_too:
+                # the north_star's form, measured beside it: row scales (a pass that stores no codes) + the tile GEMM
+                # that quantises on the way into its A stage (macaq_iu8_pfq_*); same bytes, see tests/test_gpu_pfq.py
+                fd = iu8.resolve_prefill_fused(iu8.W4, PM, n, k)
+                fbs = []
+                for layer in range(LAYERS):
+                    fb = dict(x=x.data_ptr(), w=dev_w[name][layer].data_ptr(), ws=dev_ws[name].data_ptr(), c=c.data_ptr())
+                    fb["as"] = a_s.data_ptr()
+                    fbs.append(fb)
+                with torch.cuda.stream(stream):
+                    for i in range(max(reps, warm // 4)):
+                        ctx.launch(fd, fbs[i % LAYERS], sh)
+                    f0, f1, f2 = (torch.cuda.Event(enable_timing=True) for _ in range(3))
+                    f0.record(stream)
+                    for _ in range(reps):
+                        ctx.rowscale(x.data_ptr(), a_s.data_ptr(), PM, k, sh)
+                    f1.record(stream)
+                    for i in range(reps):
+                        ctx.launch(fd, fbs[i % LAYERS], sh)
+                    f2.record(stream)
+                torch.cuda.synchronize()
+                pf[name]["fused_quant"] = dict(kernel=fd.kernel.decode(), rowscale_us=round(f0.elapsed_time(f1) * 1e3 / reps, 2),
+                                               us=round(f1.elapsed_time(f2) * 1e3 / reps, 2))
             tot_ops += ops
             tot_us += us
             tot_q_us += q_us
@@ -414,8 +437,9 @@ def main():
         return pf, tot_ops, tot_us, tot_q_us
 
     if not args.no_prefill:
-        pf, tot_ops, tot_us, tot_q_us = prefill_at(2048, 600, 60)
+        pf, tot_ops, tot_us, tot_q_us = prefill_at(2048, 600, 60, fused_too=True)
         tops = tot_ops / tot_us / 1e6
+        fq_us = sum(v["fused_quant"]["us"] + v["fused_quant"]["rowscale_us"] for v in pf.values())
         # what the matrix cores sustain on this card with such operands: the register-resident MFMA
         # loop of the probe object, fed zeros, codes like this workload's (small activations, 16*w
         # weights) and uniform random bytes. The card is power-bound under MFMA load, so the rate
@@ -443,6 +467,9 @@ def main():
             torch.cuda.synchronize()
             probe[tag] = round(pblocks * 4 * piters * 16 * 65536.0 / (e0.elapsed_time(e1) * 1e3) / 1e6, 1)
         out["prefill_m2048"] = dict(value=round(tops, 1), unit="TOPS", with_quant=round(tot_ops / (tot_us + tot_q_us) / 1e6, 1),
+                                    fused_quant=dict(tops=round(tot_ops / fq_us / 1e6, 1), vs_two_launch=round((tot_us + tot_q_us) / fq_us, 3),
+                                                     note="row-scale pass + macaq_iu8_pfq_* (quantisation fused into the A-tile load), "
+                                                          "per linear under per_linear.*.fused_quant; the launch law keeps producer + GEMM"),
                                     per_linear=pf, mfma_probe_tops=probe,
                                     frac_of_probe_workload_like=round(tops / probe["workload_like"], 4),
                                     roofline=dict(bound="mfma", achieved=round(tops / 1e3, 4), peak=INT8_PEAK_TOPS / 1e3,

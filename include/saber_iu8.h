@@ -296,6 +296,18 @@ int saber_iu8_resolve_fused(int wkind, uint32_t m, uint32_t n, uint32_t k, saber
 int saber_iu8_linear_fused(saber_iu8_ctx *ctx, int wkind, const void *x_bf16, const void *w, const float *ws,
                            void *c_bf16, void *q, float *scale, uint32_t m, uint32_t n, uint32_t k, void *stream);
 
+/* The tile GEMM with the per-token quantisation fused into its A-tile load (kernels macaq_iu8_pfq_*):
+ * x bf16 [m,k] and the rows' scales a_scale f32 [m] -- from saber_iu8_rowscale (the producer's scale
+ * without its codes) or carried from whatever made the rows -- instead of stored codes; c holds the
+ * bytes of saber_iu8_quant + saber_iu8_gemm. No counterpart among the reference's symbols: its
+ * prefill tile reads codes a producer stored (crates/saber-kernels/hip/macaq_iu8.hip:174-280,
+ * producers hip/mxfp4_hadi8.hip:22-58). saber_iu8_resolve_prefill_fused picks the cell; any
+ * macaq_iu8_pfq_* kernel is reachable through saber_iu8_describe by name. */
+int saber_iu8_rowscale(saber_iu8_ctx *ctx, const void *x_bf16, float *scale, uint32_t m, uint32_t k, void *stream);
+int saber_iu8_resolve_prefill_fused(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *out);
+int saber_iu8_linear_prefill_fused(saber_iu8_ctx *ctx, int wkind, const void *x_bf16, const float *a_scale, const void *w,
+                                   const float *w_scale, void *c_bf16, uint32_t m, uint32_t n, uint32_t k, void *stream);
+
 /* Workspace bytes the resolved GEMM needs (both 0 when it does not split). Ask before every
  * saber_iu8_gemm of a new shape: the law splits K in one band (K >= 16384, 49..128 rows, few tiles),
  * and such a launch with `partial` / `counter` NULL is refused (SABER_IU8_E_ARG). */

@@ -22,6 +22,9 @@ static const Signature SIG_PAIR = {{"a", K::Buffer},  {"as", K::Buffer}, {"w", K
                                    {"nb_b", K::I32}};
 static const Signature SIG_PF = {{"a", K::Buffer}, {"w", K::Buffer}, {"as", K::Buffer}, {"ws", K::Buffer},
                                  {"c", K::Buffer}, {"m", K::I32},    {"n", K::I32},     {"k", K::I32}};
+static const Signature SIG_PFQ = {{"x", K::Buffer}, {"w", K::Buffer}, {"as", K::Buffer}, {"ws", K::Buffer},
+                                  {"c", K::Buffer}, {"m", K::I32},    {"n", K::I32},     {"k", K::I32}};
+static const Signature SIG_ROWSCALE = {{"x", K::Buffer}, {"scale", K::Buffer}, {"k", K::I32}};
 static const Signature SIG_QUANT = {{"x", K::Buffer}, {"q", K::Buffer}, {"scale", K::Buffer}, {"k", K::I32}};
 static const Signature SIG_QUANT_ROWS = {{"x", K::Buffer}, {"q", K::Buffer},       {"scale", K::Buffer},
                                          {"k", K::I32},    {"row_tok", K::Buffer}, {"meta", K::Buffer}};
@@ -73,6 +76,8 @@ static bool starts(const std::string &s, const char *p) { return s.rfind(p, 0) =
 const Signature *signature_for(const std::string &k) {
   if (starts(k, "macaq_iu8_dec_")) return &SIG_DEC;
   if (starts(k, "macaq_iu8_decq_")) return &SIG_DECQ;
+  if (starts(k, "macaq_iu8_pfq_")) return &SIG_PFQ;
+  if (starts(k, "macaq_i8_rowscale_")) return &SIG_ROWSCALE;
   if (starts(k, "macaq_iu8_pf_")) return k.size() > 3 && k.compare(k.size() - 3, 3, "_ks") == 0 ? &SIG_DEC : &SIG_PF;
   if (starts(k, "macaq_iu8f_pair_") || starts(k, "macaq_iu8f_pairb_")) return &SIG_PAIR;
   if (starts(k, "add_rms_quant_hadi8_")) return &SIG_HAD_ARQ;

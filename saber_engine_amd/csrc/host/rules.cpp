@@ -186,6 +186,22 @@ int describe(const std::string &kernel, uint32_t m, uint32_t n, uint32_t k, uint
       if (!signature_for(kernel)) return fail(SABER_IU8_E_RULE, kernel + ": no such split form");
       return describe_pf(*v, m, n, k, ks, out);
     }
+  // the tile GEMM with the quantisation fused into its A-tile load: the geometry of the cell it names
+  if (kernel.rfind("macaq_iu8_pfq_", 0) == 0)
+    if (const PfVariant *v = pf_variant("macaq_iu8_pf_" + kernel.substr(14))) {
+      // the cells that have a fused-quant form (registers for the bf16 pieces in flight, whole A fragments a wave)
+      static const char *const PFQ[] = {"w4_t128x128", "w8_t128x128", "w4_t128x128_o2", "w4_t256x160", "w8_t256x160"};
+      bool has = false;
+      for (const char *c : PFQ) has = has || kernel.substr(14) == c;
+      if (!has || ks != 1) return fail(SABER_IU8_E_RULE, kernel + ": no such fused-quant form");
+      if ((uint64_t)m * k * 2 > 0xFFFFFFFFull) return fail(SABER_IU8_E_RULE, fmt("%s: %u rows of %u bf16 pass 4 GiB", kernel.c_str(), m, k));
+      if (int rc = describe_pf(*v, m, n, k, 0, out)) return rc;
+      copy_name(out->kernel, sizeof out->kernel, kernel);
+      copy_name(out->op, sizeof out->op, v->w8 ? "linear_i8a8_pfq" : "linear_i4a8_pfq");
+      if (int rc = fill_slots(kernel, out)) return rc;
+      set_i32(out, "m", m), set_i32(out, "n", n), set_i32(out, "k", k);
+      return 0;
+    }
   // a name of the reference's symbol set that this object does not carry (gfx1201 tile shapes): the
   // request is for the op at this shape, and the gfx950 law picks the cell
   int w8 = 0;
@@ -418,6 +434,21 @@ static std::string row_form(const char *base, uint32_t rows, uint32_t width) {
 
 int resolve_quant(uint32_t m, uint32_t k, saber_iu8_desc *out) {
   return describe_rows("quant_i8", row_form("macaq_i8_quant", m, k).c_str(), m, k, "k", out);
+}
+
+int resolve_rowscale(uint32_t m, uint32_t k, saber_iu8_desc *out) {
+  const uint32_t slots = (k + 4095) / 4096;
+  const std::string name = std::string("macaq_i8_rowscale_t256") + (slots <= 1 ? "_g1" : slots <= 2 ? "_g2" : "");
+  return describe_rows("rowscale_i8", name.c_str(), m, k, "k", out);
+}
+
+// The fused-quant tile GEMM of a shape: the 128 x 128 cell while few tiles would leave CUs idle on the
+// larger one, else the 256 x 160 cell (the widest whose registers hold the bf16 pieces in flight).
+int resolve_prefill_fused(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *out) {
+  if (wkind != SABER_IU8_W4 && wkind != SABER_IU8_W8) return fail(SABER_IU8_E_ARG, "unknown weight kind");
+  const char *tag = wkind == SABER_IU8_W8 ? "w8" : "w4";
+  const uint64_t big = (uint64_t)((m + 255) / 256) * ((n + 159) / 160);
+  return describe(fmt("macaq_iu8_pfq_%s_%s", tag, big >= CU_COUNT ? "t256x160" : "t128x128"), m, n, k, 1, out);
 }
 
 int resolve_quant_rowmajor(uint32_t m, uint32_t k, saber_iu8_desc *out) {

@@ -47,6 +47,9 @@ int resolve_quant(uint32_t m, uint32_t k, saber_iu8_desc *out);
 bool fused_holds(uint32_t m, uint32_t k);
 int resolve_fused(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *out);
 int resolve_silu_mul_quant(uint32_t rows, uint32_t n, saber_iu8_desc *out);
+// The rows' scales alone, and the tile GEMM that makes the codes itself from bf16 rows + scales.
+int resolve_rowscale(uint32_t m, uint32_t k, saber_iu8_desc *out);
+int resolve_prefill_fused(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *out);
 // Quantisation to row-major codes (q[row * k + col]).
 int resolve_quant_rowmajor(uint32_t m, uint32_t k, saber_iu8_desc *out);
 // Quantisation through a row map (output row r = input row row_tok[r]).

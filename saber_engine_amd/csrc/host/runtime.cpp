@@ -401,6 +401,26 @@ int saber_iu8_linear_fused(saber_iu8_ctx *ctx, int wkind, const void *x, const v
   return saber_iu8_launch(ctx, &d, b, 6, stream);
 }
 
+int saber_iu8_rowscale(saber_iu8_ctx *ctx, const void *x, float *scale, uint32_t m, uint32_t k, void *stream) {
+  saber_iu8_desc d;
+  if (int rc = resolve_rowscale(m, k, &d)) return rc;
+  const saber_iu8_binding b[] = {{"x", (void *)x}, {"scale", scale}};
+  return saber_iu8_launch(ctx, &d, b, 2, stream);
+}
+
+int saber_iu8_resolve_prefill_fused(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *out) {
+  if (!out) return fail(SABER_IU8_E_ARG, "resolve_prefill_fused: null descriptor");
+  return resolve_prefill_fused(wkind, m, n, k, out);
+}
+
+int saber_iu8_linear_prefill_fused(saber_iu8_ctx *ctx, int wkind, const void *x, const float *as, const void *w, const float *ws,
+                                   void *c, uint32_t m, uint32_t n, uint32_t k, void *stream) {
+  saber_iu8_desc d;
+  if (int rc = resolve_prefill_fused(wkind, m, n, k, &d)) return rc;
+  const saber_iu8_binding b[] = {{"x", (void *)x}, {"w", (void *)w}, {"as", (void *)as}, {"ws", (void *)ws}, {"c", c}};
+  return saber_iu8_launch(ctx, &d, b, 5, stream);
+}
+
 int saber_iu8_gemm_workspace(int wkind, uint32_t m, uint32_t n, uint32_t k, uint64_t *partial_bytes, uint64_t *counter_bytes) {
   saber_iu8_desc d;
   if (int rc = resolve(wkind, m, n, k, &d)) return rc;

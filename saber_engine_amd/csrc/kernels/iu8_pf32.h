@@ -96,7 +96,15 @@ constexpr int iu8_pf32_lds_bytes() {
 // all past the tile's rows, or all but the first, runs the K loop in a form with none, or one, of
 // its TM row blocks -- the same loads, barriers and stage walk, a fraction of the MFMAs and LDS reads
 // -- so such a tile costs its operand traffic instead of a full tile's matrix work.
-template <bool W8, int WMW, int WNW, int TM, int TN, bool ACC, int STMAX, bool DEEP = false, bool SPARSE = false, bool ARM = false, bool EXT_LDS = false, class TileAt>
+//
+// AQ (the per-token quantisation fused into the A-tile load): A is the bf16 activation matrix itself,
+// row-major [M, K], and `as` holds the rows' scales (max(amax / 127, 1e-30), from a row-maximum pass
+// or carried from the producer of the rows). The A fragments of a step cannot go to LDS by LDS-DMA
+// then: each wave loads the bf16 pieces of its fragments into registers a step ahead (32 bytes a lane
+// a fragment), turns them into codes by the law's own routine (iu8_code4_rcp: the bytes of the
+// producer kernel) one step later and writes the fragment into its stage; the weights keep their
+// LDS-DMA stream. One conversion a workgroup and step, whatever the columns of the tile.
+template <bool W8, int WMW, int WNW, int TM, int TN, bool ACC, int STMAX, bool DEEP = false, bool SPARSE = false, bool ARM = false, bool EXT_LDS = false, bool AQ = false, class TileAt>
 __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const float *__restrict__ as,
                                              void *__restrict__ Cv, int N, int K, TileAt tile_at,
                                              int *__restrict__ P = nullptr, int *__restrict__ cnt = nullptr,
@@ -109,7 +117,8 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
   // a wave moves whole 1-KiB fragments: wave w moves fragments w, w + NWAVE, ... of A and of W
   constexpr int A_FR = A_BYTES / 1024, W_FR = W_BYTES / 1024;
   constexpr int A_PER = (A_FR + NWAVE - 1) / NWAVE, W_PER = (W_FR + NWAVE - 1) / NWAVE;
-  constexpr int PER = A_FR / NWAVE + W_FR / NWAVE;  // wave-loads every wave issues a step (some issue one more)
+  // wave-loads every wave issues a step (some issue one more); AQ: two 16-byte loads a fragment of A
+  constexpr int PER = (AQ ? 2 : 1) * (A_FR / NWAVE) + W_FR / NWAVE;
   // as many stages as asked for and as fit the 160 KiB of LDS, at least two
   constexpr int NFIT = 160 * 1024 / STAGE;
   constexpr int NST = STMAX < 2 ? 2 : (STMAX < NFIT ? STMAX : (NFIT < 2 ? 2 : NFIT));
@@ -118,6 +127,7 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
   static_assert((NST - 2) * (PER + (A_X > 0) + (W_X > 0)) <= 63, "the in-flight count fits s_waitcnt's vmcnt field");
   static_assert(!DEEP || NST >= 3, "the deep form reads a stage a step ahead of its MFMAs");
   static_assert(!(DEEP && SPARSE), "the sparse forms exist for the phased loop only");
+  static_assert(!AQ || (!DEEP && !SPARSE && !ARM && A_FR % NWAVE == 0), "the fused-quant form: phased loop, whole A fragments a wave");
   // EXT_LDS: the stages live in the caller's LDS block (1-KiB aligned, iu8_pf32_lds_bytes of this cell),
   // for a kernel that runs two cells one after the other in the same memory
   iu8_u8 *smem;
@@ -152,12 +162,17 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
   if (!tile_at(0, L)) return;
   int lr = 0, ls = s_lo;
   unsigned ga[A_PER], gw[W_PER], gaN[A_PER], gwN[W_PER];
-  auto addr_of = [&](const iu8_tile &t, unsigned (&oa)[A_PER], unsigned (&ow)[W_PER]) {
+  // AQ: the scale of this lane's row in every fragment, for the stream's tile and the one after it
+  float qs[AQ ? A_PER : 1], qsN[AQ ? A_PER : 1];
+  auto addr_of = [&](const iu8_tile &t, unsigned (&oa)[A_PER], unsigned (&ow)[W_PER], float (&os)[AQ ? A_PER : 1]) {
 #pragma unroll
     for (int p = 0; p < A_PER; ++p) {
       const int f = min(p * NWAVE + wave, A_FR - 1);  // fragment (mt = f/2, kt2 = f%2) of the step
       const int ar = iu8_arow(t.R, t.mbase + (f >> 1) * 16 + (lane & 15));  // rows past the edge: the last one
-      if constexpr (ARM) oa[p] = (unsigned)((size_t)ar * K + (f & 1) * 64 + (lane >> 4) * 16);
+      if constexpr (AQ) {  // bf16 rows: 2 bytes an element
+        oa[p] = (unsigned)(((size_t)ar * K + (f & 1) * 64 + (lane >> 4) * 16) * 2);
+        os[p] = as[ar];
+      } else if constexpr (ARM) oa[p] = (unsigned)((size_t)ar * K + (f & 1) * 64 + (lane >> 4) * 16);
       else oa[p] = (unsigned)(((size_t)(ar >> 4) * ktiles + (f & 1)) * 1024 + ((ar & 15) + 16 * (lane >> 4)) * 16);
     }
 #pragma unroll
@@ -167,11 +182,11 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
       ow[p] = (unsigned)((size_t)nt * ksteps * WSTEP + (f % (WSTEP / 1024)) * 1024 + lane * 16);
     }
   };
-  addr_of(L, ga, gw);
+  addr_of(L, ga, gw, qs);
   // The next tile's descriptor and addresses (a gathered tile reads its row map for them) are
   // fetched a whole tile ahead, so the stream never waits for them when it crosses into that tile.
   bool haveN = tile_at(1, Nx);
-  if (haveN) addr_of(Nx, gaN, gwN);
+  if (haveN) addr_of(Nx, gaN, gwN, qsN);
   // The load is written as asm: the compiler models an LDS-DMA load as touching both memories and
   // then drains every counter to zero at each later LDS read, which would serialise the operand
   // pipeline below. Its completion is tracked by hand (vmcnt, before the step's barrier).
@@ -183,17 +198,63 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
                  : "memory", "m0");
   };
   const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) iu8_u8 *)smem;
-  auto issue = [&](int stage) {  // the load stream's step -> LDS stage
-    const unsigned sA = lds0 + stage * STAGE, sW = sA + A_BYTES;
+  // AQ: the bf16 pieces of every fragment of A this wave owns (two 16-byte loads a fragment) and the
+  // scale of their rows. Fragment p is loaded in phase p % 3 of a step, right behind the conversion of
+  // the pieces it replaces, and converted a whole step later: a step of latency cover, one register
+  // set. Loads return in order, so the compiler's own wait for a fragment's pieces also vouches for
+  // every DMA issued before them.
+  iu8_v4u aq[AQ ? A_PER : 1][2];
+  float aq_sc[AQ ? A_PER : 1];
+  auto step_k = [&]() {
     int kk = ls + L.rot;
     if (kk >= s_hi) kk -= s_hi - s_lo;
+    return kk;
+  };
+  auto issue = [&](int stage) {  // the load stream's step -> LDS stage
+    const unsigned sA = lds0 + stage * STAGE, sW = sA + A_BYTES;
+    const int kk = step_k();
     const iu8_u8 *As = A + (size_t)kk * (ARM ? 128 : 2048), *Ws = L.W + (size_t)kk * WSTEP;
+    if constexpr (!AQ) {
 #pragma unroll
-    for (int p = 0; p < A_PER; ++p)
-      if (A_FR % NWAVE == 0 || p * NWAVE + wave < A_FR) dma(As, ga[p], sA + (p * NWAVE + wave) * 1024);
+      for (int p = 0; p < A_PER; ++p)
+        if (A_FR % NWAVE == 0 || p * NWAVE + wave < A_FR) dma(As, ga[p], sA + (p * NWAVE + wave) * 1024);
+    }
 #pragma unroll
     for (int p = 0; p < W_PER; ++p)
       if (W_FR % NWAVE == 0 || p * NWAVE + wave < W_FR) dma(Ws, gw[p], sW + (p * NWAVE + wave) * 1024);
+  };
+  auto aq_load = [&](int p) {  // fragment p of the load stream's step into registers
+    if constexpr (AQ) {
+      const iu8_u8 *As = A + (size_t)step_k() * 256;
+      aq[p][0] = *(const iu8_v4u *)(As + ga[p]);
+      aq[p][1] = *(const iu8_v4u *)(As + ga[p] + 16);
+      aq_sc[p] = qs[p];
+    }
+  };
+  auto aq_commit = [&](int p, int stage) {  // the pieces of fragment p -> codes -> the fragment in `stage`
+    if constexpr (AQ) {
+      const float sc = aq_sc[p], rcp = __fdiv_rn(1.f, sc);
+      unsigned d[4];
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int w = 0; w < 2; ++w) {
+          const unsigned u0 = aq[p][h][2 * w], u1 = aq[p][h][2 * w + 1];
+          d[h * 2 + w] = iu8_code4_rcp(__uint_as_float(u0 << 16), __uint_as_float(u0 & 0xFFFF0000u), __uint_as_float(u1 << 16),
+                                       __uint_as_float(u1 & 0xFFFF0000u), sc, rcp);
+        }
+      *(iu8_v4u *)&smem[stage * STAGE + (p * NWAVE + wave) * 1024 + lane * 16] = iu8_v4u{d[0], d[1], d[2], d[3]};
+    }
+  };
+  // phase ph of a step: the fragments p = ph, ph + 3, ... are converted into stage `cst`, then re-loaded
+  auto aq_phase = [&](int ph, int cst) {
+    if constexpr (AQ) {
+#pragma unroll
+      for (int p = ph; p < A_PER; p += 3) {
+        aq_commit(p, cst);
+        aq_load(p);
+      }
+    }
   };
   auto advance = [&]() {  // next step of the stream; past the last tile it keeps re-loading the last step
     if (++ls == s_hi) {
@@ -203,8 +264,12 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
         for (int p = 0; p < A_PER; ++p) ga[p] = gaN[p];
 #pragma unroll
         for (int p = 0; p < W_PER; ++p) gw[p] = gwN[p];
+        if constexpr (AQ) {
+#pragma unroll
+          for (int p = 0; p < A_PER; ++p) qs[p] = qsN[p];
+        }
         haveN = tile_at(lr + 1, Nx);
-        if (haveN) addr_of(Nx, gaN, gwN);
+        if (haveN) addr_of(Nx, gaN, gwN, qsN);
       } else {
         ls = s_hi - 1;
       }
@@ -299,8 +364,17 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
 #pragma unroll
   for (int s0 = 0; s0 < NST - 1; ++s0) {
     issue(s0);
+    if constexpr (AQ) {  // the last step issued here stays in registers for the first step's phases
+#pragma unroll
+      for (int p = 0; p < A_PER; ++p) aq_load(p);
+      if (s0 < NST - 2) {
+#pragma unroll
+        for (int p = 0; p < A_PER; ++p) aq_commit(p, s0);
+      }
+    }
     advance();
   }
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   wait_step(false);
   __builtin_amdgcn_s_barrier();
   // deep form: register sets of one whole step, [set][sub-step f = 2p + kt2]
@@ -421,17 +495,27 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
             fetch_w8(sW, 1, 0, 1);
             fetch_w4(sW, 1);
           }
-          issue(stl);
+          // AQ: the pieces loaded a step ago become fragments of the stage NST-1 steps ahead (the one
+          // this step's DMA of the weights is for... a step later: the loads ran one step behind it)
+          const int cst = st + NST - 2 >= NST ? st - 2 : st + NST - 2;
+          if constexpr (!AQ) issue(stl);
+          aq_phase(0, cst);
           mfmas(0, 0, 0, nl);
           IU8_PHASE_ORDER(NL + NW, NL);
           // phase 1
           fetch_a(sA, 0, 1, 0, nl);
           if constexpr (NL > 0) fetch_w8(sW, 0, 1, 0);
+          aq_phase(1, cst);
           mfmas(1, 0, 1, nl);
           IU8_PHASE_ORDER(NL + (W8 ? NW : 0), NL);
           // phase 2
           fetch_a(sA, 1, 1, 1, nl);
           if constexpr (NL > 0) fetch_w8(sW, 1, 1, 1);
+          aq_phase(2, cst);
+          // AQ: the weights' DMA leaves behind the step's last register load. The compiler counts its own
+          // loads only, so its wait for a fragment's pieces asks for as many more of the oldest loads as
+          // DMAs were issued since; in this order those are register loads of a step ago, not a fresh DMA.
+          if constexpr (AQ) issue(stl);
           mfmas(0, 1, 0, nl);
           IU8_PHASE_ORDER(NL + (W8 ? NW : 0), NL);
           // phase 3, behind the barrier: every wave's reads of this stage are done and the next step's

@@ -5,6 +5,7 @@
 // A fragment order (iu8_common.h), scale f32 per row.
 //
 //   macaq_i8_quant_t256           x bf16 [M,K] -> q, scale                 (grid M, block 256)
+//   macaq_i8_rowscale_t256        the rows' scales alone (the pass in front of macaq_iu8_pfq_*)
 //   macaq_i8_quant_rm_t256        the same with the codes row-major, q[row * K + col] (the operand a
 //                                 grouped GEMM gathers whole token rows from)
 //   macaq_i8_quant_rows_t256      the first through a row map: output row r = input row row_tok[r]
@@ -49,7 +50,8 @@ static __device__ __forceinline__ float i8q_block_max(float v) {
 }
 
 // codes of one row from v[g][16] (f32 values), written in A fragment order (RM: row-major, K bytes a row)
-template <int I8Q_MAXG, bool RM = false>
+// SCALE_ONLY: the row's scale alone (the row-maximum pass in front of a GEMM that makes the codes itself)
+template <int I8Q_MAXG, bool RM = false, bool SCALE_ONLY = false>
 static __device__ __forceinline__ void i8q_tail(float (&v)[I8Q_MAXG][16], int G, iu8_u8 *__restrict__ q,
                                                 float *__restrict__ scale, int row, int K) {
   const int tid = threadIdx.x;
@@ -64,6 +66,7 @@ static __device__ __forceinline__ void i8q_tail(float (&v)[I8Q_MAXG][16], int G,
   const float sc = fmaxf(__fdiv_rn(amax, 127.f), 1e-30f);
   const float rcp = __fdiv_rn(1.f, sc);
   if (tid == 0) scale[row] = sc;
+  if constexpr (SCALE_ONLY) return;
   iu8_u8 *qrow = q + (size_t)(row >> 4) * (K >> 6) * 1024 + (row & 15) * 16;
 #pragma unroll
   for (int i = 0; i < I8Q_MAXG; ++i) {
@@ -82,7 +85,7 @@ static __device__ __forceinline__ void i8q_tail(float (&v)[I8Q_MAXG][16], int G,
 // `row_tok` / `meta` (optional, may be null): with them output row r is the quantised input row
 // row_tok[r] (the expert-major rows of a routed layer, gathered here once so that the grouped GEMM
 // reads whole fragments); pad rows (row_tok < 0) and rows past meta[1] are skipped.
-template <int I8Q_MAXG, bool RM = false>
+template <int I8Q_MAXG, bool RM = false, bool SCALE_ONLY = false>
 static __device__ __forceinline__ void i8q_quant_body(const unsigned short *__restrict__ x, unsigned char *__restrict__ q,
                                                       float *__restrict__ scale, int k,
                                                       const int *__restrict__ row_tok = nullptr,
@@ -109,7 +112,7 @@ static __device__ __forceinline__ void i8q_quant_body(const unsigned short *__re
       v[i][8 + 2 * w + 1] = __uint_as_float(hi[w] & 0xFFFF0000u);
     }
   }
-  i8q_tail<I8Q_MAXG, RM>(v, G, q, scale, row, k);
+  i8q_tail<I8Q_MAXG, RM, SCALE_ONLY>(v, G, q, scale, row, k);
 }
 #define I8Q_QUANT(name, MAXG)                                                                                   \
   extern "C" __global__ __launch_bounds__(I8Q_T) void name(const unsigned short *__restrict__ x,                \
@@ -122,6 +125,16 @@ I8Q_QUANT(macaq_i8_quant_t256_g5, 5)
 I8Q_QUANT(macaq_i8_quant_t256_g2, 2)
 I8Q_QUANT(macaq_i8_quant_t256_g1, 1)
 #undef I8Q_QUANT
+// the rows' scales alone: x bf16 [M, K] -> scale f32 [M] (what macaq_i8_quant_* stores beside its codes)
+#define I8Q_ROWSCALE(name, MAXG)                                                                                \
+  extern "C" __global__ __launch_bounds__(I8Q_T) void name(const unsigned short *__restrict__ x,                \
+                                                           float *__restrict__ scale, int k) {                  \
+    i8q_quant_body<MAXG, false, true>(x, nullptr, scale, k);                                                    \
+  }
+I8Q_ROWSCALE(macaq_i8_rowscale_t256, 8)
+I8Q_ROWSCALE(macaq_i8_rowscale_t256_g2, 2)
+I8Q_ROWSCALE(macaq_i8_rowscale_t256_g1, 1)
+#undef I8Q_ROWSCALE
 // row-major codes (q[row * k + col]): the operand a routed layer's grouped GEMM gathers token rows from
 #define I8Q_QUANT_RM(name, MAXG)                                                                                \
   extern "C" __global__ __launch_bounds__(I8Q_T) void name(const unsigned short *__restrict__ x,                \

@@ -83,3 +83,38 @@ IU8_PF32K(macaq_iu8_pf_w4_t64x128_s_ks, false, 2, 2, 1, 2, 5, 2, true)
 #undef IU8_PF32K
 #define IU8_PF_VARIANT(name, W8, WMW, WNW, TM, TN, ACC, ST, OCC, DEEP) IU8_PF32(name, W8, WMW, WNW, TM, TN, ACC, ST, OCC, DEEP)
 #include "iu8_variants.def"
+
+// The tile GEMM with the per-token quantisation fused into its A-tile load (symbols `macaq_iu8_pfq_*`,
+// the cell named by the suffix): `x` is the bf16 activation matrix [m, k] itself, `as` the rows' scales
+// (macaq_i8_rowscale_*, or carried from the producer of the rows); the codes are made on the way into
+// the A stage by the routine the producer kernel uses, so c holds the bytes of producer + GEMM. No
+// counterpart among the reference's symbols: its prefill reads codes a producer stored
+// (crates/saber-kernels/hip/macaq_iu8.hip:174-280). The conversion is VALU work that shares the
+// CU with the MFMAs -- about 11 * BM wave instructions a step against BM * BN / 32 MFMA cycles a SIMD --
+// and measured on this card the fused cells take 2.3-3.1x the time of their plain twins (1.8-3.8x of
+// producer + the law's GEMM over the four 27B-class shapes at 256, 2048 and 8192 rows), so the launch law
+// does not pick them: they are kept, tested and reachable by name. The 256 x 256 cell has no registers
+// left for the pieces in flight (it spilt, and still was the least slow at 2.05-2.3x), so it has no
+// fused form here.
+#define IU8_PFQ(name, W8, WMW, WNW, TM, TN, ST, OCC)                                                               \
+  extern "C" __global__ __launch_bounds__(WMW * WNW * 64)                                                         \
+      __attribute__((amdgpu_waves_per_eu(WMW * WNW * OCC / 4, WMW * WNW * OCC / 4))) void name(                    \
+      const unsigned short *__restrict__ x, const unsigned char *__restrict__ w, const float *__restrict__ as,    \
+      const float *__restrict__ ws, unsigned short *__restrict__ c, int m, int n, int k) {                         \
+    constexpr int BM = WMW * TM * 32, BN = WNW * TN * 32;                                                          \
+    const int gx = (n + BN - 1) / BN, gy = (m + BM - 1) / BM;                                                      \
+    const iu8_rows R{nullptr, 0, m};                                                                               \
+    iu8_pf32_run<W8, WMW, WNW, TM, TN, false, ST, false, false, false, false, true>(                               \
+        (const iu8_u8 *)x, as, c, n, k, [&](int r, iu8_tile &t) {                                                  \
+          int bx, by;                                                                                              \
+          if (!iu8_dense_tile_at(r, gx, gy, bx, by)) return false;                                                 \
+          t = iu8_tile{R, by * BM, bx * (BN / 16), w, ws, by * gx + bx};                                           \
+          return true;                                                                                             \
+        });                                                                                                        \
+  }
+IU8_PFQ(macaq_iu8_pfq_w4_t128x128, false, 4, 2, 1, 2, 3, 1)
+IU8_PFQ(macaq_iu8_pfq_w8_t128x128, true, 4, 2, 1, 2, 3, 1)
+IU8_PFQ(macaq_iu8_pfq_w4_t128x128_o2, false, 2, 2, 2, 2, 3, 2)
+IU8_PFQ(macaq_iu8_pfq_w4_t256x160, false, 8, 1, 1, 5, 3, 1)
+IU8_PFQ(macaq_iu8_pfq_w8_t256x160, true, 8, 1, 1, 5, 3, 1)
+#undef IU8_PFQ

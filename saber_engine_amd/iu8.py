@@ -110,6 +110,8 @@ def lib():
         L.saber_iu8_quant.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32, C.c_uint32, C.c_void_p]
         L.saber_iu8_quant_rowmajor.argtypes = L.saber_iu8_quant.argtypes
         L.saber_iu8_gemm.argtypes = [C.c_void_p, C.c_int] + [C.c_void_p] * 5 + [C.c_uint32] * 3 + [C.c_void_p] * 3
+        L.saber_iu8_rowscale.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32, C.c_uint32, C.c_void_p]
+        L.saber_iu8_linear_prefill_fused.argtypes = [C.c_void_p, C.c_int] + [C.c_void_p] * 5 + [C.c_uint32] * 3 + [C.c_void_p]
         L.saber_iu8_gemm_static.argtypes = [C.c_void_p, C.c_int] + [C.c_void_p] * 5 + [C.c_uint32] * 3 + [C.c_void_p]
         L.saber_iu8_static_workspace_bytes.restype = C.c_uint64
         L.saber_iu8_gemm_acc.argtypes = [C.c_void_p, C.c_int] + [C.c_void_p] * 3 + [C.c_uint32] * 3 + [C.c_void_p]
@@ -194,6 +196,12 @@ def fused_holds(m, k):
 def resolve_fused(wkind, m, n, k):
     d = Desc()
     _check(lib().saber_iu8_resolve_fused(wkind, m, n, k, C.byref(d)))
+    return d
+
+
+def resolve_prefill_fused(wkind, m, n, k):
+    d = Desc()
+    _check(lib().saber_iu8_resolve_prefill_fused(wkind, m, n, k, C.byref(d)))
     return d
 
 
@@ -338,6 +346,12 @@ class Context:
 
     def gemm(self, wkind, a, a_scale, w, w_scale, c, m, n, k, partial=None, counter=None, stream=0):
         _check(lib().saber_iu8_gemm(self._h, wkind, a, a_scale, w, w_scale, c, m, n, k, partial, counter, stream))
+
+    def rowscale(self, x, scale, m, k, stream=0):
+        _check(lib().saber_iu8_rowscale(self._h, x, scale, m, k, stream))
+
+    def linear_prefill_fused(self, wkind, x, a_scale, w, w_scale, c, m, n, k, stream=0):
+        _check(lib().saber_iu8_linear_prefill_fused(self._h, wkind, x, a_scale, w, w_scale, c, m, n, k, stream))
 
     def gemm_static(self, wkind, a, a_scale, w, w_scale, c, m, n, k, stream=0):
         """gemm() with the split-K workspaces in the library's static device array: allocates nothing."""

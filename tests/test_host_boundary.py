@@ -148,6 +148,21 @@ def test_reference_symbol_names_are_answered_by_the_law():
         iu8.describe("macaq_iu8f_pf_w4_bm128", 400, 5120, 17408, ks=2)
 
 
+def test_fused_quant_tile_gemm_descriptors():
+    """macaq_iu8_pfq_*: the geometry of the cell the suffix names, the pf kernarg list with `x` for `a`."""
+    d = iu8.describe("macaq_iu8_pfq_w4_t256x160", 2048, 5120, 17408)
+    u = iu8.describe("macaq_iu8_pf_w4_t256x160", 2048, 5120, 17408)
+    assert tuple(d.grid) == tuple(u.grid) and d.block[0] == u.block[0] == 512 and d.kernarg_bytes == 52 and d.op == b"linear_i4a8_pfq"
+    assert [d.args[i].name.decode() for i in range(d.n_args)] == ["x", "w", "as", "ws", "c", "m", "n", "k"]
+    assert iu8.resolve_prefill_fused(iu8.W4, 2048, 34816, 5120).kernel == b"macaq_iu8_pfq_w4_t256x160"
+    assert iu8.resolve_prefill_fused(iu8.W8, 256, 5120, 5120).kernel == b"macaq_iu8_pfq_w8_t128x128"
+    for bad in (lambda: iu8.describe("macaq_iu8_pfq_w4_t64x64_s", 256, 256, 256), lambda: iu8.describe("macaq_iu8_pfq_w4_t256x160", 256, 256, 256, ks=2),
+                lambda: iu8.resolve_prefill_fused(iu8.W4, 0, 256, 256), lambda: iu8.describe("macaq_iu8_pfq_w4_t128x128", 500000, 128, 5120)):
+        with pytest.raises(iu8.IU8Error) as e:
+            bad()
+        assert e.value.code == iu8.E_RULE
+
+
 def test_band_table_is_the_launch_law():
     """prebuilt/gfx950/macaq_iu8.band.toml (the law as data, the gfx950 counterpart of the reference's
     PF_BAND / PF_TILES tables, macaq_iu8.rs:150-212) is what the library writes today, and every row
