@@ -263,6 +263,60 @@ def main():
                                 frac_of_probe=round(nb / us / 1e3 / hbm_probe, 4), read_probe_us=round(pus, 2))
         del gl
 
+    # ---- the MLP of the step (gate+up -> SiLU * up + requantisation -> down) as ONE persistent launch
+    # (macaq_iu8f_mlp_w4_tm1) beside the three launches it replaces (fused linear, silu-mul-quant
+    # producer, GEMV), both as graphs walking the weight copies. More work than the step's two linears
+    # (the activation between them), so it is reported here and not part of `value`.
+    mlp = None
+    (_, n_gu, hid), (_, _, inter) = [l for l in linears if l[0] == "gate_up"][0], [l for l in linears if l[0] == "down"][0]
+    if fused and n_gu == 2 * inter and iu8.fused_holds(M, inter):
+        p_rows = torch.zeros((M, inter), dtype=torch.int16, device=dev)
+        state = torch.zeros(iu8.MLP_CHAIN_STATE_BYTES // 4, dtype=torch.int32, device=dev)
+        q_dn = torch.zeros(iu8.a_bytes(M, inter), dtype=torch.uint8, device=dev)
+        s_dn = torch.zeros(M, dtype=torch.float32, device=dev)
+        d_silu, d_dn = iu8.resolve_silu_mul_quant(M, inter), descs["down"]
+
+        def chain(layer):
+            ctx.mlp_chain(dev_x["gate_up"].data_ptr(), dev_w["gate_up"][layer].data_ptr(), dev_ws["gate_up"].data_ptr(),
+                          dev_w["down"][layer].data_ptr(), dev_ws["down"].data_ptr(), None, p_rows.data_ptr(), state.data_ptr(),
+                          dev_c["down"].data_ptr(), M, hid, inter, stream=sh)
+
+        def three(layer):
+            launch_fused("gate_up", layer)
+            ctx.launch(d_silu, dict(gu=dev_c["gate_up"].data_ptr(), q=q_dn.data_ptr(), scale=s_dn.data_ptr()), sh)
+            b = dict(a=q_dn.data_ptr(), w=dev_w["down"][layer].data_ptr(), ws=dev_ws["down"].data_ptr(), c=dev_c["down"].data_ptr(),
+                     decode_partial=partial.data_ptr(), decode_counter=counter.data_ptr())
+            b["as"] = s_dn.data_ptr()
+            ctx.launch(d_dn, b, sh)
+
+        times, bits = {}, {}
+        for tag, fn in (("three_launches", three), ("chain", chain)):
+            gl = torch.cuda.CUDAGraph()
+            with torch.cuda.stream(stream):
+                fn(0)
+            stream.synchronize()
+            with torch.cuda.graph(gl, stream=stream):
+                for i in range(K_steps):
+                    fn(i % LAYERS)
+            with torch.cuda.stream(stream):
+                gl.replay()
+                l0, l1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                l0.record(stream)
+                gl.replay()
+                l1.record(stream)
+            torch.cuda.synchronize()
+            times[tag] = l0.elapsed_time(l1) * 1e3 / K_steps
+            bits[tag] = dev_c["down"].clone()
+            del gl
+        wb = (n_gu * hid + hid * inter) // 2
+        mlp = dict(kernel="macaq_iu8f_mlp_w4_tm1", weight_bytes=wb, us_chain=round(times["chain"], 2),
+                   us_three_launches=round(times["three_launches"], 2),
+                   us_two_linears_alone=round(per_linear["gate_up"]["us"] + per_linear["down"]["us"], 2),
+                   gbps_chain=round(wb / times["chain"] / 1e3, 1), same_bytes=bool(torch.equal(bits["chain"], bits["three_launches"])),
+                   state_status=int(state[iu8.MLP_CHAIN_STATUS_OFFSET // 4].item()))
+        launch_fused("down", (K_steps - 1) % LAYERS)   # dev_c["down"] back to the step's own output for the spot check below
+        stream.synchronize()
+
     # ---- parity spot check against the CPU oracle, and the CPU baseline beside it
     out = dict(metric="W4A8 GEMM GB/s (%HBM) at M=1; int8 TOPS (%MFMA peak) at M=2048", value=round(value, 1), unit="GB/s",
                n_gpus=1, steps=K_steps, warmup=W_steps, ms_per_step=round(ms_per_step, 5), higher_is_better=True,
@@ -275,7 +329,7 @@ def main():
                            warm_cache_gbps=round(step_bytes / (warm_ms * 1e-3) / 1e9, 1),
                            hbm_frac_of_probe=round(value / hbm_probe, 4)),
                roofline=roofline)
-    out["decode_m%d" % M] = dict(per_linear=per_linear, note="one launch a linear, cold weights, graph replay; read_probe_us = a plain "
+    out["decode_m%d" % M] = dict(per_linear=per_linear, mlp_chain=mlp, note="one launch a linear, cold weights, graph replay; read_probe_us = a plain "
                                  "streaming read of the same weight bytes, cold the same way; down is the 5120x17408 GEMV")
 
     if not args.no_cpu:

@@ -296,6 +296,30 @@ int saber_iu8_resolve_fused(int wkind, uint32_t m, uint32_t n, uint32_t k, saber
 int saber_iu8_linear_fused(saber_iu8_ctx *ctx, int wkind, const void *x_bf16, const void *w, const float *ws,
                            void *c_bf16, void *q, float *scale, uint32_t m, uint32_t n, uint32_t k, void *stream);
 
+/* The dense decode MLP as ONE persistent launch: gate+up linear -> SiLU(gate) * up with its
+ * per-token requantisation -> down linear, for at most 4 rows whose codes fit the fused form at both
+ * widths (saber_iu8_fused_holds(m, hidden) and (m, inter)). The dense twin of the reference's routed
+ * back half, which chains gate_up -> silu-quant -> down in one persistent launch with device-counter
+ * hand-overs (crates/saber-kernels/hip/moe_grouped.hip:1656-1765, crates/saber-kernels/src/moe.rs:341-345);
+ * its dense MLP is three launches (crates/saber-kernels/src/macaq_iu8.rs:864-875), whose bytes this
+ * launch reproduces. x bf16 [m, hidden]; w_gu W4 [2*inter, hidden] (gate rows, then up rows) with
+ * ws_gu f32 [2*inter]; w_dn W4 [hidden, inter] with ws_dn f32 [hidden]; c bf16 [m, hidden].
+ * Workspaces (the descriptor lists them): gu bf16 [m, 2*inter] and p bf16 [m, inter], undefined at
+ * entry; state, SABER_IU8_MLP_CHAIN_STATE_BYTES, zero before the first launch: the workgroups meet
+ * through it (an arrival word a workgroup, stamped with a generation the kernel advances), and a
+ * launch that completes leaves it ready for the next. All workgroups must be resident at once: the
+ * launch is refused (SABER_IU8_E_RULE) on a device that does not hold the grid. A meeting waits at
+ * most `spin` polls (0: the default, about a second); a launch that gives up leaves a non-zero word
+ * at state + SABER_IU8_MLP_CHAIN_STATUS_OFFSET and an undefined c: after synchronising, a caller
+ * that shares the GPU with other work checks that word and, if set, zeroes `state` and runs the
+ * three launches. Launches that share one `state` must not overlap. Asynchronous. */
+#define SABER_IU8_MLP_CHAIN_STATE_BYTES (12 * 1024)
+#define SABER_IU8_MLP_CHAIN_STATUS_OFFSET (10 * 1024 + 8)
+int saber_iu8_resolve_mlp_chain(uint32_t m, uint32_t hidden, uint32_t inter, uint32_t spin, saber_iu8_desc *out);
+int saber_iu8_mlp_chain(saber_iu8_ctx *ctx, const void *x_bf16, const void *w_gu, const float *ws_gu, const void *w_dn,
+                        const float *ws_dn, void *gu, void *p, void *state, void *c, uint32_t m, uint32_t hidden, uint32_t inter,
+                        uint32_t spin, void *stream);
+
 /* The tile GEMM with the per-token quantisation fused into its A-tile load (kernels macaq_iu8_pfq_*):
  * x bf16 [m,k] and the rows' scales a_scale f32 [m] -- from saber_iu8_rowscale (the producer's scale
  * without its codes) or carried from whatever made the rows -- instead of stored codes; c holds the

@@ -20,6 +20,11 @@ static const Signature SIG_PAIR = {{"a", K::Buffer},  {"as", K::Buffer}, {"w", K
                                    {"c_b", K::Buffer}, {"m", K::I32},    {"k", K::I32},     {"n", K::I32},
                                    {"ks", K::I32},    {"nb", K::I32},    {"n_b", K::I32},   {"ks_b", K::I32},
                                    {"nb_b", K::I32}};
+// the decode MLP chain (no counterpart list in the reference: its dense MLP is three launches)
+static const Signature SIG_MLP = {{"x", K::Buffer},    {"w", K::Buffer},      {"ws", K::Buffer}, {"w_b", K::Buffer},
+                                  {"ws_b", K::Buffer}, {"gu", K::Buffer},     {"p", K::Buffer},  {"state", K::Buffer},
+                                  {"c", K::Buffer},    {"m", K::I32},         {"k", K::I32},     {"n", K::I32},
+                                  {"spin", K::I32}};
 static const Signature SIG_PF = {{"a", K::Buffer}, {"w", K::Buffer}, {"as", K::Buffer}, {"ws", K::Buffer},
                                  {"c", K::Buffer}, {"m", K::I32},    {"n", K::I32},     {"k", K::I32}};
 static const Signature SIG_PFQ = {{"x", K::Buffer}, {"w", K::Buffer}, {"as", K::Buffer}, {"ws", K::Buffer},
@@ -80,6 +85,7 @@ const Signature *signature_for(const std::string &k) {
   if (starts(k, "macaq_i8_rowscale_")) return &SIG_ROWSCALE;
   if (starts(k, "macaq_iu8_pf_")) return k.size() > 3 && k.compare(k.size() - 3, 3, "_ks") == 0 ? &SIG_DEC : &SIG_PF;
   if (starts(k, "macaq_iu8f_pair_") || starts(k, "macaq_iu8f_pairb_")) return &SIG_PAIR;
+  if (starts(k, "macaq_iu8f_mlp_")) return &SIG_MLP;
   if (starts(k, "add_rms_quant_hadi8_")) return &SIG_HAD_ARQ;
   if (starts(k, "silu_mul_quant_hadi8_")) return &SIG_HAD_SMQ;
   if (starts(k, "quant_hadi8_")) return &SIG_HAD_Q;

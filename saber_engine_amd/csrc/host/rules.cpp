@@ -424,6 +424,39 @@ int resolve_fused(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc 
   return 0;
 }
 
+// The decode MLP as one persistent launch (kernels/iu8_chain.h): both linears in the fused form's
+// bounds, every workgroup resident at once (two a CU: the runtime checks what the card really
+// holds), at most 8 column blocks of either linear a workgroup.
+int resolve_mlp_chain(uint32_t m, uint32_t hidden, uint32_t inter, uint32_t spin, saber_iu8_desc *d) {
+  const char *op = "mlp_chain_i4a8";
+  if (inter > 0x3FFFFFFFu) return fail(SABER_IU8_E_RULE, fmt("%s: intermediate width %u", op, inter));
+  if (int rc = check_shape(op, m, 2 * inter, hidden)) return rc;
+  if (int rc = check_shape(op, m, hidden, inter)) return rc;
+  if (!fused_holds(m, hidden) || !fused_holds(m, inter))
+    return fail(SABER_IU8_E_RULE, fmt("%s: %u rows of %u / %u do not fit the fused form (at most 4 rows, 20 KiB of codes)", op, m,
+                                      hidden, inter));
+  const uint32_t grid = 2 * CU_COUNT, nblk = std::max((2 * inter + 31) / 32, (hidden + 31) / 32);
+  if (nblk > 8 * grid)
+    return fail(SABER_IU8_E_RULE, fmt("%s: %u column blocks are more than the %u resident workgroups walk (8 each)", op, nblk, grid));
+  const char *name = "macaq_iu8f_mlp_w4_tm1";
+  memset(d, 0, sizeof *d);
+  copy_name(d->op, sizeof d->op, op);
+  copy_name(d->plugin, sizeof d->plugin, "macaq_iu8f");
+  copy_name(d->kernel, sizeof d->kernel, name);
+  d->grid[0] = grid, d->grid[1] = 1, d->grid[2] = 1;
+  d->block[0] = 512, d->block[1] = 1, d->block[2] = 1;
+  d->n_launches = 1;
+  d->ks = 1;
+  if (int rc = fill_slots(name, d)) return rc;
+  set_i32(d, "m", m);
+  set_i32(d, "k", hidden);
+  set_i32(d, "n", inter);
+  set_i32(d, "spin", spin ? spin : MLP_CHAIN_SPIN);
+  add_ws(d, "p", SABER_IU8_WS_SCRATCH, (uint64_t)m * inter * 2, 0);
+  add_ws(d, "state", SABER_IU8_WS_PERSISTENT, MLP_CHAIN_STATE_BYTES, 1);
+  return 0;
+}
+
 // The row kernels' register forms: the narrowest that holds the row (4,096 elements a group slot).
 // Many narrow rows go a wave a row (`base`_w64), the rest a workgroup a row (`base`_t256...).
 static std::string row_form(const char *base, uint32_t rows, uint32_t width) {

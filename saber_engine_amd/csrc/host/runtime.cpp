@@ -22,6 +22,7 @@ using namespace iu8;
 struct LoadedKernel {
   hipFunction_t fn;
   uint32_t max_threads;  // the code object's max_flat_workgroup_size: the block its indexing is written for
+  int64_t resident;      // workgroups of that size the device holds at once (kernels that meet inside a launch), else 0
 };
 struct saber_iu8_ctx {
   int device = 0;
@@ -95,7 +96,17 @@ static int load_one(saber_iu8_ctx *ctx, const std::string &manifest_path) {
   for (const KernelDecl &k : m.kernel) {
     hipFunction_t fn;
     if ((e = hipModuleGetFunction(&fn, mod, k.name.c_str())) != hipSuccess) return hip_fail(("hipModuleGetFunction " + k.name).c_str(), e);
-    ctx->fn[k.name] = LoadedKernel{fn, k.max_flat_workgroup_size};
+    int64_t resident = 0;
+    if (k.name.rfind("macaq_iu8f_mlp_", 0) == 0) {
+      // asked once, at load: the launch itself may run under stream capture
+      int per_cu = 0, cus = 0;
+      if ((e = hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, fn, (int)k.max_flat_workgroup_size, 0)) != hipSuccess)
+        return hip_fail("hipModuleOccupancyMaxActiveBlocksPerMultiprocessor", e);
+      if ((e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, ctx->device)) != hipSuccess)
+        return hip_fail("hipDeviceGetAttribute", e);
+      resident = (int64_t)per_cu * cus;
+    }
+    ctx->fn[k.name] = LoadedKernel{fn, k.max_flat_workgroup_size, resident};
     ctx->counters.kernels_loaded++;
   }
   return 0;
@@ -331,7 +342,33 @@ int saber_iu8_has_kernel(const saber_iu8_ctx *ctx, const char *kernel) {
 
 // What a hand-edited descriptor could get wrong for a kernel whose bounds depend on its grid: the
 // fused decode linear keeps at most 8 column blocks' weight scales a workgroup and 20 KiB of codes.
-static int launch_guard(const saber_iu8_desc *d) {
+static int i32_arg(const saber_iu8_desc *d, const char *name) {
+  for (uint32_t i = 0; i < d->n_args; ++i)
+    if (d->args[i].kind == SABER_IU8_ARG_I32 && !strcmp(d->args[i].name, name)) return (int)d->args[i].ival;
+  return 0;
+}
+
+// The decode MLP chain's workgroups meet inside the launch: a grid the card cannot hold all at once
+// would wait for workgroups that never start (until the kernel's bounded wait gives up), so it is
+// refused here from what the loaded kernel's registers and LDS let reside.
+static int chain_guard(const LoadedKernel &lk, const saber_iu8_desc *d) {
+  const int64_t m = i32_arg(d, "m"), h = i32_arg(d, "k"), i = i32_arg(d, "n");
+  if (m <= 0 || h <= 0 || i <= 0 || !fused_holds((uint32_t)m, (uint32_t)h) || !fused_holds((uint32_t)m, (uint32_t)i) ||
+      h % 128 || i % 128)
+    return fail(SABER_IU8_E_RULE, fmt("%s: %lld rows of %lld / %lld do not fit the fused form", d->kernel, (long long)m, (long long)h,
+                                      (long long)i));
+  const int64_t nblk = std::max((2 * i + 31) / 32, (h + 31) / 32);
+  if ((int64_t)d->grid[0] * 8 < nblk || d->grid[0] > MLP_CHAIN_MAX_GRID || d->grid[1] != 1 || d->grid[2] != 1 || i32_arg(d, "spin") <= 0)
+    return fail(SABER_IU8_E_RULE, fmt("%s: grid %u x %u x %u: %lld column blocks at most 8 a workgroup, at most %u workgroups, a spin limit",
+                                      d->kernel, d->grid[0], d->grid[1], d->grid[2], (long long)nblk, MLP_CHAIN_MAX_GRID));
+  if (lk.resident < (int64_t)d->grid[0])
+    return fail(SABER_IU8_E_RULE, fmt("%s: %u workgroups must be resident at once; this device holds %lld", d->kernel, d->grid[0],
+                                      (long long)lk.resident));
+  return 0;
+}
+
+static int launch_guard(const LoadedKernel &lk, const saber_iu8_desc *d) {
+  if (strncmp(d->kernel, "macaq_iu8f_mlp_", 15) == 0) return chain_guard(lk, d);
   if (strncmp(d->kernel, "macaq_iu8_decq_", 15) != 0) return 0;
   int64_t m = 0, n = 0, k = 0;
   for (uint32_t i = 0; i < d->n_args; ++i) {
@@ -363,7 +400,7 @@ int saber_iu8_launch(saber_iu8_ctx *ctx, const saber_iu8_desc *d, const saber_iu
   if (threads != it->second.max_threads)
     return fail(SABER_IU8_E_RULE, fmt("%s: a block of %llu threads; the gfx950 kernel is written for %u (use this object's launch law)",
                                       d->kernel, (unsigned long long)threads, it->second.max_threads));
-  if (int rc = launch_guard(d)) return rc;
+  if (int rc = launch_guard(it->second, d)) return rc;
   alignas(16) uint8_t image[256];
   uint32_t bytes = 0;
   if (int rc = saber_iu8_pack_kernarg(d, bufs, n_bufs, image, sizeof image, &bytes)) return rc;
@@ -399,6 +436,23 @@ int saber_iu8_linear_fused(saber_iu8_ctx *ctx, int wkind, const void *x, const v
   if (!scale) set_null(&d, "scale");
   const saber_iu8_binding b[] = {{"x", (void *)x}, {"w", (void *)w}, {"ws", (void *)ws}, {"c", c}, {"q", q}, {"scale", scale}};
   return saber_iu8_launch(ctx, &d, b, 6, stream);
+}
+
+int saber_iu8_resolve_mlp_chain(uint32_t m, uint32_t hidden, uint32_t inter, uint32_t spin, saber_iu8_desc *out) {
+  if (!out) return fail(SABER_IU8_E_ARG, "resolve_mlp_chain: null descriptor");
+  return resolve_mlp_chain(m, hidden, inter, spin, out);
+}
+
+int saber_iu8_mlp_chain(saber_iu8_ctx *ctx, const void *x, const void *w_gu, const float *ws_gu, const void *w_dn,
+                        const float *ws_dn, void *gu, void *p, void *state, void *c, uint32_t m, uint32_t hidden, uint32_t inter,
+                        uint32_t spin, void *stream) {
+  saber_iu8_desc d;
+  if (int rc = resolve_mlp_chain(m, hidden, inter, spin, &d)) return rc;
+  if (!gu) set_null(&d, "gu");  // the [gate | up] rows are a tap: the kernel tests the pointer
+  const saber_iu8_binding b[] = {{"x", (void *)x},         {"w", (void *)w_gu}, {"ws", (void *)ws_gu}, {"w_b", (void *)w_dn},
+                                 {"ws_b", (void *)ws_dn}, {"gu", gu},          {"p", p},              {"state", state},
+                                 {"c", c}};
+  return saber_iu8_launch(ctx, &d, b, 9, stream);
 }
 
 int saber_iu8_rowscale(saber_iu8_ctx *ctx, const void *x, float *scale, uint32_t m, uint32_t k, void *stream) {

@@ -18,13 +18,46 @@
 
 #define IU8_DECQ_MAXB 8  // column blocks a workgroup: gridDim.x >= ceil(blocks / 8)
 
-template <bool W8, int NT, int KW, int WPB, int D>
+// CH (a launch that chains the MLP's two linears through memory, iu8_chain.h): 0 = a launch of its own.
+// 1 = the chain's first linear, gate and up PAIRED: W holds 2N rows (N gate rows, then N up rows), a
+// column block is ONE 16-column tile of the product p = bf16(bf16(silu(gate)) * up), whose gate tile
+// goes to the waves wn = 0 and whose up tile to the waves wn = 1 (WN = 2, NT = 1). The up wave leaves
+// its bf16 values in LDS, the gate wave combines them a block later (behind that block's own
+// meeting, so the exchange costs no barrier of its own), stores p straight through to memory
+// (coherent for the other workgroups of the launch, whatever XCD they run on) and keeps the rows'
+// maxima of |p|, which end in `hook.slot` (4 floats, this workgroup's). C, if not null, receives
+// [gate | up] as a launch of its own would store them (bf16 [M, 2N]).
+// 2 = the chain's second linear: its rows are the first's output, so the weight ring starts first,
+// then `hook.wait()` returns when every workgroup's share of the rows is in memory, the rows are
+// loaded coherently, and their maxima come from `hook.amax(out)` (found by the producers) instead of a
+// pass over the rows.
+static __device__ __forceinline__ float iu8_silu_bf16(float x) {  // as the producer kernels compute it (macaq_i8q: i8q_silu_bf16)
+#pragma clang fp contract(off)
+  return iu8_bf16_f32((unsigned short)iu8_bf16_bits(x / (1.f + expf(-x))));
+}
+struct iu8_decq_pairhook {
+  unsigned short *p;  // bf16 [M, N]
+  float *slot;        // this workgroup's 4 maxima
+};
+struct iu8_decq_nohook {
+  __device__ bool wait() const { return true; }
+  __device__ void amax(float[4]) const {}
+};
+static __device__ __forceinline__ iu8_v4u iu8_decq_ld_coherent(const iu8_v4u *p) {
+  const unsigned long long lo = __hip_atomic_load((const unsigned long long *)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+  const unsigned long long hi = __hip_atomic_load((const unsigned long long *)p + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+  return iu8_v4u{(unsigned)lo, (unsigned)(lo >> 32), (unsigned)hi, (unsigned)(hi >> 32)};
+}
+template <bool W8, int NT, int KW, int WPB, int D, int CH = 0, class Hook = iu8_decq_nohook>
 __device__ __forceinline__ void iu8_decq_body(const unsigned short *__restrict__ X, const iu8_u8 *__restrict__ W,
                                               const float *__restrict__ ws, iu8_u8 *__restrict__ qout,
                                               float *__restrict__ sout, unsigned short *__restrict__ C, int M, int N,
-                                              int K) {
+                                              int K, const Hook hook = Hook{}) {
   static_assert(KW > 1 && WPB % KW == 0, "k-waves divide the workgroup");
   constexpr int WN = WPB / KW;
+  constexpr bool PAIRED = CH == 1;
+  static_assert(!PAIRED || (WN == 2 && NT == 1 && !W8), "the paired form: a gate wave and an up wave a tile");
+  constexpr int WNB = PAIRED ? 1 : WN;  // column-tile groups of the OUTPUT a block
   constexpr int NTHR = WPB * 64;
   constexpr int WSTEP = W8 ? 2048 : 1024;  // bytes of one 16-row weight tile per 128-deep K step
   constexpr int WV = W8 ? 2 : 1;           // 16-byte loads a lane per step per tile
@@ -34,15 +67,21 @@ __device__ __forceinline__ void iu8_decq_body(const unsigned short *__restrict__
   __shared__ __attribute__((aligned(16))) int s_red[2][RED];
   __shared__ float s_amax[WPB][4];
   __shared__ float s_ws[IU8_DECQ_MAXB][WN * NT * 16];  // the epilogue's weight scales (W4: already / 16)
+  __shared__ __attribute__((aligned(8))) unsigned s_up[PAIRED ? 2 : 1][PAIRED ? 128 : 2];  // the up wave's bf16 values, two blocks
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wk = wave % KW, wn = wave / KW;
   const int ntiles = N >> 4, steps = K >> 7;
   const int ml = lane & 15, lg = lane >> 4;
-  const int T = wk < steps ? (steps - wk + KW - 1) / KW : 0;  // this wave's steps of a block: wk + t*KW
-  const int nblk = (ntiles + WN * NT - 1) / (WN * NT);
   const int G = gridDim.x;
+  const int T = wk < steps ? (steps - wk + KW - 1) / KW : 0;  // this wave's steps of a block: wk + t*KW
+  const int nblk = (ntiles + WNB * NT - 1) / (WNB * NT);
+  // the weight tile of this wave's j-th tile in the workgroup's block b (paired: the up rows follow the N gate rows)
+  auto tile_of = [&](int b, int j) {
+    if constexpr (PAIRED) return wn * ntiles + min((int)blockIdx.x + b * G, ntiles - 1);
+    else return min((((int)blockIdx.x + b * G) * WN + wn) * NT + j, ntiles - 1);  // a tile past N re-reads the last one and stores nothing
+  };
   const int nb = (int)blockIdx.x < nblk ? (nblk - (int)blockIdx.x + G - 1) / G : 0;  // this workgroup's blocks
   const int TT = nb * T;
 
@@ -52,9 +91,11 @@ __device__ __forceinline__ void iu8_decq_body(const unsigned short *__restrict__
   constexpr int X_PER = (ABYTES / 8 + NTHR - 1) / NTHR;
   iu8_v4u xreg[X_PER];
   const int k8 = K >> 3, x_pieces = M * k8;
+  if constexpr (CH != 2) {
 #pragma unroll
-  for (int p = 0; p < X_PER; ++p)
-    if (p * NTHR + tid < x_pieces) xreg[p] = *((const iu8_v4u *)X + p * NTHR + tid);
+    for (int p = 0; p < X_PER; ++p)
+      if (p * NTHR + tid < x_pieces) xreg[p] = *((const iu8_v4u *)X + p * NTHR + tid);
+  }
 
   // ---- this workgroup's weight scales, all blocks: loaded now, put in LDS behind the ring's issue
   // (a store here would wait out the load's whole latency in front of the weight loads)
@@ -63,20 +104,23 @@ __device__ __forceinline__ void iu8_decq_body(const unsigned short *__restrict__
 #pragma unroll
   for (int p = 0; p < WS_PER; ++p) {
     const int i = p * NTHR + tid, b = i / (WN * NT * 16), c = i - b * (WN * NT * 16);
-    const int n = ((int)blockIdx.x + b * G) * (WN * NT * 16) + c;
-    wsreg[p] = (i < min(nb, IU8_DECQ_MAXB) * (WN * NT * 16) && n < N) ? iu8_wsu<W8>(ws, n) : 0.f;
+    int n;
+    bool in;
+    if constexpr (PAIRED) {
+      const int t = (int)blockIdx.x + b * G;
+      n = (c >> 4) * N + t * 16 + (c & 15), in = t < ntiles;
+    } else {
+      n = ((int)blockIdx.x + b * G) * (WN * NT * 16) + c, in = n < N;
+    }
+    wsreg[p] = (i < min(nb, IU8_DECQ_MAXB) * (WN * NT * 16) && in) ? iu8_wsu<W8>(ws, n) : 0.f;
   }
 
   // ---- the issue side of the ring: block ib, step it, this lane's address in every tile
   int ib = 0, it = 0;
   const iu8_u8 *ip[NT];
   auto set_ip = [&](int b) {
-    const int nt0 = (((int)blockIdx.x + b * G) * WN + wn) * NT;
 #pragma unroll
-    for (int j = 0; j < NT; ++j) {
-      const int ntj = min(nt0 + j, ntiles - 1);  // a tile past N re-reads the last one and stores nothing
-      ip[j] = W + ((size_t)ntj * steps + wk) * WSTEP + lane * 16;
-    }
+    for (int j = 0; j < NT; ++j) ip[j] = W + ((size_t)tile_of(b, j) * steps + wk) * WSTEP + lane * 16;
   };
   set_ip(0);
   iu8_v4u ring[D][NT][WV];
@@ -98,6 +142,24 @@ __device__ __forceinline__ void iu8_decq_body(const unsigned short *__restrict__
   // all order-free maxima; sc = max(amax / 127, 1e-30); codes by the exact reciprocal path
   float qsc[4] = {1.f, 1.f, 1.f, 1.f};
   {
+    if constexpr (CH == 2) {
+      // the chain's second linear: weights first (they do not depend on the first linear), then the
+      // rows once every producer's share is in memory; no pass for the maxima
+#pragma unroll
+      for (int i = 0; i < D; ++i)
+        if (i < TT) issue(i);
+      if (!hook.wait()) return;  // a producer never arrived (the launch reports it): give up as a whole
+#pragma unroll
+      for (int p = 0; p < X_PER; ++p)
+        if (p * NTHR + tid < x_pieces) xreg[p] = iu8_decq_ld_coherent((const iu8_v4u *)X + p * NTHR + tid);
+#pragma unroll
+      for (int p = 0; p < WS_PER; ++p)
+        if (p * NTHR + tid < WS_ALL) (&s_ws[0][0])[p * NTHR + tid] = wsreg[p];
+      float a4[4];
+      hook.amax(a4);  // the whole workgroup: the maxima over the producers' shares
+#pragma unroll
+      for (int r = 0; r < 4; ++r) s_amax[0][r] = a4[r];
+    } else {
     float am[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int p = 0; p < X_PER; ++p) {
@@ -135,14 +197,17 @@ __device__ __forceinline__ void iu8_decq_body(const unsigned short *__restrict__
 #pragma unroll
     for (int p = 0; p < WS_PER; ++p)
       if (p * NTHR + tid < WS_ALL) (&s_ws[0][0])[p * NTHR + tid] = wsreg[p];
+    }
     __syncthreads();
     float qrcp[4] = {1.f, 1.f, 1.f, 1.f};
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       if (r >= M) break;
       float a = s_amax[0][r];
+      if constexpr (CH != 2) {
 #pragma unroll
-      for (int w = 1; w < WPB; ++w) a = fmaxf(a, s_amax[w][r]);
+        for (int w = 1; w < WPB; ++w) a = fmaxf(a, s_amax[w][r]);
+      }
       qsc[r] = fmaxf(__fdiv_rn(a, 127.f), 1e-30f);
       qrcp[r] = __fdiv_rn(1.f, qsc[r]);
     }
@@ -183,6 +248,29 @@ __device__ __forceinline__ void iu8_decq_body(const unsigned short *__restrict__
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
   };
+  // the paired form's gate wave: its bf16 gate values of the block before, the rows' running maxima
+  iu8_v2u g_prev = iu8_v2u{0, 0};
+  float pmax = 0.f;
+  auto pair_done = [&](int b) {  // p of the workgroup's block b: the gate wave's values x the up wave's, out of LDS
+#pragma clang fp contract(off)
+    if constexpr (PAIRED) {
+      const iu8_v2u u = *(const iu8_v2u *)&s_up[b & 1][lane * 2];
+      const int tile = (int)blockIdx.x + b * G;
+      if (tile >= ntiles || ml >= M) return;
+      const unsigned gw[2] = {g_prev.x, g_prev.y}, uw[2] = {u.x, u.y};
+      unsigned o[2];
+#pragma unroll
+      for (int w = 0; w < 2; ++w) {
+        const float g0 = __uint_as_float(gw[w] << 16), g1 = __uint_as_float(gw[w] & 0xFFFF0000u);
+        const float u0 = __uint_as_float(uw[w] << 16), u1 = __uint_as_float(uw[w] & 0xFFFF0000u);
+        const unsigned b0 = iu8_bf16_bits(iu8_silu_bf16(g0) * u0), b1 = iu8_bf16_bits(iu8_silu_bf16(g1) * u1);
+        o[w] = b0 | (b1 << 16);
+        pmax = fmaxf(pmax, fmaxf(fabsf(iu8_bf16_f32((unsigned short)b0)), fabsf(iu8_bf16_f32((unsigned short)b1))));
+      }
+      __hip_atomic_store((unsigned long long *)(hook.p + (size_t)ml * N + tile * 16 + lg * 4),
+                         (unsigned long long)o[0] | ((unsigned long long)o[1] << 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
+  };
   auto block_end = [&]() {
     int *red = s_red[cb & 1];
     if (wk > 0) {
@@ -195,17 +283,33 @@ __device__ __forceinline__ void iu8_decq_body(const unsigned short *__restrict__
       for (int q = 0; q < KW - 1; ++q)
 #pragma unroll
         for (int j = 0; j < NT; ++j) acc[j] += *(const iu8_v4i *)&red[((q * WN + wn) * NT + j) * 256 + lane * 4];
-      const int nt0 = (((int)blockIdx.x + cb * G) * WN + wn) * NT;
-#pragma unroll
-      for (int j = 0; j < NT; ++j) {
-        if (nt0 + j >= ntiles || ml >= M) continue;
-        const int n = (nt0 + j) * 16 + lg * 4;
-        const float *wsu = &s_ws[min(cb, IU8_DECQ_MAXB - 1)][(wn * NT + j) * 16 + lg * 4];
-        const float am = ml == 0 ? qsc[0] : ml == 1 ? qsc[1] : ml == 2 ? qsc[2] : qsc[3];
+      const float am = ml == 0 ? qsc[0] : ml == 1 ? qsc[1] : ml == 2 ? qsc[2] : qsc[3];
+      if constexpr (PAIRED) {
+        const int tile = (int)blockIdx.x + cb * G;
+        const float *wsu = &s_ws[min(cb, IU8_DECQ_MAXB - 1)][wn * 16 + lg * 4];
         unsigned h[4];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) h[r] = iu8_bf16_bits(iu8_epi(acc[j][r], am, wsu[r]));
-        *(iu8_v2u *)(C + (size_t)ml * N + n) = iu8_v2u{h[0] | (h[1] << 16), h[2] | (h[3] << 16)};
+        for (int r = 0; r < 4; ++r) h[r] = iu8_bf16_bits(iu8_epi(acc[0][r], am, wsu[r]));
+        const iu8_v2u out = iu8_v2u{h[0] | (h[1] << 16), h[2] | (h[3] << 16)};
+        if (C != nullptr && tile < ntiles && ml < M) *(iu8_v2u *)(C + (size_t)ml * 2 * N + wn * N + tile * 16 + lg * 4) = out;
+        if (wn == 1) {
+          *(iu8_v2u *)&s_up[cb & 1][lane * 2] = out;  // read by the gate wave behind the NEXT meeting
+        } else {
+          if (cb > 0) pair_done(cb - 1);  // the up wave stored these before the meeting just passed
+          g_prev = out;
+        }
+      } else {
+        const int nt0 = (((int)blockIdx.x + cb * G) * WN + wn) * NT;
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+          if (nt0 + j >= ntiles || ml >= M) continue;
+          const int n = (nt0 + j) * 16 + lg * 4;
+          const float *wsu = &s_ws[min(cb, IU8_DECQ_MAXB - 1)][(wn * NT + j) * 16 + lg * 4];
+          unsigned h[4];
+#pragma unroll
+          for (int r = 0; r < 4; ++r) h[r] = iu8_bf16_bits(iu8_epi(acc[j][r], am, wsu[r]));
+          *(iu8_v2u *)(C + (size_t)ml * N + n) = iu8_v2u{h[0] | (h[1] << 16), h[2] | (h[3] << 16)};
+        }
       }
     }
 #pragma unroll
@@ -236,23 +340,36 @@ __device__ __forceinline__ void iu8_decq_body(const unsigned short *__restrict__
 
   if (T == 0) {  // a k-wave past a short K: no steps, but it meets the others once a block
     for (int b = 0; b < nb; ++b) block_end();
-    return;
-  }
-  int L0 = 0;
-  for (; L0 + 2 * D <= TT; L0 += D) {  // steady state: every slot consumed and re-issued
+  } else {
+    int L0 = 0;
+    for (; L0 + 2 * D <= TT; L0 += D) {  // steady state: every slot consumed and re-issued
 #pragma unroll
-    for (int i = 0; i < D; ++i) {
-      consume(i);
-      issue(i);
+      for (int i = 0; i < D; ++i) {
+        consume(i);
+        issue(i);
+      }
+    }
+    for (; L0 < TT; L0 += D) {  // drain
+#pragma unroll
+      for (int i = 0; i < D; ++i) {
+        if (L0 + i < TT) {
+          consume(i);
+          if (L0 + i + D < TT) issue(i);
+        }
+      }
     }
   }
-  for (; L0 < TT; L0 += D) {  // drain
-#pragma unroll
-    for (int i = 0; i < D; ++i) {
-      if (L0 + i < TT) {
-        consume(i);
-        if (L0 + i + D < TT) issue(i);
-      }
+  if constexpr (PAIRED) {
+    // the last block's pair, behind one more meeting; then this workgroup's maxima: a lane holds row
+    // ml's over its 4 columns of every block, the four lanes of a row meet by two exchanges
+    meet();
+    if (wk == 0 && wn == 0) {
+      if (nb > 0) pair_done(nb - 1);
+      pmax = fmaxf(pmax, __shfl_xor(pmax, 16));
+      pmax = fmaxf(pmax, __shfl_xor(pmax, 32));
+      if (lane < 4)  // all four words, every launch: nothing of an earlier launch survives
+        __hip_atomic_store((unsigned *)hook.slot + lane, lane < M ? __float_as_uint(pmax) : 0u, __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_SYSTEM);
     }
   }
 }

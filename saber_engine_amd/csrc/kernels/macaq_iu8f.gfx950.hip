@@ -12,6 +12,7 @@
 // problem's workgroups in front of problem 0's (the reference's ba-first order,
 // crates/saber-kernels/src/macaq_iu8.rs:549-553): the same bytes, the small half not in the tail.
 #include "iu8_gemm.h"
+#include "iu8_chain.h"
 
 #define IU8F_PAIR(name, TM, NT, KW, WPB, D, ALDS, BFIRST)                                                                \
   extern "C" __global__ __launch_bounds__(WPB * 64) void name(                                                      \
@@ -31,3 +32,19 @@
 #define IU8_PAIR_VARIANT(name, TM, NT, KW, WPB, D, ALDS, BFIRST) IU8F_PAIR(name, TM, NT, KW, WPB, D, ALDS, BFIRST)
 #include "iu8_variants.def"
 #undef IU8F_PAIR
+
+// THE DECODE MLP CHAIN: gate+up linear -> SiLU(gate) * up with its per-token requantisation -> down
+// linear, one persistent launch for at most 4 rows (iu8_chain.h). `w` / `ws` are the gate and up
+// weights as one [2n, k] operand (gate rows first), `w_b` / `ws_b` the down weights [k, n]; `gu`
+// (bf16 [m, 2n]) and `p` (bf16 [m, n]) are the launch's working rows; `state` is the 12 KiB block
+// the workgroups meet through (zero before the first launch, ready for the next after a launch that
+// completes; the word at 10 KiB + 8 non-zero: a meeting timed out, c is not valid).
+// The grid is the host's: every workgroup resident at once, at most 512 of them, at most 8 column
+// blocks of either linear a workgroup.
+extern "C" __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) void macaq_iu8f_mlp_w4_tm1(
+    const unsigned short *__restrict__ x, const unsigned char *__restrict__ w, const float *__restrict__ ws,
+    const unsigned char *__restrict__ w_b, const float *__restrict__ ws_b, unsigned short *__restrict__ gu,
+    unsigned short *__restrict__ p, unsigned char *__restrict__ state, unsigned short *__restrict__ c, int m, int k, int n,
+    int spin) {
+  iu8_chain_mlp<1, 4, 8, 8>(x, w, ws, w_b, ws_b, gu, p, state, c, m, k, n, spin);
+}

@@ -122,6 +122,8 @@ def lib():
         L.saber_iu8_band_toml.argtypes = [C.c_char_p, C.c_size_t, C.POINTER(C.c_size_t)]
         L.saber_iu8_gemm_pair.argtypes = [C.c_void_p] * 6 + [C.c_uint32] + [C.c_void_p] * 3 + [C.c_uint32] * 3 + [C.c_void_p]
         L.saber_iu8_linear_fused.argtypes = [C.c_void_p, C.c_int] + [C.c_void_p] * 6 + [C.c_uint32] * 3 + [C.c_void_p]
+        L.saber_iu8_resolve_mlp_chain.argtypes = [C.c_uint32] * 4 + [C.c_void_p]
+        L.saber_iu8_mlp_chain.argtypes = [C.c_void_p] * 10 + [C.c_uint32] * 4 + [C.c_void_p]
         L.saber_iu8_quant_had.argtypes = [C.c_void_p] * 4 + [C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p]
         L.saber_iu8_silu_mul_quant_had.argtypes = [C.c_void_p] * 4 + [C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p]
         L.saber_iu8_add_rms_quant_had.argtypes = [C.c_void_p] * 7 + [C.c_uint32, C.c_uint32, C.c_float, C.c_void_p, C.c_void_p]
@@ -196,6 +198,16 @@ def fused_holds(m, k):
 def resolve_fused(wkind, m, n, k):
     d = Desc()
     _check(lib().saber_iu8_resolve_fused(wkind, m, n, k, C.byref(d)))
+    return d
+
+
+MLP_CHAIN_STATE_BYTES = 12 * 1024
+MLP_CHAIN_STATUS_OFFSET = 10 * 1024 + 8
+
+
+def resolve_mlp_chain(m, hidden, inter, spin=0):
+    d = Desc()
+    _check(lib().saber_iu8_resolve_mlp_chain(m, hidden, inter, spin, C.byref(d)))
     return d
 
 
@@ -362,6 +374,12 @@ class Context:
 
     def linear_fused(self, wkind, x, w, w_scale, c, m, n, k, q=None, scale=None, stream=0):
         _check(lib().saber_iu8_linear_fused(self._h, wkind, x, w, w_scale, c, q, scale, m, n, k, stream))
+
+    def mlp_chain(self, x, w_gu, ws_gu, w_dn, ws_dn, gu, p, state, c, m, hidden, inter, spin=0, stream=0):
+        """gate+up -> SiLU * up + requant -> down in one persistent launch; `state` (MLP_CHAIN_STATE_BYTES)
+        zero before the first use. A non-zero word at state + MLP_CHAIN_STATUS_OFFSET after the launch:
+        a meeting timed out, c is undefined."""
+        _check(lib().saber_iu8_mlp_chain(self._h, x, w_gu, ws_gu, w_dn, ws_dn, gu, p, state, c, m, hidden, inter, spin, stream))
 
     def quant_had(self, x, q, scale, m, k, had_t, stream=0):
         _check(lib().saber_iu8_quant_had(self._h, x, q, scale, m, k, had_t, stream))

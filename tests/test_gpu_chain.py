@@ -1,0 +1,124 @@
+"""GPU parity of the dense decode MLP as one persistent launch (macaq_iu8f_mlp_w4_tm1): gate+up
+linear -> SiLU * up + requantisation -> down linear. Bit-exact against the oracle's three steps and
+against the library's own three launches; the launch's working rows are checked too; the bounded
+wait of its meetings is exercised from the host with a one-poll limit (every workgroup still exits
+normally)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import ref
+from saber_engine_amd import iu8, synth
+from tests.gpu_util import dev_bf16_bits, dev_f32, dev_u8, host_u16, say
+
+pytestmark = pytest.mark.gpu
+GEN = iu8.MLP_CHAIN_STATUS_OFFSET // 4 - 2              # the generation word; the status word two words on
+
+
+class Mlp:
+    def __init__(self, M, H, I, seed):
+        rng = np.random.default_rng(seed)
+        self.M, self.H, self.I = M, H, I
+        self.Wgu, self.wsgu = synth.weights(rng, 2 * I, H, False)
+        self.Wdn, self.wsdn = synth.weights(rng, H, I, False)
+        self.X = synth.activations(rng, M, H)
+        self.x = dev_bf16_bits(self.X)
+        self.wgu, self.wsg = dev_u8(iu8.repack_w4(self.Wgu)), dev_f32(self.wsgu)
+        self.wdn, self.wsd = dev_u8(iu8.repack_w4(self.Wdn)), dev_f32(self.wsdn)
+        self.gu = torch.full((M, 2 * I), 0x7FC0, dtype=torch.int16, device="cuda")
+        self.p = torch.full((M, I), 0x7FC0, dtype=torch.int16, device="cuda")
+        self.state = torch.zeros(iu8.MLP_CHAIN_STATE_BYTES // 4, dtype=torch.int32, device="cuda")
+        self.c = torch.full((M, H), 0x7FC0, dtype=torch.int16, device="cuda")
+
+    def oracle(self):
+        gu = ref.linear(self.X, self.Wgu, self.wsgu, False, threads=16)["C"]
+        _, _, p = ref.silu_mul_quant(gu)
+        c = ref.linear(p, self.Wdn, self.wsdn, False, threads=16)["C"]
+        return gu, p, c
+
+    def chain(self, ctx, spin=0, tap=True):
+        ctx.mlp_chain(self.x.data_ptr(), self.wgu.data_ptr(), self.wsg.data_ptr(), self.wdn.data_ptr(), self.wsd.data_ptr(),
+                      self.gu.data_ptr() if tap else None, self.p.data_ptr(), self.state.data_ptr(), self.c.data_ptr(),
+                      self.M, self.H, self.I, spin=spin)
+        torch.cuda.synchronize()
+
+    def three_launches(self, ctx):
+        M, H, I = self.M, self.H, self.I
+        gu = torch.full((M, 2 * I), 0x7FC0, dtype=torch.int16, device="cuda")
+        q = torch.zeros(iu8.a_bytes(M, I), dtype=torch.uint8, device="cuda")
+        s = torch.zeros(M, dtype=torch.float32, device="cuda")
+        c = torch.full((M, H), 0x7FC0, dtype=torch.int16, device="cuda")
+        ctx.linear_fused(iu8.W4, self.x.data_ptr(), self.wgu.data_ptr(), self.wsg.data_ptr(), gu.data_ptr(), M, 2 * I, H)
+        ctx.launch(iu8.resolve_silu_mul_quant(M, I), dict(gu=gu.data_ptr(), q=q.data_ptr(), scale=s.data_ptr()))
+        ctx.gemm_static(iu8.W4, q.data_ptr(), s.data_ptr(), self.wdn.data_ptr(), self.wsd.data_ptr(), c.data_ptr(), M, H, I)
+        torch.cuda.synchronize()
+        return host_u16(gu), host_u16(c)
+
+
+# rows, hidden, intermediate: the benchmark layer at one row (5120 / 17408); the most rows the form
+# holds at a narrower layer; two rows at the widest they fit; three rows (staged as four) with K
+# steps that do not divide among the k-waves (11 and 23); fewer column blocks than workgroups
+SHAPES = [(1, 5120, 17408), (4, 5120, 5120), (2, 2048, 10240), (3, 1408, 2944), (1, 384, 384)]
+
+
+@pytest.mark.parametrize("M,H,I", SHAPES)
+def test_chain_matches_the_oracle_and_the_three_launches(ctx, M, H, I):
+    say(f"mlp chain M={M} H={H} I={I}")
+    d = iu8.resolve_mlp_chain(M, H, I)
+    assert d.kernel == b"macaq_iu8f_mlp_w4_tm1" and d.grid[0] == 512 and d.block[0] == 512
+    assert {w.name: w.bytes for w in d.workspaces[:d.n_workspaces]} == {b"p": M * I * 2, b"state": iu8.MLP_CHAIN_STATE_BYTES}
+    mlp = Mlp(M, H, I, seed=M + I)
+    want_gu, want_p, want_c = mlp.oracle()
+    for rep in range(3):                                # launches in a row on one state block: no clearing between
+        mlp.c.fill_(0x7FC0)
+        mlp.chain(ctx)
+        gen, _, status = mlp.state[GEN:GEN + 3].cpu().tolist()
+        assert (gen, status) == (rep + 1, 0), "a completed launch advances the generation and raises nothing"
+        np.testing.assert_array_equal(host_u16(mlp.gu), want_gu)
+        np.testing.assert_array_equal(host_u16(mlp.p), want_p)
+        np.testing.assert_array_equal(host_u16(mlp.c), want_c)
+    mlp.gu.fill_(0x7FC0), mlp.c.fill_(0x7FC0)            # without the [gate | up] tap: nothing stored there
+    mlp.chain(ctx, tap=False)
+    assert (mlp.gu == 0x7FC0).all().item()
+    np.testing.assert_array_equal(host_u16(mlp.c), want_c)
+    gu3, c3 = mlp.three_launches(ctx)
+    np.testing.assert_array_equal(gu3, want_gu)
+    np.testing.assert_array_equal(c3, want_c)
+
+
+def test_chain_meeting_gives_up_after_its_poll_limit_and_says_so(ctx):
+    """One poll a meeting: the first workgroup to look finds the others not yet arrived, raises the
+    status word and leaves, and every other workgroup leaves at its next meeting. The launch ends by
+    itself; after the host clears `state` the same buffers give the right bytes."""
+    M, H, I = 1, 1024, 2048
+    say(f"mlp chain poll limit M={M} H={H} I={I}")
+    mlp = Mlp(M, H, I, seed=5)
+    mlp.chain(ctx, spin=1)
+    assert mlp.state[GEN + 2].item() != 0, "a meeting that ran out of polls raises the status word"
+    mlp.state.zero_()
+    mlp.chain(ctx)
+    assert mlp.state[GEN:GEN + 3].cpu().tolist() == [1, 0, 0]
+    np.testing.assert_array_equal(host_u16(mlp.c), mlp.oracle()[2])
+
+
+def test_chain_refuses_what_the_form_does_not_hold(ctx):
+    for m, h, i, word in ((5, 1024, 2048, "fused form"), (4, 5120, 17408, "fused form"), (1, 5120, 17400, "multiple"),
+                          (0, 1024, 2048, "nothing")):
+        with pytest.raises(iu8.IU8Error) as e:
+            iu8.resolve_mlp_chain(m, h, i)
+        assert e.value.code == iu8.E_RULE and word in str(e.value)
+    # a grid the kernel's bounds or the device's residency do not allow is refused at launch
+    d = iu8.resolve_mlp_chain(1, 1024, 2048)
+    x = torch.zeros(1 << 16, dtype=torch.uint8, device="cuda")
+    bufs = {k: x.data_ptr() for k in ("x", "w", "ws", "w_b", "ws_b", "gu", "p", "state", "c")}
+    assert x.numel() >= iu8.MLP_CHAIN_STATE_BYTES
+    before = ctx.counters().launches
+    d.grid[0] = 4096
+    with pytest.raises(iu8.IU8Error) as e:
+        ctx.launch(d, bufs)
+    assert e.value.code == iu8.E_RULE and "at most 512 workgroups" in str(e.value)
+    d.grid[0] = 8                                       # 128 column blocks of gate+up: more than 8 x 8
+    with pytest.raises(iu8.IU8Error) as e:
+        ctx.launch(d, bufs)
+    assert e.value.code == iu8.E_RULE and "column blocks" in str(e.value)
+    assert ctx.counters().launches == before

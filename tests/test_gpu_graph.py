@@ -1,7 +1,7 @@
 """Capture legality and re-entrancy (launch conventions of crates/saber-exec/src/launch.rs:590-660: no
 allocation, no synchronisation, one launch an op, kernels re-entrant across graph replays): a launch
 train of every kind of launch this library makes -- fused decode linear, producer + GEMV, the decode
-pair, a tile GEMM whose law splits K (arrival counters), the quarter-tile 256x256 cell, a routed layer
+pair, the decode MLP chain, a tile GEMM whose law splits K (arrival counters), the quarter-tile 256x256 cell, a routed layer
 -- is captured into one HIP graph and replayed several times with other work in between; every
 replay's bytes equal the eager run's."""
 import numpy as np
@@ -61,6 +61,20 @@ def test_launch_train_replays_bit_identically(ctx):
     train.append(lambda: ctx.quant(xp.data_ptr(), qp.data_ptr(), sp.data_ptr(), M, K, stream=sh))
     train.append(lambda: ctx.gemm_pair(qp.data_ptr(), sp.data_ptr(), w0.data_ptr(), sd0.data_ptr(), c0.data_ptr(), n0,
                                        w1.data_ptr(), sd1.data_ptr(), c1.data_ptr(), n1, M, K, stream=sh))
+    # the decode MLP as one persistent launch: its workgroups meet through a state block whose
+    # generation the kernel itself advances, so a replay needs nothing cleared or re-stamped
+    Mc, Hc, Ic = 2, 1024, 2560
+    Wg, sg = synth.weights(rng, 2 * Ic, Hc, False)
+    Wd, sdn = synth.weights(rng, Hc, Ic, False)
+    xc = dev_bf16_bits(synth.activations(rng, Mc, Hc))
+    wg, wd, sgd, sdd = dev_u8(iu8.repack_w4(Wg)), dev_u8(iu8.repack_w4(Wd)), dev_f32(sg), dev_f32(sdn)
+    pc = torch.zeros((Mc, Ic), dtype=torch.int16, device="cuda")
+    cc = torch.zeros((Mc, Hc), dtype=torch.int16, device="cuda")
+    state = torch.zeros(iu8.MLP_CHAIN_STATE_BYTES // 4, dtype=torch.int32, device="cuda")
+    keep.extend([xc, wg, wd, sgd, sdd, pc, state])
+    outs.append(cc)
+    train.append(lambda: ctx.mlp_chain(xc.data_ptr(), wg.data_ptr(), sgd.data_ptr(), wd.data_ptr(), sdd.data_ptr(), None,
+                                       pc.data_ptr(), state.data_ptr(), cc.data_ptr(), Mc, Hc, Ic, stream=sh))
     # a routed layer (router's arrival counter, tile tables rebuilt every replay)
     case = synth.moe_case(T=150, E=128, topk=8, H=512, I=256, seed=3, experts=4)
     layer = MoeLayerIU8(ctx, 150, 128, 8, 512, 256)
