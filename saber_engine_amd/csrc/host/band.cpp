@@ -130,6 +130,27 @@ std::string band_toml() {
   put(o, "rows_max", 4);
   put(o, "staged_code_bytes", 20 * 1024);
   put(o, "column_blocks_per_workgroup_max", 8);
+  put(o, "threads", 1024);
+  put(o, "column_block", 32);
+  o += "# workgroups for b = ceil(n / 32) column blocks: b while b <= cu_count, else equal shares\n";
+  o += "# ceil(b / min(8, ceil(b / cu_count))); the layer shapes:\n";
+  for (const Shape &sh : SHAPES) {
+    saber_iu8_desc d;
+    if (resolve_fused(SABER_IU8_W4, 1, sh.n, sh.k, &d)) continue;
+    o += fmt("grid.%s = %u\n", sh.op, d.grid[0]);
+  }
+  o += "\n[mlp_chain]\n";
+  o += "# macaq_iu8f_mlp_w4_tm1: gate+up -> SiLU * up + requantisation -> down in one persistent launch while\n";
+  o += "# the rows fit the fused form at both widths; every workgroup resident (one a CU)\n";
+  put(o, "threads", 1024);
+  put(o, "state_bytes", MLP_CHAIN_STATE_BYTES);
+  put(o, "spin_default", MLP_CHAIN_SPIN);
+  put(o, "workgroups_max", MLP_CHAIN_MAX_GRID);
+  {
+    saber_iu8_desc d;
+    if (!resolve_mlp_chain(1, 5120, 17408, 0, &d)) o += fmt("grid.hidden5120_inter17408 = %u\n", d.grid[0]);
+    if (!resolve_mlp_chain(4, 5120, 5120, 0, &d)) o += fmt("grid.hidden5120_inter5120 = %u\n", d.grid[0]);
+  }
   o += "\n[pair]\n# block order by tm: true = the second problem's workgroups first (macaq_iu8f_pairb_*)\n";
   {
     saber_iu8_desc a, b, p;

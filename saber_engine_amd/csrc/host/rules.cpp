@@ -397,6 +397,12 @@ bool fused_holds(uint32_t m, uint32_t k) {
   return (uint64_t)mr * k <= 20 * 1024;
 }
 
+uint32_t fused_grid(uint32_t nblk) {
+  if (nblk <= CU_COUNT) return nblk;
+  const uint32_t per = std::min<uint32_t>(8, (nblk + CU_COUNT - 1) / CU_COUNT);
+  return (nblk + per - 1) / per;
+}
+
 int resolve_fused(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *d) {
   if (wkind != SABER_IU8_W4 && wkind != SABER_IU8_W8) return fail(SABER_IU8_E_ARG, "unknown weight kind");
   const char *op = wkind == SABER_IU8_W8 ? "linear_i8a8_fused" : "linear_i4a8_fused";
@@ -408,13 +414,11 @@ int resolve_fused(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc 
   copy_name(d->op, sizeof d->op, op);
   copy_name(d->plugin, sizeof d->plugin, "macaq_iu8");
   copy_name(d->kernel, sizeof d->kernel, name);
-  // 8 waves: 4 k-waves x 2 weight tiles = 32 columns a block. Persistent past two workgroups a CU
-  // (what its registers let reside): the workgroups walk the blocks, at most 8 each.
-  const uint32_t nblk = (n + 31) / 32, resident = 2 * CU_COUNT;
-  uint32_t grid = nblk;
-  if (nblk > resident) grid = std::max(resident, ((nblk + 7) / 8 + CU_COUNT - 1) / CU_COUNT * CU_COUNT);
-  d->grid[0] = grid, d->grid[1] = 1, d->grid[2] = 1;
-  d->block[0] = 512, d->block[1] = 1, d->block[2] = 1;
+  // 16 waves: 8 k-waves x 2 weight tiles = 32 columns a block, one workgroup a CU. Past one block a
+  // CU the workgroups walk the blocks in equal shares (1,088 blocks: 218 workgroups x 5, measured 15.8 us
+  // against 16.2 on 256 workgroups with 4 or 5), at most 8 each (the kernel's scale table).
+  d->grid[0] = fused_grid((n + 31) / 32), d->grid[1] = 1, d->grid[2] = 1;
+  d->block[0] = 1024, d->block[1] = 1, d->block[2] = 1;
   d->n_launches = 1;
   d->ks = 1;
   if (int rc = fill_slots(name, d)) return rc;
@@ -435,16 +439,18 @@ int resolve_mlp_chain(uint32_t m, uint32_t hidden, uint32_t inter, uint32_t spin
   if (!fused_holds(m, hidden) || !fused_holds(m, inter))
     return fail(SABER_IU8_E_RULE, fmt("%s: %u rows of %u / %u do not fit the fused form (at most 4 rows, 20 KiB of codes)", op, m,
                                       hidden, inter));
-  const uint32_t grid = 2 * CU_COUNT, nblk = std::max((2 * inter + 31) / 32, (hidden + 31) / 32);
-  if (nblk > 8 * grid)
-    return fail(SABER_IU8_E_RULE, fmt("%s: %u column blocks are more than the %u resident workgroups walk (8 each)", op, nblk, grid));
+  // the first linear walks inter / 16 paired tiles, the second hidden / 32 column blocks; one workgroup a CU
+  const uint32_t nblk = std::max(inter / 16, (hidden + 31) / 32);
+  if (nblk > 8 * CU_COUNT)
+    return fail(SABER_IU8_E_RULE, fmt("%s: %u column blocks are more than the %u resident workgroups walk (8 each)", op, nblk, CU_COUNT));
+  const uint32_t grid = std::max(fused_grid(inter / 16), fused_grid((hidden + 31) / 32));
   const char *name = "macaq_iu8f_mlp_w4_tm1";
   memset(d, 0, sizeof *d);
   copy_name(d->op, sizeof d->op, op);
   copy_name(d->plugin, sizeof d->plugin, "macaq_iu8f");
   copy_name(d->kernel, sizeof d->kernel, name);
   d->grid[0] = grid, d->grid[1] = 1, d->grid[2] = 1;
-  d->block[0] = 512, d->block[1] = 1, d->block[2] = 1;
+  d->block[0] = 1024, d->block[1] = 1, d->block[2] = 1;
   d->n_launches = 1;
   d->ks = 1;
   if (int rc = fill_slots(name, d)) return rc;

@@ -357,7 +357,7 @@ static int chain_guard(const LoadedKernel &lk, const saber_iu8_desc *d) {
       h % 128 || i % 128)
     return fail(SABER_IU8_E_RULE, fmt("%s: %lld rows of %lld / %lld do not fit the fused form", d->kernel, (long long)m, (long long)h,
                                       (long long)i));
-  const int64_t nblk = std::max((2 * i + 31) / 32, (h + 31) / 32);
+  const int64_t nblk = std::max(i / 16, (h + 31) / 32);
   if ((int64_t)d->grid[0] * 8 < nblk || d->grid[0] > MLP_CHAIN_MAX_GRID || d->grid[1] != 1 || d->grid[2] != 1 || i32_arg(d, "spin") <= 0)
     return fail(SABER_IU8_E_RULE, fmt("%s: grid %u x %u x %u: %lld column blocks at most 8 a workgroup, at most %u workgroups, a spin limit",
                                       d->kernel, d->grid[0], d->grid[1], d->grid[2], (long long)nblk, MLP_CHAIN_MAX_GRID));
@@ -380,7 +380,7 @@ static int launch_guard(const LoadedKernel &lk, const saber_iu8_desc *d) {
   if (m <= 0 || n <= 0 || k <= 0 || !fused_holds((uint32_t)m, (uint32_t)k))
     return fail(SABER_IU8_E_RULE, fmt("%s: %lld rows of %lld do not fit the fused form", d->kernel, (long long)m, (long long)k));
   const int64_t nblk = (n + 31) / 32;
-  if ((int64_t)d->grid[0] * 8 < nblk || d->grid[1] != 1 || d->grid[2] != 1 || d->block[0] != 512)
+  if ((int64_t)d->grid[0] * 8 < nblk || d->grid[1] != 1 || d->grid[2] != 1)
     return fail(SABER_IU8_E_RULE, fmt("%s: grid %u x %u x %u of %u threads cannot walk %lld column blocks (at most 8 a workgroup)",
                                       d->kernel, d->grid[0], d->grid[1], d->grid[2], d->block[0], (long long)nblk));
   return 0;

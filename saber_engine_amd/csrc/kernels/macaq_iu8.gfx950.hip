@@ -38,7 +38,12 @@
 // reference fuses producers the other way round (norm/activation + quant in front of an int8 GEMM,
 // crates/saber-kernels/hip/mxfp4_hadi8.hip); this is the same law inside the GEMV's prologue, where
 // it hides behind the first weight loads.
-#define IU8_DECQ(name, W8, D) IU8_DECQX(name, W8, 1, 4, 8, D)  /* the default decode cell's geometry */
+// Geometry: 16 waves a workgroup (one workgroup a CU, 4 waves a SIMD) as 8 k-waves x 2 column tiles, a
+// ring of 4 steps a wave. Measured against 8 waves (4 k-waves x 2 tiles, two workgroups a CU) with a ring
+// of 8 -- the same bytes in flight a CU: QKV 5.99 -> 5.56 us, O 5.57 -> 5.20, gate+up 16.4 -> 15.8, down
+// 12.8 -> 10.7 at one row: the rows' quantisation, which every workgroup repeats in front of its first
+// MFMA, is spread over twice the lanes, and a CU's waves all see one set of staged codes. Ring depths
+// 2/3/5/6 and 16 k-waves on 16-column blocks measured slower on every shape.
 #define IU8_DECQX(name, W8, NT, KW, WPB, D)                                                                            \
   extern "C" __global__ __launch_bounds__(WPB * 64) __attribute__((amdgpu_waves_per_eu(4, 4))) void name(              \
       const unsigned short *__restrict__ x, const unsigned char *__restrict__ w, const float *__restrict__ ws,     \
@@ -46,9 +51,8 @@
       int k) {                                                                                                     \
     iu8_decq_body<W8, NT, KW, WPB, D>(x, w, ws, q, scale, c, m, n, k);                                             \
   }
-IU8_DECQ(macaq_iu8_decq_w4_tm1, false, 8)
-IU8_DECQ(macaq_iu8_decq_w8_tm1, true, 4)
-#undef IU8_DECQ
+IU8_DECQX(macaq_iu8_decq_w4_tm1, false, 1, 8, 16, 4)
+IU8_DECQX(macaq_iu8_decq_w8_tm1, true, 1, 8, 16, 2)
 #undef IU8_DECQX
 
 // Cells with K split over gridDim.z (symbol suffix `_ks`, the decode kernarg list: the two workspaces

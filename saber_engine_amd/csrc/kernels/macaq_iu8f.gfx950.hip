@@ -39,12 +39,12 @@
 // (bf16 [m, 2n]) and `p` (bf16 [m, n]) are the launch's working rows; `state` is the 12 KiB block
 // the workgroups meet through (zero before the first launch, ready for the next after a launch that
 // completes; the word at 10 KiB + 8 non-zero: a meeting timed out, c is not valid).
-// The grid is the host's: every workgroup resident at once, at most 512 of them, at most 8 column
-// blocks of either linear a workgroup.
-extern "C" __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) void macaq_iu8f_mlp_w4_tm1(
+// The grid is the host's: every workgroup resident at once (one a CU: 16 waves), at most 512 of them,
+// at most 8 column blocks of either linear a workgroup.
+extern "C" __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4))) void macaq_iu8f_mlp_w4_tm1(
     const unsigned short *__restrict__ x, const unsigned char *__restrict__ w, const float *__restrict__ ws,
     const unsigned char *__restrict__ w_b, const float *__restrict__ ws_b, unsigned short *__restrict__ gu,
     unsigned short *__restrict__ p, unsigned char *__restrict__ state, unsigned short *__restrict__ c, int m, int k, int n,
     int spin) {
-  iu8_chain_mlp<1, 4, 8, 8>(x, w, ws, w_b, ws_b, gu, p, state, c, m, k, n, spin);
+  iu8_chain_mlp<1, 8, 16, 4>(x, w, ws, w_b, ws_b, gu, p, state, c, m, k, n, spin);
 }

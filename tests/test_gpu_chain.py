@@ -65,7 +65,8 @@ SHAPES = [(1, 5120, 17408), (4, 5120, 5120), (2, 2048, 10240), (3, 1408, 2944), 
 def test_chain_matches_the_oracle_and_the_three_launches(ctx, M, H, I):
     say(f"mlp chain M={M} H={H} I={I}")
     d = iu8.resolve_mlp_chain(M, H, I)
-    assert d.kernel == b"macaq_iu8f_mlp_w4_tm1" and d.grid[0] == 512 and d.block[0] == 512
+    assert d.kernel == b"macaq_iu8f_mlp_w4_tm1" and d.block[0] == 1024
+    assert d.grid[0] <= 256 and d.grid[0] * 8 >= max(I // 16, H // 32)      # one workgroup a CU, at most 8 blocks each
     assert {w.name: w.bytes for w in d.workspaces[:d.n_workspaces]} == {b"p": M * I * 2, b"state": iu8.MLP_CHAIN_STATE_BYTES}
     mlp = Mlp(M, H, I, seed=M + I)
     want_gu, want_p, want_c = mlp.oracle()
@@ -117,6 +118,10 @@ def test_chain_refuses_what_the_form_does_not_hold(ctx):
     with pytest.raises(iu8.IU8Error) as e:
         ctx.launch(d, bufs)
     assert e.value.code == iu8.E_RULE and "at most 512 workgroups" in str(e.value)
+    d.grid[0] = 300                                     # fits the state block, but one 16-wave workgroup a CU: 256 at once
+    with pytest.raises(iu8.IU8Error) as e:
+        ctx.launch(d, bufs)
+    assert e.value.code == iu8.E_RULE and "resident" in str(e.value)
     d.grid[0] = 8                                       # 128 column blocks of gate+up: more than 8 x 8
     with pytest.raises(iu8.IU8Error) as e:
         ctx.launch(d, bufs)

@@ -196,6 +196,19 @@ def test_band_table_is_the_launch_law():
     assert len(names) == 45 and names["macaq_iu8_pf_w4_tn4_lbk64"].startswith("same name") and names["macaq_iu8f_arnq_hadi8_w4_tm1"] == "none"
     assert t["moe"]["tile_blocks_1_last_tokens"] == 112 and t["moe"]["tile_blocks_8_last_tokens"] == 2047
     assert t["pair"]["second_first"] == [True] * 4
+    # the fused decode linear's grid law and the chain's, as the tables state them
+    f = t["fused_decode_linear"]
+    for op, grid in f["grid"].items():
+        n, k = next((b["n"], b["k"]) for b in t["band"] if b["op"] == op)
+        d = iu8.resolve_fused(iu8.W4, 1, n, k)
+        blocks = -(-n // f["column_block"])
+        assert d.grid[0] == grid and d.block[0] == f["threads"] and grid * f["column_blocks_per_workgroup_max"] >= blocks
+        assert grid == (blocks if blocks <= 256 else -(-blocks // min(8, -(-blocks // 256))))
+    assert f["grid"]["gate_up"] == 218 and f["grid"]["down"] == 160
+    c = t["mlp_chain"]
+    d = iu8.resolve_mlp_chain(1, 5120, 17408)
+    assert d.grid[0] == c["grid"]["hidden5120_inter17408"] <= 256 and d.block[0] == c["threads"]
+    assert d.workspace("state").bytes == c["state_bytes"] == iu8.MLP_CHAIN_STATE_BYTES and d.arg("spin").ival == c["spin_default"]
 
 
 def test_operands_past_4_gib_are_refused_by_the_tile_gemm():
