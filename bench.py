@@ -269,7 +269,7 @@ def main():
     # (the activation between them), so it is reported here and not part of `value`.
     mlp = None
     (_, n_gu, hid), (_, _, inter) = [l for l in linears if l[0] == "gate_up"][0], [l for l in linears if l[0] == "down"][0]
-    if fused and n_gu == 2 * inter and iu8.fused_holds(M, inter):
+    if fused and n_gu == 2 * inter and iu8.mlp_chain_holds(M, hid, inter):
         p_rows = torch.zeros((M, inter), dtype=torch.int16, device=dev)
         state = torch.zeros(iu8.MLP_CHAIN_STATE_BYTES // 4, dtype=torch.int32, device=dev)
         q_dn = torch.zeros(iu8.a_bytes(M, inter), dtype=torch.uint8, device=dev)

@@ -284,8 +284,10 @@ int saber_iu8_gemm_pair(saber_iu8_ctx *ctx, const void *a, const float *a_scale,
                         uint32_t n, const void *w_b, const float *w_scale_b, void *c_b, uint32_t n_b, uint32_t m, uint32_t k,
                         void *stream);
 
-/* The whole decode linear in one launch where the shape allows (at most 4 rows whose codes fit the
- * kernel's 20 KiB staging area; saber_iu8_fused_holds): per-token quantisation fused into the
+/* The whole decode linear in one launch where that is the faster form (saber_iu8_fused_holds: up to
+ * 4 rows whose codes, rows rounded up to a power of two, fit 20 KiB of LDS -- kernel `_tm1` -- or up
+ * to 3 rows in 80 KiB -- kernel `_tm1_a80`, which itself holds up to 16 rows and is reachable by name
+ * through saber_iu8_describe_raw): per-token quantisation fused into the
  * GEMV's activation staging. x bf16 [m,k]; q (A edge) and scale f32 [m] are optional outputs (NULL:
  * not stored) with the bytes saber_iu8_quant would write. Other shapes are refused
  * (SABER_IU8_E_RULE): run saber_iu8_quant + saber_iu8_gemm. No counterpart among the reference's
@@ -298,7 +300,7 @@ int saber_iu8_linear_fused(saber_iu8_ctx *ctx, int wkind, const void *x_bf16, co
 
 /* The dense decode MLP as ONE persistent launch: gate+up linear -> SiLU(gate) * up with its
  * per-token requantisation -> down linear, for at most 4 rows whose codes fit the fused form at both
- * widths (saber_iu8_fused_holds(m, hidden) and (m, inter)). The dense twin of the reference's routed
+ * widths (saber_iu8_mlp_chain_holds: at most 4 rows, 20 KiB of codes at hidden and at inter). The dense twin of the reference's routed
  * back half, which chains gate_up -> silu-quant -> down in one persistent launch with device-counter
  * hand-overs (crates/saber-kernels/hip/moe_grouped.hip:1656-1765, crates/saber-kernels/src/moe.rs:341-345);
  * its dense MLP is three launches (crates/saber-kernels/src/macaq_iu8.rs:864-875), whose bytes this
@@ -315,6 +317,7 @@ int saber_iu8_linear_fused(saber_iu8_ctx *ctx, int wkind, const void *x_bf16, co
  * three launches. Launches that share one `state` must not overlap. Asynchronous. */
 #define SABER_IU8_MLP_CHAIN_STATE_BYTES (12 * 1024)
 #define SABER_IU8_MLP_CHAIN_STATUS_OFFSET (10 * 1024 + 8)
+int saber_iu8_mlp_chain_holds(uint32_t m, uint32_t hidden, uint32_t inter);
 int saber_iu8_resolve_mlp_chain(uint32_t m, uint32_t hidden, uint32_t inter, uint32_t spin, saber_iu8_desc *out);
 int saber_iu8_mlp_chain(saber_iu8_ctx *ctx, const void *x_bf16, const void *w_gu, const float *ws_gu, const void *w_dn,
                         const float *ws_dn, void *gu, void *p, void *state, void *c, uint32_t m, uint32_t hidden, uint32_t inter,

@@ -388,14 +388,22 @@ static int describe_rows(const char *op, const char *kernel, uint32_t rows, uint
   return 0;
 }
 
-// The fused form quantises up to 4 rows whose int8 codes (rows rounded up to a power of two) fit
-// the kernel's 20 KiB staging area.
-bool fused_holds(uint32_t m, uint32_t k) {
-  if (m == 0 || m > 4) return false;
+// The fused forms quantise rows whose int8 codes (rows rounded up to a power of two) fit the kernel's
+// staging area: up to 4 rows in 20 KiB (`_tm1`), up to 16 rows in 80 KiB (`_tm1_a80`). Every workgroup
+// repeats the rows' quantisation (about 0.7 us a row of 5,120 on this card), a producer launch costs
+// about 3 us once: the law takes the 80 KiB form for up to 3 rows (down at 2 rows: 14.5 against 17.4 us
+// as producer + GEMV; at 4 rows 17.8 against 17.6; QKV at 5 / 8 / 16 rows 9.3 / 10.7 / 15.8 against
+// 8.8 / 8.9 / 9.4). The kernel itself holds what `fused_form_holds` says, by name.
+static uint64_t staged_bytes(uint32_t m, uint32_t k) {
   uint32_t mr = 1;
   while (mr < m) mr *= 2;
-  return (uint64_t)mr * k <= 20 * 1024;
+  return (uint64_t)mr * k;
 }
+bool fused_small_holds(uint32_t m, uint32_t k) { return m >= 1 && m <= 4 && staged_bytes(m, k) <= 20 * 1024; }
+bool fused_form_holds(bool a80, uint32_t m, uint32_t k) {
+  return a80 ? m >= 1 && m <= 16 && staged_bytes(m, k) <= 80 * 1024 : fused_small_holds(m, k);
+}
+bool fused_holds(uint32_t m, uint32_t k) { return fused_small_holds(m, k) || (m <= 3 && fused_form_holds(true, m, k)); }
 
 uint32_t fused_grid(uint32_t nblk) {
   if (nblk <= CU_COUNT) return nblk;
@@ -408,8 +416,8 @@ int resolve_fused(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc 
   const char *op = wkind == SABER_IU8_W8 ? "linear_i8a8_fused" : "linear_i4a8_fused";
   if (int rc = check_shape(op, m, n, k)) return rc;
   if (!fused_holds(m, k))
-    return fail(SABER_IU8_E_RULE, fmt("%s: %u rows of %u do not fit the fused form (at most 4 rows, 20 KiB of codes)", op, m, k));
-  const std::string name = fmt("macaq_iu8_decq_%s_tm1", wkind == SABER_IU8_W8 ? "w8" : "w4");
+    return fail(SABER_IU8_E_RULE, fmt("%s: %u rows of %u are not a fused launch (up to 4 rows in 20 KiB of codes, up to 3 rows in 80 KiB)", op, m, k));
+  const std::string name = fmt("macaq_iu8_decq_%s_tm1%s", wkind == SABER_IU8_W8 ? "w8" : "w4", fused_small_holds(m, k) ? "" : "_a80");
   memset(d, 0, sizeof *d);
   copy_name(d->op, sizeof d->op, op);
   copy_name(d->plugin, sizeof d->plugin, "macaq_iu8");
@@ -436,7 +444,7 @@ int resolve_mlp_chain(uint32_t m, uint32_t hidden, uint32_t inter, uint32_t spin
   if (inter > 0x3FFFFFFFu) return fail(SABER_IU8_E_RULE, fmt("%s: intermediate width %u", op, inter));
   if (int rc = check_shape(op, m, 2 * inter, hidden)) return rc;
   if (int rc = check_shape(op, m, hidden, inter)) return rc;
-  if (!fused_holds(m, hidden) || !fused_holds(m, inter))
+  if (!fused_small_holds(m, hidden) || !fused_small_holds(m, inter))
     return fail(SABER_IU8_E_RULE, fmt("%s: %u rows of %u / %u do not fit the fused form (at most 4 rows, 20 KiB of codes)", op, m,
                                       hidden, inter));
   // the first linear walks inter / 16 paired tiles, the second hidden / 32 column blocks; one workgroup a CU

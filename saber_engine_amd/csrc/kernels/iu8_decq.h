@@ -48,7 +48,7 @@ static __device__ __forceinline__ iu8_v4u iu8_decq_ld_coherent(const iu8_v4u *p)
   const unsigned long long hi = __hip_atomic_load((const unsigned long long *)p + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
   return iu8_v4u{(unsigned)lo, (unsigned)(lo >> 32), (unsigned)hi, (unsigned)(hi >> 32)};
 }
-template <bool W8, int NT, int KW, int WPB, int D, int CH = 0, class Hook = iu8_decq_nohook>
+template <bool W8, int NT, int KW, int WPB, int D, int CH = 0, class Hook = iu8_decq_nohook, int AKB = 20>
 __device__ __forceinline__ void iu8_decq_body(const unsigned short *__restrict__ X, const iu8_u8 *__restrict__ W,
                                               const float *__restrict__ ws, iu8_u8 *__restrict__ qout,
                                               float *__restrict__ sout, unsigned short *__restrict__ C, int M, int N,
@@ -61,11 +61,18 @@ __device__ __forceinline__ void iu8_decq_body(const unsigned short *__restrict__
   constexpr int NTHR = WPB * 64;
   constexpr int WSTEP = W8 ? 2048 : 1024;  // bytes of one 16-row weight tile per 128-deep K step
   constexpr int WV = W8 ? 2 : 1;           // 16-byte loads a lane per step per tile
-  constexpr int ABYTES = 20 * 1024;        // staged codes: pow2(M) * K bytes
+  constexpr int ABYTES = AKB * 1024;       // staged codes: pow2(M) * K bytes
+  // BIG (more than 20 KiB staged): up to 16 rows. The rows' maxima meet by LDS integer max (a wave's
+  // pieces of one load lie in one row when K is a multiple of 512: then one lane a wave), scales and
+  // reciprocals are made once a row by 16 lanes, and a lane reads its row's scale for the epilogue.
+  constexpr bool BIG = AKB > 20;
+  static_assert(!BIG || CH == 0, "the chain's forms stage at most 20 KiB");
   constexpr int RED = (KW - 1) * WN * NT * 256;  // ints of one partial area
   __shared__ __attribute__((aligned(16))) iu8_u8 s_a[ABYTES];
   __shared__ __attribute__((aligned(16))) int s_red[2][RED];
   __shared__ float s_amax[WPB][4];
+  __shared__ unsigned s_rowmax[BIG ? 16 : 1];
+  __shared__ float s_rsc[BIG ? 16 : 1], s_rrcp[BIG ? 16 : 1];
   __shared__ float s_ws[IU8_DECQ_MAXB][WN * NT * 16];  // the epilogue's weight scales (W4: already / 16)
   __shared__ __attribute__((aligned(8))) unsigned s_up[PAIRED ? 2 : 1][PAIRED ? 128 : 2];  // the up wave's bf16 values, two blocks
 
@@ -141,6 +148,67 @@ __device__ __forceinline__ void iu8_decq_body(const unsigned short *__restrict__
   // ---- quantise the rows: amax lane -> wave (butterfly) -> workgroup (LDS),
   // all order-free maxima; sc = max(amax / 127, 1e-30); codes by the exact reciprocal path
   float qsc[4] = {1.f, 1.f, 1.f, 1.f};
+  float my_sc = 1.f;  // BIG: the scale of this lane's row (ml)
+  if constexpr (BIG) {
+    if (tid < 16) s_rowmax[tid] = 0u;
+    __syncthreads();
+    const bool wave_rows = (k8 & 63) == 0;  // a wave's 64 pieces of one load lie in one row
+#pragma unroll
+    for (int p = 0; p < X_PER; ++p) {
+      const int piece = p * NTHR + tid;
+      const bool live = piece < x_pieces;
+      const int row = live ? piece / k8 : 0;
+      float m8 = 0.f;
+      if (live) {
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          m8 = fmaxf(m8, fabsf(__uint_as_float(xreg[p][w] << 16)));
+          m8 = fmaxf(m8, fabsf(__uint_as_float(xreg[p][w] & 0xFFFF0000u)));
+        }
+      }
+      if (wave_rows) {  // x_pieces is then a multiple of 64: a wave is live or not as a whole
+        m8 = iu8_wave_max_nonneg(m8);
+        if (lane == 0 && live) __hip_atomic_fetch_max(&s_rowmax[row], __float_as_uint(m8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      } else if (live) {
+        __hip_atomic_fetch_max(&s_rowmax[row], __float_as_uint(m8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < D; ++i)
+      if (i < TT) issue(i);
+#pragma unroll
+    for (int p = 0; p < WS_PER; ++p)
+      if (p * NTHR + tid < WS_ALL) (&s_ws[0][0])[p * NTHR + tid] = wsreg[p];
+    __syncthreads();
+    if (tid < 16) {
+      const float sc = fmaxf(__fdiv_rn(__uint_as_float(s_rowmax[tid]), 127.f), 1e-30f);
+      s_rsc[tid] = sc;
+      s_rrcp[tid] = __fdiv_rn(1.f, sc);
+    }
+    __syncthreads();
+    const bool out0 = blockIdx.x == 0 && qout != nullptr;
+    if (blockIdx.x == 0 && sout != nullptr && tid < M) sout[tid] = s_rsc[tid];
+    my_sc = s_rsc[ml];
+#pragma unroll
+    for (int p = 0; p < X_PER; ++p) {
+      const int piece = p * NTHR + tid;
+      if (piece >= x_pieces) continue;
+      const int row = piece / k8, k = (piece - row * k8) << 3;
+      const float sc = s_rsc[row], rcp = s_rrcp[row];
+      float f[8];
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        f[2 * w] = __uint_as_float(xreg[p][w] << 16);
+        f[2 * w + 1] = __uint_as_float(xreg[p][w] & 0xFFFF0000u);
+      }
+      const unsigned d0 = iu8_code4_rcp(f[0], f[1], f[2], f[3], sc, rcp);
+      const unsigned d1 = iu8_code4_rcp(f[4], f[5], f[6], f[7], sc, rcp);
+      const int kt = k >> 6, g = (k >> 4) & 3, half = (k >> 3) & 1;
+      *(iu8_v2u *)&s_a[((((kt * 4 + g) << mr_shift) + row) << 4) + half * 8] = iu8_v2u{d0, d1};
+      if (out0) *(iu8_v2u *)(qout + (size_t)kt * 1024 + (row + 16 * g) * 16 + half * 8) = iu8_v2u{d0, d1};
+    }
+    __syncthreads();
+  } else
   {
     if constexpr (CH == 2) {
       // the chain's second linear: weights first (they do not depend on the first linear), then the
@@ -283,7 +351,7 @@ __device__ __forceinline__ void iu8_decq_body(const unsigned short *__restrict__
       for (int q = 0; q < KW - 1; ++q)
 #pragma unroll
         for (int j = 0; j < NT; ++j) acc[j] += *(const iu8_v4i *)&red[((q * WN + wn) * NT + j) * 256 + lane * 4];
-      const float am = ml == 0 ? qsc[0] : ml == 1 ? qsc[1] : ml == 2 ? qsc[2] : qsc[3];
+      const float am = BIG ? my_sc : ml == 0 ? qsc[0] : ml == 1 ? qsc[1] : ml == 2 ? qsc[2] : qsc[3];
       if constexpr (PAIRED) {
         const int tile = (int)blockIdx.x + cb * G;
         const float *wsu = &s_ws[min(cb, IU8_DECQ_MAXB - 1)][wn * 16 + lg * 4];

@@ -44,16 +44,22 @@
 // 12.8 -> 10.7 at one row: the rows' quantisation, which every workgroup repeats in front of its first
 // MFMA, is spread over twice the lanes, and a CU's waves all see one set of staged codes. Ring depths
 // 2/3/5/6 and 16 k-waves on 16-column blocks measured slower on every shape.
-#define IU8_DECQX(name, W8, NT, KW, WPB, D)                                                                            \
+// `_a80`: the same launch for up to 16 rows whose codes (rows rounded up to a power of two) fit 80 KiB of
+// LDS -- 16 rows of K = 5120, 4 rows of K = 17408 -- in place of a producer launch + GEMV.
+#define IU8_DECQX(name, W8, NT, KW, WPB, D) IU8_DECQA(name, W8, NT, KW, WPB, D, 20)
+#define IU8_DECQA(name, W8, NT, KW, WPB, D, AKB)                                                                       \
   extern "C" __global__ __launch_bounds__(WPB * 64) __attribute__((amdgpu_waves_per_eu(4, 4))) void name(              \
       const unsigned short *__restrict__ x, const unsigned char *__restrict__ w, const float *__restrict__ ws,     \
       unsigned char *__restrict__ q, float *__restrict__ scale, unsigned short *__restrict__ c, int m, int n,      \
       int k) {                                                                                                     \
-    iu8_decq_body<W8, NT, KW, WPB, D>(x, w, ws, q, scale, c, m, n, k);                                             \
+    iu8_decq_body<W8, NT, KW, WPB, D, 0, iu8_decq_nohook, AKB>(x, w, ws, q, scale, c, m, n, k);                    \
   }
 IU8_DECQX(macaq_iu8_decq_w4_tm1, false, 1, 8, 16, 4)
 IU8_DECQX(macaq_iu8_decq_w8_tm1, true, 1, 8, 16, 2)
+IU8_DECQA(macaq_iu8_decq_w4_tm1_a80, false, 1, 8, 16, 4, 80)
+IU8_DECQA(macaq_iu8_decq_w8_tm1_a80, true, 1, 8, 16, 2, 80)
 #undef IU8_DECQX
+#undef IU8_DECQA
 
 // Cells with K split over gridDim.z (symbol suffix `_ks`, the decode kernarg list: the two workspaces
 // in front of c), for the rows between the regimes, where few tiles leave CUs idle. Measured, the

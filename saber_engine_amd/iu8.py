@@ -116,6 +116,7 @@ def lib():
         L.saber_iu8_static_workspace_bytes.restype = C.c_uint64
         L.saber_iu8_gemm_acc.argtypes = [C.c_void_p, C.c_int] + [C.c_void_p] * 3 + [C.c_uint32] * 3 + [C.c_void_p]
         L.saber_iu8_fused_holds.argtypes = [C.c_uint32, C.c_uint32]
+        L.saber_iu8_mlp_chain_holds.argtypes = [C.c_uint32] * 3
         L.saber_iu8_pair.argtypes = [C.POINTER(Desc)] * 3
         L.saber_iu8_pair_ordered.argtypes = [C.POINTER(Desc)] * 2 + [C.c_int, C.POINTER(Desc)]
         L.saber_iu8_load_plugin.argtypes = [C.c_void_p, C.c_char_p]
@@ -193,6 +194,18 @@ def band_toml():
 
 def fused_holds(m, k):
     return bool(lib().saber_iu8_fused_holds(m, k))
+
+
+def fused_small_holds(m, k):
+    """Up to 4 rows whose codes fit 20 KiB: the `_tm1` fused kernel."""
+    mr = 1
+    while mr < m:
+        mr *= 2
+    return 1 <= m <= 4 and mr * k <= 20 * 1024
+
+
+def mlp_chain_holds(m, hidden, inter):
+    return bool(lib().saber_iu8_mlp_chain_holds(m, hidden, inter))
 
 
 def resolve_fused(wkind, m, n, k):

@@ -47,7 +47,7 @@ def test_config1_decode_layer_set_as_the_fused_launches_the_benchmark_times(ctx,
     """The hot path as bench.py launches it: one fused quant + GEMV launch a linear
     (macaq_iu8_decq_w4_tm1), on the four full layer shapes, against the oracle."""
     for name, n, k in synth.LAYER_LINEARS:
-        if not iu8.fused_holds(M, k):          # down at M = 4: 4 x 17408 codes do not fit the staged form
+        if not iu8.fused_holds(M, k):          # down at M = 4: producer + GEMV is the faster form
             assert (name, M) == ("down", 4)
             continue
         say(f"config 1, fused launch: {name} M={M} N={n} K={k}")

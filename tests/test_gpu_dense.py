@@ -91,9 +91,48 @@ def test_fused_linear_walks_column_blocks(ctx, M, N, K, grid):
         assert e.value.code == iu8.E_RULE
 
 
+@pytest.mark.parametrize("M,N,K,grid", [(2, 5120, 17408, None),    # what the law launches it for: down at 2 and 3 rows
+                                          (3, 352, 17408, None),
+                                          (16, 480, 5120, None),     # the most rows; K a multiple of 512: a wave's pieces lie in one row
+                                          (16, 7168, 5120, None),
+                                          (9, 208, 4992, 2),         # K = 39 steps, not a multiple of 512: rows change inside a wave
+                                          (5, 1104, 640, 5),         # several blocks a workgroup, an odd tile count, k-waves with no step
+                                          (4, 96, 17408, None),      # 4 rows of the widest K
+                                          (1, 64, 128, None)])       # one step
+def test_fused_decode_linear_80_kib_form(ctx, M, N, K, grid):
+    """macaq_iu8_decq_{w4,w8}_tm1_a80: up to 16 rows staged in 80 KiB, the bytes of producer + GEMV.
+    The law launches it for up to 3 rows; the other shapes reach it by name."""
+    for w8 in (False, True):
+        say(f"fused decode linear, 80 KiB form: M={M} N={N} K={K} grid={grid} w8={w8}")
+        case = synth.dense_case(M, N, K, w8=w8, seed=31 + M)
+        r = ref.linear(case["X"], case["W"], case["ws"], w8, threads=8)
+        wk, tag = (iu8.W8, "w8") if w8 else (iu8.W4, "w4")
+        x, wf, ws = dev_bf16_bits(case["X"]), dev_u8(iu8.repack_weights(case["W"], w8)), dev_f32(case["ws"])
+        c = torch.full((M, N), 0x7FC0, dtype=torch.int16, device="cuda")
+        q = torch.full((iu8.a_bytes(M, K),), 0x55, dtype=torch.uint8, device="cuda")
+        s = torch.zeros(M, dtype=torch.float32, device="cuda")
+        if M <= 3 and grid is None and not iu8.fused_small_holds(M, K):
+            d = iu8.resolve_fused(wk, M, N, K)
+            assert d.kernel.decode() == f"macaq_iu8_decq_{tag}_tm1_a80" and d.block[0] == 1024
+        else:
+            nblk = (N + 31) // 32
+            d = iu8.describe_raw(f"macaq_iu8_decq_{tag}_tm1_a80", (grid or min(nblk, 256), 1, 1), 1024, m=M, n=N, k=K)
+        ctx.launch(d, dict(x=x.data_ptr(), w=wf.data_ptr(), ws=ws.data_ptr(), c=c.data_ptr(), q=q.data_ptr(), scale=s.data_ptr()))
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(host_u16(c), r["C"])
+        np.testing.assert_array_equal(iu8.unpack_a(q.cpu().numpy(), M, K), r["q"])
+        np.testing.assert_array_equal(s.cpu().numpy().view(np.uint32), r["a_scale"].view(np.uint32))
+    # what the kernel does not hold is refused at launch, by name
+    d = iu8.describe_raw("macaq_iu8_decq_w4_tm1_a80", (1, 1, 1), 1024, m=17, n=64, k=128)
+    with pytest.raises(iu8.IU8Error) as e:
+        ctx.launch(d, dict(x=x.data_ptr(), w=wf.data_ptr(), ws=ws.data_ptr(), c=c.data_ptr(), q=q.data_ptr(), scale=s.data_ptr()))
+    assert e.value.code == iu8.E_RULE
+
+
 def test_fused_form_refuses_what_it_does_not_hold(ctx):
-    assert not iu8.fused_holds(5, 1024) and not iu8.fused_holds(2, 17408) and not iu8.fused_holds(4, 5248)
+    assert not iu8.fused_holds(5, 1024) and not iu8.fused_holds(4, 17408) and not iu8.fused_holds(4, 5248)
     assert iu8.fused_holds(1, 17408) and iu8.fused_holds(4, 5120) and iu8.fused_holds(2, 10240)
+    assert iu8.fused_holds(2, 17408) and iu8.fused_holds(3, 17408) and not iu8.fused_small_holds(2, 17408)   # the 80 KiB form
     with pytest.raises(iu8.IU8Error) as e:
         iu8.resolve_fused(iu8.W4, 5, 256, 1024)
     assert e.value.code == iu8.E_RULE
