@@ -335,7 +335,8 @@ uint32_t pf_split(bool w8, uint32_t m, uint32_t n, uint32_t k, const PfVariant *
 // band tables (crates/saber-kernels/src/macaq_iu8.rs:150-212).
 const PfVariant *pf_cell(bool w8, uint32_t m, uint32_t n, uint32_t k) {
   static const struct { const char *tile; double tops_per_cu; } CELLS[] = {
-      {"tn4_lbk64", 13.27}, {"t256x224", 11.27}, {"t256x160", 9.98}, {"t128x128", 7.85},
+      {"tn4_lbk64", 13.27}, {"t256x320", 12.8}, {"t256x224", 11.27}, {"t128x320", 10.45}, {"t256x160", 9.98},
+      {"t128x256", 8.8},    {"t128x128", 7.85},
       {"t128x128_o2", 8.68}, {"t128x64_s", 6.21}, {"t64x128_s", 7.24}, {"t64x64_s", 5.96}};
   constexpr double FIXED_US = 2.78, CU_GBPS = 90.0, L2_TBPS = 17.7;
   const PfVariant *best = nullptr;

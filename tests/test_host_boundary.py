@@ -275,11 +275,15 @@ def test_prefill_launch_is_persistent_and_covers_the_output():
 
 def test_prefill_cells_of_the_benchmark_shapes():
     # speed data of this card: the cell that was fastest in the sweep of each shape
-    want = {(2048, 34816, 5120): "tn4_lbk64", (2048, 7168, 5120): "tn4_lbk64", (2048, 5120, 17408): "t256x160",
-            (2048, 5120, 5120): "t256x160", (8192, 34816, 5120): "tn4_lbk64",
+    want = {(2048, 34816, 5120): "tn4_lbk64", (2048, 7168, 5120): "tn4_lbk64", (2048, 5120, 17408): "t128x320",
+            (2048, 5120, 5120): "t128x320", (8192, 34816, 5120): "tn4_lbk64",
+            # N = 5120 is 16 column blocks of 320: two even rounds of 256 x 320 tiles at 8,192 rows
+            (8192, 5120, 17408): "t256x320", (8192, 5120, 5120): "t256x320", (4096, 5120, 17408): "t256x320",
+            (512, 34816, 5120): "t256x320",
             # up to M of about 512 the launch is bound by what the CUs pull from L2: small tiles on every CU
-            (256, 5120, 17408): "t64x128_s", (128, 5120, 17408): "t64x128_s_ks", (128, 5120, 5120): "t64x64_s", (256, 34816, 5120): "t256x160",
-            (1024, 5120, 5120): "t128x128_o2", (1024, 7168, 5120): "t128x128_o2"}
+            (256, 5120, 17408): "t64x128_s", (128, 5120, 17408): "t64x128_s_ks", (128, 5120, 5120): "t64x64_s", (256, 34816, 5120): "t128x320",
+            (1024, 5120, 5120): "t128x256", (1024, 7168, 5120): "t128x256", (512, 5120, 5120): "t128x128"}
+    assert iu8.resolve(iu8.W8, 8192, 5120, 17408).kernel.decode() == "macaq_iu8_pf_w8_tn4_lbk64"      # no int8-weight 256 x 320 cell
     for (m, n, k), tile in want.items():
         assert iu8.resolve(iu8.W4, m, n, k).kernel.decode() == "macaq_iu8_pf_w4_" + tile, (m, n, k)
     with pytest.raises(iu8.IU8Error):
