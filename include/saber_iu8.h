@@ -143,6 +143,14 @@ int saber_iu8_describe(const char *kernel, uint32_t m, uint32_t n, uint32_t k, u
  * this library. *need (optional) receives the bytes required; buf may be NULL to ask for it. */
 int saber_iu8_band_toml(char *buf, size_t cap, size_t *need);
 
+/* The target as the planner's DeviceProfile (crates/saber-plan/src/device.rs:168-193; the reference's
+ * gfx1201 instance: device.rs:208-258) as TOML text in that struct's field names and serde shape:
+ * CU count, LDS, wave sizes, capability bits, the matrix shapes, Infinity Cache and VRAM sizes, and
+ * the bandwidths with their provenance (DRAM measured on this card; PCIe and xGMI nominal: never
+ * valid for sizing, as the reference says of such numbers). Committed as
+ * prebuilt/gfx950/device_profile.toml; same calling convention as saber_iu8_band_toml. */
+int saber_iu8_device_profile_toml(char *buf, size_t cap, size_t *need);
+
 /* The activation producer's descriptor (i8_twin's role, macaq_iu8.rs:881-916): bf16 [m,k] rows
  * -> int8 A edge + f32 scales. */
 int saber_iu8_resolve_quant(uint32_t m, uint32_t k, saber_iu8_desc *out);

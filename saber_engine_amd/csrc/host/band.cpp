@@ -264,7 +264,67 @@ std::string band_toml() {
   return o;
 }
 
+// The target as the planner's DeviceProfile would hold it (crates/saber-plan/src/device.rs:168-193; the
+// gfx1201 instance: device.rs:208-258), in that struct's field names and its serde shape (an enum
+// variant with fields is a one-key table, a unit variant a string), so the Rust side can read it with
+// the derive it already has. The matrix shapes are this target's MFMA forms under the struct's WMMA name.
+std::string device_profile_toml() {
+  std::string o;
+  o += "# gfx950 (MI355X) as crates/saber-plan/src/device.rs::DeviceProfile: field names and serde shape of that\n";
+  o += "# struct. Written by saber_iu8_device_profile_toml; the build step regenerates it.\n";
+  put(o, "gfx_target", std::string("gfx950"));
+  put(o, "name", std::string("AMD Instinct MI355X"));
+  put(o, "cu_count", CU_COUNT);
+  put(o, "lds_bytes", 160 * 1024);
+  o += "wave_sizes = [64]\n";
+  put(o, "infinity_cache_bytes", 256ull << 20);
+  put(o, "vram_bytes", 288ull << 30);
+  o += "\n[caps]\n";
+  putb(o, "fp8_wmma", true);
+  putb(o, "int8_wmma", true);
+  putb(o, "int4_wmma", false);  // no int4 matrix form: W4 is unpacked to int8 in registers
+  putb(o, "sparse_2_4_swmmac", true);
+  putb(o, "lds_dma", true);
+  putb(o, "nontemporal_loads", true);
+  putb(o, "lds_transpose_read", true);
+  o += "\n[bandwidths.dram]\n";
+  o += "# a streaming read of 1 GiB (four times the Infinity Cache), every workgroup a contiguous span; a\n";
+  o += "# grid-stride walk reads 5,000-6,800; the published figure is 8,000\n";
+  o += "gbs = 7050.0\n";
+  o += "source = { measured_here = { harness = \"iu8_probe_read, 1 GiB in contiguous spans\", when = \"2026-11-25\" } }\n";
+  o += "\n[bandwidths.pcie_h2d]\ngbs = 64.0\nsource = \"nominal\"\n";
+  o += "\n[bandwidths.p2p]\n# one xGMI link; this build runs on one GPU and never measured it\ngbs = 153.6\nsource = \"nominal\"\n";
+  struct Shape { uint32_t m, n, k; const char *ab, *acc; bool sparse; };
+  static const Shape MFMA[] = {
+      {16, 16, 64, "iu8", "i32", false},      {32, 32, 32, "iu8", "i32", false},     {16, 16, 32, "bf16", "f32", false},
+      {32, 32, 16, "bf16", "f32", false},     {16, 16, 32, "fp16", "f32", false},    {32, 32, 16, "fp16", "f32", false},
+      {16, 16, 128, "fp8_e4m3", "f32", false}, {32, 32, 64, "fp8_e4m3", "f32", false}, {16, 16, 128, "fp8_e5m2", "f32", false},
+      {32, 32, 64, "fp8_e5m2", "f32", false},  {16, 16, 128, "iu8", "i32", true},      {32, 32, 64, "iu8", "i32", true}};
+  for (const Shape &w : MFMA) {
+    o += "\n[[wmma_shapes]]\n";
+    put(o, "m", w.m);
+    put(o, "n", w.n);
+    put(o, "k", w.k);
+    put(o, "a_dtype", std::string(w.ab));
+    put(o, "b_dtype", std::string(w.ab));
+    put(o, "acc_dtype", std::string(w.acc));
+    putb(o, "sparse_2_4", w.sparse);
+  }
+  return o;
+}
+
 }  // namespace iu8
+
+static int text_out(const std::string &t, const char *what, char *buf, size_t cap, size_t *need) {
+  if (need) *need = t.size() + 1;
+  if (!buf || cap < t.size() + 1) return buf ? iu8::fail(SABER_IU8_E_ARG, std::string(what) + ": buffer too small") : 0;
+  memcpy(buf, t.c_str(), t.size() + 1);
+  return 0;
+}
+
+extern "C" int saber_iu8_device_profile_toml(char *buf, size_t cap, size_t *need) {
+  return text_out(iu8::device_profile_toml(), "device_profile_toml", buf, cap, need);
+}
 
 extern "C" int saber_iu8_band_toml(char *buf, size_t cap, size_t *need) {
   const std::string t = iu8::band_toml();

@@ -23,6 +23,7 @@ struct MpVal {
 struct MpReader {
   const uint8_t *p, *end;
   bool ok = true;
+  int depth = 0;  // containers open: a note nests four or five deep; a crafted one must not eat the stack
   uint64_t be(int n) {
     if (end - p < n) {
       ok = false;
@@ -55,10 +56,15 @@ struct MpReader {
   }
   MpVal value() {
     MpVal v;
-    if (p >= end) {
+    if (p >= end || depth > 32) {
       ok = false;
       return v;
     }
+    struct Nest {
+      int &d;
+      explicit Nest(int &x) : d(x) { ++d; }
+      ~Nest() { --d; }
+    } nest(depth);
     const uint8_t t = *p++;
     if (t <= 0x7f) { v.kind = MpVal::Int; v.i = t; }
     else if (t >= 0xe0) { v.kind = MpVal::Int; v.i = (int8_t)t; }
@@ -131,7 +137,9 @@ static bool parse_elf(const std::vector<uint8_t> &b, size_t base, size_t size, C
   rd(b, base + 58, shentsize);
   rd(b, base + 60, shnum);
   if (machine != 224) return bad("ELF machine is not EM_AMDGPU");
-  if (shoff == 0 || shentsize < 64 || shoff + (uint64_t)shentsize * shnum > size) return bad("bad section table");
+  uint64_t sh_end = 0;
+  if (shoff == 0 || shentsize < 64 || __builtin_add_overflow(shoff, (uint64_t)shentsize * shnum, &sh_end) || sh_end > size)
+    return bad("bad section table");
   for (uint16_t i = 0; i < shnum; ++i) {
     const size_t sh = base + shoff + (size_t)i * shentsize;
     uint32_t type = 0;
@@ -139,7 +147,8 @@ static bool parse_elf(const std::vector<uint8_t> &b, size_t base, size_t size, C
     rd(b, sh + 4, type);
     rd(b, sh + 24, off);
     rd(b, sh + 32, sz);
-    if (type != 7 /* SHT_NOTE */ || off + sz > size) continue;
+    uint64_t sec_end = 0;
+    if (type != 7 /* SHT_NOTE */ || __builtin_add_overflow(off, sz, &sec_end) || sec_end > size) continue;
     size_t p = base + off;
     const size_t end = p + sz;
     while (p + 12 <= end) {

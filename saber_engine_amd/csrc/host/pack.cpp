@@ -202,7 +202,9 @@ extern "C" int saber_iu8_pack_open(const char *path, const uint8_t *expected_pla
     if (r.data_off < cursor)
       return bad(fmt("record %u (%s): data_off %llu is below %llu; the table must be sorted by data_off and records must not overlap after padding",
                      i, r.name, (unsigned long long)r.data_off, (unsigned long long)cursor));
-    if (r.length > h.file_bytes || align_up(r.data_off + r.length) > h.file_bytes)
+    uint64_t rec_end = 0;  // a data_off near 2^64 must not wrap past the check
+    if (r.length > h.file_bytes || __builtin_add_overflow(r.data_off, r.length, &rec_end) || rec_end > h.file_bytes ||
+        align_up(rec_end) > h.file_bytes)
       return bad(fmt("record %u (%s): runs past file_bytes", i, r.name));
     unsigned __int128 bits = dtype_bits(r.dtype);
     for (uint32_t d = 0; d < r.ndim; ++d) {

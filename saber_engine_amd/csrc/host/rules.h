@@ -66,6 +66,7 @@ int resolve_quant_rows(uint32_t rows, uint32_t k, saber_iu8_desc *out);
 // The reference's symbol names this object answers through its launch law (band.cpp).
 int ref_symbol_by_law(const std::string &kernel, int *w8, const char **note);
 std::string band_toml();
+std::string device_profile_toml();
 
 // Fills name/offset/size of every slot from the kernel's signature; kinds default to BUFFER.
 int fill_slots(const std::string &kernel, saber_iu8_desc *d);

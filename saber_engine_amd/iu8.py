@@ -20,6 +20,7 @@ PREBUILT = os.path.join(ROOT, "prebuilt", "gfx950")
 # the parity suite's test-only object (accumulator and table taps), outside the plugin directory
 TAPS_MANIFEST = os.path.join(PREBUILT, "taps", "iu8_taps.manifest.toml")
 BAND_TABLE = os.path.join(PREBUILT, "macaq_iu8.band.toml")
+DEVICE_PROFILE = os.path.join(PREBUILT, "device_profile.toml")
 
 W4, W8 = 0, 1
 ARG_BUFFER, ARG_NULL_BUFFER, ARG_I32, ARG_F32, ARG_I64 = 0, 1, 2, 3, 4
@@ -121,6 +122,7 @@ def lib():
         L.saber_iu8_pair_ordered.argtypes = [C.POINTER(Desc)] * 2 + [C.c_int, C.POINTER(Desc)]
         L.saber_iu8_load_plugin.argtypes = [C.c_void_p, C.c_char_p]
         L.saber_iu8_band_toml.argtypes = [C.c_char_p, C.c_size_t, C.POINTER(C.c_size_t)]
+        L.saber_iu8_device_profile_toml.argtypes = [C.c_char_p, C.c_size_t, C.POINTER(C.c_size_t)]
         L.saber_iu8_gemm_pair.argtypes = [C.c_void_p] * 6 + [C.c_uint32] + [C.c_void_p] * 3 + [C.c_uint32] * 3 + [C.c_void_p]
         L.saber_iu8_linear_fused.argtypes = [C.c_void_p, C.c_int] + [C.c_void_p] * 6 + [C.c_uint32] * 3 + [C.c_void_p]
         L.saber_iu8_resolve_mlp_chain.argtypes = [C.c_uint32] * 4 + [C.c_void_p]
@@ -189,6 +191,15 @@ def band_toml():
     lib().saber_iu8_band_toml(None, 0, C.byref(need))
     buf = C.create_string_buffer(need.value)
     _check(lib().saber_iu8_band_toml(buf, need.value, None))
+    return buf.value.decode()
+
+
+def device_profile_toml():
+    """The target's DeviceProfile as TOML text (what the build step writes to DEVICE_PROFILE)."""
+    need = C.c_size_t(0)
+    lib().saber_iu8_device_profile_toml(None, 0, C.byref(need))
+    buf = C.create_string_buffer(need.value)
+    _check(lib().saber_iu8_device_profile_toml(buf, need.value, None))
     return buf.value.decode()
 
 

@@ -37,6 +37,7 @@ PLUGINS = ("macaq_iu8", "macaq_iu8f", "macaq_i8q", "mxfp4_hadi8", "attn_glue_had
 TAPS = ("iu8_taps",)
 TAPS_DIR = os.path.join(PREBUILT, "taps")
 BAND = os.path.join(PREBUILT, "macaq_iu8.band.toml")
+DEVICE_PROFILE = os.path.join(PREBUILT, "device_profile.toml")
 
 
 def candidates(stem, arch):
@@ -117,21 +118,33 @@ def build_plugin(stem, out_dir=PREBUILT):
     return hsaco, manifest
 
 
+def _text_of(entry):
+    L = _lib()
+    fn = getattr(L, entry)
+    need = ctypes.c_size_t(0)
+    fn(None, ctypes.c_size_t(0), ctypes.byref(need))
+    buf = ctypes.create_string_buffer(need.value)
+    if fn(buf, ctypes.c_size_t(need.value), None) != 0:
+        raise RuntimeError(entry + ": " + L.saber_iu8_last_error().decode())
+    return buf.value.decode()
+
+
 def band_text():
     """The launch law as TOML text, straight from the host library."""
-    L = _lib()
-    need = ctypes.c_size_t(0)
-    L.saber_iu8_band_toml(None, ctypes.c_size_t(0), ctypes.byref(need))
-    buf = ctypes.create_string_buffer(need.value)
-    if L.saber_iu8_band_toml(buf, ctypes.c_size_t(need.value), None) != 0:
-        raise RuntimeError("band table: " + L.saber_iu8_last_error().decode())
-    return buf.value.decode()
+    return _text_of("saber_iu8_band_toml")
+
+
+def device_profile_text():
+    """The target's DeviceProfile as TOML text, straight from the host library."""
+    return _text_of("saber_iu8_device_profile_toml")
 
 
 def write_band(path=BAND):
     os.makedirs(os.path.dirname(path), exist_ok=True)
     with open(path, "w") as f:
         f.write(band_text())
+    with open(DEVICE_PROFILE, "w") as f:
+        f.write(device_profile_text())
     return path
 
 

@@ -211,6 +211,31 @@ def test_band_table_is_the_launch_law():
     assert d.workspace("state").bytes == c["state_bytes"] == iu8.MLP_CHAIN_STATE_BYTES and d.arg("spin").ival == c["spin_default"]
 
 
+def test_device_profile_is_the_planners_struct_as_data():
+    """prebuilt/gfx950/device_profile.toml carries every field of the planner's DeviceProfile
+    (crates/saber-plan/src/device.rs:168-193) in its serde shape, is what the library writes today, and
+    agrees with the launch law's own constants; no bandwidth is given without its provenance."""
+    import tomli
+
+    text = open(iu8.DEVICE_PROFILE).read()
+    assert text == iu8.device_profile_toml(), "stale device profile: run python -m saber_engine_amd.kbuild"
+    p = tomli.loads(text)
+    assert set(p) == {"gfx_target", "name", "cu_count", "wmma_shapes", "lds_bytes", "wave_sizes", "caps", "bandwidths",
+                      "infinity_cache_bytes", "vram_bytes"}
+    assert p["gfx_target"] == "gfx950" and p["wave_sizes"] == [64] and p["lds_bytes"] == 160 * 1024
+    assert p["cu_count"] == tomli.loads(open(iu8.BAND_TABLE).read())["cu_count"] == 256
+    assert set(p["caps"]) == {"fp8_wmma", "int8_wmma", "int4_wmma", "sparse_2_4_swmmac", "lds_dma", "nontemporal_loads", "lds_transpose_read"}
+    assert p["caps"]["int8_wmma"] and p["caps"]["lds_dma"] and not p["caps"]["int4_wmma"]
+    for w in p["wmma_shapes"]:
+        assert set(w) == {"m", "n", "k", "a_dtype", "b_dtype", "acc_dtype", "sparse_2_4"}
+    dense_i8 = {(w["m"], w["n"], w["k"]) for w in p["wmma_shapes"] if w["a_dtype"] == "iu8" and not w["sparse_2_4"]}
+    assert dense_i8 == {(16, 16, 64), (32, 32, 32)}           # the two forms the decode and the tile GEMM are written on
+    assert set(p["bandwidths"]) == {"dram", "pcie_h2d", "p2p"}
+    dram = p["bandwidths"]["dram"]
+    assert 5000 < dram["gbs"] < 8000 and set(dram["source"]["measured_here"]) == {"harness", "when"}
+    assert p["bandwidths"]["pcie_h2d"]["source"] == "nominal" and p["bandwidths"]["p2p"]["source"] == "nominal"
+
+
 def test_operands_past_4_gib_are_refused_by_the_tile_gemm():
     with pytest.raises(iu8.IU8Error) as e:
         iu8.resolve(iu8.W4, 300000, 5120, 17408)            # A: 300,000 x 17,408 bytes
@@ -399,6 +424,39 @@ def test_tampered_code_object_is_refused(tmp_path):
     open(tmp_path / "macaq_iu8.hsaco", "wb").write(bytes(blob))
     rc, refusal, _ = iu8.manifest_validate(path)
     assert rc in (iu8.E_VALIDATE, iu8.E_PARSE)
+
+
+def _elf_with_note(desc, sh_offset=None, sh_size=None):
+    """A minimal little-endian ELF64 for EM_AMDGPU whose only real section is one metadata note."""
+    note = struct.pack("<III", 7, len(desc), 32) + b"AMDGPU\0\0" + desc + b"\0" * (-len(desc) % 4)
+    off = 64
+    shoff = off + len(note)
+    hdr = bytearray(64)
+    hdr[0:6] = b"\x7fELF\x02\x01"
+    struct.pack_into("<HH", hdr, 16, 3, 224)
+    struct.pack_into("<Q", hdr, 40, shoff)
+    struct.pack_into("<HHHHHH", hdr, 52, 64, 0, 0, 64, 2, 0)
+    sh = bytearray(128)
+    struct.pack_into("<I", sh, 64 + 4, 7)
+    struct.pack_into("<QQ", sh, 64 + 24, off if sh_offset is None else sh_offset, len(note) if sh_size is None else sh_size)
+    return bytes(hdr) + note + bytes(sh)
+
+
+@pytest.mark.parametrize("what,blob", [
+    ("a note nested 200,000 arrays deep", _elf_with_note(b"\x91" * 200000 + b"\xc0")),
+    ("a note nested 200,000 maps deep", _elf_with_note(b"\x81\xa1k" * 200000 + b"\xc0")),
+    ("a note section whose offset + size wraps 64 bits", _elf_with_note(b"\x80", sh_offset=2**64 - 8, sh_size=64)),
+    ("a section table whose end wraps 64 bits", _elf_with_note(b"\x80")[:40] + struct.pack("<Q", 2**64 - 64) + _elf_with_note(b"\x80")[48:]),
+])
+def test_crafted_code_objects_are_parse_errors_not_crashes(tmp_path, what, blob):
+    """The code-object reader's bounds: a msgpack note that nests without end is refused at a fixed depth
+    (it must not recurse down the stack), and section ranges that wrap around 2^64 are not ranges."""
+    path = tmp_path / "crafted.hsaco"
+    path.write_bytes(blob)
+    rc = iu8.lib().saber_iu8_manifest_write(str(path).encode(), b"crafted", b"gfx950", b"crafted.hip", b"0" * 64, b"", b"0" * 64,
+                                           str(tmp_path / "crafted.manifest.toml").encode())
+    assert rc == iu8.E_PARSE, (what, rc, iu8.lib().saber_iu8_last_error().decode())
+    assert not (tmp_path / "crafted.manifest.toml").exists()
 
 
 def test_schema_version_and_garbage_are_parse_errors(tmp_path):

@@ -141,6 +141,7 @@ def mutations(raw):
     yield "records out of order", fix(put(raw, REC + 24, "<Q", doff - 4096)), iu8.E_PARSE, "sorted"
     yield "length against shape", fix(put(raw, REC + 32, "<Q", 48 * 128 - 1)), iu8.E_PARSE, "imply"
     yield "past the file", fix(put(raw, REC + 24, "<Q", len(raw))), iu8.E_PARSE, "past"
+    yield "data_off + length wraps 64 bits", fix(put(raw, REC + 24, "<Q", 2**64 - 4096)), iu8.E_PARSE, "past"
     yield "table hash", put(raw, REC + 12, "<I", 18), iu8.E_VALIDATE, "table hash"
     names = raw.find(b"L0.down.wi4s")                                           # rename to its neighbour's name + pad
     dup = bytearray(raw)
@@ -156,7 +157,7 @@ def test_every_open_rule_refuses(tmp_path, case):
             Pack(write(tmp_path, bad, "bad.pack"))
         assert e.value.code == code and word in str(e.value), (name, str(e.value))
         n += 1
-    assert n == 30
+    assert n == 31
 
 
 def test_duplicate_names_and_chunk_entries_refuse(tmp_path, case):
