@@ -383,9 +383,12 @@ int saber_iu8_gemm_acc(saber_iu8_ctx *ctx, int wkind, const void *a, const void 
  * (crates/saber-kernels/hip/moe_route.hip, crates/saber-kernels/src/moe.rs) with the iu8 GEMM at
  * 128 experts, top-8 (the one router symbol this build ships: other widths are refused). */
 
-/* Geometry caps (crates/saber-kernels/src/moe.rs:691-708), no shared expert. */
+/* Geometry caps (crates/saber-kernels/src/moe.rs:691-708); the `_shared` forms add the shared expert's
+ * rows (every token once, padded to 16) and tiles. */
 uint32_t saber_iu8_moe_rows_cap(uint32_t tokens, uint32_t topk, uint32_t experts);
 uint32_t saber_iu8_moe_tiles_cap(uint32_t tokens, uint32_t topk, uint32_t experts, uint32_t tile_blocks);
+uint32_t saber_iu8_moe_rows_cap_shared(uint32_t tokens, uint32_t topk, uint32_t experts);
+uint32_t saber_iu8_moe_tiles_cap_shared(uint32_t tokens, uint32_t topk, uint32_t experts, uint32_t tile_blocks);
 /* tile_blocks the grouped law picks for `tokens`: 1 (16-row tiles, weight-streaming cells) while an
  * expert averages <= 7 routes, 8 (128-row MFMA tiles) below 128 routes an expert, 16 (256-row) from there. */
 uint32_t saber_iu8_moe_tile_blocks(uint32_t tokens, uint32_t topk, uint32_t experts);
@@ -402,12 +405,17 @@ typedef struct {
   int32_t *tile_row0;   /* [tiles_cap] */
   int32_t *tile_rows;   /* [tiles_cap] */
   int32_t *expert_cnt;  /* [experts] */
-  int32_t *meta;        /* [8]: [0] tiles, [1] rows, [3] routes, [4] experts touched */
+  int32_t *meta;        /* [8]: [0] tiles, [1] rows, [2] first shared row or -1, [3] routes, [4] experts touched */
   int32_t *blk_cnt;     /* [ceil(T / 32) * experts]  scratch (the router uses the first ceil(T / 128) * experts) */
   int32_t *rank;        /* [T * topk]                scratch */
   int32_t *arrive;      /* [1]  persistent: zeroed once by the caller, left zero */
   const uint16_t *silu_lut; /* optional (may be NULL): [65536] as saber_iu8_silu_table wrote it; with it
                              * saber_iu8_moe_silu_mul_quant reads the bf16 silu from the table on large row counts */
+  const uint16_t *sgate;    /* optional (may be NULL): bf16 [T], the shared expert's gate logits. Given, the layer has a
+                             * shared expert (crates/saber-kernels/hip/moe_route.hip:244-272, 299-321): the router appends
+                             * every token as a row of expert index `experts` (its weights are entry `experts` of the
+                             * grouped GEMMs' pointer table), sized by the `_shared` caps, and the combine adds
+                             * sigmoid(sgate[t]) * Y[shared row of t] */
 } saber_iu8_moe_tables;
 
 /* Router + expert-major sort + tile table, one launch. logits bf16 [T, experts]. */

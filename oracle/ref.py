@@ -36,6 +36,8 @@ def lib():
         L.w4a8_epilogue.argtypes = [C.c_int32, C.c_float, C.c_float, C.c_int]
         L.w4a8_exp_nonpos.restype = C.c_float
         L.w4a8_exp_nonpos.argtypes = [C.c_float]
+        L.w4a8_sigmoid.restype = C.c_float
+        L.w4a8_sigmoid.argtypes = [C.c_float]
         L.w4a8_silu_bf16.restype = C.c_uint16
         L.w4a8_silu_bf16.argtypes = [C.c_uint16]
         L.w4a8_a_tiled_gfx12.restype = C.c_uint64
@@ -201,6 +203,25 @@ def combine(Y_bits, topk_w, route_pos, H):
     T, topk = w.shape
     out = np.empty((T, H), np.uint16)
     lib().w4a8_combine(_p(Y), _p(w), _p(rp), C.c_int(T), C.c_int(topk), C.c_int(H), _p(out))
+    return out
+
+
+def sigmoid(g):
+    """The shared expert's gate: f32 sigmoid by the router's IEEE-only exp, elementwise."""
+    g = np.ascontiguousarray(g, dtype=np.float32).ravel()
+    L = lib()
+    return np.array([L.w4a8_sigmoid(C.c_float(float(v))) for v in g], dtype=np.float32)
+
+
+def combine_shared(Y_bits, topk_w, route_pos, sgate_bits, sh0, H):
+    """combine() plus sigmoid(sgate[t]) * Y[sh0 + t]: the layer with a shared expert."""
+    Y = _c(Y_bits, np.uint16)
+    w = _c(topk_w, np.float32)
+    rp = _c(route_pos, np.int32)
+    sg = _c(sgate_bits, np.uint16)
+    T, topk = w.shape
+    out = np.empty((T, H), np.uint16)
+    lib().w4a8_combine_shared(_p(Y), _p(w), _p(rp), _p(sg), C.c_int(int(sh0)), C.c_int(T), C.c_int(topk), C.c_int(H), _p(out))
     return out
 
 

@@ -491,6 +491,40 @@ void w4a8_combine(const uint16_t *Y, const float *topk_w, const int32_t *route_p
     }
 }
 
+/* sigmoid(g) of the shared expert's gate (hip/moe_route.hip:59-63): e = exp(-|g|) by the router's
+ * IEEE-only exp, then 1 / (1 + e) for g >= 0 and e / (1 + e) below, IEEE divides. */
+float w4a8_sigmoid(float g) {
+  volatile float e = w4a8_exp_nonpos(-fabsf(g));
+  volatile float d = 1.f + e;
+  volatile float r = g >= 0.f ? 1.f / d : e / d;
+  return r;
+}
+
+/* The combine of a layer with a shared expert (hip/moe_route.hip:299-321): the routes' sum as in
+ * w4a8_combine, then + sigmoid(f32(sgate[t])) * f32(Y[sh0 + t]) (the product rounded before the add),
+ * one bf16 rounding. sh0 < 0 or sgate NULL: the plain combine. */
+void w4a8_combine_shared(const uint16_t *Y, const float *topk_w, const int32_t *route_pos, const uint16_t *sgate, int sh0,
+                         int T, int topk, int H, uint16_t *out) {
+  const int shared = sh0 >= 0 && sgate != NULL;
+  for (int t = 0; t < T; ++t) {
+    const float sg = shared ? w4a8_sigmoid(w4a8_bf16_f32(sgate[t])) : 0.f;
+    for (int h = 0; h < H; ++h) {
+      volatile float acc = 0.f;
+      for (int k = 0; k < topk; ++k) {
+        const int p = route_pos[(size_t)t * topk + k];
+        if (p < 0) continue;
+        volatile float pr = topk_w[(size_t)t * topk + k] * w4a8_bf16_f32(Y[(size_t)p * H + h]);
+        acc = acc + pr;
+      }
+      if (shared) {
+        volatile float pr = sg * w4a8_bf16_f32(Y[(size_t)(sh0 + t) * H + h]);
+        acc = acc + pr;
+      }
+      out[(size_t)t * H + h] = w4a8_bf16_rne(acc);
+    }
+  }
+}
+
 /* ------------------------------------------------------------------ the MoE layer end to end */
 
 /* Flash-Next-style expert layer under the iu8 law, one expert at a time (the grouped

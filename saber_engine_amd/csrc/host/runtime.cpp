@@ -662,6 +662,13 @@ uint32_t saber_iu8_moe_tiles_cap(uint32_t tokens, uint32_t topk, uint32_t expert
   const uint32_t r = tokens * topk;
   return std::min(r, experts) + r / (16u * std::max(tile_blocks, 1u)) + 1u;
 }
+uint32_t saber_iu8_moe_rows_cap_shared(uint32_t tokens, uint32_t topk, uint32_t experts) {
+  return saber_iu8_moe_rows_cap(tokens, topk, experts) + (tokens + 15) / 16 * 16;
+}
+uint32_t saber_iu8_moe_tiles_cap_shared(uint32_t tokens, uint32_t topk, uint32_t experts, uint32_t tile_blocks) {
+  const uint32_t g = std::max(tile_blocks, 1u);
+  return saber_iu8_moe_tiles_cap(tokens, topk, experts, tile_blocks) + ((tokens + 15) / 16 + g - 1) / g;
+}
 // Rows a tile (x16). 16-row tiles on the streaming cell while routes are few (up to 7 routes an
 // expert on average); above, the MFMA cells, whose sparse forms make a thinly filled tile cost about
 // its weight traffic and which stream an expert's weights once instead of once a 16-row tile:
@@ -701,7 +708,7 @@ int saber_iu8_moe_route(saber_iu8_ctx *ctx, const void *logits, uint32_t tokens,
   set_i32(&d, "e_lo", 0);
   set_i32(&d, "e_loc", experts);
   set_i32(&d, "tile_blocks", tile_blocks);
-  set_i32(&d, "with_shared", 0);
+  set_i32(&d, "with_shared", t->sgate ? 1 : 0);
   const saber_iu8_binding b[] = {{"logits", (void *)logits},      {"topk_ids", t->topk_ids},   {"topk_w", t->topk_w},
                                  {"route_pos", t->route_pos},     {"row_tok", t->row_tok},     {"row_route", t->row_route},
                                  {"tile_expert", t->tile_expert}, {"tile_row0", t->tile_row0}, {"tile_rows", t->tile_rows},
@@ -723,7 +730,7 @@ int saber_iu8_moe_route_quant(saber_iu8_ctx *ctx, const void *logits, const void
   set_i32(&d, "e_lo", 0);
   set_i32(&d, "e_loc", experts);
   set_i32(&d, "tile_blocks", tile_blocks);
-  set_i32(&d, "with_shared", 0);
+  set_i32(&d, "with_shared", t->sgate ? 1 : 0);
   set_i32(&d, "k", k);
   const saber_iu8_binding b[] = {{"logits", (void *)logits},      {"topk_ids", t->topk_ids},   {"topk_w", t->topk_w},
                                  {"route_pos", t->route_pos},     {"row_tok", t->row_tok},     {"row_route", t->row_route},
@@ -745,7 +752,8 @@ int saber_iu8_moe_grouped(saber_iu8_ctx *ctx, const void *a, const float *as, co
   const bool dec = tile_blocks == 1;
   // the MFMA cells address A with 32-bit byte offsets: token-major codes (gather 1, 2) or rows_cap rows
   if (!dec) {
-    const uint64_t a_rows = gather ? (uint64_t)(tokens + 15) / 16 * 16 : saber_iu8_moe_rows_cap(tokens, topk, experts);
+    const uint64_t a_rows = gather ? (uint64_t)(tokens + 15) / 16 * 16
+                                   : t->sgate ? saber_iu8_moe_rows_cap_shared(tokens, topk, experts) : saber_iu8_moe_rows_cap(tokens, topk, experts);
     if (a_rows * k > 0xFFFFFFFFull || (uint64_t)n * k / 2 > 0xFFFFFFFFull)
       return fail(SABER_IU8_E_RULE, fmt("moe_grouped: %llu rows of K=%u (or an expert's %u x %u weights) pass 4 GiB, more than the tile GEMM addresses",
                                         (unsigned long long)a_rows, k, n, k));
@@ -766,7 +774,9 @@ int saber_iu8_moe_grouped(saber_iu8_ctx *ctx, const void *a, const float *as, co
   saber_iu8_desc d;
   // the streaming cell: a workgroup a (column block, tile), static worst-case grid; the MFMA cell:
   // persistent, one workgroup a CU over the live work items
-  const uint32_t tiles_cap = saber_iu8_moe_tiles_cap(tokens, topk, experts, tile_blocks), gx = (n + bn - 1) / bn;
+  const uint32_t tiles_cap = t->sgate ? saber_iu8_moe_tiles_cap_shared(tokens, topk, experts, tile_blocks)
+                                      : saber_iu8_moe_tiles_cap(tokens, topk, experts, tile_blocks);
+  const uint32_t gx = (n + bn - 1) / bn;
   const uint64_t items = (uint64_t)gx * tiles_cap;
   if (int rc = dec ? raw_desc(name.c_str(), gx, tiles_cap, block, &d)
                    : raw_desc(name.c_str(), (uint32_t)(items < CU_COUNT ? items : CU_COUNT), 1, block, &d))
@@ -821,9 +831,10 @@ int saber_iu8_moe_combine(saber_iu8_ctx *ctx, const void *y, const saber_iu8_moe
   saber_iu8_desc d;
   if (int rc = raw_desc("moe_iu8_combine_bf16", tokens, 1, 256, &d)) return rc;
   set_i32(&d, "h", h);
-  set_null(&d, "sgate");
-  const saber_iu8_binding b[] = {{"y", (void *)y}, {"topk_w", t->topk_w}, {"route_pos", t->route_pos}, {"meta", t->meta}, {"out", out}};
-  return saber_iu8_launch(ctx, &d, b, 5, stream);
+  if (!t->sgate) set_null(&d, "sgate");  // no shared expert: the kernel tests the pointer
+  const saber_iu8_binding b[] = {{"y", (void *)y},   {"topk_w", t->topk_w}, {"route_pos", t->route_pos},
+                                 {"meta", t->meta}, {"out", out},          {"sgate", (void *)t->sgate}};
+  return saber_iu8_launch(ctx, &d, b, t->sgate ? 6 : 5, stream);
 }
 
 int saber_iu8_silu_table(saber_iu8_ctx *ctx, void *out, void *stream) {

@@ -685,7 +685,17 @@ MOE_GROUPED_PF(moe_iu8_grouped_w4_pf16_g0, moe_grouped_pf_one, 0, 2, 4, 4, 2, 3)
 #undef MOE_GROUPED_PF
 
 // ---------------------------------------------------------------------------- combine
-// One workgroup a token, 8 bf16 a thread-step.
+// sigmoid(g) from the router's IEEE-only exp (crates/saber-kernels/hip/moe_route.hip:59-63): e = exp(-|g|),
+// 1 / (1 + e) for g >= 0, e / (1 + e) below; IEEE divides.
+static __device__ __forceinline__ float moe_sigmoid(float g) {
+#pragma clang fp contract(off)
+  const float e = moe_exp_nonpos(-fabsf(g));
+  const float d = 1.f + e;
+  return g >= 0.f ? __fdiv_rn(1.f, d) : __fdiv_rn(e, d);
+}
+// One workgroup a token, 8 bf16 a thread-step: out[t] = bf16(sum over the token's routes in top-k order of
+// w * Y[route's row], then + sigmoid(sgate[t]) * Y[shared row t] when the layer has a shared expert
+// (meta[2] >= 0 and sgate given), f32, one bf16 rounding (crates/saber-kernels/hip/moe_route.hip:287-329).
 extern "C" __global__ __launch_bounds__(256) void moe_iu8_combine_bf16(
     const unsigned short *__restrict__ y, const float *__restrict__ topk_w, const int *__restrict__ route_pos,
     const unsigned short *__restrict__ sgate, const int *__restrict__ meta, unsigned short *__restrict__ out, int h) {
@@ -698,8 +708,9 @@ extern "C" __global__ __launch_bounds__(256) void moe_iu8_combine_bf16(
     s_w[threadIdx.x] = topk_w[(size_t)t * MOE_TOPK + threadIdx.x];
   }
   __syncthreads();
-  (void)sgate;  // the shared-expert gate term is not part of this object's layer
-  (void)meta;
+  const int sh0 = meta[2];
+  const bool shared = sh0 >= 0 && sgate != nullptr;
+  const float sg = shared ? moe_sigmoid(iu8_bf16_f32(sgate[t])) : 0.f;
   for (int g = threadIdx.x; g < h / 8; g += 256) {
     float acc[8];
 #pragma unroll
@@ -713,6 +724,14 @@ extern "C" __global__ __launch_bounds__(256) void moe_iu8_combine_bf16(
       for (int q = 0; q < 4; ++q) {
         acc[2 * q] = acc[2 * q] + w * __uint_as_float(v[q] << 16);
         acc[2 * q + 1] = acc[2 * q + 1] + w * __uint_as_float(v[q] & 0xFFFF0000u);
+      }
+    }
+    if (shared) {
+      const iu8_v4u v = ((const iu8_v4u *)(y + (size_t)(sh0 + t) * h))[g];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        acc[2 * q] = acc[2 * q] + sg * __uint_as_float(v[q] << 16);
+        acc[2 * q + 1] = acc[2 * q + 1] + sg * __uint_as_float(v[q] & 0xFFFF0000u);
       }
     }
     iu8_v4u o;

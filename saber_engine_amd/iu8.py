@@ -71,7 +71,7 @@ class Counters(C.Structure):
 
 
 MOE_TABLE_FIELDS = ("topk_ids", "topk_w", "route_pos", "row_tok", "row_route", "tile_expert", "tile_row0", "tile_rows",
-                    "expert_cnt", "meta", "blk_cnt", "rank", "arrive", "silu_lut")
+                    "expert_cnt", "meta", "blk_cnt", "rank", "arrive", "silu_lut", "sgate")
 
 
 class MoeTables(C.Structure):
@@ -135,11 +135,12 @@ def lib():
         L.saber_iu8_attn_gate_quant_had.argtypes = [C.c_void_p] * 5 + [C.c_uint32] * 4 + [C.c_void_p, C.c_void_p]
         L.saber_iu8_get_counters.argtypes = [C.c_void_p, C.POINTER(Counters)]
         L.saber_iu8_has_kernel.argtypes = [C.c_void_p, C.c_char_p]
-        for fn in ("saber_iu8_moe_rows_cap", "saber_iu8_moe_tile_blocks"):
+        for fn in ("saber_iu8_moe_rows_cap", "saber_iu8_moe_rows_cap_shared", "saber_iu8_moe_tile_blocks"):
             getattr(L, fn).restype = C.c_uint32
             getattr(L, fn).argtypes = [C.c_uint32] * 3
-        L.saber_iu8_moe_tiles_cap.restype = C.c_uint32
-        L.saber_iu8_moe_tiles_cap.argtypes = [C.c_uint32] * 4
+        for fn in ("saber_iu8_moe_tiles_cap", "saber_iu8_moe_tiles_cap_shared"):
+            getattr(L, fn).restype = C.c_uint32
+            getattr(L, fn).argtypes = [C.c_uint32] * 4
         L.saber_iu8_moe_route.argtypes = [C.c_void_p, C.c_void_p] + [C.c_uint32] * 4 + [C.POINTER(MoeTables), C.c_void_p]
         L.saber_iu8_moe_route_quant.argtypes = [C.c_void_p] * 5 + [C.c_uint32] * 5 + [C.POINTER(MoeTables), C.c_void_p]
         L.saber_iu8_moe_grouped.argtypes = ([C.c_void_p] * 5 + [C.c_uint32, C.c_uint32, C.c_int] + [C.c_uint32] * 4 +
@@ -449,12 +450,12 @@ class Context:
         _check(lib().saber_iu8_silu_table(self._h, out, stream))
 
 
-def moe_rows_cap(tokens, topk, experts):
-    return lib().saber_iu8_moe_rows_cap(tokens, topk, experts)
+def moe_rows_cap(tokens, topk, experts, shared=False):
+    return (lib().saber_iu8_moe_rows_cap_shared if shared else lib().saber_iu8_moe_rows_cap)(tokens, topk, experts)
 
 
-def moe_tiles_cap(tokens, topk, experts, tile_blocks):
-    return lib().saber_iu8_moe_tiles_cap(tokens, topk, experts, tile_blocks)
+def moe_tiles_cap(tokens, topk, experts, tile_blocks, shared=False):
+    return (lib().saber_iu8_moe_tiles_cap_shared if shared else lib().saber_iu8_moe_tiles_cap)(tokens, topk, experts, tile_blocks)
 
 
 def moe_tile_blocks(tokens, topk, experts):

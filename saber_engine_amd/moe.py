@@ -10,11 +10,15 @@ from . import iu8
 
 
 class MoeLayerIU8:
-    def __init__(self, ctx, tokens, experts=128, topk=8, hidden=4096, inter=1536, tile_blocks=None, device="cuda"):
+    def __init__(self, ctx, tokens, experts=128, topk=8, hidden=4096, inter=1536, tile_blocks=None, device="cuda", shared=False):
+        """shared: the layer has a shared expert (crates/saber-kernels/src/moe.rs:688-711): every token also
+        runs through expert index `experts`, whose weights are the last entry given to set_weights, and
+        the combine adds sigmoid(sgate[t]) times that row."""
         self.ctx, self.T, self.E, self.topk, self.H, self.I = ctx, tokens, experts, topk, hidden, inter
+        self.shared = bool(shared)
         self.tb = tile_blocks or iu8.moe_tile_blocks(tokens, topk, experts)
-        self.rows_cap = iu8.moe_rows_cap(tokens, topk, experts)
-        self.tiles_cap = iu8.moe_tiles_cap(tokens, topk, experts, self.tb)
+        self.rows_cap = iu8.moe_rows_cap(tokens, topk, experts, self.shared)
+        self.tiles_cap = iu8.moe_tiles_cap(tokens, topk, experts, self.tb, self.shared)
         i32 = dict(dtype=torch.int32, device=device)
         R = tokens * topk
         self.buf = dict(
@@ -29,7 +33,11 @@ class MoeLayerIU8:
         self.buf["silu_lut"] = torch.zeros(65536, dtype=torch.int16, device=device)
         ctx.silu_table(self.buf["silu_lut"].data_ptr())
         torch.cuda.synchronize()
-        self.tables = iu8.MoeTables(*[self.buf[n].data_ptr() for n in iu8.MOE_TABLE_FIELDS])
+        # the shared expert's gate logits, bf16 [T]: bound into the tables only when the layer has one
+        self.sgate = torch.zeros(tokens, dtype=torch.int16, device=device) if self.shared else None
+        ptr = {n: self.buf[n].data_ptr() for n in self.buf}
+        ptr["sgate"] = self.sgate.data_ptr() if self.shared else None
+        self.tables = iu8.MoeTables(*[ptr[n] for n in iu8.MOE_TABLE_FIELDS])
         u8 = dict(dtype=torch.uint8, device=device)
         # tokens are quantised once and the grouped gate+up GEMM gathers their rows: the streaming cell
         # (16-row tiles) from the A edge, the MFMA cells from row-major codes (whole 64-byte runs a row)
@@ -44,16 +52,19 @@ class MoeLayerIU8:
         self.xptr_gu = self.xptr_dn = None
 
     def set_weights(self, wgu_frag, wsgu, wdn_frag, wsdn):
-        """Per-expert gfx950 W4 fragments [E, 2I*H/2] / [E, H*I/2] (uint8) and scales [E,2I] / [E,H] (f32) on device."""
+        """Per-expert gfx950 W4 fragments [E, 2I*H/2] / [E, H*I/2] (uint8) and scales [E,2I] / [E,H] (f32) on device;
+        E + 1 of each with a shared expert (the shared expert's last)."""
         self._w = (wgu_frag, wsgu, wdn_frag, wsdn)
-        E = self.E
+        E = self.E + (1 if self.shared else 0)
+        assert wgu_frag.shape[0] >= E and wdn_frag.shape[0] >= E
         gu = [[wgu_frag[e].data_ptr(), wsgu[e].data_ptr()] for e in range(E)]
         dn = [[wdn_frag[e].data_ptr(), wsdn[e].data_ptr()] for e in range(E)]
         self.xptr_gu = torch.tensor(np.array(gu, np.int64).ravel(), device=wgu_frag.device)
         self.xptr_dn = torch.tensor(np.array(dn, np.int64).ravel(), device=wgu_frag.device)
 
     def forward(self, x, logits, stream=0):
-        """x bf16 bits [T,H] (int16 tensor), logits bf16 bits [T,E]; every launch on `stream`."""
+        """x bf16 bits [T,H] (int16 tensor), logits bf16 bits [T,E]; with a shared expert its gate logits
+        (bf16 bits [T]) are read from self.sgate, which the caller fills; every launch on `stream`."""
         c, T, E, k, H, I = self.ctx, self.T, self.E, self.topk, self.H, self.I
         if self.gather == 1 and H <= 16384:   # few tokens: the router and the quantisation in one launch
             c.moe_route_quant(logits.data_ptr(), x.data_ptr(), self.q1.data_ptr(), self.s1.data_ptr(), T, E, k, H, self.tb,

@@ -77,6 +77,63 @@ def test_moe_layer_small_experts(ctx, T, tb):
     check_layer(layer, case)
 
 
+@pytest.mark.parametrize("T,tb", [(1, None), (16, None), (37, None), (100, 8), (300, None), (300, 1), (520, 16)])
+def test_moe_layer_with_a_shared_expert(ctx, T, tb):
+    """The layer with a shared expert (crates/saber-kernels/hip/moe_route.hip:244-272, 299-321): the router
+    appends every token as a row of expert index 128 behind the routed rows (meta[2] = its first row, tiles
+    of `tile_blocks` blocks, pad rows marked), both grouped GEMMs and the SiLU*up requant run those rows
+    on the shared expert's weights, and the combine adds sigmoid(sgate[t]) times the token's shared row.
+    Expected: the oracle's routed layer, the shared expert as a dense MLP of the oracle's linears over all
+    tokens, and the oracle's combine with the gate term."""
+    E, k, H, I = 128, 8, 512, 256
+    say(f"moe layer with a shared expert T={T} tile_blocks={tb}")
+    case = synth.moe_case(T=T, E=E, topk=k, H=H, I=I, seed=100 + T, experts=6)
+    rng = np.random.default_rng(T)
+    Wgu_s, wsgu_s = synth.weights(rng, 2 * I, H, False)
+    Wdn_s, wsdn_s = synth.weights(rng, H, I, False)
+    sgate = synth.f32_to_bf16_bits((2.5 * rng.standard_normal(T)).astype(np.float32))
+    layer = MoeLayerIU8(ctx, T, E, k, H, I, tile_blocks=tb, shared=True)
+    wgu = torch.from_numpy(np.stack([iu8.repack_w4(case["Wgu"][e]) for e in range(E)] + [iu8.repack_w4(Wgu_s)])).cuda()
+    wdn = torch.from_numpy(np.stack([iu8.repack_w4(case["Wdn"][e]) for e in range(E)] + [iu8.repack_w4(Wdn_s)])).cuda()
+    layer.set_weights(wgu, torch.from_numpy(np.concatenate([case["wsgu"], wsgu_s[None]])).cuda(), wdn,
+                      torch.from_numpy(np.concatenate([case["wsdn"], wsdn_s[None]])).cuda())
+    layer.sgate.copy_(dev_bf16_bits(sgate))
+    for t in (layer.gu, layer.y, layer.out):
+        t.fill_(0x7FC0)
+    x, lg = dev_bf16_bits(case["X"]), dev_bf16_bits(case["logits"])
+    layer.forward(x, lg)
+    layer.forward(x, lg)
+    torch.cuda.synchronize()
+    # ---- the tables: the routed part as without a shared expert, then the shared rows and tiles
+    ids, w = ref.route(case["logits"], k)
+    lay = ref.sort_layout(ids, E, layer.tb)
+    b = {n: t.cpu().numpy() for n, t in layer.buf.items()}
+    rows, nt, G = lay["rows"], lay["tiles"], layer.tb
+    sh_blocks = (T + 15) // 16
+    sh_tiles = -(-sh_blocks // G)
+    assert b["meta"][:6].tolist() == [nt + sh_tiles, rows + sh_blocks * 16, rows, T * k, int((lay["expert_cnt"] > 0).sum()), rows]
+    assert layer.rows_cap >= rows + sh_blocks * 16 and layer.tiles_cap >= nt + sh_tiles and int(b["arrive"][0]) == 0
+    np.testing.assert_array_equal(b["row_tok"][:rows], lay["row_tok"])
+    np.testing.assert_array_equal(b["row_tok"][rows:rows + sh_blocks * 16], np.where(np.arange(sh_blocks * 16) < T, np.arange(sh_blocks * 16), -1))
+    np.testing.assert_array_equal(b["tile_expert"][:nt + sh_tiles], np.concatenate([lay["tile_expert"], np.full(sh_tiles, E)]))
+    np.testing.assert_array_equal(b["tile_row0"][nt:nt + sh_tiles], rows + 16 * G * np.arange(sh_tiles))
+    np.testing.assert_array_equal(b["tile_rows"][nt:nt + sh_tiles], np.minimum(16 * G, T - 16 * G * np.arange(sh_tiles)))
+    np.testing.assert_array_equal(b["route_pos"].reshape(T, k), lay["route_pos"])
+    # ---- the arithmetic
+    r = ref.moe_layer(case["X"], w, lay, case["Wgu"], case["wsgu"], case["Wdn"], case["wsdn"], I, threads=8)
+    live = lay["row_tok"] >= 0
+    np.testing.assert_array_equal(host_u16(layer.y)[:rows][live], r["Y"][live])
+    gu_s = ref.linear(case["X"], Wgu_s, wsgu_s, False, threads=8)["C"]
+    _, _, p_s = ref.silu_mul_quant(gu_s)
+    y_s = ref.linear(p_s, Wdn_s, wsdn_s, False, threads=8)["C"]
+    np.testing.assert_array_equal(host_u16(layer.gu)[rows:rows + T], gu_s)
+    np.testing.assert_array_equal(host_u16(layer.y)[rows:rows + T], y_s)
+    Y = np.concatenate([r["Y"], y_s])
+    want = ref.combine_shared(Y, w, lay["route_pos"], sgate, rows, H)
+    np.testing.assert_array_equal(host_u16(layer.out), want)
+    assert (want != r["out"]).any()                      # the gate term is in the output
+
+
 def test_moe_layer_streamed_rows_cell(ctx):
     """K past the short-K form and more routes than the LDS staging is sized for: the streaming cell
     that reads the rows beside the weights (gate+up), the short-K cell (down)."""

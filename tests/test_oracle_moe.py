@@ -194,6 +194,50 @@ def test_combine_is_an_ordered_f32_sum_with_one_rounding():
     assert (acc_r != acc).any()
 
 
+def test_sigmoid_is_the_logistic_within_rounding_and_matches_the_f32_restatement():
+    """The shared expert's gate (hip/moe_route.hip:59-63). Pinned by a numpy-f32 restatement built on the
+    pinned exp (bit-equal), by float64 (a few ulp), and by what the function must satisfy whatever the
+    exp's last bit: s(0) = 1/2, s(g) + s(-g) = 1 within an ulp, monotone, saturating ends."""
+    gs = np.concatenate([np.linspace(-30, 30, 2401), [0.0, -0.0, 1e-8, -1e-8, 90.0, -90.0, 1e30, -1e30]]).astype(np.float32)
+    got = ref.sigmoid(gs)
+    e = exp_nonpos_np(-np.abs(gs))
+    d = (np.float32(1) + e).astype(np.float32)
+    want = np.where(gs >= 0, (np.float32(1) / d).astype(np.float32), (e / d).astype(np.float32)).astype(np.float32)
+    np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32))
+    true = 1.0 / (1.0 + np.exp(-gs.astype(np.float64)))
+    live = np.abs(gs) < 60
+    assert np.max(np.abs(got[live] - true[live]) / true[live]) < 4e-7
+    assert got[gs == 0][0] == 0.5 and got[-2] == 1.0 and got[-1] == 0.0
+    half = np.linspace(0, 30, 1201).astype(np.float32)
+    assert np.max(np.abs(ref.sigmoid(half) + ref.sigmoid(-half) - 1.0)) <= 1.2e-7
+    line = ref.sigmoid(np.linspace(-30, 30, 2401).astype(np.float32))
+    assert (np.diff(line) >= 0).all()
+
+
+def test_combine_shared_adds_the_gated_shared_row_last():
+    rng = np.random.default_rng(16)
+    T, topk, H, rows = 7, 8, 64, 150
+    sh0 = 128
+    Y = synth.f32_to_bf16_bits(rng.standard_normal((rows, H)).astype(np.float32))
+    w = rng.random((T, topk)).astype(np.float32)
+    pos = rng.integers(0, sh0, (T, topk)).astype(np.int32)
+    pos[4, 0] = -1
+    sgate = synth.f32_to_bf16_bits((3 * rng.standard_normal(T)).astype(np.float32))
+    out = ref.combine_shared(Y, w, pos, sgate, sh0, H)
+    yf = synth.bf16_bits_to_f32(Y)
+    acc = np.zeros((T, H), np.float32)
+    for k in range(topk):
+        live = pos[:, k] >= 0
+        pr = (w[:, k, None].astype(np.float64) * yf[np.maximum(pos[:, k], 0)].astype(np.float64)).astype(np.float32)
+        acc = np.where(live[:, None], (acc + pr).astype(np.float32), acc)
+    sg = ref.sigmoid(synth.bf16_bits_to_f32(sgate))
+    pr = (sg[:, None].astype(np.float64) * yf[sh0:sh0 + T].astype(np.float64)).astype(np.float32)
+    np.testing.assert_array_equal(out, synth.f32_to_bf16_bits((acc + pr).astype(np.float32)))
+    # without shared rows it is the plain combine; and the shared term is really there
+    np.testing.assert_array_equal(ref.combine_shared(Y, w, pos, sgate, -1, H), ref.combine(Y, w, pos, H))
+    assert (out != ref.combine(Y, w, pos, H)).any()
+
+
 def test_moe_layer_equals_per_route_composition():
     c = synth.moe_case(T=6, E=16, topk=2, H=256, I=128, seed=3)
     ids, w = ref.route(c["logits"], 2)
