@@ -27,6 +27,7 @@
 typedef int iu8_v4i __attribute__((ext_vector_type(4)));
 typedef unsigned iu8_v4u __attribute__((ext_vector_type(4)));
 typedef unsigned iu8_v2u __attribute__((ext_vector_type(2)));
+typedef float iu8_v4f __attribute__((ext_vector_type(4)));
 typedef unsigned char iu8_u8;
 
 // D[n][m] += sum_k W[n][k] * A[m][k] over 64 k: src0 = weight operand (lane: row n = l%16),

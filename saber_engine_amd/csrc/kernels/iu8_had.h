@@ -11,42 +11,45 @@
 
 #define HAD_MAXG 5  // 8-element groups a thread: K <= 40 * T
 
-static __device__ __forceinline__ float had_dpp_xor1(float v) {
-  return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, false));
-}
-static __device__ __forceinline__ float had_dpp_xor2(float v) {
-  return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, false));
+// One butterfly stage across lanes: the pair is (this lane, the lane CTRL's quad permute brings in);
+// the lane whose bit is clear holds the pair's low element and keeps the sum, the other the difference
+// low - high. A DPP move copies registers exactly, in a 64-wide wave as in a 32-wide one.
+template <int CTRL>
+static __device__ __forceinline__ void had_lane_stage(float (&v)[8], bool holds_high) {
+#pragma clang fp contract(off)
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const float other = __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v[j]), CTRL, 0xF, 0xF, false));
+    v[j] = holds_high ? other - v[j] : v[j] + other;
+  }
 }
 
-// v[8]: this lane's 8 values of its group; t8: the group's 8 entries of t. In place.
+// The 32-point transform (crates/saber-kernels/hip/macaq_had.h:47-83) of the block whose elements
+// 8*(lane & 3) .. + 7 this lane holds in v: multiply by the block's t, the unnormalised Sylvester
+// butterfly over element bits 0..4 in that order -- bits 0..2 pair registers, bits 3 and 4 pair lanes
+// (xor 1, xor 2) -- each stage (low, high) -> (low + high, low - high), then one multiply by
+// (float)(1 / sqrt(32)). t8: the 8 entries of t for this lane's elements. In place.
 static __device__ __forceinline__ void had32(float (&v)[8], const float *__restrict__ t8, int lane) {
 #pragma clang fp contract(off)
-  const float4 ta = ((const float4 *)t8)[0], tb = ((const float4 *)t8)[1];
-  v[0] = v[0] * ta.x, v[1] = v[1] * ta.y, v[2] = v[2] * ta.z, v[3] = v[3] * ta.w;
-  v[4] = v[4] * tb.x, v[5] = v[5] * tb.y, v[6] = v[6] * tb.z, v[7] = v[7] * tb.w;
+  const iu8_v4f t_lo = *(const iu8_v4f *)t8, t_hi = *(const iu8_v4f *)(t8 + 4);
 #pragma unroll
-  for (int s = 1; s < 8; s <<= 1) {
+  for (int j = 0; j < 4; ++j) v[j] = v[j] * t_lo[j], v[j + 4] = v[j + 4] * t_hi[j];
+#pragma unroll
+  for (int bit = 0; bit < 3; ++bit) {
+    const int span = 1 << bit;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      if (j & s) continue;
-      const float lo = v[j], hi = v[j | s];
-      v[j] = lo + hi;
-      v[j | s] = lo - hi;
+      if (j & span) continue;  // j is the pair's low element
+      const float low = v[j], high = v[j + span];
+      v[j] = low + high;
+      v[j + span] = low - high;
     }
   }
-  const bool b0 = (lane & 1) != 0, b1 = (lane & 2) != 0;
+  had_lane_stage<0xB1>(v, (lane & 1) != 0);  // quad_perm [1,0,3,2]: element bit 3
+  had_lane_stage<0x4E>(v, (lane & 2) != 0);  // quad_perm [2,3,0,1]: element bit 4
+  const float inv_sqrt32 = __uint_as_float(0x3E3504F3u);
 #pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    const float p = had_dpp_xor1(v[j]);
-    v[j] = b0 ? (p - v[j]) : (v[j] + p);
-  }
-#pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    const float p = had_dpp_xor2(v[j]);
-    v[j] = b1 ? (p - v[j]) : (v[j] + p);
-  }
-#pragma unroll
-  for (int j = 0; j < 8; ++j) v[j] = v[j] * __uint_as_float(0x3E3504F3u);
+  for (int j = 0; j < 8; ++j) v[j] = v[j] * inv_sqrt32;
 }
 
 // The row of workgroup b: the 8 A tiles of a full group of 128 rows go one to an XCD (consecutive

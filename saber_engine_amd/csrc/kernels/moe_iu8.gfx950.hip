@@ -30,24 +30,23 @@
 #define MOE_THREADS 1024
 #define MOE_CHUNK 36864  // rows of the placement tables held in LDS at a time (144 KiB)
 
-// e^x for x <= 0 from IEEE-rounded mul/add/rint/ldexp only (the law of
-// crates/saber-kernels/hip/moe_route.hip:43-57: n = rint(x*log2e), two-step Cody-Waite reduction,
-// degree-7 Taylor by Horner, ldexp; x <= -80 or NaN -> 0).
+// e^x for x <= 0 from IEEE-rounded multiply / add / rint / ldexp only, so that every implementation of
+// the router gives the same bits (the law of crates/saber-kernels/hip/moe_route.hip:43-57):
+// n = rint(x * log2(e)); r = x - n * ln2 in two Cody-Waite pieces; e^r by the degree-7 Taylor
+// polynomial in Horner form (coefficients 1/7! ... 1/2!, 1, 1 as f32 bit patterns); result * 2^n.
+// x <= -80 or NaN gives 0.
 static __device__ __forceinline__ float moe_exp_nonpos(float x) {
 #pragma clang fp contract(off)
+  constexpr unsigned LOG2E = 0x3FB8AA3Bu, LN2_HEAD = 0x3F317200u, LN2_TAIL = 0x35BFBE8Eu;
+  constexpr unsigned TAYLOR[8] = {0x39500D01u, 0x3AB60B61u, 0x3C088889u, 0x3D2AAAABu, 0x3E2AAAABu, 0x3F000000u, 0x3F800000u, 0x3F800000u};
   if (!(x > -80.f)) return 0.f;
-  const float n = __builtin_rintf(x * __uint_as_float(0x3FB8AA3Bu));
-  float r = x - n * __uint_as_float(0x3F317200u);
-  r = r - n * __uint_as_float(0x35BFBE8Eu);
-  float p = __uint_as_float(0x39500D01u);
-  p = p * r + __uint_as_float(0x3AB60B61u);
-  p = p * r + __uint_as_float(0x3C088889u);
-  p = p * r + __uint_as_float(0x3D2AAAABu);
-  p = p * r + __uint_as_float(0x3E2AAAABu);
-  p = p * r + 0.5f;
-  p = p * r + 1.f;
-  p = p * r + 1.f;
-  return __builtin_ldexpf(p, (int)n);
+  const float n = __builtin_rintf(x * __uint_as_float(LOG2E));
+  float r = x - n * __uint_as_float(LN2_HEAD);
+  r = r - n * __uint_as_float(LN2_TAIL);
+  float poly = __uint_as_float(TAYLOR[0]);
+#pragma unroll
+  for (int i = 1; i < 8; ++i) poly = poly * r + __uint_as_float(TAYLOR[i]);
+  return __builtin_ldexpf(poly, (int)n);
 }
 
 // Lane exchanges inside a token's 8 lanes without the LDS crossbar's latency: DPP quad permutes for
