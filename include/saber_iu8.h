@@ -293,8 +293,8 @@ int saber_iu8_gemm_pair(saber_iu8_ctx *ctx, const void *a, const float *a_scale,
                         void *stream);
 
 /* The whole decode linear in one launch where that is the faster form (saber_iu8_fused_holds: up to
- * 4 rows whose codes, rows rounded up to a power of two, fit 20 KiB of LDS -- kernel `_tm1` -- or up
- * to 3 rows in 80 KiB -- kernel `_tm1_a80`, which itself holds up to 16 rows and is reachable by name
+ * 4 rows whose codes, rows rounded up to a power of two, fit 20 KiB of LDS -- kernel `_tm1` -- or
+ * 80 KiB -- kernel `_tm1_a80`, which itself holds up to 16 rows and is reachable by name
  * through saber_iu8_describe_raw): per-token quantisation fused into the
  * GEMV's activation staging. x bf16 [m,k]; q (A edge) and scale f32 [m] are optional outputs (NULL:
  * not stored) with the bytes saber_iu8_quant would write. Other shapes are refused

@@ -391,10 +391,10 @@ static int describe_rows(const char *op, const char *kernel, uint32_t rows, uint
 
 // The fused forms quantise rows whose int8 codes (rows rounded up to a power of two) fit the kernel's
 // staging area: up to 4 rows in 20 KiB (`_tm1`), up to 16 rows in 80 KiB (`_tm1_a80`). Every workgroup
-// repeats the rows' quantisation (about 0.7 us a row of 5,120 on this card), a producer launch costs
-// about 3 us once: the law takes the 80 KiB form for up to 3 rows (down at 2 rows: 14.5 against 17.4 us
-// as producer + GEMV; at 4 rows 17.8 against 17.6; QKV at 5 / 8 / 16 rows 9.3 / 10.7 / 15.8 against
-// 8.8 / 8.9 / 9.4). The kernel itself holds what `fused_form_holds` says, by name.
+// repeats the rows' quantisation (about 0.5 us a row of 5,120 on this card), a producer launch costs
+// about 3 us once: the law takes the 80 KiB form for up to 4 rows (down at 2 rows: 14.4 against 17.3 us
+// as producer + GEMV; at 4 rows 16.0 against 17.4; QKV at 5 / 6 / 8 rows 9.0 / 9.2 / 9.9 against 8.8). The
+// kernel itself holds what `fused_form_holds` says, by name.
 static uint64_t staged_bytes(uint32_t m, uint32_t k) {
   uint32_t mr = 1;
   while (mr < m) mr *= 2;
@@ -404,7 +404,7 @@ bool fused_small_holds(uint32_t m, uint32_t k) { return m >= 1 && m <= 4 && stag
 bool fused_form_holds(bool a80, uint32_t m, uint32_t k) {
   return a80 ? m >= 1 && m <= 16 && staged_bytes(m, k) <= 80 * 1024 : fused_small_holds(m, k);
 }
-bool fused_holds(uint32_t m, uint32_t k) { return fused_small_holds(m, k) || (m <= 3 && fused_form_holds(true, m, k)); }
+bool fused_holds(uint32_t m, uint32_t k) { return fused_small_holds(m, k) || (m <= 4 && fused_form_holds(true, m, k)); }
 
 uint32_t fused_grid(uint32_t nblk) {
   if (nblk <= CU_COUNT) return nblk;
@@ -417,7 +417,7 @@ int resolve_fused(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc 
   const char *op = wkind == SABER_IU8_W8 ? "linear_i8a8_fused" : "linear_i4a8_fused";
   if (int rc = check_shape(op, m, n, k)) return rc;
   if (!fused_holds(m, k))
-    return fail(SABER_IU8_E_RULE, fmt("%s: %u rows of %u are not a fused launch (up to 4 rows in 20 KiB of codes, up to 3 rows in 80 KiB)", op, m, k));
+    return fail(SABER_IU8_E_RULE, fmt("%s: %u rows of %u are not a fused launch (up to 4 rows, 20 KiB of codes or 80 KiB)", op, m, k));
   const std::string name = fmt("macaq_iu8_decq_%s_tm1%s", wkind == SABER_IU8_W8 ? "w8" : "w4", fused_small_holds(m, k) ? "" : "_a80");
   memset(d, 0, sizeof *d);
   copy_name(d->op, sizeof d->op, op);

@@ -44,7 +44,7 @@ int pair(const saber_iu8_desc &first, const saber_iu8_desc &second, saber_iu8_de
 const DecVariant *pair_variant(const std::string &name);
 int resolve_quant(uint32_t m, uint32_t k, saber_iu8_desc *out);
 // The fused quant + GEMV of a decode linear; refuses (by name) shapes it does not hold.
-bool fused_holds(uint32_t m, uint32_t k);        // the law: a fused launch is what runs (20 KiB form, or the 80 KiB form up to 3 rows)
+bool fused_holds(uint32_t m, uint32_t k);        // the law: a fused launch is what runs (up to 4 rows: the 20 KiB form, else the 80 KiB form)
 bool fused_form_holds(bool a80, uint32_t m, uint32_t k);  // what the kernel itself holds: `_tm1` 4 rows / 20 KiB, `_tm1_a80` 16 rows / 80 KiB
 bool fused_small_holds(uint32_t m, uint32_t k);  // the 20 KiB form: up to 4 rows (`_tm1`, and both linears of the MLP chain)
 uint32_t fused_grid(uint32_t nblk);  // workgroups for nblk column blocks: one a CU, then equal shares of at most 8

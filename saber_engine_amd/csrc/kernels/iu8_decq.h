@@ -153,11 +153,17 @@ __device__ __forceinline__ void iu8_decq_body(const unsigned short *__restrict__
     if (tid < 16) s_rowmax[tid] = 0u;
     __syncthreads();
     const bool wave_rows = (k8 & 63) == 0;  // a wave's 64 pieces of one load lie in one row
+    // piece p * NTHR + tid = (row, col) in pieces of 8: two divides here, then steps of NTHR pieces
+    const int row_step = NTHR / k8, col_step = NTHR - row_step * k8;
+    int row = tid / k8, col = tid - row * k8;
+    auto next_piece = [&]() {
+      row += row_step, col += col_step;
+      if (col >= k8) col -= k8, ++row;
+    };
 #pragma unroll
-    for (int p = 0; p < X_PER; ++p) {
+    for (int p = 0; p < X_PER; ++p, next_piece()) {
       const int piece = p * NTHR + tid;
       const bool live = piece < x_pieces;
-      const int row = live ? piece / k8 : 0;
       float m8 = 0.f;
       if (live) {
 #pragma unroll
@@ -168,11 +174,13 @@ __device__ __forceinline__ void iu8_decq_body(const unsigned short *__restrict__
       }
       if (wave_rows) {  // x_pieces is then a multiple of 64: a wave is live or not as a whole
         m8 = iu8_wave_max_nonneg(m8);
-        if (lane == 0 && live) __hip_atomic_fetch_max(&s_rowmax[row], __float_as_uint(m8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        if (lane == 0 && live) __hip_atomic_fetch_max(&s_rowmax[row & 15], __float_as_uint(m8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
       } else if (live) {
-        __hip_atomic_fetch_max(&s_rowmax[row], __float_as_uint(m8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        __hip_atomic_fetch_max(&s_rowmax[row & 15], __float_as_uint(m8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
       }
     }
+    row = tid / k8, col = tid - row * k8;
+    asm volatile("" : "+v"(row), "+v"(col));  // walked again from here: not ten (row, col) pairs kept in registers
 #pragma unroll
     for (int i = 0; i < D; ++i)
       if (i < TT) issue(i);
@@ -190,10 +198,10 @@ __device__ __forceinline__ void iu8_decq_body(const unsigned short *__restrict__
     if (blockIdx.x == 0 && sout != nullptr && tid < M) sout[tid] = s_rsc[tid];
     my_sc = s_rsc[ml];
 #pragma unroll
-    for (int p = 0; p < X_PER; ++p) {
+    for (int p = 0; p < X_PER; ++p, next_piece()) {
       const int piece = p * NTHR + tid;
       if (piece >= x_pieces) continue;
-      const int row = piece / k8, k = (piece - row * k8) << 3;
+      const int k = col << 3;
       const float sc = s_rsc[row], rcp = s_rrcp[row];
       float f[8];
 #pragma unroll
