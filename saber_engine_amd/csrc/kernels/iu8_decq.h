@@ -71,7 +71,7 @@ __device__ __forceinline__ void iu8_decq_body(const unsigned short *__restrict__
   __shared__ __attribute__((aligned(16))) iu8_u8 s_a[ABYTES];
   __shared__ __attribute__((aligned(16))) int s_red[2][RED];
   __shared__ float s_amax[WPB][4];
-  __shared__ float s_sq[2][4];  // scale and reciprocal a row, made once a workgroup when there are several rows
+  __shared__ float s_sq[2][4];  // scale and reciprocal a row, made once a workgroup
   __shared__ unsigned s_rowmax[BIG ? 16 : 1];
   __shared__ float s_rsc[BIG ? 16 : 1], s_rrcp[BIG ? 16 : 1];
   __shared__ float s_ws[IU8_DECQ_MAXB][WN * NT * 16];  // the epilogue's weight scales (W4: already / 16)
@@ -277,29 +277,22 @@ __device__ __forceinline__ void iu8_decq_body(const unsigned short *__restrict__
     }
     __syncthreads();
     float qrcp[4] = {1.f, 1.f, 1.f, 1.f};
-    if (M == 1) {  // one row: every lane makes the scale itself (two divides cost less than a meeting)
-      float a = s_amax[0][0];
+    // lane r makes row r's scale and reciprocal (two IEEE divides) once a workgroup; every lane making them
+    // for itself cost more than this hand-over: 16 partial maxima to read and 20 instructions a row and lane
+    // (one row: QKV 5.75 -> 5.56 us, O 5.53 -> 5.34, gate+up 16.9 -> 16.5; four rows: QKV 7.8 -> 6.9)
+    if (tid < 4) {
+      float a = s_amax[0][tid];
       if constexpr (CH != 2) {
 #pragma unroll
-        for (int w = 1; w < WPB; ++w) a = fmaxf(a, s_amax[w][0]);
+        for (int w = 1; w < WPB; ++w) a = fmaxf(a, s_amax[w][tid]);
       }
-      qsc[0] = fmaxf(__fdiv_rn(a, 127.f), 1e-30f);
-      qrcp[0] = __fdiv_rn(1.f, qsc[0]);
-    } else {  // several rows: lane r makes row r's scale and reciprocal, once a workgroup
-      if (tid < 4) {
-        float a = s_amax[0][tid];
-        if constexpr (CH != 2) {
-#pragma unroll
-          for (int w = 1; w < WPB; ++w) a = fmaxf(a, s_amax[w][tid]);
-        }
-        const float sc = fmaxf(__fdiv_rn(a, 127.f), 1e-30f);
-        s_sq[0][tid] = sc;
-        s_sq[1][tid] = __fdiv_rn(1.f, sc);
-      }
-      __syncthreads();
-#pragma unroll
-      for (int r = 0; r < 4; ++r) qsc[r] = s_sq[0][r], qrcp[r] = s_sq[1][r];
+      const float sc = fmaxf(__fdiv_rn(a, 127.f), 1e-30f);
+      s_sq[0][tid] = sc;
+      s_sq[1][tid] = __fdiv_rn(1.f, sc);
     }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < 4; ++r) qsc[r] = s_sq[0][r], qrcp[r] = s_sq[1][r];
     const bool out0 = blockIdx.x == 0 && qout != nullptr;
     if (blockIdx.x == 0 && sout != nullptr && tid < M)
       sout[tid] = tid == 0 ? qsc[0] : tid == 1 ? qsc[1] : tid == 2 ? qsc[2] : qsc[3];
