@@ -314,17 +314,19 @@ int saber_iu8_linear_fused(saber_iu8_ctx *ctx, int wkind, const void *x_bf16, co
  * its dense MLP is three launches (crates/saber-kernels/src/macaq_iu8.rs:864-875), whose bytes this
  * launch reproduces. x bf16 [m, hidden]; w_gu W4 [2*inter, hidden] (gate rows, then up rows) with
  * ws_gu f32 [2*inter]; w_dn W4 [hidden, inter] with ws_dn f32 [hidden]; c bf16 [m, hidden].
- * Workspaces (the descriptor lists them): gu bf16 [m, 2*inter] and p bf16 [m, inter], undefined at
- * entry; state, SABER_IU8_MLP_CHAIN_STATE_BYTES, zero before the first launch: the workgroups meet
- * through it (an arrival word a workgroup, stamped with a generation the kernel advances), and a
- * launch that completes leaves it ready for the next. All workgroups must be resident at once: the
- * launch is refused (SABER_IU8_E_RULE) on a device that does not hold the grid. A meeting waits at
- * most `spin` polls (0: the default, about a second); a launch that gives up leaves a non-zero word
- * at state + SABER_IU8_MLP_CHAIN_STATUS_OFFSET and an undefined c: after synchronising, a caller
- * that shares the GPU with other work checks that word and, if set, zeroes `state` and runs the
- * three launches. Launches that share one `state` must not overlap. Asynchronous. */
-#define SABER_IU8_MLP_CHAIN_STATE_BYTES (12 * 1024)
-#define SABER_IU8_MLP_CHAIN_STATUS_OFFSET (10 * 1024 + 8)
+ * Workspaces (the descriptor lists them): p bf16 [m, inter], scratch (undefined at entry); state,
+ * SABER_IU8_MLP_CHAIN_STATE_BYTES, persistent in the reference's sense (include/saber_abi.h:163-174):
+ * zeroed once when allocated and left zero by a launch that completes, except its first 8 KiB (the
+ * workgroups' maxima), which every launch rewrites before reading. gu bf16 [m, 2*inter] is an optional
+ * tap (NULL: not stored). The workgroups meet through `state` (an arrival word a workgroup), so all
+ * of them must be resident at once: the launch is refused (SABER_IU8_E_RULE) on a device that does
+ * not hold the grid. A wait lasts at most `spin` polls (0: the default, about a second); a launch
+ * that gives up leaves a non-zero word at state + SABER_IU8_MLP_CHAIN_STATUS_OFFSET and an undefined
+ * c: after synchronising, a caller that shares the GPU with other work checks that word and, if set,
+ * zeroes `state` and runs the three launches. Launches that share one `state` must not overlap.
+ * Asynchronous. */
+#define SABER_IU8_MLP_CHAIN_STATE_BYTES (13 * 1024)
+#define SABER_IU8_MLP_CHAIN_STATUS_OFFSET (12 * 1024)
 int saber_iu8_mlp_chain_holds(uint32_t m, uint32_t hidden, uint32_t inter);
 int saber_iu8_resolve_mlp_chain(uint32_t m, uint32_t hidden, uint32_t inter, uint32_t spin, saber_iu8_desc *out);
 int saber_iu8_mlp_chain(saber_iu8_ctx *ctx, const void *x_bf16, const void *w_gu, const float *ws_gu, const void *w_dn,

@@ -50,7 +50,7 @@ bool fused_small_holds(uint32_t m, uint32_t k);  // the 20 KiB form: up to 4 row
 uint32_t fused_grid(uint32_t nblk);  // workgroups for nblk column blocks: one a CU, then equal shares of at most 8
 int resolve_fused(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *out);
 // The decode MLP (gate+up -> SiLU * up + requant -> down) as one persistent launch; spin 0 = the default.
-constexpr uint32_t MLP_CHAIN_STATE_BYTES = 12 * 1024;  // the kernel's state block (kernels/iu8_chain.h)
+constexpr uint32_t MLP_CHAIN_STATE_BYTES = 13 * 1024;  // the kernel's state block (kernels/iu8_chain.h)
 constexpr uint32_t MLP_CHAIN_MAX_GRID = 512;           // arrival words and maxima slots in the state block
 constexpr uint32_t MLP_CHAIN_SPIN = 1u << 20;  // polls a meeting waits at most (about a microsecond each)
 int resolve_mlp_chain(uint32_t m, uint32_t hidden, uint32_t inter, uint32_t spin, saber_iu8_desc *out);

@@ -22,91 +22,115 @@
 // launches -- a chain with the activation as a phase of its own between two meetings ran no faster
 // than the three launches, which is why the activation sits in the first linear's epilogue.
 //
-// A meeting is a word a workgroup, not a shared counter: a workgroup that arrives stores the
-// launch's generation and the phase into its own word (straight through to memory, behind its
-// completed data stores), and a waiting workgroup reads all the words at once, one a lane. 512
-// read-modify-writes of one counter a meeting, which the memory system performs one after another
-// (about 20 ns each), cost 10 us a meeting (measured); the words cost a store and a load. The generation lives
-// in the state block and is advanced by workgroup 0 once every workgroup has read it, so the words
-// never need clearing: a launch that completes leaves the state block ready for the next one.
+// The meeting is a word a workgroup, not a shared counter: a workgroup that arrives stores 1 into its
+// own word (straight through to memory, behind its completed data stores); the LAST workgroup of the
+// grid collects -- it reads all the words at once, one a lane, and when all are set stores the `go`
+// word, which every waiting workgroup polls with one lane. (512 read-modify-writes of one counter a
+// meeting, which the memory system performs one after another at about 20 ns each, cost 10 us a
+// meeting; every workgroup reading all the words itself -- 512 x 2 KB a microsecond out of one memory
+// channel -- held the workgroups still streaming weights back by 3-5 us. Both measured.)
+// The state block is a Persistent workspace in the reference's sense (include/saber_abi.h:163-174:
+// zeroed once when allocated, left zero by the kernel): a workgroup that has seen `go` sets its
+// `passed` word, and the collector -- at once when it has no column block of the second linear, else
+// behind its own -- waits until every waiting workgroup has passed and then clears the words, the
+// passed words and `go`. A launch that completes leaves every word it wrote at zero except the
+// maxima slots, which every launch rewrites in full before reading them.
 //
-// A meeting polls at most `spin` times (a bounded wait: about a microsecond a poll); past that the
-// workgroup raises the status word and leaves, and so does every other one at its next meeting, so
-// a launch that cannot complete ends instead of hanging. The host then zeroes the state block
-// before it is used again.
+// A wait polls at most `spin` times (a bounded wait: about a microsecond a poll); past that the
+// workgroup raises the status word and leaves, and so does every other one at its next look, so a
+// launch that cannot complete ends instead of hanging; nothing is cleared then, and the host zeroes
+// the state block before it is used again.
 //
 // The state block (IU8_CHAIN_STATE_BYTES, zero before the first launch):
 //   [0, 8 KiB)        512 slots of 4 floats: a workgroup's maxima of |p|, a row
-//   [8 KiB, 10 KiB)   512 arrival words
-//   [10 KiB]          generation;  [10 KiB + 8]  status (non-zero: a meeting timed out);  [10 KiB + 12]  go
+//   [8 KiB, 10 KiB)   512 arrival words          [10 KiB, 12 KiB)  512 passed words
+//   [12 KiB]          status (non-zero: a wait timed out);  [12 KiB + 4]  go
 #pragma once
 #include "iu8_decq.h"
 
 #define IU8_CHAIN_MAXG 512
-#define IU8_CHAIN_STATE_BYTES (12 * 1024)
+#define IU8_CHAIN_STATE_BYTES (13 * 1024)
 #define IU8_CHAIN_WORDS_OFF (8 * 1024)
-#define IU8_CHAIN_GEN_OFF (10 * 1024)
+#define IU8_CHAIN_PASSED_OFF (10 * 1024)
+#define IU8_CHAIN_STATUS_OFF (12 * 1024)
 
 struct iu8_chain_sync {
-  unsigned *words;  // arrival words, one a workgroup
-  int *status;      // status[0] != 0: a meeting timed out; status[1]: the collector's `go` word (8-byte aligned pair)
-  unsigned base;    // 4 * the launch's generation: phase ph of this launch is the value base + ph
-  int spin;         // polls a meeting waits at most
+  unsigned *words;   // arrival words, one a workgroup
+  unsigned *passed;  // a waiting workgroup has seen `go`
+  int *status;       // status[0] != 0: a wait timed out; status[1]: the collector's `go` word (an 8-byte aligned pair)
+  int nwait;         // workgroups that wait at the meeting: those with a column block of the second linear
+  int spin;          // polls a wait lasts at most
 };
+static __device__ __forceinline__ unsigned iu8_chain_ld(const unsigned *p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+static __device__ __forceinline__ void iu8_chain_st(unsigned *p, unsigned v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
 
 // This workgroup's stores are in memory, then its word says so.
-static __device__ __forceinline__ void iu8_chain_arrive(const iu8_chain_sync &S, unsigned phase) {
+static __device__ __forceinline__ void iu8_chain_arrive(const iu8_chain_sync &S) {
   iu8_stores_done();
   __syncthreads();
-  if (threadIdx.x == 0) __hip_atomic_store(S.words + blockIdx.x, S.base + phase, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+  if (threadIdx.x == 0) iu8_chain_st(S.words + blockIdx.x, 1u);
 }
-// Returns true once every workgroup's word has reached `phase`, false when the wait ran out or
-// another workgroup's did (status raised). Workgroup 0 collects: it reads all the words at once, one
-// a lane (gridDim.x <= blockDim.x), and when all have arrived stores the `go` word; every other
-// workgroup polls that one word with one lane. (Every workgroup reading all the words -- 512 x 2 KB a
-// microsecond out of one memory channel -- held back the workgroups still streaming their weights
-// through that channel by 3-5 us, measured from timestamps inside the kernel.)
-static __device__ __forceinline__ bool iu8_chain_wait(const iu8_chain_sync &S, unsigned phase) {
-  const unsigned target = S.base + phase;
-  unsigned *go = (unsigned *)S.status + 1;
+// The whole workgroup: true once `n` words from `w` on are all set, false when the polls ran out or a
+// wait elsewhere did (status raised). n <= blockDim.x: one word a lane.
+static __device__ __forceinline__ bool iu8_chain_all_set(const iu8_chain_sync &S, const unsigned *w, int n) {
   bool ok = false;
-  if (blockIdx.x == 0) {
-    const bool mine = threadIdx.x < gridDim.x;
-    for (int n = 0; n < S.spin; ++n) {
-      int pending = 0;
-      if (mine) pending = (int)(__hip_atomic_load(S.words + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) - target) < 0;
-      if (threadIdx.x == blockDim.x - 1) pending |= 2 * (__hip_atomic_load(S.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) != 0);
-      const int any = __syncthreads_or(pending);
-      if (any & 2) break;
-      if (any == 0) {
-        ok = true;
-        break;
-      }
+  for (int i = 0; i < S.spin; ++i) {
+    int pending = (int)threadIdx.x < n && iu8_chain_ld(w + threadIdx.x) == 0u;
+    if (threadIdx.x == blockDim.x - 1) pending |= 2 * (iu8_chain_ld((const unsigned *)S.status) != 0u);
+    const int any = __syncthreads_or(pending);
+    if (any & 2) break;
+    if (any == 0) {
+      ok = true;
+      break;
     }
-    if (threadIdx.x == 0) {
-      if (ok) __hip_atomic_store(go, target, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-      else __hip_atomic_store(S.status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-    }
+  }
+  if (!ok && threadIdx.x == 0) iu8_chain_st((unsigned *)S.status, 1u);
+  return ok;
+}
+// The collector's first half: every workgroup has arrived -> `go`.
+static __device__ __forceinline__ bool iu8_chain_collect(const iu8_chain_sync &S) {
+  const bool ok = iu8_chain_all_set(S, S.words, (int)gridDim.x);
+  if (ok && threadIdx.x == 0) iu8_chain_st((unsigned *)S.status + 1, 1u);
+  return ok;
+}
+// The collector's second half: every waiting workgroup has seen `go` -> everything back to zero.
+static __device__ __forceinline__ void iu8_chain_clear(const iu8_chain_sync &S) {
+  if (!iu8_chain_all_set(S, S.passed, S.nwait)) return;
+  if ((int)threadIdx.x < (int)gridDim.x) iu8_chain_st(S.words + threadIdx.x, 0u);
+  if ((int)threadIdx.x < S.nwait) iu8_chain_st(S.passed + threadIdx.x, 0u);
+  if (threadIdx.x == 0) iu8_chain_st((unsigned *)S.status + 1, 0u);
+}
+// A waiting workgroup: true once `go` is set (and says that it has seen it), false when the polls ran
+// out or a wait elsewhere did. The collector itself collects here.
+static __device__ __forceinline__ bool iu8_chain_wait(const iu8_chain_sync &S) {
+  if (blockIdx.x == gridDim.x - 1) {
+    const bool ok = iu8_chain_collect(S);
+    if (ok && threadIdx.x == 0) iu8_chain_st(S.passed + blockIdx.x, 1u);
     return ok;
   }
   __shared__ int s_ok;
   if (threadIdx.x == 0) {
     int good = 0;
-    for (int n = 0; n < S.spin; ++n) {
+    for (int i = 0; i < S.spin; ++i) {
       // status and go, one 8-byte load
       const unsigned long long v = __hip_atomic_load((const unsigned long long *)S.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
       if ((unsigned)v != 0u) break;
-      if ((int)((unsigned)(v >> 32) - target) >= 0) {
+      if ((unsigned)(v >> 32) != 0u) {
         good = 1;
         break;
       }
       __builtin_amdgcn_s_sleep(2);
     }
-    if (!good) __hip_atomic_store(S.status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    if (good) iu8_chain_st(S.passed + blockIdx.x, 1u);
+    else iu8_chain_st((unsigned *)S.status, 1u);
     s_ok = good;
   }
   __syncthreads();
-  ok = s_ok != 0;
+  const bool ok = s_ok != 0;
   __syncthreads();
   return ok;
 }
@@ -115,7 +139,7 @@ static __device__ __forceinline__ bool iu8_chain_wait(const iu8_chain_sync &S, u
 struct iu8_chain_hook {
   iu8_chain_sync S;
   const float *slots;
-  __device__ bool wait() const { return iu8_chain_wait(S, 1u); }
+  __device__ bool wait() const { return iu8_chain_wait(S); }
   __device__ void amax(float out[4]) const {
     __shared__ float s_m[16][4];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -148,21 +172,23 @@ __device__ __forceinline__ void iu8_chain_mlp(const unsigned short *__restrict__
                                               unsigned short *__restrict__ c, int M, int H, int I, int spin) {
   static_assert(WPB * 64 >= IU8_CHAIN_MAXG, "a lane an arrival word");
   float *slots = (float *)state;
-  unsigned *gen = (unsigned *)(state + IU8_CHAIN_GEN_OFF);
-  // the generation: read by every workgroup before it arrives, advanced by workgroup 0 behind the
-  // meeting -- when every workgroup has arrived and so has read it
-  const unsigned g = __hip_atomic_load(gen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-  const iu8_chain_sync S{(unsigned *)(state + IU8_CHAIN_WORDS_OFF), (int *)(gen + 2), 4u * g, spin};
+  constexpr int BLK2 = (WPB / KW) * NT * 16;  // columns of the second linear a workgroup and block
+  const int G = gridDim.x;
+  const iu8_chain_sync S{(unsigned *)(state + IU8_CHAIN_WORDS_OFF), (unsigned *)(state + IU8_CHAIN_PASSED_OFF),
+                         (int *)(state + IU8_CHAIN_STATUS_OFF), min(G, (H + BLK2 - 1) / BLK2), spin};
+  const bool collector = (int)blockIdx.x == G - 1;
   // phase 1: [gate | up] = x . Wgu^T (quantisation of x fused), p and this workgroup's maxima from its
   // epilogue, stored through; gu (may be null) is a tap
   iu8_decq_body<false, NT, KW, WPB, D, 1>(x, w_gu, ws_gu, nullptr, nullptr, gu, M, I, H,
                                           iu8_decq_pairhook{p, slots + blockIdx.x * 4});
-  iu8_chain_arrive(S, 1u);
-  // a workgroup with no column block of the second linear is done (workgroup 0 always has one)
-  constexpr int BLK2 = (WPB / KW) * NT * 16;
-  if ((int)blockIdx.x * BLK2 >= H) return;
+  iu8_chain_arrive(S);
+  if ((int)blockIdx.x >= S.nwait) {
+    // no column block of the second linear: done -- but the collector collects, and clears at once
+    if (collector && iu8_chain_collect(S)) iu8_chain_clear(S);
+    return;
+  }
   // phase 2: c = p . Wdn^T; the hook waits for the meeting behind the first weight loads
   iu8_decq_body<false, NT, KW, WPB, D, 2>(p, w_dn, ws_dn, nullptr, nullptr, c, M, H, I, iu8_chain_hook{S, slots});
-  if (blockIdx.x == 0 && threadIdx.x == 0 && __hip_atomic_load(S.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) == 0)
-    __hip_atomic_store(gen, g + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+  // (one answer for the whole workgroup: the clear holds barriers)
+  if (collector && __syncthreads_or(iu8_chain_ld((const unsigned *)S.status) != 0u) == 0) iu8_chain_clear(S);
 }

@@ -36,9 +36,9 @@
 // THE DECODE MLP CHAIN: gate+up linear -> SiLU(gate) * up with its per-token requantisation -> down
 // linear, one persistent launch for at most 4 rows (iu8_chain.h). `w` / `ws` are the gate and up
 // weights as one [2n, k] operand (gate rows first), `w_b` / `ws_b` the down weights [k, n]; `gu`
-// (bf16 [m, 2n]) and `p` (bf16 [m, n]) are the launch's working rows; `state` is the 12 KiB block
-// the workgroups meet through (zero before the first launch, ready for the next after a launch that
-// completes; the word at 10 KiB + 8 non-zero: a meeting timed out, c is not valid).
+// (bf16 [m, 2n]) and `p` (bf16 [m, n]) are the launch's working rows; `state` is the 13 KiB block
+// the workgroups meet through (zero before the first launch, left zero past its first 8 KiB by a launch
+// that completes; the word at 12 KiB non-zero: a wait timed out, c is not valid).
 // The grid is the host's: every workgroup resident at once (one a CU: 16 waves), at most 512 of them,
 // at most 8 column blocks of either linear a workgroup.
 extern "C" __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4))) void macaq_iu8f_mlp_w4_tm1(

@@ -226,8 +226,8 @@ def resolve_fused(wkind, m, n, k):
     return d
 
 
-MLP_CHAIN_STATE_BYTES = 12 * 1024
-MLP_CHAIN_STATUS_OFFSET = 10 * 1024 + 8
+MLP_CHAIN_STATE_BYTES = 13 * 1024
+MLP_CHAIN_STATUS_OFFSET = 12 * 1024
 
 
 def resolve_mlp_chain(m, hidden, inter, spin=0):

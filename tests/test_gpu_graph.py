@@ -61,8 +61,8 @@ def test_launch_train_replays_bit_identically(ctx):
     train.append(lambda: ctx.quant(xp.data_ptr(), qp.data_ptr(), sp.data_ptr(), M, K, stream=sh))
     train.append(lambda: ctx.gemm_pair(qp.data_ptr(), sp.data_ptr(), w0.data_ptr(), sd0.data_ptr(), c0.data_ptr(), n0,
                                        w1.data_ptr(), sd1.data_ptr(), c1.data_ptr(), n1, M, K, stream=sh))
-    # the decode MLP as one persistent launch: its workgroups meet through a state block whose
-    # generation the kernel itself advances, so a replay needs nothing cleared or re-stamped
+    # the decode MLP as one persistent launch: its workgroups meet through a state block that the
+    # kernel itself leaves at zero, so a replay needs nothing cleared between launches
     Mc, Hc, Ic = 2, 1024, 2560
     Wg, sg = synth.weights(rng, 2 * Ic, Hc, False)
     Wd, sdn = synth.weights(rng, Hc, Ic, False)
