@@ -427,8 +427,11 @@ int saber_iu8_moe_route(saber_iu8_ctx *ctx, const void *logits_bf16, uint32_t to
 /* The router and the per-token quantisation of the layer's input in one launch (the two are
  * independent; in the reference they are two operators, moe_route.hip:108-284 and the int8 producer
  * mxfp4_hadi8.hip:22-58): what saber_iu8_moe_route and saber_iu8_quant(x, q, scale, tokens, k) would
- * write, for the few-token regime where a layer's time is its launches. x bf16 [tokens, k], q in the
- * A fragment order ([ceil(tokens/16)*16, k] bytes), scale f32 [tokens]; K % 128 == 0, K <= 16384. */
+ * write (tile_blocks 1: q in the A fragment order, [ceil(tokens/16)*16, k] bytes, what the streaming
+ * cell gathers from) or saber_iu8_quant_rowmajor (tile_blocks 8 / 16: q row-major [tokens, k], what
+ * the MFMA cells gather from). With few tokens a layer's time is its launches; with many, the
+ * router's tail -- one workgroup lays out the tables -- runs beside the quantisation instead of in
+ * front of it. x bf16 [tokens, k], scale f32 [tokens]; K % 128 == 0, K <= 16384. */
 int saber_iu8_moe_route_quant(saber_iu8_ctx *ctx, const void *logits_bf16, const void *x_bf16, void *q, float *scale,
                               uint32_t tokens, uint32_t experts, uint32_t topk, uint32_t k, uint32_t tile_blocks,
                               const saber_iu8_moe_tables *t, void *stream);

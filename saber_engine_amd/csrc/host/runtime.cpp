@@ -724,8 +724,12 @@ int saber_iu8_moe_route_quant(saber_iu8_ctx *ctx, const void *logits, const void
   if (tile_blocks == 0) return fail(SABER_IU8_E_RULE, "moe_route_quant: tile_blocks 0");
   if (k == 0 || k % 128 != 0 || k > 16384)
     return fail(SABER_IU8_E_RULE, fmt("moe_route_quant: K=%u must be a multiple of 128 (the slab) up to 16384 (a 16-element group a thread)", k));
+  // a row on 256, 512 or 1,024 threads by its length: 4, 2 or 1 rows a quantising workgroup (the kernel's own rule)
+  const uint32_t groups = k / 16, rows_wg = groups <= 256 ? 4 : groups <= 512 ? 2 : 1;
   saber_iu8_desc d;
-  if (int rc = raw_desc("moe_iu8_routeq_topk8_sort_e128", (tokens + 127) / 128 + tokens, 1, 1024, &d)) return rc;
+  if (int rc = raw_desc(tile_blocks == 1 ? "moe_iu8_routeq_topk8_sort_e128" : "moe_iu8_routeq_rm_topk8_sort_e128",
+                        (tokens + 127) / 128 + (tokens + rows_wg - 1) / rows_wg, 1, 1024, &d))
+    return rc;
   set_i32(&d, "t", tokens);
   set_i32(&d, "e_lo", 0);
   set_i32(&d, "e_loc", experts);

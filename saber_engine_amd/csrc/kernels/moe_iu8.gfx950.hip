@@ -380,11 +380,16 @@ extern "C" __global__ __launch_bounds__(MOE_THREADS) void moe_iu8_route_topk8_so
                  tile_expert, tile_row0, tile_rows, expert_cnt, meta, blk_cnt, rank, arrive, gridDim.x, blockIdx.x);
 }
 
-// The router and the tokens' quantisation in one launch, for the few-token regime where a layer's time
-// is its launches: the two do not depend on each other, so the first ceil(T / 128) workgroups route and
-// workgroup ceil(T / 128) + t quantises token t (x bf16 [T, k] -> codes in the A fragment order +
-// scale[t]; macaq_i8.h:10-13, one 16-element group a thread, k <= 16,384). grid [ceil(T/128) + T, 1, 1].
-extern "C" __global__ __launch_bounds__(MOE_THREADS) void moe_iu8_routeq_topk8_sort_e128(
+// The router and the tokens' quantisation in one launch: the two do not depend on each other, so the
+// first ceil(T / 128) workgroups route and the ones behind them quantise the tokens (x bf16 [T, k] ->
+// codes + scale[t]; macaq_i8.h:10-13, one 16-element group a thread, k <= 16,384), a row on 256, 512
+// or 1,024 threads by its length, so 4, 2 or 1 rows a workgroup. With few tokens a layer's time is
+// its launches; with many the router's tail (one workgroup lays out the tables) runs beside the
+// quantisation instead of in front of it. Codes in the A fragment order (RM false, for the streaming
+// cell) or row-major (RM true, for the MFMA cells' gather). grid [ceil(T/128) + ceil(T / rows a
+// workgroup), 1, 1].
+template <bool RM>
+static __device__ __forceinline__ void moe_routeq_body(
     const unsigned short *__restrict__ logits, int T, int e_lo, int e_loc, int tile_blocks, int with_shared,
     int *__restrict__ topk_ids, float *__restrict__ topk_w, int *__restrict__ route_pos, int *__restrict__ row_tok,
     int *__restrict__ row_route, int *__restrict__ tile_expert, int *__restrict__ tile_row0,
@@ -399,11 +404,14 @@ extern "C" __global__ __launch_bounds__(MOE_THREADS) void moe_iu8_routeq_topk8_s
     return;
   }
   __shared__ float s_max[MOE_THREADS / 64];
-  const int row = blockIdx.x - nblk, g = threadIdx.x, G = k >> 4;
+  const int G = k >> 4, span = G <= 256 ? 256 : G <= 512 ? 512 : 1024;  // threads a row
+  const int sub = threadIdx.x / span, g = threadIdx.x - sub * span;
+  const int row = ((int)blockIdx.x - nblk) * (MOE_THREADS / span) + sub;
+  const bool mine = row < T && g < G;
   float v[16];
 #pragma unroll
   for (int j = 0; j < 16; ++j) v[j] = 0.f;
-  if (g < G) {
+  if (mine) {
     const unsigned short *xr = x + (size_t)row * k + g * 16;
     const iu8_v4u lo = *(const iu8_v4u *)xr, hi = *(const iu8_v4u *)(xr + 8);
 #pragma unroll
@@ -420,19 +428,39 @@ extern "C" __global__ __launch_bounds__(MOE_THREADS) void moe_iu8_routeq_topk8_s
   amax = iu8_wave_max_nonneg(amax);
   if ((threadIdx.x & 63) == 0) s_max[threadIdx.x >> 6] = amax;
   __syncthreads();
-#pragma unroll
-  for (int w = 0; w < MOE_THREADS / 64; ++w) amax = fmaxf(amax, s_max[w]);
+  const int w0 = sub * (span >> 6);  // the waves of this row
+  amax = s_max[w0];
+  for (int w = 1; w < (span >> 6); ++w) amax = fmaxf(amax, s_max[w0 + w]);
   const float sc = fmaxf(__fdiv_rn(amax, 127.f), 1e-30f), rcp = __fdiv_rn(1.f, sc);
-  if (threadIdx.x == 0) scale[row] = sc;
-  if (g < G) {
+  if (g == 0 && row < T) scale[row] = sc;
+  if (mine) {
     unsigned d[4];
 #pragma unroll
     for (int w = 0; w < 4; ++w) d[w] = iu8_code4_rcp(v[w * 4], v[w * 4 + 1], v[w * 4 + 2], v[w * 4 + 3], sc, rcp);
-    // fragment (row / 16, k / 64): 1 KiB; the 16 bytes of (row % 16, k chunk (g & 3)) at (row % 16 + 16 * chunk) * 16
-    *(iu8_v4u *)(q + ((size_t)(row >> 4) * (k >> 6) + (g >> 2)) * 1024 + (g & 3) * 256 + (row & 15) * 16) =
-        iu8_v4u{d[0], d[1], d[2], d[3]};
+    if constexpr (RM) {
+      *(iu8_v4u *)(q + (size_t)row * k + g * 16) = iu8_v4u{d[0], d[1], d[2], d[3]};
+    } else {
+      // fragment (row / 16, k / 64): 1 KiB; the 16 bytes of (row % 16, k chunk (g & 3)) at (row % 16 + 16 * chunk) * 16
+      *(iu8_v4u *)(q + ((size_t)(row >> 4) * (k >> 6) + (g >> 2)) * 1024 + (g & 3) * 256 + (row & 15) * 16) =
+          iu8_v4u{d[0], d[1], d[2], d[3]};
+    }
   }
 }
+#define MOE_ROUTEQ(name, RM)                                                                                          \
+  extern "C" __global__ __launch_bounds__(MOE_THREADS) void name(                                                      \
+      const unsigned short *__restrict__ logits, int T, int e_lo, int e_loc, int tile_blocks, int with_shared,          \
+      int *__restrict__ topk_ids, float *__restrict__ topk_w, int *__restrict__ route_pos, int *__restrict__ row_tok,   \
+      int *__restrict__ row_route, int *__restrict__ tile_expert, int *__restrict__ tile_row0,                          \
+      int *__restrict__ tile_rows, int *__restrict__ expert_cnt, int *__restrict__ meta, int *__restrict__ blk_cnt,     \
+      int *__restrict__ rank, int *__restrict__ arrive, const unsigned short *__restrict__ x,                           \
+      unsigned char *__restrict__ q, float *__restrict__ scale, int k) {                                                \
+    moe_routeq_body<RM>(logits, T, e_lo, e_loc, tile_blocks, with_shared, topk_ids, topk_w, route_pos, row_tok,         \
+                        row_route, tile_expert, tile_row0, tile_rows, expert_cnt, meta, blk_cnt, rank, arrive, x, q,    \
+                        scale, k);                                                                                      \
+  }
+MOE_ROUTEQ(moe_iu8_routeq_topk8_sort_e128, false)
+MOE_ROUTEQ(moe_iu8_routeq_rm_topk8_sort_e128, true)
+#undef MOE_ROUTEQ
 
 // ---------------------------------------------------------------------------- grouped GEMMs
 // grid [ceil(N / BN), tiles_cap, 1]: blockIdx.y is a tile; a workgroup whose tile is past the live

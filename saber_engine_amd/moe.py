@@ -66,7 +66,7 @@ class MoeLayerIU8:
         """x bf16 bits [T,H] (int16 tensor), logits bf16 bits [T,E]; with a shared expert its gate logits
         (bf16 bits [T]) are read from self.sgate, which the caller fills; every launch on `stream`."""
         c, T, E, k, H, I = self.ctx, self.T, self.E, self.topk, self.H, self.I
-        if self.gather == 1 and H <= 16384:   # few tokens: the router and the quantisation in one launch
+        if H <= 16384:   # the router and the tokens' quantisation, which do not depend on each other, in one launch
             c.moe_route_quant(logits.data_ptr(), x.data_ptr(), self.q1.data_ptr(), self.s1.data_ptr(), T, E, k, H, self.tb,
                               self.tables, stream)
         else:
