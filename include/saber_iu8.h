@@ -459,6 +459,28 @@ int saber_iu8_moe_quant_rows(saber_iu8_ctx *ctx, const void *x_bf16, void *q, fl
 int saber_iu8_moe_silu_mul_quant(saber_iu8_ctx *ctx, const void *gu_bf16, void *q, float *scale, uint32_t n,
                                  uint32_t rows_cap, const saber_iu8_moe_tables *t, void *stream);
 
+/* The routed back half with few tokens as two launches instead of three (16-row tiles only,
+ * tile_blocks 1, and an intermediate width whose 16 rows fit the second launch's LDS:
+ * saber_iu8_moe_back_holds). The reference chains gate_up -> silu-quant -> down inside its persistent
+ * back half (crates/saber-kernels/hip/moe_grouped.hip:1656-1765, crates/saber-kernels/src/moe.rs:341-345);
+ * here the activation sits in the first GEMM's epilogue and the requantisation in front of the second
+ * GEMM's K loop, with the bytes of saber_iu8_moe_grouped -> saber_iu8_moe_silu_mul_quant ->
+ * saber_iu8_moe_grouped.
+ *   saber_iu8_moe_gate_up_act: a / as the token-major A edge and scales (gathered through row_tok),
+ *     xptr the experts' gate+up weights ([2 * inter, k]: gate rows, then up rows) and scales;
+ *     p bf16 [rows_cap, inter] = bf16(bf16(silu(gate)) * up).
+ *   saber_iu8_moe_down_rows: p as written above, quantised per row in front of the K loop (K = inter);
+ *     xptr the experts' down weights ([n, inter]) and scales; y bf16 [rows_cap, n]. */
+int saber_iu8_moe_back_holds(uint32_t tile_blocks, uint32_t inter);
+/* The launch law's pick: the two-launch form where it holds and an expert has at most 2.5 routes on average. */
+int saber_iu8_moe_back_pays(uint32_t tokens, uint32_t topk, uint32_t experts, uint32_t tile_blocks, uint32_t inter);
+int saber_iu8_moe_gate_up_act(saber_iu8_ctx *ctx, const void *a, const float *as, const void *xptr, void *p_bf16,
+                              uint32_t inter, uint32_t k, uint32_t tokens, uint32_t experts, uint32_t topk,
+                              uint32_t tile_blocks, const saber_iu8_moe_tables *t, void *stream);
+int saber_iu8_moe_down_rows(saber_iu8_ctx *ctx, const void *p_bf16, const void *xptr, void *y_bf16, uint32_t n,
+                            uint32_t inter, uint32_t tokens, uint32_t experts, uint32_t topk, uint32_t tile_blocks,
+                            const saber_iu8_moe_tables *t, void *stream);
+
 /* Weighted combine: out[t] = bf16(sum_k w[t,k] * Y[pos(t,k)]) in top-k order; y bf16 [rows_cap, h]. */
 int saber_iu8_moe_combine(saber_iu8_ctx *ctx, const void *y_bf16, const saber_iu8_moe_tables *t, void *out_bf16,
                           uint32_t tokens, uint32_t topk, uint32_t h, void *stream);

@@ -183,6 +183,15 @@ std::string band_toml() {
     put(o, "tile_blocks_1_last_tokens", t1);
     put(o, "tile_blocks_8_last_tokens", t8);
     put(o, "tile_blocks_above", 16);
+    // the back half as two launches (activation in gate+up's epilogue, requantisation in front of down's K loop)
+    uint32_t tf = 0;
+    for (uint32_t t = 1; t <= t1; ++t)
+      if (saber_iu8_moe_back_pays(t, 8, 128, 1, 1536)) tf = t;
+    put(o, "fused_back_last_tokens", tf);
+    uint32_t imax = 0;
+    for (uint32_t i = 128; i <= 8192; i += 128)
+      if (saber_iu8_moe_back_holds(1, i)) imax = i;
+    put(o, "fused_back_inter_max", imax);
   }
 
   // ---- cells

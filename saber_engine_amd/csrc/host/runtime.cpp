@@ -796,6 +796,59 @@ int saber_iu8_moe_grouped(saber_iu8_ctx *ctx, const void *a, const float *as, co
   return saber_iu8_launch(ctx, &d, b, sizeof b / sizeof b[0], stream);
 }
 
+// The back half with few tokens: 16 rows of `inter` codes must fit the second launch's 24 KiB of staged rows.
+int saber_iu8_moe_back_holds(uint32_t tile_blocks, uint32_t inter) {
+  return tile_blocks == 1 && inter != 0 && inter % 128 == 0 && (uint64_t)16 * inter <= 24 * 1024;
+}
+
+// ... and pays while an expert has few rows: every workgroup of a tile repeats the tile's requantisation and the
+// gate+up epilogue spends an exp and a divide a value on the few lanes that hold live rows. Measured on the 128-expert
+// top-8 layer (hidden 4096, inter 1536): 144.9 -> 139.9 us a layer at 16 tokens, 197.9 -> 193.0 at 32, even at 48,
+// 242.4 -> 247.7 at 64: up to 2.5 routes an expert.
+int saber_iu8_moe_back_pays(uint32_t tokens, uint32_t topk, uint32_t experts, uint32_t tile_blocks, uint32_t inter) {
+  return saber_iu8_moe_back_holds(tile_blocks, inter) && experts != 0 && (uint64_t)tokens * topk * 2 <= (uint64_t)experts * 5;
+}
+
+static int moe_back_launch(saber_iu8_ctx *ctx, const std::string &name, uint32_t gx, const void *a,
+                           const float *as, const void *xptr, void *c, uint32_t n, uint32_t k, uint32_t tokens,
+                           uint32_t experts, uint32_t topk, const saber_iu8_moe_tables *t, void *stream) {
+  const uint32_t tiles_cap = t->sgate ? saber_iu8_moe_tiles_cap_shared(tokens, topk, experts, 1) : saber_iu8_moe_tiles_cap(tokens, topk, experts, 1);
+  saber_iu8_desc d;
+  if (int rc = raw_desc(name.c_str(), gx, tiles_cap, 512, &d)) return rc;
+  set_i32(&d, "n", n);
+  set_i32(&d, "k", k);
+  set_i32(&d, "pmax", 0);
+  set_null(&d, "p");
+  set_null(&d, "cnt");
+  if (!as) set_null(&d, "as");
+  const saber_iu8_binding b[] = {{"a", (void *)a},           {"xptr", (void *)xptr},         {"tile_expert", t->tile_expert},
+                                 {"tile_row0", t->tile_row0}, {"tile_rows", t->tile_rows},   {"row_tok", t->row_tok},
+                                 {"meta", t->meta},           {"c", c},                      {"as", (void *)as}};
+  return saber_iu8_launch(ctx, &d, b, as ? 9 : 8, stream);  // without scales the last binding is left out
+}
+
+int saber_iu8_moe_gate_up_act(saber_iu8_ctx *ctx, const void *a, const float *as, const void *xptr, void *p, uint32_t inter,
+                              uint32_t k, uint32_t tokens, uint32_t experts, uint32_t topk, uint32_t tile_blocks,
+                              const saber_iu8_moe_tables *t, void *stream) {
+  if (int rc = moe_check("moe_gate_up_act", tokens, experts, topk, t)) return rc;
+  if (!saber_iu8_moe_back_holds(tile_blocks, inter) || k == 0 || k % 128 != 0)
+    return fail(SABER_IU8_E_RULE, fmt("moe_gate_up_act: tile_blocks %u, inter %u, K=%u; the fused back half is the 16-row cell's "
+                                      "(tile_blocks 1), inter a multiple of 128 up to 1536, K a multiple of 128", tile_blocks, inter, k));
+  return moe_back_launch(ctx, "moe_iu8_grouped_w4_decpa_g1", (inter + 15) / 16, a, as, xptr, p, 2 * inter, k, tokens, experts, topk,
+                         t, stream);
+}
+
+int saber_iu8_moe_down_rows(saber_iu8_ctx *ctx, const void *p, const void *xptr, void *y, uint32_t n, uint32_t inter,
+                            uint32_t tokens, uint32_t experts, uint32_t topk, uint32_t tile_blocks,
+                            const saber_iu8_moe_tables *t, void *stream) {
+  if (int rc = moe_check("moe_down_rows", tokens, experts, topk, t)) return rc;
+  if (!saber_iu8_moe_back_holds(tile_blocks, inter) || n == 0 || n % 16 != 0)
+    return fail(SABER_IU8_E_RULE, fmt("moe_down_rows: tile_blocks %u, inter %u, N=%u; the fused back half is the 16-row cell's "
+                                      "(tile_blocks 1), inter a multiple of 128 up to 1536, N a multiple of 16", tile_blocks, inter, n));
+  return moe_back_launch(ctx, "moe_iu8_grouped_w4_deckq_g0", (n + 63) / 64, p, nullptr, xptr, y, n, inter, tokens,
+                         experts, topk, t, stream);
+}
+
 int saber_iu8_moe_quant_rows(saber_iu8_ctx *ctx, const void *x, void *q, float *scale, uint32_t k, uint32_t rows_cap,
                              const saber_iu8_moe_tables *t, void *stream) {
   if (!t) return fail(SABER_IU8_E_ARG, "moe_quant_rows: null tables");

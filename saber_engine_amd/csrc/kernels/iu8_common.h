@@ -51,6 +51,12 @@ static __device__ __forceinline__ unsigned iu8_bf16_bits(float x) {
   return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
 }
 static __device__ __forceinline__ float iu8_bf16_f32(unsigned short b) { return __uint_as_float((unsigned)b << 16); }
+// bf16(silu(x)) as the producer kernels compute it (macaq_i8q: i8q_silu_bf16; the law
+// crates/saber-kernels/hip/mxfp4_hadi8.hip:118-146): x / (1 + expf(-x)), IEEE divide, one bf16 rounding.
+static __device__ __forceinline__ float iu8_silu_bf16(float x) {
+#pragma clang fp contract(off)
+  return iu8_bf16_f32((unsigned short)iu8_bf16_bits(x / (1.f + expf(-x))));
+}
 
 template <bool W8>
 static __device__ __forceinline__ float iu8_wsu(const float *__restrict__ ws, int n) {

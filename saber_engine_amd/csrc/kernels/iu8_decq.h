@@ -31,10 +31,6 @@
 // then `hook.wait()` returns when every workgroup's share of the rows is in memory, the rows are
 // loaded coherently, and their maxima come from `hook.amax(out)` (found by the producers) instead of a
 // pass over the rows.
-static __device__ __forceinline__ float iu8_silu_bf16(float x) {  // as the producer kernels compute it (macaq_i8q: i8q_silu_bf16)
-#pragma clang fp contract(off)
-  return iu8_bf16_f32((unsigned short)iu8_bf16_bits(x / (1.f + expf(-x))));
-}
 struct iu8_decq_pairhook {
   unsigned short *p;  // bf16 [M, N]
   float *slot;        // this workgroup's 4 maxima

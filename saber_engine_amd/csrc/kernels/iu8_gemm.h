@@ -33,7 +33,17 @@ static __device__ __forceinline__ iu8_blk iu8_blk_of_grid() {
 }
 
 // ============================================================================ decode band
-template <int TM, bool W8, int NT, int KW, int WPB, int D, int ALDS, bool ACC>
+// MODE 1, the gate+up projection of an MLP with the activation in its epilogue: W holds N/2 gate rows
+// and then N/2 up rows, a wave's two tiles are the gate tile and the up tile of the same 16 columns,
+// and C is p = bf16(bf16(silu(gate)) * up), bf16 [rows, N/2] -- what the three steps (this GEMM to
+// bf16, SiLU * up, bf16) write (crates/saber-kernels/hip/mxfp4_hadi8.hip:118-146), without the
+// [gate | up] matrix in memory. A column block is WN*16 columns of p.
+// MODE 2, the projection behind it: A is those bf16 rows themselves ([rows, K], in place), quantised
+// here by the per-token law (crates/saber-kernels/hip/macaq_i8.h:10-13) into the staged LDS form, the
+// scales kept in LDS for the epilogue; `as` is not read. The tile's rows must fit: pow2(rows) * K <=
+// ALDS KiB (the host's rule). Every workgroup of a tile repeats its rows' quantisation, which is what
+// a producer launch in front would cost once -- worth it for the few rows an expert has in decode.
+template <int TM, bool W8, int NT, int KW, int WPB, int D, int ALDS, bool ACC, int MODE = 0>
 __device__ __forceinline__ void iu8_dec_body(const iu8_u8 *__restrict__ A, const iu8_u8 *__restrict__ W,
                                              const float *__restrict__ as, const float *__restrict__ ws,
                                              int *__restrict__ P, int *__restrict__ cnt, void *__restrict__ Cv,
@@ -41,6 +51,9 @@ __device__ __forceinline__ void iu8_dec_body(const iu8_u8 *__restrict__ A, const
   const int M = R.rows;
   static_assert(WPB % KW == 0, "k-waves divide the workgroup");
   static_assert(ALDS == 0 || TM == 1, "LDS staging of A is the M <= 16 form");
+  constexpr bool PAIR = MODE == 1, AQ = MODE == 2;
+  static_assert(!PAIR || (NT == 2 && TM == 1 && !W8 && !ACC), "the paired form: a gate tile and an up tile a wave");
+  static_assert(!AQ || (ALDS > 0 && !ACC), "rows quantised here are staged in LDS");
   constexpr int WN = WPB / KW;
   constexpr int NTHR = WPB * 64;
   constexpr int WSTEP = W8 ? 2048 : 1024;  // bytes of one 16-row weight tile per 128-deep K step
@@ -68,7 +81,8 @@ __device__ __forceinline__ void iu8_dec_body(const iu8_u8 *__restrict__ A, const
   const iu8_u8 *wp[NT];
 #pragma unroll
   for (int j = 0; j < NT; ++j) {
-    const int ntj = min(nt0 + j, ntiles - 1);  // a tile past N re-reads the last one and stores nothing
+    // a tile past N re-reads the last one and stores nothing; paired: tile j = 0 of the gate rows, 1 of the up rows
+    const int ntj = PAIR ? j * (ntiles >> 1) + min(B.bx * WN + wn, (ntiles >> 1) - 1) : min(nt0 + j, ntiles - 1);
     wp[j] = W + ((size_t)ntj * steps + s_lo + wk) * WSTEP + lane * 16;
   }
 
@@ -87,11 +101,30 @@ __device__ __forceinline__ void iu8_dec_body(const iu8_u8 *__restrict__ A, const
   constexpr bool A_INREG = A_PER <= 8;
   iu8_v4u areg[A_INREG ? A_PER : 1];
   int a_pieces = 0;
+  // rows quantised here (AQ): 16-element groups of the bf16 rows, group i = row * K/16 + k/16; a thread's
+  // first group stays in registers (all of them for up to NTHR groups: 5 rows of 1,536), later ones are
+  // read again for the codes, out of the cache
+  iu8_v4u xraw[2];
+  __shared__ unsigned s_rmax[AQ ? 16 : 1];
+  __shared__ float s_rsc[AQ ? 16 : 1], s_rrcp[AQ ? 16 : 1];
+  const int k16 = K >> 4, q_groups = M * k16;
+  auto q_src = [&](int i) {
+    const int row = i / k16, g = i - row * k16;
+    return (const iu8_v4u *)((const unsigned short *)A + (size_t)iu8_arow(R, row) * K + g * 16);
+  };
   if constexpr (ALDS > 0) {
     while ((1 << mr_shift) < M) ++mr_shift;
     a_pieces = ((s_hi - s_lo) * 2 * 4) << mr_shift;
     staged = M <= 16 && a_pieces * 16 <= ABYTES;
-    if (staged) {
+    if constexpr (AQ) {
+      if (!staged || Z != 1) return;  // the host's rule keeps such a launch out; nothing is stored
+      if (tid < 16) s_rmax[tid] = 0u;
+      if (tid < q_groups) {
+        const iu8_v4u *src = q_src(tid);
+        xraw[0] = src[0];
+        xraw[1] = src[1];
+      }
+    } else if (staged) {
       auto a_src = [&](int piece) {
         const int r = piece & ((1 << mr_shift) - 1), g = (piece >> mr_shift) & 3, kt = piece >> (mr_shift + 2);
         const int ar = iu8_arow(R, r);
@@ -179,7 +212,50 @@ __device__ __forceinline__ void iu8_dec_body(const iu8_u8 *__restrict__ A, const
 #pragma unroll
       for (int i = 0; i < D; ++i)
         if (i < T) issue(i, i);
-      if constexpr (A_INREG) {
+      if constexpr (AQ) {
+#pragma clang fp contract(off)
+        // the rows' maxima (f32 maxima of |x| as the producers take them, met by an integer max in LDS:
+        // non-negative floats order as their bit patterns), scales by 16 lanes, codes into the staged form
+        auto val = [&](const iu8_v4u (&x)[2], int j) {
+          const unsigned w = x[j >> 3][(j >> 1) & 3];
+          return __uint_as_float((j & 1) ? (w & 0xFFFF0000u) : (w << 16));
+        };
+        auto group_max = [&](const iu8_v4u (&x)[2], int i) {
+          float mx = 0.f;
+#pragma unroll
+          for (int j = 0; j < 16; ++j) mx = fmaxf(mx, fabsf(val(x, j)));
+          atomicMax(&s_rmax[i / k16], __float_as_uint(mx));
+        };
+        auto group_codes = [&](const iu8_v4u (&x)[2], int i) {
+          const int row = i / k16, g = i - row * k16;
+          const float sc = s_rsc[row], rcp = s_rrcp[row];
+          unsigned d[4];
+#pragma unroll
+          for (int w = 0; w < 4; ++w) d[w] = iu8_code4_rcp(val(x, w * 4), val(x, w * 4 + 1), val(x, w * 4 + 2), val(x, w * 4 + 3), sc, rcp);
+          // staged piece ((kt * 4 + chunk) * MR + row): the 16 codes of k = kt * 64 + chunk * 16, i.e. group g = kt * 4 + chunk
+          *(iu8_v4u *)&s_mem[((g << mr_shift) + row) << 4] = iu8_v4u{d[0], d[1], d[2], d[3]};
+        };
+        __syncthreads();
+        if (tid < q_groups) group_max(xraw, tid);
+        for (int i = tid + NTHR; i < q_groups; i += NTHR) {
+          const iu8_v4u *src = q_src(i);
+          const iu8_v4u x[2] = {src[0], src[1]};
+          group_max(x, i);
+        }
+        __syncthreads();
+        if (tid < 16) {
+          const float sc = fmaxf(__fdiv_rn(__uint_as_float(s_rmax[tid]), 127.f), 1e-30f);
+          s_rsc[tid] = sc;
+          s_rrcp[tid] = __fdiv_rn(1.f, sc);
+        }
+        __syncthreads();
+        if (tid < q_groups) group_codes(xraw, tid);
+        for (int i = tid + NTHR; i < q_groups; i += NTHR) {
+          const iu8_v4u *src = q_src(i);
+          const iu8_v4u x[2] = {src[0], src[1]};
+          group_codes(x, i);
+        }
+      } else if constexpr (A_INREG) {
 #pragma unroll
         for (int p = 0; p < A_PER; ++p)
           if (p * NTHR + tid < a_pieces) *(iu8_v4u *)&s_mem[(p * NTHR + tid) * 16] = areg[p];
@@ -247,6 +323,22 @@ __device__ __forceinline__ void iu8_dec_body(const iu8_u8 *__restrict__ A, const
   }
 
   const int nq = lg * 4;
+  if constexpr (PAIR) {
+#pragma clang fp contract(off)
+    const int tp = B.bx * WN + wn, half = N >> 1;  // this wave's tile of p
+    if (wk != 0 || tp >= (ntiles >> 1) || ml >= M) return;
+    const int n = tp * 16 + nq;
+    const float am = as[iu8_arow(R, ml)];
+    unsigned h[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const float g = iu8_bf16_f32((unsigned short)iu8_bf16_bits(iu8_epi(acc[0][0][r], am, iu8_wsu<W8>(ws, n + r))));
+      const float u = iu8_bf16_f32((unsigned short)iu8_bf16_bits(iu8_epi(acc[0][1][r], am, iu8_wsu<W8>(ws, half + n + r))));
+      h[r] = iu8_bf16_bits(iu8_silu_bf16(g) * u);
+    }
+    *(iu8_v2u *)((unsigned short *)Cv + (size_t)(R.row0 + ml) * half + n) = iu8_v2u{h[0] | (h[1] << 16), h[2] | (h[3] << 16)};
+    return;
+  }
   if (Z == 1) {
     if (wk != 0) return;
 #pragma unroll
@@ -264,7 +356,7 @@ __device__ __forceinline__ void iu8_dec_body(const iu8_u8 *__restrict__ A, const
         if constexpr (ACC) {
           *(iu8_v4i *)((int *)Cv + crow + n) = acc[i][j];
         } else {
-          const float am = as[iu8_arow(R, m)];
+          const float am = AQ ? s_rsc[m] : as[iu8_arow(R, m)];
           unsigned h[4];
 #pragma unroll
           for (int r = 0; r < 4; ++r) h[r] = iu8_bf16_bits(iu8_epi(acc[i][j][r], am, wsu[r]));

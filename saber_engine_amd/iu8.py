@@ -146,6 +146,12 @@ def lib():
         L.saber_iu8_moe_grouped.argtypes = ([C.c_void_p] * 5 + [C.c_uint32, C.c_uint32, C.c_int] + [C.c_uint32] * 4 +
                                             [C.POINTER(MoeTables), C.c_void_p])
         L.saber_iu8_moe_quant_rows.argtypes = [C.c_void_p] * 4 + [C.c_uint32, C.c_uint32, C.POINTER(MoeTables), C.c_void_p]
+        L.saber_iu8_moe_back_holds.restype = C.c_int
+        L.saber_iu8_moe_back_holds.argtypes = [C.c_uint32, C.c_uint32]
+        L.saber_iu8_moe_back_pays.restype = C.c_int
+        L.saber_iu8_moe_back_pays.argtypes = [C.c_uint32] * 5
+        L.saber_iu8_moe_gate_up_act.argtypes = [C.c_void_p] * 5 + [C.c_uint32] * 6 + [C.POINTER(MoeTables), C.c_void_p]
+        L.saber_iu8_moe_down_rows.argtypes = [C.c_void_p] * 4 + [C.c_uint32] * 6 + [C.POINTER(MoeTables), C.c_void_p]
         L.saber_iu8_moe_silu_mul_quant.argtypes = [C.c_void_p] * 4 + [C.c_uint32, C.c_uint32, C.POINTER(MoeTables), C.c_void_p]
         L.saber_iu8_moe_combine.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(MoeTables), C.c_void_p] + [C.c_uint32] * 3 + [C.c_void_p]
         L.saber_iu8_silu_table.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
@@ -437,6 +443,14 @@ class Context:
         _check(lib().saber_iu8_moe_grouped(self._h, a, a_scale, xptr, c, n, k, int(gather), tokens, experts, topk,
                                            tile_blocks, C.byref(tables), stream))
 
+    def moe_gate_up_act(self, a, a_scale, xptr, p, inter, k, tokens, experts, topk, tile_blocks, tables, stream=0):
+        _check(lib().saber_iu8_moe_gate_up_act(self._h, a, a_scale, xptr, p, inter, k, tokens, experts, topk, tile_blocks,
+                                               C.byref(tables), stream))
+
+    def moe_down_rows(self, p, xptr, y, n, inter, tokens, experts, topk, tile_blocks, tables, stream=0):
+        _check(lib().saber_iu8_moe_down_rows(self._h, p, xptr, y, n, inter, tokens, experts, topk, tile_blocks,
+                                             C.byref(tables), stream))
+
     def moe_quant_rows(self, x, q, scale, k, rows_cap, tables, stream=0):
         _check(lib().saber_iu8_moe_quant_rows(self._h, x, q, scale, k, rows_cap, C.byref(tables), stream))
 
@@ -460,6 +474,16 @@ def moe_tiles_cap(tokens, topk, experts, tile_blocks, shared=False):
 
 def moe_tile_blocks(tokens, topk, experts):
     return lib().saber_iu8_moe_tile_blocks(tokens, topk, experts)
+
+
+def moe_back_pays(tokens, topk, experts, tile_blocks, inter):
+    """The launch law's pick between the two-launch back half and the three launches."""
+    return bool(lib().saber_iu8_moe_back_pays(tokens, topk, experts, tile_blocks, inter))
+
+
+def moe_back_holds(tile_blocks, inter):
+    """The routed back half as two launches (activation in gate+up's epilogue, requantisation in front of down's K loop)."""
+    return bool(lib().saber_iu8_moe_back_holds(tile_blocks, inter))
 
 
 def gemm_workspace(wkind, m, n, k):

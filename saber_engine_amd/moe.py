@@ -1,5 +1,6 @@
-"""The routed-expert layer as a launch train over the C ABI: route+sort -> per-token quant ->
-grouped gate+up (token rows gathered) -> SiLU*up requant -> grouped down -> weighted combine.  The train and
+"""The routed-expert layer as a launch train over the C ABI: route+sort with the per-token quant ->
+grouped gate+up (token rows gathered) -> SiLU*up requant -> grouped down -> weighted combine; with few
+tokens (16-row tiles) the activation rides in gate+up's epilogue and the requant in front of down's K loop.  The train and
 its buffers follow the reference's MoE block (crates/saber-kernels/src/moe.rs:9-28, 142-171); the
 arithmetic of every GEMM is the iu8 contract.  torch is used for device memory only.
 """
@@ -10,7 +11,8 @@ from . import iu8
 
 
 class MoeLayerIU8:
-    def __init__(self, ctx, tokens, experts=128, topk=8, hidden=4096, inter=1536, tile_blocks=None, device="cuda", shared=False):
+    def __init__(self, ctx, tokens, experts=128, topk=8, hidden=4096, inter=1536, tile_blocks=None, device="cuda", shared=False,
+                 fused_back=None):
         """shared: the layer has a shared expert (crates/saber-kernels/src/moe.rs:688-711): every token also
         runs through expert index `experts`, whose weights are the last entry given to set_weights, and
         the combine adds sigmoid(sgate[t]) times that row."""
@@ -44,6 +46,9 @@ class MoeLayerIU8:
         self.gather = 1 if self.tb == 1 else 2
         self.q1 = torch.zeros(max(iu8.a_bytes(tokens, hidden), tokens * hidden), **u8)
         self.s1 = torch.zeros(tokens, dtype=torch.float32, device=device)
+        # few tokens: the back half as two launches, p = silu(gate) * up straight out of the first GEMM
+        self.fused_back = iu8.moe_back_pays(tokens, topk, experts, self.tb, inter) if fused_back is None else bool(fused_back)
+        self.p = torch.zeros((self.rows_cap, inter), dtype=torch.int16, device=device) if self.fused_back else None
         self.gu = torch.zeros((self.rows_cap, 2 * inter), dtype=torch.int16, device=device)
         self.q2 = torch.zeros(iu8.a_bytes(self.rows_cap, inter), **u8)
         self.s2 = torch.zeros(self.rows_cap, dtype=torch.float32, device=device)
@@ -75,10 +80,16 @@ class MoeLayerIU8:
                 c.quant(x.data_ptr(), self.q1.data_ptr(), self.s1.data_ptr(), T, H, stream)
             else:
                 c.quant_rowmajor(x.data_ptr(), self.q1.data_ptr(), self.s1.data_ptr(), T, H, stream)
-        c.moe_grouped(self.q1.data_ptr(), self.s1.data_ptr(), self.xptr_gu.data_ptr(), self.gu.data_ptr(), 2 * I, H,
-                      self.gather, T, E, k, self.tb, self.tables, stream)
-        c.moe_silu_mul_quant(self.gu.data_ptr(), self.q2.data_ptr(), self.s2.data_ptr(), I, self.rows_cap, self.tables, stream)
-        c.moe_grouped(self.q2.data_ptr(), self.s2.data_ptr(), self.xptr_dn.data_ptr(), self.y.data_ptr(), H, I, False,
-                      T, E, k, self.tb, self.tables, stream)
+        if self.fused_back:
+            c.moe_gate_up_act(self.q1.data_ptr(), self.s1.data_ptr(), self.xptr_gu.data_ptr(), self.p.data_ptr(), I, H,
+                              T, E, k, self.tb, self.tables, stream)
+            c.moe_down_rows(self.p.data_ptr(), self.xptr_dn.data_ptr(), self.y.data_ptr(), H, I, T, E, k, self.tb,
+                            self.tables, stream)
+        else:
+            c.moe_grouped(self.q1.data_ptr(), self.s1.data_ptr(), self.xptr_gu.data_ptr(), self.gu.data_ptr(), 2 * I, H,
+                          self.gather, T, E, k, self.tb, self.tables, stream)
+            c.moe_silu_mul_quant(self.gu.data_ptr(), self.q2.data_ptr(), self.s2.data_ptr(), I, self.rows_cap, self.tables, stream)
+            c.moe_grouped(self.q2.data_ptr(), self.s2.data_ptr(), self.xptr_dn.data_ptr(), self.y.data_ptr(), H, I, False,
+                          T, E, k, self.tb, self.tables, stream)
         c.moe_combine(self.y.data_ptr(), self.tables, self.out.data_ptr(), T, k, H, stream)
         return self.out

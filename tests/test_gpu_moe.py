@@ -24,16 +24,15 @@ def test_device_silu_equals_host_formula_on_all_65536_inputs(ctx):
     assert bad.size == 0, [(hex(i), hex(got[i]), hex(want[i])) for i in bad[:8]]
 
 
-def run_layer(ctx, case, tile_blocks=None):
+def run_layer(ctx, case, tile_blocks=None, fused_back=None):
     T, E, k, H, I = case["T"], case["E"], case["topk"], case["H"], case["I"]
-    layer = MoeLayerIU8(ctx, T, E, k, H, I, tile_blocks=tile_blocks)
+    layer = MoeLayerIU8(ctx, T, E, k, H, I, tile_blocks=tile_blocks, fused_back=fused_back)
     wgu = torch.from_numpy(np.stack([iu8.repack_w4(case["Wgu"][e]) for e in range(E)])).cuda()
     wdn = torch.from_numpy(np.stack([iu8.repack_w4(case["Wdn"][e]) for e in range(E)])).cuda()
     layer.set_weights(wgu, torch.from_numpy(case["wsgu"]).cuda(), wdn, torch.from_numpy(case["wsdn"]).cuda())
     # poison what the kernels must overwrite
-    layer.gu.fill_(0x7FC0)
-    layer.y.fill_(0x7FC0)
-    layer.out.fill_(0x7FC0)
+    for t in (layer.gu, layer.y, layer.out) + ((layer.p,) if layer.fused_back else ()):
+        t.fill_(0x7FC0)
     x, lg = dev_bf16_bits(case["X"]), dev_bf16_bits(case["logits"])
     layer.forward(x, lg)
     layer.forward(x, lg)            # twice: the arrival counter must have been left at zero
@@ -60,7 +59,9 @@ def check_layer(layer, case, taps=True):
     r = ref.moe_layer(case["X"], w, lay, case["Wgu"], case["wsgu"], case["Wdn"], case["wsdn"], I, threads=8, taps=taps)
     live = lay["row_tok"] >= 0
     rows = lay["rows"]
-    if taps:
+    if taps and layer.fused_back:   # the activation sits in gate+up's epilogue: p is the tap
+        np.testing.assert_array_equal(host_u16(layer.p)[:rows][live], ref.silu_mul_quant(r["gu"][live])[2])
+    elif taps:
         np.testing.assert_array_equal(host_u16(layer.gu)[:rows][live], r["gu"][live])
         q2 = iu8.unpack_a(layer.q2.cpu().numpy(), rows, I)
         np.testing.assert_array_equal(q2[live], r["q2"][live])
@@ -75,6 +76,32 @@ def test_moe_layer_small_experts(ctx, T, tb):
     case = synth.moe_case(T=T, E=128, topk=8, H=512, I=256, seed=T, experts=8)
     layer = run_layer(ctx, case, tile_blocks=tb)
     check_layer(layer, case)
+
+
+@pytest.mark.parametrize("T,H,I", [(1, 512, 256), (16, 4096, 1536), (37, 512, 1536), (100, 640, 384), (112, 1024, 256), (300, 512, 256)])
+def test_moe_back_half_in_two_launches(ctx, T, H, I):
+    """Few tokens (16-row tiles): gate+up with SiLU * up in its epilogue, then down with p's per-token
+    quantisation in front of its K loop. Same bytes as the three launches (grouped gate+up, SiLU * up
+    requant, grouped down) and as the oracle; staged and row-streaming gate+up forms (by routes an
+    expert), tiles of 1 to 16 rows, the widest intermediate the form holds. Other tile sizes are refused."""
+    say(f"moe back half in two launches T={T} H={H} I={I}")
+    case = synth.moe_case(T=T, E=128, topk=8, H=H, I=I, seed=T + I, experts=8)
+    fused = run_layer(ctx, case, tile_blocks=1, fused_back=True)
+    three = run_layer(ctx, case, tile_blocks=1, fused_back=False)
+    assert fused.fused_back and not three.fused_back and iu8.moe_back_holds(1, I)
+    rows = int(fused.buf["meta"][1].item())
+    live = fused.buf["row_tok"][:rows] >= 0
+    assert torch.equal(fused.y[:rows][live], three.y[:rows][live])
+    assert torch.equal(fused.out, three.out)
+    check_layer(fused, case)
+    assert not iu8.moe_back_holds(8, I) and not iu8.moe_back_holds(1, 1664) and not iu8.moe_back_holds(1, 200)
+    with pytest.raises(iu8.IU8Error) as e:
+        ctx.moe_gate_up_act(fused.q1.data_ptr(), fused.s1.data_ptr(), fused.xptr_gu.data_ptr(), fused.p.data_ptr(), I, H,
+                            T, 128, 8, 8, fused.tables)
+    assert e.value.code == iu8.E_RULE
+    with pytest.raises(iu8.IU8Error) as e:
+        ctx.moe_down_rows(fused.p.data_ptr(), fused.xptr_dn.data_ptr(), fused.y.data_ptr(), H, 1664, T, 128, 8, 1, fused.tables)
+    assert e.value.code == iu8.E_RULE
 
 
 @pytest.mark.parametrize("T,tb", [(1, None), (16, None), (37, None), (100, 8), (300, None), (300, 1), (520, 16)])
@@ -126,7 +153,10 @@ def test_moe_layer_with_a_shared_expert(ctx, T, tb):
     gu_s = ref.linear(case["X"], Wgu_s, wsgu_s, False, threads=8)["C"]
     _, _, p_s = ref.silu_mul_quant(gu_s)
     y_s = ref.linear(p_s, Wdn_s, wsdn_s, False, threads=8)["C"]
-    np.testing.assert_array_equal(host_u16(layer.gu)[rows:rows + T], gu_s)
+    if layer.fused_back:
+        np.testing.assert_array_equal(host_u16(layer.p)[rows:rows + T], p_s)
+    else:
+        np.testing.assert_array_equal(host_u16(layer.gu)[rows:rows + T], gu_s)
     np.testing.assert_array_equal(host_u16(layer.y)[rows:rows + T], y_s)
     Y = np.concatenate([r["Y"], y_s])
     want = ref.combine_shared(Y, w, lay["route_pos"], sgate, rows, H)
