@@ -51,6 +51,14 @@ static __device__ __forceinline__ unsigned iu8_bf16_bits(float x) {
   return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
 }
 static __device__ __forceinline__ float iu8_bf16_f32(unsigned short b) { return __uint_as_float((unsigned)b << 16); }
+typedef float iu8_v2f __attribute__((ext_vector_type(2)));
+typedef __bf16 iu8_v2bf __attribute__((ext_vector_type(2)));
+
+// two f32 -> packed bf16, round to nearest even (v_cvt_pk_bf16_f32); lo in bits 0..15
+static __device__ __forceinline__ unsigned iu8_bf16_pack(float lo, float hi) {
+  const iu8_v2bf r = __builtin_convertvector(iu8_v2f{lo, hi}, iu8_v2bf);
+  return *(const unsigned *)&r;
+}
 // bf16(silu(x)) as the producer kernels compute it (macaq_i8q: i8q_silu_bf16; the law
 // crates/saber-kernels/hip/mxfp4_hadi8.hip:118-146): x / (1 + expf(-x)), IEEE divide, one bf16 rounding.
 static __device__ __forceinline__ float iu8_silu_bf16(float x) {

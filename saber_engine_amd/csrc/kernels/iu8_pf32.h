@@ -32,14 +32,6 @@
 #include "iu8_gemm.h"
 
 typedef int iu8_v16i __attribute__((ext_vector_type(16)));
-typedef float iu8_v2f __attribute__((ext_vector_type(2)));
-typedef __bf16 iu8_v2bf __attribute__((ext_vector_type(2)));
-
-// two f32 -> packed bf16, round to nearest even (v_cvt_pk_bf16_f32); lo in bits 0..15
-static __device__ __forceinline__ unsigned iu8_bf16_pack(float lo, float hi) {
-  const iu8_v2bf r = __builtin_convertvector(iu8_v2f{lo, hi}, iu8_v2bf);
-  return *(const unsigned *)&r;
-}
 
 // One tile of work: rows [mbase, mbase + BM) of the row map R against the 16-row weight tiles from
 // nt0 of W (with row scales ws).

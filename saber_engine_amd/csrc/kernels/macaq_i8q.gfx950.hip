@@ -322,9 +322,11 @@ extern "C" __global__ __launch_bounds__(1024) void macaq_i8_silu_mul_quant_lut_w
       vu.u[0] = *(const iu8_v4u *)(gr + n + g * 16);
       vu.u[1] = *(const iu8_v4u *)(gr + n + g * 16 + 8);
 #pragma unroll
-      for (int j = 0; j < 16; ++j) {
-        const float t = iu8_bf16_f32(s_lut[vg.h[j]]);
-        v[i][j] = iu8_bf16_f32((unsigned short)iu8_bf16_bits(t * iu8_bf16_f32(vu.h[j])));
+      for (int j = 0; j < 16; j += 2) {  // two products a v_cvt_pk_bf16_f32
+        const float t0 = iu8_bf16_f32(s_lut[vg.h[j]]), t1 = iu8_bf16_f32(s_lut[vg.h[j + 1]]);
+        const unsigned p2 = iu8_bf16_pack(t0 * iu8_bf16_f32(vu.h[j]), t1 * iu8_bf16_f32(vu.h[j + 1]));
+        v[i][j] = __uint_as_float(p2 << 16);
+        v[i][j + 1] = __uint_as_float(p2 & 0xFFFF0000u);
       }
     }
     i8q_tail_w64(v, G, q, scale, row, n);
