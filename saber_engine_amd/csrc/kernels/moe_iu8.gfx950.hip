@@ -754,11 +754,16 @@ extern "C" __global__ __launch_bounds__(256) void moe_iu8_combine_bf16(
     float acc[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) acc[j] = 0.f;
+    // the routes' rows are requested together (a route that is not local, p < 0, reads row 0 and is not added):
+    // one latency a group instead of eight in a row; the adds keep the top-k order
+    iu8_v4u rows[MOE_TOPK];
+#pragma unroll
+    for (int k = 0; k < MOE_TOPK; ++k) rows[k] = ((const iu8_v4u *)(y + (size_t)max(s_pos[k], 0) * h))[g];
+#pragma unroll
     for (int k = 0; k < MOE_TOPK; ++k) {
-      const int p = s_pos[k];
-      if (p < 0) continue;
+      if (s_pos[k] < 0) continue;
       const float w = s_w[k];
-      const iu8_v4u v = ((const iu8_v4u *)(y + (size_t)p * h))[g];
+      const iu8_v4u v = rows[k];
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         acc[2 * q] = acc[2 * q] + w * __uint_as_float(v[q] << 16);
