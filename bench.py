@@ -632,7 +632,7 @@ def main():
             live = int((layer.buf["expert_cnt"] > 0).sum().item())
             wbytes = live * (2 * I * H // 2 + H * I // 2 + 4 * (2 * I + H))
             ops = 2.0 * T * topk * (2 * I * H + H * I)
-            moe["t%d" % T] = dict(layer_us=round(us, 1), launches=4 if layer.fused_back else 5, tile_rows=16 * layer.tb, experts_touched=live,
+            moe["t%d" % T] = dict(layer_us=round(us, 1), launches=(4 if layer.fused_back else 5) + (1 if T > 128 and layer.tb != 1 else 0), tile_rows=16 * layer.tb, experts_touched=live,
                                   weight_gbps=round(wbytes / us / 1e3, 1), tops=round(ops / us / 1e6, 1),
                                   bound="hbm" if T == 16 else "mfma",
                                   frac=round((wbytes / us / 1e3) / HBM_PEAK_GBPS if T == 16 else (ops / us / 1e6) / INT8_PEAK_TOPS, 4))

@@ -420,7 +420,9 @@ typedef struct {
                              * sigmoid(sgate[t]) * Y[shared row of t] */
 } saber_iu8_moe_tables;
 
-/* Router + expert-major sort + tile table, one launch. logits bf16 [T, experts]. */
+/* Router + expert-major sort + tile table (crates/saber-kernels/hip/moe_route.hip:108-284). logits bf16
+ * [T, experts]. One launch up to 128 tokens (one routing workgroup); above, two: routing with the
+ * workgroups' counts and ranks, then the layout with every workgroup placing its own routes. */
 int saber_iu8_moe_route(saber_iu8_ctx *ctx, const void *logits_bf16, uint32_t tokens, uint32_t experts, uint32_t topk,
                         uint32_t tile_blocks, const saber_iu8_moe_tables *t, void *stream);
 

@@ -698,23 +698,46 @@ static int raw_desc(const char *kernel, uint32_t gx, uint32_t gy, uint32_t block
   return saber_iu8_describe_raw(kernel, "moe_iu8", grid, block, d);
 }
 
+// The router's launches. One routing workgroup (up to 128 tokens) lays out its tables itself. With more, the routing
+// launch stops behind the workgroups' counts and ranks and a second launch of as many workgroups lays out the tables,
+// every workgroup placing its own routes (moe_iu8_route_place_e128): the one-launch form's last arriver does that
+// alone (4,096 tokens: 22 of its 38 us). `x` given: the tokens' quantisation rides in the routing launch.
+static int moe_route_launches(saber_iu8_ctx *ctx, const void *logits, const void *x, void *q, float *scale, uint32_t tokens,
+                              uint32_t experts, uint32_t k, uint32_t tile_blocks, const saber_iu8_moe_tables *t, void *stream) {
+  const uint32_t nblk = (tokens + 127) / 128;
+  const bool two = nblk > 1;
+  // a row on 256, 512 or 1,024 threads by its length: 4, 2 or 1 rows a quantising workgroup (the kernel's own rule)
+  const uint32_t groups = k / 16, rows_wg = groups <= 256 ? 4 : groups <= 512 ? 2 : 1;
+  const bool rm = tile_blocks != 1;
+  const std::string name = !x ? (two ? "moe_iu8_route_part_topk8_sort_e128" : "moe_iu8_route_topk8_sort_e128")
+                              : std::string("moe_iu8_routeq_") + (rm ? "rm_" : "") + (two && rm ? "part_" : "") + "topk8_sort_e128";
+  const bool part = name.find("_part_") != std::string::npos;
+  auto launch = [&](const std::string &kernel, uint32_t gx, bool with_x) {
+    saber_iu8_desc d;
+    if (int rc = raw_desc(kernel.c_str(), gx, 1, 1024, &d)) return rc;
+    set_i32(&d, "t", tokens);
+    set_i32(&d, "e_lo", 0);
+    set_i32(&d, "e_loc", experts);
+    set_i32(&d, "tile_blocks", tile_blocks);
+    set_i32(&d, "with_shared", t->sgate ? 1 : 0);
+    if (with_x) set_i32(&d, "k", k);
+    const saber_iu8_binding b[] = {{"logits", (void *)logits},      {"topk_ids", t->topk_ids},   {"topk_w", t->topk_w},
+                                   {"route_pos", t->route_pos},     {"row_tok", t->row_tok},     {"row_route", t->row_route},
+                                   {"tile_expert", t->tile_expert}, {"tile_row0", t->tile_row0}, {"tile_rows", t->tile_rows},
+                                   {"expert_cnt", t->expert_cnt},   {"meta", t->meta},           {"blk_cnt", t->blk_cnt},
+                                   {"rank", t->rank},               {"arrive", t->arrive},       {"x", (void *)x},
+                                   {"q", q},                        {"scale", scale}};
+    return saber_iu8_launch(ctx, &d, b, with_x ? 17 : 14, stream);
+  };
+  if (int rc = launch(name, nblk + (x ? (tokens + rows_wg - 1) / rows_wg : 0), x != nullptr)) return rc;
+  return part ? launch("moe_iu8_route_place_e128", nblk, false) : 0;
+}
+
 int saber_iu8_moe_route(saber_iu8_ctx *ctx, const void *logits, uint32_t tokens, uint32_t experts, uint32_t topk,
                         uint32_t tile_blocks, const saber_iu8_moe_tables *t, void *stream) {
   if (int rc = moe_check("moe_route", tokens, experts, topk, t)) return rc;
   if (tile_blocks == 0) return fail(SABER_IU8_E_RULE, "moe_route: tile_blocks 0");
-  saber_iu8_desc d;
-  if (int rc = raw_desc("moe_iu8_route_topk8_sort_e128", (tokens + 127) / 128, 1, 1024, &d)) return rc;
-  set_i32(&d, "t", tokens);
-  set_i32(&d, "e_lo", 0);
-  set_i32(&d, "e_loc", experts);
-  set_i32(&d, "tile_blocks", tile_blocks);
-  set_i32(&d, "with_shared", t->sgate ? 1 : 0);
-  const saber_iu8_binding b[] = {{"logits", (void *)logits},      {"topk_ids", t->topk_ids},   {"topk_w", t->topk_w},
-                                 {"route_pos", t->route_pos},     {"row_tok", t->row_tok},     {"row_route", t->row_route},
-                                 {"tile_expert", t->tile_expert}, {"tile_row0", t->tile_row0}, {"tile_rows", t->tile_rows},
-                                 {"expert_cnt", t->expert_cnt},   {"meta", t->meta},           {"blk_cnt", t->blk_cnt},
-                                 {"rank", t->rank},               {"arrive", t->arrive}};
-  return saber_iu8_launch(ctx, &d, b, sizeof b / sizeof b[0], stream);
+  return moe_route_launches(ctx, logits, nullptr, nullptr, nullptr, tokens, experts, 0, tile_blocks, t, stream);
 }
 
 int saber_iu8_moe_route_quant(saber_iu8_ctx *ctx, const void *logits, const void *x, void *q, float *scale, uint32_t tokens,
@@ -722,27 +745,9 @@ int saber_iu8_moe_route_quant(saber_iu8_ctx *ctx, const void *logits, const void
                               const saber_iu8_moe_tables *t, void *stream) {
   if (int rc = moe_check("moe_route_quant", tokens, experts, topk, t)) return rc;
   if (tile_blocks == 0) return fail(SABER_IU8_E_RULE, "moe_route_quant: tile_blocks 0");
-  if (k == 0 || k % 128 != 0 || k > 16384)
+  if (!x || k == 0 || k % 128 != 0 || k > 16384)
     return fail(SABER_IU8_E_RULE, fmt("moe_route_quant: K=%u must be a multiple of 128 (the slab) up to 16384 (a 16-element group a thread)", k));
-  // a row on 256, 512 or 1,024 threads by its length: 4, 2 or 1 rows a quantising workgroup (the kernel's own rule)
-  const uint32_t groups = k / 16, rows_wg = groups <= 256 ? 4 : groups <= 512 ? 2 : 1;
-  saber_iu8_desc d;
-  if (int rc = raw_desc(tile_blocks == 1 ? "moe_iu8_routeq_topk8_sort_e128" : "moe_iu8_routeq_rm_topk8_sort_e128",
-                        (tokens + 127) / 128 + (tokens + rows_wg - 1) / rows_wg, 1, 1024, &d))
-    return rc;
-  set_i32(&d, "t", tokens);
-  set_i32(&d, "e_lo", 0);
-  set_i32(&d, "e_loc", experts);
-  set_i32(&d, "tile_blocks", tile_blocks);
-  set_i32(&d, "with_shared", t->sgate ? 1 : 0);
-  set_i32(&d, "k", k);
-  const saber_iu8_binding b[] = {{"logits", (void *)logits},      {"topk_ids", t->topk_ids},   {"topk_w", t->topk_w},
-                                 {"route_pos", t->route_pos},     {"row_tok", t->row_tok},     {"row_route", t->row_route},
-                                 {"tile_expert", t->tile_expert}, {"tile_row0", t->tile_row0}, {"tile_rows", t->tile_rows},
-                                 {"expert_cnt", t->expert_cnt},   {"meta", t->meta},           {"blk_cnt", t->blk_cnt},
-                                 {"rank", t->rank},               {"arrive", t->arrive},       {"x", (void *)x},
-                                 {"q", q},                        {"scale", scale}};
-  return saber_iu8_launch(ctx, &d, b, sizeof b / sizeof b[0], stream);
+  return moe_route_launches(ctx, logits, x, q, scale, tokens, experts, k, tile_blocks, t, stream);
 }
 
 int saber_iu8_moe_grouped(saber_iu8_ctx *ctx, const void *a, const float *as, const void *xptr, void *c, uint32_t n,

@@ -87,7 +87,10 @@ static __device__ __forceinline__ int moe_exscan(int v, int *s_wave, int *total)
   return base + x - v;
 }
 
-// The router's workgroup `blk` of `nblk` (128 tokens each).
+// The router's workgroup `blk` of `nblk` (128 tokens each). PART: the workgroup stops behind its own
+// counts and ranks (phases 1 and 2); the tables are then laid out by moe_iu8_route_place_e128, a launch
+// of its own in which every workgroup places its own routes.
+template <bool PART = false>
 static __device__ __forceinline__ void moe_route_body(
     const unsigned short *__restrict__ logits, int T, int e_lo, int e_loc, int tile_blocks, int with_shared,
     int *__restrict__ topk_ids, float *__restrict__ topk_w, int *__restrict__ route_pos, int *__restrict__ row_tok,
@@ -222,6 +225,7 @@ static __device__ __forceinline__ void moe_route_body(
   const bool solo = nblk == 1;
   if (!solo) {
     for (int e = tid; e < e_loc; e += MOE_THREADS) blk_cnt[(size_t)blk * e_loc + e] = s_cnt[e];
+    if constexpr (PART) return;
     __syncthreads();
     if (tid == 0) {
       __threadfence();
@@ -380,6 +384,132 @@ extern "C" __global__ __launch_bounds__(MOE_THREADS) void moe_iu8_route_topk8_so
                  tile_expert, tile_row0, tile_rows, expert_cnt, meta, blk_cnt, rank, arrive, gridDim.x, blockIdx.x);
 }
 
+extern "C" __global__ __launch_bounds__(MOE_THREADS) void moe_iu8_route_part_topk8_sort_e128(
+    const unsigned short *__restrict__ logits, int T, int e_lo, int e_loc, int tile_blocks, int with_shared,
+    int *__restrict__ topk_ids, float *__restrict__ topk_w, int *__restrict__ route_pos, int *__restrict__ row_tok,
+    int *__restrict__ row_route, int *__restrict__ tile_expert, int *__restrict__ tile_row0,
+    int *__restrict__ tile_rows, int *__restrict__ expert_cnt, int *__restrict__ meta, int *__restrict__ blk_cnt,
+    int *__restrict__ rank, int *__restrict__ arrive) {
+  moe_route_body<true>(logits, T, e_lo, e_loc, tile_blocks, with_shared, topk_ids, topk_w, route_pos, row_tok, row_route,
+                       tile_expert, tile_row0, tile_rows, expert_cnt, meta, blk_cnt, rank, arrive, gridDim.x, blockIdx.x);
+}
+
+// The tables behind moe_iu8_route*_part_*: workgroup b (of ceil(T / 128), the part launch's routing
+// workgroups) sums the workgroups' per-expert counts -- every workgroup the totals, and the counts of
+// the workgroups in front of it as its own base -- lays out the experts' offsets like the one-launch
+// router, and places its own 1,024 routes; workgroup 0 also writes the tile table, the counts, meta,
+// the pad rows and a shared expert's rows. No workgroup waits for another: with more than one routing
+// workgroup the one-launch form's last arriver lays out and places everything alone (4,096 tokens:
+// 22 of its 38 us). Same tables: a route's row is the same sum. Kernarg list of the router (logits,
+// topk_w and arrive are not touched). grid [ceil(T / 128), 1, 1].
+extern "C" __global__ __launch_bounds__(MOE_THREADS) void moe_iu8_route_place_e128(
+    const unsigned short *__restrict__ logits, int T, int e_lo, int e_loc, int tile_blocks, int with_shared,
+    int *__restrict__ topk_ids, float *__restrict__ topk_w, int *__restrict__ route_pos, int *__restrict__ row_tok,
+    int *__restrict__ row_route, int *__restrict__ tile_expert, int *__restrict__ tile_row0,
+    int *__restrict__ tile_rows, int *__restrict__ expert_cnt, int *__restrict__ meta, int *__restrict__ blk_cnt,
+    int *__restrict__ rank, int *__restrict__ arrive) {
+  constexpr int PARTS = MOE_THREADS / MOE_E;
+  __shared__ int s_all[PARTS][MOE_E], s_mine[PARTS][MOE_E];
+  __shared__ int s_cnt[MOE_E], s_base[MOE_E], s_off[MOE_E], s_toff[MOE_E];
+  __shared__ int s_wave[MOE_THREADS / 64];
+  const int tid = threadIdx.x, nblk = gridDim.x, blk = blockIdx.x;
+  {
+    const int e = tid % MOE_E, part = tid / MOE_E;
+    const int chunk = (nblk + PARTS - 1) / PARTS, b_lo = min(part * chunk, nblk), b_hi = min(b_lo + chunk, nblk);
+    int all = 0, mine = 0;
+    if (e < e_loc)
+      for (int b0 = b_lo; b0 < b_hi; b0 += 8) {
+        int c[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) c[u] = b0 + u < b_hi ? blk_cnt[(size_t)(b0 + u) * e_loc + e] : 0;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          all += c[u];
+          mine += b0 + u < blk ? c[u] : 0;
+        }
+      }
+    s_all[part][e] = all;
+    s_mine[part][e] = mine;
+    __syncthreads();
+    if (part == 0) {
+      int a = 0, m = 0;
+#pragma unroll
+      for (int q = 0; q < PARTS; ++q) {
+        a += s_all[q][e];
+        m += s_mine[q][e];
+      }
+      s_cnt[e] = e < e_loc ? a : 0;
+      s_base[e] = m;
+    }
+    __syncthreads();
+  }
+  const int G = tile_blocks, TR = 16 * tile_blocks;
+  int my_rows = 0, my_tiles = 0, my_touched = 0, my_routes = 0;
+  if (tid < e_loc) {
+    const int c = s_cnt[tid], nb = (c + 15) / 16;
+    my_rows = nb * 16;
+    my_tiles = (nb + G - 1) / G;
+    my_touched = c > 0;
+    my_routes = c;
+  }
+  int rows_total, tiles_total, touched_total, routes_total;
+  const int rbase = moe_exscan(my_rows, s_wave, &rows_total);
+  const int tbase = moe_exscan(my_tiles, s_wave, &tiles_total);
+  moe_exscan(my_touched, s_wave, &touched_total);
+  moe_exscan(my_routes, s_wave, &routes_total);
+  if (tid < e_loc) {
+    s_off[tid] = rbase;
+    s_toff[tid] = tbase;
+  }
+  __syncthreads();
+  if (blk == 0) {
+    const int sh_row0 = rows_total;
+    const int sh_blocks = with_shared ? (T + 15) / 16 : 0;
+    const int sh_tiles = (sh_blocks + G - 1) / G;
+    if (tid == 0) {
+      meta[0] = tiles_total + sh_tiles;
+      meta[1] = rows_total + sh_blocks * 16;
+      meta[2] = with_shared ? sh_row0 : -1;
+      meta[3] = routes_total;
+      meta[4] = touched_total;
+      meta[5] = rows_total;
+    }
+    for (int e = tid; e < e_loc; e += MOE_THREADS) {
+      const int c = s_cnt[e], nb = (c + 15) / 16, nt = (nb + G - 1) / G;
+      expert_cnt[e] = c;
+      for (int j = 0; j < nt; ++j) {
+        tile_expert[s_toff[e] + j] = e;
+        tile_row0[s_toff[e] + j] = s_off[e] + j * TR;
+        tile_rows[s_toff[e] + j] = min(TR, c - j * TR);
+      }
+      for (int i = c; i < nb * 16; ++i) {  // the pad rows behind the expert's routes
+        row_tok[s_off[e] + i] = -1;
+        row_route[s_off[e] + i] = -1;
+      }
+    }
+    for (int j = tid; j < sh_tiles; j += MOE_THREADS) {
+      tile_expert[tiles_total + j] = e_loc;
+      tile_row0[tiles_total + j] = sh_row0 + j * TR;
+      tile_rows[tiles_total + j] = min(TR, T - j * TR);
+    }
+    for (int r = tid; r < sh_blocks * 16; r += MOE_THREADS) {
+      row_tok[sh_row0 + r] = r < T ? r : -1;
+      row_route[sh_row0 + r] = -1;
+    }
+  }
+  const int r = blk * (MOE_TPB * MOE_TOPK) + tid;  // this workgroup's routes: a thread a route
+  if (r < T * MOE_TOPK) {
+    const int le = topk_ids[r] - e_lo;
+    const bool local = le >= 0 && le < e_loc;
+    const int p = local ? s_off[le] + s_base[le] + rank[r] : -1;
+    route_pos[r] = p;
+    if (local) {
+      row_route[p] = r;
+      row_tok[p] = r / MOE_TOPK;
+    }
+  }
+}
+
 // The router and the tokens' quantisation in one launch: the two do not depend on each other, so the
 // first ceil(T / 128) workgroups route and the ones behind them quantise the tokens (x bf16 [T, k] ->
 // codes + scale[t]; macaq_i8.h:10-13, one 16-element group a thread, k <= 16,384), a row on 256, 512
@@ -388,7 +518,7 @@ extern "C" __global__ __launch_bounds__(MOE_THREADS) void moe_iu8_route_topk8_so
 // quantisation instead of in front of it. Codes in the A fragment order (RM false, for the streaming
 // cell) or row-major (RM true, for the MFMA cells' gather). grid [ceil(T/128) + ceil(T / rows a
 // workgroup), 1, 1].
-template <bool RM>
+template <bool RM, bool PART = false>
 static __device__ __forceinline__ void moe_routeq_body(
     const unsigned short *__restrict__ logits, int T, int e_lo, int e_loc, int tile_blocks, int with_shared,
     int *__restrict__ topk_ids, float *__restrict__ topk_w, int *__restrict__ route_pos, int *__restrict__ row_tok,
@@ -399,8 +529,8 @@ static __device__ __forceinline__ void moe_routeq_body(
 #pragma clang fp contract(off)
   const int nblk = (T + MOE_TPB - 1) / MOE_TPB;
   if ((int)blockIdx.x < nblk) {
-    moe_route_body(logits, T, e_lo, e_loc, tile_blocks, with_shared, topk_ids, topk_w, route_pos, row_tok, row_route,
-                   tile_expert, tile_row0, tile_rows, expert_cnt, meta, blk_cnt, rank, arrive, nblk, blockIdx.x);
+    moe_route_body<PART>(logits, T, e_lo, e_loc, tile_blocks, with_shared, topk_ids, topk_w, route_pos, row_tok, row_route,
+                         tile_expert, tile_row0, tile_rows, expert_cnt, meta, blk_cnt, rank, arrive, nblk, blockIdx.x);
     return;
   }
   __shared__ float s_max[MOE_THREADS / 64];
@@ -446,7 +576,7 @@ static __device__ __forceinline__ void moe_routeq_body(
     }
   }
 }
-#define MOE_ROUTEQ(name, RM)                                                                                          \
+#define MOE_ROUTEQ(name, RM, PART)                                                                                          \
   extern "C" __global__ __launch_bounds__(MOE_THREADS) void name(                                                      \
       const unsigned short *__restrict__ logits, int T, int e_lo, int e_loc, int tile_blocks, int with_shared,          \
       int *__restrict__ topk_ids, float *__restrict__ topk_w, int *__restrict__ route_pos, int *__restrict__ row_tok,   \
@@ -454,12 +584,13 @@ static __device__ __forceinline__ void moe_routeq_body(
       int *__restrict__ tile_rows, int *__restrict__ expert_cnt, int *__restrict__ meta, int *__restrict__ blk_cnt,     \
       int *__restrict__ rank, int *__restrict__ arrive, const unsigned short *__restrict__ x,                           \
       unsigned char *__restrict__ q, float *__restrict__ scale, int k) {                                                \
-    moe_routeq_body<RM>(logits, T, e_lo, e_loc, tile_blocks, with_shared, topk_ids, topk_w, route_pos, row_tok,         \
+    moe_routeq_body<RM, PART>(logits, T, e_lo, e_loc, tile_blocks, with_shared, topk_ids, topk_w, route_pos, row_tok,         \
                         row_route, tile_expert, tile_row0, tile_rows, expert_cnt, meta, blk_cnt, rank, arrive, x, q,    \
                         scale, k);                                                                                      \
   }
-MOE_ROUTEQ(moe_iu8_routeq_topk8_sort_e128, false)
-MOE_ROUTEQ(moe_iu8_routeq_rm_topk8_sort_e128, true)
+MOE_ROUTEQ(moe_iu8_routeq_topk8_sort_e128, false, false)
+MOE_ROUTEQ(moe_iu8_routeq_rm_topk8_sort_e128, true, false)
+MOE_ROUTEQ(moe_iu8_routeq_rm_part_topk8_sort_e128, true, true)
 #undef MOE_ROUTEQ
 
 // ---------------------------------------------------------------------------- grouped GEMMs
