@@ -78,6 +78,34 @@ def test_moe_layer_small_experts(ctx, T, tb):
     check_layer(layer, case)
 
 
+@pytest.mark.parametrize("I", [256, 1536, 2048, 2560, 4096])
+def test_silu_mul_requant_table_form(ctx, I):
+    """SiLU * up + requant over many expert-major rows, the form that reads the bf16 silu from the table in
+    LDS: rows of 256 to 4,096 elements (one to four 16-element groups a lane), pad rows skipped, against
+    the oracle's row routine (codes, scales)."""
+    T, E, k = 520, 128, 8
+    say(f"silu * up requant, table form: I={I}")
+    rng = np.random.default_rng(I)
+    layer = MoeLayerIU8(ctx, T, E, k, 128, I, tile_blocks=8)
+    assert layer.rows_cap >= 4096
+    lg = dev_bf16_bits(synth.f32_to_bf16_bits(rng.standard_normal(size=(T, E), dtype=np.float32)))
+    ctx.moe_route(lg.data_ptr(), T, E, k, layer.tb, layer.tables)
+    gu = synth.f32_to_bf16_bits((rng.standard_normal(size=(layer.rows_cap, 2 * I)) * rng.choice([0.1, 1.0, 6.0], size=(layer.rows_cap, 1))).astype(np.float32))
+    layer.gu.copy_(dev_bf16_bits(gu))
+    layer.q2.fill_(0x55)
+    layer.s2.fill_(-1.0)
+    ctx.moe_silu_mul_quant(layer.gu.data_ptr(), layer.q2.data_ptr(), layer.s2.data_ptr(), I, layer.rows_cap, layer.tables)
+    torch.cuda.synchronize()
+    rows = int(layer.buf["meta"][1].item())
+    live = layer.buf["row_tok"][:rows].cpu().numpy() >= 0
+    assert live.sum() == T * k and (~live).sum() > 0
+    want_q, want_s, _ = ref.silu_mul_quant(gu[:rows][live])
+    np.testing.assert_array_equal(iu8.unpack_a(layer.q2.cpu().numpy(), rows, I)[live], want_q)
+    s2 = layer.s2.cpu().numpy()
+    np.testing.assert_array_equal(s2[:rows][live].view(np.uint32), want_s.view(np.uint32))
+    assert (s2[:rows][~live] == -1.0).all() and (s2[rows:] == -1.0).all()      # pad rows and the rows past the live ones are left alone
+
+
 @pytest.mark.parametrize("T,H,I", [(1, 512, 256), (16, 4096, 1536), (37, 512, 1536), (100, 640, 384), (112, 1024, 256), (300, 512, 256)])
 def test_moe_back_half_in_two_launches(ctx, T, H, I):
     """Few tokens (16-row tiles): gate+up with SiLU * up in its epilogue, then down with p's per-token
