@@ -602,10 +602,12 @@ MOE_ROUTEQ(moe_iu8_routeq_rm_part_topk8_sort_e128, true, true)
       const int *__restrict__ tile_expert, const int *__restrict__ tile_row0, const int *__restrict__ tile_rows,  \
       const int *__restrict__ row_tok, const int *__restrict__ meta, const float *__restrict__ as,                \
       int *__restrict__ p, int *__restrict__ cnt, unsigned short *__restrict__ c, int n, int k, int pmax) {        \
+    /* the tile's table entries are requested beside the live count, not behind it (the tables hold gridDim.y     \
+       entries): one link less in the chain of dependent loads in front of the first weight load */               \
     const int tile = blockIdx.y;                                                                                   \
-    if (tile >= meta[0]) return;                                                                                   \
-    const int e = tile_expert[tile];                                                                               \
-    const iu8_rows R{GATHER ? row_tok : nullptr, tile_row0[tile], min(tile_rows[tile], 16)};                       \
+    const int live = meta[0], e = tile_expert[tile], row0 = tile_row0[tile], rows = tile_rows[tile];               \
+    if (tile >= live) return;                                                                                      \
+    const iu8_rows R{GATHER ? row_tok : nullptr, row0, min(rows, 16)};                                             \
     iu8_dec_body<1, false, NT, KW, WPB, D, ALDS, false, MODE>(a, (const unsigned char *)xptr[2 * e], as,           \
                                                               (const float *)xptr[2 * e + 1], p, cnt, c, R, n, k); \
   }
