@@ -474,7 +474,7 @@ int saber_iu8_moe_silu_mul_quant(saber_iu8_ctx *ctx, const void *gu_bf16, void *
  *   saber_iu8_moe_down_rows: p as written above, quantised per row in front of the K loop (K = inter);
  *     xptr the experts' down weights ([n, inter]) and scales; y bf16 [rows_cap, n]. */
 int saber_iu8_moe_back_holds(uint32_t tile_blocks, uint32_t inter);
-/* The launch law's pick: the two-launch form where it holds and an expert has at most 2.5 routes on average. */
+/* The launch law's pick: the two-launch form wherever it holds (measured faster at every token count of the 16-row regime). */
 int saber_iu8_moe_back_pays(uint32_t tokens, uint32_t topk, uint32_t experts, uint32_t tile_blocks, uint32_t inter);
 int saber_iu8_moe_gate_up_act(saber_iu8_ctx *ctx, const void *a, const float *as, const void *xptr, void *p_bf16,
                               uint32_t inter, uint32_t k, uint32_t tokens, uint32_t experts, uint32_t topk,

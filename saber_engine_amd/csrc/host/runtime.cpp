@@ -806,12 +806,12 @@ int saber_iu8_moe_back_holds(uint32_t tile_blocks, uint32_t inter) {
   return tile_blocks == 1 && inter != 0 && inter % 128 == 0 && (uint64_t)16 * inter <= 24 * 1024;
 }
 
-// ... and pays while an expert has few rows: every workgroup of a tile repeats the tile's requantisation and the
-// gate+up epilogue spends an exp and a divide a value on the few lanes that hold live rows. Measured on the 128-expert
-// top-8 layer (hidden 4096, inter 1536): 144.9 -> 139.9 us a layer at 16 tokens, 197.9 -> 193.0 at 32, even at 48,
-// 242.4 -> 247.7 at 64: up to 2.5 routes an expert.
+// ... and pays wherever it holds. Measured on the 128-expert top-8 layer (hidden 4096, inter 1536), layer in us, three
+// launches against two: 8 tokens 107.3 / 100.0, 16 tokens 145.2 / 139.4, 32 tokens 190.5 / 183.1, 64 tokens 242.0 / 226.7,
+// 112 tokens 296.5 / 271.9 (gate+up with one tile of p a wave up to 1.5 routes an expert, two above).
 int saber_iu8_moe_back_pays(uint32_t tokens, uint32_t topk, uint32_t experts, uint32_t tile_blocks, uint32_t inter) {
-  return saber_iu8_moe_back_holds(tile_blocks, inter) && experts != 0 && (uint64_t)tokens * topk * 2 <= (uint64_t)experts * 5;
+  (void)tokens, (void)topk, (void)experts;
+  return saber_iu8_moe_back_holds(tile_blocks, inter);
 }
 
 static int moe_back_launch(saber_iu8_ctx *ctx, const std::string &name, uint32_t gx, const void *a,
@@ -839,8 +839,10 @@ int saber_iu8_moe_gate_up_act(saber_iu8_ctx *ctx, const void *a, const float *as
   if (!saber_iu8_moe_back_holds(tile_blocks, inter) || k == 0 || k % 128 != 0)
     return fail(SABER_IU8_E_RULE, fmt("moe_gate_up_act: tile_blocks %u, inter %u, K=%u; the fused back half is the 16-row cell's "
                                       "(tile_blocks 1), inter a multiple of 128 up to 1536, K a multiple of 128", tile_blocks, inter, k));
-  return moe_back_launch(ctx, "moe_iu8_grouped_w4_decpa_g1", (inter + 15) / 16, a, as, xptr, p, 2 * inter, k, tokens, experts, topk,
-                         t, stream);
+  // one tile of p a wave up to 1.5 routes an expert, two above (the rows streamed beside the weights feed twice the columns)
+  const bool wide = (uint64_t)tokens * topk * 2 > (uint64_t)experts * 3;
+  return moe_back_launch(ctx, wide ? "moe_iu8_grouped_w4_decpb_g1" : "moe_iu8_grouped_w4_decpa_g1", (inter + (wide ? 31 : 15)) / (wide ? 32 : 16), a,
+                         as, xptr, p, 2 * inter, k, tokens, experts, topk, t, stream);
 }
 
 int saber_iu8_moe_down_rows(saber_iu8_ctx *ctx, const void *p, const void *xptr, void *y, uint32_t n, uint32_t inter,

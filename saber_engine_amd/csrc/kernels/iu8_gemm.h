@@ -34,10 +34,10 @@ static __device__ __forceinline__ iu8_blk iu8_blk_of_grid() {
 
 // ============================================================================ decode band
 // MODE 1, the gate+up projection of an MLP with the activation in its epilogue: W holds N/2 gate rows
-// and then N/2 up rows, a wave's two tiles are the gate tile and the up tile of the same 16 columns,
+// and then N/2 up rows, a wave's NT tiles are NT/2 gate tiles and the up tiles of the same columns,
 // and C is p = bf16(bf16(silu(gate)) * up), bf16 [rows, N/2] -- what the three steps (this GEMM to
 // bf16, SiLU * up, bf16) write (crates/saber-kernels/hip/mxfp4_hadi8.hip:118-146), without the
-// [gate | up] matrix in memory. A column block is WN*16 columns of p.
+// [gate | up] matrix in memory. A column block is WN * NT/2 * 16 columns of p.
 // MODE 2, the projection behind it: A is those bf16 rows themselves ([rows, K], in place), quantised
 // here by the per-token law (crates/saber-kernels/hip/macaq_i8.h:10-13) into the staged LDS form, the
 // scales kept in LDS for the epilogue; `as` is not read. The tile's rows must fit: pow2(rows) * K <=
@@ -52,7 +52,8 @@ __device__ __forceinline__ void iu8_dec_body(const iu8_u8 *__restrict__ A, const
   static_assert(WPB % KW == 0, "k-waves divide the workgroup");
   static_assert(ALDS == 0 || TM == 1, "LDS staging of A is the M <= 16 form");
   constexpr bool PAIR = MODE == 1, AQ = MODE == 2;
-  static_assert(!PAIR || (NT == 2 && TM == 1 && !W8 && !ACC), "the paired form: a gate tile and an up tile a wave");
+  static_assert(!PAIR || (NT % 2 == 0 && TM == 1 && !W8 && !ACC), "the paired form: gate tiles and their up tiles a wave");
+  constexpr int NP = PAIR ? NT / 2 : 1;  // tiles of p a wave (paired: tiles [0, NP) are gate tiles, [NP, NT) their up tiles)
   static_assert(!AQ || (ALDS > 0 && !ACC), "rows quantised here are staged in LDS");
   constexpr int WN = WPB / KW;
   constexpr int NTHR = WPB * 64;
@@ -82,7 +83,7 @@ __device__ __forceinline__ void iu8_dec_body(const iu8_u8 *__restrict__ A, const
 #pragma unroll
   for (int j = 0; j < NT; ++j) {
     // a tile past N re-reads the last one and stores nothing; paired: tile j = 0 of the gate rows, 1 of the up rows
-    const int ntj = PAIR ? j * (ntiles >> 1) + min(B.bx * WN + wn, (ntiles >> 1) - 1) : min(nt0 + j, ntiles - 1);
+    const int ntj = PAIR ? (j / NP) * (ntiles >> 1) + min((B.bx * WN + wn) * NP + j % NP, (ntiles >> 1) - 1) : min(nt0 + j, ntiles - 1);
     wp[j] = W + ((size_t)ntj * steps + s_lo + wk) * WSTEP + lane * 16;
   }
 
@@ -325,18 +326,23 @@ __device__ __forceinline__ void iu8_dec_body(const iu8_u8 *__restrict__ A, const
   const int nq = lg * 4;
   if constexpr (PAIR) {
 #pragma clang fp contract(off)
-    const int tp = B.bx * WN + wn, half = N >> 1;  // this wave's tile of p
-    if (wk != 0 || tp >= (ntiles >> 1) || ml >= M) return;
-    const int n = tp * 16 + nq;
+    const int half = N >> 1;
+    if (wk != 0 || ml >= M) return;
     const float am = as[iu8_arow(R, ml)];
-    unsigned h[4];
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const float g = iu8_bf16_f32((unsigned short)iu8_bf16_bits(iu8_epi(acc[0][0][r], am, iu8_wsu<W8>(ws, n + r))));
-      const float u = iu8_bf16_f32((unsigned short)iu8_bf16_bits(iu8_epi(acc[0][1][r], am, iu8_wsu<W8>(ws, half + n + r))));
-      h[r] = iu8_bf16_bits(iu8_silu_bf16(g) * u);
+    for (int jj = 0; jj < NP; ++jj) {
+      const int tp = (B.bx * WN + wn) * NP + jj;  // this wave's jj-th tile of p
+      if (tp >= (ntiles >> 1)) continue;
+      const int n = tp * 16 + nq;
+      unsigned h[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float g = iu8_bf16_f32((unsigned short)iu8_bf16_bits(iu8_epi(acc[0][jj][r], am, iu8_wsu<W8>(ws, n + r))));
+        const float u = iu8_bf16_f32((unsigned short)iu8_bf16_bits(iu8_epi(acc[0][NP + jj][r], am, iu8_wsu<W8>(ws, half + n + r))));
+        h[r] = iu8_bf16_bits(iu8_silu_bf16(g) * u);
+      }
+      *(iu8_v2u *)((unsigned short *)Cv + (size_t)(R.row0 + ml) * half + n) = iu8_v2u{h[0] | (h[1] << 16), h[2] | (h[3] << 16)};
     }
-    *(iu8_v2u *)((unsigned short *)Cv + (size_t)(R.row0 + ml) * half + n) = iu8_v2u{h[0] | (h[1] << 16), h[2] | (h[3] << 16)};
     return;
   }
   if (Z == 1) {

@@ -596,8 +596,8 @@ MOE_ROUTEQ(moe_iu8_routeq_rm_part_topk8_sort_e128, true, true)
 // ---------------------------------------------------------------------------- grouped GEMMs
 // grid [ceil(N / BN), tiles_cap, 1]: blockIdx.y is a tile; a workgroup whose tile is past the live
 // count exits whole.
-#define MOE_GROUPED_DEC(name, GATHER, NT, KW, WPB, D, ALDS, MODE)                                                \
-  extern "C" __global__ __launch_bounds__(WPB * 64) __attribute__((amdgpu_waves_per_eu(8, 8))) void name(        \
+#define MOE_GROUPED_DEC(name, GATHER, NT, KW, WPB, D, ALDS, MODE, WPE)                                              \
+  extern "C" __global__ __launch_bounds__(WPB * 64) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) void name(        \
       const unsigned char *__restrict__ a, const unsigned long long *__restrict__ xptr,                           \
       const int *__restrict__ tile_expert, const int *__restrict__ tile_row0, const int *__restrict__ tile_rows,  \
       const int *__restrict__ row_tok, const int *__restrict__ meta, const float *__restrict__ as,                \
@@ -611,17 +611,17 @@ MOE_ROUTEQ(moe_iu8_routeq_rm_part_topk8_sort_e128, true, true)
     iu8_dec_body<1, false, NT, KW, WPB, D, ALDS, false, MODE>(a, (const unsigned char *)xptr[2 * e], as,           \
                                                               (const float *)xptr[2 * e + 1], p, cnt, c, R, n, k); \
   }
-MOE_GROUPED_DEC(moe_iu8_grouped_w4_dec_g1, true, 1, 4, 8, 8, 20, 0)
-MOE_GROUPED_DEC(moe_iu8_grouped_w4_dec_g0, false, 1, 4, 8, 8, 20, 0)
+MOE_GROUPED_DEC(moe_iu8_grouped_w4_dec_g1, true, 1, 4, 8, 8, 20, 0, 8)
+MOE_GROUPED_DEC(moe_iu8_grouped_w4_dec_g0, false, 1, 4, 8, 8, 20, 0, 8)
 // The same cell with the activation rows streamed from L2 beside the weights instead of staged in
 // LDS: the staged form holds pow2(rows) * K <= 20 KiB (4 rows at K = 4096) and runs a tile that
 // does not fit without its load ring; this one keeps the ring for any tile.
 // Short K (up to 16 steps): two k-waves a tile instead of four, so a workgroup covers 64 columns and a
 // wave's ring holds its whole share (an expert's down projection, K = 1536: 50 -> 45 us at 16 tokens)
-MOE_GROUPED_DEC(moe_iu8_grouped_w4_deck_g1, true, 1, 2, 8, 6, 20, 0)
-MOE_GROUPED_DEC(moe_iu8_grouped_w4_deck_g0, false, 1, 2, 8, 6, 20, 0)
-MOE_GROUPED_DEC(moe_iu8_grouped_w4_deca_g1, true, 2, 8, 8, 2, 0, 0)
-MOE_GROUPED_DEC(moe_iu8_grouped_w4_deca_g0, false, 2, 8, 8, 2, 0, 0)
+MOE_GROUPED_DEC(moe_iu8_grouped_w4_deck_g1, true, 1, 2, 8, 6, 20, 0, 8)
+MOE_GROUPED_DEC(moe_iu8_grouped_w4_deck_g0, false, 1, 2, 8, 6, 20, 0, 8)
+MOE_GROUPED_DEC(moe_iu8_grouped_w4_deca_g1, true, 2, 8, 8, 2, 0, 0, 8)
+MOE_GROUPED_DEC(moe_iu8_grouped_w4_deca_g0, false, 2, 8, 8, 2, 0, 0, 8)
 // The back half of a routed layer with few tokens as two launches instead of three: gate+up with the
 // activation in its epilogue (a wave owns the gate tile and the up tile of 16 columns and writes
 // p = bf16(bf16(silu(gate)) * up), bf16 [rows_cap, n / 2]; the reference chains the same three steps
@@ -631,9 +631,13 @@ MOE_GROUPED_DEC(moe_iu8_grouped_w4_deca_g0, false, 2, 8, 8, 2, 0, 0)
 // routines on the same values. gate+up on the row-streaming cell: the staged forms of this epilogue
 // (its exp and divide on top of the staged rows' registers) spill inside the K loop at eight waves a
 // SIMD and measured 5 to 60 % slower.
-MOE_GROUPED_DEC(moe_iu8_grouped_w4_decpa_g1, true, 2, 8, 8, 2, 0, 1)
+MOE_GROUPED_DEC(moe_iu8_grouped_w4_decpa_g1, true, 2, 8, 8, 2, 0, 1, 8)
 
-MOE_GROUPED_DEC(moe_iu8_grouped_w4_deckq_g0, false, 1, 2, 8, 6, 24, 2)
+MOE_GROUPED_DEC(moe_iu8_grouped_w4_deckq_g0, false, 1, 2, 8, 6, 24, 2, 8)
+// two tiles of p a wave (32 columns a workgroup): the rows streamed beside the weights feed twice the
+// columns, which pays from about 1.5 routes an expert (layer at 32 tokens 187 -> 183 us, at 64 246 -> 227,
+// at 112 316 -> 272; at 8 tokens 100 -> 104)
+MOE_GROUPED_DEC(moe_iu8_grouped_w4_decpb_g1, true, 4, 8, 8, 2, 0, 1, 5)
 #undef MOE_GROUPED_DEC
 
 // The MFMA-bound cells: a persistent launch of one workgroup a CU walks the work items

@@ -110,8 +110,8 @@ def test_silu_mul_requant_table_form(ctx, I):
 def test_moe_back_half_in_two_launches(ctx, T, H, I):
     """Few tokens (16-row tiles): gate+up with SiLU * up in its epilogue, then down with p's per-token
     quantisation in front of its K loop. Same bytes as the three launches (grouped gate+up, SiLU * up
-    requant, grouped down) and as the oracle; staged and row-streaming gate+up forms (by routes an
-    expert), tiles of 1 to 16 rows, the widest intermediate the form holds. Other tile sizes are refused."""
+    requant, grouped down) and as the oracle; gate+up with one and with two tiles of p a wave (by routes
+    an expert), tiles of 1 to 16 rows, the widest intermediate the form holds. Other tile sizes are refused."""
     say(f"moe back half in two launches T={T} H={H} I={I}")
     case = synth.moe_case(T=T, E=128, topk=8, H=H, I=I, seed=T + I, experts=8)
     fused = run_layer(ctx, case, tile_blocks=1, fused_back=True)

@@ -195,8 +195,8 @@ def test_band_table_is_the_launch_law():
     names = {r["name"]: r["answer"] for r in t["reference_symbol"]}
     assert len(names) == 45 and names["macaq_iu8_pf_w4_tn4_lbk64"].startswith("same name") and names["macaq_iu8f_arnq_hadi8_w4_tm1"] == "none"
     assert t["moe"]["tile_blocks_1_last_tokens"] == 112 and t["moe"]["tile_blocks_8_last_tokens"] == 2047
-    assert t["moe"]["fused_back_last_tokens"] == 40 and t["moe"]["fused_back_inter_max"] == 1536
-    assert iu8.moe_back_pays(16, 8, 128, 1, 1536) and not iu8.moe_back_pays(64, 8, 128, 1, 1536)
+    assert t["moe"]["fused_back_last_tokens"] == 112 and t["moe"]["fused_back_inter_max"] == 1536
+    assert iu8.moe_back_pays(16, 8, 128, 1, 1536) and iu8.moe_back_pays(112, 8, 128, 1, 1536)
     assert not iu8.moe_back_pays(16, 8, 128, 8, 1536) and not iu8.moe_back_holds(1, 1664)
     assert t["pair"]["second_first"] == [True] * 4
     # the fused decode linear's grid law and the chain's, as the tables state them
