@@ -269,6 +269,37 @@ def test_route_and_quant_in_one_launch(ctx, T, H):
     assert e.value.code == iu8.E_RULE
 
 
+@pytest.mark.parametrize("T,tb", [(129, 8), (700, 8), (3000, 16)])
+def test_one_launch_router_under_the_reference_name(ctx, T, tb):
+    """Above 128 tokens the C ABI routes in two launches; the one-launch kernel under the reference's name
+    (its last workgroup to arrive lays out the tables alone) stays in the plugin for a host that launches
+    that name: same tables, arrival counter left at zero, twice in a row."""
+    say(f"one-launch router by name: T={T} tile_blocks={tb}")
+    E, k = 128, 8
+    rng = np.random.default_rng(T)
+    lg = dev_bf16_bits(synth.f32_to_bf16_bits(rng.standard_normal(size=(T, E), dtype=np.float32)))
+    two, one = MoeLayerIU8(ctx, T, E, k, 128, 128, tile_blocks=tb), MoeLayerIU8(ctx, T, E, k, 128, 128, tile_blocks=tb)
+    ctx.moe_route(lg.data_ptr(), T, E, k, tb, two.tables)
+    d = iu8.describe_raw("moe_iu8_route_topk8_sort_e128", ((T + 127) // 128, 1, 1), 1024, plugin="moe_iu8",
+                         t=T, e_lo=0, e_loc=E, tile_blocks=tb, with_shared=0)
+    bufs = dict(logits=lg.data_ptr(), **{n_: one.buf[n_].data_ptr() for n_ in (
+        "topk_ids", "topk_w", "route_pos", "row_tok", "row_route", "tile_expert", "tile_row0", "tile_rows", "expert_cnt",
+        "meta", "blk_cnt", "rank", "arrive")})
+    for _ in range(2):
+        ctx.launch(d, bufs)
+    torch.cuda.synchronize()
+    nt, rows = int(two.buf["meta"][0].item()), int(two.buf["meta"][1].item())
+    assert int(one.buf["arrive"][0].item()) == 0 and int(two.buf["arrive"][0].item()) == 0
+    for name in ("topk_ids", "topk_w", "route_pos", "expert_cnt", "meta"):
+        assert torch.equal(one.buf[name], two.buf[name]), name
+    for name in ("tile_expert", "tile_row0", "tile_rows"):
+        assert torch.equal(one.buf[name][:nt], two.buf[name][:nt]), name
+    for name in ("row_tok", "row_route"):
+        assert torch.equal(one.buf[name][:rows], two.buf[name][:rows]), name
+    ids, _ = ref.route(synth.f32_to_bf16_bits(np.random.default_rng(T).standard_normal(size=(T, E), dtype=np.float32)), k)
+    np.testing.assert_array_equal(two.buf["topk_ids"].cpu().numpy().reshape(T, k), ids)
+
+
 def test_grouped_tile_kernels_on_a_tiny_grid(ctx):
     """The tile kernels are persistent: on 3 workgroups instead of one a CU every workgroup walks more
     items than its item table holds (the 256-row kernel then resolves items as it goes, the 128-row
