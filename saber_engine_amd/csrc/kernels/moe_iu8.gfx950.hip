@@ -413,6 +413,10 @@ extern "C" __global__ __launch_bounds__(MOE_THREADS) void moe_iu8_route_place_e1
   __shared__ int s_cnt[MOE_E], s_base[MOE_E], s_off[MOE_E], s_toff[MOE_E];
   __shared__ int s_wave[MOE_THREADS / 64];
   const int tid = threadIdx.x, nblk = gridDim.x, blk = blockIdx.x;
+  // this thread's route: its expert and rank are requested now, beside the count table, not behind the scans
+  const int r = blk * (MOE_TPB * MOE_TOPK) + tid;
+  const bool mine = r < T * MOE_TOPK;
+  const int my_e = mine ? topk_ids[r] : -1, my_rank = mine ? rank[r] : 0;
   {
     const int e = tid % MOE_E, part = tid / MOE_E;
     const int chunk = (nblk + PARTS - 1) / PARTS, b_lo = min(part * chunk, nblk), b_hi = min(b_lo + chunk, nblk);
@@ -497,11 +501,10 @@ extern "C" __global__ __launch_bounds__(MOE_THREADS) void moe_iu8_route_place_e1
       row_route[sh_row0 + r] = -1;
     }
   }
-  const int r = blk * (MOE_TPB * MOE_TOPK) + tid;  // this workgroup's routes: a thread a route
-  if (r < T * MOE_TOPK) {
-    const int le = topk_ids[r] - e_lo;
+  if (mine) {  // this workgroup's routes: a thread a route
+    const int le = my_e - e_lo;
     const bool local = le >= 0 && le < e_loc;
-    const int p = local ? s_off[le] + s_base[le] + rank[r] : -1;
+    const int p = local ? s_off[le] + s_base[le] + my_rank : -1;
     route_pos[r] = p;
     if (local) {
       row_route[p] = r;
