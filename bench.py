@@ -49,6 +49,7 @@ def main():
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-moe", action="store_true")
+    ap.add_argument("--no-producers", action="store_true", help="skip the Hadamard-basis producers' section")
     ap.add_argument("--no-other-m", action="store_true", help="prefill at M = 2048 only (a profiler run that wants one M a kernel)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--probe-copy", action="store_true",
@@ -638,6 +639,58 @@ def main():
                                   frac=round((wbytes / us / 1e3) / HBM_PEAK_GBPS if T == 16 else (ops / us / 1e6) / INT8_PEAK_TOPS, 4))
             del layer, x, lg
         out["moe_e128_top8_h4096_i1536"] = moe
+    # ---- the Hadamard-basis int8 producers that feed these GEMMs in the served model (memory-bound: a pass over
+    # the bf16 rows in, the codes, scales and the new residual out), at decode and at prefill row counts
+    if not args.no_producers:
+        g = torch.Generator(device=dev)
+        g.manual_seed(1)
+
+        def bf16(*shape, scale=1.0):
+            return (torch.randn(shape, device=dev, generator=g) * scale).to(torch.bfloat16).view(torch.int16)
+
+        prod = {}
+        for PM in (16, 2048):
+            Kh, Ni, Ng, hd = 5120, 17408, 6144, 128
+            t_k = (torch.randint(0, 2, (Ni,), device=dev, generator=g).float() * 2 - 1)
+            q = torch.zeros(iu8.a_bytes(PM, Ni), dtype=torch.uint8, device=dev)
+            sc = torch.zeros(PM, dtype=torch.float32, device=dev)
+            xk, res, wk, ro = bf16(PM, Kh), bf16(PM, Kh, scale=4.0), bf16(Kh, scale=0.1), torch.zeros((PM, Kh), dtype=torch.int16, device=dev)
+            gu = bf16(PM, 2 * Ni, scale=2.0)
+            xg, zg, wg = bf16(PM, Ng, scale=2.0), bf16(PM, Ng, scale=3.0), bf16(hd)
+            core, blk = bf16(PM, Kh), bf16(PM, 2 * Kh, scale=3.0)
+            cases = {
+                "quant_had_k5120": (lambda: ctx.quant_had(xk.data_ptr(), q.data_ptr(), sc.data_ptr(), PM, Kh, t_k.data_ptr(), sh),
+                                    PM * (3 * Kh + 4)),
+                "add_rms_quant_had_k5120": (lambda: ctx.add_rms_quant_had(xk.data_ptr(), res.data_ptr(), wk.data_ptr(), q.data_ptr(), sc.data_ptr(),
+                                                                          ro.data_ptr(), PM, Kh, 1e-6, t_k.data_ptr(), sh),
+                                            PM * (7 * Kh + 4) + 2 * Kh),
+                "silu_mul_quant_had_n17408": (lambda: ctx.silu_mul_quant_had(gu.data_ptr(), q.data_ptr(), sc.data_ptr(), PM, Ni, t_k.data_ptr(), sh),
+                                              PM * (5 * Ni + 4)),
+                "gdn_norm_quant_had_n6144": (lambda: ctx.gdn_norm_quant_had(xg.data_ptr(), zg.data_ptr(), Ng, wg.data_ptr(), q.data_ptr(), sc.data_ptr(),
+                                                                            PM, Ng, 1e-6, t_k.data_ptr(), sh),
+                                             PM * (5 * Ng + 4)),
+                "attn_gate_quant_had_n5120": (lambda: ctx.attn_gate_quant_had(core.data_ptr(), blk.data_ptr(), q.data_ptr(), sc.data_ptr(), PM, Kh, hd,
+                                                                              2 * Kh, t_k.data_ptr(), sh),
+                                              PM * (5 * Kh + 4)),
+            }
+            row = {}
+            for name, (fn, nbytes) in cases.items():
+                reps = 200 if PM <= 16 else 60
+                with torch.cuda.stream(stream):
+                    for _ in range(10):
+                        fn()
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record(stream)
+                    for _ in range(reps):
+                        fn()
+                    e1.record(stream)
+                torch.cuda.synchronize()
+                us = e0.elapsed_time(e1) * 1e3 / reps
+                row[name] = dict(us=round(us, 2), bytes=int(nbytes), gbps=round(nbytes / us / 1e3, 1), hbm_frac=round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4))
+            prod["m%d" % PM] = row
+        prod["note"] = ("one launch a producer, back to back on one stream (inputs of the decode rows stay in the caches: those lines are launch latency, "
+                        "not bandwidth); bytes = bf16 rows in + codes + scales (+ the residual row out)")
+        out["hadamard_producers"] = prod
     print(json.dumps(out), flush=True)
     ctx.close()
 
