@@ -628,26 +628,35 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
       constexpr int ROWB = CB * 64 + 16, LPR = CB * 4, PIECES = 32 * LPR;
       static_assert(NWAVE * 32 * ROWB <= STAGE, "the epilogue region fits one stage");
       iu8_u8 *reg = smem + (st == 0 ? NST - 1 : st - 1) * STAGE + wave * (32 * ROWB);
+      float am[TM];
 #pragma unroll
-      for (int i = 0; i < TM; ++i) {
-        if (C.mbase + (wm * TM + i) * 32 >= M) continue;  // a row block past the tile's rows (the whole wave)
-        const int m = C.mbase + (wm * TM + i) * 32 + r32;
-        const float am = as[iu8_arow(C.R, min(m, M - 1))];
+      for (int i = 0; i < TM; ++i) am[i] = as[iu8_arow(C.R, min(C.mbase + (wm * TM + i) * 32 + r32, M - 1))];
+      // a column block's weight scales are fetched and brought to the accumulator's unit once, for all the
+      // wave's row blocks
 #pragma unroll
-        for (int jb = 0; jb < TN / CB; ++jb) {
+      for (int jb = 0; jb < TN / CB; ++jb) {
+        float4 wsu[CB][4];
+#pragma unroll
+        for (int jj = 0; jj < CB; ++jj)
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const int n = min(ncol0 + jb * (CB * 32) + jj * 32 + g * 8 + nq, N - 4);
+            const float4 w4 = *(const float4 *)(C.ws + n);
+            const float u = W8 ? 1.f : 0.0625f;  // exact: a power of two
+            wsu[jj][g] = float4{w4.x * u, w4.y * u, w4.z * u, w4.w * u};
+          }
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+          if (C.mbase + (wm * TM + i) * 32 >= M) continue;  // a row block past the tile's rows (the whole wave)
 #pragma unroll
           for (int jj = 0; jj < CB; ++jj) {
             const int j = jb * CB + jj;
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
               const int nl = jj * 32 + g * 8 + nq;
-              const int n = min(ncol0 + jb * (CB * 32) + nl, N - 4);
-              const float4 w4 = *(const float4 *)(C.ws + n);
-              const float u = W8 ? 1.f : 0.0625f;  // exact: a power of two
-              const unsigned lo = iu8_bf16_pack(iu8_epi(acc[i][j][g * 4], am, w4.x * u),
-                                                iu8_epi(acc[i][j][g * 4 + 1], am, w4.y * u));
-              const unsigned hi = iu8_bf16_pack(iu8_epi(acc[i][j][g * 4 + 2], am, w4.z * u),
-                                                iu8_epi(acc[i][j][g * 4 + 3], am, w4.w * u));
+              const float4 w4 = wsu[jj][g];
+              const unsigned lo = iu8_bf16_pack(iu8_epi(acc[i][j][g * 4], am[i], w4.x), iu8_epi(acc[i][j][g * 4 + 1], am[i], w4.y));
+              const unsigned hi = iu8_bf16_pack(iu8_epi(acc[i][j][g * 4 + 2], am[i], w4.z), iu8_epi(acc[i][j][g * 4 + 3], am[i], w4.w));
               *(iu8_v2u *)&reg[r32 * ROWB + nl * 2] = iu8_v2u{lo, hi};
             }
           }
