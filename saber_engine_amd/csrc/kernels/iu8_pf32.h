@@ -66,13 +66,14 @@ static __device__ __forceinline__ bool iu8_dense_tile_at(int r, int gx, int gy, 
   return true;
 }
 
-// LDS bytes of a cell's stages (what iu8_pf32_run declares, or expects from its caller).
+// LDS bytes of a cell (what iu8_pf32_run declares, or expects from its caller): its stages and, behind
+// them, two sets of a tile's epilogue scales (BM + BN floats each).
 template <bool W8, int WMW, int WNW, int TM, int TN, int STMAX>
 constexpr int iu8_pf32_lds_bytes() {
   constexpr int STAGE = WMW * TM * 2 * 2048 + WNW * TN * 2 * (W8 ? 2048 : 1024);
   constexpr int NFIT = 160 * 1024 / STAGE;
   constexpr int NST = STMAX < 2 ? 2 : (STMAX < NFIT ? STMAX : (NFIT < 2 ? 2 : NFIT));
-  return NST * STAGE;
+  return NST * STAGE + 2 * (WMW * TM * 32 + WNW * TN * 32) * 4;
 }
 
 // A split of K over gridDim.z (P, cnt not null): the workgroups of share z run steps [z*spb, (z+1)*spb)
@@ -126,9 +127,19 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
   if constexpr (EXT_LDS) {
     smem = ext_lds;
   } else {
-    __shared__ __attribute__((aligned(1024))) iu8_u8 own_lds[NST * STAGE];
+    __shared__ __attribute__((aligned(1024))) iu8_u8 own_lds[NST * STAGE + 2 * (BMT + BNT) * 16 * 4];
     smem = own_lds;
   }
+
+  // The epilogue's scales of a tile (its rows' activation scales, its columns' weight scales in the
+  // accumulator's unit) are put in LDS when the load stream enters the tile, a tile ahead of their use:
+  // fetched in the epilogue they were a dependent load or two (a gathered row's scale hangs on its
+  // row_tok entry) in front of the first output, with both waves of every SIMD waiting on them -- some
+  // 1.7 us an item, a tenth of an item of the routed down projection (K = 1536). Two sets: the tile being
+  // computed and the one the stream is in.
+  constexpr int BM = BMT * 16, BN = BNT * 16;
+  float(*s_am)[BM] = (float(*)[BM])(smem + NST * STAGE);
+  float(*s_wsu)[BN] = (float(*)[BN])(smem + NST * STAGE + 2 * BM * 4);
 
   // Opaque to the optimiser: a kernel that runs cells in a loop must not carry one cell's per-lane
   // addresses in registers through the other cell's K loop.
@@ -175,6 +186,15 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
     }
   };
   addr_of(L, ga, gw, qs);
+  // (with fewer K steps a tile than the stream runs ahead, it would be more than one tile ahead of the MFMAs and
+  // two sets would not do: such a launch fetches the scales in the epilogue)
+  const bool stashed = steps >= NST + (DEEP ? 1 : 0);  // the stream's lead in steps (the deep form fetches a step ahead of its MFMAs), and one to spare
+  auto stash_scales = [&](const iu8_tile &t, int set) {
+    if (!stashed) return;
+    if (tid < BM) s_am[set][tid] = as[iu8_arow(t.R, min(t.mbase + tid, t.R.rows - 1))];
+    for (int c = tid; c < BN; c += NWAVE * 64) s_wsu[set][c] = t.ws[min(t.nt0 * 16 + c, N - 1)] * (W8 ? 1.f : 0.0625f);  // exact: a power of two
+  };
+  stash_scales(L, 0);
   // The next tile's descriptor and addresses (a gathered tile reads its row map for them) are
   // fetched a whole tile ahead, so the stream never waits for them when it crosses into that tile.
   bool haveN = tile_at(1, Nx);
@@ -260,6 +280,7 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
 #pragma unroll
           for (int p = 0; p < A_PER; ++p) qs[p] = qsN[p];
         }
+        stash_scales(L, lr & 1);
         haveN = tile_at(lr + 1, Nx);
         if (haveN) addr_of(Nx, gaN, gwN, qsN);
       } else {
@@ -630,9 +651,9 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
       iu8_u8 *reg = smem + (st == 0 ? NST - 1 : st - 1) * STAGE + wave * (32 * ROWB);
       float am[TM];
 #pragma unroll
-      for (int i = 0; i < TM; ++i) am[i] = as[iu8_arow(C.R, min(C.mbase + (wm * TM + i) * 32 + r32, M - 1))];
-      // a column block's weight scales are fetched and brought to the accumulator's unit once, for all the
-      // wave's row blocks
+      for (int i = 0; i < TM; ++i)
+        am[i] = stashed ? s_am[r & 1][(wm * TM + i) * 32 + r32] : as[iu8_arow(C.R, min(C.mbase + (wm * TM + i) * 32 + r32, M - 1))];
+      // a column block's weight scales are read once, for all the wave's row blocks
 #pragma unroll
       for (int jb = 0; jb < TN / CB; ++jb) {
         float4 wsu[CB][4];
@@ -640,10 +661,13 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
         for (int jj = 0; jj < CB; ++jj)
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
-            const int n = min(ncol0 + jb * (CB * 32) + jj * 32 + g * 8 + nq, N - 4);
-            const float4 w4 = *(const float4 *)(C.ws + n);
-            const float u = W8 ? 1.f : 0.0625f;  // exact: a power of two
-            wsu[jj][g] = float4{w4.x * u, w4.y * u, w4.z * u, w4.w * u};
+            if (stashed) {
+              wsu[jj][g] = *(const float4 *)&s_wsu[r & 1][wn * TN * 32 + jb * (CB * 32) + jj * 32 + g * 8 + nq];
+            } else {
+              const float4 w4 = *(const float4 *)(C.ws + min(ncol0 + jb * (CB * 32) + jj * 32 + g * 8 + nq, N - 4));
+              const float u = W8 ? 1.f : 0.0625f;  // exact: a power of two
+              wsu[jj][g] = float4{w4.x * u, w4.y * u, w4.z * u, w4.w * u};
+            }
           }
 #pragma unroll
         for (int i = 0; i < TM; ++i) {

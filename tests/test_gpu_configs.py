@@ -109,7 +109,22 @@ def test_every_prefill_variant_gives_the_same_bytes(ctx, tag, w8):
         np.testing.assert_array_equal(run.C, r["C"])
 
 
-@pytest.mark.parametrize("shape", [(65, 16, 128), (97, 48, 256), (129, 304, 384), (4160, 1088, 256)])
+def test_prefill_several_tiles_a_workgroup_on_every_tile(ctx):
+    """More tiles than workgroups for every cell, the largest included, and seven K steps a tile: more
+    than the deepest cell's load stream runs ahead, so every cell hands a tile's epilogue scales over
+    through LDS a tile ahead (with fewer steps a cell fetches them in the epilogue: the edge shapes below
+    take that path, on two to five steps)."""
+    M, N, K = 8320, 4352, 896
+    for tag, w8 in (("w4", False), ("w8", True)):
+        case = synth.dense_case(M, N, K, w8=w8, seed=5)
+        r = ref.linear(case["X"], case["W"], case["ws"], w8, threads=8)
+        for name in all_variants(f"macaq_iu8_pf_{tag}_"):
+            say(f"prefill, several tiles a workgroup {(M, N, K)} {name}")
+            run = DenseRun(ctx, case, kernel=name, want_acc=False)
+            np.testing.assert_array_equal(run.C, r["C"])
+
+
+@pytest.mark.parametrize("shape", [(65, 16, 128), (97, 48, 256), (129, 304, 384), (4160, 1088, 256), (4160, 1088, 384), (4160, 1088, 512)])
 def test_prefill_edges_on_every_tile(ctx, shape):
     """One K step, two K steps (fewer than the LDS stages), ragged rows and columns, a tile count
     above the persistent grid (several tiles a workgroup, the load stream running across tiles)."""
