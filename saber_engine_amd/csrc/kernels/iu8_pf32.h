@@ -66,14 +66,22 @@ static __device__ __forceinline__ bool iu8_dense_tile_at(int r, int gx, int gy, 
   return true;
 }
 
-// LDS bytes of a cell (what iu8_pf32_run declares, or expects from its caller): its stages and, behind
-// them, two sets of a tile's epilogue scales (BM + BN floats each).
-template <bool W8, int WMW, int WNW, int TM, int TN, int STMAX>
+// The grouped launches' tile cells (the sparse forms, at least 128 x 256) hand a tile's epilogue scales over
+// through LDS (below): their items are short in K (an expert's down projection: 12 steps) and many a
+// workgroup. A dense launch has long tiles and often one a workgroup: there the hand-over measured 3 % slower.
+template <bool SPARSE, int WMW, int WNW, int TM, int TN>
+constexpr bool iu8_pf32_stashes() {
+  return SPARSE && WMW * TM * 32 * WNW * TN * 32 >= 128 * 256;
+}
+// LDS bytes of a cell (what iu8_pf32_run declares, or expects from its caller): its stages and, where the
+// cell stashes them (STASH: iu8_pf32_stashes), two sets of a tile's epilogue scales (BM + BN floats each)
+// behind them.
+template <bool W8, int WMW, int WNW, int TM, int TN, int STMAX, bool STASH = false>
 constexpr int iu8_pf32_lds_bytes() {
   constexpr int STAGE = WMW * TM * 2 * 2048 + WNW * TN * 2 * (W8 ? 2048 : 1024);
   constexpr int NFIT = 160 * 1024 / STAGE;
   constexpr int NST = STMAX < 2 ? 2 : (STMAX < NFIT ? STMAX : (NFIT < 2 ? 2 : NFIT));
-  return NST * STAGE + 2 * (WMW * TM * 32 + WNW * TN * 32) * 4;
+  return NST * STAGE + (STASH ? 2 * (WMW * TM * 32 + WNW * TN * 32) * 4 : 0);
 }
 
 // A split of K over gridDim.z (P, cnt not null): the workgroups of share z run steps [z*spb, (z+1)*spb)
@@ -127,12 +135,12 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
   if constexpr (EXT_LDS) {
     smem = ext_lds;
   } else {
-    __shared__ __attribute__((aligned(1024))) iu8_u8 own_lds[NST * STAGE + 2 * (BMT + BNT) * 16 * 4];
+    __shared__ __attribute__((aligned(1024))) iu8_u8 own_lds[iu8_pf32_lds_bytes<W8, WMW, WNW, TM, TN, STMAX, iu8_pf32_stashes<SPARSE, WMW, WNW, TM, TN>()>()];
     smem = own_lds;
   }
 
   // The epilogue's scales of a tile (its rows' activation scales, its columns' weight scales in the
-  // accumulator's unit) are put in LDS when the load stream enters the tile, a tile ahead of their use:
+  // weight scales) are put in LDS when the load stream enters the tile, a tile ahead of their use:
   // fetched in the epilogue they were a dependent load or two (a gathered row's scale hangs on its
   // row_tok entry) in front of the first output, with both waves of every SIMD waiting on them -- some
   // 1.7 us an item, a tenth of an item of the routed down projection (K = 1536). Two sets: the tile being
@@ -186,13 +194,28 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
     }
   };
   addr_of(L, ga, gw, qs);
+  const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) iu8_u8 *)smem;
   // (with fewer K steps a tile than the stream runs ahead, it would be more than one tile ahead of the MFMAs and
   // two sets would not do: such a launch fetches the scales in the epilogue)
-  const bool stashed = steps >= NST + (DEEP ? 1 : 0);  // the stream's lead in steps (the deep form fetches a step ahead of its MFMAs), and one to spare
+  const bool stashed = iu8_pf32_stashes<SPARSE, WMW, WNW, TM, TN>() && steps >= NST + (DEEP ? 1 : 0);  // the stream's lead in steps (the deep form fetches a step ahead of its MFMAs), and one to spare
+  // Rows in place: both tables come by LDS-DMA like the operands (a dword a lane, 64 consecutive entries a
+  // wave-load), so nothing waits for them at the crossing. Gathered rows: the row's scale hangs on its
+  // row_tok entry, an ordinary dependent load -- the crossing of such a tile waits for that entry anyway,
+  // for the operand addresses.
+  auto dma4 = [&](const void *base, unsigned off, unsigned lds) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" : : "s"(lds), "v"(off), "s"(base) : "memory", "m0");
+  };
   auto stash_scales = [&](const iu8_tile &t, int set) {
     if (!stashed) return;
-    if (tid < BM) s_am[set][tid] = as[iu8_arow(t.R, min(t.mbase + tid, t.R.rows - 1))];
-    for (int c = tid; c < BN; c += NWAVE * 64) s_wsu[set][c] = t.ws[min(t.nt0 * 16 + c, N - 1)] * (W8 ? 1.f : 0.0625f);  // exact: a power of two
+    const unsigned l_am = lds0 + NST * STAGE + set * BM * 4, l_ws = lds0 + NST * STAGE + 2 * BM * 4 + set * BN * 4;
+    if (t.R.row_tok == nullptr) {
+      if (wave < BM / 64) dma4(as, (unsigned)iu8_arow(t.R, min(t.mbase + tid, t.R.rows - 1)) * 4u, l_am + wave * 256);
+    } else if (tid < BM) {
+      s_am[set][tid] = as[iu8_arow(t.R, min(t.mbase + tid, t.R.rows - 1))];
+    }
+#pragma unroll
+    for (int c0 = 0; c0 < BN; c0 += NWAVE * 64)
+      if (c0 + tid < BN) dma4(t.ws, (unsigned)min(t.nt0 * 16 + c0 + tid, N - 1) * 4u, l_ws + (c0 + wave * 64) * 4);  // (a lane an entry: none past the set)
   };
   stash_scales(L, 0);
   // The next tile's descriptor and addresses (a gathered tile reads its row map for them) are
@@ -209,7 +232,6 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
                  : "s"(lds), "v"(off), "s"(base)
                  : "memory", "m0");
   };
-  const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) iu8_u8 *)smem;
   // AQ: the bf16 pieces of every fragment of A this wave owns (two 16-byte loads a fragment) and the
   // scale of their rows. Fragment p is loaded in phase p % 3 of a step, right behind the conversion of
   // the pieces it replaces, and converted a whole step later: a step of latency cover, one register
@@ -661,13 +683,10 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
         for (int jj = 0; jj < CB; ++jj)
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
-            if (stashed) {
-              wsu[jj][g] = *(const float4 *)&s_wsu[r & 1][wn * TN * 32 + jb * (CB * 32) + jj * 32 + g * 8 + nq];
-            } else {
-              const float4 w4 = *(const float4 *)(C.ws + min(ncol0 + jb * (CB * 32) + jj * 32 + g * 8 + nq, N - 4));
-              const float u = W8 ? 1.f : 0.0625f;  // exact: a power of two
-              wsu[jj][g] = float4{w4.x * u, w4.y * u, w4.z * u, w4.w * u};
-            }
+            const float4 w4 = stashed ? *(const float4 *)&s_wsu[r & 1][wn * TN * 32 + jb * (CB * 32) + jj * 32 + g * 8 + nq]
+                                      : *(const float4 *)(C.ws + min(ncol0 + jb * (CB * 32) + jj * 32 + g * 8 + nq, N - 4));
+            const float u = W8 ? 1.f : 0.0625f;  // exact: a power of two
+            wsu[jj][g] = float4{w4.x * u, w4.y * u, w4.z * u, w4.w * u};
           }
 #pragma unroll
         for (int i = 0; i < TM; ++i) {

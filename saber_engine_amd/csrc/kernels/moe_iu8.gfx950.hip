@@ -725,7 +725,7 @@ static __device__ __forceinline__ void moe_grouped_pf_one(
   static_assert(BN == 256 && WMW * WNW == 8, "both cells are 8 waves and 256 columns wide");
   __shared__ unsigned short s_order[MOE_ORDER_CAP];
   __shared__ moe_item s_item[MOE_ONE_ITEMS];
-  __shared__ __attribute__((aligned(1024))) iu8_u8 lds[iu8_pf32_lds_bytes<false, WMW, WNW, TM, TN, ST>()];  // one block for both walks below
+  __shared__ __attribute__((aligned(1024))) iu8_u8 lds[iu8_pf32_lds_bytes<false, WMW, WNW, TM, TN, ST, true>()];  // one block for both walks below
   const int nt = meta[0], gx = (n + BN - 1) / BN, total = nt * gx;
   const bool ordered = nt <= MOE_ORDER_CAP;
   if (ordered) moe_tile_order<WMW * WNW * 64>(tile_rows, nt, s_order);
@@ -777,7 +777,7 @@ static __device__ __forceinline__ void moe_grouped_pf_two(
     const int *__restrict__ meta, const float *__restrict__ as, unsigned short *__restrict__ c, int n, int k) {
   constexpr int BN = WNW * TN * 32;
   static_assert(BN == 256 && WMW * WNW == 8, "both cells are 8 waves and 256 columns wide");
-  constexpr int LB = iu8_pf32_lds_bytes<false, WMW, WNW, TM, TN, ST>();
+  constexpr int LB = iu8_pf32_lds_bytes<false, WMW, WNW, TM, TN, ST, true>();
   constexpr int LL = iu8_pf32_lds_bytes<false, 2, 4, 1, 2, MOE_LIGHT_ST>();
   __shared__ __attribute__((aligned(1024))) iu8_u8 lds[LB > LL ? LB : LL];
   __shared__ unsigned short s_order[MOE_ORDER_CAP];
