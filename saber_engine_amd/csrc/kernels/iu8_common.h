@@ -106,8 +106,12 @@ static __device__ __forceinline__ unsigned iu8_code4_rcp(float x0, float x1, flo
   const float off = fmaxf(fmaxf(fabsf(t0 - (u0 - MAGIC)), fabsf(t1 - (u1 - MAGIC))),
                           fmaxf(fabsf(t2 - (u2 - MAGIC)), fabsf(t3 - (u3 - MAGIC))));
   const bool near_tie = !(off <= 0.4999f);  // NaN goes to the divide as well
-  if (__builtin_expect(near_tie, 0))
+  if (__builtin_expect(near_tie, 0)) {
+    // stays a branch: without this statement the compiler now and then runs the four divides for every
+    // quad and selects afterwards (seen as a third more VALU work in a row producer)
+    asm volatile("");
     return iu8_code(x0, sc) | (iu8_code(x1, sc) << 8) | (iu8_code(x2, sc) << 16) | (iu8_code(x3, sc) << 24);
+  }
   // bytes 0,1 from (u0, u1), bytes 2,3 from (u2, u3); selector 0x0c yields a zero byte
   return __builtin_amdgcn_perm(__float_as_uint(u1), __float_as_uint(u0), 0x0c0c0400u) |
          __builtin_amdgcn_perm(__float_as_uint(u3), __float_as_uint(u2), 0x04000c0cu);

@@ -82,6 +82,72 @@ static __device__ __forceinline__ void i8q_tail(float (&v)[I8Q_MAXG][16], int G,
   }
 }
 
+// The same from a row kept as packed bf16 pairs (pk[g][w]: elements 2w and 2w + 1 of group g, as loaded; a
+// thread's groups past the row's end are zeros). The largest magnitude of finite bf16 values is
+// the largest of their bit patterns without the sign, two a packed 16-bit maximum; a thread that holds a
+// NaN (a pattern above infinity's) takes the f32 maximum instead, which passes NaNs over.
+template <int NG>
+static __device__ __forceinline__ float i8q_pk_amax(const unsigned (&pk)[NG][8]) {
+  typedef unsigned short us2 __attribute__((ext_vector_type(2)));
+  us2 m2 = {0, 0};
+#pragma unroll
+  for (int i = 0; i < NG; ++i)
+#pragma unroll
+    for (int w = 0; w < 8; ++w) m2 = __builtin_elementwise_max(m2, __builtin_bit_cast(us2, pk[i][w] & 0x7FFF7FFFu));
+  const unsigned top = m2.x > m2.y ? m2.x : m2.y;
+  float amax = __uint_as_float(top << 16);
+  if (top > 0x7F80u) {
+    amax = 0.f;
+#pragma unroll
+    for (int i = 0; i < NG; ++i)
+#pragma unroll
+      for (int w = 0; w < 8; ++w) {
+        unsigned r = pk[i][w];
+        asm volatile("" : "+v"(r));  // a value of its own: nothing of the fast path is kept alive for this one
+        amax = fmaxf(amax, fabsf(__uint_as_float(r << 16)));
+        amax = fmaxf(amax, fabsf(__uint_as_float(r & 0xFFFF0000u)));
+      }
+  }
+  return amax;
+}
+static __device__ __forceinline__ iu8_v4u i8q_pk_codes(const unsigned (&g)[8], float sc, float rcp) {
+  unsigned d[4];
+#pragma unroll
+  for (int w = 0; w < 4; ++w)
+    d[w] = iu8_code4_rcp(__uint_as_float(g[2 * w] << 16), __uint_as_float(g[2 * w] & 0xFFFF0000u),
+                         __uint_as_float(g[2 * w + 1] << 16), __uint_as_float(g[2 * w + 1] & 0xFFFF0000u), sc, rcp);
+  return iu8_v4u{d[0], d[1], d[2], d[3]};
+}
+// A group's 16 elements, zeros when the group is past the row's end. Nothing uses the registers before
+// every group of the row has been requested: a load whose data is used under the same test is waited
+// for before the next is requested -- MAXG memory latencies a row instead of one.
+static __device__ __forceinline__ void i8q_pk_load(unsigned (&g)[8], const unsigned short *p, bool live) {
+  iu8_v4u lo = {0u, 0u, 0u, 0u}, hi = {0u, 0u, 0u, 0u};
+  if (live) lo = *(const iu8_v4u *)p, hi = *(const iu8_v4u *)(p + 8);
+#pragma unroll
+  for (int w = 0; w < 4; ++w) g[w] = lo[w], g[4 + w] = hi[w];
+}
+template <int I8Q_MAXG, bool RM, bool SCALE_ONLY>
+static __device__ __forceinline__ void i8q_tail_pk(const unsigned (&pk)[I8Q_MAXG][8], int G, iu8_u8 *__restrict__ q,
+                                                   float *__restrict__ scale, int row, int K) {
+  const int tid = threadIdx.x;
+  const float amax = i8q_block_max(i8q_pk_amax(pk));
+  const float sc = fmaxf(__fdiv_rn(amax, 127.f), 1e-30f);
+  const float rcp = __fdiv_rn(1.f, sc);
+  if (tid == 0) scale[row] = sc;
+  if constexpr (SCALE_ONLY) return;
+  iu8_u8 *qrow = q + (size_t)(row >> 4) * (K >> 6) * 1024 + (row & 15) * 16;
+#pragma unroll
+  for (int i = 0; i < I8Q_MAXG; ++i) {
+    const int g = tid + i * I8Q_T;
+    if (g >= G) continue;
+    const iu8_v4u d = i8q_pk_codes(pk[i], sc, rcp);
+    if constexpr (RM) *(iu8_v4u *)(q + (size_t)row * K + g * 16) = d;
+    else *(iu8_v4u *)(qrow + (size_t)(g >> 2) * 1024 + (g & 3) * 256) = d;
+    __builtin_amdgcn_sched_barrier(0);  // a group's codes at a time: their temporaries are what fills the registers
+  }
+}
+
 // `row_tok` / `meta` (optional, may be null): with them output row r is the quantised input row
 // row_tok[r] (the expert-major rows of a routed layer, gathered here once so that the grouped GEMM
 // reads whole fragments); pad rows (row_tok < 0) and rows past meta[1] are skipped.
@@ -98,32 +164,41 @@ static __device__ __forceinline__ void i8q_quant_body(const unsigned short *__re
     if (src < 0) return;
   }
   const unsigned short *xr = x + (size_t)src * k;
-  float v[I8Q_MAXG][16];
+  if constexpr (I8Q_MAXG >= 5) {
+    // The long forms request a row's pieces all at once (i8q_pk_load) and keep them packed as they came, 8
+    // registers a group instead of 16: the form for up to 20,480 elements then runs eight waves a SIMD
+    // (2,048 rows of 17,408: 26.0 -> 21.9 us). The forms of one or two groups measured 4-8 % slower this way.
+    unsigned pk[I8Q_MAXG][8];
 #pragma unroll
-  for (int i = 0; i < I8Q_MAXG; ++i) {
-    const int g = threadIdx.x + i * I8Q_T;
-    if (g >= G) continue;
-    const iu8_v4u lo = *(const iu8_v4u *)(xr + g * 16), hi = *(const iu8_v4u *)(xr + g * 16 + 8);
+    for (int i = 0; i < I8Q_MAXG; ++i) i8q_pk_load(pk[i], xr + (threadIdx.x + i * I8Q_T) * 16, (int)threadIdx.x + i * I8Q_T < G);
+    i8q_tail_pk<I8Q_MAXG, RM, SCALE_ONLY>(pk, G, q, scale, row, k);
+  } else {
+    float v[I8Q_MAXG][16];
 #pragma unroll
-    for (int w = 0; w < 4; ++w) {
-      v[i][2 * w] = __uint_as_float(lo[w] << 16);
-      v[i][2 * w + 1] = __uint_as_float(lo[w] & 0xFFFF0000u);
-      v[i][8 + 2 * w] = __uint_as_float(hi[w] << 16);
-      v[i][8 + 2 * w + 1] = __uint_as_float(hi[w] & 0xFFFF0000u);
+    for (int i = 0; i < I8Q_MAXG; ++i) {
+      const int g = threadIdx.x + i * I8Q_T;
+      if (g >= G) continue;
+      const iu8_v4u lo = *(const iu8_v4u *)(xr + g * 16), hi = *(const iu8_v4u *)(xr + g * 16 + 8);
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        v[i][2 * w] = __uint_as_float(lo[w] << 16);
+        v[i][2 * w + 1] = __uint_as_float(lo[w] & 0xFFFF0000u);
+        v[i][8 + 2 * w] = __uint_as_float(hi[w] << 16);
+        v[i][8 + 2 * w + 1] = __uint_as_float(hi[w] & 0xFFFF0000u);
+      }
     }
+    i8q_tail<I8Q_MAXG, RM, SCALE_ONLY>(v, G, q, scale, row, k);
   }
-  i8q_tail<I8Q_MAXG, RM, SCALE_ONLY>(v, G, q, scale, row, k);
 }
-#define I8Q_QUANT(name, MAXG)                                                                                   \
-  extern "C" __global__ __launch_bounds__(I8Q_T) void name(const unsigned short *__restrict__ x,                \
-                                                           unsigned char *__restrict__ q, float *__restrict__ scale, \
-                                                           int k) {                                             \
+#define I8Q_QUANT(name, MAXG, WPE)                                                                              \
+  extern "C" __global__ __launch_bounds__(I8Q_T) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) void name(      \
+      const unsigned short *__restrict__ x, unsigned char *__restrict__ q, float *__restrict__ scale, int k) {  \
     i8q_quant_body<MAXG>(x, q, scale, k);                                                                       \
   }
-I8Q_QUANT(macaq_i8_quant_t256, 8)
-I8Q_QUANT(macaq_i8_quant_t256_g5, 5)
-I8Q_QUANT(macaq_i8_quant_t256_g2, 2)
-I8Q_QUANT(macaq_i8_quant_t256_g1, 1)
+I8Q_QUANT(macaq_i8_quant_t256, 8, 5)
+I8Q_QUANT(macaq_i8_quant_t256_g5, 5, 8)
+I8Q_QUANT(macaq_i8_quant_t256_g2, 2, 8)
+I8Q_QUANT(macaq_i8_quant_t256_g1, 1, 8)
 #undef I8Q_QUANT
 // the rows' scales alone: x bf16 [M, K] -> scale f32 [M] (what macaq_i8_quant_* stores beside its codes)
 #define I8Q_ROWSCALE(name, MAXG)                                                                                \
