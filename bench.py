@@ -658,6 +658,8 @@ def main():
             gu = bf16(PM, 2 * Ni, scale=2.0)
             xg, zg, wg = bf16(PM, Ng, scale=2.0), bf16(PM, Ng, scale=3.0), bf16(hd)
             core, blk = bf16(PM, Kh), bf16(PM, 2 * Kh, scale=3.0)
+            silu_lut = torch.zeros(65536, dtype=torch.int16, device=dev)
+            ctx.silu_table(silu_lut.data_ptr(), sh)
             cases = {
                 "quant_had_k5120": (lambda: ctx.quant_had(xk.data_ptr(), q.data_ptr(), sc.data_ptr(), PM, Kh, t_k.data_ptr(), sh),
                                     PM * (3 * Kh + 4)),
@@ -666,6 +668,9 @@ def main():
                                             PM * (7 * Kh + 4) + 2 * Kh),
                 "silu_mul_quant_had_n17408": (lambda: ctx.silu_mul_quant_had(gu.data_ptr(), q.data_ptr(), sc.data_ptr(), PM, Ni, t_k.data_ptr(), sh),
                                               PM * (5 * Ni + 4)),
+                "silu_mul_quant_had_lut_n17408": (lambda: ctx.silu_mul_quant_had_lut(gu.data_ptr(), q.data_ptr(), sc.data_ptr(), PM, Ni, t_k.data_ptr(),
+                                                                                     silu_lut.data_ptr(), sh),
+                                                  PM * (5 * Ni + 4)),
                 "gdn_norm_quant_had_n6144": (lambda: ctx.gdn_norm_quant_had(xg.data_ptr(), zg.data_ptr(), Ng, wg.data_ptr(), q.data_ptr(), sc.data_ptr(),
                                                                             PM, Ng, 1e-6, t_k.data_ptr(), sh),
                                              PM * (5 * Ng + 4)),
@@ -689,7 +694,8 @@ def main():
                 row[name] = dict(us=round(us, 2), bytes=int(nbytes), gbps=round(nbytes / us / 1e3, 1), hbm_frac=round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4))
             prod["m%d" % PM] = row
         prod["note"] = ("one launch a producer, back to back on one stream (inputs of the decode rows stay in the caches: those lines are launch latency, "
-                        "not bandwidth); bytes = bf16 rows in + codes + scales (+ the residual row out)")
+                        "not bandwidth); bytes = bf16 rows in + codes + scales (+ the residual row out); silu_mul_quant_had_lut = the same op with "
+                        "the caller's table of the bf16 silu at hand")
         out["hadamard_producers"] = prod
     print(json.dumps(out), flush=True)
     ctx.close()

@@ -266,6 +266,17 @@ int saber_iu8_quant_had(saber_iu8_ctx *ctx, const void *x_bf16, void *q, float *
                         const float *had_t, void *stream);
 int saber_iu8_silu_mul_quant_had(saber_iu8_ctx *ctx, const void *gu_bf16, void *q, float *scale, uint32_t m, uint32_t n,
                                  const float *had_t, void *stream);
+/* saber_iu8_silu_mul_quant_had with a table of the bf16 silu at hand (`silu_lut`: u16 [65536] on the device
+ * as saber_iu8_silu_table wrote it, a 128 KiB persistent workspace of the caller, filled once): for rows of
+ * SABER_IU8_SILU_LUT_MIN_WIDTH elements and more the launch reads bf16(silu(gate)) from the table's middle,
+ * which every workgroup copies into LDS (kernels silu_mul_quant_hadi8_lut_t{256,512}; the computed form
+ * spends more than half of its arithmetic on the exp and the divide and is bound by it); narrower rows, or a
+ * null table, are saber_iu8_silu_mul_quant_had. Same bytes either way: the table is the computed form's own
+ * output. No counterpart among the reference's operators: its producer computes
+ * (crates/saber-kernels/hip/mxfp4_hadi8.hip:117-146). */
+#define SABER_IU8_SILU_LUT_MIN_WIDTH 2048u
+int saber_iu8_silu_mul_quant_had_lut(saber_iu8_ctx *ctx, const void *gu_bf16, void *q, float *scale, uint32_t m, uint32_t n,
+                                     const float *had_t, const uint16_t *silu_lut, void *stream);
 int saber_iu8_add_rms_quant_had(saber_iu8_ctx *ctx, const void *y_bf16, const void *res_bf16, const void *w_bf16, void *q,
                                 float *scale, void *res_out_bf16, uint32_t m, uint32_t k, float eps, const float *had_t,
                                 void *stream);

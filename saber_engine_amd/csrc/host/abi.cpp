@@ -39,6 +39,8 @@ static const Signature SIG_HAD_ARQ = {{"y", K::Buffer},     {"res", K::Buffer}, 
                                       {"q", K::Buffer},     {"scale", K::Buffer},   {"res_out", K::Buffer},
                                       {"k", K::I32},        {"eps", K::F32},        {"had_t", K::Buffer}};
 static const Signature SIG_HAD_SMQ = {{"gu", K::Buffer}, {"q", K::Buffer}, {"scale", K::Buffer}, {"n", K::I32}, {"had_t", K::Buffer}};
+static const Signature SIG_HAD_SMQ_LUT = {{"gu", K::Buffer}, {"q", K::Buffer}, {"scale", K::Buffer}, {"n", K::I32},
+                                          {"had_t", K::Buffer}, {"lut", K::Buffer}};
 static const Signature SIG_HAD_Q = {{"x", K::Buffer}, {"q", K::Buffer}, {"scale", K::Buffer}, {"k", K::I32}, {"had_t", K::Buffer}};
 // crates/saber-kernels/src/abi.rs:652-662 and :2683-2694, `had_t` appended last
 static const Signature SIG_HAD_GNQ = {{"x", K::Buffer}, {"z", K::Buffer},     {"zs", K::I64}, {"w", K::Buffer},
@@ -87,6 +89,7 @@ const Signature *signature_for(const std::string &k) {
   if (starts(k, "macaq_iu8f_pair_") || starts(k, "macaq_iu8f_pairb_")) return &SIG_PAIR;
   if (starts(k, "macaq_iu8f_mlp_")) return &SIG_MLP;
   if (starts(k, "add_rms_quant_hadi8_")) return &SIG_HAD_ARQ;
+  if (starts(k, "silu_mul_quant_hadi8_lut_")) return &SIG_HAD_SMQ_LUT;
   if (starts(k, "silu_mul_quant_hadi8_")) return &SIG_HAD_SMQ;
   if (starts(k, "quant_hadi8_")) return &SIG_HAD_Q;
   if (starts(k, "gdn_norm_quant_hadi8_")) return &SIG_HAD_GNQ;

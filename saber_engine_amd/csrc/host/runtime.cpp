@@ -600,6 +600,20 @@ int saber_iu8_silu_mul_quant_had(saber_iu8_ctx *ctx, const void *gu, void *q, fl
   return saber_iu8_launch(ctx, &d, b, 4, stream);
 }
 
+int saber_iu8_silu_mul_quant_had_lut(saber_iu8_ctx *ctx, const void *gu, void *q, float *scale, uint32_t m, uint32_t n,
+                                     const float *had_t, const uint16_t *silu_lut, void *stream) {
+  if (!silu_lut || n < SABER_IU8_SILU_LUT_MIN_WIDTH) return saber_iu8_silu_mul_quant_had(ctx, gu, q, scale, m, n, had_t, stream);
+  saber_iu8_desc d;
+  if (int rc = had_desc("silu_mul_quant_had_i8", "silu_mul_quant", m, n, &d)) return rc;  // the shape checks, grid and block
+  const std::string name = fmt("silu_mul_quant_hadi8_lut_t%u", d.block[0]);
+  const uint32_t grid[3] = {m, 1, 1};
+  if (int rc = saber_iu8_describe_raw(name.c_str(), "mxfp4_hadi8", grid, d.block[0], &d)) return rc;
+  snprintf(d.op, sizeof d.op, "silu_mul_quant_had_i8");
+  set_i32(&d, "n", n);
+  const saber_iu8_binding b[] = {{"gu", (void *)gu}, {"q", q}, {"scale", scale}, {"had_t", (void *)had_t}, {"lut", (void *)silu_lut}};
+  return saber_iu8_launch(ctx, &d, b, 5, stream);
+}
+
 int saber_iu8_add_rms_quant_had(saber_iu8_ctx *ctx, const void *y, const void *res, const void *w, void *q, float *scale,
                                 void *res_out, uint32_t m, uint32_t k, float eps, const float *had_t, void *stream) {
   saber_iu8_desc d;

@@ -29,9 +29,8 @@ static __device__ __forceinline__ void had_lane_stage(float (&v)[8], bool holds_
 // butterfly over element bits 0..4 in that order -- bits 0..2 pair registers, bits 3 and 4 pair lanes
 // (xor 1, xor 2) -- each stage (low, high) -> (low + high, low - high), then one multiply by
 // (float)(1 / sqrt(32)). t8: the 8 entries of t for this lane's elements. In place.
-static __device__ __forceinline__ void had32(float (&v)[8], const float *__restrict__ t8, int lane) {
+static __device__ __forceinline__ void had32(float (&v)[8], iu8_v4f t_lo, iu8_v4f t_hi, int lane) {
 #pragma clang fp contract(off)
-  const iu8_v4f t_lo = *(const iu8_v4f *)t8, t_hi = *(const iu8_v4f *)(t8 + 4);
 #pragma unroll
   for (int j = 0; j < 4; ++j) v[j] = v[j] * t_lo[j], v[j + 4] = v[j + 4] * t_hi[j];
 #pragma unroll
@@ -50,6 +49,10 @@ static __device__ __forceinline__ void had32(float (&v)[8], const float *__restr
   const float inv_sqrt32 = __uint_as_float(0x3E3504F3u);
 #pragma unroll
   for (int j = 0; j < 8; ++j) v[j] = v[j] * inv_sqrt32;
+}
+
+static __device__ __forceinline__ void had32(float (&v)[8], const float *__restrict__ t8, int lane) {
+  had32(v, *(const iu8_v4f *)t8, *(const iu8_v4f *)(t8 + 4), lane);
 }
 
 // The row of workgroup b: the 8 A tiles of a full group of 128 rows go one to an XCD (consecutive

@@ -7,6 +7,7 @@
 //
 //   add_rms_quant_hadi8_t{256,512}_tiled1   v = bf16((f32(y) + f32(res)) * inv * (f32(w) + 1)), res_out = bf16(y + res)
 //   silu_mul_quant_hadi8_t{256,512}_tiled1  v = bf16(bf16(silu(gate)) * up)
+//   silu_mul_quant_hadi8_lut_t{256,512}     the same with bf16(silu(gate)) read from a table (LDS)
 //   quant_hadi8_t{256,512}_tiled1           v = x (no counterpart among the reference's symbols: the
 //                                           transform in front of the plain producer)
 //   gdn_norm_quant_hadi8_t256_tiled1        v = bf16(((x * inv_head) * w) * silu_f32(z)), per 128-element head
@@ -140,6 +141,73 @@ HAD_ARQ(add_rms_quant_hadi8_t512_tiled1, 512)
 HAD_SMQ(silu_mul_quant_hadi8_t256_tiled1, 256)
 HAD_SMQ(silu_mul_quant_hadi8_t512_tiled1, 512)
 #undef HAD_SMQ
+
+// silu_mul_quant with the bf16 silu read from a table: `lut` holds bf16(silu(x)) of every bf16 bit pattern x as
+// macaq_silu_bf16_table (code object `macaq_i8q`) wrote it, i.e. this file's own expression
+// vg / (1 + expf(-vg)) rounded to bf16, so the bytes are those of the computed form, which spends about 30 of
+// its 55 VALU operations an element on the exp and the divide and is bound by them. A workgroup copies the
+// table's middle -- magnitudes from 2^-17 up to 2^15, both signs: 2 x 4,096 entries, 16 KiB -- into LDS beside
+// its row's loads; a gate outside (one in some hundred thousand of unit-scale rows) is computed as before.
+// The kernel is the computed form otherwise (a workgroup a row, the same lane map). No counterpart among
+// the reference's symbols (`lut` behind its kernarg list).
+#define HAD_LUT_LO (110 << 7)  // first pattern without sign in the table: 2^-17
+#define HAD_LUT_N 4096         // patterns a sign: 32 exponents
+template <int T>
+static __device__ __forceinline__ void had_silu_lut_body(const unsigned short *__restrict__ gu, iu8_u8 *__restrict__ q,
+                                                         float *__restrict__ scale, int N,
+                                                         const float *__restrict__ had_t,
+                                                         const unsigned short *__restrict__ lut) {
+#pragma clang fp contract(off)
+  __shared__ __attribute__((aligned(16))) unsigned short s_lut[2 * HAD_LUT_N];
+  const int row = had_row(), tid = threadIdx.x, NV = N >> 3;
+  gu += (size_t)row * 2 * N;
+  // the row's pieces and the table are requested together, nothing is used before the last request has left
+  iu8_v4u rg[HAD_MAXG], ru[HAD_MAXG], tb[2 * HAD_LUT_N / 8 / T];
+#pragma unroll
+  for (int i = 0; i < HAD_MAXG; ++i) {
+    const int g = tid + i * T;
+    rg[i] = ru[i] = iu8_v4u{0u, 0u, 0u, 0u};
+    if (g < NV) rg[i] = *(const iu8_v4u *)(gu + (unsigned)(g * 8)), ru[i] = *(const iu8_v4u *)(gu + N + (unsigned)(g * 8));
+  }
+#pragma unroll
+  for (int c = 0; c < 2 * HAD_LUT_N / 8 / T; ++c) {
+    const int i = (c * T + tid) * 8;  // entry: sign i / HAD_LUT_N, pattern HAD_LUT_LO + i % HAD_LUT_N
+    tb[c] = *(const iu8_v4u *)(lut + (i / HAD_LUT_N) * 32768 + HAD_LUT_LO + (i & (HAD_LUT_N - 1)));
+  }
+#pragma unroll
+  for (int c = 0; c < 2 * HAD_LUT_N / 8 / T; ++c) ((iu8_v4u *)s_lut)[c * T + tid] = tb[c];
+  __syncthreads();
+  auto silu = [&](unsigned b) {  // bf16 pattern (low 16 bits) -> bf16(silu) as f32
+    const unsigned idx = (b & 0x7FFFu) - HAD_LUT_LO;
+    if (__builtin_expect(idx < (unsigned)HAD_LUT_N, 1)) return iu8_bf16_f32(s_lut[((b >> 15) << 12) | idx]);
+    const float x = iu8_bf16_f32((unsigned short)b);
+    return iu8_bf16_f32((unsigned short)iu8_bf16_bits(x / (1.f + expf(-x))));
+  };
+  float sv[HAD_MAXG][8];
+#pragma unroll
+  for (int i = 0; i < HAD_MAXG; ++i) {
+    const int g = tid + i * T;
+    if (g >= NV) continue;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {  // two products a v_cvt_pk_bf16_f32
+      const float t0 = silu(rg[i][w] & 0xFFFFu), t1 = silu(rg[i][w] >> 16);
+      const unsigned p2 = iu8_bf16_pack(t0 * __uint_as_float(ru[i][w] << 16), t1 * __uint_as_float(ru[i][w] & 0xFFFF0000u));
+      sv[i][2 * w] = __uint_as_float(p2 << 16);
+      sv[i][2 * w + 1] = __uint_as_float(p2 & 0xFFFF0000u);
+    }
+    had32(sv[i], had_t + 8 * g, tid);
+  }
+  had_tail<T>(sv, NV, q, scale, row, N);
+}
+#define HAD_SMQ_LUT(name, T)                                                                                      \
+  extern "C" __global__ __launch_bounds__(T) void name(                                                          \
+      const unsigned short *__restrict__ gu, unsigned char *__restrict__ q, float *__restrict__ scale, int N,    \
+      const float *__restrict__ had_t, const unsigned short *__restrict__ lut) {                                 \
+    had_silu_lut_body<T>(gu, q, scale, N, had_t, lut);                                                           \
+  }
+HAD_SMQ_LUT(silu_mul_quant_hadi8_lut_t256, 256)
+HAD_SMQ_LUT(silu_mul_quant_hadi8_lut_t512, 512)
+#undef HAD_SMQ_LUT
 
 #define HAD_Q(name, T)                                                                                            \
   extern "C" __global__ __launch_bounds__(T) void name(const unsigned short *__restrict__ x,                     \

@@ -129,6 +129,7 @@ def lib():
         L.saber_iu8_mlp_chain.argtypes = [C.c_void_p] * 10 + [C.c_uint32] * 4 + [C.c_void_p]
         L.saber_iu8_quant_had.argtypes = [C.c_void_p] * 4 + [C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p]
         L.saber_iu8_silu_mul_quant_had.argtypes = [C.c_void_p] * 4 + [C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p]
+        L.saber_iu8_silu_mul_quant_had_lut.argtypes = [C.c_void_p] * 4 + [C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p]
         L.saber_iu8_add_rms_quant_had.argtypes = [C.c_void_p] * 7 + [C.c_uint32, C.c_uint32, C.c_float, C.c_void_p, C.c_void_p]
         L.saber_iu8_gdn_norm_quant_had.argtypes = [C.c_void_p] * 3 + [C.c_int64] + [C.c_void_p] * 3 + [
             C.c_uint32, C.c_uint32, C.c_float, C.c_void_p, C.c_void_p]
@@ -417,6 +418,9 @@ class Context:
 
     def silu_mul_quant_had(self, gu, q, scale, m, n, had_t, stream=0):
         _check(lib().saber_iu8_silu_mul_quant_had(self._h, gu, q, scale, m, n, had_t, stream))
+
+    def silu_mul_quant_had_lut(self, gu, q, scale, m, n, had_t, silu_lut, stream=0):
+        _check(lib().saber_iu8_silu_mul_quant_had_lut(self._h, gu, q, scale, m, n, had_t, silu_lut, stream))
 
     def add_rms_quant_had(self, y, res, w, q, scale, res_out, m, k, eps, had_t, stream=0):
         _check(lib().saber_iu8_add_rms_quant_had(self._h, y, res, w, q, scale, res_out, m, k, eps, had_t, stream))

@@ -177,3 +177,32 @@ def test_quant_ties_and_near_ties_round_like_the_ieee_divide(ctx):
         ctx.linear_fused(iu8.W4, xs.data_ptr(), wf.data_ptr(), wsd.data_ptr(), c.data_ptr(), 4, 64, K, q=q4.data_ptr(), scale=s4.data_ptr())
         torch.cuda.synchronize()
         np.testing.assert_array_equal(iu8.unpack_a(q4.cpu().numpy(), 4, K), want_q[r0:r0 + 4])
+
+
+@pytest.mark.parametrize("K", [1024, 5120, 17408, 24576])
+def test_quant_rows_with_nan_and_infinity(ctx, K):
+    """Rows that hold NaNs and infinities, on every register-width form of the producer (one, two, five
+    and eight groups a thread): the row maximum passes a NaN over, a NaN's code is -127, an infinite
+    maximum makes the scale infinite (finite elements 0, the infinities themselves -127)."""
+    say(f"quant nan/inf K={K}")
+    rng = np.random.default_rng(K)
+    M = 12
+    X = synth.f32_to_bf16_bits((rng.standard_normal((M, K)) * 3).astype(np.float32))
+    nan, pinf, ninf = 0x7FC0, 0x7F80, 0xFF80
+    X[1, 17] = nan                                  # a lone NaN
+    X[2, K - 1] = pinf                              # an infinity in the row's last group
+    X[3, 0], X[3, 1] = nan, ninf                    # both in one pair
+    X[4, :] = nan                                   # nothing but NaNs: the maximum stays 0
+    X[5, 4096 % K] = 0xFFC1                         # a negative NaN with a payload
+    X[6, K // 2], X[6, K // 2 + 9] = 0x7F81, 0x7F7F  # a signalling pattern beside the largest finite value
+    X[7, np.arange(0, K, 257)] = nan                # a NaN in many threads' groups
+    want_q, want_s = ref.quant_bf16(X)
+    x = dev_bf16_bits(X)
+    for rm in (False, True):
+        q = torch.zeros(M * K if rm else iu8.a_bytes(M, K), dtype=torch.uint8, device="cuda")
+        s = torch.zeros(M, dtype=torch.float32, device="cuda")
+        (ctx.quant_rowmajor if rm else ctx.quant)(x.data_ptr(), q.data_ptr(), s.data_ptr(), M, K)
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(s.cpu().numpy().view(np.uint32), want_s.view(np.uint32))
+        got = q.cpu().numpy().view(np.int8).reshape(M, K) if rm else iu8.unpack_a(q.cpu().numpy(), M, K)
+        np.testing.assert_array_equal(got, want_q)

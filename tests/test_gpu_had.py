@@ -46,6 +46,34 @@ def test_silu_mul_quant_had(ctx, M, N):
     np.testing.assert_array_equal(iu8.unpack_a(q.cpu().numpy(), M, N), wq)
 
 
+@pytest.mark.parametrize("M,N", [(2, 2048), (130, 6144), (33, 10240), (70, 10304), (523, 17408), (19, 20480), (77, 64), (40, 1536)])
+def test_silu_mul_quant_had_table_form(ctx, M, N):
+    """For rows of SABER_IU8_SILU_LUT_MIN_WIDTH elements and more the launch reads the bf16 silu from the middle
+    of the caller's table (both thread counts a row, one to five groups a thread, full and ragged; gates
+    outside the table's range -- infinities, NaN, zeros, denormals, huge values -- take the computed branch);
+    narrower rows are the computed form. The oracle's bytes either way."""
+    say(f"silu_mul_quant_had_lut M={M} N={N}")
+    rng = np.random.default_rng(M + N)
+    gu = synth.f32_to_bf16_bits((rng.standard_normal((M, 2 * N)) * 2).astype(np.float32))
+    gu[M // 2, :8] = [0x7F80, 0xFF80, 0x7FC0, 0x0000, 0x8000, 0x7F7F, 0xFF7F, 0x0001]   # gate: inf, -inf, NaN, zeros, extremes
+    gu[0, 8:16] = [0x36FF, 0x3700, 0xB6FF, 0xB700, 0x46FF, 0x4700, 0xC6FF, 0xC700]     # both sides of the table's two edges
+    t = (rng.choice([-1.0, 1.0], size=N) * rng.uniform(0.5, 2.0, size=N)).astype(np.float32)
+    q, s = outs(M, N)
+    lut = torch.zeros(65536, dtype=torch.int16, device="cuda")
+    ctx.silu_table(lut.data_ptr())
+    gd, td = dev_bf16_bits(gu), dev_f32(t)
+    ctx.silu_mul_quant_had_lut(gd.data_ptr(), q.data_ptr(), s.data_ptr(), M, N, td.data_ptr(), lut.data_ptr())
+    torch.cuda.synchronize()
+    wq, wsc = ref.silu_mul_quant_had(gu, t)
+    np.testing.assert_array_equal(s.cpu().numpy().view(np.uint32), wsc.view(np.uint32))
+    np.testing.assert_array_equal(iu8.unpack_a(q.cpu().numpy(), M, N), wq)
+    # ... and the computed form's bytes, whichever of the two the row count picked
+    q2, s2 = outs(M, N)
+    ctx.silu_mul_quant_had(gd.data_ptr(), q2.data_ptr(), s2.data_ptr(), M, N, td.data_ptr())
+    torch.cuda.synchronize()
+    assert torch.equal(q, q2) and torch.equal(s.view(torch.int32), s2.view(torch.int32))
+
+
 @pytest.mark.parametrize("M,K", [(3, 256), (20, 5120), (9, 17408)])
 def test_add_rms_quant_had(ctx, M, K):
     say(f"add_rms_quant_had M={M} K={K}")
