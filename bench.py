@@ -660,6 +660,8 @@ def main():
             core, blk = bf16(PM, Kh), bf16(PM, 2 * Kh, scale=3.0)
             silu_lut = torch.zeros(65536, dtype=torch.int16, device=dev)
             ctx.silu_table(silu_lut.data_ptr(), sh)
+            sig_lut = torch.zeros(65536, dtype=torch.int16, device=dev)
+            ctx.sigmoid_table(sig_lut.data_ptr(), sh)
             cases = {
                 "quant_had_k5120": (lambda: ctx.quant_had(xk.data_ptr(), q.data_ptr(), sc.data_ptr(), PM, Kh, t_k.data_ptr(), sh),
                                     PM * (3 * Kh + 4)),
@@ -674,6 +676,9 @@ def main():
                 "gdn_norm_quant_had_n6144": (lambda: ctx.gdn_norm_quant_had(xg.data_ptr(), zg.data_ptr(), Ng, wg.data_ptr(), q.data_ptr(), sc.data_ptr(),
                                                                             PM, Ng, 1e-6, t_k.data_ptr(), sh),
                                              PM * (5 * Ng + 4)),
+                "attn_gate_quant_had_lut_n5120": (lambda: ctx.attn_gate_quant_had_lut(core.data_ptr(), blk.data_ptr(), q.data_ptr(), sc.data_ptr(), PM,
+                                                                                      Kh, hd, 2 * Kh, t_k.data_ptr(), sig_lut.data_ptr(), sh),
+                                                  PM * (5 * Kh + 4)),
                 "attn_gate_quant_had_n5120": (lambda: ctx.attn_gate_quant_had(core.data_ptr(), blk.data_ptr(), q.data_ptr(), sc.data_ptr(), PM, Kh, hd,
                                                                               2 * Kh, t_k.data_ptr(), sh),
                                               PM * (5 * Kh + 4)),
@@ -694,8 +699,7 @@ def main():
                 row[name] = dict(us=round(us, 2), bytes=int(nbytes), gbps=round(nbytes / us / 1e3, 1), hbm_frac=round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4))
             prod["m%d" % PM] = row
         prod["note"] = ("one launch a producer, back to back on one stream (inputs of the decode rows stay in the caches: those lines are launch latency, "
-                        "not bandwidth); bytes = bf16 rows in + codes + scales (+ the residual row out); silu_mul_quant_had_lut = the same op with "
-                        "the caller's table of the bf16 silu at hand")
+                        "not bandwidth); bytes = bf16 rows in + codes + scales (+ the residual row out); *_lut = the same op with the caller's table of its gate at hand")
         out["hadamard_producers"] = prod
     print(json.dumps(out), flush=True)
     ctx.close()

@@ -277,6 +277,17 @@ int saber_iu8_silu_mul_quant_had(saber_iu8_ctx *ctx, const void *gu_bf16, void *
 #define SABER_IU8_SILU_LUT_MIN_WIDTH 2048u
 int saber_iu8_silu_mul_quant_had_lut(saber_iu8_ctx *ctx, const void *gu_bf16, void *q, float *scale, uint32_t m, uint32_t n,
                                      const float *had_t, const uint16_t *silu_lut, void *stream);
+/* The attention output gate's producer the same way: saber_iu8_sigmoid_table writes bf16(sigmoid) of every bf16
+ * pattern (u16 [65536], 128 KiB, the kernel's own expression: crates/saber-kernels/hip/attn_glue_hadi8.hip:23-79);
+ * with it saber_iu8_attn_gate_quant_had_lut launches attn_gate_quant_hadi8_lut_t256 for rows of
+ * SABER_IU8_SILU_LUT_MIN_WIDTH elements and more, from SABER_IU8_SIGMOID_LUT_MIN_ROWS rows on (below, the copy of
+ * the table's middle costs more than the few rows' exps). The GDN norm's f32 gate was tabled too and did not
+ * gain: that kernel is not bound by its gate. */
+#define SABER_IU8_SIGMOID_LUT_MIN_ROWS 1024u
+int saber_iu8_sigmoid_table(saber_iu8_ctx *ctx, void *out_u16, void *stream);
+int saber_iu8_attn_gate_quant_had_lut(saber_iu8_ctx *ctx, const void *core_bf16, const void *gate_bf16, void *q, float *scale,
+                                      uint32_t m, uint32_t n, uint32_t head_dim, uint32_t gate_stride, const float *had_t,
+                                      const uint16_t *sigmoid_lut, void *stream);
 int saber_iu8_add_rms_quant_had(saber_iu8_ctx *ctx, const void *y_bf16, const void *res_bf16, const void *w_bf16, void *q,
                                 float *scale, void *res_out_bf16, uint32_t m, uint32_t k, float eps, const float *had_t,
                                 void *stream);

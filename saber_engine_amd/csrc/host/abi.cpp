@@ -48,6 +48,9 @@ static const Signature SIG_HAD_GNQ = {{"x", K::Buffer}, {"z", K::Buffer},     {"
                                       {"had_t", K::Buffer}};
 static const Signature SIG_HAD_AGQ = {{"core", K::Buffer}, {"gate", K::Buffer}, {"q", K::Buffer}, {"scale", K::Buffer},
                                       {"n", K::I32},       {"hd", K::I32},      {"gs", K::I32},   {"had_t", K::Buffer}};
+static const Signature SIG_HAD_AGQ_LUT = {{"core", K::Buffer}, {"gate", K::Buffer}, {"q", K::Buffer}, {"scale", K::Buffer},
+                                          {"n", K::I32},       {"hd", K::I32},      {"gs", K::I32},   {"had_t", K::Buffer},
+                                          {"lut", K::Buffer}};
 static const Signature SIG_SILU = {{"gu", K::Buffer}, {"q", K::Buffer},       {"scale", K::Buffer},
                                    {"n", K::I32},     {"row_tok", K::Buffer}, {"meta", K::Buffer}};
 static const Signature SIG_SILU_LUT = {{"gu", K::Buffer}, {"q", K::Buffer},       {"scale", K::Buffer}, {"n", K::I32},
@@ -93,8 +96,10 @@ const Signature *signature_for(const std::string &k) {
   if (starts(k, "silu_mul_quant_hadi8_")) return &SIG_HAD_SMQ;
   if (starts(k, "quant_hadi8_")) return &SIG_HAD_Q;
   if (starts(k, "gdn_norm_quant_hadi8_")) return &SIG_HAD_GNQ;
+  if (starts(k, "attn_gate_quant_hadi8_lut_")) return &SIG_HAD_AGQ_LUT;
   if (starts(k, "attn_gate_quant_hadi8_")) return &SIG_HAD_AGQ;
   if (k == "mxfp4_hadi8_silu_f32_table" || k == "attn_glue_hadi8_sigmoid_bf16_table") return &SIG_TABLE;
+  if (k == "attn_gate_sigmoid_bf16_table") return &SIG_TABLE;
   if (starts(k, "macaq_i8_quant_rows_")) return &SIG_QUANT_ROWS;
   if (starts(k, "macaq_i8_quant_")) return &SIG_QUANT;
   if (starts(k, "macaq_i8_silu_mul_quant_lut_")) return &SIG_SILU_LUT;

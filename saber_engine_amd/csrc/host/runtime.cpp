@@ -646,8 +646,8 @@ int saber_iu8_gdn_norm_quant_had(saber_iu8_ctx *ctx, const void *x, const void *
 
 // attn_gate: the reference's t256 form holds rows of at most 6,144 elements (3 groups of 8 a thread,
 // crates/saber-kernels/hip/attn_glue_hadi8.hip:33); heads of `hd` elements, a multiple of 8.
-int saber_iu8_attn_gate_quant_had(saber_iu8_ctx *ctx, const void *core, const void *gate, void *q, float *scale, uint32_t m,
-                                  uint32_t n, uint32_t head_dim, uint32_t gate_stride, const float *had_t, void *stream) {
+static int attn_gate_launch(saber_iu8_ctx *ctx, const void *core, const void *gate, void *q, float *scale, uint32_t m, uint32_t n,
+                            uint32_t head_dim, uint32_t gate_stride, const float *had_t, const uint16_t *lut, void *stream) {
   if (m == 0 || n == 0) return fail(SABER_IU8_E_RULE, fmt("attn_gate_quant_had_i8: %u rows of %u has nothing to do", m, n));
   if (n % 64 != 0 || n > 6144)
     return fail(SABER_IU8_E_RULE, fmt("attn_gate_quant_had_i8: row width %u must be a multiple of 64, at most 6144", n));
@@ -657,13 +657,24 @@ int saber_iu8_attn_gate_quant_had(saber_iu8_ctx *ctx, const void *core, const vo
     return fail(SABER_IU8_E_RULE, fmt("attn_gate_quant_had_i8: gate stride %u must cover the [q | gate] block of %u in whole 16-byte pieces", gate_stride, 2 * n));
   saber_iu8_desc d;
   const uint32_t grid[3] = {m, 1, 1};
-  if (int rc = saber_iu8_describe_raw("attn_gate_quant_hadi8_t256_tiled1", "attn_glue_hadi8", grid, 256, &d)) return rc;
+  if (int rc = saber_iu8_describe_raw(lut ? "attn_gate_quant_hadi8_lut_t256" : "attn_gate_quant_hadi8_t256_tiled1", "attn_glue_hadi8", grid, 256, &d)) return rc;
   snprintf(d.op, sizeof d.op, "attn_gate_quant_had_i8");
   set_i32(&d, "n", n);
   set_i32(&d, "hd", head_dim);
   set_i32(&d, "gs", gate_stride);
-  const saber_iu8_binding b[] = {{"core", (void *)core}, {"gate", (void *)gate}, {"q", q}, {"scale", scale}, {"had_t", (void *)had_t}};
-  return saber_iu8_launch(ctx, &d, b, 5, stream);
+  const saber_iu8_binding b[] = {{"core", (void *)core}, {"gate", (void *)gate}, {"q", q}, {"scale", scale}, {"had_t", (void *)had_t},
+                                 {"lut", (void *)lut}};
+  return saber_iu8_launch(ctx, &d, b, lut ? 6 : 5, stream);
+}
+int saber_iu8_attn_gate_quant_had(saber_iu8_ctx *ctx, const void *core, const void *gate, void *q, float *scale, uint32_t m,
+                                  uint32_t n, uint32_t head_dim, uint32_t gate_stride, const float *had_t, void *stream) {
+  return attn_gate_launch(ctx, core, gate, q, scale, m, n, head_dim, gate_stride, had_t, nullptr, stream);
+}
+int saber_iu8_attn_gate_quant_had_lut(saber_iu8_ctx *ctx, const void *core, const void *gate, void *q, float *scale, uint32_t m,
+                                      uint32_t n, uint32_t head_dim, uint32_t gate_stride, const float *had_t,
+                                      const uint16_t *sigmoid_lut, void *stream) {
+  const bool pays = n >= SABER_IU8_SILU_LUT_MIN_WIDTH && m >= SABER_IU8_SIGMOID_LUT_MIN_ROWS;
+  return attn_gate_launch(ctx, core, gate, q, scale, m, n, head_dim, gate_stride, had_t, pays ? sigmoid_lut : nullptr, stream);
 }
 
 // ---------------------------------------------------------------------------- routed experts
@@ -913,6 +924,17 @@ int saber_iu8_moe_combine(saber_iu8_ctx *ctx, const void *y, const saber_iu8_moe
   const saber_iu8_binding b[] = {{"y", (void *)y},   {"topk_w", t->topk_w}, {"route_pos", t->route_pos},
                                  {"meta", t->meta}, {"out", out},          {"sgate", (void *)t->sgate}};
   return saber_iu8_launch(ctx, &d, b, t->sgate ? 6 : 5, stream);
+}
+
+static int table_launch(saber_iu8_ctx *ctx, const char *kernel, const char *plugin, void *out, void *stream) {
+  saber_iu8_desc d;
+  const uint32_t grid[3] = {256, 1, 1};
+  if (int rc = saber_iu8_describe_raw(kernel, plugin, grid, 256, &d)) return rc;
+  const saber_iu8_binding b[] = {{"out", out}};
+  return saber_iu8_launch(ctx, &d, b, 1, stream);
+}
+int saber_iu8_sigmoid_table(saber_iu8_ctx *ctx, void *out, void *stream) {
+  return table_launch(ctx, "attn_gate_sigmoid_bf16_table", "attn_glue_hadi8", out, stream);
 }
 
 int saber_iu8_silu_table(saber_iu8_ctx *ctx, void *out, void *stream) {

@@ -13,13 +13,32 @@
 // tap kernel of the test-only object `iu8_taps` tables.
 #include "iu8_had.h"
 
-extern "C" __global__ __launch_bounds__(256) void attn_gate_quant_hadi8_t256_tiled1(
-    const unsigned short *__restrict__ core, const unsigned short *__restrict__ gate, unsigned char *__restrict__ q,
-    float *__restrict__ scale, int n, int hd, int gs, const float *__restrict__ had_t) {
+// `lut` (the table form, may be null): bf16(sigmoid) of every bf16 pattern as attn_gate_sigmoid_bf16_table wrote
+// it; the gate is then read from the table's middle in LDS (iu8_had.h) instead of computed.
+template <bool LUT>
+static __device__ __forceinline__ void attn_gate_body(const unsigned short *__restrict__ core,
+                                                      const unsigned short *__restrict__ gate, unsigned char *__restrict__ q,
+                                                      float *__restrict__ scale, int n, int hd, int gs,
+                                                      const float *__restrict__ had_t,
+                                                      const unsigned short *__restrict__ lut) {
 #pragma clang fp contract(off)
   constexpr int T = 256;
   const int row = had_row(), tid = threadIdx.x, NV = n >> 3;
   core += (size_t)row * n, gate += (size_t)row * gs;
+  __shared__ __attribute__((aligned(16))) unsigned short s_lut[LUT ? 2 * HAD_LUT_N : 8];
+  if constexpr (LUT) {
+    had_lut_copy<unsigned short, T> tb;
+    tb.request(lut, tid);
+    tb.commit(s_lut, tid);
+    __syncthreads();
+  }
+  auto sig = [&](float g) {
+    if constexpr (LUT) {
+      unsigned at;
+      if (__builtin_expect(had_lut_index(__float_as_uint(g) >> 16, at), 1)) return iu8_bf16_f32(s_lut[at]);
+    }
+    return glue_sigmoid_bf16(g);
+  };
   float sv[HAD_MAXG][8];
 #pragma unroll
   for (int i = 0; i < HAD_MAXG; ++i) {
@@ -30,9 +49,26 @@ extern "C" __global__ __launch_bounds__(256) void attn_gate_quant_hadi8_t256_til
     had_load8(core + e, vc);
     had_load8(gate + (size_t)h * 2 * hd + hd + o, vg);
 #pragma unroll
-    for (int j = 0; j < 8; ++j)
-      sv[i][j] = iu8_bf16_f32((unsigned short)iu8_bf16_bits(vc[j] * glue_sigmoid_bf16(vg[j])));
+    for (int j = 0; j < 8; ++j) sv[i][j] = iu8_bf16_f32((unsigned short)iu8_bf16_bits(vc[j] * sig(vg[j])));
     had32(sv[i], had_t + 8 * g, tid);
   }
   had_tail<T>(sv, NV, q, scale, row, n);
+}
+extern "C" __global__ __launch_bounds__(256) void attn_gate_quant_hadi8_t256_tiled1(
+    const unsigned short *__restrict__ core, const unsigned short *__restrict__ gate, unsigned char *__restrict__ q,
+    float *__restrict__ scale, int n, int hd, int gs, const float *__restrict__ had_t) {
+  attn_gate_body<false>(core, gate, q, scale, n, hd, gs, had_t, nullptr);
+}
+// the table form (no counterpart among the reference's symbols: `lut` behind its kernarg list)
+extern "C" __global__ __launch_bounds__(256) void attn_gate_quant_hadi8_lut_t256(
+    const unsigned short *__restrict__ core, const unsigned short *__restrict__ gate, unsigned char *__restrict__ q,
+    float *__restrict__ scale, int n, int hd, int gs, const float *__restrict__ had_t,
+    const unsigned short *__restrict__ lut) {
+  attn_gate_body<true>(core, gate, q, scale, n, hd, gs, had_t, lut);
+}
+// bf16(sigmoid) of all 65,536 bf16 inputs (bf16 bits [65536]): the table of attn_gate_quant_hadi8_lut_t256.
+// grid 256, block 256.
+extern "C" __global__ __launch_bounds__(256) void attn_gate_sigmoid_bf16_table(unsigned short *__restrict__ out) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  out[i] = (unsigned short)iu8_bf16_bits(glue_sigmoid_bf16(iu8_bf16_f32((unsigned short)i)));
 }

@@ -118,3 +118,35 @@ static __device__ __forceinline__ float glue_sigmoid_bf16(float g) {
 #pragma clang fp contract(off)
   return iu8_bf16_f32((unsigned short)iu8_bf16_bits(1.f / (1.f + expf(-g))));
 }
+
+// A table of a gate over all 65,536 bf16 bit patterns (bf16 or f32 entries, as a table kernel of these
+// objects wrote it with the gate's own expression) serves a producer through its middle: the patterns of
+// magnitudes 2^-17 up to 2^15, both signs, 2 x HAD_LUT_N entries, which a workgroup copies into LDS (16 KiB of
+// bf16 entries, 32 KiB of f32). A lookup returns the computed gate's bits by construction; a pattern
+// outside (zeros, denormals, huge values, infinities, NaN: one in some hundred thousand of unit-scale
+// values) is computed.
+#define HAD_LUT_LO (110 << 7)  // first pattern without sign in the table: 2^-17
+#define HAD_LUT_N 4096         // patterns a sign: 32 exponents
+// requests this thread's 16-byte pieces of the middle (T threads; E = unsigned short or float)
+template <class E, int T>
+struct had_lut_copy {
+  static constexpr int PER = 16 / sizeof(E), NP = 2 * HAD_LUT_N / PER / T;
+  iu8_v4u tb[NP];
+  __device__ __forceinline__ void request(const E *__restrict__ lut, int tid) {
+#pragma unroll
+    for (int c = 0; c < NP; ++c) {
+      const int i = (c * T + tid) * PER;  // entry: sign i / HAD_LUT_N, pattern HAD_LUT_LO + i % HAD_LUT_N
+      tb[c] = *(const iu8_v4u *)(lut + (i / HAD_LUT_N) * 32768 + HAD_LUT_LO + (i & (HAD_LUT_N - 1)));
+    }
+  }
+  __device__ __forceinline__ void commit(E *s_lut, int tid) const {  // the caller's barrier follows
+#pragma unroll
+    for (int c = 0; c < NP; ++c) ((iu8_v4u *)s_lut)[c * T + tid] = tb[c];
+  }
+};
+// the LDS index of pattern b (low 16 bits), or false when b is outside the middle
+static __device__ __forceinline__ bool had_lut_index(unsigned b, unsigned &at) {
+  const unsigned idx = (b & 0x7FFFu) - HAD_LUT_LO;
+  at = ((b >> 15) << 12) | idx;
+  return idx < (unsigned)HAD_LUT_N;
+}

@@ -150,8 +150,6 @@ HAD_SMQ(silu_mul_quant_hadi8_t512_tiled1, 512)
 // its row's loads; a gate outside (one in some hundred thousand of unit-scale rows) is computed as before.
 // The kernel is the computed form otherwise (a workgroup a row, the same lane map). No counterpart among
 // the reference's symbols (`lut` behind its kernarg list).
-#define HAD_LUT_LO (110 << 7)  // first pattern without sign in the table: 2^-17
-#define HAD_LUT_N 4096         // patterns a sign: 32 exponents
 template <int T>
 static __device__ __forceinline__ void had_silu_lut_body(const unsigned short *__restrict__ gu, iu8_u8 *__restrict__ q,
                                                          float *__restrict__ scale, int N,
@@ -162,24 +160,20 @@ static __device__ __forceinline__ void had_silu_lut_body(const unsigned short *_
   const int row = had_row(), tid = threadIdx.x, NV = N >> 3;
   gu += (size_t)row * 2 * N;
   // the row's pieces and the table are requested together, nothing is used before the last request has left
-  iu8_v4u rg[HAD_MAXG], ru[HAD_MAXG], tb[2 * HAD_LUT_N / 8 / T];
+  iu8_v4u rg[HAD_MAXG], ru[HAD_MAXG];
+  had_lut_copy<unsigned short, T> tb;
 #pragma unroll
   for (int i = 0; i < HAD_MAXG; ++i) {
     const int g = tid + i * T;
     rg[i] = ru[i] = iu8_v4u{0u, 0u, 0u, 0u};
     if (g < NV) rg[i] = *(const iu8_v4u *)(gu + (unsigned)(g * 8)), ru[i] = *(const iu8_v4u *)(gu + N + (unsigned)(g * 8));
   }
-#pragma unroll
-  for (int c = 0; c < 2 * HAD_LUT_N / 8 / T; ++c) {
-    const int i = (c * T + tid) * 8;  // entry: sign i / HAD_LUT_N, pattern HAD_LUT_LO + i % HAD_LUT_N
-    tb[c] = *(const iu8_v4u *)(lut + (i / HAD_LUT_N) * 32768 + HAD_LUT_LO + (i & (HAD_LUT_N - 1)));
-  }
-#pragma unroll
-  for (int c = 0; c < 2 * HAD_LUT_N / 8 / T; ++c) ((iu8_v4u *)s_lut)[c * T + tid] = tb[c];
+  tb.request(lut, tid);
+  tb.commit(s_lut, tid);
   __syncthreads();
   auto silu = [&](unsigned b) {  // bf16 pattern (low 16 bits) -> bf16(silu) as f32
-    const unsigned idx = (b & 0x7FFFu) - HAD_LUT_LO;
-    if (__builtin_expect(idx < (unsigned)HAD_LUT_N, 1)) return iu8_bf16_f32(s_lut[((b >> 15) << 12) | idx]);
+    unsigned at;
+    if (__builtin_expect(had_lut_index(b, at), 1)) return iu8_bf16_f32(s_lut[at]);
     const float x = iu8_bf16_f32((unsigned short)b);
     return iu8_bf16_f32((unsigned short)iu8_bf16_bits(x / (1.f + expf(-x))));
   };

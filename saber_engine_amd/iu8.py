@@ -134,6 +134,8 @@ def lib():
         L.saber_iu8_gdn_norm_quant_had.argtypes = [C.c_void_p] * 3 + [C.c_int64] + [C.c_void_p] * 3 + [
             C.c_uint32, C.c_uint32, C.c_float, C.c_void_p, C.c_void_p]
         L.saber_iu8_attn_gate_quant_had.argtypes = [C.c_void_p] * 5 + [C.c_uint32] * 4 + [C.c_void_p, C.c_void_p]
+        L.saber_iu8_attn_gate_quant_had_lut.argtypes = [C.c_void_p] * 5 + [C.c_uint32] * 4 + [C.c_void_p, C.c_void_p, C.c_void_p]
+        L.saber_iu8_sigmoid_table.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
         L.saber_iu8_get_counters.argtypes = [C.c_void_p, C.POINTER(Counters)]
         L.saber_iu8_has_kernel.argtypes = [C.c_void_p, C.c_char_p]
         for fn in ("saber_iu8_moe_rows_cap", "saber_iu8_moe_rows_cap_shared", "saber_iu8_moe_tile_blocks"):
@@ -430,6 +432,12 @@ class Context:
 
     def attn_gate_quant_had(self, core, gate, q, scale, m, n, head_dim, gate_stride, had_t, stream=0):
         _check(lib().saber_iu8_attn_gate_quant_had(self._h, core, gate, q, scale, m, n, head_dim, gate_stride, had_t, stream))
+
+    def attn_gate_quant_had_lut(self, core, gate, q, scale, m, n, head_dim, gate_stride, had_t, sigmoid_lut, stream=0):
+        _check(lib().saber_iu8_attn_gate_quant_had_lut(self._h, core, gate, q, scale, m, n, head_dim, gate_stride, had_t, sigmoid_lut, stream))
+
+    def sigmoid_table(self, out, stream=0):
+        _check(lib().saber_iu8_sigmoid_table(self._h, out, stream))
 
     def gemm_acc(self, wkind, a, w, acc, m, n, k, stream=0):
         _check(lib().saber_iu8_gemm_acc(self._h, wkind, a, w, acc, m, n, k, stream))

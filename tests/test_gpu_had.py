@@ -148,6 +148,32 @@ def test_gdn_norm_quant_had(ctx, M, H, zs_pad):
     np.testing.assert_array_equal(iu8.unpack_a(q.cpu().numpy(), M, N), wq)
 
 
+@pytest.mark.parametrize("M,H,hd,pad", [(1033, 24, 256, 0), (1024, 16, 128, 96), (1100, 48, 128, 0), (1030, 8, 128, 0), (40, 40, 128, 0)])
+def test_attn_gate_quant_had_table_form(ctx, M, H, hd, pad):
+    """The gate read from the middle of the product's own table (saber_iu8_sigmoid_table), gates outside it
+    computed; narrow rows and few rows take the computed kernel. The computed form's bytes and the oracle's."""
+    n = H * hd
+    say(f"attn_gate_quant_had_lut M={M} n={n} hd={hd} gate stride {2 * n + pad}")
+    rng = np.random.default_rng(M + n + hd + 1)
+    core = synth.f32_to_bf16_bits(rng.standard_normal((M, n)).astype(np.float32))
+    block = synth.f32_to_bf16_bits((rng.standard_normal((M, 2 * n + pad)) * 3).astype(np.float32))
+    block[M // 2, hd:hd + 12] = [0x7F80, 0xFF80, 0x7FC0, 0x0000, 0x8000, 0x7F7F, 0xFF7F, 0x0001, 0x36FF, 0x3700, 0xC6FF, 0xC700]
+    t = rng.choice([-1.0, 1.0], size=n).astype(np.float32)
+    lut = torch.zeros(65536, dtype=torch.int16, device="cuda")
+    ctx.sigmoid_table(lut.data_ptr())
+    cd, gd, td = dev_bf16_bits(core), dev_bf16_bits(block), dev_f32(t)
+    q, s = outs(M, n)
+    ctx.attn_gate_quant_had_lut(cd.data_ptr(), gd.data_ptr(), q.data_ptr(), s.data_ptr(), M, n, hd, 2 * n + pad, td.data_ptr(),
+                                lut.data_ptr())
+    q2, s2 = outs(M, n)
+    ctx.attn_gate_quant_had(cd.data_ptr(), gd.data_ptr(), q2.data_ptr(), s2.data_ptr(), M, n, hd, 2 * n + pad, td.data_ptr())
+    torch.cuda.synchronize()
+    assert torch.equal(q, q2) and torch.equal(s.view(torch.int32), s2.view(torch.int32))
+    wq, wsc = ref.attn_gate_quant_had(core, block, t, hd)
+    np.testing.assert_array_equal(s.cpu().numpy().view(np.uint32), wsc.view(np.uint32))
+    np.testing.assert_array_equal(iu8.unpack_a(q.cpu().numpy(), M, n), wq)
+
+
 @pytest.mark.parametrize("M,H,hd,pad", [(1, 1, 64, 0), (9, 24, 256, 0), (140, 16, 128, 96), (2, 48, 128, 0)])
 def test_attn_gate_quant_had(ctx, M, H, hd, pad):
     n = H * hd
