@@ -32,7 +32,7 @@ LAYERS = 6                  # distinct weight copies walked by successive steps 
 # command (FETCH_SIZE, then WRITE_SIZE), each counter scaled by what it reads for the 256 MiB copy
 # probe, and is kept in the profile summary named below. Keyed by (kernel, M); None = not measured.
 TRAFFIC_SOURCE = "profiles/macaq_iu8_decq_w4_tm1__layer_set_m1.txt"
-TRAFFIC = {("macaq_iu8_decq_w4_tm1", 1): 41735812.0, ("macaq_iu8_dec_w4_tm1", 1): 41993981.0}
+TRAFFIC = {("macaq_iu8_decq_w4_tm1", 1): 41737825.0, ("macaq_iu8_dec_w4_tm1", 1): 41995646.0}
 
 
 def alg_bytes(m, n, k, w8=False):
