@@ -16,7 +16,9 @@
 // shfl_down 16..1 inside each 32 lanes, then over the T/32 partials; gdn_norm per group
 // (x1*x1, fma x0, fma x2..x7), then the xor butterfly 8, 4, 2, 1 over the head's 16 lanes. Their
 // `rsqrtf` is the one thing not taken over: the device's approximate reciprocal square root cannot be
-// restated on a host, so inv = 1 / sqrt(x) here uses the IEEE square root and divide. gdn_norm's
+// restated on a host, so inv = 1 / sqrt(x) here uses the IEEE square root and divide (`__builtin_sqrtf`, which
+// this toolchain expands to the correctly rounded sequence; its `__fsqrt_rn` is the native approximation, an
+// ulp off now and then, which showed as a bf16 value of a row flipped once in a few million elements). gdn_norm's
 // gate silu_f32(z) = z / (1 + expf(-z)) stays in f32 and so carries the device's expf: a function of
 // a bf16 input, it is tabled by a tap kernel of the test-only object `iu8_taps` (had_silu_f32 lives
 // in iu8_had.h for both) for a checker to hold against a host's.
@@ -106,7 +108,7 @@ static __device__ __forceinline__ void had_add_rms_body(const unsigned short *__
     if (tid == 0) s_sum[0] = v;
   }
   __syncthreads();
-  const float inv = __fdiv_rn(1.f, __fsqrt_rn(__fdiv_rn(s_sum[0], (float)K) + eps));
+  const float inv = __fdiv_rn(1.f, __builtin_sqrtf(__fdiv_rn(s_sum[0], (float)K) + eps));
 #pragma unroll
   for (int i = 0; i < HAD_MAXG; ++i) {
     const int g = tid + i * T;
@@ -239,7 +241,7 @@ static __device__ __forceinline__ void had_gdn_norm_body(const unsigned short *_
 #pragma unroll
     for (int o = 8; o; o >>= 1) ssq = ssq + __shfl_xor(ssq, o, 16);
     if (!on) continue;
-    const float inv = __fdiv_rn(1.f, __fsqrt_rn(ssq * (1.f / 128.f) + eps));
+    const float inv = __fdiv_rn(1.f, __builtin_sqrtf(ssq * (1.f / 128.f) + eps));
     had_load8(z + g * 8, vz);
     had_load8(w + (g & 15) * 8, vw);
 #pragma unroll

@@ -94,6 +94,29 @@ def test_add_rms_quant_had(ctx, M, K):
     np.testing.assert_array_equal(iu8.unpack_a(q.cpu().numpy(), M, K), wq)
 
 
+@pytest.mark.parametrize("M,K", [(1024, 20480), (700, 5120)])
+def test_add_rms_quant_had_rows_of_many_magnitudes(ctx, M, K):
+    """Many rows whose sums of squares spread over fifteen orders of magnitude: the square root under `inv` must
+    be the correctly rounded one on every row (an ulp of `inv` flips a bf16 value of the row once in some
+    hundred thousand elements, and with it a code or two of that 32-block)."""
+    say(f"add_rms_quant_had, row magnitudes, M={M} K={K}")
+    rng = np.random.default_rng(K + M)
+    y = synth.f32_to_bf16_bits((rng.standard_normal((M, K)) * np.exp(rng.uniform(-12, 6, size=(M, 1)))).astype(np.float32))
+    r = synth.f32_to_bf16_bits((rng.standard_normal((M, K)) * 4 * np.exp(rng.uniform(-12, 6, size=(M, 1)))).astype(np.float32))
+    w = synth.f32_to_bf16_bits((rng.standard_normal(K) * 0.1).astype(np.float32))
+    t = (rng.choice([-1.0, 1.0], size=K) * rng.uniform(0.5, 2.0, size=K)).astype(np.float32)
+    q, s = outs(M, K)
+    ro = torch.zeros((M, K), dtype=torch.int16, device="cuda")
+    yd, rd, wd, td = dev_bf16_bits(y), dev_bf16_bits(r), dev_bf16_bits(w), dev_f32(t)
+    ctx.add_rms_quant_had(yd.data_ptr(), rd.data_ptr(), wd.data_ptr(), q.data_ptr(), s.data_ptr(), ro.data_ptr(), M, K, 1e-6,
+                          td.data_ptr())
+    torch.cuda.synchronize()
+    wq, wsc, wro = ref.add_rms_quant_had(y, r, w, t, 1e-6, 256 if K <= 10240 else 512)
+    np.testing.assert_array_equal(host_u16(ro), wro)
+    np.testing.assert_array_equal(s.cpu().numpy().view(np.uint32), wsc.view(np.uint32))
+    np.testing.assert_array_equal(iu8.unpack_a(q.cpu().numpy(), M, K), wq)
+
+
 def tap(ctx, kernel, plugin, dtype):
     """A checker's tap kernel: one value for each of the 65,536 bf16 inputs."""
     out = torch.zeros(65536, dtype=dtype, device="cuda")

@@ -1,0 +1,162 @@
+"""Seeded random-shape parity sweeps of the hot path against the CPU oracle, through the C ABI: the dense linear
+with whatever kernel the launch law picks for the shape, the routed layer, and the row producers. Bit-exact,
+like the fixed cases elsewhere; the shapes, magnitudes and special values are drawn so that the corners between
+the hand-picked cases get visited (ragged rows and columns, every regime of M, rows whose magnitudes spread over
+many orders, infinities, NaN, zeros and denormals in the producers' inputs)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import ref
+from saber_engine_amd import iu8, synth
+from tests.gpu_util import DenseRun, assert_dense_matches, dev_bf16_bits, dev_f32, host_u16, say
+from tests.test_gpu_moe import check_layer, run_layer
+
+pytestmark = pytest.mark.gpu
+
+ROWS = [1, 2, 3, 4, 5, 8, 15, 16, 17, 31, 33, 48, 49, 63, 64, 65, 100, 127, 128, 129, 200, 255, 256, 257, 300, 511, 513,
+        700, 1000, 1025, 1500, 2048, 2100, 3000]
+
+
+def test_dense_linear_random_shapes(ctx):
+    rng = np.random.default_rng(20240)
+    for n in range(160):
+        M, w8 = int(rng.choice(ROWS)), bool(rng.integers(0, 2))
+        N, K = int(rng.integers(1, 321)) * 16, int(rng.integers(1, 41)) * 128
+        if rng.random() < 0.2:
+            N = int(rng.choice([5120, 7168, 4352]))
+        if rng.random() < 0.2:
+            K = int(rng.choice([5120, 17408, 1536, 4096]))
+        while M * N * K > 6e9:
+            N = max(16, (N // 2) // 16 * 16)
+        say(f"sweep dense {n}: M={M} N={N} K={K} w8={w8}")
+        case = synth.dense_case(M, N, K, w8=w8, seed=int(rng.integers(0, 1 << 30)))
+        r = ref.linear(case["X"], case["W"], case["ws"], w8, threads=8)
+        run = DenseRun(ctx, case, want_acc=(M <= 64))
+        assert_dense_matches(run, r, w8)
+        if iu8.fused_holds(M, K):      # the fused decode linear on the same operands
+            c = torch.zeros((M, N), dtype=torch.int16, device="cuda")
+            ctx.linear_fused(iu8.W8 if w8 else iu8.W4, run.dev["x"].data_ptr(), run.dev["wf"].data_ptr(), run.dev["ws"].data_ptr(),
+                             c.data_ptr(), M, N, K)
+            torch.cuda.synchronize()
+            np.testing.assert_array_equal(host_u16(c), r["C"])
+
+
+def test_routed_layer_random_shapes(ctx):
+    rng = np.random.default_rng(20241)
+    tokens = [1, 2, 5, 13, 16, 17, 31, 48, 64, 90, 111, 112, 113, 128, 129, 200, 256, 300, 480, 512, 700, 1000, 1500, 2047, 2048, 2500]
+    for n in range(60):
+        T, H, I = int(rng.choice(tokens)), int(rng.choice([256, 512, 640, 1024])), int(rng.choice([128, 256, 384, 512, 1536]))
+        tb = rng.choice([None, None, 1, 8, 16])
+        tb = None if tb is None or (T > 600 and tb == 1) else int(tb)
+        skew = rng.random() < 0.3
+        say(f"sweep routed layer {n}: T={T} H={H} I={I} tile_blocks={tb} skew={skew}")
+        case = synth.moe_case(T=T, E=128, topk=8, H=H, I=I, seed=int(rng.integers(0, 1 << 30)), experts=4)
+        if skew:      # a few hot experts: long tile runs beside many nearly empty tiles
+            lg = synth.bf16_bits_to_f32(case["logits"])
+            lg[:, rng.integers(0, 128, size=3)] += np.float32(rng.uniform(1.0, 5.0))
+            case["logits"] = synth.f32_to_bf16_bits(lg)
+        layer = run_layer(ctx, case, tile_blocks=tb)
+        check_layer(layer, case)
+        del layer
+
+
+def test_row_producers_random_shapes(ctx):
+    rng = np.random.default_rng(20242)
+    tab = torch.zeros(65536, dtype=torch.float32, device="cuda")
+    ctx.launch(iu8.describe_raw("mxfp4_hadi8_silu_f32_table", (256, 1, 1), 256, plugin="mxfp4_hadi8"), dict(out=tab.data_ptr()))
+    silu_lut = torch.zeros(65536, dtype=torch.int16, device="cuda")
+    sig_lut = torch.zeros(65536, dtype=torch.int16, device="cuda")
+    ctx.silu_table(silu_lut.data_ptr())
+    ctx.sigmoid_table(sig_lut.data_ptr())
+    torch.cuda.synchronize()
+    silu_tab = tab.cpu().numpy()      # the GDN norm's f32 gate is the card's own expf: its table goes to the oracle
+
+    def outs(M, K):
+        return (torch.full((iu8.a_bytes(M, K),), 0x55, dtype=torch.uint8, device="cuda"), torch.zeros(M, dtype=torch.float32, device="cuda"))
+
+    def bits(shape, scale):
+        x = (rng.standard_normal(shape) * scale).astype(np.float32)
+        if rng.random() < 0.3:        # rows of very different magnitudes
+            x *= np.exp(rng.uniform(-12, 6, size=(shape[0], 1))).astype(np.float32)
+        b = synth.f32_to_bf16_bits(x)
+        if rng.random() < 0.3:        # a few special patterns
+            b.reshape(-1)[rng.integers(0, b.size, size=6)] = [0x7F80, 0xFF80, 0x7FC0, 0x0000, 0x8000, 0x0001]
+        return b
+
+    def check(q, s, M, K, wq, wsc):
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(s.cpu().numpy().view(np.uint32), wsc.view(np.uint32))
+        np.testing.assert_array_equal(iu8.unpack_a(q.cpu().numpy(), M, K), wq)
+
+    ops = ["quant", "quant_rm", "quant_had", "silu_had", "silu_had_lut", "add_rms", "add_rms", "gdn", "attn", "attn_lut"]
+    for n in range(240):
+        M, K = int(rng.choice([1, 2, 3, 7, 8, 9, 15, 16, 17, 33, 100, 128, 130, 500, 1024, 1030, 2048])), int(rng.integers(1, 321)) * 64
+        if rng.random() < 0.25:
+            K = int(rng.choice([5120, 17408, 1536, 4096, 6144, 20480]))
+        while M * K > 6e6:
+            M = max(1, M // 2)
+        op = str(rng.choice(ops))
+        say(f"sweep producer {n}: {op} M={M} K={K}")
+        t = (rng.choice([-1.0, 1.0], size=K) * rng.uniform(0.5, 2.0, size=K)).astype(np.float32)
+        td = dev_f32(t)
+        q, s = outs(M, K)
+        if op in ("quant", "quant_rm"):
+            X = bits((M, K), 2.0)
+            xd = dev_bf16_bits(X)
+            wq, wsc = ref.quant_bf16(X)
+            if op == "quant":
+                ctx.quant(xd.data_ptr(), q.data_ptr(), s.data_ptr(), M, K)
+                check(q, s, M, K, wq, wsc)
+            else:
+                qr = torch.zeros(M * K, dtype=torch.uint8, device="cuda")
+                ctx.quant_rowmajor(xd.data_ptr(), qr.data_ptr(), s.data_ptr(), M, K)
+                torch.cuda.synchronize()
+                np.testing.assert_array_equal(qr.cpu().numpy().view(np.int8).reshape(M, K), wq)
+                np.testing.assert_array_equal(s.cpu().numpy().view(np.uint32), wsc.view(np.uint32))
+        elif op == "quant_had":
+            X = bits((M, K), 2.0)
+            xd = dev_bf16_bits(X)
+            ctx.quant_had(xd.data_ptr(), q.data_ptr(), s.data_ptr(), M, K, td.data_ptr())
+            check(q, s, M, K, *ref.quant_had(X, t))
+        elif op in ("silu_had", "silu_had_lut"):
+            gu = bits((M, 2 * K), 2.0)
+            gd = dev_bf16_bits(gu)
+            if op == "silu_had":
+                ctx.silu_mul_quant_had(gd.data_ptr(), q.data_ptr(), s.data_ptr(), M, K, td.data_ptr())
+            else:
+                ctx.silu_mul_quant_had_lut(gd.data_ptr(), q.data_ptr(), s.data_ptr(), M, K, td.data_ptr(), silu_lut.data_ptr())
+            check(q, s, M, K, *ref.silu_mul_quant_had(gu, t))
+        elif op == "add_rms":
+            y, r = bits((M, K), 1.0), bits((M, K), 4.0)
+            w = synth.f32_to_bf16_bits((rng.standard_normal(K) * 0.1).astype(np.float32))
+            ro = torch.zeros((M, K), dtype=torch.int16, device="cuda")
+            yd, rd, wd = dev_bf16_bits(y), dev_bf16_bits(r), dev_bf16_bits(w)
+            ctx.add_rms_quant_had(yd.data_ptr(), rd.data_ptr(), wd.data_ptr(), q.data_ptr(), s.data_ptr(), ro.data_ptr(), M, K, 1e-6, td.data_ptr())
+            wq, wsc, wro = ref.add_rms_quant_had(y, r, w, t, 1e-6, 256 if K <= 10240 else 512)
+            check(q, s, M, K, wq, wsc)
+            np.testing.assert_array_equal(host_u16(ro), wro)
+        elif op == "gdn":
+            N, pad = max(128, min(K, 10240) // 128 * 128), int(rng.choice([0, 8, 64]))
+            q, s = outs(M, N)
+            x, z = bits((M, N), 2.0), bits((M, N + pad), 3.0)
+            w = synth.f32_to_bf16_bits((1 + rng.standard_normal(128) * 0.1).astype(np.float32))
+            t2 = np.resize(t, N).astype(np.float32)
+            td2, xd, zd, wd = dev_f32(t2), dev_bf16_bits(x), dev_bf16_bits(z), dev_bf16_bits(w)
+            ctx.gdn_norm_quant_had(xd.data_ptr(), zd.data_ptr(), N + pad, wd.data_ptr(), q.data_ptr(), s.data_ptr(), M, N, 1e-6, td2.data_ptr())
+            check(q, s, M, N, *ref.gdn_norm_quant_had(x, z[:, :N], w, t2, 1e-6, silu_tab=silu_tab))
+        else:
+            hd = int(rng.choice([64, 128, 256]))
+            n_ = max(1, min(K, 6144) // hd) * hd
+            if n_ % 64:
+                continue
+            q, s = outs(M, n_)
+            t2 = np.resize(t, n_).astype(np.float32)
+            core, blk = bits((M, n_), 1.0), bits((M, 2 * n_), 3.0)
+            td2, cd, gd = dev_f32(t2), dev_bf16_bits(core), dev_bf16_bits(blk)
+            if op == "attn":
+                ctx.attn_gate_quant_had(cd.data_ptr(), gd.data_ptr(), q.data_ptr(), s.data_ptr(), M, n_, hd, 2 * n_, td2.data_ptr())
+            else:
+                ctx.attn_gate_quant_had_lut(cd.data_ptr(), gd.data_ptr(), q.data_ptr(), s.data_ptr(), M, n_, hd, 2 * n_, td2.data_ptr(),
+                                            sig_lut.data_ptr())
+            check(q, s, M, n_, *ref.attn_gate_quant_had(core, blk, t2, hd))
