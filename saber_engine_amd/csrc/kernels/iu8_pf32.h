@@ -179,7 +179,10 @@ __device__ __forceinline__ void iu8_pf32_run(const iu8_u8 *__restrict__ A, const
 #pragma unroll
     for (int p = 0; p < A_PER; ++p) {
       const int f = min(p * NWAVE + wave, A_FR - 1);  // fragment (mt = f/2, kt2 = f%2) of the step
-      const int ar = iu8_arow(t.R, t.mbase + (f >> 1) * 16 + (lane & 15));  // rows past the edge: the last one
+      // rows past the edge: the last one of the padded 16-row tile (the int8 operand is padded to whole tiles); the
+      // fused-quant form reads the caller's bf16 rows and their scales, which hold exactly `rows` rows: the last live one
+      const int mrow = t.mbase + (f >> 1) * 16 + (lane & 15);
+      const int ar = iu8_arow(t.R, AQ ? min(mrow, t.R.rows - 1) : mrow);
       if constexpr (AQ) {  // bf16 rows: 2 bytes an element
         oa[p] = (unsigned)(((size_t)ar * K + (f & 1) * 64 + (lane >> 4) * 16) * 2);
         os[p] = as[ar];
