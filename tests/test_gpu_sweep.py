@@ -3,6 +3,9 @@ with whatever kernel the launch law picks for the shape, the routed layer, and t
 like the fixed cases elsewhere; the shapes, magnitudes and special values are drawn so that the corners between
 the hand-picked cases get visited (ragged rows and columns, every regime of M, rows whose magnitudes spread over
 many orders, infinities, NaN, zeros and denormals in the producers' inputs)."""
+import os
+import re
+
 import numpy as np
 import pytest
 import torch
@@ -11,6 +14,7 @@ from oracle import ref
 from saber_engine_amd import iu8, synth
 from tests.gpu_util import DenseRun, assert_dense_matches, dev_bf16_bits, dev_f32, host_u16, say
 from tests.test_gpu_moe import check_layer, run_layer
+from tests.test_gpu_pfq import CELLS as PFQ_CELLS, run_pfq
 
 pytestmark = pytest.mark.gpu
 
@@ -40,6 +44,52 @@ def test_dense_linear_random_shapes(ctx):
                              c.data_ptr(), M, N, K)
             torch.cuda.synchronize()
             np.testing.assert_array_equal(host_u16(c), r["C"])
+
+
+def test_named_cells_random_shapes(ctx):
+    """Every dense cell by its name -- the tile cells at any row count, the streaming cells with K shared over one to
+    three workgroups, the `_ks` tile cells, the fused-quant cells -- on random ragged shapes: what the host's
+    rule lets through gives the oracle's bytes (and leaves the arrival counters at zero), the rest is refused."""
+    rng = np.random.default_rng(20243)
+    text = open(os.path.join(iu8.PKG, "csrc", "kernels", "iu8_variants.def")).read()
+    names = [n for n in re.findall(r"^IU8_(?:DEC|PF)_VARIANT\((\w+),", text, flags=re.M) if not n.endswith("_acc")]
+    split = ["macaq_iu8_pf_w4_t128x128_ks", "macaq_iu8_pf_w8_t128x128_ks", "macaq_iu8_pf_w4_t256x160_ks", "macaq_iu8_pf_w8_t256x160_ks",
+             "macaq_iu8_pf_w4_t64x128_s_ks"]
+    ran = 0
+    for n in range(320):
+        kind, ks = str(rng.choice(["pf", "pf", "dec", "ks", "pfq"])), 1
+        if kind == "dec":
+            name, M, ks = str(rng.choice([x for x in names if "_dec_" in x])), int(rng.integers(1, 65)), int(rng.integers(1, 4))
+        elif kind == "ks":
+            name, M, ks = str(rng.choice(split)), int(rng.choice([33, 64, 65, 100, 128, 200, 256, 300, 513])), int(rng.integers(1, 5))
+        elif kind == "pfq":
+            w8 = bool(rng.integers(0, 2))
+            name, M = f"macaq_iu8_pfq_{'w8' if w8 else 'w4'}_{rng.choice(PFQ_CELLS[w8])}", int(rng.choice([65, 100, 128, 129, 200, 256, 300, 513, 1000]))
+        else:
+            name = str(rng.choice([x for x in names if "_pf_" in x]))
+            M = int(rng.choice([1, 17, 64, 65, 100, 128, 129, 200, 256, 257, 300, 511, 513, 700, 1025, 2100]))
+        w8 = "_w8_" in name
+        N, K = int(rng.integers(1, 161)) * 16, int(rng.integers(1, 25)) * 128
+        while M * N * K > 3e9:
+            N = max(16, (N // 2) // 16 * 16)
+        say(f"sweep named {n}: {name} ks={ks} M={M} N={N} K={K}")
+        case = synth.dense_case(M, N, K, w8=w8, seed=int(rng.integers(0, 1 << 30)))
+        try:
+            iu8.describe(name, M, N, K, ks)
+        except iu8.IU8Error:
+            continue                     # the host's rule: more rows than the cell holds, more shares than K steps
+        r = ref.linear(case["X"], case["W"], case["ws"], w8, threads=8)
+        if kind == "pfq":
+            s, c = run_pfq(ctx, case, name)
+            np.testing.assert_array_equal(s.view(np.uint32), r["a_scale"].view(np.uint32))
+            np.testing.assert_array_equal(c, r["C"])
+        else:
+            run = DenseRun(ctx, case, kernel=name, ks=ks, want_acc=False)
+            np.testing.assert_array_equal(run.C, r["C"])
+            if run.counter is not None:
+                assert not run.counter.cpu().numpy().any()
+        ran += 1
+    assert ran >= 200
 
 
 def test_routed_layer_random_shapes(ctx):
