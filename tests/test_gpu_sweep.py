@@ -12,8 +12,10 @@ import torch
 
 from oracle import ref
 from saber_engine_amd import iu8, synth
-from tests.gpu_util import DenseRun, assert_dense_matches, dev_bf16_bits, dev_f32, host_u16, say
+from tests.gpu_util import DenseRun, assert_dense_matches, dev_bf16_bits, dev_f32, dev_u8, host_u16, say
+from tests.test_gpu_chain import SLOTS, Mlp
 from tests.test_gpu_moe import check_layer, run_layer
+from tests.test_gpu_pair import halves
 from tests.test_gpu_pfq import CELLS as PFQ_CELLS, run_pfq
 
 pytestmark = pytest.mark.gpu
@@ -90,6 +92,71 @@ def test_named_cells_random_shapes(ctx):
                 assert not run.counter.cpu().numpy().any()
         ran += 1
     assert ran >= 200
+
+
+def test_pair_chain_static_gemm_and_back_half_random_shapes(ctx):
+    """The decode pair, the decode MLP chain (two launches in a row on one state block), the GEMM on the
+    library's static workspace (twice in a row) and the routed layer's back half as two and as three launches."""
+    rng = np.random.default_rng(20244)
+    for n in range(150):
+        kind = str(rng.choice(["pair", "chain", "static", "back", "back"]))
+        if kind == "pair":
+            M, K = int(rng.integers(1, 49)), int(rng.integers(1, 41)) * 128
+            n0, n1 = int(rng.integers(1, 200)) * 16, int(rng.integers(1, 40)) * 16
+            say(f"sweep {n}: pair M={M} K={K} N={n0}+{n1}")
+            X, (W0, ws0), (W1, ws1) = halves(rng, M, K, n0, n1)
+            xd = dev_bf16_bits(X)
+            q = torch.zeros(iu8.a_bytes(M, K), dtype=torch.uint8, device="cuda")
+            s = torch.zeros(M, dtype=torch.float32, device="cuda")
+            ctx.quant(xd.data_ptr(), q.data_ptr(), s.data_ptr(), M, K)
+            w0, w1, s0, s1 = dev_u8(iu8.repack_w4(W0)), dev_u8(iu8.repack_w4(W1)), dev_f32(ws0), dev_f32(ws1)
+            c0 = torch.full((M, n0), 0x7FC0, dtype=torch.int16, device="cuda")
+            c1 = torch.full((M, n1), 0x7FC0, dtype=torch.int16, device="cuda")
+            ctx.gemm_pair(q.data_ptr(), s.data_ptr(), w0.data_ptr(), s0.data_ptr(), c0.data_ptr(), n0,
+                          w1.data_ptr(), s1.data_ptr(), c1.data_ptr(), n1, M, K)
+            torch.cuda.synchronize()
+            np.testing.assert_array_equal(host_u16(c0), ref.linear(X, W0, ws0, False, threads=8)["C"])
+            np.testing.assert_array_equal(host_u16(c1), ref.linear(X, W1, ws1, False, threads=8)["C"])
+        elif kind == "chain":
+            M = int(rng.integers(1, 5))
+            cap = 20480 // (1 << (M - 1).bit_length()) // 128        # the fused form's staged rows: pow2(M) * width <= 20 KiB
+            H, I = int(rng.integers(1, cap + 1)) * 128, int(rng.integers(1, cap + 1)) * 128
+            say(f"sweep {n}: chain M={M} H={H} I={I}")
+            assert iu8.mlp_chain_holds(M, H, I)
+            mlp = Mlp(M, H, I, seed=int(rng.integers(0, 1 << 30)))
+            gu, p, c = mlp.oracle()
+            for _ in range(2):
+                mlp.chain(ctx)
+                assert not mlp.state[SLOTS:].any().item()
+                np.testing.assert_array_equal(host_u16(mlp.gu), gu)
+                np.testing.assert_array_equal(host_u16(mlp.p), p)
+                np.testing.assert_array_equal(host_u16(mlp.c), c)
+        elif kind == "static":
+            M, w8 = int(rng.choice([1, 3, 16, 17, 40, 64, 65, 100, 128, 200, 300])), bool(rng.integers(0, 2))
+            N, K = int(rng.integers(1, 200)) * 16, int(rng.integers(1, 137)) * 128
+            while M * N * K > 3e9:
+                N = max(16, (N // 2) // 16 * 16)
+            say(f"sweep {n}: static-workspace GEMM M={M} N={N} K={K} w8={w8}")
+            case = synth.dense_case(M, N, K, w8=w8, seed=int(rng.integers(0, 1 << 30)))
+            r = ref.linear(case["X"], case["W"], case["ws"], w8, threads=8)
+            x, wf, ws = dev_bf16_bits(case["X"]), dev_u8(iu8.repack_weights(case["W"], w8)), dev_f32(case["ws"])
+            q = torch.zeros(iu8.a_bytes(M, K), dtype=torch.uint8, device="cuda")
+            s = torch.zeros(M, dtype=torch.float32, device="cuda")
+            c = torch.full((M, N), 0x7FC0, dtype=torch.int16, device="cuda")
+            ctx.quant(x.data_ptr(), q.data_ptr(), s.data_ptr(), M, K)
+            for _ in range(2):
+                ctx.gemm_static(iu8.W8 if w8 else iu8.W4, q.data_ptr(), s.data_ptr(), wf.data_ptr(), ws.data_ptr(), c.data_ptr(), M, N, K)
+                torch.cuda.synchronize()
+                np.testing.assert_array_equal(host_u16(c), r["C"])
+        else:
+            T, H = int(rng.choice([1, 3, 8, 16, 33, 64, 100, 112, 113, 200, 300])), int(rng.choice([256, 512, 1024]))
+            I, fused = int(rng.choice([128, 256, 640, 1536])), bool(rng.integers(0, 2))
+            say(f"sweep {n}: routed back half T={T} H={H} I={I} two launches={fused}")
+            assert iu8.moe_back_holds(1, I)
+            case = synth.moe_case(T=T, E=128, topk=8, H=H, I=I, seed=int(rng.integers(0, 1 << 30)), experts=4)
+            layer = run_layer(ctx, case, tile_blocks=1, fused_back=fused)
+            check_layer(layer, case)
+            del layer
 
 
 def test_routed_layer_random_shapes(ctx):
