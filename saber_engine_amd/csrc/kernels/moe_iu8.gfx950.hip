@@ -222,10 +222,16 @@ static __device__ __forceinline__ void moe_route_body(
   __syncthreads();
   // A lone workgroup (up to 128 tokens) is its own last arriver: its counts are the totals, its
   // routes' bases are zero, and no hand-over through memory is needed.
+  if constexpr (PART) {
+    // (also with one workgroup: the placement launch sums the counts whatever their number, and a launch that
+    // ends here holds none of the layout's LDS -- 144 KiB of row tables that would leave one workgroup a CU to
+    // the quantising workgroups of the same launch)
+    for (int e = tid; e < e_loc; e += MOE_THREADS) blk_cnt[(size_t)blk * e_loc + e] = s_cnt[e];
+    return;
+  }
   const bool solo = nblk == 1;
   if (!solo) {
     for (int e = tid; e < e_loc; e += MOE_THREADS) blk_cnt[(size_t)blk * e_loc + e] = s_cnt[e];
-    if constexpr (PART) return;
     __syncthreads();
     if (tid == 0) {
       __threadfence();
