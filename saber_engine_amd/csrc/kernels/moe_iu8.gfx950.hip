@@ -64,27 +64,38 @@ static __device__ __forceinline__ float moe_dppf(float v) {
   return __int_as_float(moe_dpp<CTRL>(__float_as_int(v)));
 }
 
-// exclusive scan of one int a thread over the 256-thread workgroup; *total = the sum
-static __device__ __forceinline__ int moe_exscan(int v, int *s_wave, int *total) {
+// The layout's four scans over the experts (rows, tiles, touched experts, routes) in one pass: one round of
+// shuffles and one pair of barriers for all four. base[] = the exclusive prefixes, total[] = the sums, in that order.
+static __device__ __forceinline__ void moe_exscan4(int rows, int tiles, int touched, int routes, int (*s_wave4)[4],
+                                                   int (&base)[4], int (&total)[4]) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  int x = v;
+  const int v[4] = {rows, tiles, touched, routes};
+  int x[4] = {rows, tiles, touched, routes};
 #pragma unroll
   for (int o = 1; o < 64; o <<= 1) {
-    const int y = __shfl_up(x, o, 64);
-    if (lane >= o) x += y;
+#pragma unroll
+    for (int f = 0; f < 4; ++f) {
+      const int y = __shfl_up(x[f], o, 64);
+      if (lane >= o) x[f] += y;
+    }
   }
-  if (lane == 63) s_wave[wave] = x;
+  if (lane == 63) {
+#pragma unroll
+    for (int f = 0; f < 4; ++f) s_wave4[wave][f] = x[f];
+  }
   __syncthreads();
-  int base = 0, all = 0;
+#pragma unroll
+  for (int f = 0; f < 4; ++f) base[f] = x[f] - v[f], total[f] = 0;
 #pragma unroll
   for (int w = 0; w < MOE_THREADS / 64; ++w) {
-    const int s = s_wave[w];
-    if (w < wave) base += s;
-    all += s;
+#pragma unroll
+    for (int f = 0; f < 4; ++f) {
+      const int t = s_wave4[w][f];
+      if (w < wave) base[f] += t;
+      total[f] += t;
+    }
   }
   __syncthreads();
-  *total = all;
-  return base + x - v;
 }
 
 // The router's workgroup `blk` of `nblk` (128 tokens each). PART: the workgroup stops behind its own
@@ -104,7 +115,7 @@ static __device__ __forceinline__ void moe_route_body(
   __shared__ unsigned s_mask[MOE_E][MOE_TPB / 32];
   __shared__ int s_cnt[MOE_E];
   __shared__ int s_off[MOE_E], s_toff[MOE_E];
-  __shared__ int s_wave[MOE_THREADS / 64];
+  __shared__ int s_wave[MOE_THREADS / 64][4];
   __shared__ int s_last;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int t0 = blk * MOE_TPB;
@@ -298,11 +309,10 @@ static __device__ __forceinline__ void moe_route_body(
     my_touched = c > 0;
     my_routes = c;
   }
-  int rows_total, tiles_total, touched_total, routes_total;
-  const int rbase = moe_exscan(my_rows, s_wave, &rows_total);
-  const int tbase = moe_exscan(my_tiles, s_wave, &tiles_total);
-  moe_exscan(my_touched, s_wave, &touched_total);
-  moe_exscan(my_routes, s_wave, &routes_total);
+  int sbase[4], stotal[4];
+  moe_exscan4(my_rows, my_tiles, my_touched, my_routes, s_wave, sbase, stotal);
+  const int rbase = sbase[0], tbase = sbase[1];
+  const int rows_total = stotal[0], tiles_total = stotal[1], touched_total = stotal[2], routes_total = stotal[3];
   if (tid < e_loc) {
     s_off[tid] = rbase;
     s_toff[tid] = tbase;
@@ -417,7 +427,7 @@ extern "C" __global__ __launch_bounds__(MOE_THREADS) void moe_iu8_route_place_e1
   constexpr int PARTS = MOE_THREADS / MOE_E;
   __shared__ int s_all[PARTS][MOE_E], s_mine[PARTS][MOE_E];
   __shared__ int s_cnt[MOE_E], s_base[MOE_E], s_off[MOE_E], s_toff[MOE_E];
-  __shared__ int s_wave[MOE_THREADS / 64];
+  __shared__ int s_wave[MOE_THREADS / 64][4];
   const int tid = threadIdx.x, nblk = gridDim.x, blk = blockIdx.x;
   // this thread's route: its expert and rank are requested now, beside the count table, not behind the scans
   const int r = blk * (MOE_TPB * MOE_TOPK) + tid;
@@ -462,11 +472,10 @@ extern "C" __global__ __launch_bounds__(MOE_THREADS) void moe_iu8_route_place_e1
     my_touched = c > 0;
     my_routes = c;
   }
-  int rows_total, tiles_total, touched_total, routes_total;
-  const int rbase = moe_exscan(my_rows, s_wave, &rows_total);
-  const int tbase = moe_exscan(my_tiles, s_wave, &tiles_total);
-  moe_exscan(my_touched, s_wave, &touched_total);
-  moe_exscan(my_routes, s_wave, &routes_total);
+  int sbase[4], stotal[4];
+  moe_exscan4(my_rows, my_tiles, my_touched, my_routes, s_wave, sbase, stotal);
+  const int rbase = sbase[0], tbase = sbase[1];
+  const int rows_total = stotal[0], tiles_total = stotal[1], touched_total = stotal[2], routes_total = stotal[3];
   if (tid < e_loc) {
     s_off[tid] = rbase;
     s_toff[tid] = tbase;
