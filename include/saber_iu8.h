@@ -430,7 +430,7 @@ typedef struct {
   int32_t *tile_rows;   /* [tiles_cap] */
   int32_t *expert_cnt;  /* [experts] */
   int32_t *meta;        /* [8]: [0] tiles, [1] rows, [2] first shared row or -1, [3] routes, [4] experts touched */
-  int32_t *blk_cnt;     /* [ceil(T / 32) * experts]  scratch (the router uses the first ceil(T / 128) * experts) */
+  int32_t *blk_cnt;     /* [ceil(T / 32) * experts]  scratch (the one-launch router uses the first ceil(T / 128) * experts) */
   int32_t *rank;        /* [T * topk]                scratch */
   int32_t *arrive;      /* [1]  persistent: zeroed once by the caller, left zero */
   const uint16_t *silu_lut; /* optional (may be NULL): [65536] as saber_iu8_silu_table wrote it; with it
@@ -444,7 +444,8 @@ typedef struct {
 
 /* Router + expert-major sort + tile table (crates/saber-kernels/hip/moe_route.hip:108-284). logits bf16
  * [T, experts]. One launch up to 128 tokens (one routing workgroup); above, two: routing with the
- * workgroups' counts and ranks, then the layout with every workgroup placing its own routes. */
+ * workgroups' counts and ranks (32 tokens a workgroup: blk_cnt is used in full), then the layout with every
+ * workgroup placing its own routes. */
 int saber_iu8_moe_route(saber_iu8_ctx *ctx, const void *logits_bf16, uint32_t tokens, uint32_t experts, uint32_t topk,
                         uint32_t tile_blocks, const saber_iu8_moe_tables *t, void *stream);
 

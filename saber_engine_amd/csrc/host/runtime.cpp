@@ -737,9 +737,9 @@ static int moe_route_launches(saber_iu8_ctx *ctx, const void *logits, const void
   const std::string name = !x ? (two ? "moe_iu8_route_part_topk8_sort_e128" : "moe_iu8_route_topk8_sort_e128")
                               : std::string("moe_iu8_routeq_") + (rm ? "rm_" : "") + (two && rm ? "part_" : "") + "topk8_sort_e128";
   const bool part = name.find("_part_") != std::string::npos;
-  auto launch = [&](const std::string &kernel, uint32_t gx, bool with_x) {
+  auto launch = [&](const std::string &kernel, uint32_t gx, bool with_x, uint32_t block = 1024) {
     saber_iu8_desc d;
-    if (int rc = raw_desc(kernel.c_str(), gx, 1, 1024, &d)) return rc;
+    if (int rc = raw_desc(kernel.c_str(), gx, 1, block, &d)) return rc;
     set_i32(&d, "t", tokens);
     set_i32(&d, "e_lo", 0);
     set_i32(&d, "e_loc", experts);
@@ -754,8 +754,11 @@ static int moe_route_launches(saber_iu8_ctx *ctx, const void *logits, const void
                                    {"q", q},                        {"scale", scale}};
     return saber_iu8_launch(ctx, &d, b, with_x ? 17 : 14, stream);
   };
-  if (int rc = launch(name, nblk + (x ? (tokens + rows_wg - 1) / rows_wg : 0), x != nullptr)) return rc;
-  return part ? launch("moe_iu8_route_place_e128", nblk, false) : 0;
+  if (part) {  // routing workgroups of 32 tokens on 256 threads, a quantising workgroup a token row
+    if (int rc = launch(name, (tokens + 31) / 32 + (x ? tokens : 0), x != nullptr, 256)) return rc;
+    return launch("moe_iu8_route_place_e128", nblk, false);
+  }
+  return launch(name, nblk + (x ? (tokens + rows_wg - 1) / rows_wg : 0), x != nullptr);
 }
 
 int saber_iu8_moe_route(saber_iu8_ctx *ctx, const void *logits, uint32_t tokens, uint32_t experts, uint32_t topk,

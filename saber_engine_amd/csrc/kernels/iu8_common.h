@@ -117,6 +117,42 @@ static __device__ __forceinline__ unsigned iu8_code4_rcp(float x0, float x1, flo
          __builtin_amdgcn_perm(__float_as_uint(u3), __float_as_uint(u2), 0x04000c0cu);
 }
 
+// The per-token law from a row kept as packed bf16 pairs (pk[g][w]: elements 2w and 2w + 1 of 16-element group g, as
+// loaded; a thread's groups past the row's end are zeros). The largest magnitude of finite bf16 values is
+// the largest of their bit patterns without the sign, two a packed 16-bit maximum; a thread that holds a
+// NaN (a pattern above infinity's) takes the f32 maximum instead, which passes NaNs over.
+template <int NG>
+static __device__ __forceinline__ float iu8_pk_amax(const unsigned (&pk)[NG][8]) {
+  typedef unsigned short us2 __attribute__((ext_vector_type(2)));
+  us2 m2 = {0, 0};
+#pragma unroll
+  for (int i = 0; i < NG; ++i)
+#pragma unroll
+    for (int w = 0; w < 8; ++w) m2 = __builtin_elementwise_max(m2, __builtin_bit_cast(us2, pk[i][w] & 0x7FFF7FFFu));
+  const unsigned top = m2.x > m2.y ? m2.x : m2.y;
+  float amax = __uint_as_float(top << 16);
+  if (top > 0x7F80u) {
+    amax = 0.f;
+#pragma unroll
+    for (int i = 0; i < NG; ++i)
+#pragma unroll
+      for (int w = 0; w < 8; ++w) {
+        unsigned r = pk[i][w];
+        asm volatile("" : "+v"(r));  // a value of its own: nothing of the fast path is kept alive for this one
+        amax = fmaxf(amax, fabsf(__uint_as_float(r << 16)));
+        amax = fmaxf(amax, fabsf(__uint_as_float(r & 0xFFFF0000u)));
+      }
+  }
+  return amax;
+}
+static __device__ __forceinline__ iu8_v4u iu8_pk_codes(const unsigned (&g)[8], float sc, float rcp) {
+  unsigned d[4];
+#pragma unroll
+  for (int w = 0; w < 4; ++w)
+    d[w] = iu8_code4_rcp(__uint_as_float(g[2 * w] << 16), __uint_as_float(g[2 * w] & 0xFFFF0000u),
+                         __uint_as_float(g[2 * w + 1] << 16), __uint_as_float(g[2 * w + 1] & 0xFFFF0000u), sc, rcp);
+  return iu8_v4u{d[0], d[1], d[2], d[3]};
+}
 // Maximum over the 64 lanes of a wave of values that are non-negative and never NaN (row maxima of
 // |x|): DPP inside each 16-lane row (partners xor 1, xor 2, the half-row and the row mirror), then the
 // four rows' values through scalar registers, where the unsigned order of the bit patterns is the

@@ -82,42 +82,6 @@ static __device__ __forceinline__ void i8q_tail(float (&v)[I8Q_MAXG][16], int G,
   }
 }
 
-// The same from a row kept as packed bf16 pairs (pk[g][w]: elements 2w and 2w + 1 of group g, as loaded; a
-// thread's groups past the row's end are zeros). The largest magnitude of finite bf16 values is
-// the largest of their bit patterns without the sign, two a packed 16-bit maximum; a thread that holds a
-// NaN (a pattern above infinity's) takes the f32 maximum instead, which passes NaNs over.
-template <int NG>
-static __device__ __forceinline__ float i8q_pk_amax(const unsigned (&pk)[NG][8]) {
-  typedef unsigned short us2 __attribute__((ext_vector_type(2)));
-  us2 m2 = {0, 0};
-#pragma unroll
-  for (int i = 0; i < NG; ++i)
-#pragma unroll
-    for (int w = 0; w < 8; ++w) m2 = __builtin_elementwise_max(m2, __builtin_bit_cast(us2, pk[i][w] & 0x7FFF7FFFu));
-  const unsigned top = m2.x > m2.y ? m2.x : m2.y;
-  float amax = __uint_as_float(top << 16);
-  if (top > 0x7F80u) {
-    amax = 0.f;
-#pragma unroll
-    for (int i = 0; i < NG; ++i)
-#pragma unroll
-      for (int w = 0; w < 8; ++w) {
-        unsigned r = pk[i][w];
-        asm volatile("" : "+v"(r));  // a value of its own: nothing of the fast path is kept alive for this one
-        amax = fmaxf(amax, fabsf(__uint_as_float(r << 16)));
-        amax = fmaxf(amax, fabsf(__uint_as_float(r & 0xFFFF0000u)));
-      }
-  }
-  return amax;
-}
-static __device__ __forceinline__ iu8_v4u i8q_pk_codes(const unsigned (&g)[8], float sc, float rcp) {
-  unsigned d[4];
-#pragma unroll
-  for (int w = 0; w < 4; ++w)
-    d[w] = iu8_code4_rcp(__uint_as_float(g[2 * w] << 16), __uint_as_float(g[2 * w] & 0xFFFF0000u),
-                         __uint_as_float(g[2 * w + 1] << 16), __uint_as_float(g[2 * w + 1] & 0xFFFF0000u), sc, rcp);
-  return iu8_v4u{d[0], d[1], d[2], d[3]};
-}
 // A group's 16 elements, zeros when the group is past the row's end. Nothing uses the registers before
 // every group of the row has been requested: a load whose data is used under the same test is waited
 // for before the next is requested -- MAXG memory latencies a row instead of one.
@@ -131,7 +95,7 @@ template <int I8Q_MAXG, bool RM, bool SCALE_ONLY>
 static __device__ __forceinline__ void i8q_tail_pk(const unsigned (&pk)[I8Q_MAXG][8], int G, iu8_u8 *__restrict__ q,
                                                    float *__restrict__ scale, int row, int K) {
   const int tid = threadIdx.x;
-  const float amax = i8q_block_max(i8q_pk_amax(pk));
+  const float amax = i8q_block_max(iu8_pk_amax(pk));
   const float sc = fmaxf(__fdiv_rn(amax, 127.f), 1e-30f);
   const float rcp = __fdiv_rn(1.f, sc);
   if (tid == 0) scale[row] = sc;
@@ -141,7 +105,7 @@ static __device__ __forceinline__ void i8q_tail_pk(const unsigned (&pk)[I8Q_MAXG
   for (int i = 0; i < I8Q_MAXG; ++i) {
     const int g = tid + i * I8Q_T;
     if (g >= G) continue;
-    const iu8_v4u d = i8q_pk_codes(pk[i], sc, rcp);
+    const iu8_v4u d = iu8_pk_codes(pk[i], sc, rcp);
     if constexpr (RM) *(iu8_v4u *)(q + (size_t)row * K + g * 16) = d;
     else *(iu8_v4u *)(qrow + (size_t)(g >> 2) * 1024 + (g & 3) * 256) = d;
     __builtin_amdgcn_sched_barrier(0);  // a group's codes at a time: their temporaries are what fills the registers

@@ -27,6 +27,7 @@
 #define MOE_E 128
 #define MOE_TOPK 8
 #define MOE_TPB 128
+#define MOE_PTPB 32  // tokens a routing workgroup of the part launches (256 threads)
 #define MOE_THREADS 1024
 #define MOE_CHUNK 36864  // rows of the placement tables held in LDS at a time (144 KiB)
 
@@ -101,7 +102,12 @@ static __device__ __forceinline__ void moe_exscan4(int rows, int tiles, int touc
 // The router's workgroup `blk` of `nblk` (128 tokens each). PART: the workgroup stops behind its own
 // counts and ranks (phases 1 and 2); the tables are then laid out by moe_iu8_route_place_e128, a launch
 // of its own in which every workgroup places its own routes.
-template <bool PART = false>
+// TPB: tokens a workgroup, on TPB * 8 threads. The one-launch forms take 128 (the layout's scans and its placement
+// are written for 1,024 threads); the part launches take MOE_PTPB = 32: the routing of a token is a long chain of
+// dependent arithmetic (128 exps, eight rounds of arg-max), and with 128 tokens a workgroup it runs four waves a
+// SIMD deep on T / 128 CUs while the rest of the card idles or quantises -- 32 tokens a workgroup put a wave a SIMD
+// on four times the CUs.
+template <bool PART = false, int TPB = MOE_TPB>
 static __device__ __forceinline__ void moe_route_body(
     const unsigned short *__restrict__ logits, int T, int e_lo, int e_loc, int tile_blocks, int with_shared,
     int *__restrict__ topk_ids, float *__restrict__ topk_w, int *__restrict__ route_pos, int *__restrict__ row_tok,
@@ -109,20 +115,22 @@ static __device__ __forceinline__ void moe_route_body(
     int *__restrict__ tile_rows, int *__restrict__ expert_cnt, int *__restrict__ meta, int *__restrict__ blk_cnt,
     int *__restrict__ rank, int *__restrict__ arrive, const int nblk, const int blk) {
 #pragma clang fp contract(off)
-  __shared__ __attribute__((aligned(16))) int s_ids[MOE_TPB * MOE_TOPK];
+  constexpr int NTHR = TPB * MOE_TOPK;
+  static_assert(PART || TPB == MOE_TPB, "the layout behind the routing runs on 1,024 threads");
+  __shared__ __attribute__((aligned(16))) int s_ids[TPB * MOE_TOPK];
   __shared__ int s_part[MOE_THREADS / MOE_E][MOE_E];
   __shared__ int s_rows[MOE_CHUNK];
-  __shared__ unsigned s_mask[MOE_E][MOE_TPB / 32];
+  __shared__ unsigned s_mask[MOE_E][TPB / 32];
   __shared__ int s_cnt[MOE_E];
   __shared__ int s_off[MOE_E], s_toff[MOE_E];
   __shared__ int s_wave[MOE_THREADS / 64][4];
   __shared__ int s_last;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int t0 = blk * MOE_TPB;
+  const int t0 = blk * TPB;
 
-  for (int e = tid; e < MOE_E; e += MOE_THREADS) s_cnt[e] = 0;
-  for (int i = tid; i < MOE_E * (MOE_TPB / 32); i += MOE_THREADS) s_mask[i / (MOE_TPB / 32)][i % (MOE_TPB / 32)] = 0u;
-  for (int i = tid; i < MOE_TPB * MOE_TOPK; i += MOE_THREADS) s_ids[i] = -1;
+  for (int e = tid; e < MOE_E; e += NTHR) s_cnt[e] = 0;
+  for (int i = tid; i < MOE_E * (TPB / 32); i += NTHR) s_mask[i / (TPB / 32)][i % (TPB / 32)] = 0u;
+  for (int i = tid; i < TPB * MOE_TOPK; i += NTHR) s_ids[i] = -1;
   __syncthreads();
 
   // ---- phase 1: 8 lanes a token (a wave = 8 tokens); lane group g owns experts [16g, 16g + 16).
@@ -208,26 +216,26 @@ static __device__ __forceinline__ void moe_route_body(
   // ---- phase 2: this workgroup's per-expert counts and each route's rank among the earlier
   // tokens of this workgroup routed to the same expert (a token's experts are distinct): a bit a
   // token in the expert's 128-bit mask, the rank is the count of the bits below the token's
-  for (int i = tid; i < MOE_TPB * MOE_TOPK; i += MOE_THREADS) {
+  for (int i = tid; i < TPB * MOE_TOPK; i += NTHR) {
     const int e = s_ids[i], le = e - e_lo, tl = i / MOE_TOPK;
     if (e >= 0 && le >= 0 && le < e_loc) atomicOr(&s_mask[le][tl >> 5], 1u << (tl & 31));
   }
   __syncthreads();
-  for (int i = tid; i < MOE_TPB * MOE_TOPK; i += MOE_THREADS) {
+  for (int i = tid; i < TPB * MOE_TOPK; i += NTHR) {
     const int e = s_ids[i], le = e - e_lo, tl = i / MOE_TOPK;
     if (e < 0 || le < 0 || le >= e_loc) continue;
     int rk = 0;
 #pragma unroll
-    for (int w = 0; w < MOE_TPB / 32; ++w) {
+    for (int w = 0; w < TPB / 32; ++w) {
       const unsigned m = s_mask[le][w];
       rk += __popc(w < (tl >> 5) ? m : w == (tl >> 5) ? m & ((1u << (tl & 31)) - 1u) : 0u);
     }
     rank[(size_t)t0 * MOE_TOPK + i] = rk;
   }
-  for (int e = tid; e < e_loc; e += MOE_THREADS) {
+  for (int e = tid; e < e_loc; e += NTHR) {
     int c = 0;
 #pragma unroll
-    for (int w = 0; w < MOE_TPB / 32; ++w) c += __popc(s_mask[e][w]);
+    for (int w = 0; w < TPB / 32; ++w) c += __popc(s_mask[e][w]);
     s_cnt[e] = c;
   }
   __syncthreads();
@@ -237,7 +245,7 @@ static __device__ __forceinline__ void moe_route_body(
     // (also with one workgroup: the placement launch sums the counts whatever their number, and a launch that
     // ends here holds none of the layout's LDS -- 144 KiB of row tables that would leave one workgroup a CU to
     // the quantising workgroups of the same launch)
-    for (int e = tid; e < e_loc; e += MOE_THREADS) blk_cnt[(size_t)blk * e_loc + e] = s_cnt[e];
+    for (int e = tid; e < e_loc; e += NTHR) blk_cnt[(size_t)blk * e_loc + e] = s_cnt[e];
     return;
   }
   const bool solo = nblk == 1;
@@ -400,14 +408,14 @@ extern "C" __global__ __launch_bounds__(MOE_THREADS) void moe_iu8_route_topk8_so
                  tile_expert, tile_row0, tile_rows, expert_cnt, meta, blk_cnt, rank, arrive, gridDim.x, blockIdx.x);
 }
 
-extern "C" __global__ __launch_bounds__(MOE_THREADS) void moe_iu8_route_part_topk8_sort_e128(
+extern "C" __global__ __launch_bounds__(MOE_PTPB * MOE_TOPK) void moe_iu8_route_part_topk8_sort_e128(
     const unsigned short *__restrict__ logits, int T, int e_lo, int e_loc, int tile_blocks, int with_shared,
     int *__restrict__ topk_ids, float *__restrict__ topk_w, int *__restrict__ route_pos, int *__restrict__ row_tok,
     int *__restrict__ row_route, int *__restrict__ tile_expert, int *__restrict__ tile_row0,
     int *__restrict__ tile_rows, int *__restrict__ expert_cnt, int *__restrict__ meta, int *__restrict__ blk_cnt,
     int *__restrict__ rank, int *__restrict__ arrive) {
-  moe_route_body<true>(logits, T, e_lo, e_loc, tile_blocks, with_shared, topk_ids, topk_w, route_pos, row_tok, row_route,
-                       tile_expert, tile_row0, tile_rows, expert_cnt, meta, blk_cnt, rank, arrive, gridDim.x, blockIdx.x);
+  moe_route_body<true, MOE_PTPB>(logits, T, e_lo, e_loc, tile_blocks, with_shared, topk_ids, topk_w, route_pos, row_tok, row_route,
+                                 tile_expert, tile_row0, tile_rows, expert_cnt, meta, blk_cnt, rank, arrive, gridDim.x, blockIdx.x);
 }
 
 // The tables behind moe_iu8_route*_part_*: workgroup b (of ceil(T / 128), the part launch's routing
@@ -428,13 +436,18 @@ extern "C" __global__ __launch_bounds__(MOE_THREADS) void moe_iu8_route_place_e1
   __shared__ int s_all[PARTS][MOE_E], s_mine[PARTS][MOE_E];
   __shared__ int s_cnt[MOE_E], s_base[MOE_E], s_off[MOE_E], s_toff[MOE_E];
   __shared__ int s_wave[MOE_THREADS / 64][4];
-  const int tid = threadIdx.x, nblk = gridDim.x, blk = blockIdx.x;
+  // the part launch counted and ranked in blocks of MOE_PTPB tokens: SUB of them make this workgroup's 128 tokens
+  constexpr int SUB = MOE_TPB / MOE_PTPB;
+  static_assert(SUB <= PARTS, "a thread group a sub-block");
+  __shared__ int s_sub[SUB][MOE_E];
+  const int tid = threadIdx.x, nblk = (T + MOE_PTPB - 1) / MOE_PTPB, blk = blockIdx.x * SUB;
   // this thread's route: its expert and rank are requested now, beside the count table, not behind the scans
-  const int r = blk * (MOE_TPB * MOE_TOPK) + tid;
+  const int r = blockIdx.x * (MOE_TPB * MOE_TOPK) + tid;
   const bool mine = r < T * MOE_TOPK;
   const int my_e = mine ? topk_ids[r] : -1, my_rank = mine ? rank[r] : 0;
   {
     const int e = tid % MOE_E, part = tid / MOE_E;
+    if (part < SUB) s_sub[part][e] = (e < e_loc && blk + part < nblk) ? blk_cnt[(size_t)(blk + part) * e_loc + e] : 0;
     const int chunk = (nblk + PARTS - 1) / PARTS, b_lo = min(part * chunk, nblk), b_hi = min(b_lo + chunk, nblk);
     int all = 0, mine = 0;
     if (e < e_loc)
@@ -481,7 +494,7 @@ extern "C" __global__ __launch_bounds__(MOE_THREADS) void moe_iu8_route_place_e1
     s_toff[tid] = tbase;
   }
   __syncthreads();
-  if (blk == 0) {
+  if (blockIdx.x == 0) {
     const int sh_row0 = rows_total;
     const int sh_blocks = with_shared ? (T + 15) / 16 : 0;
     const int sh_tiles = (sh_blocks + G - 1) / G;
@@ -519,7 +532,12 @@ extern "C" __global__ __launch_bounds__(MOE_THREADS) void moe_iu8_route_place_e1
   if (mine) {  // this workgroup's routes: a thread a route
     const int le = my_e - e_lo;
     const bool local = le >= 0 && le < e_loc;
-    const int p = local ? s_off[le] + s_base[le] + my_rank : -1;
+    int p = -1;
+    if (local) {  // the experts' offset, the routes of the blocks in front of this route's 32-token block, its rank there
+      p = s_off[le] + s_base[le] + my_rank;
+#pragma unroll
+      for (int j = 0; j + 1 < SUB; ++j) p += j < tid / (MOE_PTPB * MOE_TOPK) ? s_sub[j][le] : 0;
+    }
     route_pos[r] = p;
     if (local) {
       row_route[p] = r;
@@ -536,7 +554,7 @@ extern "C" __global__ __launch_bounds__(MOE_THREADS) void moe_iu8_route_place_e1
 // quantisation instead of in front of it. Codes in the A fragment order (RM false, for the streaming
 // cell) or row-major (RM true, for the MFMA cells' gather). grid [ceil(T/128) + ceil(T / rows a
 // workgroup), 1, 1].
-template <bool RM, bool PART = false>
+template <bool RM, bool PART = false>  // (PART: kept for the one-launch body's own use; the part launch has its own kernel below)
 static __device__ __forceinline__ void moe_routeq_body(
     const unsigned short *__restrict__ logits, int T, int e_lo, int e_loc, int tile_blocks, int with_shared,
     int *__restrict__ topk_ids, float *__restrict__ topk_w, int *__restrict__ route_pos, int *__restrict__ row_tok,
@@ -608,8 +626,56 @@ static __device__ __forceinline__ void moe_routeq_body(
   }
 MOE_ROUTEQ(moe_iu8_routeq_topk8_sort_e128, false, false)
 MOE_ROUTEQ(moe_iu8_routeq_rm_topk8_sort_e128, true, false)
-MOE_ROUTEQ(moe_iu8_routeq_rm_part_topk8_sort_e128, true, true)
 #undef MOE_ROUTEQ
+// The part form of the same launch (above 128 tokens, row-major codes): workgroups of 256 threads, the first
+// ceil(T / 32) route 32 tokens each (moe_route_body), each of the T behind them quantises one token row, a thread
+// up to four 16-element groups (k <= 16,384). grid [ceil(T / 32) + T, 1, 1]; moe_iu8_route_place_e128 follows.
+extern "C" __global__ __launch_bounds__(MOE_PTPB * MOE_TOPK) void moe_iu8_routeq_rm_part_topk8_sort_e128(
+    const unsigned short *__restrict__ logits, int T, int e_lo, int e_loc, int tile_blocks, int with_shared,
+    int *__restrict__ topk_ids, float *__restrict__ topk_w, int *__restrict__ route_pos, int *__restrict__ row_tok,
+    int *__restrict__ row_route, int *__restrict__ tile_expert, int *__restrict__ tile_row0,
+    int *__restrict__ tile_rows, int *__restrict__ expert_cnt, int *__restrict__ meta, int *__restrict__ blk_cnt,
+    int *__restrict__ rank, int *__restrict__ arrive, const unsigned short *__restrict__ x,
+    unsigned char *__restrict__ q, float *__restrict__ scale, int k) {
+#pragma clang fp contract(off)
+  constexpr int NTHR = MOE_PTPB * MOE_TOPK, NG = 4;
+  const int nblk = (T + MOE_PTPB - 1) / MOE_PTPB;
+  if ((int)blockIdx.x < nblk) {
+    moe_route_body<true, MOE_PTPB>(logits, T, e_lo, e_loc, tile_blocks, with_shared, topk_ids, topk_w, route_pos, row_tok, row_route,
+                                   tile_expert, tile_row0, tile_rows, expert_cnt, meta, blk_cnt, rank, arrive, nblk, blockIdx.x);
+    return;
+  }
+  __shared__ float s_max[NTHR / 64];
+  const int row = (int)blockIdx.x - nblk, tid = threadIdx.x, G = k >> 4;
+  if (row >= T) return;
+  const unsigned short *xr = x + (size_t)row * k;
+  // the row's pieces are requested all at once and stay packed as they came; groups past the row's end are zeros
+  unsigned pk[NG][8];
+#pragma unroll
+  for (int i = 0; i < NG; ++i) {
+    const int g = tid + i * NTHR;
+    iu8_v4u lo = {0u, 0u, 0u, 0u}, hi = {0u, 0u, 0u, 0u};
+    if (g < G) lo = *(const iu8_v4u *)(xr + (unsigned)(g * 16)), hi = *(const iu8_v4u *)(xr + (unsigned)(g * 16) + 8);
+#pragma unroll
+    for (int w = 0; w < 4; ++w) pk[i][w] = lo[w], pk[i][4 + w] = hi[w];
+  }
+  float amax = iu8_pk_amax(pk);
+  amax = iu8_wave_max_nonneg(amax);
+  if ((tid & 63) == 0) s_max[tid >> 6] = amax;
+  __syncthreads();
+  amax = s_max[0];
+#pragma unroll
+  for (int w = 1; w < NTHR / 64; ++w) amax = fmaxf(amax, s_max[w]);
+  const float sc = fmaxf(__fdiv_rn(amax, 127.f), 1e-30f), rcp = __fdiv_rn(1.f, sc);
+  if (tid == 0) scale[row] = sc;
+#pragma unroll
+  for (int i = 0; i < NG; ++i) {
+    const int g = tid + i * NTHR;
+    if (g >= G) continue;
+    *(iu8_v4u *)(q + (size_t)row * k + (unsigned)(g * 16)) = iu8_pk_codes(pk[i], sc, rcp);
+    __builtin_amdgcn_sched_barrier(0);  // a group's codes at a time (registers)
+  }
+}
 
 // ---------------------------------------------------------------------------- grouped GEMMs
 // grid [ceil(N / BN), tiles_cap, 1]: blockIdx.y is a tile; a workgroup whose tile is past the live
