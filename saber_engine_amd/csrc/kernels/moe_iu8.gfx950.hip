@@ -554,7 +554,7 @@ extern "C" __global__ __launch_bounds__(MOE_THREADS) void moe_iu8_route_place_e1
 // quantisation instead of in front of it. Codes in the A fragment order (RM false, for the streaming
 // cell) or row-major (RM true, for the MFMA cells' gather). grid [ceil(T/128) + ceil(T / rows a
 // workgroup), 1, 1].
-template <bool RM, bool PART = false>  // (PART: kept for the one-launch body's own use; the part launch has its own kernel below)
+template <bool RM>
 static __device__ __forceinline__ void moe_routeq_body(
     const unsigned short *__restrict__ logits, int T, int e_lo, int e_loc, int tile_blocks, int with_shared,
     int *__restrict__ topk_ids, float *__restrict__ topk_w, int *__restrict__ route_pos, int *__restrict__ row_tok,
@@ -565,8 +565,8 @@ static __device__ __forceinline__ void moe_routeq_body(
 #pragma clang fp contract(off)
   const int nblk = (T + MOE_TPB - 1) / MOE_TPB;
   if ((int)blockIdx.x < nblk) {
-    moe_route_body<PART>(logits, T, e_lo, e_loc, tile_blocks, with_shared, topk_ids, topk_w, route_pos, row_tok, row_route,
-                         tile_expert, tile_row0, tile_rows, expert_cnt, meta, blk_cnt, rank, arrive, nblk, blockIdx.x);
+    moe_route_body<false>(logits, T, e_lo, e_loc, tile_blocks, with_shared, topk_ids, topk_w, route_pos, row_tok, row_route,
+                          tile_expert, tile_row0, tile_rows, expert_cnt, meta, blk_cnt, rank, arrive, nblk, blockIdx.x);
     return;
   }
   __shared__ float s_max[MOE_THREADS / 64];
@@ -612,7 +612,7 @@ static __device__ __forceinline__ void moe_routeq_body(
     }
   }
 }
-#define MOE_ROUTEQ(name, RM, PART)                                                                                          \
+#define MOE_ROUTEQ(name, RM)                                                                                                \
   extern "C" __global__ __launch_bounds__(MOE_THREADS) void name(                                                      \
       const unsigned short *__restrict__ logits, int T, int e_lo, int e_loc, int tile_blocks, int with_shared,          \
       int *__restrict__ topk_ids, float *__restrict__ topk_w, int *__restrict__ route_pos, int *__restrict__ row_tok,   \
@@ -620,12 +620,12 @@ static __device__ __forceinline__ void moe_routeq_body(
       int *__restrict__ tile_rows, int *__restrict__ expert_cnt, int *__restrict__ meta, int *__restrict__ blk_cnt,     \
       int *__restrict__ rank, int *__restrict__ arrive, const unsigned short *__restrict__ x,                           \
       unsigned char *__restrict__ q, float *__restrict__ scale, int k) {                                                \
-    moe_routeq_body<RM, PART>(logits, T, e_lo, e_loc, tile_blocks, with_shared, topk_ids, topk_w, route_pos, row_tok,         \
+    moe_routeq_body<RM>(logits, T, e_lo, e_loc, tile_blocks, with_shared, topk_ids, topk_w, route_pos, row_tok,               \
                         row_route, tile_expert, tile_row0, tile_rows, expert_cnt, meta, blk_cnt, rank, arrive, x, q,    \
                         scale, k);                                                                                      \
   }
-MOE_ROUTEQ(moe_iu8_routeq_topk8_sort_e128, false, false)
-MOE_ROUTEQ(moe_iu8_routeq_rm_topk8_sort_e128, true, false)
+MOE_ROUTEQ(moe_iu8_routeq_topk8_sort_e128, false)
+MOE_ROUTEQ(moe_iu8_routeq_rm_topk8_sort_e128, true)
 #undef MOE_ROUTEQ
 // The part form of the same launch (above 128 tokens, row-major codes): workgroups of 256 threads, the first
 // ceil(T / 32) route 32 tokens each (moe_route_body), each of the T behind them quantises one token row, a thread
