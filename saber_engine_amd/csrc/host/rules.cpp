@@ -324,24 +324,33 @@ uint32_t pf_split(bool w8, uint32_t m, uint32_t n, uint32_t k, const PfVariant *
 }
 
 // The prefill cell of a shape: the tile whose estimated time is least. A launch's time is a fixed
-// cost plus the largest of three: the matrix work of the busiest CU over the cell's measured rate
+// cost, a cost a tile the busiest workgroup runs (pipeline fill, epilogue, tile switch: what a cell pays
+// whatever K is) and the largest of three: the matrix work of the busiest CU over the cell's measured rate
 // (co-resident workgroups of a two-a-CU cell share the CU's matrix units), the bytes that CU pulls in
 // (its tiles' A rows and W columns, K deep) over what one CU takes from L2, and all tiles' bytes over
 // what the L2s deliver together -- the last two are what bind for M up to about 512, where the A rows
 // are re-read once a column block, so small tiles that put every CU to work win there and the large
-// ones take over as the matrix work grows. The constants are this card's speed data (least-squares fit
-// of 520 timings: the four 27B-class shapes x M = 65..8192 x ten cells; the picked cell is within 2 %
-// of the best measured one on 47 of the 52 shapes and within 13 % on all), as the reference keeps its
-// band tables (crates/saber-kernels/src/macaq_iu8.rs:150-212).
+// ones take over as the matrix work grows. The constants are this card's speed data, one table a weight
+// kind (int8 weights are twice the bytes a tile and have no unpack: the cells rank differently), fitted to
+// sustained timings of every cell on the four 27B-class shapes x 14 row counts from 65 to 8,192 (W4: 574
+// timings, the pick is the fastest measured cell on 52 of 56 shape x M points and within 3.4 % on all;
+// W8, output-side shapes: every pick the fastest), as the reference keeps its band tables
+// (crates/saber-kernels/src/macaq_iu8.rs:150-212). One table for both kinds had sent the int8-weight
+// O and down projections at 2,048 rows to the 128 x 320 cell, 17-22 % behind the 256 x 160 cell there.
 const PfVariant *pf_cell(bool w8, uint32_t m, uint32_t n, uint32_t k) {
-  static const struct { const char *tile; double tops_per_cu; } CELLS[] = {
-      {"tn4_lbk64", 13.27}, {"t256x320", 12.8}, {"t256x224", 11.27}, {"t128x320", 10.45}, {"t256x160", 9.98},
-      {"t128x256", 8.8},    {"t128x128", 7.85},
-      {"t128x128_o2", 8.68}, {"t128x64_s", 6.21}, {"t64x128_s", 7.24}, {"t64x64_s", 5.96}};
-  constexpr double FIXED_US = 2.78, CU_GBPS = 90.0, L2_TBPS = 17.7;
+  struct Cell { const char *tile; double tops_per_cu, tile_us; };
+  struct Law { double fixed_us, cu_gbps, l2_tbps, lone; Cell cells[11]; };
+  static const Law W4 = {0.000, 90.000, 15.307, 1.182,
+                         {{"tn4_lbk64", 13.221, 1.279}, {"t256x320", 12.785, 0.000}, {"t256x224", 12.417, 6.000}, {"t128x320", 10.591, 6.000}, {"t256x160", 10.445, 4.215}, {"t128x256", 10.338, 6.000}, {"t128x128", 8.480, 1.193}, {"t128x128_o2", 10.406, 3.795}, {"t128x64_s", 5.778, 2.108}, {"t64x128_s", 6.950, 2.992}, {"t64x64_s", 6.696, 0.873}}};
+  static const Law W8 = {1.532, 93.036, 20.882, 1.564,
+                         {{"tn4_lbk64", 15.504, 4.658}, {"t256x320", 12.800, 0.000}, {"t256x224", 11.270, 0.000}, {"t128x320", 8.171, 2.815}, {"t256x160", 11.863, 0.544}, {"t128x256", 9.363, 0.196}, {"t128x128", 9.013, 0.068}, {"t128x128_o2", 9.722, 0.808}, {"t128x64_s", 5.244, 1.816}, {"t64x128_s", 5.976, 0.853}, {"t64x64_s", 5.960, 0.040}}};
+  const Law &law = w8 ? W8 : W4;
+  double quarter_rate = 0;
+  for (const auto &c : law.cells)
+    if (!strcmp(c.tile, "t128x128")) quarter_rate = c.tops_per_cu;
   const PfVariant *best = nullptr;
   double best_t = 0;
-  for (const auto &c : CELLS) {
+  for (const auto &c : law.cells) {
     const PfVariant *v = pf_variant(fmt("macaq_iu8_pf_%s_%s", w8 ? "w8" : "w4", c.tile));
     if (!v) continue;
     const double bm = v->block_m(), bn = v->block_n();
@@ -353,15 +362,15 @@ const PfVariant *pf_cell(bool w8, uint32_t m, uint32_t n, uint32_t k) {
     // 128 x 128 cell, each a quarter of the work at that cell's rate
     const uint64_t q = tiles / grid, rem = tiles - q * grid;
     if (!strcmp(c.tile, "tn4_lbk64") && q >= 1 && rem > 0 && 2 * rem <= grid)
-      cu_tiles = (double)q + (double)((4 * rem + grid - 1) / grid) * 0.25 * (13.27 / 7.85);
+      cu_tiles = (double)q + (double)((4 * rem + grid - 1) / grid) * 0.25 * (c.tops_per_cu / quarter_rate);
     const double tile_bytes = bm * k + bn * k * (w8 ? 1.0 : 0.5);
     const double t_mfma = cu_tiles * bm * bn * k * 2.0 / (c.tops_per_cu * 1e6);
-    const double t_cu = cu_tiles * tile_bytes / (CU_GBPS * 1e3);
-    const double t_l2 = (double)tiles * tile_bytes / (L2_TBPS * 1e6);
+    const double t_cu = cu_tiles * tile_bytes / (law.cu_gbps * 1e3);
+    const double t_l2 = (double)tiles * tile_bytes / (law.l2_tbps * 1e6);
     // the two-a-CU 128 x 128 cell alone on a CU (no more workgroups than CUs) has four waves to hide
-    // its latencies with and measured 9-12 % behind the eight-wave 128 x 128 cell there
-    const double lone = (!strcmp(c.tile, "t128x128_o2") && grid <= CU_COUNT) ? 1.15 : 1.0;
-    const double t = FIXED_US + lone * std::max(t_mfma, std::max(t_cu, t_l2));
+    // its latencies with and measured well behind the eight-wave 128 x 128 cell there
+    const double lone = (!strcmp(c.tile, "t128x128_o2") && grid <= CU_COUNT) ? law.lone : 1.0;
+    const double t = law.fixed_us + (double)per_wg * c.tile_us + lone * std::max(t_mfma, std::max(t_cu, t_l2));
     if (!best || t < best_t) best = v, best_t = t;
   }
   return best;
