@@ -130,6 +130,10 @@ std::string band_toml() {
   put(o, "rows_max", 4);
   put(o, "staged_code_bytes", 20 * 1024);
   put(o, "column_blocks_per_workgroup_max", 8);
+  o += "# macaq_iu8_decq_{w4,w8}_r1: one row; the row's codes are made just in time inside the weight stream\n";
+  put(o, "r1_rows", 1);
+  put(o, "r1_k_min", FUSED_R1_MIN_K);
+  put(o, "r1_k_max", 20 * 1024);
   o += "# macaq_iu8_decq_{w4,w8}_tm1_a80: the same launch with 80 KiB of staged codes; the kernel holds up to 16\n";
   o += "# rows, the law launches it for up to 4 (every workgroup repeats the quantisation: more rows lose to\n";
   o += "# producer + GEMV)\n";

@@ -434,7 +434,14 @@ int resolve_fused(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc 
   if (int rc = check_shape(op, m, n, k)) return rc;
   if (!fused_holds(m, k))
     return fail(SABER_IU8_E_RULE, fmt("%s: %u rows of %u are not a fused launch (up to 4 rows, 20 KiB of codes or 80 KiB)", op, m, k));
-  const std::string name = fmt("macaq_iu8_decq_%s_tm1%s", wkind == SABER_IU8_W8 ? "w8" : "w4", fused_small_holds(m, k) ? "" : "_a80");
+  // one long row: the form that makes the row's codes just in time inside the weight stream (`_r1`). Measured on
+  // this card against the several-row form at one row (cold weights, graph replay, N = 5120): K = 8,192 6.47
+  // against 6.91 us, 12,288 7.82 against 8.38, 17,408 9.88 against 10.7-11.4, 20,480 10.97 against 11.83; at
+  // K = 5,120 it loses (5.64 against 5.17: there a thread of the several-row form converts one piece at most,
+  // which is what this form's first chunk costs, and its two column groups convert every piece twice)
+  const std::string name = m == 1 && k >= FUSED_R1_MIN_K && fused_small_holds(m, k)
+                               ? fmt("macaq_iu8_decq_%s_r1", wkind == SABER_IU8_W8 ? "w8" : "w4")
+                               : fmt("macaq_iu8_decq_%s_tm1%s", wkind == SABER_IU8_W8 ? "w8" : "w4", fused_small_holds(m, k) ? "" : "_a80");
   memset(d, 0, sizeof *d);
   copy_name(d->op, sizeof d->op, op);
   copy_name(d->plugin, sizeof d->plugin, "macaq_iu8");

@@ -32,6 +32,7 @@ uint32_t pf_split(bool w8, uint32_t m, uint32_t n, uint32_t k, const PfVariant *
 constexpr uint32_t DECODE_MAX_M = 64;  // the decode band's last row count (macaq_iu8.rs:31)
 constexpr uint32_t KS_MAX = 8;         // the largest grid-level split (macaq_iu8.rs:44)
 constexpr uint32_t CU_COUNT = 256;     // MI355X compute units
+constexpr uint32_t FUSED_R1_MIN_K = 8192;   // rows at least this long take the one-row fused decode form
 
 // Grid-level split of a decode GEMM whose grid has `nblk` column blocks.
 uint32_t decode_split(uint32_t m, uint32_t n, uint32_t k, uint32_t nblk, uint32_t kw);

@@ -381,6 +381,9 @@ static int launch_guard(const LoadedKernel &lk, const saber_iu8_desc *d) {
     if (!strcmp(d->args[i].name, "k")) k = d->args[i].ival;
   }
   const bool a80 = strstr(d->kernel, "_a80") != nullptr;
+  const size_t len = strlen(d->kernel);
+  if (len > 3 && !strcmp(d->kernel + len - 3, "_r1") && m != 1)
+    return fail(SABER_IU8_E_RULE, fmt("%s: the one-row form, got %lld rows", d->kernel, (long long)m));
   if (m <= 0 || n <= 0 || k <= 0 || !fused_form_holds(a80, (uint32_t)m, (uint32_t)k))
     return fail(SABER_IU8_E_RULE, fmt("%s: %lld rows of %lld do not fit the fused form", d->kernel, (long long)m, (long long)k));
   const int64_t nblk = (n + 31) / 32;

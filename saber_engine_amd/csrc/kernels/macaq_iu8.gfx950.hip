@@ -25,6 +25,7 @@
 //           in registers just in time; the output tile goes out through LDS as whole row segments.
 #include "iu8_gemm.h"
 #include "iu8_decq.h"
+#include "iu8_decq1.h"
 #include "iu8_pf32.h"
 #include "iu8_dense_defs.h"
 
@@ -60,6 +61,21 @@ IU8_DECQA(macaq_iu8_decq_w4_tm1_a80, false, 1, 8, 16, 4, 80)
 IU8_DECQA(macaq_iu8_decq_w8_tm1_a80, true, 1, 8, 16, 2, 80)
 #undef IU8_DECQX
 #undef IU8_DECQA
+
+// One row (`_r1`, the GEMV of a single token): the same launch with the row's codes made just in time --
+// a wave converts only the K steps it multiplies, a chunk of 4 steps ahead of their use, inside the weight
+// stream (iu8_decq1.h). In front of the first MFMA stand the row's arrival, one meeting of the waves'
+// maxima and one chunk's conversion instead of the whole row's conversion behind two barriers.
+#define IU8_DECQ1(name, W8, KW, WPB, D)                                                                            \
+  extern "C" __global__ __launch_bounds__(WPB * 64) __attribute__((amdgpu_waves_per_eu(4, 4))) void name(          \
+      const unsigned short *__restrict__ x, const unsigned char *__restrict__ w, const float *__restrict__ ws,     \
+      unsigned char *__restrict__ q, float *__restrict__ scale, unsigned short *__restrict__ c, int m, int n,      \
+      int k) {                                                                                                     \
+    iu8_decq1_body<W8, KW, WPB, D>(x, w, ws, q, scale, c, n, k);                                                   \
+  }
+IU8_DECQ1(macaq_iu8_decq_w4_r1, false, 8, 16, 4)
+IU8_DECQ1(macaq_iu8_decq_w8_r1, true, 8, 16, 2)
+#undef IU8_DECQ1
 
 // Cells with K split over gridDim.z (symbol suffix `_ks`, the decode kernarg list: the two workspaces
 // in front of c), for the rows between the regimes, where few tiles leave CUs idle. Measured, the

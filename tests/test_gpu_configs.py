@@ -45,7 +45,7 @@ def test_config1_decode_layer_set(ctx, M):
 @pytest.mark.parametrize("M", [1, 4])
 def test_config1_decode_layer_set_as_the_fused_launches_the_benchmark_times(ctx, M):
     """The hot path as bench.py launches it: one fused quant + GEMV launch a linear
-    (macaq_iu8_decq_w4_tm1), on the four full layer shapes, against the oracle."""
+    (macaq_iu8_decq_w4_r1 at one row, macaq_iu8_decq_w4_tm1[_a80] at four), on the four full layer shapes, against the oracle."""
     for name, n, k in synth.LAYER_LINEARS:
         assert iu8.fused_holds(M, k)
         say(f"config 1, fused launch: {name} M={M} N={n} K={k}")
@@ -54,7 +54,8 @@ def test_config1_decode_layer_set_as_the_fused_launches_the_benchmark_times(ctx,
         x, wf, ws = dev_bf16_bits(case["X"]), dev_u8(iu8.repack_w4(case["W"])), dev_f32(case["ws"])
         c = torch.full((M, n), 0x7FC0, dtype=torch.int16, device="cuda")
         d = iu8.resolve_fused(iu8.W4, M, n, k)
-        assert d.kernel == (b"macaq_iu8_decq_w4_tm1" if iu8.fused_small_holds(M, k) else b"macaq_iu8_decq_w4_tm1_a80")   # down at 4 rows
+        # one long row (down): the just-in-time form; down at 4 rows: the 80 KiB form
+        assert d.kernel == (b"macaq_iu8_decq_w4_r1" if M == 1 and k >= 8192 else b"macaq_iu8_decq_w4_tm1" if iu8.fused_small_holds(M, k) else b"macaq_iu8_decq_w4_tm1_a80")
         for a in ("q", "scale"):                # as the benchmark launches it: no optional outputs
             d.arg(a).kind = iu8.ARG_NULL_BUFFER
         ctx.launch(d, dict(x=x.data_ptr(), w=wf.data_ptr(), ws=ws.data_ptr(), c=c.data_ptr()))

@@ -129,6 +129,95 @@ def test_fused_decode_linear_80_kib_form(ctx, M, N, K, grid):
     assert e.value.code == iu8.E_RULE
 
 
+@pytest.mark.parametrize("N,K,grid", [(5120, 17408, None),    # the benchmark's GEMV: 17 steps a k-wave, five chunks, the last of one step
+                                        (96, 20480, None),      # the longest row the form holds: 20 steps a k-wave
+                                        (7168, 5120, None),     # 5 steps a k-wave: one chunk ahead, then one step
+                                        (1040, 128, 5),         # one K step: seven k-waves without a step, several blocks a workgroup
+                                        (1104, 640, 16),        # five k-waves with one step; an odd number of 16-column tiles
+                                        (2080, 1536, 9),        # 12 steps: k-waves of 2 and 1; up to 8 blocks a workgroup
+                                        (34816, 5120, None),    # 1,088 blocks: 218 workgroups x 5, later blocks on codes in place
+                                        (272, 4224, 3),         # 33 steps: one k-wave with 5, the others 4
+                                        (64, 16512, 2)])        # 129 steps: one k-wave with 17
+def test_fused_decode_linear_one_row_form(ctx, N, K, grid):
+    """macaq_iu8_decq_{w4,w8}_r1: the row's codes made just in time, a chunk of 4 steps ahead of the MFMAs,
+    by the waves that multiply them; the bytes of producer + GEMV, optional outputs included."""
+    for w8 in (False, True):
+        say(f"fused decode linear, one-row form: N={N} K={K} grid={grid} w8={w8}")
+        case = synth.dense_case(1, N, K, w8=w8, seed=N + K)
+        r = ref.linear(case["X"], case["W"], case["ws"], w8, threads=8)
+        wk, tag = (iu8.W8, "w8") if w8 else (iu8.W4, "w4")
+        x, wf, ws = dev_bf16_bits(case["X"]), dev_u8(iu8.repack_weights(case["W"], w8)), dev_f32(case["ws"])
+        d = iu8.resolve_fused(wk, 1, N, K)
+        assert d.kernel.decode() == (f"macaq_iu8_decq_{tag}_r1" if K >= 8192 else f"macaq_iu8_decq_{tag}_tm1") and d.block[0] == 1024
+        d = iu8.describe_raw(f"macaq_iu8_decq_{tag}_r1", (grid or d.grid[0], 1, 1), 1024, m=1, n=N, k=K)   # short rows reach it by name
+        c = torch.full((1, N), 0x7FC0, dtype=torch.int16, device="cuda")
+        q = torch.full((iu8.a_bytes(1, K),), 0x55, dtype=torch.uint8, device="cuda")
+        s = torch.zeros(1, dtype=torch.float32, device="cuda")
+        ctx.launch(d, dict(x=x.data_ptr(), w=wf.data_ptr(), ws=ws.data_ptr(), c=c.data_ptr(), q=q.data_ptr(), scale=s.data_ptr()))
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(host_u16(c), r["C"])
+        np.testing.assert_array_equal(iu8.unpack_a(q.cpu().numpy(), 1, K), r["q"])
+        np.testing.assert_array_equal(s.cpu().numpy().view(np.uint32), r["a_scale"].view(np.uint32))
+        # ... and the same bytes as the several-row form at one row
+        d2 = iu8.describe_raw(f"macaq_iu8_decq_{tag}_tm1", (d.grid[0], 1, 1), 1024, m=1, n=N, k=K)
+        c2 = torch.full((1, N), 0x7FC0, dtype=torch.int16, device="cuda")
+        for a in ("q", "scale"):
+            d2.arg(a).kind = iu8.ARG_NULL_BUFFER
+        ctx.launch(d2, dict(x=x.data_ptr(), w=wf.data_ptr(), ws=ws.data_ptr(), c=c2.data_ptr()))
+        torch.cuda.synchronize()
+        assert torch.equal(c, c2)
+    d = iu8.describe_raw("macaq_iu8_decq_w4_r1", (1, 1, 1), 1024, m=2, n=64, k=128)   # more than one row: refused by name
+    with pytest.raises(iu8.IU8Error) as e:
+        ctx.launch(d, dict(x=x.data_ptr(), w=wf.data_ptr(), ws=ws.data_ptr(), c=c.data_ptr(), q=q.data_ptr(), scale=s.data_ptr()))
+    assert e.value.code == iu8.E_RULE
+
+
+def test_one_row_form_on_ties_nan_and_infinity(ctx):
+    """The one-row form on rows of crafted ties (the reciprocal path must hand them to the divide) and on rows
+    with NaNs and infinities (the packed maximum's NaN branch, an infinite scale): codes, scale and output
+    against the oracle's."""
+    say("one-row form: ties, nan, inf")
+    K, N = 2048, 64
+    rows = []
+    for amax in (127.0, 254.0, 63.5, 1.984375):
+        sc = np.float32(amax) / np.float32(127.0)
+        ks = np.arange(K, dtype=np.float32) % 126
+        xr = (ks + np.float32(0.5)) * sc * np.where(np.arange(K) % 2 == 0, 1, -1).astype(np.float32)
+        xr[0] = amax
+        b0 = synth.f32_to_bf16_bits(xr).astype(np.uint16)
+        rows.append(b0)
+        for step in (1, -1):                      # the neighbouring bf16 values of every tie
+            b = (b0.astype(np.int32) + step).astype(np.uint16)
+            b[0] = b0[0]
+            rows.append(b)
+    rng = np.random.default_rng(5)
+    base = synth.f32_to_bf16_bits((rng.standard_normal((6, K)) * 3).astype(np.float32))
+    base[0, 17] = 0x7FC0                      # a lone NaN
+    base[1, K - 1] = 0x7F80                   # an infinity in the last piece
+    base[2, 0], base[2, 1] = 0x7FC0, 0xFF80   # both in one pair
+    base[3, :] = 0x7FC0                       # nothing but NaNs: the maximum stays 0
+    base[4, np.arange(0, K, 129)] = 0xFFC1    # negative NaNs with a payload in many pieces
+    base[5, :] = 0                            # an all-zero row: scale 1e-30, codes 0
+    rows += list(base)
+    W, wsc = synth.weights(np.random.default_rng(3), N, K, False)
+    wf, wsd = dev_u8(iu8.repack_w4(W)), dev_f32(wsc)
+    for i, row in enumerate(rows):
+        X = np.ascontiguousarray(row.reshape(1, K))
+        want_q, want_s = ref.quant_bf16(X)
+        xs = dev_bf16_bits(X)
+        q = torch.zeros(iu8.a_bytes(1, K), dtype=torch.uint8, device="cuda")
+        s = torch.zeros(1, dtype=torch.float32, device="cuda")
+        c = torch.zeros((1, N), dtype=torch.int16, device="cuda")
+        d = iu8.describe_raw("macaq_iu8_decq_w4_r1", (2, 1, 1), 1024, m=1, n=N, k=K)
+        ctx.launch(d, dict(x=xs.data_ptr(), w=wf.data_ptr(), ws=wsd.data_ptr(), c=c.data_ptr(), q=q.data_ptr(), scale=s.data_ptr()))
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(s.cpu().numpy().view(np.uint32), want_s.view(np.uint32), err_msg=f"row {i}")
+        np.testing.assert_array_equal(iu8.unpack_a(q.cpu().numpy(), 1, K), want_q, err_msg=f"row {i}")
+        if i < len(rows) - 6 or i == len(rows) - 1:    # finite rows: the output too (NaN payloads of c are not pinned)
+            r = ref.linear(X, W, wsc, False, threads=4)
+            np.testing.assert_array_equal(host_u16(c), r["C"], err_msg=f"row {i}")
+
+
 def test_fused_form_refuses_what_it_does_not_hold(ctx):
     assert not iu8.fused_holds(5, 1024) and not iu8.fused_holds(4, 20608) and not iu8.fused_holds(2, 41088)
     assert iu8.fused_holds(1, 17408) and iu8.fused_holds(4, 5120) and iu8.fused_holds(2, 10240)
