@@ -343,9 +343,11 @@ int saber_iu8_linear_fused(saber_iu8_ctx *ctx, int wkind, const void *x_bf16, co
  * tap (NULL: not stored). The workgroups meet through `state` (an arrival word a workgroup), so all
  * of them must be resident at once: the launch is refused (SABER_IU8_E_RULE) on a device that does
  * not hold the grid. A wait lasts at most `spin` polls (0: the default, about a second); a launch
- * that gives up leaves a non-zero word at state + SABER_IU8_MLP_CHAIN_STATUS_OFFSET and an undefined
- * c: after synchronising, a caller that shares the GPU with other work checks that word and, if set,
- * zeroes `state` and runs the three launches. Launches that share one `state` must not overlap.
+ * that gives up leaves a non-zero word at state + SABER_IU8_MLP_CHAIN_STATUS_OFFSET and every element
+ * of c a bf16 NaN (0x7FC0) -- and so does every later launch on that state block while the word is
+ * set, e.g. the replays of a captured graph: the failure shows in the output itself. A caller that
+ * finds the word set (or NaNs where the inputs had none) zeroes `state` and runs the three launches.
+ * Launches that share one `state` must not overlap.
  * Asynchronous. */
 #define SABER_IU8_MLP_CHAIN_STATE_BYTES (13 * 1024)
 #define SABER_IU8_MLP_CHAIN_STATUS_OFFSET (12 * 1024)
@@ -375,7 +377,11 @@ int saber_iu8_gemm_workspace(int wkind, uint32_t m, uint32_t n, uint32_t k, uint
 
 /* C[m,n] bf16 = epilogue(A . W^T): a/as from the producer, w in the gfx950 fragment order, ws f32
  * [n]. `partial` (scratch) and `counter` (zeroed once by the caller, left zero) may be NULL when
- * saber_iu8_gemm_workspace reports 0. */
+ * saber_iu8_gemm_workspace reports 0.
+ * Non-finite rows: a row whose scale is infinite (an infinity among its activations) gives infinities
+ * where its accumulator is not zero and NaNs where it is (0 * inf), exactly where the contract's two
+ * multiplies make them (crates/saber-kernels/hip/macaq_iu8.hip:20-24); that an element of c is a NaN is
+ * defined, its sign and payload are not (they are the multiplier's that made it). */
 int saber_iu8_gemm(saber_iu8_ctx *ctx, int wkind, const void *a, const float *as, const void *w, const float *ws,
                    void *c_bf16, uint32_t m, uint32_t n, uint32_t k, void *partial, void *counter, void *stream);
 
@@ -392,6 +398,12 @@ int saber_iu8_gemm(saber_iu8_ctx *ctx, int wkind, const void *a, const float *as
 int saber_iu8_gemm_static(saber_iu8_ctx *ctx, int wkind, const void *a, const float *as, const void *w, const float *ws,
                           void *c_bf16, uint32_t m, uint32_t n, uint32_t k, void *stream);
 uint64_t saber_iu8_static_workspace_bytes(void);
+/* The static array's arrival counters back to zero, by a fill kernel on `stream` (no memset, so it may be
+ * captured): recovery for a process in which a split launch was cut short between a tile's first and last
+ * arrival (a device error, a destroyed stream), which leaves counters no later launch brings back to zero.
+ * Not needed in ordinary use -- every kernel leaves its counters at zero. Belongs to saber_iu8_gemm_static
+ * and, like it, has no counterpart in the reference. SABER_IU8_E_NOTLOADED when the device has no array. */
+int saber_iu8_static_workspace_reset(saber_iu8_ctx *ctx, void *stream);
 
 /* The raw int32 accumulators of the same GEMM (16 * sum(a*w) for W4, sum(a*w) for W8), int32
  * [m,n]: the parity tap. No counterpart in the reference's shipped object (its tests replay

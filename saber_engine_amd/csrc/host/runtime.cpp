@@ -30,6 +30,7 @@ struct saber_iu8_ctx {
   std::vector<hipModule_t> modules;
   std::map<std::string, LoadedKernel> fn;
   saber_iu8_counters counters{};
+  std::string static_ws_error;  // why this device has no static workspace (empty: it has one)
 };
 
 static int hip_fail(const char *what, hipError_t e) {
@@ -295,9 +296,6 @@ int saber_iu8_open(const char *prebuilt_dir, int device, saber_iu8_ctx **out) {
   }
   closedir(dp);
   std::sort(manifests.begin(), manifests.end());
-  // the library's static split-K workspace on this device (saber_iu8_gemm_static): its address is
-  // taken here, once a device, with the device current
-  if (int rc = static_ws_init(device)) return rc;
   saber_iu8_ctx *ctx = new saber_iu8_ctx();
   ctx->device = device;
   ctx->arch = arch;
@@ -316,6 +314,11 @@ int saber_iu8_open(const char *prebuilt_dir, int device, saber_iu8_ctx **out) {
     saber_iu8_close(ctx);
     return fail(SABER_IU8_E_NOTLOADED, msg);
   }
+  // The library's static split-K workspace on this device (saber_iu8_gemm_static): its address is taken here,
+  // once a device, with the device current and behind the plugin set, whose refusals say more about a device
+  // this library is not built for than a failed symbol look-up would. A failure is kept, not returned: only
+  // saber_iu8_gemm_static needs the array, and it then says why it has none.
+  if (static_ws_init(device) != 0) ctx->static_ws_error = last_error();
   *out = ctx;
   return 0;
 }
@@ -528,8 +531,14 @@ int saber_iu8_gemm_static(saber_iu8_ctx *ctx, int wkind, const void *a, const fl
     (is_partial ? partial : counter) = is_partial ? static_ws_partial(ctx->device) : static_ws_counter(ctx->device);
   }
   if (d.n_workspaces && (!partial || !counter))
-    return fail(SABER_IU8_E_NOTLOADED, fmt("gemm_static: the static workspace of device %d was not set up", ctx->device));
+    return fail(SABER_IU8_E_NOTLOADED, fmt("gemm_static: the static workspace of device %d was not set up%s%s", ctx->device,
+                                           ctx->static_ws_error.empty() ? "" : ": ", ctx->static_ws_error.c_str()));
   return launch_gemm(ctx, d, a, as, w, ws, c, partial, counter, stream);
+}
+
+int saber_iu8_static_workspace_reset(saber_iu8_ctx *ctx, void *stream) {
+  if (!ctx) return fail(SABER_IU8_E_ARG, "static_workspace_reset: null context");
+  return static_ws_reset(ctx->device, stream);
 }
 
 uint64_t saber_iu8_static_workspace_bytes(void) { return STATIC_WS_BYTES; }

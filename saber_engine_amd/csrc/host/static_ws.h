@@ -13,6 +13,8 @@ constexpr size_t STATIC_WS_BYTES = STATIC_WS_COUNTER_BYTES + STATIC_WS_PARTIAL_B
 
 // With `device` current: takes the array's address on it (once) and zero-fills it. 0 or an error code.
 int static_ws_init(int device);
+// Zero-fills the arrival counters on `stream` with a kernel (capture-legal). 0 or an error code.
+int static_ws_reset(int device, void *stream);
 void *static_ws_partial(int device);  // nullptr before static_ws_init(device)
 void *static_ws_counter(int device);
 

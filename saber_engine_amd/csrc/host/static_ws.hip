@@ -14,6 +14,8 @@
 // enters a captured graph.
 #include <hip/hip_runtime.h>
 
+#include <mutex>
+
 #include "../../../include/saber_iu8.h"
 #include "static_ws.h"
 #include "util.h"
@@ -28,6 +30,7 @@ __global__ void static_ws_fill(unsigned *p, size_t n4) {
 
 constexpr int MAX_DEVICES = 64;
 void *g_ptr[MAX_DEVICES];  // the array's address on each device, 0 = not asked for yet
+std::mutex g_mu;           // two threads opening contexts on one device: one of them sets the array up, the other waits
 
 }  // namespace
 
@@ -35,6 +38,9 @@ namespace iu8 {
 
 int static_ws_init(int device) {
   if (device < 0 || device >= MAX_DEVICES) return fail(SABER_IU8_E_ARG, fmt("static workspace: device %d out of range", device));
+  // held over the fill: a second opener must not see the address before the zeros are there, nor fill again
+  // under a launch of the first that is counting arrivals
+  std::lock_guard<std::mutex> lock(g_mu);
   if (g_ptr[device]) return 0;
   // the caller has made `device` current
   void *p = nullptr;
@@ -46,6 +52,22 @@ int static_ws_init(int device) {
   if ((e = hipGetLastError()) != hipSuccess || (e = hipStreamSynchronize(nullptr)) != hipSuccess)
     return fail(SABER_IU8_E_HIP, fmt("static workspace fill on device %d: HIP status %d (%s)", device, (int)e, hipGetErrorString(e)));
   g_ptr[device] = p;
+  return 0;
+}
+
+// The arrival counters back to zero, on the caller's stream, by the fill kernel (no memset: a caller may be
+// capturing): for a process that had a launch cut short (a device error, a killed stream) between a tile's
+// first arrival and its last, which leaves counters that no later launch would bring back to zero.
+int static_ws_reset(int device, void *stream) {
+  void *p = nullptr;
+  {
+    std::lock_guard<std::mutex> lock(g_mu);
+    p = device >= 0 && device < MAX_DEVICES ? g_ptr[device] : nullptr;
+  }
+  if (!p) return fail(SABER_IU8_E_NOTLOADED, fmt("static workspace of device %d was not set up", device));
+  hipLaunchKernelGGL(static_ws_fill, dim3(16), dim3(256), 0, (hipStream_t)stream, (unsigned *)p, STATIC_WS_COUNTER_BYTES / 4);
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(SABER_IU8_E_HIP, fmt("static workspace reset on device %d: HIP status %d (%s)", device, (int)e, hipGetErrorString(e)));
   return 0;
 }
 

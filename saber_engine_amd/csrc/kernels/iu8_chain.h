@@ -39,7 +39,9 @@
 // A wait polls at most `spin` times (a bounded wait: about a microsecond a poll); past that the
 // workgroup raises the status word and leaves, and so does every other one at its next look, so a
 // launch that cannot complete ends instead of hanging; nothing is cleared then, and the host zeroes
-// the state block before it is used again.
+// the state block before it is used again. Such a launch -- and every later one on a state block whose
+// status is still raised -- fills its output rows with bf16 NaNs (0x7FC0), so the failure shows in `c`
+// itself, also to a caller that replays a captured graph and never reads the state block.
 //
 // The state block (IU8_CHAIN_STATE_BYTES, zero before the first launch):
 //   [0, 8 KiB)        512 slots of 4 floats: a workgroup's maxima of |p|, a row

@@ -221,7 +221,20 @@ __device__ __forceinline__ void iu8_decq_body(const unsigned short *__restrict__
 #pragma unroll
       for (int i = 0; i < D; ++i)
         if (i < TT) issue(i);
-      if (!hook.wait()) return;  // a producer never arrived (the launch reports it): give up as a whole
+      if (!hook.wait()) {
+        // A producer never arrived, or the state block still carries an earlier launch's raised status: the
+        // launch gives up as a whole and says so where the caller looks -- every output this workgroup owns
+        // becomes a bf16 NaN (0x7FC0), so a replayed graph that can no longer complete does not hand back
+        // stale or half-written rows as if they were results. (The status word says the same to a host that
+        // reads the state block.)
+        constexpr int BC = WNB * NT * 16;
+        for (int i = tid; i < nb * BC * M; i += NTHR) {
+          const int b = i / (BC * M), r = (i / BC) % M, cc = i % BC;
+          const int n = ((int)blockIdx.x + b * G) * BC + cc;
+          if (n < N) C[(size_t)r * N + n] = 0x7FC0;
+        }
+        return;
+      }
 #pragma unroll
       for (int p = 0; p < X_PER; ++p)
         if (p * NTHR + tid < x_pieces) xreg[p] = iu8_decq_ld_coherent((const iu8_v4u *)X + p * NTHR + tid);

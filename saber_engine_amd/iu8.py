@@ -114,6 +114,7 @@ def lib():
         L.saber_iu8_rowscale.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32, C.c_uint32, C.c_void_p]
         L.saber_iu8_linear_prefill_fused.argtypes = [C.c_void_p, C.c_int] + [C.c_void_p] * 5 + [C.c_uint32] * 3 + [C.c_void_p]
         L.saber_iu8_gemm_static.argtypes = [C.c_void_p, C.c_int] + [C.c_void_p] * 5 + [C.c_uint32] * 3 + [C.c_void_p]
+        L.saber_iu8_static_workspace_reset.argtypes = [C.c_void_p, C.c_void_p]
         L.saber_iu8_static_workspace_bytes.restype = C.c_uint64
         L.saber_iu8_gemm_acc.argtypes = [C.c_void_p, C.c_int] + [C.c_void_p] * 3 + [C.c_uint32] * 3 + [C.c_void_p]
         L.saber_iu8_fused_holds.argtypes = [C.c_uint32, C.c_uint32]
@@ -402,6 +403,11 @@ class Context:
     def gemm_static(self, wkind, a, a_scale, w, w_scale, c, m, n, k, stream=0):
         """gemm() with the split-K workspaces in the library's static device array: allocates nothing."""
         _check(lib().saber_iu8_gemm_static(self._h, wkind, a, a_scale, w, w_scale, c, m, n, k, stream))
+
+    def static_workspace_reset(self, stream=0):
+        """The static array's arrival counters back to zero (a fill kernel on `stream`): recovery after a split
+        launch that was cut short."""
+        _check(lib().saber_iu8_static_workspace_reset(self._h, stream))
 
     def gemm_pair(self, a, a_scale, w, w_scale, c, n, w_b, w_scale_b, c_b, n_b, m, k, stream=0):
         _check(lib().saber_iu8_gemm_pair(self._h, a, a_scale, w, w_scale, c, n, w_b, w_scale_b, c_b, n_b, m, k, stream))

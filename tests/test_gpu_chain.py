@@ -94,12 +94,39 @@ def test_chain_meeting_gives_up_after_its_poll_limit_and_says_so(ctx):
     M, H, I = 1, 1024, 2048
     say(f"mlp chain poll limit M={M} H={H} I={I}")
     mlp = Mlp(M, H, I, seed=5)
+    mlp.c.zero_()
     mlp.chain(ctx, spin=1)
     assert mlp.state[STATUS].item() != 0, "a wait that ran out of polls raises the status word"
+    assert (mlp.c == 0x7FC0).all().item(), "a launch that gave up fills its output with bf16 NaNs"
+    # a later launch on the state block as it was left (a graph replay that nobody checked): it cannot
+    # complete either, and its output says so instead of carrying stale rows
+    mlp.c.zero_()
+    mlp.chain(ctx)
+    assert mlp.state[STATUS].item() != 0 and (mlp.c == 0x7FC0).all().item()
     mlp.state.zero_()
     mlp.chain(ctx)
     assert not mlp.state[SLOTS:].any().item()
     np.testing.assert_array_equal(host_u16(mlp.c), mlp.oracle()[2])
+
+
+def test_one_state_block_serves_launches_of_different_shapes_and_inputs(ctx):
+    """One state block handed from launch to launch: a larger grid then a smaller one, larger magnitudes then
+    smaller ones (the maxima slots of workgroups the second launch does not have keep the first launch's
+    values and must not reach its scales), then back; every launch against the oracle."""
+    say("mlp chain: one state block, different shapes and inputs")
+    state = torch.zeros(iu8.MLP_CHAIN_STATE_BYTES // 4, dtype=torch.int32, device="cuda")
+    big, small = Mlp(1, 5120, 17408, seed=21), Mlp(2, 1024, 2048, seed=22)
+    big.X = synth.f32_to_bf16_bits(synth.bf16_bits_to_f32(big.X) * np.float32(64.0))     # large rows first
+    big.x = dev_bf16_bits(big.X)
+    assert iu8.resolve_mlp_chain(1, 5120, 17408).grid[0] > iu8.resolve_mlp_chain(2, 1024, 2048).grid[0]
+    want = {id(m): m.oracle() for m in (big, small)}
+    for mlp in (big, small, big, small, small):
+        mlp.state = state
+        mlp.c.fill_(0x7FC0)
+        mlp.chain(ctx)
+        assert not state[SLOTS:].any().item()
+        np.testing.assert_array_equal(host_u16(mlp.p), want[id(mlp)][1])
+        np.testing.assert_array_equal(host_u16(mlp.c), want[id(mlp)][2])
 
 
 def test_chain_refuses_what_the_form_does_not_hold(ctx):

@@ -218,6 +218,37 @@ def test_one_row_form_on_ties_nan_and_infinity(ctx):
             np.testing.assert_array_equal(host_u16(c), r["C"], err_msg=f"row {i}")
 
 
+@pytest.mark.parametrize("w8", [False, True])
+@pytest.mark.parametrize("M,N,K", [(12, 256, 1024),     # the streaming body (decode band)
+                                   (200, 320, 1024)])    # the tile body (MFMA cells)
+def test_rows_with_nan_and_infinity_through_the_gemm_epilogue(ctx, M, N, K, w8):
+    """Activation rows with NaNs and infinities through producer + GEMM on both body families. A row with a
+    NaN among finite values has a finite scale (the maximum passes the NaN over) and a finite output: bit-exact.
+    A row with an infinity has an infinite scale: its outputs are infinities where the accumulator is not zero
+    (bit-exact) and NaNs where it is (0 * inf); of a NaN in c only its being one is pinned -- the sign and payload
+    come from the multiplier that made it (the card's on one side, the host's on the other), which no contract
+    of the reference fixes (crates/saber-kernels/hip/macaq_iu8.hip:20-24)."""
+    say(f"nan/inf rows through the epilogue M={M} N={N} K={K} w8={w8}")
+    case = synth.dense_case(M, N, K, w8=w8, seed=M + K)
+    X = case["X"]
+    X[1, 17] = 0x7FC0                         # a lone NaN
+    X[2, K - 1] = 0x7F80                      # +inf
+    X[3, 5], X[3, 6] = 0xFF80, 0x7FC0         # -inf beside a NaN
+    X[4, :] = 0x7FC0                          # nothing but NaNs
+    X[5, 0], X[5, 1] = 0x7F80, 0xFF80         # both infinities: codes -127 and -127, the rest 0
+    r = ref.linear(X, case["W"], case["ws"], w8, threads=8)
+    run = DenseRun(ctx, case, want_acc=True)
+    np.testing.assert_array_equal(run.q, r["q"])
+    np.testing.assert_array_equal(run.a_scale.view(np.uint32), r["a_scale"].view(np.uint32))
+    np.testing.assert_array_equal(run.acc, r["S"] if w8 else r["S"] * 16)
+    want, got = r["C"], run.C
+    nan_w, nan_g = (want & 0x7FFF) > 0x7F80, (got & 0x7FFF) > 0x7F80
+    np.testing.assert_array_equal(nan_g, nan_w)                       # NaN exactly where the law makes one
+    np.testing.assert_array_equal(got[~nan_w], want[~nan_w])          # everything else bit for bit, infinities included
+    assert nan_w[[2, 3, 5]].any() or (r["S"][[2, 3, 5]] != 0).all()   # the infinite rows were exercised either way
+    assert not nan_w[[0, 1, 4] + list(range(6, M))].any()             # rows with a finite scale never give a NaN
+
+
 def test_fused_form_refuses_what_it_does_not_hold(ctx):
     assert not iu8.fused_holds(5, 1024) and not iu8.fused_holds(4, 20608) and not iu8.fused_holds(2, 41088)
     assert iu8.fused_holds(1, 17408) and iu8.fused_holds(4, 5120) and iu8.fused_holds(2, 10240)
