@@ -494,8 +494,45 @@ def main():
                 per[name] = dict(kernel=gd.kernel.decode(), gemv_us=round(g_us, 2), gemv_gbps=round(gb / g_us / 1e3, 1),
                                  producer=qd.kernel.decode(), producer_us=round(q_us, 2))
         del g
-        return dict(us_per_step=round(us, 2), gbps=round(nbytes / us / 1e3, 1), hbm_frac=round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4),
-                    launches_per_step=nlaunch, per_linear=per)
+        res = dict(us_per_step=round(us, 2), gbps=round(nbytes / us / 1e3, 1), hbm_frac=round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4),
+                   launches_per_step=nlaunch, per_linear=per)
+        # the step's MLP as one persistent launch beside its three launches, where the rows fit the chain's forms
+        if iu8.mlp_chain_holds(DM, hid, inter):
+            p_rows = torch.zeros((DM, inter), dtype=torch.int16, device=dev)
+            state = torch.zeros(iu8.MLP_CHAIN_STATE_BYTES // 4, dtype=torch.int32, device=dev)
+            q_dn = torch.zeros(iu8.a_bytes(DM, inter), dtype=torch.uint8, device=dev)
+            s_dn = torch.zeros(DM, dtype=torch.float32, device=dev)
+            d_gu, d_silu, d_dn = iu8.resolve_fused(iu8.W4, DM, n_gu, hid), iu8.resolve_silu_mul_quant(DM, inter), iu8.resolve(iu8.W4, DM, hid, inter)
+            for j in range(d_gu.n_args):
+                if d_gu.args[j].name in (b"q", b"scale"):
+                    d_gu.args[j].kind = iu8.ARG_NULL_BUFFER
+
+            def chain(i):
+                ctx.mlp_chain(xs["gate_up"].data_ptr(), dev_w["gate_up"][i % LAYERS].data_ptr(), dev_ws["gate_up"].data_ptr(),
+                              dev_w["down"][i % LAYERS].data_ptr(), dev_ws["down"].data_ptr(), None, p_rows.data_ptr(), state.data_ptr(),
+                              cs["down"].data_ptr(), DM, hid, inter, stream=sh)
+
+            def three(i):
+                ctx.launch(d_gu, dict(x=xs["gate_up"].data_ptr(), w=dev_w["gate_up"][i % LAYERS].data_ptr(), ws=dev_ws["gate_up"].data_ptr(),
+                                      c=cs["gate_up"].data_ptr()), sh)
+                ctx.launch(d_silu, dict(gu=cs["gate_up"].data_ptr(), q=q_dn.data_ptr(), scale=s_dn.data_ptr()), sh)
+                b = dict(a=q_dn.data_ptr(), w=dev_w["down"][i % LAYERS].data_ptr(), ws=dev_ws["down"].data_ptr(), c=cs["down"].data_ptr())
+                b["as"] = s_dn.data_ptr()
+                ctx.launch(d_dn, b, sh)
+
+            with torch.cuda.stream(stream):
+                three(0)
+            stream.synchronize()
+            want = cs["down"].clone()
+            t3 = graph_us(three)
+            with torch.cuda.stream(stream):
+                chain(0)
+            stream.synchronize()
+            same = bool(torch.equal(want, cs["down"]))
+            tc = graph_us(chain)
+            res["mlp_chain"] = dict(kernel=iu8.resolve_mlp_chain(DM, hid, inter).kernel.decode(), us_chain=round(tc, 2), us_three_launches=round(t3, 2),
+                                    same_bytes=same, state_status=int(state[iu8.MLP_CHAIN_STATUS_OFFSET // 4].item()))
+        return res
 
     if M == 1 and not args.no_other_m:
         out["decode_other_m"] = {"m%d" % DM: decode_at(DM) for DM in (4, 8, 16)}

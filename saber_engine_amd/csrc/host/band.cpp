@@ -151,7 +151,8 @@ std::string band_toml() {
   }
   o += "\n[mlp_chain]\n";
   o += "# macaq_iu8f_mlp_w4_tm1: gate+up -> SiLU * up + requantisation -> down in one persistent launch while\n";
-  o += "# the rows fit the fused form at both widths; every workgroup resident (one a CU)\n";
+  o += "# the rows fit the fused form at both widths; every workgroup resident (one a CU).\n";
+  o += "# macaq_iu8f_mlp_w4_tm1_a80: the same with the second linear's rows in 80 KiB of staged codes (up to 4 rows)\n";
   put(o, "threads", 1024);
   put(o, "state_bytes", MLP_CHAIN_STATE_BYTES);
   put(o, "spin_default", MLP_CHAIN_SPIN);
@@ -160,6 +161,7 @@ std::string band_toml() {
     saber_iu8_desc d;
     if (!resolve_mlp_chain(1, 5120, 17408, 0, &d)) o += fmt("grid.hidden5120_inter17408 = %u\n", d.grid[0]);
     if (!resolve_mlp_chain(4, 5120, 5120, 0, &d)) o += fmt("grid.hidden5120_inter5120 = %u\n", d.grid[0]);
+    if (!resolve_mlp_chain(4, 5120, 17408, 0, &d)) o += fmt("a80.grid.hidden5120_inter17408_rows4 = %u\n", d.grid[0]);
   }
   o += "\n[pair]\n# block order by tm: true = the second problem's workgroups first (macaq_iu8f_pairb_*)\n";
   {

@@ -420,6 +420,11 @@ bool fused_small_holds(uint32_t m, uint32_t k) { return m >= 1 && m <= 4 && stag
 bool fused_form_holds(bool a80, uint32_t m, uint32_t k) {
   return a80 ? m >= 1 && m <= 16 && staged_bytes(m, k) <= 80 * 1024 : fused_small_holds(m, k);
 }
+// the MLP chain: the first linear's rows (hidden wide) in the 20 KiB form, the second's (intermediate wide) in
+// the 20 KiB form or, for up to 4 rows, the 80 KiB one
+bool mlp_chain_form_holds(uint32_t m, uint32_t hidden, uint32_t inter) {
+  return fused_small_holds(m, hidden) && (fused_small_holds(m, inter) || (m <= 4 && fused_form_holds(true, m, inter)));
+}
 bool fused_holds(uint32_t m, uint32_t k) { return fused_small_holds(m, k) || (m <= 4 && fused_form_holds(true, m, k)); }
 
 uint32_t fused_grid(uint32_t nblk) {
@@ -468,15 +473,16 @@ int resolve_mlp_chain(uint32_t m, uint32_t hidden, uint32_t inter, uint32_t spin
   if (inter > 0x3FFFFFFFu) return fail(SABER_IU8_E_RULE, fmt("%s: intermediate width %u", op, inter));
   if (int rc = check_shape(op, m, 2 * inter, hidden)) return rc;
   if (int rc = check_shape(op, m, hidden, inter)) return rc;
-  if (!fused_small_holds(m, hidden) || !fused_small_holds(m, inter))
-    return fail(SABER_IU8_E_RULE, fmt("%s: %u rows of %u / %u do not fit the fused form (at most 4 rows, 20 KiB of codes)", op, m,
-                                      hidden, inter));
+  if (!mlp_chain_form_holds(m, hidden, inter))
+    return fail(SABER_IU8_E_RULE, fmt("%s: %u rows of %u / %u do not fit the fused form (at most 4 rows, 20 KiB of codes at the hidden "
+                                      "width, 80 KiB at the intermediate)", op, m, hidden, inter));
   // the first linear walks inter / 16 paired tiles, the second hidden / 32 column blocks; one workgroup a CU
   const uint32_t nblk = std::max(inter / 16, (hidden + 31) / 32);
   if (nblk > 8 * CU_COUNT)
     return fail(SABER_IU8_E_RULE, fmt("%s: %u column blocks are more than the %u resident workgroups walk (8 each)", op, nblk, CU_COUNT));
   const uint32_t grid = std::max(fused_grid(inter / 16), fused_grid((hidden + 31) / 32));
-  const char *name = "macaq_iu8f_mlp_w4_tm1";
+  // the second linear's rows in 20 KiB of staged codes, else in 80 KiB (`_a80`: 2 to 4 rows of the 27B layer's 17,408)
+  const char *name = fused_small_holds(m, inter) ? "macaq_iu8f_mlp_w4_tm1" : "macaq_iu8f_mlp_w4_tm1_a80";
   memset(d, 0, sizeof *d);
   copy_name(d->op, sizeof d->op, op);
   copy_name(d->plugin, sizeof d->plugin, "macaq_iu8f");

@@ -47,7 +47,8 @@ int resolve_quant(uint32_t m, uint32_t k, saber_iu8_desc *out);
 // The fused quant + GEMV of a decode linear; refuses (by name) shapes it does not hold.
 bool fused_holds(uint32_t m, uint32_t k);        // the law: a fused launch is what runs (up to 4 rows: the 20 KiB form, else the 80 KiB form)
 bool fused_form_holds(bool a80, uint32_t m, uint32_t k);  // what the kernel itself holds: `_tm1` 4 rows / 20 KiB, `_tm1_a80` 16 rows / 80 KiB
-bool fused_small_holds(uint32_t m, uint32_t k);  // the 20 KiB form: up to 4 rows (`_tm1`, and both linears of the MLP chain)
+bool fused_small_holds(uint32_t m, uint32_t k);  // the 20 KiB form: up to 4 rows (`_tm1`, and the MLP chain's first linear)
+bool mlp_chain_form_holds(uint32_t m, uint32_t hidden, uint32_t inter);  // the chain: 20 KiB at the hidden width, 20 or 80 KiB at the intermediate
 uint32_t fused_grid(uint32_t nblk);  // workgroups for nblk column blocks: one a CU, then equal shares of at most 8
 int resolve_fused(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *out);
 // The decode MLP (gate+up -> SiLU * up + requant -> down) as one persistent launch; spin 0 = the default.

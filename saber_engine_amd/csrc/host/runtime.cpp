@@ -140,7 +140,7 @@ int saber_iu8_pair_ordered(const saber_iu8_desc *first, const saber_iu8_desc *se
 }
 int saber_iu8_fused_holds(uint32_t m, uint32_t k) { return fused_holds(m, k) ? 1 : 0; }
 int saber_iu8_mlp_chain_holds(uint32_t m, uint32_t hidden, uint32_t inter) {
-  return fused_small_holds(m, hidden) && fused_small_holds(m, inter) ? 1 : 0;
+  return mlp_chain_form_holds(m, hidden, inter) ? 1 : 0;
 }
 int saber_iu8_resolve_fused(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *out) {
   if (!out) return fail(SABER_IU8_E_ARG, "resolve_fused: null descriptor");
@@ -359,8 +359,9 @@ static int i32_arg(const saber_iu8_desc *d, const char *name) {
 // refused here from what the loaded kernel's registers and LDS let reside.
 static int chain_guard(const LoadedKernel &lk, const saber_iu8_desc *d) {
   const int64_t m = i32_arg(d, "m"), h = i32_arg(d, "k"), i = i32_arg(d, "n");
-  if (m <= 0 || h <= 0 || i <= 0 || !fused_small_holds((uint32_t)m, (uint32_t)h) || !fused_small_holds((uint32_t)m, (uint32_t)i) ||
-      h % 128 || i % 128)
+  const bool a80 = strstr(d->kernel, "_a80") != nullptr;
+  if (m <= 0 || h <= 0 || i <= 0 || !fused_small_holds((uint32_t)m, (uint32_t)h) ||
+      !(a80 ? m <= 4 && fused_form_holds(true, (uint32_t)m, (uint32_t)i) : fused_small_holds((uint32_t)m, (uint32_t)i)) || h % 128 || i % 128)
     return fail(SABER_IU8_E_RULE, fmt("%s: %lld rows of %lld / %lld do not fit the fused form", d->kernel, (long long)m, (long long)h,
                                       (long long)i));
   const int64_t nblk = std::max(i / 16, (h + 31) / 32);

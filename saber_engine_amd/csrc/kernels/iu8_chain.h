@@ -166,7 +166,10 @@ struct iu8_chain_hook {
   }
 };
 
-template <int NT, int KW, int WPB, int D>
+// AKB2: KiB of staged codes of the second linear -- 20 (pow2(M) * I <= 20 KiB) or 80 (up to 4 rows of an
+// intermediate width whose codes fit 80 KiB: the benchmark layer's 17,408 at 2 to 4 rows). The two linears
+// run one after the other, so their LDS objects lie over one block.
+template <int NT, int KW, int WPB, int D, int AKB2 = 20>
 __device__ __forceinline__ void iu8_chain_mlp(const unsigned short *__restrict__ x, const iu8_u8 *__restrict__ w_gu,
                                               const float *__restrict__ ws_gu, const iu8_u8 *__restrict__ w_dn,
                                               const float *__restrict__ ws_dn, unsigned short *__restrict__ gu,
@@ -181,7 +184,11 @@ __device__ __forceinline__ void iu8_chain_mlp(const unsigned short *__restrict__
   const bool collector = (int)blockIdx.x == G - 1;
   // phase 1: [gate | up] = x . Wgu^T (quantisation of x fused), p and this workgroup's maxima from its
   // epilogue, stored through; gu (may be null) is a tap
-  iu8_decq_body<false, NT, KW, WPB, D, 1>(x, w_gu, ws_gu, nullptr, nullptr, gu, M, I, H,
+  __shared__ union Lds {
+    iu8_decq_lds<NT, KW, WPB, 1, 20> first;
+    iu8_decq_lds<NT, KW, WPB, 2, AKB2> second;
+  } lds;
+  iu8_decq_body<false, NT, KW, WPB, D, 1>(lds.first, x, w_gu, ws_gu, nullptr, nullptr, gu, M, I, H,
                                           iu8_decq_pairhook{p, slots + blockIdx.x * 4});
   iu8_chain_arrive(S);
   if ((int)blockIdx.x >= S.nwait) {
@@ -190,7 +197,9 @@ __device__ __forceinline__ void iu8_chain_mlp(const unsigned short *__restrict__
     return;
   }
   // phase 2: c = p . Wdn^T; the hook waits for the meeting behind the first weight loads
-  iu8_decq_body<false, NT, KW, WPB, D, 2>(p, w_dn, ws_dn, nullptr, nullptr, c, M, H, I, iu8_chain_hook{S, slots});
+  // (the first linear's LDS is dead: every wave of this workgroup is past iu8_chain_arrive's barrier)
+  iu8_decq_body<false, NT, KW, WPB, D, 2, iu8_chain_hook, AKB2>(lds.second, p, w_dn, ws_dn, nullptr, nullptr, c, M, H, I,
+                                                                iu8_chain_hook{S, slots});
   // (one answer for the whole workgroup: the clear holds barriers)
   if (collector && __syncthreads_or(iu8_chain_ld((const unsigned *)S.status) != 0u) == 0) iu8_chain_clear(S);
 }

@@ -44,11 +44,27 @@ static __device__ __forceinline__ iu8_v4u iu8_decq_ld_coherent(const iu8_v4u *p)
   const unsigned long long hi = __hip_atomic_load((const unsigned long long *)p + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
   return iu8_v4u{(unsigned)lo, (unsigned)(lo >> 32), (unsigned)hi, (unsigned)(hi >> 32)};
 }
+// The body's LDS, as one object: a kernel that runs two bodies one after the other (the MLP chain) lays both
+// objects over one block of LDS; a kernel with one body declares one.
+template <int NT, int KW, int WPB, int CH, int AKB>
+struct iu8_decq_lds {
+  static constexpr int WN = WPB / KW, RED = (KW - 1) * WN * NT * 256;
+  static constexpr bool BIG = AKB > 20, PAIRED = CH == 1;
+  __attribute__((aligned(16))) iu8_u8 s_a[AKB * 1024];  // staged codes: pow2(M) * K bytes
+  __attribute__((aligned(16))) int s_red[2][RED];       // the k-waves' partials, two alternating areas
+  float s_amax[WPB][4];
+  float s_sq[2][4];  // scale and reciprocal a row, made once a workgroup
+  unsigned s_rowmax[BIG ? 16 : 1];
+  float s_rsc[BIG ? 16 : 1], s_rrcp[BIG ? 16 : 1];
+  float s_ws[IU8_DECQ_MAXB][WN * NT * 16];  // the epilogue's weight scales (W4: already / 16)
+  __attribute__((aligned(8))) unsigned s_up[PAIRED ? 2 : 1][PAIRED ? 128 : 2];  // the up wave's bf16 values, two blocks
+};
 template <bool W8, int NT, int KW, int WPB, int D, int CH = 0, class Hook = iu8_decq_nohook, int AKB = 20>
-__device__ __forceinline__ void iu8_decq_body(const unsigned short *__restrict__ X, const iu8_u8 *__restrict__ W,
-                                              const float *__restrict__ ws, iu8_u8 *__restrict__ qout,
-                                              float *__restrict__ sout, unsigned short *__restrict__ C, int M, int N,
-                                              int K, const Hook hook = Hook{}) {
+__device__ __forceinline__ void iu8_decq_body(iu8_decq_lds<NT, KW, WPB, CH, AKB> &S, const unsigned short *__restrict__ X,
+                                              const iu8_u8 *__restrict__ W, const float *__restrict__ ws,
+                                              iu8_u8 *__restrict__ qout, float *__restrict__ sout,
+                                              unsigned short *__restrict__ C, int M, int N, int K,
+                                              const Hook hook = Hook{}) {
   static_assert(KW > 1 && WPB % KW == 0, "k-waves divide the workgroup");
   constexpr int WN = WPB / KW;
   constexpr bool PAIRED = CH == 1;
@@ -62,16 +78,16 @@ __device__ __forceinline__ void iu8_decq_body(const unsigned short *__restrict__
   // pieces of one load lie in one row when K is a multiple of 512: then one lane a wave), scales and
   // reciprocals are made once a row by 16 lanes, and a lane reads its row's scale for the epilogue.
   constexpr bool BIG = AKB > 20;
-  static_assert(!BIG || CH == 0, "the chain's forms stage at most 20 KiB");
-  constexpr int RED = (KW - 1) * WN * NT * 256;  // ints of one partial area
-  __shared__ __attribute__((aligned(16))) iu8_u8 s_a[ABYTES];
-  __shared__ __attribute__((aligned(16))) int s_red[2][RED];
-  __shared__ float s_amax[WPB][4];
-  __shared__ float s_sq[2][4];  // scale and reciprocal a row, made once a workgroup
-  __shared__ unsigned s_rowmax[BIG ? 16 : 1];
-  __shared__ float s_rsc[BIG ? 16 : 1], s_rrcp[BIG ? 16 : 1];
-  __shared__ float s_ws[IU8_DECQ_MAXB][WN * NT * 16];  // the epilogue's weight scales (W4: already / 16)
-  __shared__ __attribute__((aligned(8))) unsigned s_up[PAIRED ? 2 : 1][PAIRED ? 128 : 2];  // the up wave's bf16 values, two blocks
+  static_assert(!BIG || CH != 1, "the chain's first linear stages at most 20 KiB");
+  auto &s_a = S.s_a;
+  auto &s_red = S.s_red;
+  auto &s_amax = S.s_amax;
+  auto &s_sq = S.s_sq;
+  auto &s_rowmax = S.s_rowmax;
+  auto &s_rsc = S.s_rsc;
+  auto &s_rrcp = S.s_rrcp;
+  auto &s_ws = S.s_ws;
+  auto &s_up = S.s_up;
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -142,14 +158,24 @@ __device__ __forceinline__ void iu8_decq_body(const unsigned short *__restrict__
     }
   };
 
+  // A launch of the chain that cannot complete (a producer never arrived, or the state block still carries an
+  // earlier launch's raised status) gives up as a whole and says so where the caller looks: every output this
+  // workgroup owns becomes a bf16 NaN (0x7FC0), so a replayed graph that can no longer complete does not hand
+  // back stale or half-written rows as if they were results. (The status word says the same to a host that
+  // reads the state block.)
+  auto give_up = [&]() {
+    constexpr int BC = WNB * NT * 16;
+    for (int i = tid; i < nb * BC * M; i += NTHR) {
+      const int b = i / (BC * M), r = (i / BC) % M, cc = i % BC;
+      const int n = ((int)blockIdx.x + b * G) * BC + cc;
+      if (n < N) C[(size_t)r * N + n] = 0x7FC0;
+    }
+  };
   // ---- quantise the rows: amax lane -> wave (butterfly) -> workgroup (LDS),
   // all order-free maxima; sc = max(amax / 127, 1e-30); codes by the exact reciprocal path
   float qsc[4] = {1.f, 1.f, 1.f, 1.f};
   float my_sc = 1.f;  // BIG: the scale of this lane's row (ml)
   if constexpr (BIG) {
-    if (tid < 16) s_rowmax[tid] = 0u;
-    __syncthreads();
-    const bool wave_rows = (k8 & 63) == 0;  // a wave's 64 pieces of one load lie in one row
     // piece p * NTHR + tid = (row, col) in pieces of 8: two divides here, then steps of NTHR pieces
     const int row_step = NTHR / k8, col_step = NTHR - row_step * k8;
     int row = tid / k8, col = tid - row * k8;
@@ -157,6 +183,30 @@ __device__ __forceinline__ void iu8_decq_body(const unsigned short *__restrict__
       row += row_step, col += col_step;
       if (col >= k8) col -= k8, ++row;
     };
+    if constexpr (CH == 2) {
+      // the chain's second linear on the 80 KiB form (up to 4 rows): weights first (they do not depend on the
+      // first linear), then the rows once every producer's share is in memory; the rows' maxima are the
+      // producers' (hook.amax), no pass over the rows
+#pragma unroll
+      for (int i = 0; i < D; ++i)
+        if (i < TT) issue(i);
+      if (!hook.wait()) {
+        give_up();
+        return;
+      }
+#pragma unroll
+      for (int p = 0; p < X_PER; ++p)
+        if (p * NTHR + tid < x_pieces) xreg[p] = iu8_decq_ld_coherent((const iu8_v4u *)X + p * NTHR + tid);
+#pragma unroll
+      for (int p = 0; p < WS_PER; ++p)
+        if (p * NTHR + tid < WS_ALL) (&s_ws[0][0])[p * NTHR + tid] = wsreg[p];
+      float a4[4];
+      hook.amax(a4);  // the whole workgroup: the maxima over the producers' shares
+      if (tid < 16) s_rowmax[tid] = tid < 4 ? __float_as_uint(tid == 0 ? a4[0] : tid == 1 ? a4[1] : tid == 2 ? a4[2] : a4[3]) : 0u;
+    } else {
+    if (tid < 16) s_rowmax[tid] = 0u;
+    __syncthreads();
+    const bool wave_rows = (k8 & 63) == 0;  // a wave's 64 pieces of one load lie in one row
 #pragma unroll
     for (int p = 0; p < X_PER; ++p, next_piece()) {
       const int piece = p * NTHR + tid;
@@ -184,6 +234,7 @@ __device__ __forceinline__ void iu8_decq_body(const unsigned short *__restrict__
 #pragma unroll
     for (int p = 0; p < WS_PER; ++p)
       if (p * NTHR + tid < WS_ALL) (&s_ws[0][0])[p * NTHR + tid] = wsreg[p];
+    }
     __syncthreads();
     if (tid < 16) {
       const float sc = fmaxf(__fdiv_rn(__uint_as_float(s_rowmax[tid]), 127.f), 1e-30f);
@@ -222,17 +273,7 @@ __device__ __forceinline__ void iu8_decq_body(const unsigned short *__restrict__
       for (int i = 0; i < D; ++i)
         if (i < TT) issue(i);
       if (!hook.wait()) {
-        // A producer never arrived, or the state block still carries an earlier launch's raised status: the
-        // launch gives up as a whole and says so where the caller looks -- every output this workgroup owns
-        // becomes a bf16 NaN (0x7FC0), so a replayed graph that can no longer complete does not hand back
-        // stale or half-written rows as if they were results. (The status word says the same to a host that
-        // reads the state block.)
-        constexpr int BC = WNB * NT * 16;
-        for (int i = tid; i < nb * BC * M; i += NTHR) {
-          const int b = i / (BC * M), r = (i / BC) % M, cc = i % BC;
-          const int n = ((int)blockIdx.x + b * G) * BC + cc;
-          if (n < N) C[(size_t)r * N + n] = 0x7FC0;
-        }
+        give_up();
         return;
       }
 #pragma unroll

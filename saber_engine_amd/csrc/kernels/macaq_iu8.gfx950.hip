@@ -53,7 +53,8 @@
       const unsigned short *__restrict__ x, const unsigned char *__restrict__ w, const float *__restrict__ ws,     \
       unsigned char *__restrict__ q, float *__restrict__ scale, unsigned short *__restrict__ c, int m, int n,      \
       int k) {                                                                                                     \
-    iu8_decq_body<W8, NT, KW, WPB, D, 0, iu8_decq_nohook, AKB>(x, w, ws, q, scale, c, m, n, k);                    \
+    __shared__ iu8_decq_lds<NT, KW, WPB, 0, AKB> lds;                                                              \
+    iu8_decq_body<W8, NT, KW, WPB, D, 0, iu8_decq_nohook, AKB>(lds, x, w, ws, q, scale, c, m, n, k);               \
   }
 IU8_DECQX(macaq_iu8_decq_w4_tm1, false, 1, 8, 16, 4)
 IU8_DECQX(macaq_iu8_decq_w8_tm1, true, 1, 8, 16, 2)

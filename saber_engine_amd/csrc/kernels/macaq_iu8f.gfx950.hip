@@ -48,3 +48,12 @@ extern "C" __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu
     int spin) {
   iu8_chain_mlp<1, 8, 16, 4>(x, w, ws, w_b, ws_b, gu, p, state, c, m, k, n, spin);
 }
+// `_a80`: the same launch with the second linear on the 80 KiB form -- up to 4 rows whose intermediate codes
+// (rows rounded up to a power of two) fit 80 KiB: 2 to 4 rows of the benchmark layer's 17,408.
+extern "C" __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4))) void macaq_iu8f_mlp_w4_tm1_a80(
+    const unsigned short *__restrict__ x, const unsigned char *__restrict__ w, const float *__restrict__ ws,
+    const unsigned char *__restrict__ w_b, const float *__restrict__ ws_b, unsigned short *__restrict__ gu,
+    unsigned short *__restrict__ p, unsigned char *__restrict__ state, unsigned short *__restrict__ c, int m, int k, int n,
+    int spin) {
+  iu8_chain_mlp<1, 8, 16, 4, 80>(x, w, ws, w_b, ws_b, gu, p, state, c, m, k, n, spin);
+}

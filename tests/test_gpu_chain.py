@@ -59,14 +59,16 @@ class Mlp:
 # rows, hidden, intermediate: the benchmark layer at one row (5120 / 17408); the most rows the form
 # holds at a narrower layer; two rows at the widest they fit; three rows (staged as four) with K
 # steps that do not divide among the k-waves (11 and 23); fewer column blocks than workgroups
-SHAPES = [(1, 5120, 17408), (4, 5120, 5120), (2, 2048, 10240), (3, 1408, 2944), (1, 384, 384)]
+# ... and the 80 KiB form of the second linear: 2 and 4 rows of the benchmark layer, 3 rows of a ragged width
+SHAPES = [(1, 5120, 17408), (4, 5120, 5120), (2, 2048, 10240), (3, 1408, 2944), (1, 384, 384),
+          (2, 5120, 17408), (4, 5120, 17408), (3, 640, 12672)]
 
 
 @pytest.mark.parametrize("M,H,I", SHAPES)
 def test_chain_matches_the_oracle_and_the_three_launches(ctx, M, H, I):
     say(f"mlp chain M={M} H={H} I={I}")
     d = iu8.resolve_mlp_chain(M, H, I)
-    assert d.kernel == b"macaq_iu8f_mlp_w4_tm1" and d.block[0] == 1024
+    assert d.kernel == (b"macaq_iu8f_mlp_w4_tm1" if iu8.fused_small_holds(M, I) else b"macaq_iu8f_mlp_w4_tm1_a80") and d.block[0] == 1024
     assert d.grid[0] <= 256 and d.grid[0] * 8 >= max(I // 16, H // 32)      # one workgroup a CU, at most 8 blocks each
     assert {w.name: w.bytes for w in d.workspaces[:d.n_workspaces]} == {b"p": M * I * 2, b"state": iu8.MLP_CHAIN_STATE_BYTES}
     mlp = Mlp(M, H, I, seed=M + I)
@@ -130,7 +132,7 @@ def test_one_state_block_serves_launches_of_different_shapes_and_inputs(ctx):
 
 
 def test_chain_refuses_what_the_form_does_not_hold(ctx):
-    for m, h, i, word in ((5, 1024, 2048, "fused form"), (4, 5120, 17408, "fused form"), (1, 5120, 17400, "multiple"),
+    for m, h, i, word in ((5, 1024, 2048, "fused form"), (4, 5120, 20608, "fused form"), (4, 5248, 5120, "fused form"), (1, 5120, 17400, "multiple"),
                           (0, 1024, 2048, "nothing")):
         with pytest.raises(iu8.IU8Error) as e:
             iu8.resolve_mlp_chain(m, h, i)
