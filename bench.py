@@ -32,8 +32,8 @@ LAYERS = 6                  # distinct weight copies walked by successive steps 
 # figure cannot be read inside this process: it comes from two rocprofv3 --pmc runs of this very
 # command (FETCH_SIZE, then WRITE_SIZE), each counter scaled by what it reads for the 256 MiB copy
 # probe, and is kept in the profile summary named below. Keyed by (kernel, M); None = not measured.
-TRAFFIC_SOURCE = "profiles/macaq_iu8_decq_w4_tm1__layer_set_m1.txt"
-TRAFFIC = {("macaq_iu8_decq_w4_tm1", 1): 41737825.0, ("macaq_iu8_dec_w4_tm1", 1): 41995646.0}
+TRAFFIC_SOURCE = "profiles/macaq_iu8_decq_w4__layer_set_m1.txt"
+TRAFFIC = {("macaq_iu8_decq_w4_r1 + macaq_iu8_decq_w4_tm1", 1): 41749312.0, ("macaq_iu8_dec_w4_tm1", 1): 41995646.0}
 
 
 def alg_bytes(m, n, k, w8=False):
@@ -231,10 +231,10 @@ def main():
     gemm_us = ev0.elapsed_time(ev1) * 1e3 / (K_steps * len(linears))
     if fused:   # reads the bf16 rows itself
         gemm_bytes = sum(alg_bytes(M, n, k) for _, n, k in linears) / len(linears)
-        kname = fdescs["down"].kernel.decode()
+        kname = " + ".join(sorted({d.kernel.decode() for d in fdescs.values()}))   # the step's launches: one symbol or two
     else:       # reads the int8 codes and the row scales
         gemm_bytes = sum(alg_bytes(M, n, k) - 2 * M * k + M * k + 4 * M for _, n, k in linears) / len(linears)
-        kname = descs["down"].kernel.decode()
+        kname = " + ".join(sorted({d.kernel.decode() for d in descs.values()}))
     achieved = gemm_bytes / (gemm_us * 1e-6) / 1e9
     roofline = dict(bound="hbm", kernel=kname, achieved=round(achieved, 1), peak=HBM_PEAK_GBPS,
                     unit="GB/s", frac=round(achieved / HBM_PEAK_GBPS, 4), traffic=TRAFFIC.get((kname, M)),
