@@ -144,13 +144,15 @@ __device__ __forceinline__ void iu8_dec_body(const iu8_u8 *__restrict__ A, const
   // ---- the weight ring
   iu8_v4u ring[D][NT][WV];
   iu8_v4i ringa[ALDS ? 1 : D][TM][2];  // direct-from-L2 activation operands when not staged
-  bool live[TM];
-#pragma unroll
-  for (int i = 0; i < TM; ++i) live[i] = i * 16 + ml < M;
-  const iu8_u8 *ap[TM];  // this lane's row of every activation tile, at the wave's first K step
+  // this lane's row of every activation tile, at the wave's first K step. A lane past the live rows reads the
+  // last live row again (the piece a live lane of the same load already touches: no line more from L2), and
+  // what it multiplies lands in output rows that are never stored. The loads are unconditional on purpose:
+  // under a per-lane test the compiler cannot count them and waits for every load in flight (`vmcnt(0)`) at
+  // each consume, which makes a ring of any depth a ring of one.
+  const iu8_u8 *ap[TM];
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
-    const int ar = iu8_arow(R, i * 16 + ml);
+    const int ar = iu8_arow(R, min(i * 16 + ml, M - 1));
     ap[i] = A + ((size_t)(ar >> 4) * ktiles + (size_t)(s_lo + wk) * 2) * 1024 + ((ar & 15) + 16 * lg) * 16;
   }
   auto issue = [&](int slot, int t) {
@@ -162,12 +164,8 @@ __device__ __forceinline__ void iu8_dec_body(const iu8_u8 *__restrict__ A, const
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-          ringa[ALDS ? 0 : slot][i][h] = iu8_v4i{0, 0, 0, 0};
-          if (live[i])
-            ringa[ALDS ? 0 : slot][i][h] =
-                *(const iu8_v4i *)(ap[i] + ((size_t)t * (2 * KW) + h) * 1024);
-        }
+        for (int h = 0; h < 2; ++h)
+          ringa[ALDS ? 0 : slot][i][h] = *(const iu8_v4i *)(ap[i] + ((size_t)t * (2 * KW) + h) * 1024);
     }
   };
   const int a_lane = (((lg << mr_shift) + min(ml, (1 << mr_shift) - 1)) << 4);
@@ -281,24 +279,46 @@ __device__ __forceinline__ void iu8_dec_body(const iu8_u8 *__restrict__ A, const
       __syncthreads();  // every wave is done with the staged rows before s_mem holds partials
     }
   } else {
+    // Every load of the ring is issued unconditionally and the tail is straight-line code a case, so that the
+    // compiler can count the loads in flight at each consume (`vmcnt(n)` for the slot's own loads, the rest stay
+    // in flight). Under a test -- a first ring of fewer than D steps, a drain loop that asks `is there a step D
+    // ahead` -- it cannot, and waits for every load in flight at each consume. The scheduling fences keep a
+    // slot's re-issue behind its own consume and in front of the next slot's: without them the compiler gathers
+    // the D consumes and then the D issues, i.e. waits for everything, multiplies, and only then asks for more.
+    // A wave with fewer than D steps loads its last step again into the spare slots and does not consume them.
+    if (T > 0) {
 #pragma unroll
-    for (int i = 0; i < D; ++i)
-      if (i < T) issue(i, i);
+      for (int i = 0; i < D; ++i) issue(i, min(i, T - 1));
+    }
     int t0 = 0;
-    for (; t0 + 2 * D <= T; t0 += D) {
+    auto round = [&](int t) {
+#pragma unroll
+      for (int i = 0; i < D; ++i) {
+        consume(i, t + i);
+        __builtin_amdgcn_sched_barrier(0);
+        issue(i, t + i + D);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+    for (; t0 + 2 * D <= T; t0 += D) round(t0);
+    const int rest = T - t0;  // up to 2D - 1 steps left, min(rest, D) of them in the ring
+#pragma unroll
+    for (int e = 0; e < D; ++e) {
+      if (rest - D != e) continue;  // rest = D + e: e more steps to issue
 #pragma unroll
       for (int i = 0; i < D; ++i) {
         consume(i, t0 + i);
-        issue(i, t0 + i + D);
+        __builtin_amdgcn_sched_barrier(0);
+        if (i < e) issue(i, t0 + i + D);
+        __builtin_amdgcn_sched_barrier(0);
       }
+#pragma unroll
+      for (int i = 0; i < e; ++i) consume(i, t0 + D + i);
     }
-    for (; t0 < T; t0 += D) {
+    if (rest < D) {
 #pragma unroll
       for (int i = 0; i < D; ++i)
-        if (t0 + i < T) {
-          consume(i, t0 + i);
-          if (t0 + i + D < T) issue(i, t0 + i + D);
-        }
+        if (i < rest) consume(i, i);
     }
   }
 
