@@ -94,6 +94,31 @@ def test_named_cells_random_shapes(ctx):
     assert ran >= 200
 
 
+def test_one_row_form_random_shapes(ctx):
+    """The one-row fused form by name on rows of any length it holds (128 to 20,480), ragged N, any grid the
+    host's rule lets through: c and the optional code output equal the oracle's."""
+    rng = np.random.default_rng(20248)
+    for n in range(60):
+        w8 = bool(rng.integers(0, 2))
+        tag = "w8" if w8 else "w4"
+        N, K = int(rng.integers(1, 200)) * 16, int(rng.integers(1, 161)) * 128
+        nblk = (N + 31) // 32
+        grid = int(rng.integers(max(1, (nblk + 7) // 8), min(nblk, 256) + 1))
+        say(f"sweep one-row {n}: {tag} N={N} K={K} grid={grid}")
+        case = synth.dense_case(1, N, K, w8=w8, seed=int(rng.integers(0, 1 << 30)))
+        r = ref.linear(case["X"], case["W"], case["ws"], w8, threads=8)
+        x, wf, ws = dev_bf16_bits(case["X"]), dev_u8(iu8.repack_weights(case["W"], w8)), dev_f32(case["ws"])
+        d = iu8.describe_raw(f"macaq_iu8_decq_{tag}_r1", (grid, 1, 1), 1024, m=1, n=N, k=K)
+        c = torch.full((1, N), 0x7FC0, dtype=torch.int16, device="cuda")
+        q = torch.full((iu8.a_bytes(1, K),), 0x55, dtype=torch.uint8, device="cuda")
+        s = torch.zeros(1, dtype=torch.float32, device="cuda")
+        ctx.launch(d, dict(x=x.data_ptr(), w=wf.data_ptr(), ws=ws.data_ptr(), c=c.data_ptr(), q=q.data_ptr(), scale=s.data_ptr()))
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(host_u16(c), r["C"])
+        np.testing.assert_array_equal(iu8.unpack_a(q.cpu().numpy(), 1, K), r["q"])
+        np.testing.assert_array_equal(s.cpu().numpy().view(np.uint32), r["a_scale"].view(np.uint32))
+
+
 def test_pair_chain_static_gemm_and_back_half_random_shapes(ctx):
     """The decode pair, the decode MLP chain (two launches in a row on one state block), the GEMM on the
     library's static workspace (twice in a row) and the routed layer's back half as two and as three launches."""
