@@ -324,8 +324,11 @@ def test_prefill_cells_of_the_benchmark_shapes():
         assert iu8.resolve(iu8.W4, m, n, k).kernel.decode() == "macaq_iu8_pf_w4_" + tile, (m, n, k)
     # int8 weights rank the cells differently (twice the bytes a tile, no unpack): the output-side projections
     # of the mixed sequence at 2,048 rows take 256 x 160 (O 51.6 us against 72.6 on 128 x 320, down 158.6 against 224.2)
-    want8 = {(2048, 5120, 5120): "t256x160", (2048, 5120, 17408): "t256x160", (8192, 5120, 17408): "tn4_lbk64",
-             (8192, 5120, 5120): "tn4_lbk64", (4096, 5120, 5120): "tn4_lbk64", (1024, 5120, 17408): "t128x256",
+    # from 4,096 rows the 256 x 320 cell (N = 5120: 16 column blocks, even rounds): O 91.2 us against 104.5 on 256 x 256 at
+    # 4,096 rows, down 278.5 against 313.0; at 8,192 rows 176.1 against 190.6 and 560.3 against 635.0; QKV stays (174.8 against 147.9)
+    want8 = {(2048, 5120, 5120): "t256x160", (2048, 5120, 17408): "t256x160", (8192, 5120, 17408): "t256x320",
+             (8192, 5120, 5120): "t256x320", (4096, 5120, 5120): "t256x320", (4096, 5120, 17408): "t256x320",
+             (4096, 7168, 5120): "tn4_lbk64", (8192, 7168, 5120): "tn4_lbk64", (1024, 5120, 17408): "t128x256",
              (512, 5120, 17408): "t128x128", (256, 5120, 5120): "t64x128_s", (128, 5120, 17408): "t64x64_s"}
     for (m, n, k), tile in want8.items():
         assert iu8.resolve(iu8.W8, m, n, k).kernel.decode() == "macaq_iu8_pf_w8_" + tile, (m, n, k)
@@ -415,8 +418,10 @@ def test_reference_symbols_and_lds_budget():
     for name in json.load(open(os.path.join(GOLD, "kernarg_gfx1201.json"))):
         assert f'name = "{name}"' in text and f'symbol = "{name}.kd"' in text
     assert max(int(v) for v in re.findall(r"group_segment_fixed_size = (\d+)", text)) <= 160 * 1024
-    # no kernel of the shipped objects spills to scratch
-    assert set(re.findall(r"private_segment_fixed_size = (\d+)", text)) == {"0"}
+    # no kernel of the shipped objects spills to scratch -- but for one dword that the int8-weight 256 x 320 cell
+    # parks across a tile's K loop (stored in front of the loop, read behind it)
+    spills = {n: int(b) for n, b in re.findall(r'name = "(\w+)"(?:(?!\[\[kernel\]\]).)*?private_segment_fixed_size = (\d+)', text, flags=re.S) if int(b)}
+    assert spills == {"macaq_iu8_pf_w8_t256x320": 8}, spills
 
 
 @pytest.mark.parametrize("edit,counter", [
