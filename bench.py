@@ -268,23 +268,27 @@ def main():
 
     # ---- every linear of the step by itself: the fused launch alone (graph of K launches walking the weight
     # copies), and the read probe on the same weight bytes, cold the same way. down = the 5120 x 17408 GEMV.
+    # (the side figures from here on do not depend on --steps: graphs of at least 120 launches, replayed a few
+    # times before the timed replay, so a short driver run reads the same per-linear numbers as a long one)
+    SIDE_STEPS = max(K_steps, 120)
     per_linear = {}
     for name, n, k in linears:
         gl = torch.cuda.CUDAGraph()
         with torch.cuda.graph(gl, stream=stream):
-            for i in range(K_steps):
+            for i in range(SIDE_STEPS):
                 if fused:
                     launch_fused(name, i % LAYERS)
                 else:
                     launch_gemm(name, i % LAYERS)
         with torch.cuda.stream(stream):
-            gl.replay()
+            for _ in range(4):
+                gl.replay()
             l0, l1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             l0.record(stream)
             gl.replay()
             l1.record(stream)
         torch.cuda.synchronize()
-        us = l0.elapsed_time(l1) * 1e3 / K_steps
+        us = l0.elapsed_time(l1) * 1e3 / SIDE_STEPS
         nb = alg_bytes(M, n, k) if fused else alg_bytes(M, n, k) - M * k + 4 * M
         wbytes = n * k // 2
         pus = min(sum(probe_read_us(dev_w[name][layer].data_ptr(), wbytes, g, 1) for layer in range(LAYERS)) / LAYERS for g in (512, 1024, 2048))
@@ -326,16 +330,17 @@ def main():
                 fn(0)
             stream.synchronize()
             with torch.cuda.graph(gl, stream=stream):
-                for i in range(K_steps):
+                for i in range(SIDE_STEPS):
                     fn(i % LAYERS)
             with torch.cuda.stream(stream):
-                gl.replay()
+                for _ in range(4):
+                    gl.replay()
                 l0, l1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                 l0.record(stream)
                 gl.replay()
                 l1.record(stream)
             torch.cuda.synchronize()
-            times[tag] = l0.elapsed_time(l1) * 1e3 / K_steps
+            times[tag] = l0.elapsed_time(l1) * 1e3 / SIDE_STEPS
             bits[tag] = dev_c["down"].clone()
             del gl
         wb = (n_gu * hid + hid * inter) // 2
