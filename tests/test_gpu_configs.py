@@ -63,6 +63,32 @@ def test_config1_decode_layer_set_as_the_fused_launches_the_benchmark_times(ctx,
         np.testing.assert_array_equal(host_u16(c), r["C"])
 
 
+# the iu8 linears of the reference's own 27B graph at TP = 1 (crates/saber-kernels/src/macaq_iu8.rs:931-947:
+# GDN in_proj_qkvz / in_proj_ba, gated attention qkv, out_proj / o_proj, MLP gate_up / down) -- the benchmark's
+# "27B-class" set shares only the last two with it
+SERVED_27B = [("gdn_qkvz", 16384, 5120), ("gdn_ba", 96, 5120), ("attn_qkv", 14336, 5120), ("o_proj", 5120, 6144),
+              ("gate_up", 34816, 5120), ("down", 5120, 17408)]
+
+
+@pytest.mark.parametrize("M", [1, 3, 16, 40, 300])
+def test_linear_shapes_of_the_served_27b_graph(ctx, M):
+    """Decode (fused where the law fuses, else producer + GEMM), the streamed band and a ragged prefill row count on
+    the served model's shapes, N = 96 (six column tiles: a workgroup with a dead tile) included."""
+    for name, n, k in SERVED_27B:
+        w8 = name in ("o_proj", "down") and M in (3, 40)     # the graph promotes some output-side projections to int8 rows
+        say(f"served 27B shape: {name} M={M} N={n} K={k} w8={w8}")
+        case = synth.dense_case(M, n, k, w8=w8, seed=100 + M)
+        r = ref.linear(case["X"], case["W"], case["ws"], w8, threads=16)
+        run = DenseRun(ctx, case, want_acc=False)
+        assert_dense_matches(run, r, w8)
+        if iu8.fused_holds(M, k):
+            c = torch.full((M, n), 0x7FC0, dtype=torch.int16, device="cuda")
+            ctx.linear_fused(iu8.W8 if w8 else iu8.W4, run.dev["x"].data_ptr(), run.dev["wf"].data_ptr(), run.dev["ws"].data_ptr(),
+                             c.data_ptr(), M, n, k)
+            torch.cuda.synchronize()
+            np.testing.assert_array_equal(host_u16(c), r["C"])
+
+
 def test_launch_refuses_a_block_the_kernel_is_not_written_for(ctx):
     """A descriptor under another launch law (the reference's 256-thread blocks under its own names,
     crates/saber-kernels/src/macaq_iu8.rs:429-489) is refused by name before anything is launched."""
