@@ -335,8 +335,10 @@ uint32_t pf_split(bool w8, uint32_t m, uint32_t n, uint32_t k, const PfVariant *
 // kind (int8 weights are twice the bytes a tile and have no unpack: the cells rank differently), fitted to
 // sustained timings of every cell on the four 27B-class shapes x 14 row counts from 65 to 8,192, weights
 // cold (successive launches walk copies that exceed the memory-side cache; with warm weights the 64 x 64
-// cell overtakes the 64 x 128 one at 256 rows, which no layer of a model sees). W4: 574 timings, the pick
-// is within 0.6 % of the fastest measured cell on all 56 shape x M points; W8, output-side shapes: every
+// cell overtakes the 64 x 128 one at 256 rows, which no layer of a model sees), and checked on shapes the fit had
+// not seen -- the served 27B graph's own 16384 x 5120, 14336 x 5120, 5120 x 6144 and 96 x 5120 at eight row counts,
+// which moved three small-cell rates and took the side-by-side term off the 64-row cells. W4: 850 timings, the
+// pick is within 0.6 % of the fastest measured cell on all 88 shape x M points; W8, output-side shapes: every
 // pick the fastest. The reference keeps its band tables the same way
 // (crates/saber-kernels/src/macaq_iu8.rs:150-212). One table for both kinds had sent the int8-weight
 // O and down projections at 2,048 rows to the 128 x 320 cell, 17-22 % behind the 256 x 160 cell there.
@@ -344,7 +346,7 @@ const PfVariant *pf_cell(bool w8, uint32_t m, uint32_t n, uint32_t k) {
   struct Cell { const char *tile; double tops_per_cu, tile_us; };
   struct Law { double fixed_us, cu_gbps, l2_tbps, lone, hbm_tbps, side_cap; Cell cells[11]; };
   static const Law W4 = {0.974, 90.000, 19.875, 1.422, 3.113, 2.116,
-                         {{"tn4_lbk64", 14.007, 3.223}, {"t256x320", 13.568, 4.138}, {"t256x224", 13.814, 14.000}, {"t128x320", 11.147, 7.968}, {"t256x160", 11.173, 8.857}, {"t128x256", 9.046, 1.844}, {"t128x128", 8.314, 2.045}, {"t128x128_o2", 9.622, 3.231}, {"t128x64_s", 4.711, 1.952}, {"t64x128_s", 7.589, 2.027}, {"t64x64_s", 6.116, 1.829}}};
+                         {{"tn4_lbk64", 14.007, 3.223}, {"t256x320", 13.568, 4.138}, {"t256x224", 13.814, 14.000}, {"t128x320", 11.147, 7.968}, {"t256x160", 11.173, 8.857}, {"t128x256", 9.046, 1.844}, {"t128x128", 8.799, 2.045}, {"t128x128_o2", 9.622, 3.231}, {"t128x64_s", 4.711, 1.952}, {"t64x128_s", 6.085, 2.027}, {"t64x64_s", 5.582, 1.829}}};
   static const Law W8 = {4.419, 75.175, 18.116, 1.782, 5.234, 1.935,
                          {{"tn4_lbk64", 13.145, 0.244}, {"t256x320", 12.800, 0.000}, {"t256x224", 11.270, 0.000}, {"t128x320", 6.328, 2.194}, {"t256x160", 11.499, 0.000}, {"t128x256", 10.761, 3.251}, {"t128x128", 8.069, 0.427}, {"t128x128_o2", 8.619, 0.229}, {"t128x64_s", 4.123, 0.073}, {"t64x128_s", 6.003, 2.817}, {"t64x64_s", 5.960, 0.000}}};
   const Law &law = w8 ? W8 : W4;
@@ -373,9 +375,12 @@ const PfVariant *pf_cell(bool w8, uint32_t m, uint32_t n, uint32_t k) {
     // the two-a-CU 128 x 128 cell alone on a CU (no more workgroups than CUs) has four waves to hide
     // its latencies with and measured well behind the eight-wave 128 x 128 cell there
     const double lone = (!strcmp(c.tile, "t128x128_o2") && grid <= CU_COUNT) ? law.lone : 1.0;
-    // cold weights: the row tiles that run side by side on one column block each fetch it from memory
+    // cold weights: the row tiles that run side by side on one column block each fetch it from memory -- those of the
+    // 128- and 256-row cells; the 64-row cells' neighbours share a column block's lines (fetch over operands 1.5-1.65 at
+    // four row tiles by the counters, and the wide projections of the served graph at 65-128 rows: 16.5-18.8 us on
+    // 64 x 128 where a doubled fetch would make it 27)
     const uint64_t gx = (n + v->block_n() - 1) / v->block_n(), gy = (m + v->block_m() - 1) / v->block_m();
-    const double side = std::min<double>((double)std::min<uint64_t>(gy, std::max<uint64_t>(1, grid / gx)), law.side_cap);
+    const double side = v->block_m() == 64 ? 1.0 : std::min<double>((double)std::min<uint64_t>(gy, std::max<uint64_t>(1, grid / gx)), law.side_cap);
     const double t_hbm = ((double)n * k * (w8 ? 1.0 : 0.5) * side + (double)m * k) / (law.hbm_tbps * 1e6);
     const double t = law.fixed_us + (double)per_wg * c.tile_us + lone * std::max(std::max(t_mfma, t_hbm), std::max(t_cu, t_l2));
     if (!best || t < best_t) best = v, best_t = t;

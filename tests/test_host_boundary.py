@@ -320,6 +320,14 @@ def test_prefill_cells_of_the_benchmark_shapes():
             # 128 x 256 for down, 33.2 against 39.7 for O)
             (1024, 5120, 17408): "t128x128_o2", (1024, 5120, 5120): "t128x128_o2", (1024, 7168, 5120): "t128x128_o2",
             (512, 5120, 5120): "t128x128", (128, 34816, 5120): "t128x128_o2"}
+    # shapes the fit had not seen: the served 27B graph's own projections (crates/saber-kernels/src/macaq_iu8.rs:931-947),
+    # each pick the fastest cell of a cold sweep of all of them (65 / 128 rows of the wide ones: 16.5-18.8 us on 64 x 128
+    # against 22.5-23.4 on 128 x 64, which the law chose before the side-by-side term came off the 64-row cells)
+    want.update({(65, 16384, 5120): "t64x128_s", (128, 14336, 5120): "t64x128_s", (256, 16384, 5120): "t128x128",
+                 (512, 14336, 5120): "t128x128_o2", (2048, 16384, 5120): "tn4_lbk64", (8192, 14336, 5120): "tn4_lbk64",
+                 (128, 5120, 6144): "t64x64_s", (256, 5120, 6144): "t64x128_s", (1024, 5120, 6144): "t128x128_o2",
+                 (2048, 5120, 6144): "t128x320", (4096, 5120, 6144): "t256x320", (2048, 96, 5120): "t64x64_s",
+                 (8192, 96, 5120): "t64x64_s"})
     for (m, n, k), tile in want.items():
         assert iu8.resolve(iu8.W4, m, n, k).kernel.decode() == "macaq_iu8_pf_w4_" + tile, (m, n, k)
     # int8 weights rank the cells differently (twice the bytes a tile, no unpack): the output-side projections
