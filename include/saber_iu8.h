@@ -370,7 +370,7 @@ int saber_iu8_linear_prefill_fused(saber_iu8_ctx *ctx, int wkind, const void *x_
                                    const float *w_scale, void *c_bf16, uint32_t m, uint32_t n, uint32_t k, void *stream);
 
 /* Workspace bytes the resolved GEMM needs (both 0 when it does not split). Ask before every
- * saber_iu8_gemm of a new shape: the law splits K in one band (K >= 16384, 49..128 rows, few tiles),
+ * saber_iu8_gemm of a new shape: the law splits K in one band (K >= 16384, 33..128 rows, few tiles),
  * and such a launch with `partial` / `counter` NULL is refused (SABER_IU8_E_ARG). */
 int saber_iu8_gemm_workspace(int wkind, uint32_t m, uint32_t n, uint32_t k, uint64_t *partial_bytes,
                              uint64_t *counter_bytes);

@@ -283,7 +283,12 @@ int resolve(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *out) 
   // The decode band ends where the tile GEMM's small cells overtake the streaming form (speed data of
   // this card: 17..32 rows stream unless the output is very wide, 33..48 unless it is wide, from 49
   // rows the tiles win on every shape measured).
-  const bool stream = m <= 16 || (m <= 32 && n <= 16384) || (m <= 48 && n <= 8192);
+  // A deep, narrow linear leaves the band at 33 rows already: where the tile law shares K over workgroups
+  // (pf_split), its 64 x 128 cell overtakes the three-tile streaming form (5120 x 17408 at 33 / 40 / 48 rows:
+  // 23.7 / 23.9 / 25.8 us on four shares against 28.2 / 28.3 / 31.3; up to 32 rows streaming wins, 18.0 against 22.4).
+  const PfVariant *split_cell = nullptr;
+  const uint32_t tile_ks = pf_split(wkind == SABER_IU8_W8, m, n, k, &split_cell);
+  const bool stream = m <= 16 || (m <= 32 && n <= 16384) || (m <= 48 && n <= 8192 && tile_ks == 0);
   if (m <= DECODE_MAX_M && stream) {
     const uint32_t tm = (m + 15) / 16;
     std::string name = fmt("macaq_iu8_dec_%s_tm%u", tag, tm);
@@ -299,9 +304,7 @@ int resolve(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *out) 
     const uint32_t nblk = (n + v->block_n() - 1) / v->block_n();
     return describe_dec(*v, m, n, k, decode_split(m, n, k, nblk, v->kw), out);
   }
-  const PfVariant *split_cell = nullptr;
-  if (const uint32_t ks = pf_split(wkind == SABER_IU8_W8, m, n, k, &split_cell))
-    return describe_pf(*split_cell, m, n, k, ks, out);
+  if (tile_ks) return describe_pf(*split_cell, m, n, k, tile_ks, out);
   return describe_pf(*pf_cell(wkind == SABER_IU8_W8, m, n, k), m, n, k, 0, out);
 }
 
@@ -313,7 +316,7 @@ int resolve(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *out) 
 // the partials cost ks*M*N*4 bytes each way and the last arriver sums alone -- so the rule is this
 // narrow. The launch then needs the `decode_partial` / `decode_counter` workspaces the descriptor lists.
 uint32_t pf_split(bool w8, uint32_t m, uint32_t n, uint32_t k, const PfVariant **cell) {
-  // measured at 49..128 rows only; above, the partials (ks * M * N * 4 bytes each way) grow with M
+  // measured at 33..128 rows; above, the partials (ks * M * N * 4 bytes each way) grow with M
   if (w8 || k < 16384 || m > 128) return 0;
   const PfVariant *v = pf_variant("macaq_iu8_pf_w4_t64x128_s");
   if (!v || !signature_for(std::string(v->name) + "_ks")) return 0;

@@ -251,13 +251,15 @@ def test_operands_past_4_gib_are_refused_by_the_tile_gemm():
 def test_launch_law_shares_k_only_on_deep_narrow_tile_gemms():
     """The one band where the law splits the tile GEMM: K >= 16384 and at most 80 tiles of the
     64x128 cell; the descriptor then names the `_ks` form, its z grid and both workspaces."""
-    for m, ks, tiles in ((49, 4, 40), (64, 4, 40), (65, 3, 80), (128, 3, 80)):
+    for m, ks, tiles in ((33, 4, 40), (48, 4, 40), (49, 4, 40), (64, 4, 40), (65, 3, 80), (128, 3, 80)):
         d = iu8.resolve(iu8.W4, m, 5120, 17408)
         assert d.kernel == b"macaq_iu8_pf_w4_t64x128_s_ks" and d.ks == ks and tuple(d.grid) == (tiles, 1, ks)
         assert d.workspace("decode_partial").bytes == ks * m * 5120 * 4 and d.workspace("decode_partial").kind == iu8.WS_SCRATCH
         c = d.workspace("decode_counter")
         assert c.bytes == tiles * 4 and c.kind == iu8.WS_PERSISTENT and c.zero_once
         assert iu8.gemm_workspace(iu8.W4, m, 5120, 17408) == (ks * m * 5120 * 4, tiles * 4)
+    # up to 32 rows the streaming form keeps a deep narrow linear too (18.0 against 22.4 us)
+    assert iu8.resolve(iu8.W4, 32, 5120, 17408).kernel == b"macaq_iu8_dec_w4_tm2"
     for wk, m, n, k in ((iu8.W4, 129, 5120, 17408), (iu8.W4, 64, 5120, 16256), (iu8.W4, 64, 12288, 17408),
                         (iu8.W8, 64, 5120, 17408), (iu8.W4, 2048, 5120, 17408), (iu8.W4, 64, 5120, 5120),
                         (iu8.W4, 4096, 128, 17408), (iu8.W4, 4096, 16, 16384)):       # many rows of a narrow output: few tiles, no split

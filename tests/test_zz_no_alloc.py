@@ -37,7 +37,7 @@ def run_both(ctx, M, N, K, seed):
 
 def test_static_workspace_gemm_equals_the_caller_workspace_gemm_twice_in_a_row(ctx):
     assert iu8.lib().saber_iu8_static_workspace_bytes() == 8 * 1024 * 1024 + 64 * 1024
-    # the band where the launch law splits K (K >= 16384, 49..128 rows, at most 80 tiles): first the
+    # the band where the launch law splits K (K >= 16384, 33..128 rows, at most 80 tiles): first the
     # largest such launch of the 27B-class layer, then a smaller one on the same static array
     for (M, N, K) in ((128, 5120, 17408), (64, 384, 16384)):
         say(f"static-workspace GEMM {M}x{N}x{K}")
