@@ -43,7 +43,10 @@ static __device__ __forceinline__ iu8_blk iu8_blk_of_grid() {
 // scales kept in LDS for the epilogue; `as` is not read. The tile's rows must fit: pow2(rows) * K <=
 // ALDS KiB (the host's rule). Every workgroup of a tile repeats its rows' quantisation, which is what
 // a producer launch in front would cost once -- worth it for the few rows an expert has in decode.
-template <int TM, bool W8, int NT, int KW, int WPB, int D, int ALDS, bool ACC, int MODE = 0>
+// EXACT (the staged forms): the first ring issued by every wave and the last steps as straight-line code, so that
+// the compiler counts the loads in flight at each consume (see the streamed form's ring below). It costs registers:
+// the grouped launches, held to 64 a lane for eight waves a SIMD, keep the plain loops.
+template <int TM, bool W8, int NT, int KW, int WPB, int D, int ALDS, bool ACC, int MODE = 0, bool EXACT = true>
 __device__ __forceinline__ void iu8_dec_body(const iu8_u8 *__restrict__ A, const iu8_u8 *__restrict__ W,
                                              const float *__restrict__ as, const float *__restrict__ ws,
                                              int *__restrict__ P, int *__restrict__ cnt, void *__restrict__ Cv,
@@ -84,7 +87,8 @@ __device__ __forceinline__ void iu8_dec_body(const iu8_u8 *__restrict__ A, const
   for (int j = 0; j < NT; ++j) {
     // a tile past N re-reads the last one and stores nothing; paired: tile j = 0 of the gate rows, 1 of the up rows
     const int ntj = PAIR ? (j / NP) * (ntiles >> 1) + min((B.bx * WN + wn) * NP + j % NP, (ntiles >> 1) - 1) : min(nt0 + j, ntiles - 1);
-    wp[j] = W + ((size_t)ntj * steps + s_lo + wk) * WSTEP + lane * 16;
+    // (EXACT: a k-wave past a short K issues the first ring all the same, on the share's last step, and drops it)
+    wp[j] = W + ((size_t)ntj * steps + (EXACT && ALDS > 0 ? min(s_lo + wk, steps - 1) : s_lo + wk)) * WSTEP + lane * 16;
   }
 
   iu8_v4i acc[TM][NT];
@@ -168,6 +172,12 @@ __device__ __forceinline__ void iu8_dec_body(const iu8_u8 *__restrict__ A, const
           ringa[ALDS ? 0 : slot][i][h] = *(const iu8_v4i *)(ap[i] + ((size_t)t * (2 * KW) + h) * 1024);
     }
   };
+  auto issue_w = [&](int slot, int t) {  // the staged ring: weights alone, no run-time test around a load
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int v = 0; v < WV; ++v) ring[slot][j][v] = iu8_ldg_nt(wp[j] + (size_t)t * (KW * WSTEP) + v * 1024);
+  };
   const int a_lane = (((lg << mr_shift) + min(ml, (1 << mr_shift) - 1)) << 4);
   auto consume = [&](int slot, int t) {
     iu8_v4i a0[TM], a1[TM];
@@ -208,9 +218,14 @@ __device__ __forceinline__ void iu8_dec_body(const iu8_u8 *__restrict__ A, const
         consume(0, t);
       }
     } else {
+      if constexpr (EXACT) {
 #pragma unroll
-      for (int i = 0; i < D; ++i)
-        if (i < T) issue(i, i);
+        for (int i = 0; i < D; ++i) issue_w(i, max(min(i, T - 1), 0));
+      } else {
+#pragma unroll
+        for (int i = 0; i < D; ++i)
+          if (i < T) issue(i, i);
+      }
       if constexpr (AQ) {
 #pragma clang fp contract(off)
         // the rows' maxima (f32 maxima of |x| as the producers take them, met by an integer max in LDS:
@@ -261,20 +276,51 @@ __device__ __forceinline__ void iu8_dec_body(const iu8_u8 *__restrict__ A, const
       }
       __syncthreads();
       int t0 = 0;
-      for (; t0 + 2 * D <= T; t0 += D) {  // steady state: every slot consumed and re-issued
+      if constexpr (EXACT) {
+        for (; t0 + 2 * D <= T; t0 += D) {
 #pragma unroll
-        for (int i = 0; i < D; ++i) {
-          consume(i, t0 + i);
-          issue(i, t0 + i + D);
-        }
-      }
-      for (; t0 < T; t0 += D) {  // drain
-#pragma unroll
-        for (int i = 0; i < D; ++i)
-          if (t0 + i < T) {
+          for (int i = 0; i < D; ++i) {
             consume(i, t0 + i);
-            if (t0 + i + D < T) issue(i, t0 + i + D);
+            __builtin_amdgcn_sched_barrier(0);
+            issue_w(i, t0 + i + D);
+            __builtin_amdgcn_sched_barrier(0);
           }
+        }
+        const int rest = T - t0;  // up to 2D - 1 steps left, min(rest, D) of them in the ring
+#pragma unroll
+        for (int e = 0; e < D; ++e) {
+          if (rest - D != e) continue;  // rest = D + e: e more steps to issue
+#pragma unroll
+          for (int i = 0; i < D; ++i) {
+            consume(i, t0 + i);
+            __builtin_amdgcn_sched_barrier(0);
+            if (i < e) issue_w(i, t0 + i + D);
+            __builtin_amdgcn_sched_barrier(0);
+          }
+#pragma unroll
+          for (int i = 0; i < e; ++i) consume(i, t0 + D + i);
+        }
+        if (rest < D) {
+#pragma unroll
+          for (int i = 0; i < D; ++i)
+            if (i < rest) consume(i, t0 + i);
+        }
+      } else {
+        for (; t0 + 2 * D <= T; t0 += D) {  // steady state: every slot consumed and re-issued
+#pragma unroll
+          for (int i = 0; i < D; ++i) {
+            consume(i, t0 + i);
+            issue(i, t0 + i + D);
+          }
+        }
+        for (; t0 < T; t0 += D) {  // drain
+#pragma unroll
+          for (int i = 0; i < D; ++i)
+            if (t0 + i < T) {
+              consume(i, t0 + i);
+              if (t0 + i + D < T) issue(i, t0 + i + D);
+            }
+        }
       }
       __syncthreads();  // every wave is done with the staged rows before s_mem holds partials
     }

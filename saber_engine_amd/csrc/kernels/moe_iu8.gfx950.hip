@@ -692,7 +692,7 @@ extern "C" __global__ __launch_bounds__(MOE_PTPB * MOE_TOPK) void moe_iu8_routeq
     const int live = meta[0], e = tile_expert[tile], row0 = tile_row0[tile], rows = tile_rows[tile];               \
     if (tile >= live) return;                                                                                      \
     const iu8_rows R{GATHER ? row_tok : nullptr, row0, min(rows, 16)};                                             \
-    iu8_dec_body<1, false, NT, KW, WPB, D, ALDS, false, MODE>(a, (const unsigned char *)xptr[2 * e], as,           \
+    iu8_dec_body<1, false, NT, KW, WPB, D, ALDS, false, MODE, false>(a, (const unsigned char *)xptr[2 * e], as,    \
                                                               (const float *)xptr[2 * e + 1], p, cnt, c, R, n, k); \
   }
 MOE_GROUPED_DEC(moe_iu8_grouped_w4_dec_g1, true, 1, 4, 8, 8, 20, 0, 8)
