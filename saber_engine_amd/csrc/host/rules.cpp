@@ -416,9 +416,8 @@ static int describe_rows(const char *op, const char *kernel, uint32_t rows, uint
 // The fused forms quantise rows whose int8 codes (rows rounded up to a power of two) fit the kernel's
 // staging area: up to 4 rows in 20 KiB (`_tm1`), up to 16 rows in 80 KiB (`_tm1_a80`). Every workgroup
 // repeats the rows' quantisation (about 0.5 us a row of 5,120 on this card), a producer launch costs
-// about 3 us once: the law takes the 80 KiB form for up to 4 rows (down at 2 rows: 14.4 against 17.3 us
-// as producer + GEMV; at 4 rows 16.0 against 17.4; QKV at 5 / 6 / 8 rows 9.0 / 9.2 / 9.9 against 8.8). The
-// kernel itself holds what `fused_form_holds` says, by name.
+// about 3 us once. The kernel itself holds what `fused_form_holds` says, by name; what the law launches is
+// `fused_holds` below.
 static uint64_t staged_bytes(uint32_t m, uint32_t k) {
   uint32_t mr = 1;
   while (mr < m) mr *= 2;
@@ -433,7 +432,14 @@ bool fused_form_holds(bool a80, uint32_t m, uint32_t k) {
 bool mlp_chain_form_holds(uint32_t m, uint32_t hidden, uint32_t inter) {
   return fused_small_holds(m, hidden) && (fused_small_holds(m, inter) || (m <= 4 && fused_form_holds(true, m, inter)));
 }
-bool fused_holds(uint32_t m, uint32_t k) { return fused_small_holds(m, k) || (m <= 4 && fused_form_holds(true, m, k)); }
+// The law: the 20 KiB form wherever it holds (1-4 rows: 5.7 / 5.3 / 16.7 us against 8.0 / 7.4 / 19.8 as two launches
+// at one row of the 27B layer's K = 5120 shapes, 6.9 / 6.7 / 17.3 against 8.3 / 7.7 / 19.5 at four); the 80 KiB form at
+// two rows (K = 17408: 13.9 against 15.2 us, 12288: 11.4 / 11.8) and at three rows of K >= 16384 (14.8 / 15.2); elsewhere
+// it loses to producer + the streamed GEMV (four rows: 16.0 / 15.2 at K = 17408, 10.5 / 9.5 at 8192, 9.2 / 8.5 at 6144;
+// three rows: 10.0 / 9.5 at 8192, 12.0 / 11.9 at 12288).
+bool fused_holds(uint32_t m, uint32_t k) {
+  return fused_small_holds(m, k) || ((m == 2 || (m == 3 && k >= 16384)) && fused_form_holds(true, m, k));
+}
 
 uint32_t fused_grid(uint32_t nblk) {
   if (nblk <= CU_COUNT) return nblk;
@@ -446,7 +452,7 @@ int resolve_fused(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc 
   const char *op = wkind == SABER_IU8_W8 ? "linear_i8a8_fused" : "linear_i4a8_fused";
   if (int rc = check_shape(op, m, n, k)) return rc;
   if (!fused_holds(m, k))
-    return fail(SABER_IU8_E_RULE, fmt("%s: %u rows of %u are not a fused launch (up to 4 rows, 20 KiB of codes or 80 KiB)", op, m, k));
+    return fail(SABER_IU8_E_RULE, fmt("%s: %u rows of %u are not a fused launch (up to 4 rows in 20 KiB of codes; 2 rows, or 3 of K >= 16384, in 80 KiB)", op, m, k));
   // one long row: the form that makes the row's codes just in time inside the weight stream (`_r1`). Measured on
   // this card against the several-row form at one row (cold weights, graph replay, N = 5120): K = 8,192 6.47
   // against 6.91 us, 12,288 7.82 against 8.38, 17,408 9.88 against 10.7-11.4, 20,480 10.97 against 11.83; at

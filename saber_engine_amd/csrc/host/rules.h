@@ -45,7 +45,7 @@ int pair(const saber_iu8_desc &first, const saber_iu8_desc &second, saber_iu8_de
 const DecVariant *pair_variant(const std::string &name);
 int resolve_quant(uint32_t m, uint32_t k, saber_iu8_desc *out);
 // The fused quant + GEMV of a decode linear; refuses (by name) shapes it does not hold.
-bool fused_holds(uint32_t m, uint32_t k);        // the law: a fused launch is what runs (up to 4 rows: the 20 KiB form, else the 80 KiB form)
+bool fused_holds(uint32_t m, uint32_t k);        // the law: a fused launch is what runs (the 20 KiB form where it holds; the 80 KiB form at 2 rows, and at 3 of K >= 16384)
 bool fused_form_holds(bool a80, uint32_t m, uint32_t k);  // what the kernel itself holds: `_tm1` 4 rows / 20 KiB, `_tm1_a80` 16 rows / 80 KiB
 bool fused_small_holds(uint32_t m, uint32_t k);  // the 20 KiB form: up to 4 rows (`_tm1`, and the MLP chain's first linear)
 bool mlp_chain_form_holds(uint32_t m, uint32_t hidden, uint32_t inter);  // the chain: 20 KiB at the hidden width, 20 or 80 KiB at the intermediate

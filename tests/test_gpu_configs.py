@@ -42,19 +42,23 @@ def test_config1_decode_layer_set(ctx, M):
         assert_dense_matches(DenseRun(ctx, case), r, False)
 
 
-@pytest.mark.parametrize("M", [1, 4])
+@pytest.mark.parametrize("M", [1, 2, 4])
 def test_config1_decode_layer_set_as_the_fused_launches_the_benchmark_times(ctx, M):
-    """The hot path as bench.py launches it: one fused quant + GEMV launch a linear
-    (macaq_iu8_decq_w4_r1 at one row, macaq_iu8_decq_w4_tm1[_a80] at four), on the four full layer shapes, against the oracle."""
+    """The hot path as bench.py launches it: one fused quant + GEMV launch a linear where the law fuses
+    (macaq_iu8_decq_w4_r1 at one long row, macaq_iu8_decq_w4_tm1, the 80 KiB form for down at two rows), producer + GEMV
+    where it does not (down at four rows), on the four full layer shapes, against the oracle."""
     for name, n, k in synth.LAYER_LINEARS:
-        assert iu8.fused_holds(M, k)
-        say(f"config 1, fused launch: {name} M={M} N={n} K={k}")
+        say(f"config 1, as the benchmark launches it: {name} M={M} N={n} K={k}")
         case = synth.dense_case(M, n, k, seed=M)
         r = ref.linear(case["X"], case["W"], case["ws"], False, threads=16)
+        if not iu8.fused_holds(M, k):
+            assert (M, k) == (4, 17408)
+            assert_dense_matches(DenseRun(ctx, case, want_acc=False), r, False)
+            continue
         x, wf, ws = dev_bf16_bits(case["X"]), dev_u8(iu8.repack_w4(case["W"])), dev_f32(case["ws"])
         c = torch.full((M, n), 0x7FC0, dtype=torch.int16, device="cuda")
         d = iu8.resolve_fused(iu8.W4, M, n, k)
-        # one long row (down): the just-in-time form; down at 4 rows: the 80 KiB form
+        # one long row (down): the just-in-time form; down at 2 rows: the 80 KiB form
         assert d.kernel == (b"macaq_iu8_decq_w4_r1" if M == 1 and k >= 8192 else b"macaq_iu8_decq_w4_tm1" if iu8.fused_small_holds(M, k) else b"macaq_iu8_decq_w4_tm1_a80")
         for a in ("q", "scale"):                # as the benchmark launches it: no optional outputs
             d.arg(a).kind = iu8.ARG_NULL_BUFFER
