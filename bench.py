@@ -347,6 +347,7 @@ def main():
         mlp = dict(kernel="macaq_iu8f_mlp_w4_tm1", weight_bytes=wb, us_chain=round(times["chain"], 2),
                    us_three_launches=round(times["three_launches"], 2),
                    us_two_linears_alone=round(per_linear["gate_up"]["us"] + per_linear["down"]["us"], 2),
+                   chain_pays_by_law=iu8.mlp_chain_pays(M, hid, inter),
                    gbps_chain=round(wb / times["chain"] / 1e3, 1), same_bytes=bool(torch.equal(bits["chain"], bits["three_launches"])),
                    state_status=int(state[iu8.MLP_CHAIN_STATUS_OFFSET // 4].item()))
         launch_fused("down", (K_steps - 1) % LAYERS)   # dev_c["down"] back to the step's own output for the spot check below
@@ -536,7 +537,7 @@ def main():
             same = bool(torch.equal(want, cs["down"]))
             tc = graph_us(chain)
             res["mlp_chain"] = dict(kernel=iu8.resolve_mlp_chain(DM, hid, inter).kernel.decode(), us_chain=round(tc, 2), us_three_launches=round(t3, 2),
-                                    same_bytes=same, state_status=int(state[iu8.MLP_CHAIN_STATUS_OFFSET // 4].item()))
+                                    chain_pays_by_law=iu8.mlp_chain_pays(DM, hid, inter), same_bytes=same, state_status=int(state[iu8.MLP_CHAIN_STATUS_OFFSET // 4].item()))
         return res
 
     if M == 1 and not args.no_other_m:

@@ -348,11 +348,17 @@ int saber_iu8_linear_fused(saber_iu8_ctx *ctx, int wkind, const void *x_bf16, co
  * of c a bf16 NaN (0x7FC0) -- and so does every later launch on that state block while the word is
  * set, e.g. the replays of a captured graph: the failure shows in the output itself. A caller that
  * finds the word set (or NaNs where the inputs had none) zeroes `state` and runs the three launches.
- * Launches that share one `state` must not overlap.
+ * Launches that share one `state` must not overlap. Work that other streams run on the device at the
+ * same time can hold compute units the grid needs: the launch then waits for it at its meeting (up to
+ * `spin`), so keep the stream's neighbours quiet around it or use the three launches.
+ * saber_iu8_mlp_chain_pays: where the one launch measured faster than the three on this card (one row
+ * of an intermediate width of 12,288 to 20,480, two rows of 13,824 to 20,480: 4-7 % and 2-3 %); elsewhere
+ * the three launches are as fast or faster, and a caller takes those.
  * Asynchronous. */
 #define SABER_IU8_MLP_CHAIN_STATE_BYTES (13 * 1024)
 #define SABER_IU8_MLP_CHAIN_STATUS_OFFSET (12 * 1024)
 int saber_iu8_mlp_chain_holds(uint32_t m, uint32_t hidden, uint32_t inter);
+int saber_iu8_mlp_chain_pays(uint32_t m, uint32_t hidden, uint32_t inter);
 int saber_iu8_resolve_mlp_chain(uint32_t m, uint32_t hidden, uint32_t inter, uint32_t spin, saber_iu8_desc *out);
 int saber_iu8_mlp_chain(saber_iu8_ctx *ctx, const void *x_bf16, const void *w_gu, const float *ws_gu, const void *w_dn,
                         const float *ws_dn, void *gu, void *p, void *state, void *c, uint32_t m, uint32_t hidden, uint32_t inter,

@@ -150,6 +150,13 @@ std::string band_toml() {
     if (resolve_fused(SABER_IU8_W4, 1, sh.n, sh.k, &d)) continue;
     o += fmt("grid.%s = %u\n", sh.op, d.grid[0]);
   }
+  o += "\n[row_producers]\n# macaq_i8_quant_* / macaq_i8_silu_mul_quant_*: 16 waves a row (_t1024) for rows wider than\n";
+  o += "# width_over while the row count leaves the card part idle, else the narrowest 256-thread form\n";
+  put(o, "t1024_width_over", T1024_WIDTH_OVER);
+  put(o, "t1024_quant_rows_max", T1024_QUANT_ROWS);
+  put(o, "t1024_quant_rows_max_wide", T1024_QUANT_ROWS_WIDE);
+  put(o, "t1024_silu_rows_max", T1024_SILU_ROWS);
+  put(o, "t1024_wide", T1024_WIDE);
   o += "\n[mlp_chain]\n";
   o += "# macaq_iu8f_mlp_w4_tm1: gate+up -> SiLU * up + requantisation -> down in one persistent launch while\n";
   o += "# the rows fit the fused form at both widths; every workgroup resident (one a CU).\n";
@@ -158,6 +165,9 @@ std::string band_toml() {
   put(o, "state_bytes", MLP_CHAIN_STATE_BYTES);
   put(o, "spin_default", MLP_CHAIN_SPIN);
   put(o, "workgroups_max", MLP_CHAIN_MAX_GRID);
+  o += "# where the one launch measured faster than the three: rows -> least intermediate width\n";
+  put(o, "pays_one_row_inter_min", MLP_CHAIN_PAYS_INTER_1);
+  put(o, "pays_two_rows_inter_min", MLP_CHAIN_PAYS_INTER_2);
   {
     saber_iu8_desc d;
     if (!resolve_mlp_chain(1, 5120, 17408, 0, &d)) o += fmt("grid.hidden5120_inter17408 = %u\n", d.grid[0]);

@@ -404,8 +404,9 @@ static int describe_rows(const char *op, const char *kernel, uint32_t rows, uint
   const bool w64 = strlen(kernel) > 4 && !strcmp(kernel + strlen(kernel) - 4, "_w64");
   if (w64 && (rows % 4 != 0 || width > 4096))
     return fail(SABER_IU8_E_RULE, fmt("%s: %s takes a multiple of 4 rows of at most 4096, got %u of %u", op, kernel, rows, width));
+  const bool t1024 = strlen(kernel) > 6 && !strcmp(kernel + strlen(kernel) - 6, "_t1024");
   d->grid[0] = w64 ? rows / 4 : rows, d->grid[1] = 1, d->grid[2] = 1;
-  d->block[0] = 256, d->block[1] = 1, d->block[2] = 1;
+  d->block[0] = t1024 ? 1024 : 256, d->block[1] = 1, d->block[2] = 1;
   d->n_launches = 1;
   d->ks = 1;
   if (int rc = fill_slots(kernel, d)) return rc;
@@ -431,6 +432,16 @@ bool fused_form_holds(bool a80, uint32_t m, uint32_t k) {
 // the 20 KiB form or, for up to 4 rows, the 80 KiB one
 bool mlp_chain_form_holds(uint32_t m, uint32_t hidden, uint32_t inter) {
   return fused_small_holds(m, hidden) && (fused_small_holds(m, inter) || (m <= 4 && fused_form_holds(true, m, inter)));
+}
+// Where the one launch beats the three (fused gate+up linear, 16-wave activation producer, streamed down GEMV), graph
+// replay on cold weights, hidden / intermediate in us chain / three: one row 5120/17408 32.9/34.2, 5120/13824 27.4/29.2,
+// 4096/14336 25.5/27.0, 4096/12288 23.0/24.2, 8192/8192 25.9/25.8, 5120/5120 18.9/17.5; two rows 5120/17408 35.3/36.0,
+// 5120/13824 29.9/30.9, 4096/14336 28.0/28.7, 4096/12288 25.7/25.4; three rows 36.5-36.8/36.6-37.4 and 31.9/31.6; four
+// rows 38.2/37.3, 33.7/32.6, 28.6/26.2. (A meeting inside the launch costs more than the gap between two launches;
+// what the chain saves is the activation's pass over memory and one launch.)
+bool mlp_chain_pays(uint32_t m, uint32_t hidden, uint32_t inter) {
+  if (inter > 20 * 1024) return false;  // not measured past the one-row form's 20 KiB of codes
+  return mlp_chain_form_holds(m, hidden, inter) && ((m == 1 && inter >= MLP_CHAIN_PAYS_INTER_1) || (m == 2 && inter >= MLP_CHAIN_PAYS_INTER_2));
 }
 // The law: the 20 KiB form wherever it holds (1-4 rows: 5.7 / 5.3 / 16.7 us against 8.0 / 7.4 / 19.8 as two launches
 // at one row of the 27B layer's K = 5120 shapes, 6.9 / 6.7 / 17.3 against 8.3 / 7.7 / 19.5 at four); the 80 KiB form at
@@ -517,8 +528,18 @@ int resolve_mlp_chain(uint32_t m, uint32_t hidden, uint32_t inter, uint32_t spin
 
 // The row kernels' register forms: the narrowest that holds the row (4,096 elements a group slot).
 // Many narrow rows go a wave a row (`base`_w64), the rest a workgroup a row (`base`_t256...).
-static std::string row_form(const char *base, uint32_t rows, uint32_t width) {
+// Rows wider than 4,096 whose count leaves the card part idle go 16 waves a row (`base`_t1024): measured on this
+// card, graph replay, 256-thread form / 1024-thread form in us -- the quantiser at 1 / 16 / 256 rows of 5,120:
+// 2.57/2.34, 2.98/2.74, 3.41/3.20; of 17,408: 3.90/2.91, 5.09/3.92, 6.72/5.49; at 512 rows 3.98/4.52 and 7.92/7.09, at
+// 1,024 4.84/6.32 and 13.3/14.3. The activation (exp and an IEEE divide an element) at 1 / 16 / 512 rows of 5,120:
+// 6.36/4.64, 6.75/5.02, 8.22/7.13; of 17,408: 13.6/7.50, 14.3/8.06, 18.8/14.9, and 47.0/42.4 at 2,048 rows (5,120
+// there: 17.5/22.1). Rows of 4,096: the two forms are within 3 % (a thread of either owns one group).
+static std::string row_form(const char *base, uint32_t rows, uint32_t width, bool silu = false) {
   if (width <= 2048 && rows % 4 == 0 && rows >= 64) return std::string(base) + "_w64";  // up to two groups a lane
+  if (width > T1024_WIDTH_OVER &&
+      (silu ? rows <= T1024_SILU_ROWS || width >= T1024_WIDE
+            : rows <= (width >= T1024_WIDE ? T1024_QUANT_ROWS_WIDE : T1024_QUANT_ROWS)))
+    return std::string(base) + "_t1024";
   const uint32_t slots = (width + 4095) / 4096;
   return std::string(base) + "_t256" + (slots <= 1 ? "_g1" : slots <= 2 ? "_g2" : slots <= 5 ? "_g5" : "");
 }
@@ -555,7 +576,7 @@ int resolve_quant_rows(uint32_t rows, uint32_t k, saber_iu8_desc *out) {
 }
 
 int resolve_silu_mul_quant(uint32_t rows, uint32_t n, saber_iu8_desc *out) {
-  if (int rc = describe_rows("silu_mul_quant_i8", row_form("macaq_i8_silu_mul_quant", rows, n).c_str(), rows, n, "n", out)) return rc;
+  if (int rc = describe_rows("silu_mul_quant_i8", row_form("macaq_i8_silu_mul_quant", rows, n, true).c_str(), rows, n, "n", out)) return rc;
   // the dense form has no row map; the routed form binds both (set_buffer)
   set_null(out, "row_tok");
   set_null(out, "meta");

@@ -33,6 +33,13 @@ constexpr uint32_t DECODE_MAX_M = 64;  // the decode band's last row count (maca
 constexpr uint32_t KS_MAX = 8;         // the largest grid-level split (macaq_iu8.rs:44)
 constexpr uint32_t CU_COUNT = 256;     // MI355X compute units
 constexpr uint32_t FUSED_R1_MIN_K = 8192;   // rows at least this long take the one-row fused decode form
+// the activation producers' 1024-thread forms: rows wider than one group a thread of the 256-thread form, up
+// to `ROWS` of them (the quantiser / the activation), or any number of rows at least `WIDE` wide for the activation
+constexpr uint32_t MLP_CHAIN_PAYS_INTER_1 = 12288, MLP_CHAIN_PAYS_INTER_2 = 13824;  // one / two rows: the chain beats the three launches from here
+constexpr uint32_t T1024_WIDTH_OVER = 4096;
+constexpr uint32_t T1024_QUANT_ROWS = 256, T1024_QUANT_ROWS_WIDE = 512;
+constexpr uint32_t T1024_SILU_ROWS = 512;
+constexpr uint32_t T1024_WIDE = 12288;
 
 // Grid-level split of a decode GEMM whose grid has `nblk` column blocks.
 uint32_t decode_split(uint32_t m, uint32_t n, uint32_t k, uint32_t nblk, uint32_t kw);
@@ -48,6 +55,7 @@ int resolve_quant(uint32_t m, uint32_t k, saber_iu8_desc *out);
 bool fused_holds(uint32_t m, uint32_t k);        // the law: a fused launch is what runs (the 20 KiB form where it holds; the 80 KiB form at 2 rows, and at 3 of K >= 16384)
 bool fused_form_holds(bool a80, uint32_t m, uint32_t k);  // what the kernel itself holds: `_tm1` 4 rows / 20 KiB, `_tm1_a80` 16 rows / 80 KiB
 bool fused_small_holds(uint32_t m, uint32_t k);  // the 20 KiB form: up to 4 rows (`_tm1`, and the MLP chain's first linear)
+bool mlp_chain_pays(uint32_t m, uint32_t hidden, uint32_t inter);        // ... and measured faster than the three launches
 bool mlp_chain_form_holds(uint32_t m, uint32_t hidden, uint32_t inter);  // the chain: 20 KiB at the hidden width, 20 or 80 KiB at the intermediate
 uint32_t fused_grid(uint32_t nblk);  // workgroups for nblk column blocks: one a CU, then equal shares of at most 8
 int resolve_fused(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *out);

@@ -142,6 +142,9 @@ int saber_iu8_fused_holds(uint32_t m, uint32_t k) { return fused_holds(m, k) ? 1
 int saber_iu8_mlp_chain_holds(uint32_t m, uint32_t hidden, uint32_t inter) {
   return mlp_chain_form_holds(m, hidden, inter) ? 1 : 0;
 }
+int saber_iu8_mlp_chain_pays(uint32_t m, uint32_t hidden, uint32_t inter) {
+  return mlp_chain_pays(m, hidden, inter) ? 1 : 0;
+}
 int saber_iu8_resolve_fused(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *out) {
   if (!out) return fail(SABER_IU8_E_ARG, "resolve_fused: null descriptor");
   return resolve_fused(wkind, m, n, k, out);

@@ -14,6 +14,8 @@
 //                                 -> q, scale over N                       (grid M, block 256)
 //                                 (crates/saber-kernels/hip/mxfp4_hadi8.hip:118-146 without the
 //                                 Hadamard; signature crates/saber-kernels/src/abi.rs:315-320)
+//   macaq_i8_quant_t1024, macaq_i8_silu_mul_quant_t1024   the first and the fifth with 16 waves a row (block
+//                                 1024): few rows of more than 4,096 elements
 //   macaq_i8_quant_w64, macaq_i8_silu_mul_quant_w64   the same two for rows of up to 4,096 elements,
 //                                 a wave a row, four rows a workgroup (grid M/4, block 256)
 //   macaq_i8_silu_mul_quant_lut_w64   the second with the bf16 silu read from a 65,536-entry table in
@@ -38,31 +40,32 @@ static __device__ __forceinline__ int i8q_row() {
   return (b & ~127) + (b & 7) * 16 + ((b & 127) >> 3);
 }
 
+template <int T = I8Q_T>
 static __device__ __forceinline__ float i8q_block_max(float v) {
-  __shared__ float s_w[I8Q_T / 64];
+  __shared__ float s_w[T / 64];
   v = iu8_wave_max_nonneg(v);
   if ((threadIdx.x & 63) == 0) s_w[threadIdx.x >> 6] = v;
   __syncthreads();
   float r = s_w[0];
 #pragma unroll
-  for (int w = 1; w < I8Q_T / 64; ++w) r = fmaxf(r, s_w[w]);
+  for (int w = 1; w < T / 64; ++w) r = fmaxf(r, s_w[w]);
   return r;
 }
 
 // codes of one row from v[g][16] (f32 values), written in A fragment order (RM: row-major, K bytes a row)
 // SCALE_ONLY: the row's scale alone (the row-maximum pass in front of a GEMM that makes the codes itself)
-template <int I8Q_MAXG, bool RM = false, bool SCALE_ONLY = false>
+template <int I8Q_MAXG, bool RM = false, bool SCALE_ONLY = false, int T = I8Q_T>
 static __device__ __forceinline__ void i8q_tail(float (&v)[I8Q_MAXG][16], int G, iu8_u8 *__restrict__ q,
                                                 float *__restrict__ scale, int row, int K) {
   const int tid = threadIdx.x;
   float amax = 0.f;
 #pragma unroll
   for (int i = 0; i < I8Q_MAXG; ++i) {
-    if (tid + i * I8Q_T >= G) continue;
+    if (tid + i * T >= G) continue;
 #pragma unroll
     for (int j = 0; j < 16; ++j) amax = fmaxf(amax, fabsf(v[i][j]));
   }
-  amax = i8q_block_max(amax);
+  amax = i8q_block_max<T>(amax);
   const float sc = fmaxf(__fdiv_rn(amax, 127.f), 1e-30f);
   const float rcp = __fdiv_rn(1.f, sc);
   if (tid == 0) scale[row] = sc;
@@ -70,7 +73,7 @@ static __device__ __forceinline__ void i8q_tail(float (&v)[I8Q_MAXG][16], int G,
   iu8_u8 *qrow = q + (size_t)(row >> 4) * (K >> 6) * 1024 + (row & 15) * 16;
 #pragma unroll
   for (int i = 0; i < I8Q_MAXG; ++i) {
-    const int g = tid + i * I8Q_T;
+    const int g = tid + i * T;
     if (g >= G) continue;
     unsigned d[4];
 #pragma unroll
@@ -115,7 +118,7 @@ static __device__ __forceinline__ void i8q_tail_pk(const unsigned (&pk)[I8Q_MAXG
 // `row_tok` / `meta` (optional, may be null): with them output row r is the quantised input row
 // row_tok[r] (the expert-major rows of a routed layer, gathered here once so that the grouped GEMM
 // reads whole fragments); pad rows (row_tok < 0) and rows past meta[1] are skipped.
-template <int I8Q_MAXG, bool RM = false, bool SCALE_ONLY = false>
+template <int I8Q_MAXG, bool RM = false, bool SCALE_ONLY = false, int T = I8Q_T>
 static __device__ __forceinline__ void i8q_quant_body(const unsigned short *__restrict__ x, unsigned char *__restrict__ q,
                                                       float *__restrict__ scale, int k,
                                                       const int *__restrict__ row_tok = nullptr,
@@ -129,6 +132,7 @@ static __device__ __forceinline__ void i8q_quant_body(const unsigned short *__re
   }
   const unsigned short *xr = x + (size_t)src * k;
   if constexpr (I8Q_MAXG >= 5) {
+    static_assert(I8Q_MAXG < 5 || T == I8Q_T, "the packed forms are the 256-thread ones");
     // The long forms request a row's pieces all at once (i8q_pk_load) and keep them packed as they came, 8
     // registers a group instead of 16: the form for up to 20,480 elements then runs eight waves a SIMD
     // (2,048 rows of 17,408: 26.0 -> 21.9 us). The forms of one or two groups measured 4-8 % slower this way.
@@ -140,7 +144,7 @@ static __device__ __forceinline__ void i8q_quant_body(const unsigned short *__re
     float v[I8Q_MAXG][16];
 #pragma unroll
     for (int i = 0; i < I8Q_MAXG; ++i) {
-      const int g = threadIdx.x + i * I8Q_T;
+      const int g = threadIdx.x + i * T;
       if (g >= G) continue;
       const iu8_v4u lo = *(const iu8_v4u *)(xr + g * 16), hi = *(const iu8_v4u *)(xr + g * 16 + 8);
 #pragma unroll
@@ -151,7 +155,7 @@ static __device__ __forceinline__ void i8q_quant_body(const unsigned short *__re
         v[i][8 + 2 * w + 1] = __uint_as_float(hi[w] & 0xFFFF0000u);
       }
     }
-    i8q_tail<I8Q_MAXG, RM, SCALE_ONLY>(v, G, q, scale, row, k);
+    i8q_tail<I8Q_MAXG, RM, SCALE_ONLY, T>(v, G, q, scale, row, k);
   }
 }
 #define I8Q_QUANT(name, MAXG, WPE)                                                                              \
@@ -204,7 +208,7 @@ static __device__ __forceinline__ float i8q_silu_bf16(float x) {
 // `row_tok` / `meta` are optional (may be null): with them the kernel runs on the expert-major
 // rows of a routed layer and skips pad rows (row_tok < 0) and rows past meta[1]
 // (signature crates/saber-kernels/src/abi.rs:344-351).
-template <int I8Q_MAXG>
+template <int I8Q_MAXG, int T = I8Q_T>
 static __device__ __forceinline__ void i8q_silu_body(const unsigned short *__restrict__ gu, unsigned char *__restrict__ q,
                                                      float *__restrict__ scale, int n, const int *__restrict__ row_tok,
                                                      const int *__restrict__ meta) {
@@ -216,7 +220,7 @@ static __device__ __forceinline__ void i8q_silu_body(const unsigned short *__res
   float v[I8Q_MAXG][16];
 #pragma unroll
   for (int i = 0; i < I8Q_MAXG; ++i) {
-    const int g = threadIdx.x + i * I8Q_T;
+    const int g = threadIdx.x + i * T;
     if (g >= G) continue;
     union { iu8_v4u u[2]; unsigned short h[16]; } vg, vu;
     vg.u[0] = *(const iu8_v4u *)(gr + g * 16);
@@ -229,7 +233,7 @@ static __device__ __forceinline__ void i8q_silu_body(const unsigned short *__res
       v[i][j] = iu8_bf16_f32((unsigned short)iu8_bf16_bits(t * iu8_bf16_f32(vu.h[j])));
     }
   }
-  i8q_tail<I8Q_MAXG>(v, G, q, scale, row, n);
+  i8q_tail<I8Q_MAXG, false, false, T>(v, G, q, scale, row, n);
 }
 #define I8Q_SILU(name, MAXG)                                                                                     \
   extern "C" __global__ __launch_bounds__(I8Q_T) void name(                                                      \
@@ -242,6 +246,20 @@ I8Q_SILU(macaq_i8_silu_mul_quant_t256_g5, 5)
 I8Q_SILU(macaq_i8_silu_mul_quant_t256_g2, 2)
 I8Q_SILU(macaq_i8_silu_mul_quant_t256_g1, 1)
 #undef I8Q_SILU
+
+// Few long rows: 16 waves a row, a thread owns groups g = tid + i*1024 (rows of up to 32,768 elements).
+// With fewer rows than CUs a row's time is one workgroup's, and a 256-thread workgroup walks a row of
+// 17,408 in five dependent steps a thread (5 groups of loads, conversions, exps); here it is two at most.
+extern "C" __global__ __launch_bounds__(1024) void macaq_i8_quant_t1024(const unsigned short *__restrict__ x,
+                                                                        unsigned char *__restrict__ q,
+                                                                        float *__restrict__ scale, int k) {
+  i8q_quant_body<2, false, false, 1024>(x, q, scale, k);
+}
+extern "C" __global__ __launch_bounds__(1024) void macaq_i8_silu_mul_quant_t1024(
+    const unsigned short *__restrict__ gu, unsigned char *__restrict__ q, float *__restrict__ scale, int n,
+    const int *__restrict__ row_tok, const int *__restrict__ meta) {
+  i8q_silu_body<2, 1024>(gu, q, scale, n, row_tok, meta);
+}
 
 // ---------------------------------------------------------------------------- a wave a row
 // Rows of up to 4,096 elements: four rows a workgroup, one wave each, a lane owns groups

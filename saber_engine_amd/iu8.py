@@ -119,6 +119,7 @@ def lib():
         L.saber_iu8_gemm_acc.argtypes = [C.c_void_p, C.c_int] + [C.c_void_p] * 3 + [C.c_uint32] * 3 + [C.c_void_p]
         L.saber_iu8_fused_holds.argtypes = [C.c_uint32, C.c_uint32]
         L.saber_iu8_mlp_chain_holds.argtypes = [C.c_uint32] * 3
+        L.saber_iu8_mlp_chain_pays.argtypes = [C.c_uint32] * 3
         L.saber_iu8_pair.argtypes = [C.POINTER(Desc)] * 3
         L.saber_iu8_pair_ordered.argtypes = [C.POINTER(Desc)] * 2 + [C.c_int, C.POINTER(Desc)]
         L.saber_iu8_load_plugin.argtypes = [C.c_void_p, C.c_char_p]
@@ -228,6 +229,11 @@ def fused_small_holds(m, k):
 
 def mlp_chain_holds(m, hidden, inter):
     return bool(lib().saber_iu8_mlp_chain_holds(m, hidden, inter))
+
+
+def mlp_chain_pays(m, hidden, inter):
+    """The one-launch MLP measured faster than the three launches at this shape."""
+    return bool(lib().saber_iu8_mlp_chain_pays(m, hidden, inter))
 
 
 def resolve_fused(wkind, m, n, k):

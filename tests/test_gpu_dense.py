@@ -327,3 +327,41 @@ def test_quant_rows_with_nan_and_infinity(ctx, K):
         np.testing.assert_array_equal(s.cpu().numpy().view(np.uint32), want_s.view(np.uint32))
         got = q.cpu().numpy().view(np.int8).reshape(M, K) if rm else iu8.unpack_a(q.cpu().numpy(), M, K)
         np.testing.assert_array_equal(got, want_q)
+
+
+def _row_forms(base, width):
+    """Every form of a row producer that holds rows of `width`, by kernel name and block size."""
+    slots = -(-width // 4096)
+    forms = [(base + "_t256" + sfx, 256) for need, sfx in ((1, "_g1"), (2, "_g2"), (5, "_g5"), (8, "")) if slots <= need]
+    return forms + [(base + "_t1024", 1024)]
+
+
+@pytest.mark.parametrize("M,K", [(1, 17408), (3, 5120), (12, 4160), (16, 32768), (5, 64), (33, 16384), (2, 20480)])
+def test_row_producers_every_form_that_holds_the_row(ctx, M, K):
+    """The quantiser and the SiLU * up + requant producer, launched by name in each of their register
+    forms (256 threads with 1, 2, 5 or 8 groups a thread; 1024 threads with 2): the same codes and
+    scales as the oracle from all of them, on rows with a NaN and an infinity among them."""
+    say(f"row producers, every form: M={M} K={K}")
+    rng = np.random.default_rng(M * 131 + K)
+    X = synth.f32_to_bf16_bits((rng.standard_normal((M, K)) * 2).astype(np.float32))
+    GU = synth.f32_to_bf16_bits((rng.standard_normal((M, 2 * K)) * 3).astype(np.float32))
+    X[M - 1, K - 1] = 0x7FC0
+    if M > 1:
+        X[0, K // 2], GU[0, K + K // 3] = 0x7F80, 0xFF80
+    want_q, want_s = ref.quant_bf16(X)
+    want_q2, want_s2, _ = ref.silu_mul_quant(GU)
+    x, gu = dev_bf16_bits(X), dev_bf16_bits(GU)
+    law_q, law_a = iu8.resolve_quant(M, K), iu8.resolve_silu_mul_quant(M, K)
+    assert (law_q.kernel.decode(), law_q.block[0]) in _row_forms("macaq_i8_quant", K)
+    assert (law_a.kernel.decode(), law_a.block[0]) in _row_forms("macaq_i8_silu_mul_quant", K)
+    for base, src, key, resolve, wq, wsc in (("macaq_i8_quant", x, "x", iu8.resolve_quant, want_q, want_s),
+                                            ("macaq_i8_silu_mul_quant", gu, "gu", iu8.resolve_silu_mul_quant, want_q2, want_s2)):
+        for name, block in _row_forms(base, K):
+            d = resolve(M, K)
+            d.kernel, d.block[0] = name.encode(), block
+            q = torch.full((iu8.a_bytes(M, K),), 0x55, dtype=torch.uint8, device="cuda")
+            s = torch.zeros(M, dtype=torch.float32, device="cuda")
+            ctx.launch(d, {key: src.data_ptr(), "q": q.data_ptr(), "scale": s.data_ptr()})
+            torch.cuda.synchronize()
+            np.testing.assert_array_equal(s.cpu().numpy().view(np.uint32), wsc.view(np.uint32), err_msg=name)
+            np.testing.assert_array_equal(iu8.unpack_a(q.cpu().numpy(), M, K), wq, err_msg=name)

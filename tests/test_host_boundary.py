@@ -148,6 +148,22 @@ def test_reference_symbol_names_are_answered_by_the_law():
         iu8.describe("macaq_iu8f_pf_w4_bm128", 400, 5120, 17408, ks=2)
 
 
+def test_row_producer_forms_by_law():
+    """The activation producers' form for a (rows, width): a wave a row for many narrow rows, 16 waves a row
+    for rows wider than 4,096 whose count leaves the card part idle, else the narrowest 256-thread form."""
+    for rows, width, quant, act in ((1, 5120, "t1024", "t1024"), (16, 17408, "t1024", "t1024"), (256, 8192, "t1024", "t1024"),
+                                    (257, 8192, "t256_g2", "t1024"), (512, 5120, "t256_g2", "t1024"), (513, 5120, "t256_g2", "t256_g2"),
+                                    (512, 12288, "t1024", "t1024"), (2048, 17408, "t256_g5", "t1024"), (2048, 12288, "t256_g5", "t1024"),
+                                    (8, 4096, "t256_g1", "t256_g1"), (64, 2048, "w64", "w64"), (6, 2048, "t256_g1", "t256_g1"),
+                                    (1, 32768, "t1024", "t1024"), (4096, 24576, "t256", "t1024")):
+        q, a = iu8.resolve_quant(rows, width), iu8.resolve_silu_mul_quant(rows, width)
+        assert q.kernel.decode() == "macaq_i8_quant_" + quant and a.kernel.decode() == "macaq_i8_silu_mul_quant_" + act, (rows, width)
+        for d, form in ((q, quant), (a, act)):
+            assert d.block[0] == (1024 if form == "t1024" else 256) and d.grid[0] == (rows // 4 if form == "w64" else rows)
+    with pytest.raises(iu8.IU8Error):
+        iu8.resolve_quant(4, 32832)
+
+
 def test_fused_quant_tile_gemm_descriptors():
     """macaq_iu8_pfq_*: the geometry of the cell the suffix names, the pf kernarg list with `x` for `a`."""
     d = iu8.describe("macaq_iu8_pfq_w4_t256x160", 2048, 5120, 17408)
@@ -212,6 +228,15 @@ def test_band_table_is_the_launch_law():
     d = iu8.resolve_mlp_chain(1, 5120, 17408)
     assert d.grid[0] == c["grid"]["hidden5120_inter17408"] <= 256 and d.block[0] == c["threads"]
     assert d.workspace("state").bytes == c["state_bytes"] == iu8.MLP_CHAIN_STATE_BYTES and d.arg("spin").ival == c["spin_default"]
+    # where the chain measured faster than the three launches: one row of a wide intermediate, two of a wider one
+    assert c["pays_one_row_inter_min"] == 12288 and c["pays_two_rows_inter_min"] == 13824
+    for m, hid, inter, pays in ((1, 5120, 17408, True), (1, 4096, 12288, True), (1, 8192, 8192, False), (1, 5120, 5120, False),
+                                (2, 5120, 17408, True), (2, 5120, 13824, True), (2, 4096, 12288, False), (3, 5120, 17408, False),
+                                (4, 5120, 17408, False), (1, 5120, 24576, False), (5, 5120, 17408, False)):
+        assert iu8.mlp_chain_pays(m, hid, inter) == pays, (m, hid, inter)
+        assert not pays or iu8.mlp_chain_holds(m, hid, inter)
+    rp = t["row_producers"]
+    assert (rp["t1024_width_over"], rp["t1024_quant_rows_max"], rp["t1024_quant_rows_max_wide"], rp["t1024_silu_rows_max"], rp["t1024_wide"]) == (4096, 256, 512, 512, 12288)
 
 
 def test_device_profile_is_the_planners_struct_as_data():
