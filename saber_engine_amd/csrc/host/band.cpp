@@ -266,6 +266,15 @@ std::string band_toml() {
       put(o, "threads", v->threads());
       put(o, "grid", std::string("[ceil(n / block_n), 1, ks]"));
       put(o, "kernarg", std::string("dec"));
+    } else if (name == "macaq_iu8_dec_w4_tm1_s80" || name == "macaq_iu8_dec_w8_tm1_s80") {
+      put(o, "regime", std::string("decode"));
+      putb(o, "w8", name[15] == '8');
+      put(o, "rows_max", 16);
+      put(o, "k_max", 5120);
+      put(o, "block_n", 32);
+      put(o, "threads", 1024);
+      put(o, "grid", std::string("[blocks = ceil(n / 32); blocks <= cu_count ? blocks : ceil(blocks / min(8, ceil(blocks / cu_count))), 1, 1] persistent"));
+      put(o, "kernarg", std::string("dec"));
     } else if (const PfVariant *v = pf_variant(ks_form ? name.substr(0, name.size() - 3) : name)) {
       put(o, "regime", std::string("prefill"));
       putb(o, "w8", v->w8 != 0);

@@ -175,7 +175,49 @@ static int describe_pf(const PfVariant &v, uint32_t m, uint32_t n, uint32_t k, u
   return 0;
 }
 
+// The streaming decode cell of M rows: tm 16-row tiles; one tile's live rows staged in LDS when they fit the 20 KiB
+// form, else streamed from L2 beside the weights.
+static std::string dec_stream_name(const char *tag, uint32_t m, uint32_t k) {
+  const uint32_t tm = (m + 15) / 16;
+  std::string name = fmt("macaq_iu8_dec_%s_tm%u", tag, tm);
+  if (tm == 1) {
+    uint32_t mr = 1;
+    while (mr < m) mr *= 2;
+    if ((uint64_t)mr * k > 20 * 1024) name += "_a0";
+  }
+  return name;
+}
+
+// The persistent GEMV of up to 16 quantised rows whose 16-row tile is staged once a workgroup in 80 KiB of LDS
+// (`macaq_iu8_dec_{w4,w8}_tm1_s80`): the fused forms' geometry (16 waves, 32 columns a block, at most 8 blocks a
+// workgroup) on the decode kernarg list.
+bool staged80_holds(uint32_t m, uint32_t k) { return m >= 1 && m <= 16 && (uint64_t)k * 16 <= 80 * 1024; }
+static int describe_s80(bool w8, uint32_t m, uint32_t n, uint32_t k, uint32_t ks, saber_iu8_desc *d) {
+  const char *op = w8 ? "gemm_i8a8" : "gemm_i4a8";
+  const std::string name = fmt("macaq_iu8_dec_%s_tm1_s80", w8 ? "w8" : "w4");
+  if (int rc = check_shape(op, m, n, k)) return rc;
+  if (ks != 1) return fail(SABER_IU8_E_RULE, name + ": the staged form does not split K");
+  if (!staged80_holds(m, k))
+    return fail(SABER_IU8_E_RULE, fmt("%s: %u rows of %u do not fit one 16-row tile in 80 KiB (K <= 5120)", name.c_str(), m, k));
+  memset(d, 0, sizeof *d);
+  copy_name(d->op, sizeof d->op, op);
+  copy_name(d->plugin, sizeof d->plugin, "macaq_iu8");
+  copy_name(d->kernel, sizeof d->kernel, name);
+  d->grid[0] = fused_grid((n + 31) / 32), d->grid[1] = 1, d->grid[2] = 1;
+  d->block[0] = 1024, d->block[1] = 1, d->block[2] = 1;
+  d->n_launches = 1;
+  d->ks = 1;
+  if (int rc = fill_slots(name, d)) return rc;
+  set_i32(d, "m", m);
+  set_i32(d, "n", n);
+  set_i32(d, "k", k);
+  set_null(d, "decode_partial");
+  set_null(d, "decode_counter");
+  return 0;
+}
+
 int describe(const std::string &kernel, uint32_t m, uint32_t n, uint32_t k, uint32_t ks, saber_iu8_desc *out) {
+  if (kernel == "macaq_iu8_dec_w4_tm1_s80" || kernel == "macaq_iu8_dec_w8_tm1_s80") return describe_s80(kernel[15] == '8', m, n, k, ks, out);
   if (const DecVariant *v = dec_variant(kernel)) return describe_dec(*v, m, n, k, ks, out);
   if (const PfVariant *v = pf_variant(kernel)) {
     if (ks != 1) return fail(SABER_IU8_E_RULE, kernel + ": the prefill tile does not split K (its `_ks` form does)");
@@ -230,6 +272,22 @@ static bool int_arg(const saber_iu8_desc &d, const char *name, int64_t *v) {
 // tiling and one staging form), M and K.
 int pair(const saber_iu8_desc &first, const saber_iu8_desc &second, saber_iu8_desc *out, int order) {
   static const char PREFIX[] = "macaq_iu8_dec_w4_";
+  // a half the law gave the staged persistent form is paired as its streamed form: the pair kernels are that geometry
+  for (const saber_iu8_desc *h : {&first, &second})
+    if (!strcmp(h->kernel, "macaq_iu8_dec_w4_tm1_s80")) {
+      saber_iu8_desc s[2];
+      const saber_iu8_desc *in[2] = {&first, &second};
+      for (int i = 0; i < 2; ++i) {
+        int64_t hm = 0, hn = 0, hk = 0;
+        s[i] = *in[i];
+        if (!strcmp(in[i]->kernel, "macaq_iu8_dec_w4_tm1_s80")) {
+          if (!int_arg(*in[i], "m", &hm) || !int_arg(*in[i], "n", &hn) || !int_arg(*in[i], "k", &hk))
+            return fail(SABER_IU8_E_RULE, "macaq iu8 pair: a half without its m, n, k");
+          if (int rc = describe(dec_stream_name("w4", (uint32_t)hm, (uint32_t)hk), (uint32_t)hm, (uint32_t)hn, (uint32_t)hk, 1, &s[i])) return rc;
+        }
+      }
+      return pair(s[0], s[1], out, order);
+    }
   const std::string k0 = first.kernel, k1 = second.kernel;
   const DecVariant *v0 = dec_variant(k0), *v1 = dec_variant(k1);
   int64_t m0 = 0, kk0 = 0, n0 = 0, m1 = 0, kk1 = 0, n1 = 0;
@@ -290,15 +348,16 @@ int resolve(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *out) 
   const uint32_t tile_ks = pf_split(wkind == SABER_IU8_W8, m, n, k, &split_cell);
   const bool stream = m <= 16 || (m <= 32 && n <= 16384) || (m <= 48 && n <= 8192 && tile_ks == 0);
   if (m <= DECODE_MAX_M && stream) {
-    const uint32_t tm = (m + 15) / 16;
-    std::string name = fmt("macaq_iu8_dec_%s_tm%u", tag, tm);
-    if (tm == 1) {
-      // live rows staged in LDS when they fit the 20 KiB form, else streamed from L2 beside the
-      // weights (the 80 KiB staged form stays loadable by name; it measured slower on every shape)
-      uint32_t mr = 1;
-      while (mr < m) mr *= 2;
-      if ((uint64_t)mr * k > 20 * 1024) name += "_a0";
-    }
+    // Up to 16 rows of K <= 5120: the persistent form that stages the 16-row tile once a workgroup (`_s80`) where
+    // it measured faster than the streamed one, which re-reads the tile from L2 once a 32-column block. W4, 9-16
+    // rows: everywhere (gate+up 34816 x 5120 19.1 -> 16.6 us, 28672 x 4096 13.2 -> 12.1, 14336 x 5120 9.4 -> 9.0,
+    // QKV / O 6.1 / 5.9 -> 6.05 / 5.8); up to 8 rows, and int8 weights at any row count, from 64 MiB of weights
+    // (W4 5-8 rows: gate+up 16.6-17.9 -> 16.4-17.2, 28672 x 4096 even, 14336 x 5120 8.5 -> 9.0 the other way;
+    // W8: gate+up 31.3 -> 28.4, 28672 x 4096 21.0 -> 19.9, 14336 x 5120 14.3 -> 13.6, QKV 8.1 -> 8.4 the other way).
+    if (m > 4 && staged80_holds(m, k) &&
+        ((m > 8 && wkind == SABER_IU8_W4) || (uint64_t)n * k / (wkind == SABER_IU8_W8 ? 1 : 2) >= S80_MIN_BYTES))
+      return describe_s80(wkind == SABER_IU8_W8, m, n, k, 1, out);
+    const std::string name = dec_stream_name(tag, m, k);
     const DecVariant *v = dec_variant(name);
     if (!v) return fail(SABER_IU8_E_RULE, name + ": no such variant");
     const uint32_t nblk = (n + v->block_n() - 1) / v->block_n();

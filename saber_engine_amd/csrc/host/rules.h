@@ -36,6 +36,7 @@ constexpr uint32_t FUSED_R1_MIN_K = 8192;   // rows at least this long take the 
 // the activation producers' 1024-thread forms: rows wider than one group a thread of the 256-thread form, up
 // to `ROWS` of them (the quantiser / the activation), or any number of rows at least `WIDE` wide for the activation
 constexpr uint32_t MLP_CHAIN_PAYS_INTER_1 = 12288, MLP_CHAIN_PAYS_INTER_2 = 13824;  // one / two rows: the chain beats the three launches from here
+constexpr uint64_t S80_MIN_BYTES = 64ull << 20;  // the staged persistent GEMV: weights from here at up to 8 rows, and for int8 weights
 constexpr uint32_t T1024_WIDTH_OVER = 4096;
 constexpr uint32_t T1024_QUANT_ROWS = 256, T1024_QUANT_ROWS_WIDE = 512;
 constexpr uint32_t T1024_SILU_ROWS = 512;
@@ -57,6 +58,7 @@ bool fused_form_holds(bool a80, uint32_t m, uint32_t k);  // what the kernel its
 bool fused_small_holds(uint32_t m, uint32_t k);  // the 20 KiB form: up to 4 rows (`_tm1`, and the MLP chain's first linear)
 bool mlp_chain_pays(uint32_t m, uint32_t hidden, uint32_t inter);        // ... and measured faster than the three launches
 bool mlp_chain_form_holds(uint32_t m, uint32_t hidden, uint32_t inter);  // the chain: 20 KiB at the hidden width, 20 or 80 KiB at the intermediate
+bool staged80_holds(uint32_t m, uint32_t k);  // up to 16 rows of K <= 5120: one 16-row tile in 80 KiB
 uint32_t fused_grid(uint32_t nblk);  // workgroups for nblk column blocks: one a CU, then equal shares of at most 8
 int resolve_fused(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *out);
 // The decode MLP (gate+up -> SiLU * up + requant -> down) as one persistent launch; spin 0 = the default.

@@ -39,6 +39,13 @@ struct iu8_decq_nohook {
   __device__ bool wait() const { return true; }
   __device__ void amax(float[4]) const {}
 };
+// CH 3: the rows arrive quantised (`X` is the A operand of up to 16 rows, int8 codes in fragment order, which
+// is the staged order at 16 rows a tile: a straight copy into LDS) with their scales in `hook.as`.
+struct iu8_decq_codes {
+  const float *as;
+  __device__ bool wait() const { return true; }
+  __device__ void amax(float[4]) const {}
+};
 static __device__ __forceinline__ iu8_v4u iu8_decq_ld_coherent(const iu8_v4u *p) {
   const unsigned long long lo = __hip_atomic_load((const unsigned long long *)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
   const unsigned long long hi = __hip_atomic_load((const unsigned long long *)p + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
@@ -79,6 +86,7 @@ __device__ __forceinline__ void iu8_decq_body(iu8_decq_lds<NT, KW, WPB, CH, AKB>
   // reciprocals are made once a row by 16 lanes, and a lane reads its row's scale for the epilogue.
   constexpr bool BIG = AKB > 20;
   static_assert(!BIG || CH != 1, "the chain's first linear stages at most 20 KiB");
+  constexpr bool CODES = CH == 3;
   auto &s_a = S.s_a;
   auto &s_red = S.s_red;
   auto &s_amax = S.s_amax;
@@ -108,9 +116,10 @@ __device__ __forceinline__ void iu8_decq_body(iu8_decq_lds<NT, KW, WPB, CH, AKB>
   // ---- the rows' bf16 pieces (8 elements = 16 bytes; piece p = row * K/8 + k/8), loaded first
   int mr_shift = 0;
   while ((1 << mr_shift) < M) ++mr_shift;
-  constexpr int X_PER = (ABYTES / 8 + NTHR - 1) / NTHR;
+  if constexpr (CODES) mr_shift = 4;
+  constexpr int X_PER = CODES ? (ABYTES / 16 + NTHR - 1) / NTHR : (ABYTES / 8 + NTHR - 1) / NTHR;
   iu8_v4u xreg[X_PER];
-  const int k8 = K >> 3, x_pieces = M * k8;
+  const int k8 = K >> 3, x_pieces = CODES ? K : M * k8;  // CODES: 16-byte pieces of the 16-row tile, K of them
   if constexpr (CH != 2) {
 #pragma unroll
     for (int p = 0; p < X_PER; ++p)
@@ -175,7 +184,20 @@ __device__ __forceinline__ void iu8_decq_body(iu8_decq_lds<NT, KW, WPB, CH, AKB>
   // all order-free maxima; sc = max(amax / 127, 1e-30); codes by the exact reciprocal path
   float qsc[4] = {1.f, 1.f, 1.f, 1.f};
   float my_sc = 1.f;  // BIG: the scale of this lane's row (ml)
-  if constexpr (BIG) {
+  if constexpr (CODES) {
+    static_assert(!CODES || BIG, "the codes form reads its row's scale like the 80 KiB form");
+    my_sc = hook.as[min(ml, M - 1)];
+#pragma unroll
+    for (int i = 0; i < D; ++i)
+      if (i < TT) issue(i);
+#pragma unroll
+    for (int p = 0; p < WS_PER; ++p)
+      if (p * NTHR + tid < WS_ALL) (&s_ws[0][0])[p * NTHR + tid] = wsreg[p];
+#pragma unroll
+    for (int p = 0; p < X_PER; ++p)
+      if (p * NTHR + tid < x_pieces) *(iu8_v4u *)&s_a[(p * NTHR + tid) << 4] = xreg[p];
+    __syncthreads();
+  } else if constexpr (BIG) {
     // piece p * NTHR + tid = (row, col) in pieces of 8: two divides here, then steps of NTHR pieces
     const int row_step = NTHR / k8, col_step = NTHR - row_step * k8;
     int row = tid / k8, col = tid - row * k8;

@@ -63,6 +63,23 @@ IU8_DECQA(macaq_iu8_decq_w8_tm1_a80, true, 1, 8, 16, 2, 80)
 #undef IU8_DECQX
 #undef IU8_DECQA
 
+// The GEMV of up to 16 quantised rows whose 16-row tile fits 80 KiB of LDS (K <= 5120), persistent like the
+// fused forms: a workgroup copies the tile into LDS once and streams its column blocks against it. The
+// streamed form (`_a0`) reads the tile from L2 once a 32-column block -- at 16 rows of K = 5120 as many bytes
+// through L2 as the weights bring from memory.
+#define IU8_DECS(name, W8, NT, KW, WPB, D)                                                                         \
+  extern "C" __global__ __launch_bounds__(WPB * 64) __attribute__((amdgpu_waves_per_eu(4, 4))) void name(          \
+      const unsigned char *__restrict__ a, const unsigned char *__restrict__ w, const float *__restrict__ as,     \
+      const float *__restrict__ ws, int *__restrict__ decode_partial, int *__restrict__ decode_counter,           \
+      unsigned short *__restrict__ c, int m, int n, int k) {                                                       \
+    __shared__ iu8_decq_lds<NT, KW, WPB, 3, 80> lds;                                                               \
+    iu8_decq_body<W8, NT, KW, WPB, D, 3, iu8_decq_codes, 80>(lds, (const unsigned short *)a, w, ws, nullptr, nullptr, c, m, n, k, \
+                                                             iu8_decq_codes{as});                                 \
+  }
+IU8_DECS(macaq_iu8_dec_w4_tm1_s80, false, 1, 8, 16, 4)
+IU8_DECS(macaq_iu8_dec_w8_tm1_s80, true, 1, 8, 16, 2)
+#undef IU8_DECS
+
 // One row (`_r1`, the GEMV of a single token): the same launch with the row's codes made just in time --
 // a wave converts only the K steps it multiplies, a chunk of 4 steps ahead of their use, inside the weight
 // stream (iu8_decq1.h). In front of the first MFMA stand the row's arrival, one meeting of the waves'

@@ -365,3 +365,29 @@ def test_row_producers_every_form_that_holds_the_row(ctx, M, K):
             torch.cuda.synchronize()
             np.testing.assert_array_equal(s.cpu().numpy().view(np.uint32), wsc.view(np.uint32), err_msg=name)
             np.testing.assert_array_equal(iu8.unpack_a(q.cpu().numpy(), M, K), wq, err_msg=name)
+
+
+@pytest.mark.parametrize("w8", [False, True])
+@pytest.mark.parametrize("M,N,K,grid", [(16, 5120, 5120, 0), (9, 96, 5120, 0), (13, 34816, 5120, 0), (11, 7184, 640, 0), (5, 4112, 128, 0),
+                                        (1, 256, 5120, 0), (16, 2048, 3072, 8), (12, 2064, 384, 9)])
+def test_sixteen_row_tile_staged_once_a_workgroup(ctx, M, N, K, grid, w8):
+    """The persistent GEMV that copies the rows' 16-row tile into LDS once a workgroup (`_s80`), by name: full and
+    ragged row counts, a last column block of 16 columns, one K step (seven idle k-waves), five column blocks a
+    workgroup at the benchmark layer's gate+up, and grids that give a workgroup 8 blocks or an uneven share.
+    The tile's rows past M hold whatever the producer's buffer held (0x55 here): they reach no output."""
+    tag = "w8" if w8 else "w4"
+    say(f"staged 16-row tile {tag} M={M} N={N} K={K} grid={grid}")
+    case = synth.dense_case(M, N, K, w8=w8, seed=M * 11 + N + K)
+    r = ref.linear(case["X"], case["W"], case["ws"], w8, threads=16)
+    run = DenseRun(ctx, case, kernel=f"macaq_iu8_dec_{tag}_tm1_s80", want_acc=False)
+    assert run.desc.block[0] == 1024 and run.desc.grid[0] * 8 >= -(-N // 32)
+    np.testing.assert_array_equal(run.C, r["C"])
+    if grid:
+        d = iu8.describe(f"macaq_iu8_dec_{tag}_tm1_s80", M, N, K)
+        d.grid[0] = grid
+        assert grid * 8 >= -(-N // 32)
+        c = torch.full((M, N), 0x7FC0, dtype=torch.int16, device="cuda")
+        ctx.launch(d, {"a": run.dev["q"].data_ptr(), "w": run.dev["wf"].data_ptr(), "as": run.dev["a_scale"].data_ptr(),
+                       "ws": run.dev["ws"].data_ptr(), "c": c.data_ptr()})
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(host_u16(c), r["C"])

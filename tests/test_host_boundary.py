@@ -81,8 +81,38 @@ def test_decode_band_routing(wk, tag):
 def test_activation_rows_are_staged_when_they_fit():
     assert iu8.resolve(iu8.W4, 1, 5120, 17408).kernel == b"macaq_iu8_dec_w4_tm1"        # 17 KiB
     assert iu8.resolve(iu8.W4, 4, 5120, 5120).kernel == b"macaq_iu8_dec_w4_tm1"         # 20 KiB
-    assert iu8.resolve(iu8.W4, 16, 5120, 5120).kernel == b"macaq_iu8_dec_w4_tm1_a0"     # past 20 KiB: streamed
+    assert iu8.resolve(iu8.W4, 8, 5120, 5120).kernel == b"macaq_iu8_dec_w4_tm1_a0"      # past 20 KiB: streamed
     assert iu8.resolve(iu8.W4, 8, 5120, 17408).kernel == b"macaq_iu8_dec_w4_tm1_a0"     # does not fit
+    assert iu8.resolve(iu8.W4, 16, 5120, 17408).kernel == b"macaq_iu8_dec_w4_tm1_a0"
+
+
+def test_sixteen_row_tile_staged_once_a_workgroup_where_it_measured_faster():
+    """`_s80`: the persistent GEMV that copies the 16-row tile (K <= 5120: 80 KiB) into LDS once a workgroup.
+    W4 at 9-16 rows everywhere it holds; up to 8 rows, and int8 weights, from 64 MiB of weights."""
+    for wk, m, n, k, s80 in ((iu8.W4, 16, 5120, 5120, True), (iu8.W4, 9, 96, 5120, True), (iu8.W4, 16, 16384, 4096, True),
+                             (iu8.W4, 8, 5120, 5120, False), (iu8.W4, 8, 34816, 5120, True), (iu8.W4, 5, 28672, 4096, False),
+                             (iu8.W4, 4, 34816, 5120, False), (iu8.W4, 16, 5120, 5248, False), (iu8.W4, 17, 34816, 5120, False),
+                             (iu8.W8, 16, 7168, 5120, False), (iu8.W8, 16, 14336, 5120, True), (iu8.W8, 5, 34816, 5120, True),
+                             (iu8.W8, 9, 24576, 2048, False)):
+        d = iu8.resolve(wk, m, n, k)
+        tag = "w8" if wk == iu8.W8 else "w4"
+        assert (d.kernel.decode() == f"macaq_iu8_dec_{tag}_tm1_s80") == s80, (tag, m, n, k, d.kernel)
+        if s80:
+            blocks = -(-n // 32)
+            assert d.block[0] == 1024 and d.ks == 1 and d.n_workspaces == 0
+            assert d.grid[0] == (blocks if blocks <= 256 else -(-blocks // min(8, -(-blocks // 256))))
+            assert bytes(d) == bytes(iu8.describe(f"macaq_iu8_dec_{tag}_tm1_s80", m, n, k))
+    for bad in (lambda: iu8.describe("macaq_iu8_dec_w4_tm1_s80", 17, 5120, 5120), lambda: iu8.describe("macaq_iu8_dec_w4_tm1_s80", 16, 5120, 5248),
+                lambda: iu8.describe("macaq_iu8_dec_w4_tm1_s80", 16, 5120, 5120, ks=2)):
+        with pytest.raises(iu8.IU8Error) as e:
+            bad()
+        assert e.value.code == iu8.E_RULE
+    # a pair's halves stay the streamed geometry, whatever the law gives each alone
+    a, b = iu8.resolve(iu8.W4, 16, 12288, 5120), iu8.resolve(iu8.W4, 16, 96, 5120)
+    assert a.kernel == b.kernel == b"macaq_iu8_dec_w4_tm1_s80"
+    d = iu8.pair(a, b)
+    a0, b0 = iu8.describe("macaq_iu8_dec_w4_tm1_a0", 16, 12288, 5120), iu8.describe("macaq_iu8_dec_w4_tm1_a0", 16, 96, 5120)
+    assert d.kernel == b"macaq_iu8f_pairb_w4_tm1_a0" and bytes(d) == bytes(iu8.pair(a0, b0))
 
 
 def test_pair_lays_two_decode_grids_end_to_end():
