@@ -379,7 +379,9 @@ static int chain_guard(const LoadedKernel &lk, const saber_iu8_desc *d) {
 
 static int launch_guard(const LoadedKernel &lk, const saber_iu8_desc *d) {
   if (strncmp(d->kernel, "macaq_iu8f_mlp_", 15) == 0) return chain_guard(lk, d);
-  if (strncmp(d->kernel, "macaq_iu8_decq_", 15) != 0) return 0;
+  const size_t klen = strlen(d->kernel);
+  const bool s80 = klen > 4 && !strcmp(d->kernel + klen - 4, "_s80");
+  if (strncmp(d->kernel, "macaq_iu8_decq_", 15) != 0 && !s80) return 0;
   int64_t m = 0, n = 0, k = 0;
   for (uint32_t i = 0; i < d->n_args; ++i) {
     if (d->args[i].kind != SABER_IU8_ARG_I32) continue;
@@ -387,8 +389,16 @@ static int launch_guard(const LoadedKernel &lk, const saber_iu8_desc *d) {
     if (!strcmp(d->args[i].name, "n")) n = d->args[i].ival;
     if (!strcmp(d->args[i].name, "k")) k = d->args[i].ival;
   }
+  if (s80) {  // the staged tile: 16 rows x K bytes of LDS, the fused forms' block walk
+    if (m <= 0 || n <= 0 || k <= 0 || k % 128 || !staged80_holds((uint32_t)m, (uint32_t)k))
+      return fail(SABER_IU8_E_RULE, fmt("%s: %lld rows of %lld do not fit one 16-row tile in 80 KiB", d->kernel, (long long)m, (long long)k));
+    if ((int64_t)d->grid[0] * 8 < (n + 31) / 32 || d->grid[1] != 1 || d->grid[2] != 1)
+      return fail(SABER_IU8_E_RULE, fmt("%s: grid %u x %u x %u cannot walk %lld column blocks (at most 8 a workgroup)", d->kernel,
+                                        d->grid[0], d->grid[1], d->grid[2], (long long)((n + 31) / 32)));
+    return 0;
+  }
   const bool a80 = strstr(d->kernel, "_a80") != nullptr;
-  const size_t len = strlen(d->kernel);
+  const size_t len = klen;
   if (len > 3 && !strcmp(d->kernel + len - 3, "_r1") && m != 1)
     return fail(SABER_IU8_E_RULE, fmt("%s: the one-row form, got %lld rows", d->kernel, (long long)m));
   if (m <= 0 || n <= 0 || k <= 0 || !fused_form_holds(a80, (uint32_t)m, (uint32_t)k))

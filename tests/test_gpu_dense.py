@@ -387,7 +387,21 @@ def test_sixteen_row_tile_staged_once_a_workgroup(ctx, M, N, K, grid, w8):
         d.grid[0] = grid
         assert grid * 8 >= -(-N // 32)
         c = torch.full((M, N), 0x7FC0, dtype=torch.int16, device="cuda")
-        ctx.launch(d, {"a": run.dev["q"].data_ptr(), "w": run.dev["wf"].data_ptr(), "as": run.dev["a_scale"].data_ptr(),
-                       "ws": run.dev["ws"].data_ptr(), "c": c.data_ptr()})
+        bufs = {"a": run.dev["q"].data_ptr(), "w": run.dev["wf"].data_ptr(), "as": run.dev["a_scale"].data_ptr(),
+                "ws": run.dev["ws"].data_ptr(), "c": c.data_ptr()}
+        ctx.launch(d, bufs)
         torch.cuda.synchronize()
         np.testing.assert_array_equal(host_u16(c), r["C"])
+        # descriptors edited past what the kernel holds are refused at launch: more than 8 blocks a workgroup, a K
+        # whose tile passes 80 KiB, more than 16 rows
+        for field, value in (("grid", max(1, (-(-N // 32) - 1) // 8)), ("k", 5248), ("m", 17)):
+            bad = iu8.describe(f"macaq_iu8_dec_{tag}_tm1_s80", M, N, K)
+            if field == "grid":
+                if value * 8 >= -(-N // 32):
+                    continue
+                bad.grid[0] = value
+            else:
+                bad.arg(field).ival = value
+            with pytest.raises(iu8.IU8Error) as e:
+                ctx.launch(bad, bufs)
+            assert e.value.code == iu8.E_RULE, field

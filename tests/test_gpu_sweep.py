@@ -119,6 +119,31 @@ def test_one_row_form_random_shapes(ctx):
         np.testing.assert_array_equal(s.cpu().numpy().view(np.uint32), r["a_scale"].view(np.uint32))
 
 
+def test_staged_tile_form_random_shapes(ctx):
+    """The persistent GEMV that stages the rows' 16-row tile once a workgroup, by name: 1 to 16 rows of any K it holds
+    (128 to 5,120), ragged N, any grid the host's rule lets through: c equals the oracle's."""
+    rng = np.random.default_rng(20249)
+    for n in range(60):
+        w8 = bool(rng.integers(0, 2))
+        tag = "w8" if w8 else "w4"
+        M, N, K = int(rng.integers(1, 17)), int(rng.integers(1, 300)) * 16, int(rng.integers(1, 41)) * 128
+        nblk = (N + 31) // 32
+        grid = int(rng.integers(max(1, (nblk + 7) // 8), min(nblk, 256) + 1))
+        say(f"sweep staged tile {n}: {tag} M={M} N={N} K={K} grid={grid}")
+        case = synth.dense_case(M, N, K, w8=w8, seed=int(rng.integers(0, 1 << 30)))
+        r = ref.linear(case["X"], case["W"], case["ws"], w8, threads=8)
+        x, wf, ws = dev_bf16_bits(case["X"]), dev_u8(iu8.repack_weights(case["W"], w8)), dev_f32(case["ws"])
+        q = torch.full((iu8.a_bytes(M, K),), 0x55, dtype=torch.uint8, device="cuda")
+        s = torch.zeros(M, dtype=torch.float32, device="cuda")
+        ctx.quant(x.data_ptr(), q.data_ptr(), s.data_ptr(), M, K)
+        d = iu8.describe(f"macaq_iu8_dec_{tag}_tm1_s80", M, N, K)
+        d.grid[0] = grid
+        c = torch.full((M, N), 0x7FC0, dtype=torch.int16, device="cuda")
+        ctx.launch(d, {"a": q.data_ptr(), "w": wf.data_ptr(), "as": s.data_ptr(), "ws": ws.data_ptr(), "c": c.data_ptr()})
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(host_u16(c), r["C"])
+
+
 def test_pair_chain_static_gemm_and_back_half_random_shapes(ctx):
     """The decode pair, the decode MLP chain (two launches in a row on one state block), the GEMM on the
     library's static workspace (twice in a row) and the routed layer's back half as two and as three launches."""
