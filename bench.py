@@ -806,20 +806,27 @@ def main():
             }
             row = {}
             for name, (fn, nbytes) in cases.items():
-                reps = 200 if PM <= 16 else 60
+                reps = 100 if PM <= 16 else 40
                 with torch.cuda.stream(stream):
-                    for _ in range(10):
+                    for _ in range(4):
                         fn()
-                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                    e0.record(stream)
+                stream.synchronize()
+                gp = torch.cuda.CUDAGraph()      # a graph: eager launches of a few microseconds are bound by the host's launch rate
+                with torch.cuda.graph(gp, stream=stream):
                     for _ in range(reps):
                         fn()
+                with torch.cuda.stream(stream):
+                    gp.replay()
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record(stream)
+                    gp.replay()
                     e1.record(stream)
                 torch.cuda.synchronize()
                 us = e0.elapsed_time(e1) * 1e3 / reps
+                del gp
                 row[name] = dict(us=round(us, 2), bytes=int(nbytes), gbps=round(nbytes / us / 1e3, 1), hbm_frac=round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4))
             prod["m%d" % PM] = row
-        prod["note"] = ("one launch a producer, back to back on one stream (inputs of the decode rows stay in the caches: those lines are launch latency, "
+        prod["note"] = ("one launch a producer, back to back in a replayed graph (inputs of the decode rows stay in the caches: those lines are launch latency, "
                         "not bandwidth); bytes = bf16 rows in + codes + scales (+ the residual row out); *_lut = the same op with the caller's table of its gate at hand")
         out["hadamard_producers"] = prod
     print(json.dumps(out), flush=True)

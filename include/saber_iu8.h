@@ -261,7 +261,11 @@ int saber_iu8_quant_rowmajor(saber_iu8_ctx *ctx, const void *x_bf16, void *q, fl
  *                       elements apart, head h's gate at h*2*head_dim + head_dim:
  *                       bf16(core * bf16(sigmoid(gate))); n at most 6,144
  *                       (hip/attn_glue_hadi8.hip:23-79, symbol attn_gate_quant_hadi8_t256_tiled1)
- * The square-root reciprocal is IEEE here where the reference calls the device's approximate rsqrtf. */
+ * The square-root reciprocal is IEEE here where the reference calls the device's approximate rsqrtf.
+ * Up to 256 rows of 4,096 elements and more launch a 1,024-thread form of every producer but add_rms (kernels
+ * `<stem>_hadi8_t1024`, `attn_gate_quant_hadi8[_lut]_t1024`; no counterpart among the reference's symbols): the
+ * same bytes -- only add_rms's sum of squares is a tree over the workgroup -- and 15-40 % less time while the
+ * rows are fewer than the compute units. */
 int saber_iu8_quant_had(saber_iu8_ctx *ctx, const void *x_bf16, void *q, float *scale, uint32_t m, uint32_t k,
                         const float *had_t, void *stream);
 int saber_iu8_silu_mul_quant_had(saber_iu8_ctx *ctx, const void *gu_bf16, void *q, float *scale, uint32_t m, uint32_t n,
@@ -281,7 +285,8 @@ int saber_iu8_silu_mul_quant_had_lut(saber_iu8_ctx *ctx, const void *gu_bf16, vo
  * pattern (u16 [65536], 128 KiB, the kernel's own expression: crates/saber-kernels/hip/attn_glue_hadi8.hip:23-79);
  * with it saber_iu8_attn_gate_quant_had_lut launches attn_gate_quant_hadi8_lut_t256 for rows of
  * SABER_IU8_SILU_LUT_MIN_WIDTH elements and more, from SABER_IU8_SIGMOID_LUT_MIN_ROWS rows on (below, the copy of
- * the table's middle costs more than the few rows' exps). The GDN norm's f32 gate was tabled too and did not
+ * the table's middle costs more than the few rows' exps) and, as attn_gate_quant_hadi8_lut_t1024, wherever the
+ * 1,024-thread form is launched (four times the threads share the copy). The GDN norm's f32 gate was tabled too and did not
  * gain: that kernel is not bound by its gate. */
 #define SABER_IU8_SIGMOID_LUT_MIN_ROWS 1024u
 int saber_iu8_sigmoid_table(saber_iu8_ctx *ctx, void *out_u16, void *stream);

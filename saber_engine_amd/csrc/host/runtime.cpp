@@ -588,13 +588,21 @@ int saber_iu8_gemm_acc(saber_iu8_ctx *ctx, int wkind, const void *a, const void 
 
 // One workgroup a row, T = 256 threads for rows of up to 10,240 elements (5 groups of 8 a thread),
 // 512 up to 20,480 (the reference's t256 / t512 pair, crates/saber-kernels/src/macaq_iu8.rs:864-875).
-static int had_desc(const char *op, const char *stem, uint32_t rows, uint32_t width, saber_iu8_desc *d) {
+// Few rows (fewer than CUs) of 4,096 elements and more go 16 waves a row (`<stem>_hadi8_t1024`, no counterpart among the
+// reference's symbols) where the workgroup's size does not enter the result -- every producer but add_rms, whose sum
+// of squares is a tree over the workgroup: the same bytes, and on this card at 16 rows (graph replay, us) the attention
+// gate 6.9 -> 4.8 (table form 7.1 -> 4.4), the GDN norm 7.2 -> 5.7, SiLU * up of 5,120 6.6 -> 4.7 and of 17,408 9.7 -> 9.0
+// (table form 7.6 -> 6.2), the plain transform of 5,120 3.6 -> 3.1 (of 17,408 the 512-thread form is as fast: kept);
+// from 512 rows on the narrow forms win.
+static bool had_t1024(uint32_t rows, uint32_t width) { return rows <= HAD_T1024_ROWS && width >= HAD_T1024_WIDTH; }
+static int had_desc(const char *op, const char *stem, uint32_t rows, uint32_t width, saber_iu8_desc *d, bool size_free = false) {
   if (rows == 0 || width == 0) return fail(SABER_IU8_E_RULE, fmt("%s: %u rows of %u has nothing to do", op, rows, width));
   if (width % 64 != 0 || width > 20480)
     return fail(SABER_IU8_E_RULE,
                 fmt("%s: row width %u must be a multiple of 64 (whole A fragments, whole 32-blocks), at most 20480", op, width));
-  const uint32_t t = width <= 10240 ? 256 : 512;
-  const std::string name = fmt("%s_hadi8_t%u_tiled1", stem, t);
+  const bool wide = size_free && had_t1024(rows, width);
+  const uint32_t t = wide ? 1024 : width <= 10240 ? 256 : 512;
+  const std::string name = wide ? fmt("%s_hadi8_t1024", stem) : fmt("%s_hadi8_t%u_tiled1", stem, t);
   const uint32_t grid[3] = {rows, 1, 1};
   if (int rc = saber_iu8_describe_raw(name.c_str(), "mxfp4_hadi8", grid, t, d)) return rc;
   snprintf(d->op, sizeof d->op, "%s", op);
@@ -611,7 +619,7 @@ static void set_f32(saber_iu8_desc *d, const char *name, float v) {
 int saber_iu8_quant_had(saber_iu8_ctx *ctx, const void *x, void *q, float *scale, uint32_t m, uint32_t k,
                         const float *had_t, void *stream) {
   saber_iu8_desc d;
-  if (int rc = had_desc("quant_had_i8", "quant", m, k, &d)) return rc;
+  if (int rc = had_desc("quant_had_i8", "quant", m, k, &d, k <= 10240)) return rc;
   set_i32(&d, "k", k);
   const saber_iu8_binding b[] = {{"x", (void *)x}, {"q", q}, {"scale", scale}, {"had_t", (void *)had_t}};
   return saber_iu8_launch(ctx, &d, b, 4, stream);
@@ -620,7 +628,7 @@ int saber_iu8_quant_had(saber_iu8_ctx *ctx, const void *x, void *q, float *scale
 int saber_iu8_silu_mul_quant_had(saber_iu8_ctx *ctx, const void *gu, void *q, float *scale, uint32_t m, uint32_t n,
                                  const float *had_t, void *stream) {
   saber_iu8_desc d;
-  if (int rc = had_desc("silu_mul_quant_had_i8", "silu_mul_quant", m, n, &d)) return rc;
+  if (int rc = had_desc("silu_mul_quant_had_i8", "silu_mul_quant", m, n, &d, true)) return rc;
   set_i32(&d, "n", n);
   const saber_iu8_binding b[] = {{"gu", (void *)gu}, {"q", q}, {"scale", scale}, {"had_t", (void *)had_t}};
   return saber_iu8_launch(ctx, &d, b, 4, stream);
@@ -630,7 +638,7 @@ int saber_iu8_silu_mul_quant_had_lut(saber_iu8_ctx *ctx, const void *gu, void *q
                                      const float *had_t, const uint16_t *silu_lut, void *stream) {
   if (!silu_lut || n < SABER_IU8_SILU_LUT_MIN_WIDTH) return saber_iu8_silu_mul_quant_had(ctx, gu, q, scale, m, n, had_t, stream);
   saber_iu8_desc d;
-  if (int rc = had_desc("silu_mul_quant_had_i8", "silu_mul_quant", m, n, &d)) return rc;  // the shape checks, grid and block
+  if (int rc = had_desc("silu_mul_quant_had_i8", "silu_mul_quant", m, n, &d, true)) return rc;  // the shape checks, grid and block
   const std::string name = fmt("silu_mul_quant_hadi8_lut_t%u", d.block[0]);
   const uint32_t grid[3] = {m, 1, 1};
   if (int rc = saber_iu8_describe_raw(name.c_str(), "mxfp4_hadi8", grid, d.block[0], &d)) return rc;
@@ -661,7 +669,8 @@ int saber_iu8_gdn_norm_quant_had(saber_iu8_ctx *ctx, const void *x, const void *
     return fail(SABER_IU8_E_RULE, fmt("gdn_norm_quant_had_i8: z stride %lld must cover the row width %u in whole 16-byte pieces", (long long)z_stride, n));
   saber_iu8_desc d;
   const uint32_t grid[3] = {m, 1, 1};
-  if (int rc = saber_iu8_describe_raw("gdn_norm_quant_hadi8_t256_tiled1", "mxfp4_hadi8", grid, 256, &d)) return rc;
+  const bool wide = had_t1024(m, n);  // a head's sum is its 16 lanes' whatever the workgroup's size
+  if (int rc = saber_iu8_describe_raw(wide ? "gdn_norm_quant_hadi8_t1024" : "gdn_norm_quant_hadi8_t256_tiled1", "mxfp4_hadi8", grid, wide ? 1024 : 256, &d)) return rc;
   snprintf(d.op, sizeof d.op, "gdn_norm_quant_had_i8");
   set_i32(&d, "n", n);
   set_i32(&d, "zs", z_stride);
@@ -683,7 +692,10 @@ static int attn_gate_launch(saber_iu8_ctx *ctx, const void *core, const void *ga
     return fail(SABER_IU8_E_RULE, fmt("attn_gate_quant_had_i8: gate stride %u must cover the [q | gate] block of %u in whole 16-byte pieces", gate_stride, 2 * n));
   saber_iu8_desc d;
   const uint32_t grid[3] = {m, 1, 1};
-  if (int rc = saber_iu8_describe_raw(lut ? "attn_gate_quant_hadi8_lut_t256" : "attn_gate_quant_hadi8_t256_tiled1", "attn_glue_hadi8", grid, 256, &d)) return rc;
+  const bool wide = had_t1024(m, n);
+  const char *name = wide ? (lut ? "attn_gate_quant_hadi8_lut_t1024" : "attn_gate_quant_hadi8_t1024")
+                          : (lut ? "attn_gate_quant_hadi8_lut_t256" : "attn_gate_quant_hadi8_t256_tiled1");
+  if (int rc = saber_iu8_describe_raw(name, "attn_glue_hadi8", grid, wide ? 1024 : 256, &d)) return rc;
   snprintf(d.op, sizeof d.op, "attn_gate_quant_had_i8");
   set_i32(&d, "n", n);
   set_i32(&d, "hd", head_dim);
@@ -699,7 +711,8 @@ int saber_iu8_attn_gate_quant_had(saber_iu8_ctx *ctx, const void *core, const vo
 int saber_iu8_attn_gate_quant_had_lut(saber_iu8_ctx *ctx, const void *core, const void *gate, void *q, float *scale, uint32_t m,
                                       uint32_t n, uint32_t head_dim, uint32_t gate_stride, const float *had_t,
                                       const uint16_t *sigmoid_lut, void *stream) {
-  const bool pays = n >= SABER_IU8_SILU_LUT_MIN_WIDTH && m >= SABER_IU8_SIGMOID_LUT_MIN_ROWS;
+  // (the 16-wave form spreads the copy of the table's middle over four times the threads: there it pays at any row count)
+  const bool pays = n >= SABER_IU8_SILU_LUT_MIN_WIDTH && (m >= SABER_IU8_SIGMOID_LUT_MIN_ROWS || had_t1024(m, n));
   return attn_gate_launch(ctx, core, gate, q, scale, m, n, head_dim, gate_stride, had_t, pays ? sigmoid_lut : nullptr, stream);
 }
 

@@ -15,14 +15,13 @@
 
 // `lut` (the table form, may be null): bf16(sigmoid) of every bf16 pattern as attn_gate_sigmoid_bf16_table wrote
 // it; the gate is then read from the table's middle in LDS (iu8_had.h) instead of computed.
-template <bool LUT>
+template <bool LUT, int T = 256>
 static __device__ __forceinline__ void attn_gate_body(const unsigned short *__restrict__ core,
                                                       const unsigned short *__restrict__ gate, unsigned char *__restrict__ q,
                                                       float *__restrict__ scale, int n, int hd, int gs,
                                                       const float *__restrict__ had_t,
                                                       const unsigned short *__restrict__ lut) {
 #pragma clang fp contract(off)
-  constexpr int T = 256;
   const int row = had_row(), tid = threadIdx.x, NV = n >> 3;
   core += (size_t)row * n, gate += (size_t)row * gs;
   __shared__ __attribute__((aligned(16))) unsigned short s_lut[LUT ? 2 * HAD_LUT_N : 8];
@@ -65,6 +64,18 @@ extern "C" __global__ __launch_bounds__(256) void attn_gate_quant_hadi8_lut_t256
     float *__restrict__ scale, int n, int hd, int gs, const float *__restrict__ had_t,
     const unsigned short *__restrict__ lut) {
   attn_gate_body<true>(core, gate, q, scale, n, hd, gs, had_t, lut);
+}
+// 16 waves a row, for few rows (no counterpart among the reference's symbols)
+extern "C" __global__ __launch_bounds__(1024) void attn_gate_quant_hadi8_t1024(
+    const unsigned short *__restrict__ core, const unsigned short *__restrict__ gate, unsigned char *__restrict__ q,
+    float *__restrict__ scale, int n, int hd, int gs, const float *__restrict__ had_t) {
+  attn_gate_body<false, 1024>(core, gate, q, scale, n, hd, gs, had_t, nullptr);
+}
+extern "C" __global__ __launch_bounds__(1024) void attn_gate_quant_hadi8_lut_t1024(
+    const unsigned short *__restrict__ core, const unsigned short *__restrict__ gate, unsigned char *__restrict__ q,
+    float *__restrict__ scale, int n, int hd, int gs, const float *__restrict__ had_t,
+    const unsigned short *__restrict__ lut) {
+  attn_gate_body<true, 1024>(core, gate, q, scale, n, hd, gs, had_t, lut);
 }
 // bf16(sigmoid) of all 65,536 bf16 inputs (bf16 bits [65536]): the table of attn_gate_quant_hadi8_lut_t256.
 // grid 256, block 256.

@@ -142,6 +142,7 @@ HAD_ARQ(add_rms_quant_hadi8_t512_tiled1, 512)
   }
 HAD_SMQ(silu_mul_quant_hadi8_t256_tiled1, 256)
 HAD_SMQ(silu_mul_quant_hadi8_t512_tiled1, 512)
+HAD_SMQ(silu_mul_quant_hadi8_t1024, 1024)  // 16 waves a row: few long rows (no counterpart among the reference's symbols)
 #undef HAD_SMQ
 
 // silu_mul_quant with the bf16 silu read from a table: `lut` holds bf16(silu(x)) of every bf16 bit pattern x as
@@ -203,6 +204,7 @@ static __device__ __forceinline__ void had_silu_lut_body(const unsigned short *_
   }
 HAD_SMQ_LUT(silu_mul_quant_hadi8_lut_t256, 256)
 HAD_SMQ_LUT(silu_mul_quant_hadi8_lut_t512, 512)
+HAD_SMQ_LUT(silu_mul_quant_hadi8_lut_t1024, 1024)
 #undef HAD_SMQ_LUT
 
 #define HAD_Q(name, T)                                                                                            \
@@ -213,6 +215,7 @@ HAD_SMQ_LUT(silu_mul_quant_hadi8_lut_t512, 512)
   }
 HAD_Q(quant_hadi8_t256_tiled1, 256)
 HAD_Q(quant_hadi8_t512_tiled1, 512)
+HAD_Q(quant_hadi8_t1024, 1024)
 #undef HAD_Q
 
 // One workgroup a row of N = heads * 128 elements; z rows `zs` elements apart; w the head's 128 weights.
@@ -257,4 +260,11 @@ extern "C" __global__ __launch_bounds__(256) void gdn_norm_quant_hadi8_t256_tile
     const unsigned short *__restrict__ w, unsigned char *__restrict__ q, float *__restrict__ scale, int N, float eps,
     const float *__restrict__ had_t) {
   had_gdn_norm_body<256>(x, z, zs, w, q, scale, N, eps, had_t);
+}
+// 16 waves a row: few rows (a head's sum is the 16 lanes' whatever the workgroup's size, so the bits are the same)
+extern "C" __global__ __launch_bounds__(1024) void gdn_norm_quant_hadi8_t1024(
+    const unsigned short *__restrict__ x, const unsigned short *__restrict__ z, long zs,
+    const unsigned short *__restrict__ w, unsigned char *__restrict__ q, float *__restrict__ scale, int N, float eps,
+    const float *__restrict__ had_t) {
+  had_gdn_norm_body<1024>(x, z, zs, w, q, scale, N, eps, had_t);
 }

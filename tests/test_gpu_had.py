@@ -214,6 +214,64 @@ def test_attn_gate_quant_had(ctx, M, H, hd, pad):
     np.testing.assert_array_equal(iu8.unpack_a(q.cpu().numpy(), M, n), wq)
 
 
+@pytest.mark.parametrize("M,H", [(5, 40), (16, 136), (3, 80), (9, 48), (300, 32)])
+def test_every_form_of_the_producers_by_name(ctx, M, H):
+    """Each producer in each of its workgroup sizes, launched by kernel name (the reference's `_t256` / `_t512`
+    symbols are what its host launches at any row count; the `_t1024` forms are what this library's law picks for
+    few long rows): the oracle's bytes from every one. add_rms is not here: its sum of squares is a tree over the
+    workgroup, so its size is part of its law (256 threads up to 10,240 elements, 512 above)."""
+    W = H * 128
+    say(f"had producers by name M={M} W={W}")
+    rng = np.random.default_rng(M * 7 + W)
+    t = (rng.choice([-1.0, 1.0], size=W) * rng.uniform(0.5, 2.0, size=W)).astype(np.float32)
+    td = dev_f32(t)
+    sizes = [T for T in (256, 512, 1024) if W <= 40 * T]
+
+    def check(name, plugin, T, bufs, want, scalars, eps=None):
+        q, s = outs(M, W)
+        d = iu8.describe_raw(name, (M, 1, 1), T, plugin=plugin, **scalars)
+        if eps is not None:
+            d.arg("eps").kind, d.arg("eps").fval = iu8.ARG_F32, eps
+        ctx.launch(d, dict(bufs, q=q.data_ptr(), scale=s.data_ptr(), had_t=td.data_ptr()))
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(s.cpu().numpy().view(np.uint32), want[1].view(np.uint32), err_msg=name)
+        np.testing.assert_array_equal(iu8.unpack_a(q.cpu().numpy(), M, W), want[0], err_msg=name)
+
+    X = synth.activations(rng, M, W)
+    xd = dev_bf16_bits(X)
+    want = ref.quant_had(X, t)
+    for T in sizes:
+        check(f"quant_hadi8_t{T}" + ("" if T == 1024 else "_tiled1"), "mxfp4_hadi8", T, dict(x=xd.data_ptr()), want, dict(k=W))
+    gu = synth.f32_to_bf16_bits((rng.standard_normal((M, 2 * W)) * 2).astype(np.float32))
+    gu[M // 2, :4] = [0x7F80, 0x7FC0, 0x0000, 0xC700]
+    gd = dev_bf16_bits(gu)
+    lut = torch.zeros(65536, dtype=torch.int16, device="cuda")
+    ctx.silu_table(lut.data_ptr())
+    want = ref.silu_mul_quant_had(gu, t)
+    for T in sizes:
+        check(f"silu_mul_quant_hadi8_t{T}" + ("" if T == 1024 else "_tiled1"), "mxfp4_hadi8", T, dict(gu=gd.data_ptr()), want, dict(n=W))
+        check(f"silu_mul_quant_hadi8_lut_t{T}", "mxfp4_hadi8", T, dict(gu=gd.data_ptr(), lut=lut.data_ptr()), want, dict(n=W))
+    if W <= 10240:
+        z = synth.f32_to_bf16_bits((rng.standard_normal((M, W + 8)) * 3).astype(np.float32))
+        w = synth.f32_to_bf16_bits((1 + rng.standard_normal(128) * 0.1).astype(np.float32))
+        zd, wd = dev_bf16_bits(z), dev_bf16_bits(w)
+        want = ref.gdn_norm_quant_had(X, z[:, :W], w, t, 1e-6, silu_tab=device_silu_f32_table(ctx))
+        for name, T in (("gdn_norm_quant_hadi8_t256_tiled1", 256), ("gdn_norm_quant_hadi8_t1024", 1024)):
+            check(name, "mxfp4_hadi8", T, dict(x=xd.data_ptr(), z=zd.data_ptr(), w=wd.data_ptr()), want, dict(n=W, zs=W + 8), eps=1e-6)
+    if W <= 6144:
+        block = synth.f32_to_bf16_bits((rng.standard_normal((M, 2 * W + 16)) * 3).astype(np.float32))
+        bd = dev_bf16_bits(block)
+        sig = torch.zeros(65536, dtype=torch.int16, device="cuda")
+        ctx.sigmoid_table(sig.data_ptr())
+        want = ref.attn_gate_quant_had(X, block, t, 128)
+        for name, T, tab in (("attn_gate_quant_hadi8_t256_tiled1", 256, False), ("attn_gate_quant_hadi8_t1024", 1024, False),
+                             ("attn_gate_quant_hadi8_lut_t256", 256, True), ("attn_gate_quant_hadi8_lut_t1024", 1024, True)):
+            bufs = dict(core=xd.data_ptr(), gate=bd.data_ptr())
+            if tab:
+                bufs["lut"] = sig.data_ptr()
+            check(name, "attn_glue_hadi8", T, bufs, want, dict(n=W, hd=128, gs=2 * W + 16))
+
+
 def test_had_producers_feed_the_gemm(ctx):
     """The transformed codes are ordinary A operands: producer + GEMM equals the oracle's GEMM on them."""
     say("quant_had -> gemm")
