@@ -175,6 +175,7 @@ static int describe_pf(const PfVariant &v, uint32_t m, uint32_t n, uint32_t k, u
   return 0;
 }
 
+static uint64_t staged_bytes(uint32_t m, uint32_t k);
 // The streaming decode cell of M rows: tm 16-row tiles; one tile's live rows staged in LDS when they fit the 20 KiB
 // form, else streamed from L2 beside the weights.
 static std::string dec_stream_name(const char *tag, uint32_t m, uint32_t k) {
@@ -191,14 +192,14 @@ static std::string dec_stream_name(const char *tag, uint32_t m, uint32_t k) {
 // The persistent GEMV of up to 16 quantised rows whose 16-row tile is staged once a workgroup in 80 KiB of LDS
 // (`macaq_iu8_dec_{w4,w8}_tm1_s80`): the fused forms' geometry (16 waves, 32 columns a block, at most 8 blocks a
 // workgroup) on the decode kernarg list.
-bool staged80_holds(uint32_t m, uint32_t k) { return m >= 1 && m <= 16 && (uint64_t)k * 16 <= 80 * 1024; }
+bool staged80_holds(uint32_t m, uint32_t k) { return m >= 1 && m <= 16 && staged_bytes(m, k) <= 80 * 1024; }
 static int describe_s80(bool w8, uint32_t m, uint32_t n, uint32_t k, uint32_t ks, saber_iu8_desc *d) {
   const char *op = w8 ? "gemm_i8a8" : "gemm_i4a8";
   const std::string name = fmt("macaq_iu8_dec_%s_tm1_s80", w8 ? "w8" : "w4");
   if (int rc = check_shape(op, m, n, k)) return rc;
   if (ks != 1) return fail(SABER_IU8_E_RULE, name + ": the staged form does not split K");
   if (!staged80_holds(m, k))
-    return fail(SABER_IU8_E_RULE, fmt("%s: %u rows of %u do not fit one 16-row tile in 80 KiB (K <= 5120)", name.c_str(), m, k));
+    return fail(SABER_IU8_E_RULE, fmt("%s: %u rows (rounded up to a power of two) of %u do not fit 80 KiB", name.c_str(), m, k));
   memset(d, 0, sizeof *d);
   copy_name(d->op, sizeof d->op, op);
   copy_name(d->plugin, sizeof d->plugin, "macaq_iu8");
@@ -354,9 +355,14 @@ int resolve(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *out) 
     // QKV / O 6.1 / 5.9 -> 6.05 / 5.8); up to 8 rows, and int8 weights at any row count, from 64 MiB of weights
     // (W4 5-8 rows: gate+up 16.6-17.9 -> 16.4-17.2, 28672 x 4096 even, 14336 x 5120 8.5 -> 9.0 the other way;
     // W8: gate+up 31.3 -> 28.4, 28672 x 4096 21.0 -> 19.9, 14336 x 5120 14.3 -> 13.6, QKV 8.1 -> 8.4 the other way).
-    if (m > 4 && staged80_holds(m, k) &&
+    if (m > 4 && k <= 5120 && staged80_holds(m, k) &&
         ((m > 8 && wkind == SABER_IU8_W4) || (uint64_t)n * k / (wkind == SABER_IU8_W8 ? 1 : 2) >= S80_MIN_BYTES))
       return describe_s80(wkind == SABER_IU8_W8, m, n, k, 1, out);
+    // ... and 2 to 4 rows of a long K, whose live rows' codes fit the same 80 KiB (the copy takes their pieces of the
+    // tile): 5120 x 17408 at 2 / 3 / 4 rows 11.0 -> 10.5 / 10.7 / 10.7 us; at K = 6144 and 8704 (5.7 -> 5.8, 6.9 -> 6.9)
+    // and on 16384 x 8192 (12.4 -> 12.8) the streamed form stays
+    if (m >= 2 && m <= 4 && k >= 16384 && wkind == SABER_IU8_W4 && staged80_holds(m, k))
+      return describe_s80(false, m, n, k, 1, out);
     const std::string name = dec_stream_name(tag, m, k);
     const DecVariant *v = dec_variant(name);
     if (!v) return fail(SABER_IU8_E_RULE, name + ": no such variant");

@@ -40,7 +40,8 @@ struct iu8_decq_nohook {
   __device__ void amax(float[4]) const {}
 };
 // CH 3: the rows arrive quantised (`X` is the A operand of up to 16 rows, int8 codes in fragment order, which
-// is the staged order at 16 rows a tile: a straight copy into LDS) with their scales in `hook.as`.
+// is the staged order at 16 rows a tile: a straight copy into LDS; with fewer live rows, rounded up to a power of
+// two, the copy takes those rows' pieces of every 256-byte run) with their scales in `hook.as`.
 struct iu8_decq_codes {
   const float *as;
   __device__ bool wait() const { return true; }
@@ -116,11 +117,18 @@ __device__ __forceinline__ void iu8_decq_body(iu8_decq_lds<NT, KW, WPB, CH, AKB>
   // ---- the rows' bf16 pieces (8 elements = 16 bytes; piece p = row * K/8 + k/8), loaded first
   int mr_shift = 0;
   while ((1 << mr_shift) < M) ++mr_shift;
-  if constexpr (CODES) mr_shift = 4;
   constexpr int X_PER = CODES ? (ABYTES / 16 + NTHR - 1) / NTHR : (ABYTES / 8 + NTHR - 1) / NTHR;
   iu8_v4u xreg[X_PER];
-  const int k8 = K >> 3, x_pieces = CODES ? K : M * k8;  // CODES: 16-byte pieces of the 16-row tile, K of them
-  if constexpr (CH != 2) {
+  // CODES: the live rows' 16-byte pieces of the 16-row tile, (K / 16) << mr_shift of them: staged piece i is the tile's
+  // piece (i >> mr_shift) * 16 + (i & (MR - 1)) -- the tile itself at 9 to 16 rows
+  const int k8 = K >> 3, x_pieces = CODES ? (K >> 4) << mr_shift : M * k8;
+  if constexpr (CODES) {
+#pragma unroll
+    for (int p = 0; p < X_PER; ++p) {
+      const int i = p * NTHR + tid;
+      if (i < x_pieces) xreg[p] = *((const iu8_v4u *)X + ((i >> mr_shift) << 4) + (i & ((1 << mr_shift) - 1)));
+    }
+  } else if constexpr (CH != 2) {
 #pragma unroll
     for (int p = 0; p < X_PER; ++p)
       if (p * NTHR + tid < x_pieces) xreg[p] = *((const iu8_v4u *)X + p * NTHR + tid);

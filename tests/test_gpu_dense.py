@@ -369,11 +369,13 @@ def test_row_producers_every_form_that_holds_the_row(ctx, M, K):
 
 @pytest.mark.parametrize("w8", [False, True])
 @pytest.mark.parametrize("M,N,K,grid", [(16, 5120, 5120, 0), (9, 96, 5120, 0), (13, 34816, 5120, 0), (11, 7184, 640, 0), (5, 4112, 128, 0),
-                                        (1, 256, 5120, 0), (16, 2048, 3072, 8), (12, 2064, 384, 9)])
+                                        (1, 256, 5120, 0), (16, 2048, 3072, 8), (12, 2064, 384, 9),
+                                        (4, 5120, 17408, 0), (2, 272, 32768, 0), (8, 1040, 10240, 5), (3, 2064, 20480, 0), (1, 96, 17408, 0)])
 def test_sixteen_row_tile_staged_once_a_workgroup(ctx, M, N, K, grid, w8):
     """The persistent GEMV that copies the rows' 16-row tile into LDS once a workgroup (`_s80`), by name: full and
     ragged row counts, a last column block of 16 columns, one K step (seven idle k-waves), five column blocks a
-    workgroup at the benchmark layer's gate+up, and grids that give a workgroup 8 blocks or an uneven share.
+    workgroup at the benchmark layer's gate+up, grids that give a workgroup 8 blocks or an uneven share, and fewer
+    live rows of a longer K (the copy then takes the live rows' pieces of the tile: 1, 2, 4 or 8 of every 16).
     The tile's rows past M hold whatever the producer's buffer held (0x55 here): they reach no output."""
     tag = "w8" if w8 else "w4"
     say(f"staged 16-row tile {tag} M={M} N={N} K={K} grid={grid}")
@@ -394,7 +396,8 @@ def test_sixteen_row_tile_staged_once_a_workgroup(ctx, M, N, K, grid, w8):
         np.testing.assert_array_equal(host_u16(c), r["C"])
         # descriptors edited past what the kernel holds are refused at launch: more than 8 blocks a workgroup, a K
         # whose tile passes 80 KiB, more than 16 rows
-        for field, value in (("grid", max(1, (-(-N // 32) - 1) // 8)), ("k", 5248), ("m", 17)):
+        mr = 1 << (M - 1).bit_length()
+        for field, value in (("grid", max(1, (-(-N // 32) - 1) // 8)), ("k", 80 * 1024 // mr + 128), ("m", 17)):
             bad = iu8.describe(f"macaq_iu8_dec_{tag}_tm1_s80", M, N, K)
             if field == "grid":
                 if value * 8 >= -(-N // 32):

@@ -121,12 +121,15 @@ def test_one_row_form_random_shapes(ctx):
 
 def test_staged_tile_form_random_shapes(ctx):
     """The persistent GEMV that stages the rows' 16-row tile once a workgroup, by name: 1 to 16 rows of any K it holds
-    (128 to 5,120), ragged N, any grid the host's rule lets through: c equals the oracle's."""
+    (128 to 5,120 at 9 to 16 rows, up to 32,768 at one or two), ragged N, any grid the host's rule lets through: c equals the oracle's."""
     rng = np.random.default_rng(20249)
     for n in range(60):
         w8 = bool(rng.integers(0, 2))
         tag = "w8" if w8 else "w4"
-        M, N, K = int(rng.integers(1, 17)), int(rng.integers(1, 300)) * 16, int(rng.integers(1, 41)) * 128
+        M, N = int(rng.integers(1, 17)), int(rng.integers(1, 300)) * 16
+        K = int(rng.integers(1, min(32768, 80 * 1024 // (1 << (M - 1).bit_length())) // 128 + 1)) * 128      # the live rows' codes fit 80 KiB (and the producer's 32,768)
+        while M * N * K > 2e9:
+            N = max(16, (N // 2) // 16 * 16)
         nblk = (N + 31) // 32
         grid = int(rng.integers(max(1, (nblk + 7) // 8), min(nblk, 256) + 1))
         say(f"sweep staged tile {n}: {tag} M={M} N={N} K={K} grid={grid}")

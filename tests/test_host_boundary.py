@@ -84,6 +84,7 @@ def test_activation_rows_are_staged_when_they_fit():
     assert iu8.resolve(iu8.W4, 8, 5120, 5120).kernel == b"macaq_iu8_dec_w4_tm1_a0"      # past 20 KiB: streamed
     assert iu8.resolve(iu8.W4, 8, 5120, 17408).kernel == b"macaq_iu8_dec_w4_tm1_a0"     # does not fit
     assert iu8.resolve(iu8.W4, 16, 5120, 17408).kernel == b"macaq_iu8_dec_w4_tm1_a0"
+    assert iu8.resolve(iu8.W4, 3, 5120, 8704).kernel == b"macaq_iu8_dec_w4_tm1_a0"
 
 
 def test_sixteen_row_tile_staged_once_a_workgroup_where_it_measured_faster():
@@ -92,6 +93,8 @@ def test_sixteen_row_tile_staged_once_a_workgroup_where_it_measured_faster():
     for wk, m, n, k, s80 in ((iu8.W4, 16, 5120, 5120, True), (iu8.W4, 9, 96, 5120, True), (iu8.W4, 16, 16384, 4096, True),
                              (iu8.W4, 8, 5120, 5120, False), (iu8.W4, 8, 34816, 5120, True), (iu8.W4, 5, 28672, 4096, False),
                              (iu8.W4, 4, 34816, 5120, False), (iu8.W4, 16, 5120, 5248, False), (iu8.W4, 17, 34816, 5120, False),
+                             (iu8.W4, 4, 5120, 17408, True), (iu8.W4, 2, 5120, 17408, True), (iu8.W4, 1, 5120, 17408, False),
+                             (iu8.W4, 4, 5120, 20608, False), (iu8.W4, 2, 256, 32768, True), (iu8.W8, 4, 5120, 17408, False),
                              (iu8.W8, 16, 7168, 5120, False), (iu8.W8, 16, 14336, 5120, True), (iu8.W8, 5, 34816, 5120, True),
                              (iu8.W8, 9, 24576, 2048, False)):
         d = iu8.resolve(wk, m, n, k)
@@ -102,7 +105,9 @@ def test_sixteen_row_tile_staged_once_a_workgroup_where_it_measured_faster():
             assert d.block[0] == 1024 and d.ks == 1 and d.n_workspaces == 0
             assert d.grid[0] == (blocks if blocks <= 256 else -(-blocks // min(8, -(-blocks // 256))))
             assert bytes(d) == bytes(iu8.describe(f"macaq_iu8_dec_{tag}_tm1_s80", m, n, k))
+    assert iu8.describe("macaq_iu8_dec_w4_tm1_s80", 8, 5120, 10240).grid[0] == 160       # by name: whatever fits 80 KiB
     for bad in (lambda: iu8.describe("macaq_iu8_dec_w4_tm1_s80", 17, 5120, 5120), lambda: iu8.describe("macaq_iu8_dec_w4_tm1_s80", 16, 5120, 5248),
+                lambda: iu8.describe("macaq_iu8_dec_w4_tm1_s80", 5, 5120, 10368), lambda: iu8.describe("macaq_iu8_dec_w4_tm1_s80", 3, 5120, 20608),
                 lambda: iu8.describe("macaq_iu8_dec_w4_tm1_s80", 16, 5120, 5120, ks=2)):
         with pytest.raises(iu8.IU8Error) as e:
             bad()
