@@ -321,7 +321,7 @@ int saber_iu8_gemm_pair(saber_iu8_ctx *ctx, const void *a, const float *a_scale,
 
 /* The whole decode linear in one launch where that is the faster form (saber_iu8_fused_holds: up to
  * 4 rows whose codes, rows rounded up to a power of two, fit 20 KiB of LDS -- kernel `_tm1`, or `_r1` for
- * one row of K >= 8192 -- and 2 rows, or 3 rows of K >= 16384, whose codes fit 80 KiB -- kernel `_tm1_a80`,
+ * one row of K >= 8192 -- and 2 rows of K >= 16384 whose codes fit 80 KiB -- kernel `_tm1_a80`,
  * which itself holds up to 16 rows and is reachable by name through saber_iu8_describe_raw; the other
  * row counts measured slower than the two launches): per-token quantisation fused into the
  * GEMV's activation staging. x bf16 [m,k]; q (A edge) and scale f32 [m] are optional outputs (NULL:

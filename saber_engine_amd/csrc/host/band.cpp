@@ -135,12 +135,12 @@ std::string band_toml() {
   put(o, "r1_k_min", FUSED_R1_MIN_K);
   put(o, "r1_k_max", 20 * 1024);
   o += "# macaq_iu8_decq_{w4,w8}_tm1_a80: the same launch with 80 KiB of staged codes; the kernel holds up to 16\n";
-  o += "# rows, the law launches it for 2 rows, and for 3 of K >= 16384 (every workgroup repeats the quantisation:\n";
-  o += "# more rows lose to producer + GEMV)\n";
+  o += "# rows, the law launches it for 2 rows of K >= 16384 (every workgroup repeats the quantisation: more rows,\n";
+  o += "# and shorter ones, lose to producer + GEMV)\n";
   put(o, "a80_staged_code_bytes", 80 * 1024);
   put(o, "a80_rows_max", 16);
-  put(o, "a80_rows_max_by_law", 3);
-  put(o, "a80_three_rows_k_min", 16384);
+  put(o, "a80_rows_by_law", 2);
+  put(o, "a80_k_min_by_law", FUSED_A80_MIN_K);
   put(o, "threads", 1024);
   put(o, "column_block", 32);
   o += "# workgroups for b = ceil(n / 32) column blocks: b while b <= cu_count, else equal shares\n";

@@ -508,13 +508,13 @@ bool mlp_chain_pays(uint32_t m, uint32_t hidden, uint32_t inter) {
   if (inter > 20 * 1024) return false;  // not measured past the one-row form's 20 KiB of codes
   return mlp_chain_form_holds(m, hidden, inter) && ((m == 1 && inter >= MLP_CHAIN_PAYS_INTER_1) || (m == 2 && inter >= MLP_CHAIN_PAYS_INTER_2));
 }
-// The law: the 20 KiB form wherever it holds (1-4 rows: 5.7 / 5.3 / 16.7 us against 8.0 / 7.4 / 19.8 as two launches
-// at one row of the 27B layer's K = 5120 shapes, 6.9 / 6.7 / 17.3 against 8.3 / 7.7 / 19.5 at four); the 80 KiB form at
-// two rows (K = 17408: 13.9 against 15.2 us, 12288: 11.4 / 11.8) and at three rows of K >= 16384 (14.8 / 15.2); elsewhere
-// it loses to producer + the streamed GEMV (four rows: 16.0 / 15.2 at K = 17408, 10.5 / 9.5 at 8192, 9.2 / 8.5 at 6144;
-// three rows: 10.0 / 9.5 at 8192, 12.0 / 11.9 at 12288).
+// The law: the 20 KiB form wherever it holds (1-4 rows: 5.7 / 5.3 / 16.7 us against 7.8 / 7.2 / 19.7 as two launches
+// at one row of the 27B layer's K = 5120 shapes, 6.9 / 6.7 / 17.2 against 8.0 / 7.5 / 19.2 at four); the 80 KiB form at
+// two rows of K >= 16384 (K = 17408: 13.85 against 13.98 us, and a launch fewer); elsewhere it loses to the 16-wave
+// producer + the streamed or staged GEMV (two rows of K = 12288: 11.4 / 11.2; three rows of K = 17408: 14.8 / 14.1, of
+// 8192: 10.0 / 9.5; four rows: 16.0 / 14.8 at K = 17408, 10.5 / 9.5 at 8192, 9.2 / 8.5 at 6144).
 bool fused_holds(uint32_t m, uint32_t k) {
-  return fused_small_holds(m, k) || ((m == 2 || (m == 3 && k >= 16384)) && fused_form_holds(true, m, k));
+  return fused_small_holds(m, k) || (m == 2 && k >= FUSED_A80_MIN_K && fused_form_holds(true, m, k));
 }
 
 uint32_t fused_grid(uint32_t nblk) {
@@ -528,7 +528,7 @@ int resolve_fused(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc 
   const char *op = wkind == SABER_IU8_W8 ? "linear_i8a8_fused" : "linear_i4a8_fused";
   if (int rc = check_shape(op, m, n, k)) return rc;
   if (!fused_holds(m, k))
-    return fail(SABER_IU8_E_RULE, fmt("%s: %u rows of %u are not a fused launch (up to 4 rows in 20 KiB of codes; 2 rows, or 3 of K >= 16384, in 80 KiB)", op, m, k));
+    return fail(SABER_IU8_E_RULE, fmt("%s: %u rows of %u are not a fused launch (up to 4 rows in 20 KiB of codes; 2 rows of K >= 16384 in 80 KiB)", op, m, k));
   // one long row: the form that makes the row's codes just in time inside the weight stream (`_r1`). Measured on
   // this card against the several-row form at one row (cold weights, graph replay, N = 5120): K = 8,192 6.47
   // against 6.91 us, 12,288 7.82 against 8.38, 17,408 9.88 against 10.7-11.4, 20,480 10.97 against 11.83; at

@@ -32,6 +32,7 @@ uint32_t pf_split(bool w8, uint32_t m, uint32_t n, uint32_t k, const PfVariant *
 constexpr uint32_t DECODE_MAX_M = 64;  // the decode band's last row count (macaq_iu8.rs:31)
 constexpr uint32_t KS_MAX = 8;         // the largest grid-level split (macaq_iu8.rs:44)
 constexpr uint32_t CU_COUNT = 256;     // MI355X compute units
+constexpr uint32_t FUSED_A80_MIN_K = 16384;  // two rows at least this long take the 80 KiB fused form
 constexpr uint32_t FUSED_R1_MIN_K = 8192;   // rows at least this long take the one-row fused decode form
 // the activation producers' 1024-thread forms: rows wider than one group a thread of the 256-thread form, up
 // to `ROWS` of them (the quantiser / the activation), or any number of rows at least `WIDE` wide for the activation
@@ -54,7 +55,7 @@ int pair(const saber_iu8_desc &first, const saber_iu8_desc &second, saber_iu8_de
 const DecVariant *pair_variant(const std::string &name);
 int resolve_quant(uint32_t m, uint32_t k, saber_iu8_desc *out);
 // The fused quant + GEMV of a decode linear; refuses (by name) shapes it does not hold.
-bool fused_holds(uint32_t m, uint32_t k);        // the law: a fused launch is what runs (the 20 KiB form where it holds; the 80 KiB form at 2 rows, and at 3 of K >= 16384)
+bool fused_holds(uint32_t m, uint32_t k);        // the law: a fused launch is what runs (the 20 KiB form where it holds; the 80 KiB form at 2 rows of K >= 16384)
 bool fused_form_holds(bool a80, uint32_t m, uint32_t k);  // what the kernel itself holds: `_tm1` 4 rows / 20 KiB, `_tm1_a80` 16 rows / 80 KiB
 bool fused_small_holds(uint32_t m, uint32_t k);  // the 20 KiB form: up to 4 rows (`_tm1`, and the MLP chain's first linear)
 bool mlp_chain_pays(uint32_t m, uint32_t hidden, uint32_t inter);        // ... and measured faster than the three launches

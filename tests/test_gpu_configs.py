@@ -52,7 +52,7 @@ def test_config1_decode_layer_set_as_the_fused_launches_the_benchmark_times(ctx,
         case = synth.dense_case(M, n, k, seed=M)
         r = ref.linear(case["X"], case["W"], case["ws"], False, threads=16)
         if not iu8.fused_holds(M, k):
-            assert (M, k) == (4, 17408)
+            assert (M, k) in ((4, 17408), (3, 17408))
             assert_dense_matches(DenseRun(ctx, case, want_acc=False), r, False)
             continue
         x, wf, ws = dev_bf16_bits(case["X"]), dev_u8(iu8.repack_w4(case["W"])), dev_f32(case["ws"])

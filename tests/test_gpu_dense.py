@@ -91,7 +91,7 @@ def test_fused_linear_walks_column_blocks(ctx, M, N, K, grid):
         assert e.value.code == iu8.E_RULE
 
 
-@pytest.mark.parametrize("M,N,K,grid", [(2, 5120, 17408, None),    # what the law launches it for: down at 2 to 4 rows
+@pytest.mark.parametrize("M,N,K,grid", [(2, 5120, 17408, None),    # what the law launches it for: down at 2 rows
                                           (3, 352, 17408, None),
                                           (16, 480, 5120, None),     # the most rows; K a multiple of 512: a wave's pieces lie in one row
                                           (16, 7168, 5120, None),
@@ -101,7 +101,7 @@ def test_fused_linear_walks_column_blocks(ctx, M, N, K, grid):
                                           (1, 64, 128, None)])       # one step
 def test_fused_decode_linear_80_kib_form(ctx, M, N, K, grid):
     """macaq_iu8_decq_{w4,w8}_tm1_a80: up to 16 rows staged in 80 KiB, the bytes of producer + GEMV.
-    The law launches it for two rows, and for three of a long K; the other shapes reach it by name."""
+    The law launches it for two rows of a long K; the other shapes reach it by name."""
     for w8 in (False, True):
         say(f"fused decode linear, 80 KiB form: M={M} N={N} K={K} grid={grid} w8={w8}")
         case = synth.dense_case(M, N, K, w8=w8, seed=31 + M)
@@ -252,8 +252,9 @@ def test_rows_with_nan_and_infinity_through_the_gemm_epilogue(ctx, M, N, K, w8):
 def test_fused_form_refuses_what_it_does_not_hold(ctx):
     assert not iu8.fused_holds(5, 1024) and not iu8.fused_holds(4, 20608) and not iu8.fused_holds(2, 41088)
     assert iu8.fused_holds(1, 17408) and iu8.fused_holds(4, 5120) and iu8.fused_holds(2, 10240)
-    assert iu8.fused_holds(2, 17408) and iu8.fused_holds(3, 17408) and not iu8.fused_small_holds(2, 17408)   # the 80 KiB form: two rows, three of a long K
+    assert iu8.fused_holds(2, 17408) and iu8.fused_holds(2, 16384) and not iu8.fused_small_holds(2, 17408)   # the 80 KiB form: two rows of a long K
     assert not iu8.fused_holds(4, 17408) and not iu8.fused_holds(4, 5248) and not iu8.fused_holds(3, 8192)   # slower than producer + GEMV: two launches
+    assert not iu8.fused_holds(3, 17408) and not iu8.fused_holds(2, 12288)
     with pytest.raises(iu8.IU8Error) as e:
         iu8.resolve_fused(iu8.W4, 5, 256, 1024)
     assert e.value.code == iu8.E_RULE
