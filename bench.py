@@ -538,6 +538,48 @@ def main():
             tc = graph_us(chain)
             res["mlp_chain"] = dict(kernel=iu8.resolve_mlp_chain(DM, hid, inter).kernel.decode(), us_chain=round(tc, 2), us_three_launches=round(t3, 2),
                                     chain_pays_by_law=iu8.mlp_chain_pays(DM, hid, inter), same_bytes=same, state_status=int(state[iu8.MLP_CHAIN_STATUS_OFFSET // 4].item()))
+        elif iu8.gate_up_act_holds(DM, hid, inter):
+            # the step's MLP at 5-16 rows: producer -> gate+up -> SiLU*up + requant -> down, against the same with the
+            # activation in the gate+up linear's epilogue (producer -> gate+up with activation -> producer on p -> down)
+            p_rows = torch.zeros((DM, inter), dtype=torch.int16, device=dev)
+            q_dn = torch.zeros(iu8.a_bytes(DM, inter), dtype=torch.uint8, device=dev)
+            s_dn = torch.zeros(DM, dtype=torch.float32, device=dev)
+            d_q, d_gu, d_silu = iu8.resolve_quant(DM, hid), iu8.resolve(iu8.W4, DM, n_gu, hid), iu8.resolve_silu_mul_quant(DM, inter)
+            d_qp, d_dn, d_act = iu8.resolve_quant(DM, inter), iu8.resolve(iu8.W4, DM, hid, inter), iu8.resolve_gate_up_act(DM, hid, inter)
+            d_act.arg("gu").kind = iu8.ARG_NULL_BUFFER
+
+            def down(i):
+                b = dict(a=q_dn.data_ptr(), w=dev_w["down"][i % LAYERS].data_ptr(), ws=dev_ws["down"].data_ptr(), c=cs["down"].data_ptr())
+                b["as"] = s_dn.data_ptr()
+                ctx.launch(d_dn, b, sh)
+
+            def four(i):
+                ctx.launch(d_q, dict(x=xs["gate_up"].data_ptr(), q=qs["gate_up"].data_ptr(), scale=ss["gate_up"].data_ptr()), sh)
+                b = dict(a=qs["gate_up"].data_ptr(), w=dev_w["gate_up"][i % LAYERS].data_ptr(), ws=dev_ws["gate_up"].data_ptr(), c=cs["gate_up"].data_ptr())
+                b["as"] = ss["gate_up"].data_ptr()
+                ctx.launch(d_gu, b, sh)
+                ctx.launch(d_silu, dict(gu=cs["gate_up"].data_ptr(), q=q_dn.data_ptr(), scale=s_dn.data_ptr()), sh)
+                down(i)
+
+            def with_act(i):
+                ctx.launch(d_q, dict(x=xs["gate_up"].data_ptr(), q=qs["gate_up"].data_ptr(), scale=ss["gate_up"].data_ptr()), sh)
+                b = dict(a=qs["gate_up"].data_ptr(), w=dev_w["gate_up"][i % LAYERS].data_ptr(), ws=dev_ws["gate_up"].data_ptr(), p=p_rows.data_ptr())
+                b["as"] = ss["gate_up"].data_ptr()
+                ctx.launch(d_act, b, sh)
+                ctx.launch(d_qp, dict(x=p_rows.data_ptr(), q=q_dn.data_ptr(), scale=s_dn.data_ptr()), sh)
+                down(i)
+
+            with torch.cuda.stream(stream):
+                four(0)
+            stream.synchronize()
+            want = cs["down"].clone()
+            t4 = graph_us(four)
+            with torch.cuda.stream(stream):
+                with_act(0)
+            stream.synchronize()
+            same = bool(torch.equal(want, cs["down"]))
+            ta = graph_us(with_act)
+            res["mlp"] = dict(kernel=d_act.kernel.decode(), us_four_launches=round(t4, 2), us_with_activation_in_gate_up=round(ta, 2), same_bytes=same)
         return res
 
     if M == 1 and not args.no_other_m:

@@ -369,6 +369,20 @@ int saber_iu8_mlp_chain(saber_iu8_ctx *ctx, const void *x_bf16, const void *w_gu
                         const float *ws_dn, void *gu, void *p, void *state, void *c, uint32_t m, uint32_t hidden, uint32_t inter,
                         uint32_t spin, void *stream);
 
+/* The gate+up linear of a dense decode MLP with SiLU(gate) * up in its epilogue, for up to 16 quantised rows whose
+ * codes (rows rounded up to a power of two) fit 80 KiB of LDS at the hidden width (saber_iu8_gate_up_act_holds: 16 rows
+ * of 5,120): a [m, hidden] int8 codes (A edge) with a_scale f32 [m], w_gu W4 [2*inter, hidden] (gate rows, then up rows)
+ * with ws_gu f32 [2*inter] -> p bf16 [m, inter] = bf16(bf16(silu(gate)) * up); gu bf16 [m, 2*inter] is an optional tap
+ * of [gate | up] (NULL: not stored). Kernel macaq_iu8f_gateup_act_w4_s80 (plugin macaq_iu8f). The MLP is then
+ * quant -> this -> quant(p) -> down in place of quant -> linear -> silu_mul_quant -> down: the same bytes (p is what
+ * silu_mul_quant quantises), one pass less over [m, 2*inter] and no exp in a producer. The dense twin of the routed
+ * layer's saber_iu8_moe_gate_up_act; the reference's dense MLP keeps the activation in its producer
+ * (crates/saber-kernels/hip/mxfp4_hadi8.hip:117-146). Asynchronous. */
+int saber_iu8_gate_up_act_holds(uint32_t m, uint32_t hidden, uint32_t inter);
+int saber_iu8_resolve_gate_up_act(uint32_t m, uint32_t hidden, uint32_t inter, saber_iu8_desc *out);
+int saber_iu8_gate_up_act(saber_iu8_ctx *ctx, const void *a, const float *a_scale, const void *w_gu, const float *ws_gu, void *gu,
+                          void *p_bf16, uint32_t m, uint32_t hidden, uint32_t inter, void *stream);
+
 /* The tile GEMM with the per-token quantisation fused into its A-tile load (kernels macaq_iu8_pfq_*):
  * x bf16 [m,k] and the rows' scales a_scale f32 [m] -- from saber_iu8_rowscale (the producer's scale
  * without its codes) or carried from whatever made the rows -- instead of stored codes; c holds the

@@ -25,6 +25,9 @@ static const Signature SIG_MLP = {{"x", K::Buffer},    {"w", K::Buffer},      {"
                                   {"ws_b", K::Buffer}, {"gu", K::Buffer},     {"p", K::Buffer},  {"state", K::Buffer},
                                   {"c", K::Buffer},    {"m", K::I32},         {"k", K::I32},     {"n", K::I32},
                                   {"spin", K::I32}};
+// the gate+up linear with its activation in the epilogue (no counterpart list in the reference)
+static const Signature SIG_GATEUP_ACT = {{"a", K::Buffer},  {"w", K::Buffer}, {"as", K::Buffer}, {"ws", K::Buffer}, {"gu", K::Buffer},
+                                         {"p", K::Buffer},  {"m", K::I32},    {"n", K::I32},     {"k", K::I32}};
 static const Signature SIG_PF = {{"a", K::Buffer}, {"w", K::Buffer}, {"as", K::Buffer}, {"ws", K::Buffer},
                                  {"c", K::Buffer}, {"m", K::I32},    {"n", K::I32},     {"k", K::I32}};
 static const Signature SIG_PFQ = {{"x", K::Buffer}, {"w", K::Buffer}, {"as", K::Buffer}, {"ws", K::Buffer},
@@ -91,6 +94,7 @@ const Signature *signature_for(const std::string &k) {
   if (starts(k, "macaq_iu8_pf_")) return k.size() > 3 && k.compare(k.size() - 3, 3, "_ks") == 0 ? &SIG_DEC : &SIG_PF;
   if (starts(k, "macaq_iu8f_pair_") || starts(k, "macaq_iu8f_pairb_")) return &SIG_PAIR;
   if (starts(k, "macaq_iu8f_mlp_")) return &SIG_MLP;
+  if (starts(k, "macaq_iu8f_gateup_act_")) return &SIG_GATEUP_ACT;
   if (starts(k, "add_rms_quant_hadi8_")) return &SIG_HAD_ARQ;
   if (starts(k, "silu_mul_quant_hadi8_lut_")) return &SIG_HAD_SMQ_LUT;
   if (starts(k, "silu_mul_quant_hadi8_")) return &SIG_HAD_SMQ;

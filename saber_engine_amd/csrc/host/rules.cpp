@@ -591,6 +591,34 @@ int resolve_mlp_chain(uint32_t m, uint32_t hidden, uint32_t inter, uint32_t spin
   return 0;
 }
 
+// The gate+up linear of a decode MLP with SiLU(gate) * up in its epilogue (`macaq_iu8f_gateup_act_w4_s80`): the rows'
+// 16-row tile staged once a workgroup (what `_s80` holds), a column block = one 16-column tile of p.
+bool gate_up_act_holds(uint32_t m, uint32_t hidden, uint32_t inter) {
+  return m >= 1 && m <= 16 && hidden % 128 == 0 && inter % 16 == 0 && inter > 0 && staged80_holds(m, hidden) && inter / 16 <= 8 * CU_COUNT;
+}
+int resolve_gate_up_act(uint32_t m, uint32_t hidden, uint32_t inter, saber_iu8_desc *d) {
+  const char *op = "linear_i4a8_gate_up_act";
+  if (inter > 0x3FFFFFFFu) return fail(SABER_IU8_E_RULE, fmt("%s: intermediate width %u", op, inter));
+  if (int rc = check_shape(op, m, 2 * inter, hidden)) return rc;
+  if (!gate_up_act_holds(m, hidden, inter))
+    return fail(SABER_IU8_E_RULE, fmt("%s: %u rows of %u / %u: at most 16 rows whose codes (rows rounded up to a power of two) fit 80 KiB, "
+                                      "at most %u tiles of 16 columns", op, m, hidden, inter, 8 * CU_COUNT));
+  const char *name = "macaq_iu8f_gateup_act_w4_s80";
+  memset(d, 0, sizeof *d);
+  copy_name(d->op, sizeof d->op, op);
+  copy_name(d->plugin, sizeof d->plugin, "macaq_iu8f");
+  copy_name(d->kernel, sizeof d->kernel, name);
+  d->grid[0] = fused_grid(inter / 16), d->grid[1] = 1, d->grid[2] = 1;
+  d->block[0] = 1024, d->block[1] = 1, d->block[2] = 1;
+  d->n_launches = 1;
+  d->ks = 1;
+  if (int rc = fill_slots(name, d)) return rc;
+  set_i32(d, "m", m);
+  set_i32(d, "n", inter);
+  set_i32(d, "k", hidden);
+  return 0;
+}
+
 // The row kernels' register forms: the narrowest that holds the row (4,096 elements a group slot).
 // Many narrow rows go a wave a row (`base`_w64), the rest a workgroup a row (`base`_t256...).
 // Rows wider than 4,096 whose count leaves the card part idle go 16 waves a row (`base`_t1024): measured on this

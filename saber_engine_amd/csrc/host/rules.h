@@ -60,6 +60,8 @@ bool fused_form_holds(bool a80, uint32_t m, uint32_t k);  // what the kernel its
 bool fused_small_holds(uint32_t m, uint32_t k);  // the 20 KiB form: up to 4 rows (`_tm1`, and the MLP chain's first linear)
 bool mlp_chain_pays(uint32_t m, uint32_t hidden, uint32_t inter);        // ... and measured faster than the three launches
 bool mlp_chain_form_holds(uint32_t m, uint32_t hidden, uint32_t inter);  // the chain: 20 KiB at the hidden width, 20 or 80 KiB at the intermediate
+bool gate_up_act_holds(uint32_t m, uint32_t hidden, uint32_t inter);  // the gate+up linear with the activation in its epilogue
+int resolve_gate_up_act(uint32_t m, uint32_t hidden, uint32_t inter, saber_iu8_desc *out);
 bool staged80_holds(uint32_t m, uint32_t k);  // up to 16 rows whose codes (rows rounded up to a power of two) fit 80 KiB
 uint32_t fused_grid(uint32_t nblk);  // workgroups for nblk column blocks: one a CU, then equal shares of at most 8
 int resolve_fused(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *out);

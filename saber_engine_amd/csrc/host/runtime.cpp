@@ -379,6 +379,15 @@ static int chain_guard(const LoadedKernel &lk, const saber_iu8_desc *d) {
 
 static int launch_guard(const LoadedKernel &lk, const saber_iu8_desc *d) {
   if (strncmp(d->kernel, "macaq_iu8f_mlp_", 15) == 0) return chain_guard(lk, d);
+  if (strncmp(d->kernel, "macaq_iu8f_gateup_act_", 22) == 0) {
+    const int64_t m = i32_arg(d, "m"), n = i32_arg(d, "n"), k = i32_arg(d, "k");
+    if (m <= 0 || n <= 0 || k <= 0 || !gate_up_act_holds((uint32_t)m, (uint32_t)k, (uint32_t)n))
+      return fail(SABER_IU8_E_RULE, fmt("%s: %lld rows of %lld / %lld do not fit the form", d->kernel, (long long)m, (long long)k, (long long)n));
+    if ((int64_t)d->grid[0] * 8 < n / 16 || d->grid[1] != 1 || d->grid[2] != 1)
+      return fail(SABER_IU8_E_RULE, fmt("%s: grid %u x %u x %u cannot walk %lld column blocks (at most 8 a workgroup)", d->kernel,
+                                        d->grid[0], d->grid[1], d->grid[2], (long long)(n / 16)));
+    return 0;
+  }
   const size_t klen = strlen(d->kernel);
   const bool s80 = klen > 4 && !strcmp(d->kernel + klen - 4, "_s80");
   if (strncmp(d->kernel, "macaq_iu8_decq_", 15) != 0 && !s80) return 0;
@@ -477,6 +486,20 @@ int saber_iu8_mlp_chain(saber_iu8_ctx *ctx, const void *x, const void *w_gu, con
                                  {"ws_b", (void *)ws_dn}, {"gu", gu},          {"p", p},              {"state", state},
                                  {"c", c}};
   return saber_iu8_launch(ctx, &d, b, 9, stream);
+}
+
+int saber_iu8_gate_up_act_holds(uint32_t m, uint32_t hidden, uint32_t inter) { return gate_up_act_holds(m, hidden, inter) ? 1 : 0; }
+int saber_iu8_resolve_gate_up_act(uint32_t m, uint32_t hidden, uint32_t inter, saber_iu8_desc *out) {
+  if (!out) return fail(SABER_IU8_E_ARG, "resolve_gate_up_act: null descriptor");
+  return resolve_gate_up_act(m, hidden, inter, out);
+}
+int saber_iu8_gate_up_act(saber_iu8_ctx *ctx, const void *a, const float *as, const void *w_gu, const float *ws_gu, void *gu,
+                          void *p, uint32_t m, uint32_t hidden, uint32_t inter, void *stream) {
+  saber_iu8_desc d;
+  if (int rc = resolve_gate_up_act(m, hidden, inter, &d)) return rc;
+  if (!gu) set_null(&d, "gu");  // the [gate | up] rows are a tap: the kernel tests the pointer
+  const saber_iu8_binding b[] = {{"a", (void *)a}, {"w", (void *)w_gu}, {"as", (void *)as}, {"ws", (void *)ws_gu}, {"gu", gu}, {"p", p}};
+  return saber_iu8_launch(ctx, &d, b, 6, stream);
 }
 
 int saber_iu8_rowscale(saber_iu8_ctx *ctx, const void *x, float *scale, uint32_t m, uint32_t k, void *stream) {

@@ -47,6 +47,16 @@ struct iu8_decq_codes {
   __device__ bool wait() const { return true; }
   __device__ void amax(float[4]) const {}
 };
+// CH 4: both -- quantised rows in (CH 3), gate and up paired with p = bf16(bf16(silu(gate)) * up) out (CH 1): the
+// gate+up linear of a decode MLP at 5 to 16 rows with the activation in its epilogue. `slot` null: no maxima kept
+// (the rows' requantisation is a producer launch of its own behind this one).
+struct iu8_decq_codes_pair {
+  const float *as;
+  unsigned short *p;
+  float *slot;
+  __device__ bool wait() const { return true; }
+  __device__ void amax(float[4]) const {}
+};
 static __device__ __forceinline__ iu8_v4u iu8_decq_ld_coherent(const iu8_v4u *p) {
   const unsigned long long lo = __hip_atomic_load((const unsigned long long *)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
   const unsigned long long hi = __hip_atomic_load((const unsigned long long *)p + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
@@ -57,7 +67,7 @@ static __device__ __forceinline__ iu8_v4u iu8_decq_ld_coherent(const iu8_v4u *p)
 template <int NT, int KW, int WPB, int CH, int AKB>
 struct iu8_decq_lds {
   static constexpr int WN = WPB / KW, RED = (KW - 1) * WN * NT * 256;
-  static constexpr bool BIG = AKB > 20, PAIRED = CH == 1;
+  static constexpr bool BIG = AKB > 20, PAIRED = CH == 1 || CH == 4;
   __attribute__((aligned(16))) iu8_u8 s_a[AKB * 1024];  // staged codes: pow2(M) * K bytes
   __attribute__((aligned(16))) int s_red[2][RED];       // the k-waves' partials, two alternating areas
   float s_amax[WPB][4];
@@ -75,7 +85,7 @@ __device__ __forceinline__ void iu8_decq_body(iu8_decq_lds<NT, KW, WPB, CH, AKB>
                                               const Hook hook = Hook{}) {
   static_assert(KW > 1 && WPB % KW == 0, "k-waves divide the workgroup");
   constexpr int WN = WPB / KW;
-  constexpr bool PAIRED = CH == 1;
+  constexpr bool PAIRED = CH == 1 || CH == 4;
   static_assert(!PAIRED || (WN == 2 && NT == 1 && !W8), "the paired form: a gate wave and an up wave a tile");
   constexpr int WNB = PAIRED ? 1 : WN;  // column-tile groups of the OUTPUT a block
   constexpr int NTHR = WPB * 64;
@@ -87,7 +97,7 @@ __device__ __forceinline__ void iu8_decq_body(iu8_decq_lds<NT, KW, WPB, CH, AKB>
   // reciprocals are made once a row by 16 lanes, and a lane reads its row's scale for the epilogue.
   constexpr bool BIG = AKB > 20;
   static_assert(!BIG || CH != 1, "the chain's first linear stages at most 20 KiB");
-  constexpr bool CODES = CH == 3;
+  constexpr bool CODES = CH == 3 || CH == 4;
   auto &s_a = S.s_a;
   auto &s_red = S.s_red;
   auto &s_amax = S.s_amax;
@@ -529,7 +539,7 @@ __device__ __forceinline__ void iu8_decq_body(iu8_decq_lds<NT, KW, WPB, CH, AKB>
       if (nb > 0) pair_done(nb - 1);
       pmax = fmaxf(pmax, __shfl_xor(pmax, 16));
       pmax = fmaxf(pmax, __shfl_xor(pmax, 32));
-      if (lane < 4)  // all four words, every launch: nothing of an earlier launch survives
+      if (lane < 4 && hook.slot != nullptr)  // all four words, every launch: nothing of an earlier launch survives
         __hip_atomic_store((unsigned *)hook.slot + lane, lane < M ? __float_as_uint(pmax) : 0u, __ATOMIC_RELAXED,
                            __HIP_MEMORY_SCOPE_SYSTEM);
     }

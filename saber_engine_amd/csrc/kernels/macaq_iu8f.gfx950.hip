@@ -57,3 +57,18 @@ extern "C" __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu
     int spin) {
   iu8_chain_mlp<1, 8, 16, 4, 80>(x, w, ws, w_b, ws_b, gu, p, state, c, m, k, n, spin);
 }
+
+// THE GATE+UP LINEAR OF A DECODE MLP WITH ITS ACTIVATION, 5 to 16 rows: a [m, k] = the rows' int8 codes (one 16-row
+// tile, K <= 5120, staged once a workgroup as in macaq_iu8_dec_w4_tm1_s80) x w [2n, k] (gate rows, then up rows) ->
+// p bf16 [m, n] = bf16(bf16(silu(gate)) * up), the gate and up tiles of a 16-column block computed side by side by
+// the two halves of a workgroup's waves and met in its epilogue; gu (bf16 [m, 2n], may be null) is a tap of
+// [gate | up]. The dense twin of the routed layer's moe_iu8_grouped_w4_decpa_*: in place of linear ->
+// macaq_i8_silu_mul_quant_* the MLP runs this launch and the plain quantiser on p, which reads half the bytes
+// and computes no exp. Grid: the fused forms' (n / 16 column blocks, at most 8 a workgroup), block 1024.
+extern "C" __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4))) void macaq_iu8f_gateup_act_w4_s80(
+    const unsigned char *__restrict__ a, const unsigned char *__restrict__ w, const float *__restrict__ as,
+    const float *__restrict__ ws, unsigned short *__restrict__ gu, unsigned short *__restrict__ p, int m, int n, int k) {
+  __shared__ iu8_decq_lds<1, 8, 16, 4, 80> lds;
+  iu8_decq_body<false, 1, 8, 16, 4, 4, iu8_decq_codes_pair, 80>(lds, (const unsigned short *)a, w, ws, nullptr, nullptr, gu, m, n, k,
+                                                                 iu8_decq_codes_pair{as, p, nullptr});
+}

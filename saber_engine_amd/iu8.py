@@ -120,6 +120,9 @@ def lib():
         L.saber_iu8_fused_holds.argtypes = [C.c_uint32, C.c_uint32]
         L.saber_iu8_mlp_chain_holds.argtypes = [C.c_uint32] * 3
         L.saber_iu8_mlp_chain_pays.argtypes = [C.c_uint32] * 3
+        L.saber_iu8_gate_up_act_holds.argtypes = [C.c_uint32] * 3
+        L.saber_iu8_resolve_gate_up_act.argtypes = [C.c_uint32] * 3 + [C.POINTER(Desc)]
+        L.saber_iu8_gate_up_act.argtypes = [C.c_void_p] * 7 + [C.c_uint32] * 3 + [C.c_void_p]
         L.saber_iu8_pair.argtypes = [C.POINTER(Desc)] * 3
         L.saber_iu8_pair_ordered.argtypes = [C.POINTER(Desc)] * 2 + [C.c_int, C.POINTER(Desc)]
         L.saber_iu8_load_plugin.argtypes = [C.c_void_p, C.c_char_p]
@@ -229,6 +232,16 @@ def fused_small_holds(m, k):
 
 def mlp_chain_holds(m, hidden, inter):
     return bool(lib().saber_iu8_mlp_chain_holds(m, hidden, inter))
+
+
+def gate_up_act_holds(m, hidden, inter):
+    return bool(lib().saber_iu8_gate_up_act_holds(m, hidden, inter))
+
+
+def resolve_gate_up_act(m, hidden, inter):
+    d = Desc()
+    _check(lib().saber_iu8_resolve_gate_up_act(m, hidden, inter, C.byref(d)))
+    return d
 
 
 def mlp_chain_pays(m, hidden, inter):
@@ -399,6 +412,9 @@ class Context:
 
     def gemm(self, wkind, a, a_scale, w, w_scale, c, m, n, k, partial=None, counter=None, stream=0):
         _check(lib().saber_iu8_gemm(self._h, wkind, a, a_scale, w, w_scale, c, m, n, k, partial, counter, stream))
+
+    def gate_up_act(self, a, a_scale, w_gu, ws_gu, gu, p, m, hidden, inter, stream=0):
+        _check(lib().saber_iu8_gate_up_act(self._h, a, a_scale, w_gu, ws_gu, gu, p, m, hidden, inter, stream))
 
     def rowscale(self, x, scale, m, k, stream=0):
         _check(lib().saber_iu8_rowscale(self._h, x, scale, m, k, stream))

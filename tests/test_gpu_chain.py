@@ -156,3 +156,51 @@ def test_chain_refuses_what_the_form_does_not_hold(ctx):
         ctx.launch(d, bufs)
     assert e.value.code == iu8.E_RULE and "column blocks" in str(e.value)
     assert ctx.counters().launches == before
+
+
+@pytest.mark.parametrize("M,H,I,grid", [(16, 5120, 17408, 0), (8, 5120, 17408, 0), (5, 1408, 2944, 0), (13, 640, 12672, 100), (1, 384, 384, 0),
+                                         (3, 17408, 256, 0), (16, 2048, 4096, 32)])
+def test_gate_up_linear_with_the_activation_in_its_epilogue(ctx, M, H, I, grid):
+    """saber_iu8_gate_up_act: quantised rows in, p = bf16(bf16(silu(gate)) * up) out, the [gate | up] tap beside it --
+    the oracle's linear and its SiLU * up, and the plain quantiser on p gives silu_mul_quant's codes and scales. Full and
+    ragged row counts, the benchmark layer, K steps that do not divide among the k-waves, few live rows of a long K,
+    a grid that gives workgroups an uneven share."""
+    say(f"gate+up with activation M={M} H={H} I={I} grid={grid}")
+    mlp = Mlp(M, H, I, seed=3 * M + I)
+    want_gu = ref.linear(mlp.X, mlp.Wgu, mlp.wsgu, False, threads=16)["C"]
+    want_q, want_s, want_p = ref.silu_mul_quant(want_gu)
+    assert iu8.gate_up_act_holds(M, H, I)
+    q0 = torch.full((iu8.a_bytes(M, H),), 0x55, dtype=torch.uint8, device="cuda")
+    s0 = torch.zeros(M, dtype=torch.float32, device="cuda")
+    ctx.quant(mlp.x.data_ptr(), q0.data_ptr(), s0.data_ptr(), M, H)
+    for tap in (True, False):
+        gu = torch.full((M, 2 * I), 0x7FC0, dtype=torch.int16, device="cuda")
+        p = torch.full((M, I), 0x7FC0, dtype=torch.int16, device="cuda")
+        if grid:
+            d = iu8.resolve_gate_up_act(M, H, I)
+            assert grid * 8 >= I // 16
+            d.grid[0] = grid
+            if not tap:
+                d.arg("gu").kind = iu8.ARG_NULL_BUFFER
+            bufs = {"a": q0.data_ptr(), "w": mlp.wgu.data_ptr(), "as": s0.data_ptr(), "ws": mlp.wsg.data_ptr(), "p": p.data_ptr()}
+            if tap:
+                bufs["gu"] = gu.data_ptr()
+            ctx.launch(d, bufs)
+        else:
+            ctx.gate_up_act(q0.data_ptr(), s0.data_ptr(), mlp.wgu.data_ptr(), mlp.wsg.data_ptr(), gu.data_ptr() if tap else None, p.data_ptr(), M, H, I)
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(host_u16(p), want_p)
+        if tap:
+            np.testing.assert_array_equal(host_u16(gu), want_gu)
+        else:
+            assert (host_u16(gu) == 0x7FC0).all()
+    q = torch.full((iu8.a_bytes(M, I),), 0x55, dtype=torch.uint8, device="cuda")
+    s = torch.zeros(M, dtype=torch.float32, device="cuda")
+    ctx.quant(p.data_ptr(), q.data_ptr(), s.data_ptr(), M, I)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(s.cpu().numpy().view(np.uint32), want_s.view(np.uint32))
+    np.testing.assert_array_equal(iu8.unpack_a(q.cpu().numpy(), M, I), want_q)
+    for bad in (lambda: iu8.resolve_gate_up_act(17, H, I), lambda: iu8.resolve_gate_up_act(16, 5248, I), lambda: iu8.resolve_gate_up_act(M, H, I + 8)):
+        with pytest.raises(iu8.IU8Error) as e:
+            bad()
+        assert e.value.code == iu8.E_RULE

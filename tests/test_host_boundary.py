@@ -199,6 +199,22 @@ def test_row_producer_forms_by_law():
         iu8.resolve_quant(4, 32832)
 
 
+def test_gate_up_with_activation_descriptor():
+    """saber_iu8_resolve_gate_up_act: the fused forms' grid over inter / 16 column blocks, 1,024 threads, the kernarg list
+    (a, w, as, ws, gu, p, m, n, k) with n = the intermediate width; what does not fit is refused by name."""
+    d = iu8.resolve_gate_up_act(16, 5120, 17408)
+    assert d.kernel == b"macaq_iu8f_gateup_act_w4_s80" and d.plugin == b"macaq_iu8f" and d.op == b"linear_i4a8_gate_up_act"
+    assert tuple(d.grid) == (218, 1, 1) and d.block[0] == 1024 and d.n_workspaces == 0 and d.kernarg_bytes == 60
+    assert [d.args[i].name.decode() for i in range(d.n_args)] == ["a", "w", "as", "ws", "gu", "p", "m", "n", "k"]
+    assert (d.arg("m").ival, d.arg("n").ival, d.arg("k").ival) == (16, 17408, 5120)
+    assert iu8.resolve_gate_up_act(3, 17408, 256).grid[0] == 16 and iu8.gate_up_act_holds(4, 20480, 64)
+    for m, h, i in ((17, 5120, 17408), (16, 5248, 17408), (5, 10368, 1024), (8, 5120, 17400), (0, 5120, 17408), (16, 5120, 16 * 2049)):
+        assert not iu8.gate_up_act_holds(m, h, i), (m, h, i)
+        with pytest.raises(iu8.IU8Error) as e:
+            iu8.resolve_gate_up_act(m, h, i)
+        assert e.value.code == iu8.E_RULE
+
+
 def test_fused_quant_tile_gemm_descriptors():
     """macaq_iu8_pfq_*: the geometry of the cell the suffix names, the pf kernarg list with `x` for `a`."""
     d = iu8.describe("macaq_iu8_pfq_w4_t256x160", 2048, 5120, 17408)
