@@ -262,10 +262,10 @@ int saber_iu8_quant_rowmajor(saber_iu8_ctx *ctx, const void *x_bf16, void *q, fl
  *                       bf16(core * bf16(sigmoid(gate))); n at most 6,144
  *                       (hip/attn_glue_hadi8.hip:23-79, symbol attn_gate_quant_hadi8_t256_tiled1)
  * The square-root reciprocal is IEEE here where the reference calls the device's approximate rsqrtf.
- * Up to 256 rows of 4,096 elements and more launch a 1,024-thread form of every producer but add_rms (kernels
+ * Up to 256 rows of 4,096 elements and more launch a 1,024-thread form of every producer (kernels
  * `<stem>_hadi8_t1024`, `attn_gate_quant_hadi8[_lut]_t1024`; no counterpart among the reference's symbols): the
- * same bytes -- only add_rms's sum of squares is a tree over the workgroup -- and 15-40 % less time while the
- * rows are fewer than the compute units. */
+ * same bytes -- add_rms, whose sum of squares is a tree over the workgroup, keeps the 256-thread form's order there
+ * (rows of up to 8,192) -- and 15-40 % less time while the rows are fewer than the compute units. */
 int saber_iu8_quant_had(saber_iu8_ctx *ctx, const void *x_bf16, void *q, float *scale, uint32_t m, uint32_t k,
                         const float *had_t, void *stream);
 int saber_iu8_silu_mul_quant_had(saber_iu8_ctx *ctx, const void *gu_bf16, void *q, float *scale, uint32_t m, uint32_t n,

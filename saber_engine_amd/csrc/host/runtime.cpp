@@ -613,7 +613,7 @@ int saber_iu8_gemm_acc(saber_iu8_ctx *ctx, int wkind, const void *a, const void 
 // 512 up to 20,480 (the reference's t256 / t512 pair, crates/saber-kernels/src/macaq_iu8.rs:864-875).
 // Few rows (fewer than CUs) of 4,096 elements and more go 16 waves a row (`<stem>_hadi8_t1024`, no counterpart among the
 // reference's symbols) where the workgroup's size does not enter the result -- every producer but add_rms, whose sum
-// of squares is a tree over the workgroup: the same bytes, and on this card at 16 rows (graph replay, us) the attention
+// of squares is a tree over the workgroup and whose 16-wave form keeps the 256-thread order (6.4 -> 4.7 at 16 rows of 5,120): the same bytes, and on this card at 16 rows (graph replay, us) the attention
 // gate 6.9 -> 4.8 (table form 7.1 -> 4.4), the GDN norm 7.2 -> 5.7, SiLU * up of 5,120 6.6 -> 4.7 and of 17,408 9.7 -> 9.0
 // (table form 7.6 -> 6.2), the plain transform of 5,120 3.6 -> 3.1 (of 17,408 the 512-thread form is as fast: kept);
 // from 512 rows on the narrow forms win.
@@ -674,7 +674,8 @@ int saber_iu8_silu_mul_quant_had_lut(saber_iu8_ctx *ctx, const void *gu, void *q
 int saber_iu8_add_rms_quant_had(saber_iu8_ctx *ctx, const void *y, const void *res, const void *w, void *q, float *scale,
                                 void *res_out, uint32_t m, uint32_t k, float eps, const float *had_t, void *stream) {
   saber_iu8_desc d;
-  if (int rc = had_desc("add_rms_quant_had_i8", "add_rms_quant", m, k, &d)) return rc;
+  // the 16-wave form carries the 256-thread form's sum order (a chain handed through LDS): one group a thread, K <= 8192
+  if (int rc = had_desc("add_rms_quant_had_i8", "add_rms_quant", m, k, &d, k <= 8192)) return rc;
   set_i32(&d, "k", k);
   set_f32(&d, "eps", eps);
   const saber_iu8_binding b[] = {{"y", (void *)y}, {"res", (void *)res}, {"w", (void *)w}, {"q", q},

@@ -123,6 +123,79 @@ static __device__ __forceinline__ void had_add_rms_body(const unsigned short *__
   had_tail<T>(sv, NV, q, scale, row, K);
 }
 
+// add_rms for few rows of up to 8,192 elements, 16 waves a row, with the sum of squares in the 256-thread form's order
+// (which is part of its law: thread t of 256 runs one fma chain over its groups t, t + 256, t + 512, t + 768 in turn, then
+// the 32-lane and 8-partial trees). Here thread tid owns group tid, and the chain of "thread" t = tid % 256 is handed
+// from slice tid / 256 to the next through LDS -- four short turns -- while everything else (the loads, y + res and its
+// store, the weights, the transform, the codes) runs on four times the threads. Same bits as
+// add_rms_quant_hadi8_t256_tiled1.
+static __device__ __forceinline__ void had_add_rms_v256_body(const unsigned short *__restrict__ y,
+                                                             const unsigned short *__restrict__ res,
+                                                             const unsigned short *__restrict__ w, iu8_u8 *__restrict__ q,
+                                                             float *__restrict__ scale, unsigned short *__restrict__ res_out,
+                                                             int K, float eps, const float *__restrict__ had_t) {
+#pragma clang fp contract(off)
+  constexpr int T = 1024, V = 256;
+  __shared__ float s_chain[V];
+  __shared__ float s_sum[V / 32];
+  const int row = had_row(), tid = threadIdx.x, NV = K >> 3, g = tid, t = tid & (V - 1), slice = tid >> 8;
+  const bool live = g < NV;
+  y += (size_t)row * K, res += (size_t)row * K, res_out += (size_t)row * K;
+  float sv[HAD_MAXG][8];
+  float vw[8];
+  if (live) {
+    float vy[8], vr[8];
+    had_load8(y + g * 8, vy);
+    had_load8(res + g * 8, vr);
+    had_load8(w + g * 8, vw);
+    unsigned o[4];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) sv[0][j] = vy[j] + vr[j];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) o[j] = iu8_bf16_bits(sv[0][2 * j]) | (iu8_bf16_bits(sv[0][2 * j + 1]) << 16);
+    *(iu8_v4u *)(res_out + g * 8) = iu8_v4u{o[0], o[1], o[2], o[3]};
+  }
+  for (int turn = 0; turn < T / V; ++turn) {
+    if (slice == turn) {
+      float ssq = turn ? s_chain[t] : 0.f;
+      if (live) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) ssq = __builtin_fmaf(sv[0][j], sv[0][j], ssq);
+      }
+      s_chain[t] = ssq;
+    }
+    __syncthreads();
+  }
+  if (tid < V) {
+    float ssq = s_chain[tid];
+#pragma unroll
+    for (int o = 16; o; o >>= 1) ssq = ssq + __shfl_down(ssq, o, 32);
+    if ((tid & 31) == 0) s_sum[tid >> 5] = ssq;
+  }
+  __syncthreads();
+  if (tid < V / 32) {
+    float v = s_sum[tid];
+#pragma unroll
+    for (int o = V / 64; o; o >>= 1) v = v + __shfl_down(v, o, 32);
+    if (tid == 0) s_sum[0] = v;
+  }
+  __syncthreads();
+  const float inv = __fdiv_rn(1.f, __builtin_sqrtf(__fdiv_rn(s_sum[0], (float)K) + eps));
+  if (live) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      sv[0][j] = iu8_bf16_f32((unsigned short)iu8_bf16_bits((sv[0][j] * inv) * (vw[j] + 1.f)));
+    had32(sv[0], had_t + 8 * g, tid);
+  }
+  had_tail<T>(sv, NV, q, scale, row, K);
+}
+extern "C" __global__ __launch_bounds__(1024) void add_rms_quant_hadi8_t1024(
+    const unsigned short *__restrict__ y, const unsigned short *__restrict__ res, const unsigned short *__restrict__ w,
+    unsigned char *__restrict__ q, float *__restrict__ scale, unsigned short *__restrict__ res_out, int K, float eps,
+    const float *__restrict__ had_t) {
+  had_add_rms_v256_body(y, res, w, q, scale, res_out, K, eps, had_t);
+}
+
 #define HAD_ARQ(name, T)                                                                                          \
   extern "C" __global__ __launch_bounds__(T) void name(                                                          \
       const unsigned short *__restrict__ y, const unsigned short *__restrict__ res,                              \

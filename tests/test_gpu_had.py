@@ -94,7 +94,7 @@ def test_add_rms_quant_had(ctx, M, K):
     np.testing.assert_array_equal(iu8.unpack_a(q.cpu().numpy(), M, K), wq)
 
 
-@pytest.mark.parametrize("M,K", [(1024, 20480), (700, 5120)])
+@pytest.mark.parametrize("M,K", [(1024, 20480), (700, 5120), (200, 8192), (256, 4160)])
 def test_add_rms_quant_had_rows_of_many_magnitudes(ctx, M, K):
     """Many rows whose sums of squares spread over fifteen orders of magnitude: the square root under `inv` must
     be the correctly rounded one on every row (an ulp of `inv` flips a bf16 value of the row once in some
@@ -218,8 +218,7 @@ def test_attn_gate_quant_had(ctx, M, H, hd, pad):
 def test_every_form_of_the_producers_by_name(ctx, M, H):
     """Each producer in each of its workgroup sizes, launched by kernel name (the reference's `_t256` / `_t512`
     symbols are what its host launches at any row count; the `_t1024` forms are what this library's law picks for
-    few long rows): the oracle's bytes from every one. add_rms is not here: its sum of squares is a tree over the
-    workgroup, so its size is part of its law (256 threads up to 10,240 elements, 512 above)."""
+    few long rows): the oracle's bytes from every one."""
     W = H * 128
     say(f"had producers by name M={M} W={W}")
     rng = np.random.default_rng(M * 7 + W)
@@ -251,6 +250,17 @@ def test_every_form_of_the_producers_by_name(ctx, M, H):
     for T in sizes:
         check(f"silu_mul_quant_hadi8_t{T}" + ("" if T == 1024 else "_tiled1"), "mxfp4_hadi8", T, dict(gu=gd.data_ptr()), want, dict(n=W))
         check(f"silu_mul_quant_hadi8_lut_t{T}", "mxfp4_hadi8", T, dict(gu=gd.data_ptr(), lut=lut.data_ptr()), want, dict(n=W))
+    # add_rms: its sum of squares is a tree over 256 threads (rows up to 10,240) or 512 (above); the 16-wave form for
+    # rows up to 8,192 hands the 256-thread form's chains through LDS, so it is held to that form's oracle
+    res = synth.f32_to_bf16_bits((rng.standard_normal((M, W)) * 4).astype(np.float32))
+    wn = synth.f32_to_bf16_bits((rng.standard_normal(W) * 0.1).astype(np.float32))
+    rd, wnd = dev_bf16_bits(res), dev_bf16_bits(wn)
+    for name, T in [("add_rms_quant_hadi8_t256_tiled1", 256)] * (W <= 10240) + [("add_rms_quant_hadi8_t512_tiled1", 512)] * (W > 10240) + \
+                   [("add_rms_quant_hadi8_t1024", 1024)] * (W <= 8192):
+        wq, wsc, wro = ref.add_rms_quant_had(X, res, wn, t, 1e-6, 256 if W <= 10240 else 512)
+        ro = torch.zeros((M, W), dtype=torch.int16, device="cuda")
+        check(name, "mxfp4_hadi8", T, dict(y=xd.data_ptr(), res=rd.data_ptr(), w=wnd.data_ptr(), res_out=ro.data_ptr()), (wq, wsc), dict(k=W), eps=1e-6)
+        np.testing.assert_array_equal(host_u16(ro), wro, err_msg=name)
     if W <= 10240:
         z = synth.f32_to_bf16_bits((rng.standard_normal((M, W + 8)) * 3).astype(np.float32))
         w = synth.f32_to_bf16_bits((1 + rng.standard_normal(128) * 0.1).astype(np.float32))
