@@ -200,6 +200,16 @@ def test_gate_up_linear_with_the_activation_in_its_epilogue(ctx, M, H, I, grid):
     torch.cuda.synchronize()
     np.testing.assert_array_equal(s.cpu().numpy().view(np.uint32), want_s.view(np.uint32))
     np.testing.assert_array_equal(iu8.unpack_a(q.cpu().numpy(), M, I), want_q)
+    if I % 64 == 0:   # ... and in the Hadamard basis: the transform + quantiser on p is silu_mul_quant_had on [gate | up]
+        t = (np.random.default_rng(I).choice([-1.0, 1.0], size=I) * np.random.default_rng(I + 1).uniform(0.5, 2.0, size=I)).astype(np.float32)
+        td = dev_f32(t)
+        qh = torch.full((iu8.a_bytes(M, I),), 0x55, dtype=torch.uint8, device="cuda")
+        sh = torch.zeros(M, dtype=torch.float32, device="cuda")
+        ctx.quant_had(p.data_ptr(), qh.data_ptr(), sh.data_ptr(), M, I, td.data_ptr())
+        torch.cuda.synchronize()
+        hq, hs = ref.silu_mul_quant_had(want_gu, t)
+        np.testing.assert_array_equal(sh.cpu().numpy().view(np.uint32), hs.view(np.uint32))
+        np.testing.assert_array_equal(iu8.unpack_a(qh.cpu().numpy(), M, I), hq)
     for bad in (lambda: iu8.resolve_gate_up_act(17, H, I), lambda: iu8.resolve_gate_up_act(16, 5248, I), lambda: iu8.resolve_gate_up_act(M, H, I + 8)):
         with pytest.raises(iu8.IU8Error) as e:
             bad()
