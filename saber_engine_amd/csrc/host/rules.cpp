@@ -355,8 +355,13 @@ int resolve(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *out) 
     // QKV / O 6.1 / 5.9 -> 6.05 / 5.8); up to 8 rows, and int8 weights at any row count, from 64 MiB of weights
     // (W4 5-8 rows: gate+up 16.6-17.9 -> 16.4-17.2, 28672 x 4096 even, 14336 x 5120 8.5 -> 9.0 the other way;
     // W8: gate+up 31.3 -> 28.4, 28672 x 4096 21.0 -> 19.9, 14336 x 5120 14.3 -> 13.6, QKV 8.1 -> 8.4 the other way).
-    if (m > 4 && k <= 5120 && staged80_holds(m, k) &&
-        ((m > 8 && wkind == SABER_IU8_W4) || (uint64_t)n * k / (wkind == SABER_IU8_W8 ? 1 : 2) >= S80_MIN_BYTES))
+    // A wide N (from 24,576 columns: three and more column blocks a workgroup) takes it at any row count, also against the
+    // staged 20 KiB form of 1-4 rows, which starts a workgroup a block (W4 gate+up at 1 / 2 / 4 rows 17.6 / 16.4 / 16.7 ->
+    // 16.6 / 15.8 / 16.35, 24576 x 2048 7.5-7.6 -> 6.85-6.9, 28672 x 4096 12.1-12.25 -> 11.2-11.9; W8 gate+up 29.2-30.8 ->
+    // 27.9-29.0; at 14336 columns and fewer it loses 0.1-0.7 us there).
+    if (k <= 5120 && staged80_holds(m, k) &&
+        ((m > 8 && wkind == SABER_IU8_W4) || n >= S80_MIN_N ||
+         (m > 4 && (uint64_t)n * k / (wkind == SABER_IU8_W8 ? 1 : 2) >= S80_MIN_BYTES)))
       return describe_s80(wkind == SABER_IU8_W8, m, n, k, 1, out);
     // ... and 2 to 4 rows of a long K, whose live rows' codes fit the same 80 KiB (the copy takes their pieces of the
     // tile): 5120 x 17408 at 2 / 3 / 4 rows 11.0 -> 10.5 / 10.7 / 10.7 us; at K = 6144 and 8704 (5.7 -> 5.8, 6.9 -> 6.9)

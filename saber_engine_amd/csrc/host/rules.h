@@ -37,6 +37,7 @@ constexpr uint32_t FUSED_R1_MIN_K = 8192;   // rows at least this long take the 
 // the activation producers' 1024-thread forms: rows wider than one group a thread of the 256-thread form, up
 // to `ROWS` of them (the quantiser / the activation), or any number of rows at least `WIDE` wide for the activation
 constexpr uint32_t MLP_CHAIN_PAYS_INTER_1 = 12288, MLP_CHAIN_PAYS_INTER_2 = 13824;  // one / two rows: the chain beats the three launches from here
+constexpr uint32_t S80_MIN_N = 24576;            // the staged persistent GEMV: columns from here at any row count
 constexpr uint64_t S80_MIN_BYTES = 64ull << 20;  // the staged persistent GEMV: weights from here at up to 8 rows, and for int8 weights
 constexpr uint32_t HAD_T1024_ROWS = 256, HAD_T1024_WIDTH = 4096;  // the Hadamard-basis producers' 16-wave forms: up to / from
 constexpr uint32_t T1024_WIDTH_OVER = 4096;

@@ -73,8 +73,12 @@ IU8_DECQA(macaq_iu8_decq_w8_tm1_a80, true, 1, 8, 16, 2, 80)
       const float *__restrict__ ws, int *__restrict__ decode_partial, int *__restrict__ decode_counter,           \
       unsigned short *__restrict__ c, int m, int n, int k) {                                                       \
     __shared__ iu8_decq_lds<NT, KW, WPB, 3, 80> lds;                                                               \
-    iu8_decq_body<W8, NT, KW, WPB, D, 3, iu8_decq_codes, 80>(lds, (const unsigned short *)a, w, ws, nullptr, nullptr, c, m, n, k, \
-                                                             iu8_decq_codes{as});                                 \
+    if (m > 8)                                                                                                     \
+      iu8_decq_body<W8, NT, KW, WPB, D, 3, iu8_decq_codes, 80, 4>(lds, (const unsigned short *)a, w, ws, nullptr, nullptr, c, m, n, \
+                                                                  k, iu8_decq_codes{as});                          \
+    else                                                                                                           \
+      iu8_decq_body<W8, NT, KW, WPB, D, 3, iu8_decq_codes, 80>(lds, (const unsigned short *)a, w, ws, nullptr, nullptr, c, m, n, k, \
+                                                               iu8_decq_codes{as});                               \
   }
 IU8_DECS(macaq_iu8_dec_w4_tm1_s80, false, 1, 8, 16, 4)
 IU8_DECS(macaq_iu8_dec_w8_tm1_s80, true, 1, 8, 16, 2)

@@ -69,6 +69,10 @@ extern "C" __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu
     const unsigned char *__restrict__ a, const unsigned char *__restrict__ w, const float *__restrict__ as,
     const float *__restrict__ ws, unsigned short *__restrict__ gu, unsigned short *__restrict__ p, int m, int n, int k) {
   __shared__ iu8_decq_lds<1, 8, 16, 4, 80> lds;
-  iu8_decq_body<false, 1, 8, 16, 4, 4, iu8_decq_codes_pair, 80>(lds, (const unsigned short *)a, w, ws, nullptr, nullptr, gu, m, n, k,
-                                                                 iu8_decq_codes_pair{as, p, nullptr});
+  if (m > 8)
+    iu8_decq_body<false, 1, 8, 16, 4, 4, iu8_decq_codes_pair, 80, 4>(lds, (const unsigned short *)a, w, ws, nullptr, nullptr, gu, m, n,
+                                                                      k, iu8_decq_codes_pair{as, p, nullptr});
+  else
+    iu8_decq_body<false, 1, 8, 16, 4, 4, iu8_decq_codes_pair, 80>(lds, (const unsigned short *)a, w, ws, nullptr, nullptr, gu, m, n, k,
+                                                                   iu8_decq_codes_pair{as, p, nullptr});
 }

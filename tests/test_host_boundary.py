@@ -89,14 +89,16 @@ def test_activation_rows_are_staged_when_they_fit():
 
 def test_sixteen_row_tile_staged_once_a_workgroup_where_it_measured_faster():
     """`_s80`: the persistent GEMV that copies the 16-row tile (K <= 5120: 80 KiB) into LDS once a workgroup.
-    W4 at 9-16 rows everywhere it holds; up to 8 rows, and int8 weights, from 64 MiB of weights."""
+    W4 at 9-16 rows everywhere it holds; up to 8 rows, and int8 weights, from 64 MiB of weights (5 rows and more) or
+    24,576 columns (any row count)."""
     for wk, m, n, k, s80 in ((iu8.W4, 16, 5120, 5120, True), (iu8.W4, 9, 96, 5120, True), (iu8.W4, 16, 16384, 4096, True),
-                             (iu8.W4, 8, 5120, 5120, False), (iu8.W4, 8, 34816, 5120, True), (iu8.W4, 5, 28672, 4096, False),
-                             (iu8.W4, 4, 34816, 5120, False), (iu8.W4, 16, 5120, 5248, False), (iu8.W4, 17, 34816, 5120, False),
+                             (iu8.W4, 8, 5120, 5120, False), (iu8.W4, 8, 34816, 5120, True), (iu8.W4, 5, 28672, 4096, True),
+                             (iu8.W4, 4, 34816, 5120, True), (iu8.W4, 1, 24576, 2048, True), (iu8.W8, 2, 34816, 5120, True),
+                             (iu8.W4, 4, 16384, 5120, False), (iu8.W8, 3, 14336, 5120, False), (iu8.W4, 16, 5120, 5248, False), (iu8.W4, 17, 34816, 5120, False),
                              (iu8.W4, 4, 5120, 17408, True), (iu8.W4, 2, 5120, 17408, True), (iu8.W4, 1, 5120, 17408, False),
                              (iu8.W4, 4, 5120, 20608, False), (iu8.W4, 2, 256, 32768, True), (iu8.W8, 4, 5120, 17408, False),
                              (iu8.W8, 16, 7168, 5120, False), (iu8.W8, 16, 14336, 5120, True), (iu8.W8, 5, 34816, 5120, True),
-                             (iu8.W8, 9, 24576, 2048, False)):
+                             (iu8.W8, 9, 24576, 2048, True)):
         d = iu8.resolve(wk, m, n, k)
         tag = "w8" if wk == iu8.W8 else "w4"
         assert (d.kernel.decode() == f"macaq_iu8_dec_{tag}_tm1_s80") == s80, (tag, m, n, k, d.kernel)
