@@ -266,11 +266,12 @@ std::string band_toml() {
       put(o, "threads", v->threads());
       put(o, "grid", std::string("[ceil(n / block_n), 1, ks]"));
       put(o, "kernarg", std::string("dec"));
-    } else if (name == "macaq_iu8_dec_w4_tm1_s80" || name == "macaq_iu8_dec_w8_tm1_s80") {
+    } else if (name.rfind("macaq_iu8_dec_w4_tm1_s80", 0) == 0 || name.rfind("macaq_iu8_dec_w8_tm1_s80", 0) == 0) {
       put(o, "regime", std::string("decode"));
       putb(o, "w8", name[15] == '8');
       put(o, "rows_max", 16);
-      put(o, "k_max", 5120);
+      if (name.back() == 'r') put(o, "staged_code_bytes_max", 80 * 1024);  // rows rounded up to a power of two x K
+      else put(o, "k_max", 5120);
       put(o, "block_n", 32);
       put(o, "threads", 1024);
       put(o, "grid", std::string("[blocks = ceil(n / 32); blocks <= cu_count ? blocks : ceil(blocks / min(8, ceil(blocks / cu_count))), 1, 1] persistent"));

@@ -193,13 +193,17 @@ static std::string dec_stream_name(const char *tag, uint32_t m, uint32_t k) {
 // (`macaq_iu8_dec_{w4,w8}_tm1_s80`): the fused forms' geometry (16 waves, 32 columns a block, at most 8 blocks a
 // workgroup) on the decode kernarg list.
 bool staged80_holds(uint32_t m, uint32_t k) { return m >= 1 && m <= 16 && staged_bytes(m, k) <= 80 * 1024; }
-static int describe_s80(bool w8, uint32_t m, uint32_t n, uint32_t k, uint32_t ks, saber_iu8_desc *d) {
+static bool staged80_tile_holds(uint32_t m, uint32_t k) { return m >= 1 && m <= 16 && (uint64_t)k * 16 <= 80 * 1024; }
+// `rows_form`: the kernel that takes the live rows' pieces of the tile (`_s80r`: few rows of a long K); else the
+// whole-tile kernel (`_s80`, K <= 5120 at any row count)
+static int describe_s80(bool w8, bool rows_form, uint32_t m, uint32_t n, uint32_t k, uint32_t ks, saber_iu8_desc *d) {
   const char *op = w8 ? "gemm_i8a8" : "gemm_i4a8";
-  const std::string name = fmt("macaq_iu8_dec_%s_tm1_s80", w8 ? "w8" : "w4");
+  const std::string name = fmt("macaq_iu8_dec_%s_tm1_s80%s", w8 ? "w8" : "w4", rows_form ? "r" : "");
   if (int rc = check_shape(op, m, n, k)) return rc;
   if (ks != 1) return fail(SABER_IU8_E_RULE, name + ": the staged form does not split K");
-  if (!staged80_holds(m, k))
-    return fail(SABER_IU8_E_RULE, fmt("%s: %u rows (rounded up to a power of two) of %u do not fit 80 KiB", name.c_str(), m, k));
+  if (rows_form ? !staged80_holds(m, k) : !staged80_tile_holds(m, k))
+    return fail(SABER_IU8_E_RULE, rows_form ? fmt("%s: %u rows (rounded up to a power of two) of %u do not fit 80 KiB", name.c_str(), m, k)
+                                            : fmt("%s: %u rows of %u do not fit one 16-row tile in 80 KiB (K <= 5120)", name.c_str(), m, k));
   memset(d, 0, sizeof *d);
   copy_name(d->op, sizeof d->op, op);
   copy_name(d->plugin, sizeof d->plugin, "macaq_iu8");
@@ -218,7 +222,8 @@ static int describe_s80(bool w8, uint32_t m, uint32_t n, uint32_t k, uint32_t ks
 }
 
 int describe(const std::string &kernel, uint32_t m, uint32_t n, uint32_t k, uint32_t ks, saber_iu8_desc *out) {
-  if (kernel == "macaq_iu8_dec_w4_tm1_s80" || kernel == "macaq_iu8_dec_w8_tm1_s80") return describe_s80(kernel[15] == '8', m, n, k, ks, out);
+  if (kernel == "macaq_iu8_dec_w4_tm1_s80" || kernel == "macaq_iu8_dec_w8_tm1_s80") return describe_s80(kernel[15] == '8', false, m, n, k, ks, out);
+  if (kernel == "macaq_iu8_dec_w4_tm1_s80r" || kernel == "macaq_iu8_dec_w8_tm1_s80r") return describe_s80(kernel[15] == '8', true, m, n, k, ks, out);
   if (const DecVariant *v = dec_variant(kernel)) return describe_dec(*v, m, n, k, ks, out);
   if (const PfVariant *v = pf_variant(kernel)) {
     if (ks != 1) return fail(SABER_IU8_E_RULE, kernel + ": the prefill tile does not split K (its `_ks` form does)");
@@ -275,13 +280,13 @@ int pair(const saber_iu8_desc &first, const saber_iu8_desc &second, saber_iu8_de
   static const char PREFIX[] = "macaq_iu8_dec_w4_";
   // a half the law gave the staged persistent form is paired as its streamed form: the pair kernels are that geometry
   for (const saber_iu8_desc *h : {&first, &second})
-    if (!strcmp(h->kernel, "macaq_iu8_dec_w4_tm1_s80")) {
+    if (!strncmp(h->kernel, "macaq_iu8_dec_w4_tm1_s80", 24)) {
       saber_iu8_desc s[2];
       const saber_iu8_desc *in[2] = {&first, &second};
       for (int i = 0; i < 2; ++i) {
         int64_t hm = 0, hn = 0, hk = 0;
         s[i] = *in[i];
-        if (!strcmp(in[i]->kernel, "macaq_iu8_dec_w4_tm1_s80")) {
+        if (!strncmp(in[i]->kernel, "macaq_iu8_dec_w4_tm1_s80", 24)) {
           if (!int_arg(*in[i], "m", &hm) || !int_arg(*in[i], "n", &hn) || !int_arg(*in[i], "k", &hk))
             return fail(SABER_IU8_E_RULE, "macaq iu8 pair: a half without its m, n, k");
           if (int rc = describe(dec_stream_name("w4", (uint32_t)hm, (uint32_t)hk), (uint32_t)hm, (uint32_t)hn, (uint32_t)hk, 1, &s[i])) return rc;
@@ -362,12 +367,12 @@ int resolve(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *out) 
     if (k <= 5120 && staged80_holds(m, k) &&
         ((m > 8 && wkind == SABER_IU8_W4) || n >= S80_MIN_N ||
          (m > 4 && (uint64_t)n * k / (wkind == SABER_IU8_W8 ? 1 : 2) >= S80_MIN_BYTES)))
-      return describe_s80(wkind == SABER_IU8_W8, m, n, k, 1, out);
+      return describe_s80(wkind == SABER_IU8_W8, false, m, n, k, 1, out);
     // ... and 2 to 4 rows of a long K, whose live rows' codes fit the same 80 KiB (the copy takes their pieces of the
     // tile): 5120 x 17408 at 2 / 3 / 4 rows 11.0 -> 10.5 / 10.7 / 10.7 us; at K = 6144 and 8704 (5.7 -> 5.8, 6.9 -> 6.9)
     // and on 16384 x 8192 (12.4 -> 12.8) the streamed form stays
     if (m >= 2 && m <= 4 && k >= 16384 && wkind == SABER_IU8_W4 && staged80_holds(m, k))
-      return describe_s80(false, m, n, k, 1, out);
+      return describe_s80(false, true, m, n, k, 1, out);
     const std::string name = dec_stream_name(tag, m, k);
     const DecVariant *v = dec_variant(name);
     if (!v) return fail(SABER_IU8_E_RULE, name + ": no such variant");

@@ -389,7 +389,8 @@ static int launch_guard(const LoadedKernel &lk, const saber_iu8_desc *d) {
     return 0;
   }
   const size_t klen = strlen(d->kernel);
-  const bool s80 = klen > 4 && !strcmp(d->kernel + klen - 4, "_s80");
+  const bool s80r = klen > 5 && !strcmp(d->kernel + klen - 5, "_s80r");
+  const bool s80 = s80r || (klen > 4 && !strcmp(d->kernel + klen - 4, "_s80"));
   if (strncmp(d->kernel, "macaq_iu8_decq_", 15) != 0 && !s80) return 0;
   int64_t m = 0, n = 0, k = 0;
   for (uint32_t i = 0; i < d->n_args; ++i) {
@@ -399,7 +400,8 @@ static int launch_guard(const LoadedKernel &lk, const saber_iu8_desc *d) {
     if (!strcmp(d->args[i].name, "k")) k = d->args[i].ival;
   }
   if (s80) {  // the staged tile: 16 rows x K bytes of LDS, the fused forms' block walk
-    if (m <= 0 || n <= 0 || k <= 0 || k % 128 || !staged80_holds((uint32_t)m, (uint32_t)k))
+    // the whole-tile kernel indexes 16 rows a K step whatever M is; the rows kernel the live rows rounded up to a power of two
+    if (m <= 0 || n <= 0 || k <= 0 || k % 128 || m > 16 || (s80r ? !staged80_holds((uint32_t)m, (uint32_t)k) : (int64_t)k * 16 > 80 * 1024))
       return fail(SABER_IU8_E_RULE, fmt("%s: %lld rows of %lld do not fit one 16-row tile in 80 KiB", d->kernel, (long long)m, (long long)k));
     if ((int64_t)d->grid[0] * 8 < (n + 31) / 32 || d->grid[1] != 1 || d->grid[2] != 1)
       return fail(SABER_IU8_E_RULE, fmt("%s: grid %u x %u x %u cannot walk %lld column blocks (at most 8 a workgroup)", d->kernel,

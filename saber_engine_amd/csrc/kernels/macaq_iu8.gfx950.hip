@@ -66,22 +66,23 @@ IU8_DECQA(macaq_iu8_decq_w8_tm1_a80, true, 1, 8, 16, 2, 80)
 // The GEMV of up to 16 quantised rows whose 16-row tile fits 80 KiB of LDS (K <= 5120), persistent like the
 // fused forms: a workgroup copies the tile into LDS once and streams its column blocks against it. The
 // streamed form (`_a0`) reads the tile from L2 once a 32-column block -- at 16 rows of K = 5120 as many bytes
-// through L2 as the weights bring from memory.
-#define IU8_DECS(name, W8, NT, KW, WPB, D)                                                                         \
+// through L2 as the weights bring from memory. `_s80r`: the same for fewer live rows of a longer K (the rows
+// rounded up to a power of two x K <= 80 KiB: 4 rows of 20,480), whose copy takes the live rows' pieces of the
+// tile; a kernel of its own because the row shift is then a register in every LDS index of the K loop, which
+// costs the whole-tile launches 0.1-0.4 us.
+#define IU8_DECS(name, W8, NT, KW, WPB, D, MRS)                                                                    \
   extern "C" __global__ __launch_bounds__(WPB * 64) __attribute__((amdgpu_waves_per_eu(4, 4))) void name(          \
       const unsigned char *__restrict__ a, const unsigned char *__restrict__ w, const float *__restrict__ as,     \
       const float *__restrict__ ws, int *__restrict__ decode_partial, int *__restrict__ decode_counter,           \
       unsigned short *__restrict__ c, int m, int n, int k) {                                                       \
     __shared__ iu8_decq_lds<NT, KW, WPB, 3, 80> lds;                                                               \
-    if (m > 8)                                                                                                     \
-      iu8_decq_body<W8, NT, KW, WPB, D, 3, iu8_decq_codes, 80, 4>(lds, (const unsigned short *)a, w, ws, nullptr, nullptr, c, m, n, \
+    iu8_decq_body<W8, NT, KW, WPB, D, 3, iu8_decq_codes, 80, MRS>(lds, (const unsigned short *)a, w, ws, nullptr, nullptr, c, m, n, \
                                                                   k, iu8_decq_codes{as});                          \
-    else                                                                                                           \
-      iu8_decq_body<W8, NT, KW, WPB, D, 3, iu8_decq_codes, 80>(lds, (const unsigned short *)a, w, ws, nullptr, nullptr, c, m, n, k, \
-                                                               iu8_decq_codes{as});                               \
   }
-IU8_DECS(macaq_iu8_dec_w4_tm1_s80, false, 1, 8, 16, 4)
-IU8_DECS(macaq_iu8_dec_w8_tm1_s80, true, 1, 8, 16, 2)
+IU8_DECS(macaq_iu8_dec_w4_tm1_s80, false, 1, 8, 16, 4, 4)
+IU8_DECS(macaq_iu8_dec_w8_tm1_s80, true, 1, 8, 16, 2, 4)
+IU8_DECS(macaq_iu8_dec_w4_tm1_s80r, false, 1, 8, 16, 4, -1)
+IU8_DECS(macaq_iu8_dec_w8_tm1_s80r, true, 1, 8, 16, 2, -1)
 #undef IU8_DECS
 
 // One row (`_r1`, the GEMV of a single token): the same launch with the row's codes made just in time --

@@ -379,14 +379,17 @@ def test_sixteen_row_tile_staged_once_a_workgroup(ctx, M, N, K, grid, w8):
     live rows of a longer K (the copy then takes the live rows' pieces of the tile: 1, 2, 4 or 8 of every 16).
     The tile's rows past M hold whatever the producer's buffer held (0x55 here): they reach no output."""
     tag = "w8" if w8 else "w4"
-    say(f"staged 16-row tile {tag} M={M} N={N} K={K} grid={grid}")
+    # the whole-tile kernel holds K <= 5120 at any row count; the rows kernel (`_s80r`) whatever fits 80 KiB, taken
+    # here for the longer K and, for every other case below it, so that both kernels see short and long loops
+    name = f"macaq_iu8_dec_{tag}_tm1_s80" + ("r" if K > 5120 or (M + N // 16) % 2 else "")
+    say(f"staged 16-row tile {name} M={M} N={N} K={K} grid={grid}")
     case = synth.dense_case(M, N, K, w8=w8, seed=M * 11 + N + K)
     r = ref.linear(case["X"], case["W"], case["ws"], w8, threads=16)
-    run = DenseRun(ctx, case, kernel=f"macaq_iu8_dec_{tag}_tm1_s80", want_acc=False)
+    run = DenseRun(ctx, case, kernel=name, want_acc=False)
     assert run.desc.block[0] == 1024 and run.desc.grid[0] * 8 >= -(-N // 32)
     np.testing.assert_array_equal(run.C, r["C"])
     if grid:
-        d = iu8.describe(f"macaq_iu8_dec_{tag}_tm1_s80", M, N, K)
+        d = iu8.describe(name, M, N, K)
         d.grid[0] = grid
         assert grid * 8 >= -(-N // 32)
         c = torch.full((M, N), 0x7FC0, dtype=torch.int16, device="cuda")
@@ -398,8 +401,8 @@ def test_sixteen_row_tile_staged_once_a_workgroup(ctx, M, N, K, grid, w8):
         # descriptors edited past what the kernel holds are refused at launch: more than 8 blocks a workgroup, a K
         # whose tile passes 80 KiB, more than 16 rows
         mr = 1 << (M - 1).bit_length()
-        for field, value in (("grid", max(1, (-(-N // 32) - 1) // 8)), ("k", 80 * 1024 // mr + 128), ("m", 17)):
-            bad = iu8.describe(f"macaq_iu8_dec_{tag}_tm1_s80", M, N, K)
+        for field, value in (("grid", max(1, (-(-N // 32) - 1) // 8)), ("k", 80 * 1024 // (mr if name.endswith("r") else 16) + 128), ("m", 17)):
+            bad = iu8.describe(name, M, N, K)
             if field == "grid":
                 if value * 8 >= -(-N // 32):
                     continue

@@ -101,15 +101,19 @@ def test_sixteen_row_tile_staged_once_a_workgroup_where_it_measured_faster():
                              (iu8.W8, 9, 24576, 2048, True)):
         d = iu8.resolve(wk, m, n, k)
         tag = "w8" if wk == iu8.W8 else "w4"
-        assert (d.kernel.decode() == f"macaq_iu8_dec_{tag}_tm1_s80") == s80, (tag, m, n, k, d.kernel)
+        # the whole-tile kernel while the 16-row tile fits (K <= 5120); the rows kernel (`_s80r`) for fewer rows of a longer K
+        name = f"macaq_iu8_dec_{tag}_tm1_s80" + ("" if k <= 5120 else "r")
+        assert (d.kernel.decode() == name) == s80 and d.kernel.decode().startswith(f"macaq_iu8_dec_{tag}_tm1_s80") == s80, (tag, m, n, k, d.kernel)
         if s80:
             blocks = -(-n // 32)
             assert d.block[0] == 1024 and d.ks == 1 and d.n_workspaces == 0
             assert d.grid[0] == (blocks if blocks <= 256 else -(-blocks // min(8, -(-blocks // 256))))
-            assert bytes(d) == bytes(iu8.describe(f"macaq_iu8_dec_{tag}_tm1_s80", m, n, k))
-    assert iu8.describe("macaq_iu8_dec_w4_tm1_s80", 8, 5120, 10240).grid[0] == 160       # by name: whatever fits 80 KiB
+            assert bytes(d) == bytes(iu8.describe(name, m, n, k))
+    assert iu8.describe("macaq_iu8_dec_w4_tm1_s80r", 8, 5120, 10240).grid[0] == 160       # by name: whatever fits 80 KiB
+    assert iu8.describe("macaq_iu8_dec_w4_tm1_s80", 3, 5120, 5120).grid[0] == 160 and iu8.describe("macaq_iu8_dec_w8_tm1_s80r", 16, 64, 5120).grid[0] == 2
     for bad in (lambda: iu8.describe("macaq_iu8_dec_w4_tm1_s80", 17, 5120, 5120), lambda: iu8.describe("macaq_iu8_dec_w4_tm1_s80", 16, 5120, 5248),
-                lambda: iu8.describe("macaq_iu8_dec_w4_tm1_s80", 5, 5120, 10368), lambda: iu8.describe("macaq_iu8_dec_w4_tm1_s80", 3, 5120, 20608),
+                lambda: iu8.describe("macaq_iu8_dec_w4_tm1_s80", 4, 5120, 17408), lambda: iu8.describe("macaq_iu8_dec_w4_tm1_s80r", 17, 5120, 128),
+                lambda: iu8.describe("macaq_iu8_dec_w4_tm1_s80r", 5, 5120, 10368), lambda: iu8.describe("macaq_iu8_dec_w4_tm1_s80r", 3, 5120, 20608),
                 lambda: iu8.describe("macaq_iu8_dec_w4_tm1_s80", 16, 5120, 5120, ks=2)):
         with pytest.raises(iu8.IU8Error) as e:
             bad()
