@@ -684,7 +684,35 @@ def main():
                 e1.record(stream)
             torch.cuda.synchronize()
             probe[tag] = round(4 * pblocks * 4 * piters * 16 * 65536.0 / (e0.elapsed_time(e1) * 1e3) / 1e6, 1)
-        out["prefill_m2048"] = dict(value=round(tops, 1), unit="TOPS", with_quant=round(tot_ops / (tot_us + tot_q_us) / 1e6, 1),
+        # a second reference point: the vendor library's plain int8 x int8 -> int32 GEMM (torch._int_mm) on the same
+        # four shapes, operands distributed like this workload's already unpacked (no W4 unpack, no scaling, int32 out,
+        # one warm weight matrix; the better of its two B orders) -- what a tuned library sustains on this card
+        lib = None
+        try:
+            lib, lib_ops, lib_us = {}, 0.0, 0.0
+            for name, n, k in linears:
+                la = torch.round(torch.randn((2048, k), device=dev, generator=g) * 2.1).clamp(-127, 127).to(torch.int8)
+                lw = torch.randint(-8, 8, (n, k), device=dev, generator=g, dtype=torch.int8) * 16
+                best = None
+                for lb in (lw.t(), lw.t().contiguous()):
+                    for _ in range(max(30, int(0.1 / (4096.0 * n * k / 2.5e15)))):
+                        lc = torch._int_mm(la, lb)
+                    l0, l1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    l0.record()
+                    for _ in range(20):
+                        lc = torch._int_mm(la, lb)
+                    l1.record()
+                    torch.cuda.synchronize()
+                    lus = l0.elapsed_time(l1) * 1e3 / 20
+                    best = lus if best is None else min(best, lus)
+                lib[name] = dict(us=round(best, 2), tops=round(4096.0 * n * k / best / 1e6, 1))
+                lib_ops += 4096.0 * n * k
+                lib_us += best
+                del la, lw, lb, lc
+            lib["value"] = round(lib_ops / lib_us / 1e6, 1)
+        except Exception as e:   # a torch build without the int8 GEMM: the figure is a side note, never the product path
+            lib = dict(error=str(e)[:120])
+        out["prefill_m2048"] = dict(value=round(tops, 1), unit="TOPS", library_int8_gemm=lib, with_quant=round(tot_ops / (tot_us + tot_q_us) / 1e6, 1),
                                     fused_quant=dict(tops=round(tot_ops / fq_us / 1e6, 1), vs_two_launch=round((tot_us + tot_q_us) / fq_us, 3),
                                                      note="row-scale pass + macaq_iu8_pfq_* (quantisation fused into the A-tile load), "
                                                           "per linear under per_linear.*.fused_quant; the launch law keeps producer + GEMM"),
