@@ -796,6 +796,12 @@ static __device__ __forceinline__ int moe_tile_order(const int *__restrict__ til
   return heavy_total;
 }
 // one cell, items in the sorted order
+// Workgroup b of a grid of G in the order in which an XCD's workgroups follow each other: b % 8 is the XCD (the
+// hardware deals consecutive ids round-robin), so XCD x holds positions x * G/8 ... of the walk. A grid that is not
+// whole eighths keeps its ids.
+static __device__ __forceinline__ int moe_xcd_run(unsigned b, int G) {
+  return (G & 7) == 0 ? (int)(b & 7) * (G >> 3) + (int)(b >> 3) : (int)b;
+}
 #define MOE_ONE_ITEMS 64  // items a workgroup resolves up front (16,384 items a launch of 256 workgroups)
 template <int GATHER, int WMW, int WNW, int TM, int TN, int ST>
 static __device__ __forceinline__ void moe_grouped_pf_one(
@@ -810,13 +816,22 @@ static __device__ __forceinline__ void moe_grouped_pf_one(
   const int nt = meta[0], gx = (n + BN - 1) / BN, total = nt * gx;
   const bool ordered = nt <= MOE_ORDER_CAP;
   if (ordered) moe_tile_order<WMW * WNW * 64>(tile_rows, nt, s_order);
-  auto resolve = [&](int id, moe_item &it) {
-    const int slot = id / gx, bx = id - slot * gx, tile = ordered ? (int)s_order[slot] : slot;
+  // Consecutive workgroup ids are dealt round-robin over the 8 XCDs, consecutive item ids are the column blocks of
+  // one tile. With a grid of whole eighths an XCD's workgroups take a run of item ids (`moe_xcd_run`), so a tile's
+  // column blocks share the tile's rows in one L2, or two (dealt by workgroup id they spread over all eight and
+  // every XCD fetched the rows for itself: the L2-miss fetch of a launch at 4,096 tokens was twice its operands).
+  const int G = gridDim.x, wv = moe_xcd_run(blockIdx.x, G);
+  const int rounds = (total + G - 1) / G;
+  auto resolve = [&](int q, moe_item &it) {  // this workgroup's item of round q; false past its last
+    const int j = wv + q * G;
+    const int slot = j / gx, bx = j % gx;
+    if (slot >= nt) return false;
+    const int tile = ordered ? (int)s_order[slot] : slot;
     const int e = tile_expert[tile];
     it = moe_item{tile_row0[tile], min(tile_rows[tile], WMW * TM * 32), bx * (BN / 16), 0,
                   (const unsigned char *)xptr[2 * e], (const float *)xptr[2 * e + 1]};
+    return true;
   };
-  const int G = gridDim.x, rounds = (total + G - 1) / G;
   if (rounds <= MOE_ONE_ITEMS) {
     // An item's descriptor hangs on a chain of dependent loads (order -> tile table -> expert pointers);
     // fetched where the load stream crosses into the item, every link drains the stream. The
@@ -824,8 +839,7 @@ static __device__ __forceinline__ void moe_grouped_pf_one(
     const int q = threadIdx.x;
     if (q < rounds) {
       moe_item it{0, -1, 0, 0, nullptr, nullptr};
-      const int id = (int)blockIdx.x + q * G;
-      if (id < total) resolve(id, it);
+      resolve(q, it);
       s_item[q] = it;
     }
     __syncthreads();
@@ -842,10 +856,8 @@ static __device__ __forceinline__ void moe_grouped_pf_one(
     return;
   }
   iu8_pf32_run<false, WMW, WNW, TM, TN, false, ST, false, true, GATHER == 2, true>(a, as, c, n, k, [&](int r, iu8_tile &t) {
-    const int id = (int)blockIdx.x + r * G;
-    if (id >= total) return false;
     moe_item it;
-    resolve(id, it);
+    if (r >= rounds || !resolve(r, it)) return false;
     t = iu8_tile{iu8_rows{GATHER ? row_tok : nullptr, it.row0, it.rows}, 0, it.nt0, it.W, it.ws};
     return true;
   }, nullptr, nullptr, lds);
@@ -881,7 +893,7 @@ static __device__ __forceinline__ void moe_grouped_pf_two(
   /* a launch of more rounds than the item table holds runs in epochs of that many */
   for (int ep = 0;; ++ep) {
     {
-      const int gx = (n + BN - 1) / BN, G = gridDim.x, w = blockIdx.x;
+      const int gx = (n + BN - 1) / BN, G = gridDim.x, w = moe_xcd_run(blockIdx.x, G);
       const int hi = heavy * gx, li = (nt - heavy) * gx;
       const int h0 = ep * MOE_HEAVY_ROUNDS, l0 = ep * MOE_LIGHT_ROUNDS;
       const int rounds = max(0, min((hi + G - 1) / G - h0, MOE_HEAVY_ROUNDS));
