@@ -176,6 +176,11 @@ def main():
     with torch.cuda.stream(stream):
         for _ in range(settle_replays):
             g_all.replay()
+        # the last settling replays go out the way the timed one does -- a replay, then a synchronisation -- so that
+        # the host's side of that pair (its caches, the wake-up from a short wait instead of a 30 ms one) is settled too
+        for _ in range(4):
+            torch.cuda.synchronize()
+            g_all.replay()
 
     # ---- the timed region: exactly K steps, one graph replay, bracketed by synchronisation; the host clock gives
     # ms_per_step and `value`, HIP events on the replay's stream give the same K steps without the host's
