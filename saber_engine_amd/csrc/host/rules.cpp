@@ -384,19 +384,25 @@ int resolve(int wkind, uint32_t m, uint32_t n, uint32_t k, saber_iu8_desc *out) 
 }
 
 // K shares of a tile launch (0: none). A deep, narrow linear at a few dozen rows gives the unsplit
-// law so few tiles that two thirds of the CUs idle through hundreds of K steps; there, 3-4 workgroups
+// law so few tiles that half to two thirds of the CUs idle through hundreds of K steps; there, 2-4 workgroups
 // a tile of the 64x128 cell, each on a share of K, measured 9-19 % faster although the partials
 // travel through memory (5120 x 17408: M=64 34.1 -> 28.6 us, M=128 33.6 -> 30.7 us). On every other
-// shape timed (K <= 6144 at any M, more than 80 tiles at any K) the unsplit cell won by 1.3-3x --
+// shape timed (K <= 6144 at any M, more than 128 tiles at any K, 256 rows and more) the unsplit cell won --
 // the partials cost ks*M*N*4 bytes each way and the last arriver sums alone -- so the rule is this
 // narrow. The launch then needs the `decode_partial` / `decode_counter` workspaces the descriptor lists.
 uint32_t pf_split(bool w8, uint32_t m, uint32_t n, uint32_t k, const PfVariant **cell) {
-  // measured at 33..128 rows; above, the partials (ks * M * N * 4 bytes each way) grow with M
-  if (w8 || k < 16384 || m > 128) return 0;
+  // measured at 33..192 rows; above, the partials (ks * M * N * 4 bytes each way) grow with M (at 256 rows the unsplit
+  // cell is level or ahead: 5120 x 17408 43.9 against 43.9-58.6 us). Up to 128 tiles, i.e. two shares at least:
+  // 81-128 tiles on two shares against the law's unsplit pick, us -- 5120 x 17408 at 129 / 160 / 192 rows 33.7 / 34.1 /
+  // 35.3 against 35.4 / 36.7 / 36.5, 5120 x 20480 38.2 / 38.8 / 38.4 against 40.4 / 42.1 / 42.5, 4096 x 16384 31.0 / 31.4 /
+  // 32.0 against 32.3 / 33.4 / 33.6; 8192 x 16384 at 96 / 128 rows 33.0 / 34.6 against 36.4 / 37.9, 12288 x 16384 at
+  // 49 / 64 rows 33.3 / 34.6 against 35.8 / 35.5; 72 tiles on three shares (3072 x 16384 at 129-192 rows) 28.1-28.7
+  // against 31.7-32.0.
+  if (w8 || k < 16384 || m > 192) return 0;
   const PfVariant *v = pf_variant("macaq_iu8_pf_w4_t64x128_s");
   if (!v || !signature_for(std::string(v->name) + "_ks")) return 0;
   const uint64_t tiles = (uint64_t)((n + v->block_n() - 1) / v->block_n()) * ((m + v->block_m() - 1) / v->block_m());
-  if (tiles > 80) return 0;
+  if (tiles > 128) return 0;
   *cell = v;
   return (uint32_t)std::min<uint64_t>(4, CU_COUNT / tiles);
 }

@@ -207,9 +207,10 @@ def test_tile_gemm_with_k_split_over_workgroups(ctx, shape, splits):
         iu8.describe("macaq_iu8_pf_w4_t128x128", 200, 272, 640, ks=2)             # the plain cell does not split
 
 
-@pytest.mark.parametrize("shape,ks", [((64, 384, 16384), 4), ((100, 640, 17408), 4), ((128, 5120, 17408), 3)])
+@pytest.mark.parametrize("shape,ks", [((64, 384, 16384), 4), ((100, 640, 17408), 4), ((128, 5120, 17408), 3),
+                                      ((129, 5120, 17408), 2), ((192, 3072, 16384), 3), ((77, 8192, 16384), 2)])
 def test_launch_law_splits_deep_narrow_tile_gemm(ctx, shape, ks):
-    """Where the law shares K over workgroups (K >= 16384, at most 80 tiles of the 64x128 cell) the
+    """Where the law shares K over workgroups (K >= 16384, up to 192 rows, at most 128 tiles of the 64x128 cell) the
     descriptor lists the workspaces and the launch through it gives the oracle's bytes."""
     M, N, K = shape
     say(f"law-split tile GEMM {shape}")

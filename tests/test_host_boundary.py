@@ -331,9 +331,13 @@ def test_operands_past_4_gib_are_refused_by_the_tile_gemm():
 
 
 def test_launch_law_shares_k_only_on_deep_narrow_tile_gemms():
-    """The one band where the law splits the tile GEMM: K >= 16384 and at most 80 tiles of the
-    64x128 cell; the descriptor then names the `_ks` form, its z grid and both workspaces."""
-    for m, ks, tiles in ((33, 4, 40), (48, 4, 40), (49, 4, 40), (64, 4, 40), (65, 3, 80), (128, 3, 80)):
+    """The one band where the law splits the tile GEMM: K >= 16384, up to 192 rows and at most 128 tiles of the
+    64x128 cell (two shares at least); the descriptor then names the `_ks` form, its z grid and both workspaces."""
+    for wk, m, n, k, ks in ((iu8.W4, 64, 12288, 17408, 2), (iu8.W4, 128, 8192, 16384, 2), (iu8.W4, 160, 3072, 16384, 3)):
+        d = iu8.resolve(wk, m, n, k)
+        tiles = -(-m // 64) * (n // 128)
+        assert d.kernel == b"macaq_iu8_pf_w4_t64x128_s_ks" and d.ks == ks and tuple(d.grid) == (tiles, 1, ks), (m, n, k)
+    for m, ks, tiles in ((33, 4, 40), (48, 4, 40), (49, 4, 40), (64, 4, 40), (65, 3, 80), (128, 3, 80), (129, 2, 120), (192, 2, 120)):
         d = iu8.resolve(iu8.W4, m, 5120, 17408)
         assert d.kernel == b"macaq_iu8_pf_w4_t64x128_s_ks" and d.ks == ks and tuple(d.grid) == (tiles, 1, ks)
         assert d.workspace("decode_partial").bytes == ks * m * 5120 * 4 and d.workspace("decode_partial").kind == iu8.WS_SCRATCH
@@ -342,7 +346,7 @@ def test_launch_law_shares_k_only_on_deep_narrow_tile_gemms():
         assert iu8.gemm_workspace(iu8.W4, m, 5120, 17408) == (ks * m * 5120 * 4, tiles * 4)
     # up to 32 rows the streaming form keeps a deep narrow linear too (18.0 against 22.4 us)
     assert iu8.resolve(iu8.W4, 32, 5120, 17408).kernel == b"macaq_iu8_dec_w4_tm2"
-    for wk, m, n, k in ((iu8.W4, 129, 5120, 17408), (iu8.W4, 64, 5120, 16256), (iu8.W4, 64, 12288, 17408),
+    for wk, m, n, k in ((iu8.W4, 193, 5120, 17408), (iu8.W4, 64, 5120, 16256), (iu8.W4, 64, 16512, 17408), (iu8.W4, 129, 8192, 16384),
                         (iu8.W8, 64, 5120, 17408), (iu8.W4, 2048, 5120, 17408), (iu8.W4, 64, 5120, 5120),
                         (iu8.W4, 4096, 128, 17408), (iu8.W4, 4096, 16, 16384)):       # many rows of a narrow output: few tiles, no split
         d = iu8.resolve(wk, m, n, k)
