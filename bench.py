@@ -54,6 +54,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-moe", action="store_true")
     ap.add_argument("--no-producers", action="store_true", help="skip the Hadamard-basis producers' section")
+    ap.add_argument("--no-library", action="store_true", help="skip the vendor library's int8 GEMM reference figure (a child process)")
     ap.add_argument("--no-other-m", action="store_true", help="prefill at M = 2048 only (a profiler run that wants one M a kernel)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--probe-copy", action="store_true",
@@ -691,31 +692,17 @@ def main():
             probe[tag] = round(4 * pblocks * 4 * piters * 16 * 65536.0 / (e0.elapsed_time(e1) * 1e3) / 1e6, 1)
         # a second reference point: the vendor library's plain int8 x int8 -> int32 GEMM (torch._int_mm) on the same
         # four shapes, operands distributed like this workload's already unpacked (no W4 unpack, no scaling, int32 out,
-        # one warm weight matrix; the better of its two B orders) -- what a tuned library sustains on this card
-        lib = None
+        # one warm weight matrix; the better of its two B orders) -- what a tuned library sustains on this card. It runs
+        # as a child process (saber_engine_amd/library_ref.py): whatever the library does, this line is still printed.
+        profiled = any(k.startswith(("ROCPROF", "ROCP_")) for k in os.environ) or "rocprof" in os.environ.get("LD_PRELOAD", "")
         try:
-            lib, lib_ops, lib_us = {}, 0.0, 0.0
-            for name, n, k in linears:
-                la = torch.round(torch.randn((2048, k), device=dev, generator=g) * 2.1).clamp(-127, 127).to(torch.int8)
-                lw = torch.randint(-8, 8, (n, k), device=dev, generator=g, dtype=torch.int8) * 16
-                best = None
-                for lb in (lw.t(), lw.t().contiguous()):
-                    for _ in range(max(30, int(0.1 / (4096.0 * n * k / 2.5e15)))):
-                        lc = torch._int_mm(la, lb)
-                    l0, l1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                    l0.record()
-                    for _ in range(20):
-                        lc = torch._int_mm(la, lb)
-                    l1.record()
-                    torch.cuda.synchronize()
-                    lus = l0.elapsed_time(l1) * 1e3 / 20
-                    best = lus if best is None else min(best, lus)
-                lib[name] = dict(us=round(best, 2), tops=round(4096.0 * n * k / best / 1e6, 1))
-                lib_ops += 4096.0 * n * k
-                lib_us += best
-                del la, lw, lb, lc
-            lib["value"] = round(lib_ops / lib_us / 1e6, 1)
-        except Exception as e:   # a torch build without the int8 GEMM: the figure is a side note, never the product path
+            import subprocess
+            if args.no_library or profiled:   # no child process under a profiler's preloaded library
+                raise RuntimeError("skipped (--no-library, or running under a profiler)")
+            child = subprocess.run([sys.executable, "-m", "saber_engine_amd.library_ref", "2048"], cwd=ROOT, timeout=180,
+                                   stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
+            lib = json.loads(child.stdout.strip().splitlines()[-1]) if child.returncode == 0 else dict(error="exit %d" % child.returncode)
+        except Exception as e:   # a side note, never the product path
             lib = dict(error=str(e)[:120])
         out["prefill_m2048"] = dict(value=round(tops, 1), unit="TOPS", library_int8_gemm=lib, with_quant=round(tot_ops / (tot_us + tot_q_us) / 1e6, 1),
                                     fused_quant=dict(tops=round(tot_ops / fq_us / 1e6, 1), vs_two_launch=round((tot_us + tot_q_us) / fq_us, 3),
